@@ -1,0 +1,142 @@
+"""Writes the golden fixtures under tests/golden/ (data only).
+
+The reference's pytest files are parsed as TEXT with `ast` (nothing from the
+reference is imported or executed): for every hist-method test the literal
+arguments of its `run_regression(depth, true_values, json.loads('<model>'),
+trees)` call are copied into a JSON fixture, together with the data set the
+test trains on (Boston rows 0..9, Iris) taken from the CSV files that ship
+with scikit-learn.  The quantiser / histogram / gain vectors of the
+reference's C++ tests are small enough to be written out here by the formulas
+those tests state (file:line given per case).
+
+Run once in the build container:  python tests/golden/make_fixtures.py
+"""
+import ast
+import csv
+import json
+import os
+import sys
+
+REF = os.environ.get("ARBORETUM_REFERENCE", "/root/reference")
+HERE = os.path.dirname(os.path.abspath(__file__))
+
+
+def _calls(path):
+    tree = ast.parse(open(path).read())
+    out = {}
+    for fn in tree.body:
+        if not isinstance(fn, ast.FunctionDef) or not fn.name.startswith("test_"):
+            continue
+        for node in ast.walk(fn):
+            if isinstance(node, ast.Call) and getattr(node.func, "id", "") == "run_regression":
+                depth = ast.literal_eval(node.args[0])
+                values = ast.literal_eval(node.args[1])
+                model = json.loads(ast.literal_eval(node.args[2].args[0]))
+                trees = ast.literal_eval(node.args[3]) if len(node.args) > 3 else 1
+                out[fn.name] = {"max_depth": depth, "trees": trees, "true_values": values,
+                                "true_model": model}
+    return out
+
+
+def _config_of(path):
+    """The literal `config = {...}` dict of run_regression, names left as strings."""
+    tree = ast.parse(open(path).read())
+    for fn in tree.body:
+        if isinstance(fn, ast.FunctionDef) and fn.name == "run_regression":
+            for node in ast.walk(fn):
+                if isinstance(node, ast.Assign) and getattr(node.targets[0], "id", "") == "config":
+                    def ev(n):
+                        if isinstance(n, ast.Dict):
+                            return {ev(k): ev(v) for k, v in zip(n.keys, n.values)}
+                        if isinstance(n, ast.Name):
+                            return "$" + n.id
+                        return ast.literal_eval(n)
+                    return ev(node.value)
+    raise RuntimeError("config not found in " + path)
+
+
+def boston10():
+    import sklearn
+    p = os.path.join(os.path.dirname(sklearn.__file__), "datasets", "data", "boston_house_prices.csv")
+    if not os.path.exists(p):
+        p = "/opt/conda/lib/python3.9/site-packages/sklearn/datasets/data/boston_house_prices.csv"
+    rows = list(csv.reader(open(p)))[2:12]
+    X = [[float(v) for v in r[:13]] for r in rows]
+    y = [float(r[13]) for r in rows]
+    return X, y
+
+
+def iris():
+    import sklearn
+    p = os.path.join(os.path.dirname(sklearn.__file__), "datasets", "data", "iris.csv")
+    rows = list(csv.reader(open(p)))[1:]
+    X = [[float(v) for v in r[:4]] for r in rows]
+    t = [int(r[4]) for r in rows]
+    return X, t
+
+
+def main():
+    reg = os.path.join(REF, "tests/py/test_hist_regregression.py")
+    log = os.path.join(REF, "tests/py/test_hist_logregression.py")
+    X, y = boston10()
+    json.dump({"source": "tests/py/test_hist_regregression.py:13-56 (config), :58-138 (cases)",
+               "X": X, "y": y, "config": _config_of(reg), "cases": _calls(reg)},
+              open(os.path.join(HERE, "hist_regression_boston10.json"), "w"))
+    X, t = iris()
+    json.dump({"source": "tests/py/test_hist_logregression.py:9-66 (config), :69-162 (cases)",
+               "X": X, "target": t, "config": _config_of(log), "cases": _calls(log)},
+              open(os.path.join(HERE, "hist_logistic_iris.json"), "w"))
+
+    # ---- quantiser goldens, tests/cpp/test_datamatrix.cu
+    q = []
+    q.append({"name": "HistWideRange", "cite": "tests/cpp/test_datamatrix.cu:25-46", "hist_size": 8,
+              "x": [float(128 - i) for i in range(128)],
+              "bins": [8 - (i // 16) - 1 for i in range(128)], "bits": 4})
+    q.append({"name": "Hist255", "cite": "tests/cpp/test_datamatrix.cu:48-72", "hist_size": 255,
+              "x": [float(i) for i in range(1024)],
+              "bins": [(i // 4) if i < 1020 else 254 for i in range(1024)], "bits": 8})
+    q.append({"name": "HistSkewedRange", "cite": "tests/cpp/test_datamatrix.cu:74-112", "hist_size": 4,
+              "x": [10, 0, 11, 1, 0, 2, 3, 0, 0, 0, 0, 0], "bins": [3, 0, 3, 1, 0, 2, 3, 0, 0, 0, 0, 0],
+              "bits": 3})
+    q.append({"name": "HistTinyRange1", "cite": "tests/cpp/test_datamatrix.cu:114-152", "hist_size": 4,
+              "x": [0, 0, 0, 1, 0, 2, 0, 0, 0, 0, 0, 0], "bins": [0, 0, 0, 1, 0, 2, 0, 0, 0, 0, 0, 0],
+              "bits": 2})
+    q.append({"name": "HistTinyRange2", "cite": "tests/cpp/test_datamatrix.cu:154-197", "hist_size": 4,
+              "x": [10, 10, 10, 1, 10, 2, 10, 10, 10, 10, 10, 10], "bins": [0] * 12, "bits": 1,
+              "first_threshold_inf": True})
+    json.dump(q, open(os.path.join(HERE, "quantiser.json"), "w"))
+
+    # ---- gain / arg-max goldens, tests/cpp/test_hist.cu
+    g = []
+    # :80-121 root: 32 rows, grad (i,1), bin i/8, hist 4 -> idx 1, gain 2048
+    g.append({"name": "RootSearch", "cite": "tests/cpp/test_hist.cu:80-121", "hist_size": 4,
+              "params": [0, 0, 0, 0, 0, 0], "nodes": [
+                  {"bins": [i // 8 for i in range(32)], "g": [float(i) for i in range(32)],
+                   "h": [1.0] * 32, "best_bin": 1, "gain": 2048.0}]})
+    # :123-259 level 1: node 0 = positions 0..15 (bin p/2), node 1 = positions
+    # 16..31 (bin 7-(p-16)/2), grad (p*p,1): best global idx 4 and 11
+    g.append({"name": "Level1Search", "cite": "tests/cpp/test_hist.cu:123-259", "hist_size": 8,
+              "params": [0, 0, 0, 0, 0, 0], "nodes": [
+                  {"bins": [p // 2 for p in range(16)], "g": [float(p * p) for p in range(16)],
+                   "h": [1.0] * 16, "best_bin": 4, "gain": 64026.672,
+                   "sums": [1, 13, 41, 85, 145, 221, 313, 421]},
+                  {"bins": [7 - (p - 16) // 2 for p in range(16, 32)],
+                   "g": [float(p * p) for p in range(16, 32)], "h": [1.0] * 16, "best_bin": 3,
+                   "gain": 565504.0, "sums": [1861, 1625, 1405, 1201, 1013, 841, 685, 545]}]})
+    json.dump(g, open(os.path.join(HERE, "gain.json"), "w"))
+
+    # ---- histogram goldens, tests/cpp/test_hist_sum.cu:425-599 (asymmetric, both orientations)
+    h = [{"name": "Asymmetric10", "cite": "tests/cpp/test_hist_sum.cu:425-536", "hist_size": 4,
+          "rows": 1280, "split_at": 10,
+          "count": [3, 3, 2, 2, 317, 317, 318, 318],
+          "sum": [12.0, 15.0, 8.0, 10.0, 204148.0, 204465.0, 204792.0, 205110.0]},
+         {"name": "Asymmetric1270", "cite": "tests/cpp/test_hist_sum.cu:538-599", "hist_size": 4,
+          "rows": 1280, "split_at": 1270,
+          "count": [318, 318, 317, 317, 2, 2, 3, 3],
+          "sum": [201612.0, 201930.0, 200978.0, 201295.0, 2548.0, 2550.0, 3822.0, 3825.0]}]
+    json.dump(h, open(os.path.join(HERE, "hist_sum.json"), "w"))
+    print("fixtures written to", HERE)
+
+
+if __name__ == "__main__":
+    sys.exit(main())

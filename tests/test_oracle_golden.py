@@ -1,0 +1,242 @@
+"""Pins the CPU checker against every golden vector the reference's own tests
+hold for the histogram path (no GPU needed)."""
+import itertools
+import math
+
+import numpy as np
+import pytest
+
+from conftest import concrete_config, load_golden
+
+
+# ---------------------------------------------------------------- quantiser
+@pytest.mark.parametrize("case", load_golden("quantiser.json"), ids=lambda c: c["name"])
+def test_quantiser_golden(oracle, case):
+    thr, bins, size = oracle.quantize_column(np.array(case["x"], np.float32), case["hist_size"])
+    assert bins.tolist() == case["bins"]
+    assert int(size).bit_length() == case["bits"]          # io.cu:411: 32 - clz(size)
+    if case.get("first_threshold_inf"):
+        assert np.isinf(thr[0])
+
+
+def test_quantiser_midpoints_when_rows_fit(oracle):
+    # rows <= hist_size: thresholds are the midpoints of consecutive distinct values
+    x = np.array([3.0, 1.0, 2.0, 2.0, 7.5, -1.0], np.float32)
+    thr, bins, size = oracle.quantize_column(x, 16)
+    u = np.unique(x)
+    assert size == len(u)
+    assert np.array_equal(thr[:size - 1], ((u[1:] + u[:-1]) * 0.5).astype(np.float32))
+    assert np.array_equal(bins, np.searchsorted(u, x))
+
+
+def test_quantiser_nan_goes_to_bin_size(oracle):
+    x = np.array([0.0, np.nan, 1.0, 2.0, np.nan, 3.0], np.float32)
+    thr, bins, size = oracle.quantize_column(x, 8)
+    assert size == 4
+    assert bins.tolist() == [0, 4, 1, 2, 4, 3]
+
+
+def test_quantiser_gap_drops_trailing(oracle):
+    # 100 distinct, then 1000 equal, then 900 distinct with B = 20: everything
+    # after the first unset threshold is dropped (io.cu:403-408)
+    x = np.concatenate([np.arange(100), np.full(1000, 100.0), 101 + np.arange(900)]).astype(np.float32)
+    thr, bins, size = oracle.quantize_column(x, 20)
+    assert size == 2
+    assert bins.max() == 1
+
+
+# ------------------------------------------------------------ gain / arg-max
+def _scan(oracle, kind, bins, g, h, B, params):
+    mls, mcw, ga, gr, lam, alpha = params
+    G = np.zeros(B)
+    H = np.zeros(B)
+    C = np.zeros(B, np.int64)
+    for b_, g_, h_ in zip(bins, g, h):
+        G[b_] += g_
+        H[b_] += h_
+        C[b_] += 1
+    best, bg = -1, 0.0
+    gains = []
+    for b_ in range(B):
+        gl, hl, cl = G[:b_ + 1].sum(), H[:b_ + 1].sum(), int(C[:b_ + 1].sum())
+        v = oracle.lib().orc_gain(kind, gl, hl, cl, G.sum(), H.sum(), int(C.sum()), mls, mcw, ga, gr,
+                                  lam, alpha, 0.0)
+        gains.append(v)
+        if v > 0 and v >= bg:
+            best, bg = b_, v
+    return best, bg, G, gains
+
+
+@pytest.mark.parametrize("case", load_golden("gain.json"), ids=lambda c: c["name"])
+@pytest.mark.parametrize("kind", [2, 3])
+def test_gain_golden(oracle, case, kind):
+    for node in case["nodes"]:
+        best, bg, G, _ = _scan(oracle, kind, node["bins"], node["g"], node["h"], case["hist_size"],
+                               case["params"])
+        assert best == node["best_bin"]
+        assert bg == pytest.approx(node["gain"], rel=4e-7)   # ASSERT_FLOAT_EQ: 4 ulp
+        if "sums" in node:
+            assert G.tolist() == node["sums"]
+
+
+@pytest.mark.parametrize("kind", [0, 1, 2, 3])
+def test_gain_closed_form(oracle, kind):
+    # alpha = 0: side gain = G^2/(H+lambda); gain = GL^2/(HL+l) + GR^2/(HR+l) - GT^2/(HT+l)
+    rng = np.random.default_rng(1)
+    for _ in range(200):
+        cl, cr = int(rng.integers(1, 50)), int(rng.integers(1, 50))
+        gl, gr = rng.normal() * cl, rng.normal() * cr
+        if kind < 2:
+            hl, hr = float(cl), float(cr)
+        else:
+            hl, hr = rng.uniform(0.5, 1) * cl, rng.uniform(0.5, 1) * cr
+        lam = float(rng.uniform(0, 2))
+        v = oracle.lib().orc_gain(kind, gl, hl, cl, gl + gr, hl + hr, cl + cr, 1, 0.0, 0.0, 0.0, lam,
+                                  0.0, 0.0)
+        ref = gl * gl / (hl + lam) + gr * gr / (hr + lam) - (gl + gr) ** 2 / (hl + hr + lam)
+        assert v == pytest.approx(max(ref, 0.0), rel=2e-4, abs=1e-4)
+
+
+def test_gain_guards(oracle):
+    g = oracle.lib().orc_gain
+    # min_leaf_size on either side
+    assert g(2, 1.0, 1.0, 1, 3.0, 4.0, 4, 2, 0.0, 0, 0, 1.0, 0, 0) == 0.0
+    # min_child_weight on |H| (pair form only, gain.cu:160-162)
+    assert g(2, 1.0, 0.5, 5, -3.0, 4.0, 10, 1, 1.0, 0, 0, 1.0, 0, 0) == 0.0
+    assert g(0, 1.0, 0.0, 5, -3.0, 0.0, 10, 1, 100.0, 0, 0, 1.0, 0, 0) == 0.0  # weights forced to 0
+    # gamma_absolute
+    v = g(2, 4.0, 2.0, 2, 0.0, 4.0, 4, 1, 0.0, 0, 0, 0.0, 0, 0)
+    assert v == pytest.approx(16.0)
+    assert g(2, 4.0, 2.0, 2, 0.0, 4.0, 4, 1, 0.0, 16.0, 0, 0.0, 0, 0) == 0.0
+    # L1: |G| <= alpha gives weight 0
+    assert oracle.lib().orc_weight(2, 0.5, 2.0, 3, 1, 0.0, 1.0, 0.75, 0.0) == 0.0
+    assert oracle.lib().orc_weight(2, -2.0, 2.0, 3, 1, 0.0, 1.0, 0.5, 0.0) == pytest.approx(-0.5)
+    assert oracle.lib().orc_weight(2, -20.0, 2.0, 3, 1, 0.0, 1.0, 0.5, 1.5) == -1.5   # max_leaf_weight
+
+
+# ---------------------------------------------------------------- histograms
+@pytest.mark.parametrize("case", load_golden("hist_sum.json"), ids=lambda c: c["name"])
+def test_hist_sum_golden(oracle, case):
+    n, B = case["rows"], case["hist_size"]
+    g = np.arange(n, dtype=np.float32)
+    bins = (np.arange(n) % B).astype(np.uint8).reshape(n, 1)
+    shift = oracle.lib().orc_fix_shift(float(g.max()))
+    first = np.arange(n) < case["split_at"]
+    h0 = oracle.hist_fixed_u8(bins, g, None, shift, 0, sel=first)
+    h1 = oracle.hist_fixed_u8(bins, g, None, shift, 0, sel=~first)
+    par = oracle.hist_fixed_u8(bins, g, None, shift, 0)
+    # sibling subtraction is exact on the integers
+    assert np.array_equal(par - h0, h1)
+    got_c = np.concatenate([h0[0, :B, 2], h1[0, :B, 2]])
+    got_s = np.concatenate([h0[0, :B, 0], h1[0, :B, 0]]) * 2.0 ** -shift
+    assert got_c.tolist() == case["count"]
+    assert got_s.tolist() == case["sum"]
+
+
+def test_fixed_point_scale(oracle):
+    L = oracle.lib()
+    assert L.orc_fix_shift(1.0) == 29 and L.orc_fix_shift(0.99) == 30 and L.orc_fix_shift(0.0) == 30
+    assert L.orc_to_fixed(1.0, 30) == 1 << 30
+    assert L.orc_to_fixed(-0.25, 32) == -(1 << 30)
+    assert L.orc_to_fixed(float("nan"), 30) == 0
+
+
+def test_expf_within_one_ulp_of_libm(oracle):
+    xs = np.concatenate([np.linspace(-100, 88, 20001), np.random.default_rng(0).normal(size=20000) * 5])
+    xs = xs.astype(np.float32)
+    ours = np.array([oracle.lib().orc_expf(float(x)) for x in xs], np.float32)
+    ref = np.exp(xs.astype(np.float64))
+    ok = np.isfinite(ref) & (ref > 1e-37)
+    ulp = np.spacing(ref[ok].astype(np.float32)).astype(np.float64)
+    assert np.all(np.abs(ours[ok].astype(np.float64) - ref[ok]) <= 0.5000001 * ulp + 0)
+
+
+# ------------------------------------------------- end-to-end golden models
+def _run_cases(oracle, fixture, X, y):
+    combos = list(itertools.product([True, False], repeat=3))
+    for name, case in fixture["cases"].items():
+        for dp, trick, upload in combos:
+            for accum in (0, 1):
+                cfg = concrete_config(fixture["config"], double_precision=dp, use_hist_trick=trick,
+                                      upload_features=upload, depth=case["max_depth"])
+                b = oracle.Booster(X, y=y, config=cfg, accum=accum)
+                b.grow(case["trees"])
+                for i in range(case["trees"]):
+                    pred = b.predict(X, i + 1)
+                    assert np.allclose(pred, case["true_values"][i]), (name, dp, trick, accum, i)
+                model = b.model_dict()
+                true = case["true_model"]["model"]
+                assert len(true) == len(model["model"])
+                for tt, ct in zip(true, model["model"]):
+                    assert np.allclose(tt["weights"], ct["weights"], rtol=1e-4, atol=1e-6), name
+                    assert tt["nodes"] == ct["nodes"], (name, dp, trick, accum)
+
+
+def test_golden_regression_boston(oracle):
+    fx = load_golden("hist_regression_boston10.json")
+    _run_cases(oracle, fx, np.array(fx["X"], np.float32), np.array(fx["y"], np.float32))
+
+
+def test_golden_logistic_iris(oracle):
+    fx = load_golden("hist_logistic_iris.json")
+    X = np.array(fx["X"], np.float32)
+    y = (np.array(fx["target"]) != 2).astype(np.float32)
+    _run_cases(oracle, fx, X, y)
+
+
+# ------------------------------------------------------------- invariants
+@pytest.mark.parametrize("objective", [0, 1])
+def test_invariants_random(oracle, objective):
+    rng = np.random.default_rng(5)
+    n, F = 3000, 7
+    X = rng.normal(size=(n, F)).astype(np.float32)
+    X[rng.random((n, F)) < 0.05] = np.nan
+    w = rng.normal(size=F)
+    s = np.nan_to_num(X) @ w
+    y = (s + 0.1 * rng.normal(size=n)).astype(np.float32) if objective == 0 else (s > 0).astype(np.float32)
+    cfg = {"objective": objective, "method": 1,
+           "internals": {"hist_size": 31, "double_precision": True},
+           "tree": {"max_depth": 4, "eta": 0.3, "lambda": 1.0}}
+    b = oracle.Booster(X, y=y, config=cfg)
+    b.grow(1)
+    leaf = b.leaf()
+    bins = b.bins()
+    tr = b.tree(0)
+    # the leaf of every row equals a host traversal on its bins
+    D = 5
+    for i in range(0, n, 7):
+        nd = 0
+        for level in range(D - 1):
+            idx = (1 << level) - 1 + nd
+            q, f = tr["quantized"][idx], tr["fid"][idx]
+            right = int(q >= 0 and bins[i, f] >= q + 1)
+            nd = nd * 2 + right
+        assert nd == leaf[i]
+    # counts: sum over bins = node size; parent = left + right on the integers
+    for level in range(D - 1):
+        h = b.level_hist(level)
+        tot = h[:, :, :, 2].sum(axis=2)
+        assert np.all(tot == tot[:, :1])
+        if level > 0:
+            hp = b.level_hist(level - 1)
+            assert np.array_equal(h[0::2] + h[1::2], hp)
+    # with and without the subtraction trick: identical integers, identical tree
+    cfg2 = dict(cfg, internals=dict(cfg["internals"], use_hist_subtraction_trick=False))
+    b2 = oracle.Booster(X, y=y, config=cfg2)
+    b2.grow(1)
+    assert np.array_equal(b2.leaf(), leaf)
+    for level in range(D - 1):
+        assert np.array_equal(b.level_hist(level), b2.level_hist(level))
+    # fixed-point sums against native double accumulation: 1e-5 relative
+    b3 = oracle.Booster(X, y=y, config=cfg, accum=1)
+    b3.grow(1)
+    assert np.array_equal(b3.leaf(), leaf)
+    for level in range(D - 1):
+        a, c = b.level_hist(level, mode=1), b3.level_hist(level, mode=1)
+        assert np.allclose(a, c, rtol=1e-5, atol=1e-6)
+    # training-set prediction equals the tracked y_hat except where the raw-value
+    # walk differs from the bin walk: a value exactly on a threshold, or a NaN
+    # in an unsplit node (threshold +INF sends NaN right, training keeps it left)
+    tracked = b.yhat() if objective == 0 else 1 / (1 + np.exp(-b.yhat().astype(np.float64)))
+    clean = ~np.isnan(X).any(axis=1)
+    assert np.allclose(b.predict(X)[clean], tracked[clean], atol=1e-5)
