@@ -1,0 +1,227 @@
+#include "booster.h"
+
+#include <algorithm>
+#include <cmath>
+#include <cstring>
+#include <limits>
+#include <stdexcept>
+#include <thread>
+
+namespace arb {
+
+void ParallelFor(size_t n, const std::function<void(size_t, size_t)> &fn) {
+  unsigned hw = std::thread::hardware_concurrency();
+  size_t nt = std::max<size_t>(1, std::min<size_t>(hw ? hw : 1, 16));
+  if (n < 65536 || nt == 1) {
+    fn(0, n);
+    return;
+  }
+  std::vector<std::thread> th;
+  size_t chunk = (n + nt - 1) / nt;
+  for (size_t t = 0; t < nt; ++t) {
+    size_t b = t * chunk, e = std::min(n, b + chunk);
+    if (b >= e) break;
+    th.emplace_back([&fn, b, e] { fn(b, e); });
+  }
+  for (auto &t : th) t.join();
+}
+
+DataMatrix::DataMatrix(size_t rows, size_t columns, size_t columns_category)
+    : rows(rows), columns_dense(columns), columns_category(columns_category) {}
+
+DataMatrix::~DataMatrix() {
+  if (device) FreeDeviceMatrix(device);
+}
+
+RegTree::RegTree(unsigned depth, unsigned label) : depth(depth), label(label) {
+  const size_t internal = ((size_t)1 << (depth - 1)) - 1;
+  fid.assign(internal, 0);
+  threshold.assign(internal, std::numeric_limits<float>::infinity());
+  quantized.assign(internal, -1);
+  gain.assign(internal, 0.0f);
+  weights.assign((size_t)1 << (depth - 1), 0.0f);
+}
+
+void RegTree::Predict(const DataMatrix &data, float *out) const {
+  const size_t offset = ((size_t)1 << (depth - 1)) - 1;
+  const size_t F = data.columns_dense;
+  ParallelFor(data.rows, [&](size_t b, size_t e) {
+    for (size_t i = b; i < e; ++i) {
+      size_t id = 0;
+      for (unsigned j = 1; j < depth; ++j) {
+        const unsigned f = fid[id];
+        // a feature id outside the matrix (foreign model) behaves like NaN: right
+        const bool left = f < F && data.value(f, i) < threshold[id];
+        id = left ? 2 * id + 1 : 2 * id + 2;
+      }
+      out[i + (size_t)label * data.rows] += weights[id - offset];
+    }
+  });
+}
+
+Garden::Garden(const Configuration &c) : cfg(c) {
+  // src/core/garden.cu:571-583 accepts objectives 0 and 1 only; the soft-max
+  // ids (param.h:12-13) are implemented here from the formula the reference
+  // leaves in a comment (objective.cu:60-89).
+  switch (cfg.objective) {
+    case kLinearRegression:
+    case kLogisticRegression:
+    case kSoftMaxOneVsAll:
+    case kSoftMaxOptimal:
+      break;
+    default:
+      throw std::runtime_error("Unknown objective function");
+  }
+  if (cfg.tree.depth < 2) throw std::runtime_error("max_depth must be at least 1");
+  if (cfg.tree.depth >= 32) throw std::runtime_error("unsupported depth");  // garden.cu:536
+  if (cfg.tree.labels_count < 1) throw std::runtime_error("labels_count must be at least 1");
+}
+
+Garden::~Garden() {}
+
+float Garden::IntoInternal(float v) const {
+  if (cfg.objective == kLogisticRegression) return std::log(v / (1 - v));
+  return v;
+}
+
+void Garden::FromInternal(const std::vector<float> &in, std::vector<float> *out) const {
+  out->resize(in.size());
+  if (cfg.objective == kLinearRegression) {
+    *out = in;
+  } else if (cfg.objective == kLogisticRegression) {  // objective.h:58-69
+    for (size_t i = 0; i < in.size(); ++i) (*out)[i] = (float)(1.0 / (1.0 + (double)std::exp(-in[i])));
+  } else {  // objective.h:80-113: class-major in, row-major out
+    const size_t K = cfg.tree.labels_count;
+    const size_t n = in.size() / K;
+    std::vector<double> v(K);
+    for (size_t i = 0; i < n; ++i) {
+      double sum = 0.0;
+      for (size_t k = 0; k < K; ++k) {
+        v[k] = std::exp((double)in[i + n * k]);
+        sum += v[k];
+      }
+      for (size_t k = 0; k < K; ++k) (*out)[i * K + k] = (float)(v[k] / sum);
+    }
+  }
+}
+
+void Garden::GrowTree(DataMatrix *data, const float *grad) {
+  if (cfg.method != kHist) throw std::runtime_error("only method 1 (hist) is implemented");
+  if (grad != nullptr) throw std::runtime_error("user-supplied gradients are not supported");
+  if (cfg.objective >= kSoftMaxOneVsAll) {
+    if (data->labels.size() != data->rows) throw std::runtime_error("labels are not set");
+  } else if (data->y.size() != data->rows) {
+    throw std::runtime_error("y is not set");
+  }
+  // colsample checks of InitGrowingTree, garden.cu:126-140
+  const size_t columns = data->columns_dense;
+  if ((int)(cfg.tree.colsample_bytree * columns) == 0)
+    throw std::runtime_error("colsample_bytree is too small");
+  if ((int)(cfg.tree.colsample_bytree * cfg.tree.colsample_bylevel * columns) == 0)
+    throw std::runtime_error("colsample_bytree and colsample_bylevel are too small");
+  if ((size_t)(cfg.tree.colsample_bytree * cfg.tree.colsample_bylevel * columns) != columns)
+    throw std::runtime_error("column sampling below 1.0 is not implemented");
+  if (DeviceCount() <= 0) throw std::runtime_error("no HIP device available: training needs an MI355X");
+  if (!builder_) {
+    QuantiseOnDevice(data, cfg.internal.hist_size, cfg.verbose.data);
+    builder_.reset(CreateTreeBuilder(cfg, data));
+    builder_->SetInspect(inspect_);
+    builder_->EnableTiming(timing_);
+    bound_ = data;
+  } else if (bound_ != data) {
+    throw std::runtime_error("booster is bound to another data matrix");
+  }
+  builder_->GrowRound(&trees_);
+}
+
+void Garden::Predict(const DataMatrix *data, std::vector<float> *out, int n_rounds) const {
+  const size_t K = cfg.tree.labels_count;
+  std::vector<float> tmp(data->rows * K, IntoInternal(cfg.tree.initial_y));
+  const long long use = std::min<long long>(n_rounds, (long long)trees_.size());
+  for (long long t = 0; t < use; ++t) trees_[t].Predict(*data, tmp.data());
+  FromInternal(tmp, out);
+}
+
+void Garden::UpdateByLastTree(DataMatrix *data) {
+  const size_t K = cfg.tree.labels_count;
+  if (data->y_hat.empty()) data->y_hat.assign(data->rows * K, IntoInternal(cfg.tree.initial_y));
+  if (trees_.size() < K) return;
+  for (size_t t = trees_.size() - K; t < trees_.size(); ++t) trees_[t].Predict(*data, data->y_hat.data());
+}
+
+void Garden::GetY(const DataMatrix *data, std::vector<float> *out) const {
+  FromInternal(data->y_hat, out);
+}
+
+// src/core/model_helper.cpp:16-23, json_conversion.h:13-40
+const char *Garden::GetModel() {
+  using json::Value;
+  Value root = Value::MakeObject();
+  root["configuration"] = cfg.ToJson();
+  Value model = Value::MakeArray();
+  for (const RegTree &t : trees_) {
+    Value jt = Value::MakeObject();
+    Value nodes = Value::MakeArray();
+    const size_t internal = ((size_t)1 << (t.depth - 1)) - 1;
+    const size_t total = ((size_t)1 << t.depth) - 1;
+    for (size_t id = 0; id < total; ++id) {
+      Value n = Value::MakeObject();
+      n["id"] = Value::MakeInt((int64_t)id);
+      const bool leaf = id >= internal;
+      n["leaf"] = Value::MakeBool(leaf);
+      if (!leaf) {
+        n["left"] = Value::MakeInt((int64_t)(2 * id + 1));
+        n["right"] = Value::MakeInt((int64_t)(2 * id + 2));
+        n["threshold"] = Value::MakeFloat(t.threshold[id]);  // non-finite prints as null
+        n["fid"] = Value::MakeInt(t.fid[id]);
+      } else {
+        n["idx"] = Value::MakeInt((int64_t)(id - internal));
+      }
+      nodes.push(n);
+    }
+    jt["nodes"] = nodes;
+    Value w = Value::MakeArray();
+    for (float x : t.weights) w.push(Value::MakeFloat(x));
+    jt["weights"] = w;
+    jt["depth"] = Value::MakeInt(t.depth);
+    model.push(jt);
+  }
+  root["model"] = model;
+  model_.clear();
+  json::Dump(root, model_);
+  return model_.c_str();
+}
+
+// src/core/model_helper.cpp:25-30, json_conversion.h:26-52, garden.cu:667-677.
+// A tree without "depth" takes the booster's depth.
+void Garden::Restore(const char *json_model) {
+  json::Value j = json::Parse(json_model);
+  const json::Value *model = j.find("model");
+  if (!model || !model->is_array()) throw std::runtime_error("model: missing \"model\" array");
+  std::vector<RegTree> loaded;
+  for (const json::Value &jt : *model->a) {
+    unsigned depth = cfg.tree.depth;
+    if (const json::Value *d = jt.find("depth")) depth = (unsigned)d->number();
+    if (depth < 2 || depth >= 32) throw std::runtime_error("model: bad tree depth");
+    RegTree t(depth, 0);  // label forced to 0 as in the reference
+    const json::Value *nodes = jt.find("nodes");
+    const json::Value *weights = jt.find("weights");
+    if (!nodes || !nodes->is_array() || !weights || !weights->is_array())
+      throw std::runtime_error("model: tree needs \"nodes\" and \"weights\"");
+    if (weights->a->size() != t.weights.size()) throw std::runtime_error("model: wrong number of weights");
+    for (size_t k = 0; k < t.weights.size(); ++k) t.weights[k] = (float)(*weights->a)[k].number();
+    for (const json::Value &n : *nodes->a) {
+      const json::Value *id = n.find("id");
+      if (!id) throw std::runtime_error("model: node without id");
+      const size_t i = (size_t)id->number();
+      if (i >= t.fid.size()) continue;  // leaf record
+      if (const json::Value *th = n.find("threshold"))
+        t.threshold[i] = th->is_null() ? std::numeric_limits<float>::infinity() : (float)th->number();
+      if (const json::Value *f = n.find("fid")) t.fid[i] = (unsigned)f->number();
+    }
+    loaded.push_back(std::move(t));
+  }
+  for (RegTree &t : loaded) trees_.push_back(std::move(t));
+}
+
+}  // namespace arb

@@ -1,0 +1,141 @@
+// Host-side objects behind the C-ABI: the data matrix, the regression tree,
+// the booster ("Garden") and the interface of the GPU tree builder.
+// Counterparts in the reference: io::DataMatrix (src/io/io.h:15-83), RegTree
+// (src/core/garden.h:32-127), Garden (src/core/garden.h:141-160).
+#ifndef ARBORETUM_AMD_BOOSTER_H_
+#define ARBORETUM_AMD_BOOSTER_H_
+
+#include <cstdint>
+#include <functional>
+#include <memory>
+#include <string>
+#include <vector>
+
+#include "config.h"
+
+namespace arb {
+
+// Runs fn(begin, end) over [0, n) on a few host threads.
+void ParallelFor(size_t n, const std::function<void(size_t, size_t)> &fn);
+
+struct DeviceMatrix;  // quantised bins resident in HBM (device_builder.hip)
+
+class DataMatrix {
+ public:
+  DataMatrix(size_t rows, size_t columns, size_t columns_category);
+  ~DataMatrix();
+
+  const size_t rows;
+  const size_t columns_dense;
+  const size_t columns_category;
+
+  // Column-major host store, one contiguous vector per feature (io.h:22).
+  std::vector<std::vector<float>> data;
+  // Pre-quantised input: row-major [rows][columns_dense] bin ids instead of
+  // floats (extension; `data` is then empty).
+  std::vector<uint8_t> prebinned;
+  bool is_prebinned = false;
+  std::vector<std::vector<unsigned>> data_categories;
+
+  std::vector<float> y;
+  std::vector<float> y_hat;
+  std::vector<unsigned char> labels;
+  std::vector<float> weights;
+
+  // Quantiser output (io.h:24, 32): thresholds[f] has hist_size entries,
+  // reduced_size[f] real bins.
+  bool quantised = false;
+  int hist_size = 0;
+  std::vector<std::vector<float>> thresholds;
+  std::vector<int> reduced_size;
+  DeviceMatrix *device = nullptr;
+
+  // Feature value as seen by host prediction.
+  inline float value(size_t f, size_t i) const {
+    return is_prebinned ? (float)prebinned[i * columns_dense + f] : data[f][i];
+  }
+};
+
+// Heap-ordered tree (src/core/reg_tree.h:16-45, garden.h:32-67).
+struct RegTree {
+  unsigned depth = 0;  // internal depth: depth-1 split levels, 2^(depth-1) leaves
+  unsigned label = 0;
+  std::vector<unsigned> fid;      // 2^(depth-1)-1 internal nodes
+  std::vector<float> threshold;
+  std::vector<int> quantized;     // split bin, -1 when the node was not split
+  std::vector<float> gain;
+  std::vector<float> weights;     // 2^(depth-1)
+
+  RegTree() {}
+  RegTree(unsigned depth, unsigned label);
+  // RegTree::Predict, garden.h:70-90: x < threshold -> left; adds the leaf
+  // weight to out[i + label * rows].
+  void Predict(const DataMatrix &data, float *out) const;
+};
+
+struct BuilderTimings {  // accumulated GPU milliseconds per kernel class
+  double grad = 0, hist_root = 0, hist_deep = 0, reduce = 0, split = 0, partition = 0, leaf = 0, plan = 0;
+  unsigned long long hist_root_launches = 0, hist_deep_launches = 0;
+  unsigned long long hist_root_rows = 0, hist_deep_rows = 0;
+};
+
+// GPU tree builder bound to one (configuration, data matrix) pair.
+class TreeBuilder {
+ public:
+  virtual ~TreeBuilder() {}
+  // One boosting round: gradients, labels_count trees, prediction update.
+  virtual void GrowRound(std::vector<RegTree> *trees) = 0;
+  // Inspection (tests, benchmark).
+  virtual void SetInspect(bool on) = 0;
+  virtual void GetLeaves(uint32_t *out) = 0;               // leaf of every row, last tree
+  virtual void GetYHat(float *out) = 0;                    // labels_count * rows
+  virtual void GetGrad(float *g, float *h) = 0;            // labels_count * rows each
+  virtual int GetLevelHist(int level, int64_t *out) = 0;   // [node][F][256][3], needs inspect
+  virtual void GetShifts(int *shift_g, int *shift_h) = 0;
+  virtual void EnableTiming(bool on) = 0;
+  virtual BuilderTimings GetTimings() = 0;
+  virtual unsigned long long RowsScanned() = 0;            // rows accumulated into histograms
+  virtual void Synchronize() = 0;
+};
+
+// device_builder.hip
+void QuantiseOnDevice(DataMatrix *data, int hist_size, bool verbose);
+void FreeDeviceMatrix(DeviceMatrix *m);
+void GetDeviceBins(const DataMatrix &data, uint8_t *out);  // row-major [rows][F]
+TreeBuilder *CreateTreeBuilder(const Configuration &cfg, DataMatrix *data);
+int DeviceCount();
+
+class Garden {
+ public:
+  explicit Garden(const Configuration &cfg);
+  ~Garden();
+  const Configuration cfg;
+
+  void GrowTree(DataMatrix *data, const float *grad);        // garden.cu:585-625
+  void Predict(const DataMatrix *data, std::vector<float> *out, int n_rounds) const;  // :643-657
+  void UpdateByLastTree(DataMatrix *data);                   // :627-635
+  void GetY(const DataMatrix *data, std::vector<float> *out) const;  // :637-641
+  const char *GetModel();                                    // :659-665
+  void Restore(const char *json_model);                      // :667-677
+
+  float IntoInternal(float v) const;                         // objective.h:20,55-57
+  void FromInternal(const std::vector<float> &in, std::vector<float> *out) const;
+
+  // Inspection / timing switches; they also apply to a builder created later.
+  void SetInspect(bool on) { inspect_ = on; if (builder_) builder_->SetInspect(on); }
+  void SetTiming(bool on) { timing_ = on; if (builder_) builder_->EnableTiming(on); }
+
+  TreeBuilder *builder() { return builder_.get(); }
+  size_t num_trees() const { return trees_.size(); }
+  const RegTree &tree(size_t i) const { return trees_[i]; }
+
+ private:
+  std::unique_ptr<TreeBuilder> builder_;
+  DataMatrix *bound_ = nullptr;
+  std::vector<RegTree> trees_;
+  std::string model_;
+  bool inspect_ = false, timing_ = false;
+};
+
+}  // namespace arb
+#endif  // ARBORETUM_AMD_BOOSTER_H_

@@ -1,0 +1,1304 @@
+// GPU tree builder for gfx950 (MI355X): quantised bins resident in HBM, one
+// stream, O(1) kernel launches per tree level and no host synchronisation
+// inside a tree.
+//
+// Data layout.  Bins are uint8, four features packed in one uint32 ("quad"),
+// stored quad-column-major: quad q of row r is bins[q * stride + r].  Every
+// row pass therefore reads and writes fully coalesced 256-byte wave
+// transactions.  Rows of one tree node are kept contiguous: after the split of
+// level k is known, a stable partition moves (bins, grad, hess, row id) from
+// the level-k order into the level-(k+1) order (ping-pong buffers).  Every
+// tree starts again from the original order, so y and y_hat never move.
+//
+// Histograms.  One workgroup owns a contiguous row range of one node and a
+// private histogram in LDS: two 64-bit words per (feature, bin),
+//   word0 = count << 47 | sum of g_q   (g_q fixed point, |g_q| <= 2^30)
+//   word1 = sum of h_q
+// so one update costs two ds_add_u64 (one for the squared objective).  A range
+// holds at most 64512 rows, which keeps both fields exact.  Each workgroup
+// writes its LDS histogram to a private slab in HBM; a reduce kernel adds the
+// slabs of a node, and derives the larger sibling as parent - smaller child.
+// All sums are integers: the result does not depend on scheduling.
+//
+// What replaces what (reference file:line):
+//   k_bin_assign      build_histogram              src/io/io.cu:293-312
+//   k_grad_*          update_grad                  src/core/objective.cu:15-56
+//   k_root_total      cub::DeviceReduce::Sum       src/core/garden.cu:432-435
+//   k_hist            hist_sum_node / hist_sum_multi_node
+//                                                  src/core/hist_grad_sum.cu:109-215,262-406
+//   k_hist_reduce     update_multi_node + global atomics
+//                                                  src/core/hist_grad_sum.cu:6-33
+//   k_split_scan      DeviceScan + hist_gain_kernel
+//                                                  src/core/hist_tree_grower.cu:9-35,393-416
+//   k_split_select    hist_apply_candidates        src/core/hist_tree_grower.cu:37-102
+//   k_part_*          apply_split, set_segment, CreatePartitioningIndexes,
+//                     scatter_kernel               src/core/builder.h:51-59,107-123,287-300
+//   k_leaf_*          UpdateLeafWeight, update_by_last_tree
+//                                                  src/core/garden.cu:45-76,487-503
+#include <hip/hip_runtime.h>
+
+#include <algorithm>
+#include <atomic>
+#include <cmath>
+#include <cstdio>
+#include <cstring>
+#include <limits>
+#include <stdexcept>
+#include <string>
+#include <thread>
+#include <vector>
+
+#include "booster.h"
+#include "gain.h"
+
+namespace arb {
+namespace {
+
+#define HIP_OK(expr)                                                                        \
+  do {                                                                                      \
+    hipError_t e_ = (expr);                                                                 \
+    if (e_ != hipSuccess)                                                                   \
+      throw std::runtime_error(std::string("HIP error: ") + hipGetErrorString(e_) + " in " #expr); \
+  } while (0)
+
+constexpr int kSlots = 256;               // histogram slots per feature (uint8 bins)
+constexpr int kHistThreads = 1024;        // one workgroup per CU, 16 waves
+constexpr int kPartThreads = 256;
+constexpr unsigned kPartRows = 4096;      // rows per partition work item
+constexpr unsigned kMaxHistRows = 64512;  // rows per histogram work item (< 2^16)
+constexpr int kCountShift = 47;           // word0 = count << 47 | g
+constexpr int kMaxPlanNodes = 4096;       // nodes per level the planner handles
+constexpr size_t kLdsBudget = 160 * 1024;
+
+struct NodeSum {
+  long long g;
+  long long h;
+  unsigned long long c;
+};
+
+struct SplitRec {
+  float gain;
+  int fid;   // -1: not split (every row stays left)
+  int bin;
+  unsigned pad;
+  NodeSum left;
+};
+
+struct WorkItem {
+  unsigned node;
+  unsigned begin;  // row range in the current order
+  unsigned end;
+  unsigned first;  // index of the first work item of this node
+};
+
+// --------------------------------------------------------------- quantiser
+// bin(x) = first l in [0,size] with x <= v[l], v[t] = thr[t] for t < size-1,
+// +INF above (src/core/cuda_helpers.h:207-222, src/io/io.cu:297-302); NaN
+// compares false everywhere and lands in bin `size`.
+__global__ void k_bin_assign(const float *__restrict__ x, int ncols, const float *__restrict__ thr,
+                             int thr_stride, const int *__restrict__ sizes,
+                             uint32_t *__restrict__ out, size_t n) {
+  __shared__ float s_thr[4][kSlots];
+  __shared__ int s_size[4];
+  for (int i = threadIdx.x; i < 4 * kSlots; i += blockDim.x) {
+    const int c = i >> 8, t = i & 255;
+    float v = INFINITY;
+    if (c < ncols && t < sizes[c] - 1) v = thr[(size_t)c * thr_stride + t];
+    s_thr[c][t] = v;
+  }
+  if (threadIdx.x < 4) s_size[threadIdx.x] = threadIdx.x < ncols ? sizes[threadIdx.x] : 0;
+  __syncthreads();
+  for (size_t r = (size_t)blockIdx.x * blockDim.x + threadIdx.x; r < n;
+       r += (size_t)gridDim.x * blockDim.x) {
+    uint32_t packed = 0;
+#pragma unroll
+    for (int c = 0; c < 4; ++c) {
+      if (c < ncols) {
+        const float v = x[(size_t)c * n + r];
+        unsigned l = 0, h = (unsigned)s_size[c];
+        while (l < h) {
+          const unsigned mid = (l + h) >> 1;
+          if (v <= s_thr[c][mid])
+            h = mid;
+          else
+            l = mid + 1;
+        }
+        packed |= l << (8 * c);
+      }
+    }
+    out[r] = packed;
+  }
+}
+
+// row-major uint8 [n][F] -> quads
+__global__ void k_pack_prebinned(const uint8_t *__restrict__ in, int F, int Q,
+                                 uint32_t *__restrict__ out, size_t stride, size_t n) {
+  for (size_t r = (size_t)blockIdx.x * blockDim.x + threadIdx.x; r < n;
+       r += (size_t)gridDim.x * blockDim.x) {
+    for (int q = 0; q < Q; ++q) {
+      uint32_t packed = 0;
+      for (int c = 0; c < 4; ++c) {
+        const int f = q * 4 + c;
+        if (f < F) packed |= (uint32_t)in[r * F + f] << (8 * c);
+      }
+      out[(size_t)q * stride + r] = packed;
+    }
+  }
+}
+
+// ------------------------------------------------------------- objectives
+__device__ __forceinline__ float WaveMaxF(float v) {
+  for (int off = 32; off > 0; off >>= 1) v = fmaxf(v, __shfl_down(v, off));
+  return v;
+}
+__device__ __forceinline__ long long WaveSumLL(long long v) {
+  for (int off = 32; off > 0; off >>= 1) v += __shfl_down(v, off);
+  return v;
+}
+
+// squared error: g = y - y_hat (objective.cu:28-38); also max |g| for the
+// fixed-point scale
+__global__ void k_grad_squared(const float *__restrict__ y, const float *__restrict__ yhat,
+                               float *__restrict__ g, size_t n, unsigned *__restrict__ gmax_bits) {
+  float m = 0.0f;
+  for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < n;
+       i += (size_t)gridDim.x * blockDim.x) {
+    const float v = y[i] - yhat[i];
+    g[i] = v;
+    const float a = fabsf(v);
+    if (a > m) m = a;  // NaN never raises the maximum
+  }
+  m = WaveMaxF(m);
+  if ((threadIdx.x & 63) == 0) atomicMax(gmax_bits, __float_as_uint(m));
+}
+
+__global__ void k_set_shift(const unsigned *__restrict__ gmax_bits, int *__restrict__ shifts) {
+  if (threadIdx.x == 0 && blockIdx.x == 0) {
+    shifts[0] = FixShiftFromMax(__uint_as_float(*gmax_bits));
+    shifts[1] = 0;
+  }
+}
+
+// logistic: s = sigmoid(y_hat), g = y - s, h = s(1-s) (objective.cu:43-56)
+__global__ void k_grad_logistic(const float *__restrict__ y, const float *__restrict__ yhat,
+                                float *__restrict__ g, float *__restrict__ h, size_t n) {
+  for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < n;
+       i += (size_t)gridDim.x * blockDim.x) {
+    const float s = SigmoidF(yhat[i]);
+    g[i] = y[i] - s;
+    h[i] = s * (1.0f - s);
+  }
+}
+
+// soft-max: p = softmax(y_hat[., row]), g_k = [label == k] - p_k,
+// h_k = 2 p_k (1 - p_k) (formula in the comment at objective.cu:60-89).
+// y_hat, g, h are class-major [K][n].
+__global__ void k_grad_softmax(const uint8_t *__restrict__ labels, const float *__restrict__ yhat,
+                               float *__restrict__ g, float *__restrict__ h, size_t n, int K) {
+  for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < n;
+       i += (size_t)gridDim.x * blockDim.x) {
+    double mx = -1e300;
+    for (int k = 0; k < K; ++k) mx = fmax(mx, (double)yhat[i + (size_t)k * n]);
+    double sum = 0.0;
+    for (int k = 0; k < K; ++k) sum += (double)ExpF((float)((double)yhat[i + (size_t)k * n] - mx));
+    const int lab = labels[i];
+    for (int k = 0; k < K; ++k) {
+      const double e = (double)ExpF((float)((double)yhat[i + (size_t)k * n] - mx));
+      const float pk = (float)(e / sum);
+      g[i + (size_t)k * n] = (lab == k ? 1.0f : 0.0f) - pk;
+      h[i + (size_t)k * n] = 2.0f * pk * (1.0f - pk);
+    }
+  }
+}
+
+// Root totals in fixed point.
+template <bool PAIR>
+__global__ void k_root_total(const float *__restrict__ g, const float *__restrict__ h,
+                             const int *__restrict__ shifts, size_t n, NodeSum *__restrict__ tot) {
+  const int sg = shifts[0], sh = shifts[1];
+  long long a = 0, b = 0;
+  for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < n;
+       i += (size_t)gridDim.x * blockDim.x) {
+    a += ToFixed(g[i], sg);
+    if (PAIR) b += ToFixed(h[i], sh);
+  }
+  a = WaveSumLL(a);
+  if (PAIR) b = WaveSumLL(b);
+  if ((threadIdx.x & 63) == 0) {
+    atomicAdd((unsigned long long *)&tot->g, (unsigned long long)a);
+    if (PAIR) atomicAdd((unsigned long long *)&tot->h, (unsigned long long)b);
+  }
+}
+
+__global__ void k_init_root(NodeSum *tot, unsigned *seg_start, unsigned long long n,
+                            unsigned *gmax_bits) {
+  if (threadIdx.x == 0 && blockIdx.x == 0) {
+    tot[0].g = 0;
+    tot[0].h = 0;
+    tot[0].c = n;
+    seg_start[0] = 0;
+    if (gmax_bits) *gmax_bits = 0;
+  }
+}
+
+// ------------------------------------------------------------------ planner
+// Splits the row ranges of the selected nodes of a level into work items of
+// at most `rows_per_item` rows.  select: 0 = every node, 1 = the smaller
+// child of each sibling pair, ties -> left (hist_grad_sum.cu:279-294).
+// One workgroup.
+__global__ void __launch_bounds__(1024)
+k_plan(const NodeSum *__restrict__ tot, const unsigned *__restrict__ seg_start, int L, int select,
+       unsigned rows_per_item, WorkItem *__restrict__ work, unsigned *__restrict__ n_work,
+       unsigned *__restrict__ node_first, unsigned *__restrict__ node_items,
+       unsigned long long *__restrict__ rows_scanned, unsigned max_items) {
+  __shared__ unsigned s_base[kMaxPlanNodes + 1];
+  __shared__ unsigned s_wave[16];
+  __shared__ unsigned s_carry;
+  __shared__ unsigned long long s_rows;
+  const int tid = threadIdx.x;
+  if (tid == 0) {
+    s_carry = 0;
+    s_rows = 0;
+  }
+  __syncthreads();
+  for (int base = 0; base < L; base += 1024) {
+    const int nd = base + tid;
+    unsigned cnt = 0;
+    if (nd < L) {
+      const unsigned long long len = tot[nd].c;
+      bool sel = true;
+      if (select == 1) {
+        const unsigned long long sib = tot[nd ^ 1].c;
+        sel = (nd & 1) ? (len < sib) : (len <= sib);
+      }
+      if (sel && len > 0) {
+        cnt = (unsigned)((len + rows_per_item - 1) / rows_per_item);
+        atomicAdd(&s_rows, len);
+      }
+      node_items[nd] = sel ? cnt : 0xffffffffu;  // 0xffffffff marks "not selected"
+    }
+    // block exclusive scan of cnt
+    unsigned incl = cnt;
+    for (int off = 1; off < 64; off <<= 1) {
+      const unsigned o = __shfl_up(incl, off);
+      if ((tid & 63) >= off) incl += o;
+    }
+    if ((tid & 63) == 63) s_wave[tid >> 6] = incl;
+    __syncthreads();
+    unsigned wave_off = 0;
+    for (int w = 0; w < (tid >> 6); ++w) wave_off += s_wave[w];
+    const unsigned excl = s_carry + wave_off + incl - cnt;
+    if (nd < L) {
+      s_base[nd] = excl;
+      node_first[nd] = excl;
+    }
+    __syncthreads();
+    if (tid == 1023) s_carry = excl + cnt;
+    __syncthreads();
+  }
+  const unsigned total = s_carry;
+  if (tid == 0) {
+    s_base[L] = total;
+    *n_work = total <= max_items ? total : 0;  // never exceed the launch bound
+    if (rows_scanned) *rows_scanned += s_rows;
+  }
+  __syncthreads();
+  if (total > max_items) return;
+  for (unsigned w = tid; w < total; w += 1024) {
+    int lo = 0, hi = L;  // last node with s_base[node] <= w and items > 0
+    while (hi - lo > 1) {
+      const int mid = (lo + hi) >> 1;
+      if (s_base[mid] <= w)
+        lo = mid;
+      else
+        hi = mid;
+    }
+    const unsigned start = seg_start[lo];
+    const unsigned len = (unsigned)tot[lo].c;
+    const unsigned k = w - s_base[lo];
+    WorkItem it;
+    it.node = lo;
+    it.begin = start + k * rows_per_item;
+    it.end = min(start + len, it.begin + rows_per_item);
+    it.first = s_base[lo];
+    work[w] = it;
+  }
+}
+
+// ---------------------------------------------------------------- histogram
+// One workgroup per work item.  LDS: nq*1024 word0 entries, then (PAIR) as
+// many word1 entries.  Handles quads [q0, q0+nq).
+template <bool PAIR>
+__global__ void __launch_bounds__(kHistThreads)
+k_hist(const uint32_t *__restrict__ bins, size_t stride, int q0, int nq, int F,
+       const float *__restrict__ g, const float *__restrict__ h, const int *__restrict__ shifts,
+       const WorkItem *__restrict__ work, const unsigned *__restrict__ n_work,
+       unsigned long long *__restrict__ slab, int nbin_total) {
+  extern __shared__ unsigned long long lds[];
+  const unsigned w = blockIdx.x;
+  if (w >= *n_work) return;
+  const WorkItem it = work[w];
+  const int nbin = nq * 4 * kSlots;
+  const int words = PAIR ? 2 * nbin : nbin;
+  for (int i = threadIdx.x; i < words; i += kHistThreads) lds[i] = 0ull;
+  __syncthreads();
+  const int sg = shifts[0], sh = shifts[1];
+  unsigned long long *lds1 = lds + nbin;
+  for (unsigned r = it.begin + threadIdx.x; r < it.end; r += kHistThreads) {
+    const unsigned long long w0 = (1ull << kCountShift) + (unsigned long long)ToFixed(g[r], sg);
+    unsigned long long w1 = 0;
+    if (PAIR) w1 = (unsigned long long)ToFixed(h[r], sh);
+    for (int q = 0; q < nq; ++q) {
+      const uint32_t b4 = bins[(size_t)(q0 + q) * stride + r];
+#pragma unroll
+      for (int c = 0; c < 4; ++c) {
+        if ((q0 + q) * 4 + c < F) {
+          const unsigned idx = (unsigned)(q * 4 + c) * kSlots + ((b4 >> (8 * c)) & 255u);
+          atomicAdd(&lds[idx], w0);
+          if (PAIR) atomicAdd(&lds1[idx], w1);
+        }
+      }
+    }
+  }
+  __syncthreads();
+  // slab layout per work item: word0[nbin_total], word1[nbin_total]
+  unsigned long long *out = slab + (size_t)w * nbin_total * (PAIR ? 2 : 1) + (size_t)q0 * 4 * kSlots;
+  for (int i = threadIdx.x; i < nbin; i += kHistThreads) {
+    out[i] = lds[i];
+    if (PAIR) out[nbin_total + i] = lds1[i];
+  }
+}
+
+// Adds the slabs of every selected node; with `trick` also writes the sibling
+// as parent - node.  grid (nbin_total/64, L), 1024 threads = 64 entries x 16
+// slab lanes.
+template <bool PAIR>
+__global__ void __launch_bounds__(1024)
+k_hist_reduce(const unsigned long long *__restrict__ slab, int nbin_total,
+              const unsigned *__restrict__ node_first, const unsigned *__restrict__ node_items,
+              long long *__restrict__ hg, long long *__restrict__ hh, unsigned *__restrict__ hc,
+              const long long *__restrict__ pg, const long long *__restrict__ ph,
+              const unsigned *__restrict__ pc, int trick) {
+  __shared__ long long s_g[16][64];
+  __shared__ long long s_h[16][64];
+  __shared__ unsigned s_c[16][64];
+  const int nd = blockIdx.y;
+  const unsigned items = node_items[nd];
+  if (items == 0xffffffffu) return;  // derived from its sibling
+  const int e = threadIdx.x & 63, lane = threadIdx.x >> 6;
+  const int entry = blockIdx.x * 64 + e;
+  const unsigned first = node_first[nd];
+  long long ag = 0, ah = 0;
+  unsigned ac = 0;
+  for (unsigned s = lane; s < items; s += 16) {
+    const unsigned long long *p = slab + (size_t)(first + s) * nbin_total * (PAIR ? 2 : 1);
+    const unsigned long long w0 = p[entry];
+    const long long gq = ((long long)(w0 << (64 - kCountShift))) >> (64 - kCountShift);
+    ag += gq;
+    ac += (unsigned)((w0 - (unsigned long long)gq) >> kCountShift);
+    if (PAIR) ah += (long long)p[nbin_total + entry];
+  }
+  s_g[lane][e] = ag;
+  s_h[lane][e] = ah;
+  s_c[lane][e] = ac;
+  __syncthreads();
+  if (lane == 0) {
+    for (int k = 1; k < 16; ++k) {
+      ag += s_g[k][e];
+      ah += s_h[k][e];
+      ac += s_c[k][e];
+    }
+    const size_t o = (size_t)nd * nbin_total + entry;
+    hg[o] = ag;
+    hh[o] = ah;
+    hc[o] = ac;
+    if (trick) {
+      const size_t po = (size_t)(nd >> 1) * nbin_total + entry;
+      const size_t so = (size_t)(nd ^ 1) * nbin_total + entry;
+      hg[so] = pg[po] - ag;
+      hh[so] = ph[po] - ah;
+      hc[so] = pc[po] - ac;
+    }
+  }
+}
+
+// --------------------------------------------------------------- split scan
+struct Cand {
+  float gain;
+  int bin;
+  NodeSum left;
+};
+
+// One wave per (feature, node): inclusive prefix over the 256 slots, gain per
+// bin < hist_size, arg-max with ties to the HIGHEST bin (builder.h:39-49),
+// only gains > 0 (hist_tree_grower.cu:31).
+template <bool PAIR, bool F64>
+__global__ void __launch_bounds__(64)
+k_split_scan(const long long *__restrict__ hg, const long long *__restrict__ hh,
+             const unsigned *__restrict__ hc, int nbin_total, int F,
+             const NodeSum *__restrict__ tot, const int *__restrict__ shifts, GainParams gp,
+             int hist_size, Cand *__restrict__ cand) {
+  const int f = blockIdx.x, nd = blockIdx.y, lane = threadIdx.x;
+  const NodeSum t = tot[nd];
+  Cand best;
+  best.gain = 0.0f;
+  best.bin = -1;
+  best.left.g = best.left.h = 0;
+  best.left.c = 0;
+  if (t.c != 0) {
+    const int sg = shifts[0], sh = shifts[1];
+    const size_t base = (size_t)nd * nbin_total + (size_t)f * kSlots + lane * 4;
+    long long g4[4], h4[4];
+    unsigned long long c4[4];
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      g4[j] = hg[base + j];
+      h4[j] = PAIR ? hh[base + j] : 0;
+      c4[j] = hc[base + j];
+    }
+#pragma unroll
+    for (int j = 1; j < 4; ++j) {
+      g4[j] += g4[j - 1];
+      h4[j] += h4[j - 1];
+      c4[j] += c4[j - 1];
+    }
+    long long ig = g4[3], ih = h4[3];
+    unsigned long long ic = c4[3];
+    for (int off = 1; off < 64; off <<= 1) {
+      const long long og = __shfl_up(ig, off);
+      const long long oh = __shfl_up(ih, off);
+      const unsigned long long oc = __shfl_up(ic, off);
+      if (lane >= off) {
+        ig += og;
+        ih += oh;
+        ic += oc;
+      }
+    }
+    const long long eg = ig - g4[3], eh = ih - h4[3];
+    const unsigned long long ec = ic - c4[3];
+    const double GT = FromFixed<F64>(t.g, sg);
+    const double HT = PAIR ? FromFixed<F64>(t.h, sh) : 0.0;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const int bin = lane * 4 + j;
+      if (bin < hist_size) {
+        const long long lg = eg + g4[j], lh = eh + h4[j];
+        const unsigned long long lc = ec + c4[j];
+        const double GL = FromFixed<F64>(lg, sg);
+        const double HL = PAIR ? FromFixed<F64>(lh, sh) : 0.0;
+        const float gn = SplitGain<PAIR, F64>(GL, HL, lc, GT, HT, t.c, gp);
+        if (gn > 0.0f && gn >= best.gain) {
+          best.gain = gn;
+          best.bin = bin;
+          best.left.g = lg;
+          best.left.h = lh;
+          best.left.c = lc;
+        }
+      }
+    }
+    for (int off = 32; off > 0; off >>= 1) {
+      const float og = __shfl_down(best.gain, off);
+      const int ob = __shfl_down(best.bin, off);
+      const long long olg = __shfl_down(best.left.g, off);
+      const long long olh = __shfl_down(best.left.h, off);
+      const unsigned long long olc = __shfl_down(best.left.c, off);
+      if (ob >= 0 && (best.bin < 0 || og > best.gain || (og == best.gain && ob > best.bin))) {
+        best.gain = og;
+        best.bin = ob;
+        best.left.g = olg;
+        best.left.h = olh;
+        best.left.c = olc;
+      }
+    }
+  }
+  if (lane == 0) cand[(size_t)nd * F + f] = best;
+}
+
+// One thread per node: best candidate over features (higher gain, then lower
+// feature id: hist_tree_grower.cu:59-60), children totals and row ranges,
+// node record.  A node without a candidate keeps every row left.
+__global__ void k_split_select(const Cand *__restrict__ cand, int F, int L,
+                               const NodeSum *__restrict__ tot,
+                               const unsigned *__restrict__ seg_start,
+                               NodeSum *__restrict__ tot_next, unsigned *__restrict__ seg_next,
+                               SplitRec *__restrict__ split, int *__restrict__ t_fid,
+                               int *__restrict__ t_bin, float *__restrict__ t_gain, int heap_off) {
+  const int nd = blockIdx.x * blockDim.x + threadIdx.x;
+  if (nd >= L) return;
+  const NodeSum t = tot[nd];
+  SplitRec rec;
+  rec.gain = 0.0f;
+  rec.fid = -1;
+  rec.bin = -1;
+  rec.pad = 0;
+  rec.left = t;
+  if (t.c != 0) {
+    for (int f = 0; f < F; ++f) {
+      const Cand c = cand[(size_t)nd * F + f];
+      if (c.bin >= 0 && (rec.fid < 0 || rec.gain < c.gain)) {
+        rec.gain = c.gain;
+        rec.fid = f;
+        rec.bin = c.bin;
+        rec.left = c.left;
+      }
+    }
+  }
+  split[nd] = rec;
+  NodeSum r;
+  r.g = t.g - rec.left.g;
+  r.h = t.h - rec.left.h;
+  r.c = t.c - rec.left.c;
+  tot_next[2 * nd] = rec.left;
+  tot_next[2 * nd + 1] = r;
+  const unsigned start = seg_start[nd];
+  seg_next[2 * nd] = start;
+  seg_next[2 * nd + 1] = start + (unsigned)rec.left.c;
+  t_fid[heap_off + nd] = rec.fid < 0 ? 0 : rec.fid;  // garden.cu:471-481
+  t_bin[heap_off + nd] = rec.fid < 0 ? -1 : rec.bin;
+  t_gain[heap_off + nd] = rec.gain;
+}
+
+// ---------------------------------------------------------------- partition
+__device__ __forceinline__ bool GoesRight(const uint32_t *__restrict__ bins, size_t stride,
+                                          const SplitRec &s, unsigned r) {
+  // builder.h:107-123: bin >= q + 1 goes right
+  if (s.fid < 0) return false;
+  const uint32_t b4 = bins[(size_t)(s.fid >> 2) * stride + r];
+  return (int)((b4 >> (8 * (s.fid & 3))) & 255u) > s.bin;
+}
+
+__global__ void __launch_bounds__(kPartThreads)
+k_part_count(const uint32_t *__restrict__ bins, size_t stride, const SplitRec *__restrict__ split,
+             const WorkItem *__restrict__ work, const unsigned *__restrict__ n_work,
+             unsigned *__restrict__ item_left) {
+  __shared__ unsigned s_cnt[kPartThreads / 64];
+  const unsigned w = blockIdx.x;
+  if (w >= *n_work) return;
+  const WorkItem it = work[w];
+  const SplitRec s = split[it.node];
+  unsigned cnt = 0;
+  for (unsigned r = it.begin + threadIdx.x; r < it.end; r += kPartThreads)
+    cnt += GoesRight(bins, stride, s, r) ? 0u : 1u;
+  for (int off = 32; off > 0; off >>= 1) cnt += __shfl_down(cnt, off);
+  if ((threadIdx.x & 63) == 0) s_cnt[threadIdx.x >> 6] = cnt;
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    unsigned t = 0;
+    for (int k = 0; k < kPartThreads / 64; ++k) t += s_cnt[k];
+    item_left[w] = t;
+  }
+}
+
+// Exclusive scan of item_left over all work items.  One workgroup.
+__global__ void __launch_bounds__(1024)
+k_part_scan(const unsigned *__restrict__ item_left, const unsigned *__restrict__ n_work,
+            unsigned *__restrict__ excl) {
+  __shared__ unsigned s_part[1024];
+  const unsigned n = *n_work;
+  const unsigned per = (n + 1023) / 1024;
+  const unsigned b = threadIdx.x * per, e = min(n, b + per);
+  unsigned sum = 0;
+  for (unsigned i = b; i < e; ++i) sum += item_left[i];
+  s_part[threadIdx.x] = sum;
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    unsigned run = 0;
+    for (int i = 0; i < 1024; ++i) {
+      const unsigned v = s_part[i];
+      s_part[i] = run;
+      run += v;
+    }
+  }
+  __syncthreads();
+  unsigned run = s_part[threadIdx.x];
+  for (unsigned i = b; i < e; ++i) {
+    excl[i] = run;
+    run += item_left[i];
+  }
+}
+
+// Stable partition of one work item's rows into the children ranges.
+template <bool PAIR>
+__global__ void __launch_bounds__(kPartThreads)
+k_partition(const uint32_t *__restrict__ bins, uint32_t *__restrict__ bins_out, size_t stride, int Q,
+            const float *__restrict__ g, float *__restrict__ g_out, const float *__restrict__ h,
+            float *__restrict__ h_out, const unsigned *__restrict__ rowid,
+            unsigned *__restrict__ rowid_out, const SplitRec *__restrict__ split,
+            const unsigned *__restrict__ seg_start, const WorkItem *__restrict__ work,
+            const unsigned *__restrict__ n_work, const unsigned *__restrict__ excl) {
+  __shared__ unsigned s_cnt[kPartThreads / 64];
+  const unsigned w = blockIdx.x;
+  if (w >= *n_work) return;
+  const WorkItem it = work[w];
+  const SplitRec s = split[it.node];
+  const unsigned start = seg_start[it.node];
+  const unsigned lefts_before = excl[w] - excl[it.first];
+  unsigned lo = start + lefts_before;
+  unsigned ro = start + (unsigned)s.left.c + (it.begin - start) - lefts_before;
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  for (unsigned base = it.begin; base < it.end; base += kPartThreads) {
+    const unsigned r = base + threadIdx.x;
+    const bool valid = r < it.end;
+    const bool right = valid && GoesRight(bins, stride, s, r);
+    const bool left = valid && !right;
+    const unsigned long long lm = __ballot(left);
+    const unsigned long long below = (1ull << lane) - 1ull;
+    if (lane == 0) s_cnt[wave] = (unsigned)__popcll(lm);
+    __syncthreads();
+    unsigned left_waves = 0, left_tile = 0;
+#pragma unroll
+    for (int k = 0; k < kPartThreads / 64; ++k) {
+      const unsigned c = s_cnt[k];
+      if (k < wave) left_waves += c;
+      left_tile += c;
+    }
+    const unsigned lrank = left_waves + (unsigned)__popcll(lm & below);
+    const unsigned rrank = (unsigned)threadIdx.x - lrank;  // invalid lanes only sit above valid ones
+    const unsigned tile_valid = min((unsigned)kPartThreads, it.end - base);
+    if (valid) {
+      const unsigned d = left ? lo + lrank : ro + rrank;
+      for (int q = 0; q < Q; ++q) bins_out[(size_t)q * stride + d] = bins[(size_t)q * stride + r];
+      g_out[d] = g[r];
+      if (PAIR) h_out[d] = h[r];
+      rowid_out[d] = rowid ? rowid[r] : r;
+    }
+    lo += left_tile;
+    ro += tile_valid - left_tile;
+    __syncthreads();
+  }
+}
+
+// --------------------------------------------------------------- leaves
+// UpdateLeafWeight (garden.cu:487-503, split.cu:25-35): left = Weight(left
+// sum), right = Weight(parent - left) with the subtraction in the sum type.
+template <bool PAIR, bool F64>
+__global__ void k_leaf_weights(const SplitRec *__restrict__ split, const NodeSum *__restrict__ tot,
+                               int L, const int *__restrict__ shifts, GainParams gp, float eta,
+                               float *__restrict__ weights) {
+  const int nd = blockIdx.x * blockDim.x + threadIdx.x;
+  if (nd >= L) return;
+  const int sg = shifts[0], sh = shifts[1];
+  const SplitRec s = split[nd];
+  const NodeSum t = tot[nd];
+  const double GL = FromFixed<F64>(s.left.g, sg), HL = PAIR ? FromFixed<F64>(s.left.h, sh) : 0.0;
+  const double GP = FromFixed<F64>(t.g, sg), HP = PAIR ? FromFixed<F64>(t.h, sh) : 0.0;
+  double GR, HR;
+  if (F64) {
+    GR = GP - GL;
+    HR = HP - HL;
+  } else {
+    GR = (double)((float)GP - (float)GL);
+    HR = (double)((float)HP - (float)HL);
+  }
+  weights[2 * nd] = LeafWeight<PAIR, F64>(GL, HL, (unsigned)s.left.c, gp) * eta;
+  weights[2 * nd + 1] = LeafWeight<PAIR, F64>(GR, HR, (unsigned)(t.c - s.left.c), gp) * eta;
+}
+
+// leaf id of every row of the last split level, scattered to original order
+__global__ void __launch_bounds__(kPartThreads)
+k_leaf_assign(const uint32_t *__restrict__ bins, size_t stride, const unsigned *__restrict__ rowid,
+              const SplitRec *__restrict__ split, const WorkItem *__restrict__ work,
+              const unsigned *__restrict__ n_work, unsigned *__restrict__ leaf_of) {
+  const unsigned w = blockIdx.x;
+  if (w >= *n_work) return;
+  const WorkItem it = work[w];
+  const SplitRec s = split[it.node];
+  for (unsigned r = it.begin + threadIdx.x; r < it.end; r += kPartThreads) {
+    const unsigned leaf = it.node * 2 + (GoesRight(bins, stride, s, r) ? 1u : 0u);
+    leaf_of[rowid ? rowid[r] : r] = leaf;
+  }
+}
+
+// update_by_last_tree (garden.cu:45-76): y_hat += weight of the row's leaf
+__global__ void k_update_yhat(float *__restrict__ yhat, const unsigned *__restrict__ leaf_of,
+                              const float *__restrict__ weights, size_t n) {
+  for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < n;
+       i += (size_t)gridDim.x * blockDim.x)
+    yhat[i] += weights[leaf_of[i]];
+}
+
+__global__ void k_fill_f32(float *p, float v, size_t n) {
+  for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < n;
+       i += (size_t)gridDim.x * blockDim.x)
+    p[i] = v;
+}
+
+template <typename T>
+T *DevAlloc(size_t n) {
+  void *p = nullptr;
+  HIP_OK(hipMalloc(&p, std::max<size_t>(n, 1) * sizeof(T)));
+  return static_cast<T *>(p);
+}
+
+inline int GridFor(size_t n, int block, int cap = 4096) {
+  size_t g = (n + block - 1) / block;
+  return (int)std::max<size_t>(1, std::min<size_t>(g, cap));
+}
+
+}  // namespace
+
+struct DeviceMatrix {
+  size_t rows = 0, stride = 0;
+  int F = 0, Q = 0;
+  uint32_t *bins = nullptr;  // [Q][stride]
+};
+
+int DeviceCount() {
+  int n = 0;
+  if (hipGetDeviceCount(&n) != hipSuccess) return 0;
+  return n;
+}
+
+void FreeDeviceMatrix(DeviceMatrix *m) {
+  if (!m) return;
+  if (m->bins) (void)hipFree(m->bins);
+  delete m;
+}
+
+// Thresholds of one column, from the sorted column: the k-th change of value
+// at sorted position i writes its midpoint to slot min(k+1, i/seg+1) - 2,
+// lowest midpoint wins (src/io/io.cu:349-410, 255-270, 27-153).
+static void ThresholdsFromSorted(const std::vector<float> &s, int hist_size, std::vector<float> *thr,
+                                 int *size) {
+  const size_t n = s.size();
+  thr->assign(hist_size, std::numeric_limits<float>::infinity());
+  unsigned seg = (unsigned)(n / (size_t)hist_size);
+  if (seg < 1) seg = 1;
+  unsigned k = 0;
+  for (size_t i = 1; i < n; ++i) {
+    if (s[i] != s[i - 1]) {
+      ++k;
+      const float mid = (float)((double)(float)(s[i] + s[i - 1]) * 0.5);
+      const long long slot = (long long)std::min<unsigned long long>(k + 1ull, i / seg + 1ull) - 2;
+      if (slot >= 0 && slot < hist_size && mid < (*thr)[slot]) (*thr)[slot] = mid;
+    }
+  }
+  int unique = 0;
+  while (unique < hist_size && !std::isinf((*thr)[unique])) ++unique;
+  ++unique;
+  *size = std::min(unique, hist_size);
+}
+
+void QuantiseOnDevice(DataMatrix *data, int hist_size, bool verbose) {
+  if (data->quantised) {
+    if (data->hist_size != hist_size) throw std::runtime_error("data matrix was quantised with another hist_size");
+    return;
+  }
+  if (hist_size < 1) throw std::runtime_error("hist_size must be positive");
+  const size_t n = data->rows;
+  const int F = (int)data->columns_dense;
+  if (n == 0 || F == 0) throw std::runtime_error("empty data matrix");
+  if (n >= 0xffffffffull) throw std::runtime_error("too many rows");
+  std::unique_ptr<DeviceMatrix, void (*)(DeviceMatrix *)> dm(new DeviceMatrix(), FreeDeviceMatrix);
+  dm->rows = n;
+  dm->F = F;
+  dm->Q = (F + 3) / 4;
+  dm->stride = (n + 63) / 64 * 64;
+  dm->bins = DevAlloc<uint32_t>((size_t)dm->Q * dm->stride);
+  data->thresholds.assign(F, {});
+  data->reduced_size.assign(F, 0);
+
+  if (data->is_prebinned) {
+    for (int f = 0; f < F; ++f) {
+      data->thresholds[f].resize(hist_size);
+      for (int k = 0; k < hist_size; ++k) data->thresholds[f][k] = (float)k + 0.5f;
+      data->reduced_size[f] = std::min(hist_size, kSlots);
+    }
+    uint8_t *d_in = DevAlloc<uint8_t>(n * F);
+    HIP_OK(hipMemcpy(d_in, data->prebinned.data(), n * F, hipMemcpyHostToDevice));
+    hipLaunchKernelGGL(k_pack_prebinned, dim3(GridFor(n, 256)), dim3(256), 0, 0, d_in, F, dm->Q,
+                       dm->bins, dm->stride, n);
+    HIP_OK(hipDeviceSynchronize());
+    HIP_OK(hipFree(d_in));
+  } else {
+    // thresholds: host sort per column (NaN last), columns in parallel
+    std::vector<char> has_nan(F, 0);
+    {
+      std::vector<std::thread> th;
+      unsigned hw = std::thread::hardware_concurrency();
+      const int nt = std::max(1, std::min<int>(hw ? hw : 1, std::min(F, 16)));
+      std::atomic<int> next{0};
+      for (int t = 0; t < nt; ++t)
+        th.emplace_back([&] {
+          std::vector<float> s;
+          for (;;) {
+            const int f = next.fetch_add(1);
+            if (f >= F) break;
+            s = data->data[f];
+            auto mid = std::partition(s.begin(), s.end(), [](float v) { return v == v; });
+            has_nan[f] = mid != s.end();
+            std::sort(s.begin(), mid);
+            ThresholdsFromSorted(s, hist_size, &data->thresholds[f], &data->reduced_size[f]);
+          }
+        });
+      for (auto &t : th) t.join();
+    }
+    for (int f = 0; f < F; ++f) {
+      if (data->reduced_size[f] + (has_nan[f] ? 1 : 0) > kSlots)
+        throw std::runtime_error("a feature needs more than 256 bin ids: 16-bit bins are not implemented");
+      if (verbose)
+        printf("feature %d has been reduced to %d bits \n", f,
+               32 - __builtin_clz((unsigned)data->reduced_size[f]));
+    }
+    float *d_x = DevAlloc<float>(4 * n);
+    float *d_thr = DevAlloc<float>(4 * (size_t)hist_size);
+    int *d_size = DevAlloc<int>(4);
+    for (int q = 0; q < dm->Q; ++q) {
+      const int nc = std::min(4, F - q * 4);
+      int sizes[4] = {0, 0, 0, 0};
+      for (int c = 0; c < nc; ++c) {
+        const int f = q * 4 + c;
+        HIP_OK(hipMemcpy(d_x + (size_t)c * n, data->data[f].data(), n * sizeof(float), hipMemcpyHostToDevice));
+        HIP_OK(hipMemcpy(d_thr + (size_t)c * hist_size, data->thresholds[f].data(),
+                         hist_size * sizeof(float), hipMemcpyHostToDevice));
+        sizes[c] = data->reduced_size[f];
+      }
+      HIP_OK(hipMemcpy(d_size, sizes, sizeof(sizes), hipMemcpyHostToDevice));
+      hipLaunchKernelGGL(k_bin_assign, dim3(GridFor(n, 256)), dim3(256), 0, 0, d_x, nc, d_thr,
+                         hist_size, d_size, dm->bins + (size_t)q * dm->stride, n);
+      HIP_OK(hipGetLastError());
+      HIP_OK(hipDeviceSynchronize());
+    }
+    HIP_OK(hipFree(d_x));
+    HIP_OK(hipFree(d_thr));
+    HIP_OK(hipFree(d_size));
+  }
+  data->device = dm.release();
+  data->hist_size = hist_size;
+  data->quantised = true;
+}
+
+void GetDeviceBins(const DataMatrix &data, uint8_t *out) {
+  const DeviceMatrix *dm = data.device;
+  if (!dm) throw std::runtime_error("data matrix is not quantised");
+  std::vector<uint32_t> q((size_t)dm->Q * dm->stride);
+  HIP_OK(hipMemcpy(q.data(), dm->bins, q.size() * sizeof(uint32_t), hipMemcpyDeviceToHost));
+  for (size_t r = 0; r < dm->rows; ++r)
+    for (int f = 0; f < dm->F; ++f)
+      out[r * dm->F + f] = (uint8_t)(q[(size_t)(f >> 2) * dm->stride + r] >> (8 * (f & 3)));
+}
+
+// ===================================================================== builder
+namespace {
+
+struct RowBuffers {
+  uint32_t *bins = nullptr;
+  float *g = nullptr, *h = nullptr;
+  unsigned *rowid = nullptr;
+};
+
+class HipTreeBuilder : public TreeBuilder {
+ public:
+  HipTreeBuilder(const Configuration &cfg, DataMatrix *data) : cfg_(cfg), data_(data) {
+    dm_ = data->device;
+    n_ = dm_->rows;
+    F_ = dm_->F;
+    Q_ = dm_->Q;
+    stride_ = dm_->stride;
+    K_ = (int)cfg.tree.labels_count;
+    D_ = (int)cfg.tree.depth;
+    pair_ = cfg.objective != kLinearRegression;
+    f64_ = cfg.internal.double_precision;
+    trick_ = cfg.internal.use_hist_subtraction_trick;
+    nbin_total_ = Q_ * 4 * kSlots;
+    if (cfg.objective >= kSoftMaxOneVsAll && K_ < 2) throw std::runtime_error("soft-max needs labels_count >= 2");
+    if (cfg.objective < kSoftMaxOneVsAll && K_ != 1) throw std::runtime_error("labels_count must be 1 for this objective");
+    const int last_nodes = 1 << (D_ - 2);
+    if (last_nodes > kMaxPlanNodes) throw std::runtime_error("unsupported depth: at most 4096 nodes per level");
+    HIP_OK(hipStreamCreateWithFlags(&stream_, hipStreamNonBlocking));
+
+    // quads per histogram launch, limited by LDS
+    const size_t per_quad = (size_t)4 * kSlots * 8 * (pair_ ? 2 : 1);
+    quads_per_group_ = (int)std::max<size_t>(1, std::min<size_t>((kLdsBudget - 1024) / per_quad, Q_));
+    lds_bytes_ = (size_t)quads_per_group_ * per_quad;
+    if (pair_)
+      HIP_OK(hipFuncSetAttribute((const void *)k_hist<true>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes_));
+    else
+      HIP_OK(hipFuncSetAttribute((const void *)k_hist<false>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes_));
+
+    // per-row state in original order
+    d_y_ = DevAlloc<float>(n_);
+    d_labels_ = DevAlloc<uint8_t>(n_);
+    d_yhat_ = DevAlloc<float>(n_ * K_);
+    d_g_ = DevAlloc<float>(n_ * K_);
+    d_h_ = DevAlloc<float>(n_ * K_);
+    d_leaf_ = DevAlloc<unsigned>(n_);
+    if (!data->y.empty()) HIP_OK(hipMemcpy(d_y_, data->y.data(), n_ * sizeof(float), hipMemcpyHostToDevice));
+    if (!data->labels.empty()) HIP_OK(hipMemcpy(d_labels_, data->labels.data(), n_, hipMemcpyHostToDevice));
+    float init = cfg.tree.initial_y;
+    if (cfg.objective == kLogisticRegression) init = std::log(init / (1 - init));  // objective.h:55-57
+    hipLaunchKernelGGL(k_fill_f32, dim3(GridFor(n_ * K_, 256)), dim3(256), 0, stream_, d_yhat_, init, n_ * K_);
+    data->y_hat.assign(n_ * K_, init);  // garden.cu:104
+
+    // ping-pong row buffers (not needed when the tree has a single split level)
+    if (D_ > 2) {
+      for (int b = 0; b < 2; ++b) {
+        buf_[b].bins = DevAlloc<uint32_t>((size_t)Q_ * stride_);
+        buf_[b].g = DevAlloc<float>(n_);
+        buf_[b].h = DevAlloc<float>(n_);
+        buf_[b].rowid = DevAlloc<unsigned>(n_);
+      }
+    }
+    // level state
+    const int max_nodes = 1 << (D_ - 1);
+    for (int b = 0; b < 2; ++b) {
+      d_tot_[b] = DevAlloc<NodeSum>(max_nodes);
+      d_seg_[b] = DevAlloc<unsigned>(max_nodes);
+      d_hg_[b] = DevAlloc<long long>((size_t)last_nodes * nbin_total_);
+      d_hh_[b] = DevAlloc<long long>((size_t)last_nodes * nbin_total_);
+      d_hc_[b] = DevAlloc<unsigned>((size_t)last_nodes * nbin_total_);
+    }
+    d_split_ = DevAlloc<SplitRec>(last_nodes);
+    d_cand_ = DevAlloc<Cand>((size_t)last_nodes * F_);
+    d_node_first_ = DevAlloc<unsigned>(last_nodes);
+    d_node_items_ = DevAlloc<unsigned>(last_nodes);
+    max_hist_items_ = (unsigned)(n_ / HistRowsPerItem(n_)) + last_nodes + 2;
+    max_part_items_ = (unsigned)(n_ / kPartRows + 1) + last_nodes;
+    d_hwork_ = DevAlloc<WorkItem>(max_hist_items_);
+    d_pwork_ = DevAlloc<WorkItem>(max_part_items_);
+    d_nwork_ = DevAlloc<unsigned>(2);
+    d_item_left_ = DevAlloc<unsigned>(max_part_items_);
+    d_excl_ = DevAlloc<unsigned>(max_part_items_);
+    d_slab_ = DevAlloc<unsigned long long>((size_t)max_hist_items_ * nbin_total_ * (pair_ ? 2 : 1));
+    d_shifts_ = DevAlloc<int>(2);
+    d_gmax_ = DevAlloc<unsigned>(1);
+    d_rows_scanned_ = DevAlloc<unsigned long long>(1);
+    HIP_OK(hipMemsetAsync(d_rows_scanned_, 0, sizeof(unsigned long long), stream_));
+    const int internal = (1 << (D_ - 1)) - 1;
+    d_tfid_ = DevAlloc<int>(internal);
+    d_tbin_ = DevAlloc<int>(internal);
+    d_tgain_ = DevAlloc<float>(internal);
+    d_weights_ = DevAlloc<float>(max_nodes);
+    int shifts[2] = {30, 0};
+    if (cfg.objective == kLogisticRegression) shifts[1] = 32;  // 0 <= h <= 1/4
+    if (cfg.objective >= kSoftMaxOneVsAll) shifts[1] = 31;     // 0 <= h <= 1/2
+    HIP_OK(hipMemcpyAsync(d_shifts_, shifts, sizeof(shifts), hipMemcpyHostToDevice, stream_));
+    HIP_OK(hipStreamSynchronize(stream_));
+  }
+
+  ~HipTreeBuilder() override {
+    (void)hipStreamSynchronize(stream_);
+    void *ptrs[] = {d_y_, d_labels_, d_yhat_, d_g_, d_h_, d_leaf_, d_split_, d_cand_, d_node_first_,
+                    d_node_items_, d_hwork_, d_pwork_, d_nwork_, d_item_left_, d_excl_, d_slab_,
+                    d_shifts_, d_gmax_, d_rows_scanned_, d_tfid_, d_tbin_, d_tgain_, d_weights_};
+    for (void *p : ptrs)
+      if (p) (void)hipFree(p);
+    for (int b = 0; b < 2; ++b) {
+      void *q[] = {buf_[b].bins, buf_[b].g, buf_[b].h, buf_[b].rowid, d_tot_[b], d_seg_[b],
+                   d_hg_[b], d_hh_[b], d_hc_[b]};
+      for (void *p : q)
+        if (p) (void)hipFree(p);
+    }
+    for (hipEvent_t e : event_pool_) (void)hipEventDestroy(e);
+    (void)hipStreamDestroy(stream_);
+  }
+
+  void GrowRound(std::vector<RegTree> *trees) override {
+    Mark(kGrad);
+    if (cfg_.objective == kLinearRegression) {
+      // the maximum is cleared by k_init_root of the previous tree / below
+      hipLaunchKernelGGL(k_init_root, dim3(1), dim3(64), 0, stream_, d_tot_[0], d_seg_[0],
+                         (unsigned long long)n_, d_gmax_);
+      hipLaunchKernelGGL(k_grad_squared, dim3(GridFor(n_, 256)), dim3(256), 0, stream_, d_y_, d_yhat_, d_g_, n_, d_gmax_);
+      hipLaunchKernelGGL(k_set_shift, dim3(1), dim3(64), 0, stream_, d_gmax_, d_shifts_);
+    } else if (cfg_.objective == kLogisticRegression) {
+      hipLaunchKernelGGL(k_grad_logistic, dim3(GridFor(n_, 256)), dim3(256), 0, stream_, d_y_, d_yhat_, d_g_, d_h_, n_);
+    } else {
+      hipLaunchKernelGGL(k_grad_softmax, dim3(GridFor(n_, 256)), dim3(256), 0, stream_, d_labels_, d_yhat_, d_g_, d_h_, n_, K_);
+    }
+    Mark(kNone);
+    for (int k = 0; k < K_; ++k) {
+      RegTree tree((unsigned)D_, (unsigned)k);
+      GrowOne(k, &tree);
+      trees->push_back(std::move(tree));
+    }
+    ResolveTimings();
+  }
+
+  void SetInspect(bool on) override { inspect_ = on; }
+  void GetLeaves(uint32_t *out) override {
+    HIP_OK(hipStreamSynchronize(stream_));
+    HIP_OK(hipMemcpy(out, d_leaf_, n_ * sizeof(unsigned), hipMemcpyDeviceToHost));
+  }
+  void GetYHat(float *out) override {
+    HIP_OK(hipStreamSynchronize(stream_));
+    HIP_OK(hipMemcpy(out, d_yhat_, n_ * K_ * sizeof(float), hipMemcpyDeviceToHost));
+  }
+  void GetGrad(float *g, float *h) override {
+    HIP_OK(hipStreamSynchronize(stream_));
+    HIP_OK(hipMemcpy(g, d_g_, n_ * K_ * sizeof(float), hipMemcpyDeviceToHost));
+    if (h) {
+      if (pair_)
+        HIP_OK(hipMemcpy(h, d_h_, n_ * K_ * sizeof(float), hipMemcpyDeviceToHost));
+      else
+        for (size_t i = 0; i < n_ * K_; ++i) h[i] = 1.0f;
+    }
+  }
+  int GetLevelHist(int level, int64_t *out) override {
+    if (level < 0 || level >= (int)kept_hist_.size()) return -1;
+    const std::vector<int64_t> &v = kept_hist_[level];
+    std::memcpy(out, v.data(), v.size() * sizeof(int64_t));
+    return (int)(v.size() / 3);
+  }
+  void GetShifts(int *sg, int *sh) override {
+    int s[2];
+    HIP_OK(hipStreamSynchronize(stream_));
+    HIP_OK(hipMemcpy(s, d_shifts_, sizeof(s), hipMemcpyDeviceToHost));
+    *sg = s[0];
+    *sh = s[1];
+  }
+  void EnableTiming(bool on) override { timing_ = on; }
+  BuilderTimings GetTimings() override { return timings_; }
+  unsigned long long RowsScanned() override {
+    unsigned long long v = 0;
+    HIP_OK(hipStreamSynchronize(stream_));
+    HIP_OK(hipMemcpy(&v, d_rows_scanned_, sizeof(v), hipMemcpyDeviceToHost));
+    return v;
+  }
+  void Synchronize() override { HIP_OK(hipStreamSynchronize(stream_)); }
+
+ private:
+  enum Phase { kNone = -1, kGrad = 0, kHistRoot, kHistDeep, kReduce, kSplit, kPartition, kLeaf, kPlan, kPhases };
+
+  // Timing: an event is recorded at every phase change; the time between two
+  // consecutive events is charged to the phase that was open.
+  void Mark(int phase) {
+    if (!timing_) return;
+    hipEvent_t e;
+    if (event_used_ < event_pool_.size()) {
+      e = event_pool_[event_used_];
+    } else {
+      HIP_OK(hipEventCreate(&e));
+      event_pool_.push_back(e);
+    }
+    ++event_used_;
+    HIP_OK(hipEventRecord(e, stream_));
+    marks_.push_back(phase);
+  }
+  void ResolveTimings() {
+    if (!timing_ || marks_.empty()) {
+      marks_.clear();
+      event_used_ = 0;
+      return;
+    }
+    HIP_OK(hipStreamSynchronize(stream_));
+    double *slots[kPhases] = {&timings_.grad, &timings_.hist_root, &timings_.hist_deep, &timings_.reduce,
+                              &timings_.split, &timings_.partition, &timings_.leaf, &timings_.plan};
+    for (size_t i = 0; i + 1 < marks_.size(); ++i) {
+      if (marks_[i] < 0) continue;
+      float ms = 0;
+      HIP_OK(hipEventElapsedTime(&ms, event_pool_[i], event_pool_[i + 1]));
+      *slots[marks_[i]] += ms;
+    }
+    marks_.clear();
+    event_used_ = 0;
+  }
+
+  unsigned HistRowsPerItem(size_t rows_max) const {
+    // about 512 work items per level, whole tiles, at most kMaxHistRows rows
+    size_t t = (rows_max + 511) / 512;
+    t = (t + kHistThreads - 1) / kHistThreads * kHistThreads;
+    return (unsigned)std::min<size_t>(std::max<size_t>(t, kHistThreads), kMaxHistRows);
+  }
+
+  template <bool PAIR>
+  void LaunchHist(const RowBuffers &cur, unsigned grid) {
+    for (int q0 = 0; q0 < Q_; q0 += quads_per_group_) {
+      const int nq = std::min(quads_per_group_, Q_ - q0);
+      const size_t lds = (size_t)nq * 4 * kSlots * 8 * (PAIR ? 2 : 1);
+      hipLaunchKernelGGL(k_hist<PAIR>, dim3(grid), dim3(kHistThreads), lds, stream_, cur.bins, stride_,
+                         q0, nq, F_, cur.g, cur.h, d_shifts_, d_hwork_, d_nwork_, d_slab_, nbin_total_);
+    }
+  }
+
+  void GrowOne(int label, RegTree *tree) {
+    const GainParams gp = cfg_.gain_params();
+    RowBuffers orig;
+    orig.bins = dm_->bins;
+    orig.g = d_g_ + (size_t)label * n_;
+    orig.h = d_h_ + (size_t)label * n_;
+    orig.rowid = nullptr;
+    if (inspect_) kept_hist_.assign(D_ - 1, {});
+
+    Mark(kGrad);
+    if (cfg_.objective != kLinearRegression || label > 0)
+      hipLaunchKernelGGL(k_init_root, dim3(1), dim3(64), 0, stream_, d_tot_[0], d_seg_[0],
+                         (unsigned long long)n_, (unsigned *)nullptr);
+    if (pair_)
+      hipLaunchKernelGGL(k_root_total<true>, dim3(GridFor(n_, 256, 1024)), dim3(256), 0, stream_, orig.g, orig.h, d_shifts_, n_, d_tot_[0]);
+    else
+      hipLaunchKernelGGL(k_root_total<false>, dim3(GridFor(n_, 256, 1024)), dim3(256), 0, stream_, orig.g, orig.h, d_shifts_, n_, d_tot_[0]);
+
+    int cur_state = 0;  // index into d_tot_/d_seg_
+    for (int level = 0; level + 1 < D_; ++level) {
+      const int L = 1 << level;
+      const RowBuffers &cur = level == 0 ? orig : buf_[(level - 1) & 1];
+      const bool trick = trick_ && level > 0;
+      const int hb = level & 1;  // histogram buffer of this level; parent is hb ^ 1
+      // ---- histogram of the level
+      const size_t rows_max = trick ? n_ / 2 : n_;
+      const unsigned per_item = HistRowsPerItem(rows_max);
+      const unsigned grid_bound = (unsigned)std::min<size_t>(rows_max / per_item + L + 1, max_hist_items_);
+      Mark(kPlan);
+      hipLaunchKernelGGL(k_plan, dim3(1), dim3(1024), 0, stream_, d_tot_[cur_state], d_seg_[cur_state], L,
+                         trick ? 1 : 0, per_item, d_hwork_, d_nwork_, d_node_first_, d_node_items_,
+                         d_rows_scanned_, grid_bound);
+      Mark(level == 0 ? kHistRoot : kHistDeep);
+      if (timing_) {
+        if (level == 0) {
+          timings_.hist_root_launches += (Q_ + quads_per_group_ - 1) / quads_per_group_;
+          timings_.hist_root_rows += n_;
+        } else {
+          timings_.hist_deep_launches += (Q_ + quads_per_group_ - 1) / quads_per_group_;
+        }
+      }
+      if (pair_)
+        LaunchHist<true>(cur, grid_bound);
+      else
+        LaunchHist<false>(cur, grid_bound);
+      Mark(kReduce);
+      {
+        dim3 grid(nbin_total_ / 64, L);
+        if (pair_)
+          hipLaunchKernelGGL(k_hist_reduce<true>, grid, dim3(1024), 0, stream_, d_slab_, nbin_total_, d_node_first_,
+                             d_node_items_, d_hg_[hb], d_hh_[hb], d_hc_[hb], d_hg_[hb ^ 1], d_hh_[hb ^ 1], d_hc_[hb ^ 1], trick ? 1 : 0);
+        else
+          hipLaunchKernelGGL(k_hist_reduce<false>, grid, dim3(1024), 0, stream_, d_slab_, nbin_total_, d_node_first_,
+                             d_node_items_, d_hg_[hb], d_hh_[hb], d_hc_[hb], d_hg_[hb ^ 1], d_hh_[hb ^ 1], d_hc_[hb ^ 1], trick ? 1 : 0);
+      }
+      if (inspect_) KeepHist(level, L, hb);
+      // ---- split scan and selection
+      Mark(kSplit);
+      {
+        dim3 grid(F_, L);
+        const int hs = std::min(cfg_.internal.hist_size, kSlots);
+#define ARB_SCAN(P, D) \
+  hipLaunchKernelGGL((k_split_scan<P, D>), grid, dim3(64), 0, stream_, d_hg_[hb], d_hh_[hb], d_hc_[hb], \
+                     nbin_total_, F_, d_tot_[cur_state], d_shifts_, gp, hs, d_cand_)
+        if (pair_ && f64_) ARB_SCAN(true, true);
+        else if (pair_) ARB_SCAN(true, false);
+        else if (f64_) ARB_SCAN(false, true);
+        else ARB_SCAN(false, false);
+#undef ARB_SCAN
+        hipLaunchKernelGGL(k_split_select, dim3((L + 127) / 128), dim3(128), 0, stream_, d_cand_, F_, L,
+                           d_tot_[cur_state], d_seg_[cur_state], d_tot_[cur_state ^ 1], d_seg_[cur_state ^ 1],
+                           d_split_, d_tfid_, d_tbin_, d_tgain_, L - 1);
+      }
+      // ---- move rows to the children order, or assign leaves at the last level
+      const unsigned pgrid = (unsigned)std::min<size_t>(n_ / kPartRows + L + 1, max_part_items_);
+      Mark(kPlan);
+      hipLaunchKernelGGL(k_plan, dim3(1), dim3(1024), 0, stream_, d_tot_[cur_state], d_seg_[cur_state], L, 0,
+                         kPartRows, d_pwork_, d_nwork_ + 1, d_node_first_, d_node_items_,
+                         (unsigned long long *)nullptr, pgrid);
+      Mark(level + 2 < D_ ? kPartition : kLeaf);
+      if (level + 2 < D_) {
+        const RowBuffers &nxt = buf_[level & 1];
+        hipLaunchKernelGGL(k_part_count, dim3(pgrid), dim3(kPartThreads), 0, stream_, cur.bins, stride_, d_split_,
+                           d_pwork_, d_nwork_ + 1, d_item_left_);
+        hipLaunchKernelGGL(k_part_scan, dim3(1), dim3(1024), 0, stream_, d_item_left_, d_nwork_ + 1, d_excl_);
+        if (pair_)
+          hipLaunchKernelGGL(k_partition<true>, dim3(pgrid), dim3(kPartThreads), 0, stream_, cur.bins, nxt.bins,
+                             stride_, Q_, cur.g, nxt.g, cur.h, nxt.h, cur.rowid, nxt.rowid, d_split_,
+                             d_seg_[cur_state], d_pwork_, d_nwork_ + 1, d_excl_);
+        else
+          hipLaunchKernelGGL(k_partition<false>, dim3(pgrid), dim3(kPartThreads), 0, stream_, cur.bins, nxt.bins,
+                             stride_, Q_, cur.g, nxt.g, cur.h, nxt.h, cur.rowid, nxt.rowid, d_split_,
+                             d_seg_[cur_state], d_pwork_, d_nwork_ + 1, d_excl_);
+      } else {
+        const int blocks = (L + 127) / 128;
+#define ARB_LEAF(P, D) \
+  hipLaunchKernelGGL((k_leaf_weights<P, D>), dim3(blocks), dim3(128), 0, stream_, d_split_, d_tot_[cur_state], L, \
+                     d_shifts_, gp, cfg_.tree.eta, d_weights_)
+        if (pair_ && f64_) ARB_LEAF(true, true);
+        else if (pair_) ARB_LEAF(true, false);
+        else if (f64_) ARB_LEAF(false, true);
+        else ARB_LEAF(false, false);
+#undef ARB_LEAF
+        hipLaunchKernelGGL(k_leaf_assign, dim3(pgrid), dim3(kPartThreads), 0, stream_, cur.bins, stride_, cur.rowid,
+                           d_split_, d_pwork_, d_nwork_ + 1, d_leaf_);
+        hipLaunchKernelGGL(k_update_yhat, dim3(GridFor(n_, 256)), dim3(256), 0, stream_,
+                           d_yhat_ + (size_t)label * n_, d_leaf_, d_weights_, n_);
+      }
+      cur_state ^= 1;
+    }
+    Mark(kNone);
+    HIP_OK(hipGetLastError());
+    // ---- tree record to the host (garden.cu:447-503)
+    const int internal = (1 << (D_ - 1)) - 1;
+    std::vector<int> fid(internal), bin(internal);
+    HIP_OK(hipMemcpyAsync(fid.data(), d_tfid_, internal * sizeof(int), hipMemcpyDeviceToHost, stream_));
+    HIP_OK(hipMemcpyAsync(bin.data(), d_tbin_, internal * sizeof(int), hipMemcpyDeviceToHost, stream_));
+    HIP_OK(hipMemcpyAsync(tree->gain.data(), d_tgain_, internal * sizeof(float), hipMemcpyDeviceToHost, stream_));
+    HIP_OK(hipMemcpyAsync(tree->weights.data(), d_weights_, tree->weights.size() * sizeof(float),
+                          hipMemcpyDeviceToHost, stream_));
+    HIP_OK(hipStreamSynchronize(stream_));
+    for (int i = 0; i < internal; ++i) {
+      tree->fid[i] = (unsigned)fid[i];
+      tree->quantized[i] = bin[i];
+      float thr = std::numeric_limits<float>::infinity();
+      if (bin[i] >= 0 && bin[i] < (int)data_->thresholds[fid[i]].size()) thr = data_->thresholds[fid[i]][bin[i]];
+      tree->threshold[i] = thr;
+    }
+  }
+
+  void KeepHist(int level, int L, int hb) {
+    const size_t cells = (size_t)L * nbin_total_;
+    std::vector<long long> g(cells), h(cells);
+    std::vector<unsigned> c(cells);
+    HIP_OK(hipStreamSynchronize(stream_));
+    HIP_OK(hipMemcpy(g.data(), d_hg_[hb], cells * sizeof(long long), hipMemcpyDeviceToHost));
+    HIP_OK(hipMemcpy(h.data(), d_hh_[hb], cells * sizeof(long long), hipMemcpyDeviceToHost));
+    HIP_OK(hipMemcpy(c.data(), d_hc_[hb], cells * sizeof(unsigned), hipMemcpyDeviceToHost));
+    // keep [node][F][256][3] (padding features of the last quad dropped)
+    std::vector<int64_t> &out = kept_hist_[level];
+    out.resize((size_t)L * F_ * kSlots * 3);
+    for (int nd = 0; nd < L; ++nd)
+      for (int f = 0; f < F_; ++f)
+        for (int b = 0; b < kSlots; ++b) {
+          const size_t s = (size_t)nd * nbin_total_ + (size_t)f * kSlots + b;
+          const size_t d = (((size_t)nd * F_ + f) * kSlots + b) * 3;
+          out[d] = g[s];
+          out[d + 1] = pair_ ? h[s] : 0;
+          out[d + 2] = c[s];
+        }
+  }
+
+  const Configuration cfg_;
+  DataMatrix *data_;
+  DeviceMatrix *dm_;
+  size_t n_ = 0, stride_ = 0;
+  int F_ = 0, Q_ = 0, K_ = 1, D_ = 2, nbin_total_ = 0;
+  bool pair_ = false, f64_ = false, trick_ = true, inspect_ = false, timing_ = false;
+  int quads_per_group_ = 1;
+  size_t lds_bytes_ = 0;
+  hipStream_t stream_ = nullptr;
+  float *d_y_ = nullptr, *d_yhat_ = nullptr, *d_g_ = nullptr, *d_h_ = nullptr, *d_weights_ = nullptr, *d_tgain_ = nullptr;
+  uint8_t *d_labels_ = nullptr;
+  unsigned *d_leaf_ = nullptr, *d_node_first_ = nullptr, *d_node_items_ = nullptr, *d_nwork_ = nullptr,
+           *d_item_left_ = nullptr, *d_excl_ = nullptr, *d_gmax_ = nullptr;
+  RowBuffers buf_[2];
+  NodeSum *d_tot_[2] = {nullptr, nullptr};
+  unsigned *d_seg_[2] = {nullptr, nullptr};
+  long long *d_hg_[2] = {nullptr, nullptr}, *d_hh_[2] = {nullptr, nullptr};
+  unsigned *d_hc_[2] = {nullptr, nullptr};
+  SplitRec *d_split_ = nullptr;
+  Cand *d_cand_ = nullptr;
+  WorkItem *d_hwork_ = nullptr, *d_pwork_ = nullptr;
+  unsigned max_hist_items_ = 0, max_part_items_ = 0;
+  unsigned long long *d_slab_ = nullptr, *d_rows_scanned_ = nullptr;
+  int *d_shifts_ = nullptr, *d_tfid_ = nullptr, *d_tbin_ = nullptr;
+  std::vector<std::vector<int64_t>> kept_hist_;
+  std::vector<hipEvent_t> event_pool_;
+  size_t event_used_ = 0;
+  std::vector<int> marks_;
+  BuilderTimings timings_;
+};
+
+}  // namespace
+
+TreeBuilder *CreateTreeBuilder(const Configuration &cfg, DataMatrix *data) {
+  if (!data->device) throw std::runtime_error("data matrix is not quantised");
+  return new HipTreeBuilder(cfg, data);
+}
+
+}  // namespace arb

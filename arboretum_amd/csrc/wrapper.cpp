@@ -1,0 +1,284 @@
+// extern "C" boundary: marshalling only.  Mirrors
+// python-wrapper/arboretum_wrapper.cu:16-205 (same names, argument meaning and
+// error convention) plus the extensions declared in arboretum_ext.h.
+#include <cstring>
+#include <limits>
+#include <new>
+#include <stdexcept>
+#include <string>
+
+#include "../../include/arboretum_ext.h"
+#include "booster.h"
+
+using namespace arb;
+
+namespace {
+
+thread_local std::string g_error;
+
+const char *Fail(const char *what) {
+  g_error = what ? what : "unknown error";
+  return g_error.c_str();
+}
+
+template <typename Fn>
+const char *Guard(Fn &&fn) {
+  try {
+    fn();
+    return nullptr;
+  } catch (const std::exception &e) {
+    return Fail(e.what());
+  } catch (const char *msg) {
+    return Fail(msg);
+  } catch (...) {
+    return Fail("unknown error");
+  }
+}
+
+struct GardenHandle {
+  explicit GardenHandle(const Configuration &cfg) : garden(cfg) {}
+  Garden garden;
+};
+
+DataMatrix *AsData(VoidPointer p) {
+  if (!p) throw std::runtime_error("null data matrix handle");
+  return static_cast<DataMatrix *>(p);
+}
+GardenHandle *AsGarden(VoidPointer p) {
+  if (!p) throw std::runtime_error("null booster handle");
+  return static_cast<GardenHandle *>(p);
+}
+TreeBuilder *BuilderOf(VoidPointer p) {
+  TreeBuilder *b = AsGarden(p)->garden.builder();
+  if (!b) throw std::runtime_error("no tree has been grown yet");
+  return b;
+}
+
+const char *CopyOut(const std::vector<float> &v, const float **out) {
+  float *p = new (std::nothrow) float[v.size() ? v.size() : 1];
+  if (!p) return Fail("unable to allocate array");
+  if (!v.empty()) std::memcpy(p, v.data(), v.size() * sizeof(float));
+  *out = p;
+  return nullptr;
+}
+
+}  // namespace
+
+extern "C" {
+
+const char *ACreateFromDenseMatrix(const float *data, const unsigned int *categories, int nrow,
+                                   int ncol, int ccol, float /*missing*/, VoidPointer *out) {
+  return Guard([&] {
+    if (!data || !out || nrow < 0 || ncol < 0 || ccol < 0) throw std::runtime_error("bad arguments");
+    DataMatrix *mat = new DataMatrix((size_t)nrow, (size_t)ncol, (size_t)ccol);
+    mat->data.assign(ncol, std::vector<float>((size_t)nrow));
+    const size_t rows = (size_t)nrow, cols = (size_t)ncol;
+    ParallelFor(rows, [&](size_t b, size_t e) {
+      for (size_t i = b; i < e; ++i)
+        for (size_t f = 0; f < cols; ++f) mat->data[f][i] = data[i * cols + f];
+    });
+    if (ccol > 0 && categories) {
+      mat->data_categories.assign(ccol, std::vector<unsigned>(rows));
+      for (size_t i = 0; i < rows; ++i)
+        for (int c = 0; c < ccol; ++c) mat->data_categories[c][i] = categories[i * ccol + c];
+    }
+    *out = mat;
+  });
+}
+
+const char *ASetY(VoidPointer data, const float *y) {
+  return Guard([&] {
+    DataMatrix *d = AsData(data);
+    if (!y) throw std::runtime_error("null y");
+    d->y.assign(y, y + d->rows);
+  });
+}
+
+const char *ASetLabel(VoidPointer data, const unsigned char *labels) {
+  return Guard([&] {
+    DataMatrix *d = AsData(data);
+    if (!labels) throw std::runtime_error("null labels");
+    d->labels.assign(labels, labels + d->rows);
+  });
+}
+
+const char *ASetWeights(VoidPointer data, const float *weights) {
+  return Guard([&] {
+    DataMatrix *d = AsData(data);
+    if (!weights) throw std::runtime_error("null weights");
+    d->weights.assign(weights, weights + d->rows);
+  });
+}
+
+const char *AInitGarden(const char *configuration, VoidPointer *out) {
+  return Guard([&] {
+    if (!configuration || !out) throw std::runtime_error("bad arguments");
+    *out = new GardenHandle(Configuration::Parse(configuration));
+  });
+}
+
+const char *AGrowTree(VoidPointer garden, VoidPointer data, const float *grad) {
+  return Guard([&] {
+    AsGarden(garden)->garden.GrowTree(AsData(data), grad);
+  });
+}
+
+const char *APredict(VoidPointer garden, VoidPointer data, const float **out, const int n_rounds) {
+  const char *err = nullptr;
+  std::vector<float> result;
+  err = Guard([&] {
+    if (!out) throw std::runtime_error("bad arguments");
+    AsGarden(garden)->garden.Predict(AsData(data), &result,
+                                     n_rounds == -1 ? std::numeric_limits<int>::max() : n_rounds);
+  });
+  return err ? err : CopyOut(result, out);
+}
+
+const char *ADumpModel(const char **model, VoidPointer garden) {
+  return Guard([&] {
+    if (!model) throw std::runtime_error("bad arguments");
+    *model = AsGarden(garden)->garden.GetModel();
+  });
+}
+
+const char *ALoadModel(const char *model, VoidPointer garden) {
+  return Guard([&] {
+    if (!model) throw std::runtime_error("bad arguments");
+    AsGarden(garden)->garden.Restore(model);
+  });
+}
+
+const char *AGetY(VoidPointer garden, VoidPointer data, const float **out) {
+  std::vector<float> result;
+  const char *err = Guard([&] {
+    if (!out) throw std::runtime_error("bad arguments");
+    AsGarden(garden)->garden.GetY(AsData(data), &result);
+  });
+  return err ? err : CopyOut(result, out);
+}
+
+const char *AAppendLastTree(VoidPointer garden, VoidPointer data) {
+  return Guard([&] { AsGarden(garden)->garden.UpdateByLastTree(AsData(data)); });
+}
+
+const char *AFreeDMatrix(VoidPointer ptr) {
+  return Guard([&] { delete static_cast<DataMatrix *>(ptr); });
+}
+const char *AFreeGarden(VoidPointer ptr) {
+  return Guard([&] { delete static_cast<GardenHandle *>(ptr); });
+}
+const char *ADeleteArray(float *in) {
+  delete[] in;
+  return nullptr;
+}
+
+// ------------------------------------------------------------- extensions
+const char *ADeviceCount(int *out) {
+  return Guard([&] { *out = DeviceCount(); });
+}
+
+const char *ACreateFromQuantized(const unsigned char *bins, long long nrow, int ncol, VoidPointer *out) {
+  return Guard([&] {
+    if (!bins || !out || nrow <= 0 || ncol <= 0) throw std::runtime_error("bad arguments");
+    DataMatrix *mat = new DataMatrix((size_t)nrow, (size_t)ncol, 0);
+    mat->is_prebinned = true;
+    mat->prebinned.assign(bins, bins + (size_t)nrow * ncol);
+    *out = mat;
+  });
+}
+
+const char *AQuantize(VoidPointer data, int hist_size) {
+  return Guard([&] {
+    if (DeviceCount() <= 0) throw std::runtime_error("no HIP device available: the quantiser needs an MI355X");
+    QuantiseOnDevice(AsData(data), hist_size, false);
+  });
+}
+
+const char *AGetBins(VoidPointer data, unsigned char *out) {
+  return Guard([&] { GetDeviceBins(*AsData(data), out); });
+}
+
+const char *AGetThresholds(VoidPointer data, int fid, float *thr, int *size) {
+  return Guard([&] {
+    DataMatrix *d = AsData(data);
+    if (!d->quantised) throw std::runtime_error("data matrix is not quantised");
+    if (fid < 0 || (size_t)fid >= d->columns_dense) throw std::runtime_error("feature id out of range");
+    if (thr) std::memcpy(thr, d->thresholds[fid].data(), d->thresholds[fid].size() * sizeof(float));
+    if (size) *size = d->reduced_size[fid];
+  });
+}
+
+const char *AGardenSetInspect(VoidPointer garden, int on) {
+  return Guard([&] {
+    AsGarden(garden)->garden.SetInspect(on != 0);
+  });
+}
+
+const char *AGardenNumTrees(VoidPointer garden, int *out) {
+  return Guard([&] { *out = (int)AsGarden(garden)->garden.num_trees(); });
+}
+
+const char *AGardenGetTree(VoidPointer garden, int t, int *fid, int *bin, float *threshold, float *gain,
+                           float *weights) {
+  return Guard([&] {
+    Garden &g = AsGarden(garden)->garden;
+    if (t < 0 || (size_t)t >= g.num_trees()) throw std::runtime_error("tree index out of range");
+    const RegTree &tr = g.tree(t);
+    for (size_t i = 0; i < tr.fid.size(); ++i) {
+      if (fid) fid[i] = (int)tr.fid[i];
+      if (bin) bin[i] = tr.quantized[i];
+      if (threshold) threshold[i] = tr.threshold[i];
+      if (gain) gain[i] = tr.gain[i];
+    }
+    if (weights) std::memcpy(weights, tr.weights.data(), tr.weights.size() * sizeof(float));
+  });
+}
+
+const char *AGardenGetLeaves(VoidPointer garden, unsigned *out) {
+  return Guard([&] { BuilderOf(garden)->GetLeaves(out); });
+}
+const char *AGardenGetTrainYHat(VoidPointer garden, float *out) {
+  return Guard([&] { BuilderOf(garden)->GetYHat(out); });
+}
+const char *AGardenGetGrad(VoidPointer garden, float *g, float *h) {
+  return Guard([&] { BuilderOf(garden)->GetGrad(g, h); });
+}
+const char *AGardenGetLevelHist(VoidPointer garden, int level, long long *out, int *cells) {
+  return Guard([&] {
+    const int n = BuilderOf(garden)->GetLevelHist(level, (int64_t *)out);
+    if (n < 0) throw std::runtime_error("level histogram not kept (inspect off or bad level)");
+    if (cells) *cells = n;
+  });
+}
+const char *AGardenGetShifts(VoidPointer garden, int *shift_g, int *shift_h) {
+  return Guard([&] { BuilderOf(garden)->GetShifts(shift_g, shift_h); });
+}
+const char *AGardenEnableTiming(VoidPointer garden, int on) {
+  return Guard([&] {
+    AsGarden(garden)->garden.SetTiming(on != 0);
+  });
+}
+const char *AGardenGetTimings(VoidPointer garden, double *out) {
+  return Guard([&] {
+    const BuilderTimings t = BuilderOf(garden)->GetTimings();
+    out[0] = t.grad;
+    out[1] = t.hist_root;
+    out[2] = t.hist_deep;
+    out[3] = t.reduce;
+    out[4] = t.split;
+    out[5] = t.partition;
+    out[6] = t.leaf;
+    out[7] = t.plan;
+    out[8] = (double)t.hist_root_launches;
+    out[9] = (double)t.hist_root_rows;
+    out[10] = (double)t.hist_deep_launches;
+  });
+}
+const char *AGardenRowsScanned(VoidPointer garden, unsigned long long *out) {
+  return Guard([&] { *out = BuilderOf(garden)->RowsScanned(); });
+}
+const char *AGardenSynchronize(VoidPointer garden) {
+  return Guard([&] { BuilderOf(garden)->Synchronize(); });
+}
+
+}  // extern "C"

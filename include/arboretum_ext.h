@@ -1,0 +1,72 @@
+/*
+ * Entry points of libarboretum.so that have no counterpart in the reference's
+ * wrapper (python-wrapper/arboretum_wrapper.h).  They exist for three callers:
+ * parity tests (inspection of the device-side state), the benchmark (device
+ * timings and work counters) and data that is already quantised (the
+ * reference's ABI only takes fp32 rows and an `int` row count).
+ * Same convention as arboretum_wrapper.h: NULL on success, else a message.
+ */
+#ifndef ARBORETUM_EXT_H_
+#define ARBORETUM_EXT_H_
+
+#include "arboretum_wrapper.h"
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* Number of HIP devices visible (0 on a CPU-only host). */
+const char *ADeviceCount(int *out);
+
+/* Data matrix from bin ids: `bins` row-major uint8 [nrow][ncol], copied.
+ * Thresholds are reported as bin + 0.5 and prediction walks the bin ids.
+ * Counterpart of the reference's quantised columns (src/io/io.h:65-76), which
+ * it can only produce itself from fp32 input. */
+const char *ACreateFromQuantized(const unsigned char *bins, long long nrow, int ncol,
+                                 VoidPointer *out);
+
+/* Runs the quantiser now (the reference defers it to the first AGrowTree,
+ * src/core/garden.cu:586-589).  Needs a GPU. */
+const char *AQuantize(VoidPointer data, int hist_size);
+
+/* Quantiser output: bins as row-major uint8 [nrow][ncol]; thresholds of one
+ * feature (hist_size floats, +INF where unset) and its number of real bins
+ * (DataMatrix::data_reduced_mapping / reduced_size, src/io/io.h:24,32). */
+const char *AGetBins(VoidPointer data, unsigned char *out);
+const char *AGetThresholds(VoidPointer data, int fid, float *thr, int *size);
+
+/* Inspection of the booster; valid after AGrowTree. */
+const char *AGardenSetInspect(VoidPointer garden, int on);      /* keep per-level histograms */
+const char *AGardenNumTrees(VoidPointer garden, int *out);
+/* Tree t: fid/bin/threshold/gain of the 2^(depth-1)-1 internal nodes in heap
+ * order (bin -1 = not split), 2^(depth-1) leaf weights.  Any pointer may be NULL. */
+const char *AGardenGetTree(VoidPointer garden, int t, int *fid, int *bin, float *threshold,
+                           float *gain, float *weights);
+/* Leaf index of every training row in the last tree, original row order
+ * (the reference's row2Node, src/core/garden.cu:56,67). */
+const char *AGardenGetLeaves(VoidPointer garden, unsigned *out);
+/* Device-side y_hat (internal scale) and gradients, class-major [labels][nrow]. */
+const char *AGardenGetTrainYHat(VoidPointer garden, float *out);
+const char *AGardenGetGrad(VoidPointer garden, float *g, float *h);
+/* Fixed-point histogram of one level of the last tree (needs inspect on):
+ * int64 [nodes][ncol][256][3] = (sum g_q, sum h_q, count); *cells = nodes*ncol*256. */
+const char *AGardenGetLevelHist(VoidPointer garden, int level, long long *out, int *cells);
+/* Binary exponents of the fixed-point scale: value = q * 2^-shift. */
+const char *AGardenGetShifts(VoidPointer garden, int *shift_g, int *shift_h);
+
+/* Device timings (HIP events on the builder's stream), accumulated since the
+ * call that enabled them.  out[0..8] = milliseconds in: gradients, root
+ * histogram kernel, deeper histogram kernels, slab reduce, split scan,
+ * partition, leaf update, planning; out[8] = root histogram launches,
+ * out[9] = rows read by them, out[10] = deeper histogram launches. */
+const char *AGardenEnableTiming(VoidPointer garden, int on);
+const char *AGardenGetTimings(VoidPointer garden, double *out);
+/* Rows accumulated into histograms so far (x ncol = histogram updates). */
+const char *AGardenRowsScanned(VoidPointer garden, unsigned long long *out);
+/* Waits for all device work of the booster. */
+const char *AGardenSynchronize(VoidPointer garden);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* ARBORETUM_EXT_H_ */

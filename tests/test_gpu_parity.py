@@ -1,0 +1,189 @@
+"""Parity of the HIP path (through the C-ABI) against the CPU checker and the
+reference's golden vectors.  Needs an MI355X: run with `-m gpu`."""
+import itertools
+import json
+
+import numpy as np
+import pytest
+
+from conftest import concrete_config, load_golden
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module")
+def arb():
+    import arboretum_amd
+    if arboretum_amd.device_count() < 1:
+        pytest.fail("no HIP device: the GPU tests must run on the GPU box")
+    return arboretum_amd
+
+
+def make_data(n, F, objective, seed, nan_frac=0.0):
+    rng = np.random.default_rng(seed)
+    X = rng.normal(size=(n, F)).astype(np.float32)
+    X[:, F // 2:] = np.round(X[:, F // 2:] * 4) / 4          # repeated values
+    if nan_frac:
+        X[rng.random((n, F)) < nan_frac] = np.nan
+    w = rng.normal(size=F)
+    s = np.nan_to_num(X) @ w / np.sqrt(F)
+    if objective == 0:
+        y = (s + 0.3 * rng.normal(size=n)).astype(np.float32)
+    else:
+        y = (rng.random(n) < 1 / (1 + np.exp(-2 * s))).astype(np.float32)
+    return X, y
+
+
+def assert_same_training(arb, oracle, X, y, cfg, rounds, check_hist=True):
+    """Grows `rounds` trees on both sides and compares every intermediate."""
+    D = cfg["tree"]["max_depth"] + 1
+    ob = oracle.Booster(X, y=y, config=cfg)
+    data = arb.DMatrix(X, y=y)
+    g = arb.Garden(cfg, data)
+    g.set_inspect(check_hist)
+    hs = cfg["internals"]["hist_size"]
+    for r in range(rounds):
+        ob.grow(1)
+        g.grow_tree()
+        if r == 0:
+            assert np.array_equal(data.bins(), ob.bins().astype(np.uint8)), "bins"
+            for f in range(X.shape[1]):
+                t0, s0 = ob.thresholds(f)
+                t1, s1 = data.thresholds(f, hs)
+                assert s0 == s1 and np.array_equal(t0, t1), "thresholds"
+        og, oh = ob.grad()
+        gg, gh = g.grad()
+        assert np.array_equal(og, gg), "grad round %d" % r
+        if cfg["objective"] != 0:
+            assert np.array_equal(oh, gh), "hess round %d" % r
+        assert g.shifts() == ob.shifts()
+        if check_hist:
+            for level in range(D - 1):
+                ho = ob.level_hist(level)[:, :, :hs + 1, :]
+                hg = g.level_hist(level)
+                if hs + 1 <= 256:
+                    assert np.array_equal(hg[:, :, :hs + 1, :], ho), "hist level %d round %d" % (level, r)
+                    assert not hg[:, :, hs + 1:, :].any()
+                else:
+                    assert np.array_equal(hg, ho[:, :, :256, :])
+        to, tg = ob.tree(r), g.tree(r)
+        assert np.array_equal(to["fid"], tg["fid"]), "fid round %d" % r
+        assert np.array_equal(to["quantized"], tg["quantized"]), "bin round %d" % r
+        assert np.array_equal(to["threshold"], tg["threshold"]), "threshold round %d" % r
+        assert np.array_equal(to["gain"], tg["gain"]), "gain round %d" % r
+        assert np.array_equal(to["weights"], tg["weights"]), "weights round %d" % r
+        assert np.array_equal(ob.leaf(), g.leaves()), "row->leaf round %d" % r
+        assert np.array_equal(ob.yhat(), g.train_yhat()), "y_hat round %d" % r
+    po, pg = ob.predict(X), g.predict(data)
+    assert np.allclose(po, pg, rtol=0, atol=1e-6), "predictions"
+    return ob, g
+
+
+@pytest.mark.parametrize("objective", [0, 1])
+@pytest.mark.parametrize("dp", [True, False])
+@pytest.mark.parametrize("trick", [True, False])
+def test_training_matches_oracle(arb, oracle, objective, dp, trick):
+    X, y = make_data(20000, 11, objective, seed=3, nan_frac=0.02)
+    cfg = {"objective": objective, "method": 1,
+           "internals": {"hist_size": 63, "double_precision": dp, "use_hist_subtraction_trick": trick},
+           "tree": {"max_depth": 5, "eta": 0.3, "lambda": 1.0, "min_child_weight": 1.0}}
+    assert_same_training(arb, oracle, X, y, cfg, rounds=3)
+
+
+def test_training_255_bins_28_features(arb, oracle):
+    X, y = make_data(60000, 28, 1, seed=11)
+    cfg = {"objective": 1, "method": 1,
+           "internals": {"hist_size": 255, "double_precision": True},
+           "tree": {"max_depth": 8, "eta": 0.1, "lambda": 1.0, "min_child_weight": 1.0}}
+    assert_same_training(arb, oracle, X, y, cfg, rounds=2)
+
+
+def test_training_many_features_uses_feature_groups(arb, oracle):
+    # 50 features do not fit one workgroup's LDS in the (g,h) form: two launches
+    X, y = make_data(9000, 50, 1, seed=5)
+    cfg = {"objective": 1, "method": 1, "internals": {"hist_size": 31, "double_precision": False},
+           "tree": {"max_depth": 4, "eta": 0.5, "lambda": 0.5}}
+    assert_same_training(arb, oracle, X, y, cfg, rounds=2)
+
+
+@pytest.mark.parametrize("n", [1, 2, 63, 64, 65, 1023, 1025, 4097])
+def test_ragged_row_counts(arb, oracle, n):
+    X, y = make_data(n, 5, 0, seed=n)
+    cfg = {"objective": 0, "method": 1, "internals": {"hist_size": 16, "double_precision": True},
+           "tree": {"max_depth": 3, "eta": 1.0, "lambda": 0.0, "min_child_weight": 0, "min_leaf_size": 0}}
+    assert_same_training(arb, oracle, X, y, cfg, rounds=2)
+
+
+def test_regularisation_and_guards(arb, oracle):
+    X, y = make_data(5000, 6, 1, seed=8)
+    cfg = {"objective": 1, "method": 1, "internals": {"hist_size": 40, "double_precision": False},
+           "tree": {"max_depth": 6, "eta": 0.2, "lambda": 2.0, "alpha": 0.5, "min_child_weight": 20.0,
+                    "min_leaf_size": 50, "gamma_absolute": 0.5, "gamma_relative": 0.001,
+                    "max_leaf_weight": 0.3}}
+    assert_same_training(arb, oracle, X, y, cfg, rounds=3)
+
+
+def test_max_depth_1(arb, oracle):
+    X, y = make_data(3000, 4, 0, seed=2)
+    cfg = {"objective": 0, "method": 1, "internals": {"hist_size": 255},
+           "tree": {"max_depth": 1, "eta": 0.5, "lambda": 1.0}}
+    assert_same_training(arb, oracle, X, y, cfg, rounds=2)
+
+
+def test_constant_features_give_unsplit_nodes(arb, oracle):
+    X = np.ones((500, 3), np.float32)
+    y = np.arange(500, dtype=np.float32)
+    cfg = {"objective": 0, "method": 1, "internals": {"hist_size": 8},
+           "tree": {"max_depth": 3, "eta": 0.5, "lambda": 1.0}}
+    ob, g = assert_same_training(arb, oracle, X, y, cfg, rounds=1)
+    assert (g.tree(0)["quantized"] == -1).all()
+    model = json.loads(g.dump())
+    assert all(n["threshold"] is None for n in model["model"][0]["nodes"] if not n["leaf"])
+
+
+# ------------------------------------------------------ reference goldens
+def _golden_cases(arb, fixture, X, y):
+    for name, case in fixture["cases"].items():
+        for dp, trick, upload in itertools.product([True, False], repeat=3):
+            cfg = concrete_config(fixture["config"], double_precision=dp, use_hist_trick=trick,
+                                  upload_features=upload, depth=case["max_depth"])
+            data = arb.DMatrix(X, y=y)
+            model = arb.train(cfg, data, case["trees"])
+            for i in range(case["trees"]):
+                pred = model.predict(data, i + 1)
+                assert np.allclose(pred, case["true_values"][i]), (name, dp, trick, upload, i)
+            dumped = model.dump()
+            created = json.loads(dumped)
+            true = case["true_model"]
+            assert len(true["model"]) == len(created["model"])
+            for tt, ct in zip(true["model"], created["model"]):
+                assert np.allclose(tt["weights"], ct["weights"], rtol=1e-4, atol=1e-6), name
+                assert tt["nodes"] == ct["nodes"], (name, dp, trick, upload)
+            loaded = arb.load(dumped)
+            for i in range(case["trees"]):
+                assert np.allclose(loaded.predict(data, i + 1), case["true_values"][i])
+
+
+def test_golden_hist_regression(arb):
+    fx = load_golden("hist_regression_boston10.json")
+    _golden_cases(arb, fx, np.array(fx["X"], np.float32), np.array(fx["y"], np.float32))
+
+
+def test_golden_hist_logistic(arb):
+    fx = load_golden("hist_logistic_iris.json")
+    _golden_cases(arb, fx, np.array(fx["X"], np.float32),
+                  (np.array(fx["target"]) != 2).astype(np.float32))
+
+
+@pytest.mark.parametrize("hist_size", [12, 15, 16, 31, 32, 63, 64, 127, 128, 255, 256, 511, 512, 1023])
+def test_sklearn_regressor_golden(arb, hist_size):
+    # tests/py/test_sklearn_regressor.py:9-40 of the reference (hist method)
+    fx = load_golden("hist_regression_boston10.json")
+    X, y = np.array(fx["X"], np.float32), np.array(fx["y"], np.float32)
+    want = fx["cases"]["test_single_tree_depth_1"]["true_values"][0]
+    for dp in (True, False):
+        m = arb.ArboretumRegression(max_depth=1, learning_rate=0.99999, n_estimators=1, verbosity=0,
+                                    min_child_weight=1.0, min_leaf_size=1, colsample_bytree=1.0, l1=0, l2=0,
+                                    double_precision=dp, method='hist', hist_size=hist_size)
+        m.fit(arb.DMatrix(X, y=y), y)
+        assert np.allclose(m.predict(arb.DMatrix(X)), want)
