@@ -1,0 +1,171 @@
+"""Headline benchmark: histogram tree growing at 10.5M rows x 28 features,
+256 bins, max_depth 8, logistic objective, on one MI355X.
+
+A step is one boosting iteration (one tree: gradients, 8 histogram levels,
+split scans, row partitions, leaf update) over the resident, already quantised
+matrix.  Prints ONE JSON line.
+
+  value        row*feature histogram updates per second over the whole step
+               (rows actually accumulated into histograms x 28 / step time)
+  ms_per_step  milliseconds per tree
+  roofline     the histogram kernel (k_hist): algorithmic bytes of all its
+               launches / their summed duration (HIP events on the builder's
+               stream), against 8 TB/s
+  cpu_baseline the CPU checker (oracle/, OpenMP) on a bounded row sample of the
+               same workload, timed on this host
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+import numpy as np
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+HBM_PEAK = 8.0e12  # bytes/s, MI355X
+
+
+def make_workload(rows, features=28, seed=0):
+    """BASELINE config 2: features 0-20 ~ N(0,1), 21-27 log-normal(0,1); label ~
+    Bernoulli(sigmoid(sum of 8 random depth-3 stump products + 0.5 N(0,1) + bias)),
+    bias chosen for about 53 % positives."""
+    rng = np.random.default_rng(seed)
+    X = rng.standard_normal(size=(rows, features), dtype=np.float32)
+    X[:, 21:] = np.exp(X[:, 21:])
+    score = np.zeros(rows, dtype=np.float32)
+    for _ in range(8):
+        prod = np.ones(rows, dtype=bool)
+        for _ in range(3):
+            f = int(rng.integers(0, features))
+            t = float(np.quantile(X[:200000, f], rng.uniform(0.3, 0.7)))
+            prod &= X[:, f] > t
+        score += prod
+    score += 0.5 * rng.standard_normal(size=rows, dtype=np.float32)
+    score -= np.float32(score.mean() - 0.12)
+    y = (rng.random(rows, dtype=np.float32) < 1.0 / (1.0 + np.exp(-score))).astype(np.float32)
+    return X, y
+
+
+def config(max_depth=8, hist_size=256):
+    return {"objective": 1, "method": 1,
+            "internals": {"hist_size": hist_size, "double_precision": True,
+                          "use_hist_subtraction_trick": True, "upload_features": True},
+            "tree": {"max_depth": max_depth, "eta": 0.1, "lambda": 1.0, "min_child_weight": 1.0,
+                     "min_leaf_size": 1, "colsample_bytree": 1.0, "colsample_bylevel": 1.0}}
+
+
+def cpu_baseline(X, y, cfg, sample_rows, trees):
+    """The CPU checker on the first `sample_rows` rows (same columns, same
+    configuration), all host cores."""
+    from oracle import oracle as orc
+    cores = os.cpu_count() or 1
+    try:
+        cores = len(os.sched_getaffinity(0))
+    except AttributeError:
+        pass
+    cores = min(cores, 16)
+    ob = orc.Booster(X[:sample_rows], y=y[:sample_rows], config=cfg, threads=cores)
+    t0 = time.perf_counter()
+    ob.grow(trees)
+    dt = time.perf_counter() - t0
+    return {"value": ob.updates / dt, "unit": "row*feature hist updates/s", "cores": cores, "kind": "port",
+            "sample": "first %d rows x %d features, %d trees, max_depth %d (%.1f s; quantisation not timed)"
+                      % (sample_rows, X.shape[1], trees, cfg["tree"]["max_depth"], dt),
+            "sec_per_tree_scaled_to_full_rows": dt / trees * (X.shape[0] / sample_rows)}
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=40)
+    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--rows", type=int, default=10_500_000)
+    ap.add_argument("--features", type=int, default=28)
+    ap.add_argument("--max-depth", type=int, default=8)
+    ap.add_argument("--hist-size", type=int, default=256)
+    ap.add_argument("--cpu-rows", type=int, default=2_000_000)
+    ap.add_argument("--cpu-trees", type=int, default=2)
+    ap.add_argument("--no-cpu", action="store_true")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        sys.exit("bench.py: this build runs on one GPU only (no collectives, no sharding); use --gpus 1")
+
+    import arboretum_amd as arb
+    if arb.device_count() < 1:
+        sys.exit("bench.py: no HIP device; the benchmark needs an MI355X")
+
+    X, y = make_workload(args.rows, args.features)
+    cfg = config(args.max_depth, args.hist_size)
+    data = arb.DMatrix(X, y=y)
+    t0 = time.perf_counter()
+    data.quantize(args.hist_size)
+    t_quant = time.perf_counter() - t0
+    model = arb.Garden(cfg, data)
+    model.labels_count = 1
+
+    for _ in range(args.warmup):
+        model.grow_tree()
+    model.synchronize()
+    model.enable_timing(True)
+    scanned0 = model.rows_scanned()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        model.grow_tree()
+    model.synchronize()
+    dt = time.perf_counter() - t0
+    scanned = model.rows_scanned() - scanned0
+    tm = model.timings()
+
+    F = args.features
+    updates = scanned * F
+    launches = tm["hist_root_launches"] + tm["hist_deep_launches"]
+    hist_ms = tm["hist_root_ms"] + tm["hist_deep_ms"]
+    # algorithmic bytes of the histogram kernel: every scanned row reads F bin
+    # bytes and one (g,h) pair; every level writes its nodes' histograms once
+    # (16 B per (feature, bin) cell of the nodes built directly).
+    nodes_built = args.steps * (1 + sum(1 << (l - 1) for l in range(1, args.max_depth)))
+    hist_bytes = scanned * (F + 8) + nodes_built * F * 256 * 16
+    achieved = hist_bytes / (hist_ms * 1e-3)
+    root_bytes = tm["hist_root_rows"] * (F + 8) + args.steps * F * 256 * 16
+    root_achieved = root_bytes / (tm["hist_root_ms"] * 1e-3) if tm["hist_root_ms"] > 0 else 0.0
+
+    out = {
+        "metric": "row*feature hist updates/s + sec/tree at 10M x 28 depth 8; % of HBM peak",
+        "value": updates / dt,
+        "unit": "row*feature hist updates/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": dt / args.steps * 1e3,
+        "sec_per_tree": dt / args.steps,
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "int64",
+        "data": "synthetic",
+        "config": {"workload": "binary classification %d rows x %d dense fp32 features (BASELINE configs[1]), "
+                               "%d bins, max_depth %d, logistic, eta 0.1, lambda 1, min_child_weight 1"
+                               % (args.rows, F, args.hist_size, args.max_depth),
+                   "rows": args.rows, "features": F, "bins": args.hist_size, "max_depth": args.max_depth},
+        "roofline": {"bound": "hbm", "achieved": achieved / 1e9, "peak": HBM_PEAK / 1e9, "unit": "GB/s",
+                     "frac": achieved / HBM_PEAK, "traffic": None,
+                     "kernel": "k_hist<true>", "launches": int(launches),
+                     "avg_launch_us": hist_ms * 1e3 / max(launches, 1),
+                     "root_level": {"achieved": root_achieved / 1e9, "frac": root_achieved / HBM_PEAK,
+                                    "avg_launch_us": tm["hist_root_ms"] * 1e3 / max(tm["hist_root_launches"], 1),
+                                    "updates_per_s": tm["hist_root_rows"] * F / (tm["hist_root_ms"] * 1e-3)
+                                    if tm["hist_root_ms"] > 0 else 0.0}},
+        "tree_floor_frac_of_hbm": (2.9e9 / (dt / args.steps)) / HBM_PEAK,
+        "phase_ms_per_tree": {k: v / args.steps for k, v in tm.items() if k.endswith("_ms")},
+        "quantise_s": t_quant,
+    }
+    if not args.no_cpu:
+        out["cpu_baseline"] = cpu_baseline(X, y, cfg, min(args.cpu_rows, args.rows), args.cpu_trees)
+    print(json.dumps(out))
+
+
+if __name__ == "__main__":
+    main()
