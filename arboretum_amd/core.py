@@ -233,7 +233,8 @@ class Garden(object):
         out = np.zeros(16, dtype=np.float64)
         _check(_LIB.AGardenGetTimings(self.handle, out.ctypes.data_as(ctypes.c_void_p)))
         keys = ["grad_ms", "hist_root_ms", "hist_deep_ms", "reduce_ms", "split_ms", "partition_ms", "leaf_ms",
-                "plan_ms", "hist_root_launches", "hist_root_rows", "hist_deep_launches"]
+                "plan_ms", "hist_root_launches", "hist_root_rows", "hist_deep_launches", "fused_last_ms",
+                "fused_last_launches"]
         return dict(zip(keys, out.tolist()))
 
     def rows_scanned(self):

@@ -73,10 +73,16 @@ struct RegTree {
   void Predict(const DataMatrix &data, float *out) const;
 };
 
-struct BuilderTimings {  // accumulated GPU milliseconds per kernel class
-  double grad = 0, hist_root = 0, hist_deep = 0, reduce = 0, split = 0, partition = 0, leaf = 0, plan = 0;
-  unsigned long long hist_root_launches = 0, hist_deep_launches = 0;
-  unsigned long long hist_root_rows = 0, hist_deep_rows = 0;
+// Accumulated GPU milliseconds per kernel class.  hist_root: histogram kernel
+// of the root level; hist_deep: histogram work of the deeper levels (the fused
+// partition + histogram kernel, or the histogram kernel after a stand-alone
+// partition); fused_last: the fused kernel of the last level, which moves no
+// rows; partition: left counts, offset scan and the stand-alone partition.
+struct BuilderTimings {
+  double grad = 0, hist_root = 0, hist_deep = 0, reduce = 0, split = 0, partition = 0, leaf = 0, plan = 0,
+         fused_last = 0;
+  unsigned long long hist_root_launches = 0, hist_deep_launches = 0, fused_last_launches = 0;
+  unsigned long long hist_root_rows = 0;
 };
 
 // GPU tree builder bound to one (configuration, data matrix) pair.

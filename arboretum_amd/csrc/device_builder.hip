@@ -23,7 +23,7 @@
 // What replaces what (reference file:line):
 //   k_bin_assign      build_histogram              src/io/io.cu:293-312
 //   k_grad_*          update_grad                  src/core/objective.cu:15-56
-//   k_root_total      cub::DeviceReduce::Sum       src/core/garden.cu:432-435
+//   k_root_from_hist  cub::DeviceReduce::Sum       src/core/garden.cu:432-435
 //   k_hist            hist_sum_node / hist_sum_multi_node
 //                                                  src/core/hist_grad_sum.cu:109-215,262-406
 //   k_hist_reduce     update_multi_node + global atomics
@@ -63,8 +63,9 @@ namespace {
 
 constexpr int kSlots = 256;               // histogram slots per feature (uint8 bins)
 constexpr int kHistThreads = 1024;        // one workgroup per CU, 16 waves
-constexpr int kPartThreads = 256;
-constexpr unsigned kPartRows = 4096;      // rows per partition work item
+constexpr int kItemWaves = kHistThreads / 64;  // waves per work item in row passes
+constexpr unsigned kPartRows = 16384;     // rows per work item of the stand-alone partition
+constexpr int kMaxGroupQuads = 9;         // quads per histogram launch (compile-time variants)
 constexpr unsigned kMaxHistRows = 64512;  // rows per histogram work item (< 2^16)
 constexpr int kCountShift = 47;           // word0 = count << 47 | g
 constexpr int kMaxPlanNodes = 4096;       // nodes per level the planner handles
@@ -211,27 +212,8 @@ __global__ void k_grad_softmax(const uint8_t *__restrict__ labels, const float *
   }
 }
 
-// Root totals in fixed point.
-template <bool PAIR>
-__global__ void k_root_total(const float *__restrict__ g, const float *__restrict__ h,
-                             const int *__restrict__ shifts, size_t n, NodeSum *__restrict__ tot) {
-  const int sg = shifts[0], sh = shifts[1];
-  long long a = 0, b = 0;
-  for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < n;
-       i += (size_t)gridDim.x * blockDim.x) {
-    a += ToFixed(g[i], sg);
-    if (PAIR) b += ToFixed(h[i], sh);
-  }
-  a = WaveSumLL(a);
-  if (PAIR) b = WaveSumLL(b);
-  if ((threadIdx.x & 63) == 0) {
-    atomicAdd((unsigned long long *)&tot->g, (unsigned long long)a);
-    if (PAIR) atomicAdd((unsigned long long *)&tot->h, (unsigned long long)b);
-  }
-}
-
 __global__ void k_init_root(NodeSum *tot, unsigned *seg_start, unsigned long long n,
-                            unsigned *gmax_bits) {
+                            unsigned *gmax_bits) {  // gmax_bits may be NULL
   if (threadIdx.x == 0 && blockIdx.x == 0) {
     tot[0].g = 0;
     tot[0].h = 0;
@@ -245,12 +227,16 @@ __global__ void k_init_root(NodeSum *tot, unsigned *seg_start, unsigned long lon
 // Splits the row ranges of the selected nodes of a level into work items of
 // at most `rows_per_item` rows.  select: 0 = every node, 1 = the smaller
 // child of each sibling pair, ties -> left (hist_grad_sum.cu:279-294).
+// rows_scanned (optional) is advanced by the rows that will be accumulated
+// into histograms: the selected rows, or, when `split` is given (fused
+// partition + histogram over parent nodes), the smaller side of every split.
 // One workgroup.
 __global__ void __launch_bounds__(1024)
 k_plan(const NodeSum *__restrict__ tot, const unsigned *__restrict__ seg_start, int L, int select,
        unsigned rows_per_item, WorkItem *__restrict__ work, unsigned *__restrict__ n_work,
        unsigned *__restrict__ node_first, unsigned *__restrict__ node_items,
-       unsigned long long *__restrict__ rows_scanned, unsigned max_items) {
+       unsigned long long *__restrict__ rows_scanned, const SplitRec *__restrict__ split,
+       unsigned max_items) {
   __shared__ unsigned s_base[kMaxPlanNodes + 1];
   __shared__ unsigned s_wave[16];
   __shared__ unsigned s_carry;
@@ -273,7 +259,12 @@ k_plan(const NodeSum *__restrict__ tot, const unsigned *__restrict__ seg_start, 
       }
       if (sel && len > 0) {
         cnt = (unsigned)((len + rows_per_item - 1) / rows_per_item);
-        atomicAdd(&s_rows, len);
+        unsigned long long acc = len;
+        if (split) {
+          const unsigned long long cl = split[nd].left.c;
+          acc = min(cl, len - cl);
+        }
+        atomicAdd(&s_rows, acc);
       }
       node_items[nd] = sel ? cnt : 0xffffffffu;  // 0xffffffff marks "not selected"
     }
@@ -305,7 +296,7 @@ k_plan(const NodeSum *__restrict__ tot, const unsigned *__restrict__ seg_start, 
   __syncthreads();
   if (total > max_items) return;
   for (unsigned w = tid; w < total; w += 1024) {
-    int lo = 0, hi = L;  // last node with s_base[node] <= w and items > 0
+    int lo = 0, hi = L;  // last node whose first item is <= w
     while (hi - lo > 1) {
       const int mid = (lo + hi) >> 1;
       if (s_base[mid] <= w)
@@ -325,12 +316,58 @@ k_plan(const NodeSum *__restrict__ tot, const unsigned *__restrict__ seg_start, 
   }
 }
 
+// Row sub-range of one wave inside a work item: kItemWaves equal contiguous
+// pieces, each a multiple of 64 rows.
+__device__ __forceinline__ void WaveRange(const WorkItem &it, int wave, unsigned *b, unsigned *e) {
+  const unsigned rows = it.end - it.begin;
+  const unsigned per = ((rows + kItemWaves - 1) / kItemWaves + 63u) & ~63u;
+  const unsigned wb = min(it.begin + (unsigned)wave * per, it.end);
+  *b = wb;
+  *e = min(wb + per, it.end);
+}
+
 // ---------------------------------------------------------------- histogram
-// One workgroup per work item.  LDS: nq*1024 word0 entries, then (PAIR) as
-// many word1 entries.  Handles quads [q0, q0+nq).
-template <bool PAIR>
+// Adds the four features of quad q (bins packed in b4) of one row.
+template <bool PAIR, int NQ>
+__device__ __forceinline__ void AccumulateRow(unsigned long long *__restrict__ lds,
+                                              const uint32_t (&b)[NQ], float gv, float hv, int sg,
+                                              int sh, int q_first, int F) {
+  constexpr int nbin = NQ * 4 * kSlots;
+  const unsigned long long w0 = (1ull << kCountShift) + (unsigned long long)ToFixed(gv, sg);
+  unsigned long long w1 = 0;
+  if (PAIR) w1 = (unsigned long long)ToFixed(hv, sh);
+#pragma unroll
+  for (int q = 0; q < NQ; ++q) {
+#pragma unroll
+    for (int c = 0; c < 4; ++c) {
+      // only the last quad can hold padding features
+      if (q < NQ - 1 || (q_first + q) * 4 + c < F) {
+        const unsigned idx = (unsigned)(q * 4 + c) * kSlots + ((b[q] >> (8 * c)) & 255u);
+        atomicAdd(&lds[idx], w0);
+        if (PAIR) atomicAdd(&lds[nbin + idx], w1);
+      }
+    }
+  }
+}
+
+template <bool PAIR, int NQ>
+__device__ __forceinline__ void FlushSlab(const unsigned long long *__restrict__ lds,
+                                          unsigned long long *__restrict__ slab, unsigned w,
+                                          int nbin_total, int q_first) {
+  // slab layout per work item: word0[nbin_total], word1[nbin_total]
+  constexpr int nbin = NQ * 4 * kSlots;
+  unsigned long long *out = slab + (size_t)w * nbin_total * (PAIR ? 2 : 1) + (size_t)q_first * 4 * kSlots;
+  for (int i = threadIdx.x; i < nbin; i += kHistThreads) {
+    out[i] = lds[i];
+    if (PAIR) out[nbin_total + i] = lds[nbin + i];
+  }
+}
+
+// Histogram of contiguous row ranges: one workgroup per work item, quads
+// [q0, q0+NQ).  LDS: NQ*1024 word0 entries, then (PAIR) as many word1 entries.
+template <bool PAIR, int NQ>
 __global__ void __launch_bounds__(kHistThreads)
-k_hist(const uint32_t *__restrict__ bins, size_t stride, int q0, int nq, int F,
+k_hist(const uint32_t *__restrict__ bins, size_t stride, int q0, int F,
        const float *__restrict__ g, const float *__restrict__ h, const int *__restrict__ shifts,
        const WorkItem *__restrict__ work, const unsigned *__restrict__ n_work,
        unsigned long long *__restrict__ slab, int nbin_total) {
@@ -338,56 +375,273 @@ k_hist(const uint32_t *__restrict__ bins, size_t stride, int q0, int nq, int F,
   const unsigned w = blockIdx.x;
   if (w >= *n_work) return;
   const WorkItem it = work[w];
-  const int nbin = nq * 4 * kSlots;
-  const int words = PAIR ? 2 * nbin : nbin;
+  constexpr int words = NQ * 4 * kSlots * (PAIR ? 2 : 1);
   for (int i = threadIdx.x; i < words; i += kHistThreads) lds[i] = 0ull;
   __syncthreads();
   const int sg = shifts[0], sh = shifts[1];
-  unsigned long long *lds1 = lds + nbin;
-  for (unsigned r = it.begin + threadIdx.x; r < it.end; r += kHistThreads) {
-    const unsigned long long w0 = (1ull << kCountShift) + (unsigned long long)ToFixed(g[r], sg);
-    unsigned long long w1 = 0;
-    if (PAIR) w1 = (unsigned long long)ToFixed(h[r], sh);
-    for (int q = 0; q < nq; ++q) {
-      const uint32_t b4 = bins[(size_t)(q0 + q) * stride + r];
+  const uint32_t *bq = bins + (size_t)q0 * stride;
+  for (unsigned base = it.begin; base < it.end; base += 2 * kHistThreads) {
+    const unsigned r0 = base + threadIdx.x, r1 = r0 + kHistThreads;
+    const bool v0 = r0 < it.end, v1 = r1 < it.end;
+    const unsigned a0 = v0 ? r0 : it.begin, a1 = v1 ? r1 : it.begin;
+    uint32_t b0[NQ], b1[NQ];
 #pragma unroll
-      for (int c = 0; c < 4; ++c) {
-        if ((q0 + q) * 4 + c < F) {
-          const unsigned idx = (unsigned)(q * 4 + c) * kSlots + ((b4 >> (8 * c)) & 255u);
-          atomicAdd(&lds[idx], w0);
-          if (PAIR) atomicAdd(&lds1[idx], w1);
-        }
-      }
+    for (int q = 0; q < NQ; ++q) {
+      b0[q] = bq[(size_t)q * stride + a0];
+      b1[q] = bq[(size_t)q * stride + a1];
+    }
+    const float g0 = g[a0], g1 = g[a1];
+    const float h0 = PAIR ? h[a0] : 0.0f, h1 = PAIR ? h[a1] : 0.0f;
+    if (v0) AccumulateRow<PAIR, NQ>(lds, b0, g0, h0, sg, sh, q0, F);
+    if (v1) AccumulateRow<PAIR, NQ>(lds, b1, g1, h1, sg, sh, q0, F);
+  }
+  __syncthreads();
+  FlushSlab<PAIR, NQ>(lds, slab, w, nbin_total, q0);
+}
+
+// ---------------------------------------------------------------- partition
+__device__ __forceinline__ bool GoesRight(const uint32_t *__restrict__ bins, size_t stride,
+                                          const SplitRec &s, unsigned r) {
+  // builder.h:107-123: bin >= q + 1 goes right
+  if (s.fid < 0) return false;
+  const uint32_t b4 = bins[(size_t)(s.fid >> 2) * stride + r];
+  return (int)((b4 >> (8 * (s.fid & 3))) & 255u) > s.bin;
+}
+
+// Rows going left, per (work item, wave range).
+__global__ void __launch_bounds__(kHistThreads)
+k_part_count(const uint32_t *__restrict__ bins, size_t stride, const SplitRec *__restrict__ split,
+             const WorkItem *__restrict__ work, const unsigned *__restrict__ n_work,
+             unsigned *__restrict__ wave_left) {
+  const unsigned w = blockIdx.x;
+  if (w >= *n_work) return;
+  const WorkItem it = work[w];
+  const SplitRec s = split[it.node];
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  unsigned wb, we;
+  WaveRange(it, wave, &wb, &we);
+  unsigned cnt = 0;
+  if (s.fid < 0) {
+    cnt = lane == 0 ? we - wb : 0;
+  } else {
+    const uint32_t *col = bins + (size_t)(s.fid >> 2) * stride;
+    const int sh = 8 * (s.fid & 3);
+    for (unsigned r = wb + lane; r < we; r += 64) cnt += ((int)((col[r] >> sh) & 255u) > s.bin) ? 0u : 1u;
+  }
+  for (int off = 32; off > 0; off >>= 1) cnt += __shfl_down(cnt, off);
+  if (lane == 0) wave_left[(size_t)w * kItemWaves + wave] = cnt;
+}
+
+// Exclusive scan of wave_left over all (item, wave) pairs.  One workgroup.
+__global__ void __launch_bounds__(1024)
+k_part_scan(const unsigned *__restrict__ wave_left, const unsigned *__restrict__ n_work,
+            unsigned *__restrict__ excl) {
+  __shared__ unsigned s_part[1024];
+  const unsigned n = *n_work * kItemWaves;
+  const unsigned per = (n + 1023) / 1024;
+  const unsigned b = min(n, threadIdx.x * per), e = min(n, b + per);
+  unsigned sum = 0;
+  for (unsigned i = b; i < e; ++i) sum += wave_left[i];
+  s_part[threadIdx.x] = sum;
+  __syncthreads();
+  // exclusive scan of the 1024 partial sums by the first wave
+  if (threadIdx.x < 64) {
+    const int lane = threadIdx.x;
+    unsigned v[16], t = 0;
+#pragma unroll
+    for (int k = 0; k < 16; ++k) {
+      v[k] = s_part[lane * 16 + k];
+      t += v[k];
+    }
+    unsigned incl = t;
+    for (int off = 1; off < 64; off <<= 1) {
+      const unsigned o = __shfl_up(incl, off);
+      if (lane >= off) incl += o;
+    }
+    unsigned run = incl - t;
+#pragma unroll
+    for (int k = 0; k < 16; ++k) {
+      s_part[lane * 16 + k] = run;
+      run += v[k];
     }
   }
   __syncthreads();
-  // slab layout per work item: word0[nbin_total], word1[nbin_total]
-  unsigned long long *out = slab + (size_t)w * nbin_total * (PAIR ? 2 : 1) + (size_t)q0 * 4 * kSlots;
-  for (int i = threadIdx.x; i < nbin; i += kHistThreads) {
-    out[i] = lds[i];
-    if (PAIR) out[nbin_total + i] = lds1[i];
+  unsigned run = s_part[threadIdx.x];
+  for (unsigned i = b; i < e; ++i) {
+    excl[i] = run;
+    run += wave_left[i];
   }
 }
 
-// Adds the slabs of every selected node; with `trick` also writes the sibling
-// as parent - node.  grid (nbin_total/64, L), 1024 threads = 64 entries x 16
-// slab lanes.
+// Destination offsets of one wave range: rows going left are packed in order
+// from the start of the parent's range, rows going right from the start of
+// the right child's range (stable on both sides).
+__device__ __forceinline__ void WaveOffsets(const WorkItem &it, const SplitRec &s, unsigned start,
+                                            const unsigned *__restrict__ excl, unsigned w, int wave,
+                                            unsigned wb, unsigned *lo, unsigned *ro) {
+  const unsigned lefts_before = excl[(size_t)w * kItemWaves + wave] - excl[(size_t)it.first * kItemWaves];
+  *lo = start + lefts_before;
+  *ro = start + (unsigned)s.left.c + (wb - start) - lefts_before;
+}
+
+// Fused pass over the rows of the parent nodes of a level: stable partition
+// into the children order (WRITE) and histogram of the smaller child of every
+// split in LDS.  Each wave owns a contiguous row range and runs without
+// workgroup barriers.  NQ = all quads of the matrix.
+template <bool PAIR, int NQ, bool WRITE>
+__global__ void __launch_bounds__(kHistThreads)
+k_part_hist(const uint32_t *__restrict__ bins, uint32_t *__restrict__ bins_out, size_t stride, int F,
+            const float *__restrict__ g, float *__restrict__ g_out, const float *__restrict__ h,
+            float *__restrict__ h_out, const int *__restrict__ shifts,
+            const SplitRec *__restrict__ split, const NodeSum *__restrict__ tot,
+            const unsigned *__restrict__ seg_start, const WorkItem *__restrict__ work,
+            const unsigned *__restrict__ n_work, const unsigned *__restrict__ excl,
+            unsigned long long *__restrict__ slab, int nbin_total) {
+  extern __shared__ unsigned long long lds[];
+  const unsigned w = blockIdx.x;
+  if (w >= *n_work) return;
+  const WorkItem it = work[w];
+  const SplitRec s = split[it.node];
+  const unsigned long long cl = s.left.c, cr = tot[it.node].c - cl;
+  const bool build_right = cl > cr;  // ties -> left (hist_grad_sum.cu:288-290)
+  constexpr int words = NQ * 4 * kSlots * (PAIR ? 2 : 1);
+  for (int i = threadIdx.x; i < words; i += kHistThreads) lds[i] = 0ull;
+  __syncthreads();
+  const int sg = shifts[0], sh = shifts[1];
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  unsigned wb, we;
+  WaveRange(it, wave, &wb, &we);
+  unsigned lo = 0, ro = 0;
+  if (WRITE) WaveOffsets(it, s, seg_start[it.node], excl, w, wave, wb, &lo, &ro);
+  const int fq = s.fid >> 2, fs = 8 * (s.fid & 3);
+  const unsigned long long below = (1ull << lane) - 1ull;
+  for (unsigned base = wb; base < we; base += 128) {
+    const unsigned r0 = base + lane, r1 = r0 + 64;
+    const bool v0 = r0 < we, v1 = r1 < we;
+    const unsigned a0 = v0 ? r0 : wb, a1 = v1 ? r1 : wb;
+    uint32_t b0[NQ], b1[NQ];
+#pragma unroll
+    for (int q = 0; q < NQ; ++q) {
+      b0[q] = bins[(size_t)q * stride + a0];
+      b1[q] = bins[(size_t)q * stride + a1];
+    }
+    const float g0 = g[a0], g1 = g[a1];
+    const float h0 = PAIR ? h[a0] : 0.0f, h1 = PAIR ? h[a1] : 0.0f;
+    uint32_t s0 = 0, s1 = 0;
+#pragma unroll
+    for (int q = 0; q < NQ; ++q) {
+      s0 = q == fq ? b0[q] : s0;
+      s1 = q == fq ? b1[q] : s1;
+    }
+    const bool right0 = v0 && s.fid >= 0 && (int)((s0 >> fs) & 255u) > s.bin;
+    const bool right1 = v1 && s.fid >= 0 && (int)((s1 >> fs) & 255u) > s.bin;
+    if (WRITE) {
+      const unsigned long long lm0 = __ballot(v0 && !right0), rm0 = __ballot(right0);
+      const unsigned long long lm1 = __ballot(v1 && !right1), rm1 = __ballot(right1);
+      const unsigned nl0 = (unsigned)__popcll(lm0), nr0 = (unsigned)__popcll(rm0);
+      if (v0) {
+        const unsigned d = right0 ? ro + (unsigned)__popcll(rm0 & below) : lo + (unsigned)__popcll(lm0 & below);
+#pragma unroll
+        for (int q = 0; q < NQ; ++q) bins_out[(size_t)q * stride + d] = b0[q];
+        g_out[d] = g0;
+        if (PAIR) h_out[d] = h0;
+      }
+      if (v1) {
+        const unsigned d = right1 ? ro + nr0 + (unsigned)__popcll(rm1 & below)
+                                  : lo + nl0 + (unsigned)__popcll(lm1 & below);
+#pragma unroll
+        for (int q = 0; q < NQ; ++q) bins_out[(size_t)q * stride + d] = b1[q];
+        g_out[d] = g1;
+        if (PAIR) h_out[d] = h1;
+      }
+      lo += nl0 + (unsigned)__popcll(lm1);
+      ro += nr0 + (unsigned)__popcll(rm1);
+    }
+    if (v0 && right0 == build_right) AccumulateRow<PAIR, NQ>(lds, b0, g0, h0, sg, sh, 0, F);
+    if (v1 && right1 == build_right) AccumulateRow<PAIR, NQ>(lds, b1, g1, h1, sg, sh, 0, F);
+  }
+  __syncthreads();
+  FlushSlab<PAIR, NQ>(lds, slab, w, nbin_total, 0);
+}
+
+// Stable partition alone (matrices too wide for the fused pass): any number
+// of quads, moved eight at a time.
+template <bool PAIR>
+__global__ void __launch_bounds__(kHistThreads)
+k_partition(const uint32_t *__restrict__ bins, uint32_t *__restrict__ bins_out, size_t stride, int Q,
+            const float *__restrict__ g, float *__restrict__ g_out, const float *__restrict__ h,
+            float *__restrict__ h_out, const SplitRec *__restrict__ split,
+            const unsigned *__restrict__ seg_start, const WorkItem *__restrict__ work,
+            const unsigned *__restrict__ n_work, const unsigned *__restrict__ excl) {
+  const unsigned w = blockIdx.x;
+  if (w >= *n_work) return;
+  const WorkItem it = work[w];
+  const SplitRec s = split[it.node];
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  unsigned wb, we;
+  WaveRange(it, wave, &wb, &we);
+  unsigned lo, ro;
+  WaveOffsets(it, s, seg_start[it.node], excl, w, wave, wb, &lo, &ro);
+  const unsigned long long below = (1ull << lane) - 1ull;
+  for (unsigned base = wb; base < we; base += 64) {
+    const unsigned r = base + lane;
+    const bool valid = r < we;
+    const bool right = valid && GoesRight(bins, stride, s, r);
+    const unsigned long long lm = __ballot(valid && !right), rm = __ballot(right);
+    if (valid) {
+      const unsigned d = right ? ro + (unsigned)__popcll(rm & below) : lo + (unsigned)__popcll(lm & below);
+      for (int q0 = 0; q0 < Q; q0 += 8) {
+        uint32_t v[8];
+#pragma unroll
+        for (int k = 0; k < 8; ++k)
+          if (q0 + k < Q) v[k] = bins[(size_t)(q0 + k) * stride + r];
+#pragma unroll
+        for (int k = 0; k < 8; ++k)
+          if (q0 + k < Q) bins_out[(size_t)(q0 + k) * stride + d] = v[k];
+      }
+      g_out[d] = g[r];
+      if (PAIR) h_out[d] = h[r];
+    }
+    lo += (unsigned)__popcll(lm);
+    ro += (unsigned)__popcll(rm);
+  }
+}
+
+// Adds the slabs of every directly built node of a level and, with `trick`,
+// derives its sibling as parent - node.  grid (nbin_total/64, L), 1024
+// threads = 64 entries x 16 slab lanes.
+//   by_parent = 0: slabs belong to work items of the node itself
+//               (node_items == 0xffffffff marks a derived node);
+//   by_parent = 1: slabs belong to work items of the parent (fused pass); the
+//               built child is the smaller one, ties -> left.
 template <bool PAIR>
 __global__ void __launch_bounds__(1024)
 k_hist_reduce(const unsigned long long *__restrict__ slab, int nbin_total,
               const unsigned *__restrict__ node_first, const unsigned *__restrict__ node_items,
-              long long *__restrict__ hg, long long *__restrict__ hh, unsigned *__restrict__ hc,
+              int by_parent, const SplitRec *__restrict__ parent_split,
+              const NodeSum *__restrict__ parent_tot, long long *__restrict__ hg,
+              long long *__restrict__ hh, unsigned *__restrict__ hc,
               const long long *__restrict__ pg, const long long *__restrict__ ph,
               const unsigned *__restrict__ pc, int trick) {
   __shared__ long long s_g[16][64];
   __shared__ long long s_h[16][64];
   __shared__ unsigned s_c[16][64];
   const int nd = blockIdx.y;
-  const unsigned items = node_items[nd];
-  if (items == 0xffffffffu) return;  // derived from its sibling
+  unsigned items, first;
+  if (by_parent) {
+    const int p = nd >> 1;
+    const unsigned long long cl = parent_split[p].left.c, cr = parent_tot[p].c - cl;
+    const bool build_right = cl > cr;
+    if (((nd & 1) != 0) != build_right) return;  // derived from its sibling
+    items = node_items[p];
+    first = node_first[p];
+  } else {
+    items = node_items[nd];
+    first = node_first[nd];
+    if (items == 0xffffffffu) return;  // derived from its sibling
+  }
   const int e = threadIdx.x & 63, lane = threadIdx.x >> 6;
   const int entry = blockIdx.x * 64 + e;
-  const unsigned first = node_first[nd];
   long long ag = 0, ah = 0;
   unsigned ac = 0;
   for (unsigned s = lane; s < items; s += 16) {
@@ -419,6 +673,25 @@ k_hist_reduce(const unsigned long long *__restrict__ slab, int nbin_total,
       hh[so] = ph[po] - ah;
       hc[so] = pc[po] - ac;
     }
+  }
+}
+
+// Root totals = sum over the slots of feature 0 of the root histogram (every
+// row, NaN included, sits in exactly one slot).  Replaces the reduction over
+// the gradient array of garden.cu:432-435.  One wave.
+__global__ void __launch_bounds__(64)
+k_root_from_hist(const long long *__restrict__ hg, const long long *__restrict__ hh,
+                 NodeSum *__restrict__ tot) {
+  long long a = 0, b = 0;
+  for (int i = threadIdx.x; i < kSlots; i += 64) {
+    a += hg[i];
+    b += hh[i];
+  }
+  a = WaveSumLL(a);
+  b = WaveSumLL(b);
+  if (threadIdx.x == 0) {
+    tot[0].g = a;
+    tot[0].h = b;
   }
 }
 
@@ -558,116 +831,6 @@ __global__ void k_split_select(const Cand *__restrict__ cand, int F, int L,
   t_gain[heap_off + nd] = rec.gain;
 }
 
-// ---------------------------------------------------------------- partition
-__device__ __forceinline__ bool GoesRight(const uint32_t *__restrict__ bins, size_t stride,
-                                          const SplitRec &s, unsigned r) {
-  // builder.h:107-123: bin >= q + 1 goes right
-  if (s.fid < 0) return false;
-  const uint32_t b4 = bins[(size_t)(s.fid >> 2) * stride + r];
-  return (int)((b4 >> (8 * (s.fid & 3))) & 255u) > s.bin;
-}
-
-__global__ void __launch_bounds__(kPartThreads)
-k_part_count(const uint32_t *__restrict__ bins, size_t stride, const SplitRec *__restrict__ split,
-             const WorkItem *__restrict__ work, const unsigned *__restrict__ n_work,
-             unsigned *__restrict__ item_left) {
-  __shared__ unsigned s_cnt[kPartThreads / 64];
-  const unsigned w = blockIdx.x;
-  if (w >= *n_work) return;
-  const WorkItem it = work[w];
-  const SplitRec s = split[it.node];
-  unsigned cnt = 0;
-  for (unsigned r = it.begin + threadIdx.x; r < it.end; r += kPartThreads)
-    cnt += GoesRight(bins, stride, s, r) ? 0u : 1u;
-  for (int off = 32; off > 0; off >>= 1) cnt += __shfl_down(cnt, off);
-  if ((threadIdx.x & 63) == 0) s_cnt[threadIdx.x >> 6] = cnt;
-  __syncthreads();
-  if (threadIdx.x == 0) {
-    unsigned t = 0;
-    for (int k = 0; k < kPartThreads / 64; ++k) t += s_cnt[k];
-    item_left[w] = t;
-  }
-}
-
-// Exclusive scan of item_left over all work items.  One workgroup.
-__global__ void __launch_bounds__(1024)
-k_part_scan(const unsigned *__restrict__ item_left, const unsigned *__restrict__ n_work,
-            unsigned *__restrict__ excl) {
-  __shared__ unsigned s_part[1024];
-  const unsigned n = *n_work;
-  const unsigned per = (n + 1023) / 1024;
-  const unsigned b = threadIdx.x * per, e = min(n, b + per);
-  unsigned sum = 0;
-  for (unsigned i = b; i < e; ++i) sum += item_left[i];
-  s_part[threadIdx.x] = sum;
-  __syncthreads();
-  if (threadIdx.x == 0) {
-    unsigned run = 0;
-    for (int i = 0; i < 1024; ++i) {
-      const unsigned v = s_part[i];
-      s_part[i] = run;
-      run += v;
-    }
-  }
-  __syncthreads();
-  unsigned run = s_part[threadIdx.x];
-  for (unsigned i = b; i < e; ++i) {
-    excl[i] = run;
-    run += item_left[i];
-  }
-}
-
-// Stable partition of one work item's rows into the children ranges.
-template <bool PAIR>
-__global__ void __launch_bounds__(kPartThreads)
-k_partition(const uint32_t *__restrict__ bins, uint32_t *__restrict__ bins_out, size_t stride, int Q,
-            const float *__restrict__ g, float *__restrict__ g_out, const float *__restrict__ h,
-            float *__restrict__ h_out, const unsigned *__restrict__ rowid,
-            unsigned *__restrict__ rowid_out, const SplitRec *__restrict__ split,
-            const unsigned *__restrict__ seg_start, const WorkItem *__restrict__ work,
-            const unsigned *__restrict__ n_work, const unsigned *__restrict__ excl) {
-  __shared__ unsigned s_cnt[kPartThreads / 64];
-  const unsigned w = blockIdx.x;
-  if (w >= *n_work) return;
-  const WorkItem it = work[w];
-  const SplitRec s = split[it.node];
-  const unsigned start = seg_start[it.node];
-  const unsigned lefts_before = excl[w] - excl[it.first];
-  unsigned lo = start + lefts_before;
-  unsigned ro = start + (unsigned)s.left.c + (it.begin - start) - lefts_before;
-  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-  for (unsigned base = it.begin; base < it.end; base += kPartThreads) {
-    const unsigned r = base + threadIdx.x;
-    const bool valid = r < it.end;
-    const bool right = valid && GoesRight(bins, stride, s, r);
-    const bool left = valid && !right;
-    const unsigned long long lm = __ballot(left);
-    const unsigned long long below = (1ull << lane) - 1ull;
-    if (lane == 0) s_cnt[wave] = (unsigned)__popcll(lm);
-    __syncthreads();
-    unsigned left_waves = 0, left_tile = 0;
-#pragma unroll
-    for (int k = 0; k < kPartThreads / 64; ++k) {
-      const unsigned c = s_cnt[k];
-      if (k < wave) left_waves += c;
-      left_tile += c;
-    }
-    const unsigned lrank = left_waves + (unsigned)__popcll(lm & below);
-    const unsigned rrank = (unsigned)threadIdx.x - lrank;  // invalid lanes only sit above valid ones
-    const unsigned tile_valid = min((unsigned)kPartThreads, it.end - base);
-    if (valid) {
-      const unsigned d = left ? lo + lrank : ro + rrank;
-      for (int q = 0; q < Q; ++q) bins_out[(size_t)q * stride + d] = bins[(size_t)q * stride + r];
-      g_out[d] = g[r];
-      if (PAIR) h_out[d] = h[r];
-      rowid_out[d] = rowid ? rowid[r] : r;
-    }
-    lo += left_tile;
-    ro += tile_valid - left_tile;
-    __syncthreads();
-  }
-}
-
 // --------------------------------------------------------------- leaves
 // UpdateLeafWeight (garden.cu:487-503, split.cu:25-35): left = Weight(left
 // sum), right = Weight(parent - left) with the subtraction in the sum type.
@@ -694,27 +857,56 @@ __global__ void k_leaf_weights(const SplitRec *__restrict__ split, const NodeSum
   weights[2 * nd + 1] = LeafWeight<PAIR, F64>(GR, HR, (unsigned)(t.c - s.left.c), gp) * eta;
 }
 
-// leaf id of every row of the last split level, scattered to original order
-__global__ void __launch_bounds__(kPartThreads)
-k_leaf_assign(const uint32_t *__restrict__ bins, size_t stride, const unsigned *__restrict__ rowid,
-              const SplitRec *__restrict__ split, const WorkItem *__restrict__ work,
-              const unsigned *__restrict__ n_work, unsigned *__restrict__ leaf_of) {
-  const unsigned w = blockIdx.x;
-  if (w >= *n_work) return;
-  const WorkItem it = work[w];
-  const SplitRec s = split[it.node];
-  for (unsigned r = it.begin + threadIdx.x; r < it.end; r += kPartThreads) {
-    const unsigned leaf = it.node * 2 + (GoesRight(bins, stride, s, r) ? 1u : 0u);
-    leaf_of[rowid ? rowid[r] : r] = leaf;
+// End of a tree, rows in original order: walk the tree on the row's bins
+// (bin >= q+1 goes right, builder.h:107-123), record the leaf, add its weight
+// to y_hat (update_by_last_tree, garden.cu:45-76) and, when NEXT_GRAD is not
+// 0, write the gradients of the next round (objective.cu:28-56):
+// 1 = squared (also max |g|), 2 = logistic.
+template <int NEXT_GRAD>
+__global__ void __launch_bounds__(256)
+k_final(const uint32_t *__restrict__ bins, size_t stride, const int *__restrict__ t_fid,
+        const int *__restrict__ t_bin, int depth, const float *__restrict__ weights,
+        float *__restrict__ yhat, const float *__restrict__ y, unsigned *__restrict__ leaf_of,
+        float *__restrict__ g, float *__restrict__ h, unsigned *__restrict__ gmax_bits, size_t n) {
+  extern __shared__ int s_nodes[];  // fid[internal], bin[internal]
+  const int internal = (1 << (depth - 1)) - 1;
+  for (int i = threadIdx.x; i < internal; i += blockDim.x) {
+    s_nodes[i] = t_fid[i];
+    s_nodes[internal + i] = t_bin[i];
   }
-}
-
-// update_by_last_tree (garden.cu:45-76): y_hat += weight of the row's leaf
-__global__ void k_update_yhat(float *__restrict__ yhat, const unsigned *__restrict__ leaf_of,
-                              const float *__restrict__ weights, size_t n) {
+  __syncthreads();
+  float m = 0.0f;
   for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < n;
-       i += (size_t)gridDim.x * blockDim.x)
-    yhat[i] += weights[leaf_of[i]];
+       i += (size_t)gridDim.x * blockDim.x) {
+    unsigned node = 0;
+    for (int level = 0; level + 1 < depth; ++level) {
+      const int id = (1 << level) - 1 + (int)node;
+      const int fid = s_nodes[id], bin = s_nodes[internal + id];
+      unsigned right = 0;
+      if (bin >= 0) {
+        const uint32_t b4 = bins[(size_t)(fid >> 2) * stride + i];
+        right = (int)((b4 >> (8 * (fid & 3))) & 255u) > bin ? 1u : 0u;
+      }
+      node = node * 2 + right;
+    }
+    leaf_of[i] = node;
+    const float yh = yhat[i] + weights[node];
+    yhat[i] = yh;
+    if (NEXT_GRAD == 1) {
+      const float v = y[i] - yh;
+      g[i] = v;
+      const float a = fabsf(v);
+      if (a > m) m = a;
+    } else if (NEXT_GRAD == 2) {
+      const float s = SigmoidF(yh);
+      g[i] = y[i] - s;
+      h[i] = s * (1.0f - s);
+    }
+  }
+  if (NEXT_GRAD == 1) {
+    m = WaveMaxF(m);
+    if ((threadIdx.x & 63) == 0) atomicMax(gmax_bits, __float_as_uint(m));
+  }
 }
 
 __global__ void k_fill_f32(float *p, float v, size_t n) {
@@ -884,8 +1076,86 @@ namespace {
 struct RowBuffers {
   uint32_t *bins = nullptr;
   float *g = nullptr, *h = nullptr;
-  unsigned *rowid = nullptr;
 };
+
+// Raises the dynamic LDS limit of a kernel once (needed above 64 KB).
+template <typename K>
+void AllowLds(K kernel, size_t bytes) {
+  static size_t allowed = 0;  // one instance per kernel type/pointer value below
+  (void)allowed;
+  HIP_OK(hipFuncSetAttribute((const void *)kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)bytes));
+}
+
+template <bool PAIR, int NQ>
+void LaunchHistNQ(hipStream_t st, unsigned grid, const uint32_t *bins, size_t stride, int q0, int F,
+                  const float *g, const float *h, const int *shifts, const WorkItem *work,
+                  const unsigned *n_work, unsigned long long *slab, int nbin_total) {
+  const size_t lds = (size_t)NQ * 4 * kSlots * 8 * (PAIR ? 2 : 1);
+  static bool configured = false;
+  if (!configured) {
+    AllowLds(k_hist<PAIR, NQ>, lds);
+    configured = true;
+  }
+  hipLaunchKernelGGL((k_hist<PAIR, NQ>), dim3(grid), dim3(kHistThreads), lds, st, bins, stride, q0, F, g, h,
+                     shifts, work, n_work, slab, nbin_total);
+}
+
+template <bool PAIR>
+void LaunchHist(int nq, hipStream_t st, unsigned grid, const uint32_t *bins, size_t stride, int q0, int F,
+                const float *g, const float *h, const int *shifts, const WorkItem *work,
+                const unsigned *n_work, unsigned long long *slab, int nbin_total) {
+#define ARB_CASE(N) \
+  case N: LaunchHistNQ<PAIR, N>(st, grid, bins, stride, q0, F, g, h, shifts, work, n_work, slab, nbin_total); break;
+  switch (nq) {
+    ARB_CASE(1) ARB_CASE(2) ARB_CASE(3) ARB_CASE(4) ARB_CASE(5) ARB_CASE(6) ARB_CASE(7) ARB_CASE(8) ARB_CASE(9)
+    default: throw std::runtime_error("internal: bad quad count");
+  }
+#undef ARB_CASE
+}
+
+struct FusedArgs {
+  const uint32_t *bins;
+  uint32_t *bins_out;
+  size_t stride;
+  int F;
+  const float *g;
+  float *g_out;
+  const float *h;
+  float *h_out;
+  const int *shifts;
+  const SplitRec *split;
+  const NodeSum *tot;
+  const unsigned *seg_start;
+  const WorkItem *work;
+  const unsigned *n_work;
+  const unsigned *excl;
+  unsigned long long *slab;
+  int nbin_total;
+};
+
+template <bool PAIR, int NQ, bool WRITE>
+void LaunchFusedNQ(hipStream_t st, unsigned grid, const FusedArgs &a) {
+  const size_t lds = (size_t)NQ * 4 * kSlots * 8 * (PAIR ? 2 : 1);
+  static bool configured = false;
+  if (!configured) {
+    AllowLds(k_part_hist<PAIR, NQ, WRITE>, lds);
+    configured = true;
+  }
+  hipLaunchKernelGGL((k_part_hist<PAIR, NQ, WRITE>), dim3(grid), dim3(kHistThreads), lds, st, a.bins, a.bins_out,
+                     a.stride, a.F, a.g, a.g_out, a.h, a.h_out, a.shifts, a.split, a.tot, a.seg_start, a.work,
+                     a.n_work, a.excl, a.slab, a.nbin_total);
+}
+
+template <bool PAIR, bool WRITE>
+void LaunchFused(int nq, hipStream_t st, unsigned grid, const FusedArgs &a) {
+#define ARB_CASE(N) \
+  case N: LaunchFusedNQ<PAIR, N, WRITE>(st, grid, a); break;
+  switch (nq) {
+    ARB_CASE(1) ARB_CASE(2) ARB_CASE(3) ARB_CASE(4) ARB_CASE(5) ARB_CASE(6) ARB_CASE(7) ARB_CASE(8) ARB_CASE(9)
+    default: throw std::runtime_error("internal: bad quad count");
+  }
+#undef ARB_CASE
+}
 
 class HipTreeBuilder : public TreeBuilder {
  public:
@@ -909,12 +1179,10 @@ class HipTreeBuilder : public TreeBuilder {
 
     // quads per histogram launch, limited by LDS
     const size_t per_quad = (size_t)4 * kSlots * 8 * (pair_ ? 2 : 1);
-    quads_per_group_ = (int)std::max<size_t>(1, std::min<size_t>((kLdsBudget - 1024) / per_quad, Q_));
-    lds_bytes_ = (size_t)quads_per_group_ * per_quad;
-    if (pair_)
-      HIP_OK(hipFuncSetAttribute((const void *)k_hist<true>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes_));
-    else
-      HIP_OK(hipFuncSetAttribute((const void *)k_hist<false>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes_));
+    quads_per_group_ = (int)std::min<size_t>(std::min<size_t>((kLdsBudget - 1024) / per_quad, kMaxGroupQuads), Q_);
+    // the fused partition + histogram pass holds one histogram of all
+    // features and builds only the smaller child
+    fused_ = trick_ && Q_ <= quads_per_group_;
 
     // per-row state in original order
     d_y_ = DevAlloc<float>(n_);
@@ -930,13 +1198,13 @@ class HipTreeBuilder : public TreeBuilder {
     hipLaunchKernelGGL(k_fill_f32, dim3(GridFor(n_ * K_, 256)), dim3(256), 0, stream_, d_yhat_, init, n_ * K_);
     data->y_hat.assign(n_ * K_, init);  // garden.cu:104
 
-    // ping-pong row buffers (not needed when the tree has a single split level)
+    // ping-pong row buffers in node order (not needed for a single split level)
     if (D_ > 2) {
-      for (int b = 0; b < 2; ++b) {
+      const int nbuf = (fused_ && D_ == 3) ? 0 : 2;  // fused: the last level writes nothing
+      for (int b = 0; b < nbuf; ++b) {
         buf_[b].bins = DevAlloc<uint32_t>((size_t)Q_ * stride_);
         buf_[b].g = DevAlloc<float>(n_);
         buf_[b].h = DevAlloc<float>(n_);
-        buf_[b].rowid = DevAlloc<unsigned>(n_);
       }
     }
     // level state
@@ -953,17 +1221,18 @@ class HipTreeBuilder : public TreeBuilder {
     d_node_first_ = DevAlloc<unsigned>(last_nodes);
     d_node_items_ = DevAlloc<unsigned>(last_nodes);
     max_hist_items_ = (unsigned)(n_ / HistRowsPerItem(n_)) + last_nodes + 2;
-    max_part_items_ = (unsigned)(n_ / kPartRows + 1) + last_nodes;
+    max_part_items_ = std::max<unsigned>((unsigned)(n_ / kPartRows + 1) + last_nodes, max_hist_items_);
     d_hwork_ = DevAlloc<WorkItem>(max_hist_items_);
     d_pwork_ = DevAlloc<WorkItem>(max_part_items_);
     d_nwork_ = DevAlloc<unsigned>(2);
-    d_item_left_ = DevAlloc<unsigned>(max_part_items_);
-    d_excl_ = DevAlloc<unsigned>(max_part_items_);
-    d_slab_ = DevAlloc<unsigned long long>((size_t)max_hist_items_ * nbin_total_ * (pair_ ? 2 : 1));
+    d_wave_left_ = DevAlloc<unsigned>((size_t)max_part_items_ * kItemWaves);
+    d_excl_ = DevAlloc<unsigned>((size_t)max_part_items_ * kItemWaves);
+    d_slab_ = DevAlloc<unsigned long long>((size_t)std::max(max_hist_items_, max_part_items_) * nbin_total_ * (pair_ ? 2 : 1));
     d_shifts_ = DevAlloc<int>(2);
     d_gmax_ = DevAlloc<unsigned>(1);
     d_rows_scanned_ = DevAlloc<unsigned long long>(1);
     HIP_OK(hipMemsetAsync(d_rows_scanned_, 0, sizeof(unsigned long long), stream_));
+    HIP_OK(hipMemsetAsync(d_gmax_, 0, sizeof(unsigned), stream_));
     const int internal = (1 << (D_ - 1)) - 1;
     d_tfid_ = DevAlloc<int>(internal);
     d_tbin_ = DevAlloc<int>(internal);
@@ -979,13 +1248,12 @@ class HipTreeBuilder : public TreeBuilder {
   ~HipTreeBuilder() override {
     (void)hipStreamSynchronize(stream_);
     void *ptrs[] = {d_y_, d_labels_, d_yhat_, d_g_, d_h_, d_leaf_, d_split_, d_cand_, d_node_first_,
-                    d_node_items_, d_hwork_, d_pwork_, d_nwork_, d_item_left_, d_excl_, d_slab_,
+                    d_node_items_, d_hwork_, d_pwork_, d_nwork_, d_wave_left_, d_excl_, d_slab_,
                     d_shifts_, d_gmax_, d_rows_scanned_, d_tfid_, d_tbin_, d_tgain_, d_weights_};
     for (void *p : ptrs)
       if (p) (void)hipFree(p);
     for (int b = 0; b < 2; ++b) {
-      void *q[] = {buf_[b].bins, buf_[b].g, buf_[b].h, buf_[b].rowid, d_tot_[b], d_seg_[b],
-                   d_hg_[b], d_hh_[b], d_hc_[b]};
+      void *q[] = {buf_[b].bins, buf_[b].g, buf_[b].h, d_tot_[b], d_seg_[b], d_hg_[b], d_hh_[b], d_hc_[b]};
       for (void *p : q)
         if (p) (void)hipFree(p);
     }
@@ -994,18 +1262,21 @@ class HipTreeBuilder : public TreeBuilder {
   }
 
   void GrowRound(std::vector<RegTree> *trees) override {
-    Mark(kGrad);
-    if (cfg_.objective == kLinearRegression) {
-      // the maximum is cleared by k_init_root of the previous tree / below
-      hipLaunchKernelGGL(k_init_root, dim3(1), dim3(64), 0, stream_, d_tot_[0], d_seg_[0],
-                         (unsigned long long)n_, d_gmax_);
-      hipLaunchKernelGGL(k_grad_squared, dim3(GridFor(n_, 256)), dim3(256), 0, stream_, d_y_, d_yhat_, d_g_, n_, d_gmax_);
-      hipLaunchKernelGGL(k_set_shift, dim3(1), dim3(64), 0, stream_, d_gmax_, d_shifts_);
-    } else if (cfg_.objective == kLogisticRegression) {
-      hipLaunchKernelGGL(k_grad_logistic, dim3(GridFor(n_, 256)), dim3(256), 0, stream_, d_y_, d_yhat_, d_g_, d_h_, n_);
-    } else {
-      hipLaunchKernelGGL(k_grad_softmax, dim3(GridFor(n_, 256)), dim3(256), 0, stream_, d_labels_, d_yhat_, d_g_, d_h_, n_, K_);
+    // Gradients of this round, unless the last pass of the previous tree has
+    // already written them (single-output objectives, inspection off).
+    if (!grad_ready_) {
+      Mark(kGrad);
+      if (cfg_.objective == kLinearRegression) {
+        hipLaunchKernelGGL(k_grad_squared, dim3(GridFor(n_, 256)), dim3(256), 0, stream_, d_y_, d_yhat_, d_g_, n_, d_gmax_);
+      } else if (cfg_.objective == kLogisticRegression) {
+        hipLaunchKernelGGL(k_grad_logistic, dim3(GridFor(n_, 256)), dim3(256), 0, stream_, d_y_, d_yhat_, d_g_, d_h_, n_);
+      } else {
+        hipLaunchKernelGGL(k_grad_softmax, dim3(GridFor(n_, 256)), dim3(256), 0, stream_, d_labels_, d_yhat_, d_g_, d_h_, n_, K_);
+      }
     }
+    if (cfg_.objective == kLinearRegression)
+      hipLaunchKernelGGL(k_set_shift, dim3(1), dim3(64), 0, stream_, d_gmax_, d_shifts_);
+    grad_ready_ = false;
     Mark(kNone);
     for (int k = 0; k < K_; ++k) {
       RegTree tree((unsigned)D_, (unsigned)k);
@@ -1025,6 +1296,7 @@ class HipTreeBuilder : public TreeBuilder {
     HIP_OK(hipMemcpy(out, d_yhat_, n_ * K_ * sizeof(float), hipMemcpyDeviceToHost));
   }
   void GetGrad(float *g, float *h) override {
+    if (!inspect_) throw std::runtime_error("gradients of the last round are only kept with inspection on");
     HIP_OK(hipStreamSynchronize(stream_));
     HIP_OK(hipMemcpy(g, d_g_, n_ * K_ * sizeof(float), hipMemcpyDeviceToHost));
     if (h) {
@@ -1041,6 +1313,8 @@ class HipTreeBuilder : public TreeBuilder {
     return (int)(v.size() / 3);
   }
   void GetShifts(int *sg, int *sh) override {
+    if (!inspect_ && cfg_.objective == kLinearRegression)
+      throw std::runtime_error("the scale of the last round is only kept with inspection on");
     int s[2];
     HIP_OK(hipStreamSynchronize(stream_));
     HIP_OK(hipMemcpy(s, d_shifts_, sizeof(s), hipMemcpyDeviceToHost));
@@ -1058,7 +1332,7 @@ class HipTreeBuilder : public TreeBuilder {
   void Synchronize() override { HIP_OK(hipStreamSynchronize(stream_)); }
 
  private:
-  enum Phase { kNone = -1, kGrad = 0, kHistRoot, kHistDeep, kReduce, kSplit, kPartition, kLeaf, kPlan, kPhases };
+  enum Phase { kNone = -1, kGrad = 0, kHistRoot, kHistDeep, kReduce, kSplit, kPartition, kLeaf, kPlan, kFusedLast, kPhases };
 
   // Timing: an event is recorded at every phase change; the time between two
   // consecutive events is charged to the phase that was open.
@@ -1083,7 +1357,7 @@ class HipTreeBuilder : public TreeBuilder {
     }
     HIP_OK(hipStreamSynchronize(stream_));
     double *slots[kPhases] = {&timings_.grad, &timings_.hist_root, &timings_.hist_deep, &timings_.reduce,
-                              &timings_.split, &timings_.partition, &timings_.leaf, &timings_.plan};
+                              &timings_.split, &timings_.partition, &timings_.leaf, &timings_.plan, &timings_.fused_last};
     for (size_t i = 0; i + 1 < marks_.size(); ++i) {
       if (marks_[i] < 0) continue;
       float ms = 0;
@@ -1094,21 +1368,49 @@ class HipTreeBuilder : public TreeBuilder {
     event_used_ = 0;
   }
 
-  unsigned HistRowsPerItem(size_t rows_max) const {
-    // about 512 work items per level, whole tiles, at most kMaxHistRows rows
+  static unsigned HistRowsPerItem(size_t rows_max) {
+    // about 512 work items per level, whole 1024-row tiles, at most kMaxHistRows rows
     size_t t = (rows_max + 511) / 512;
     t = (t + kHistThreads - 1) / kHistThreads * kHistThreads;
     return (unsigned)std::min<size_t>(std::max<size_t>(t, kHistThreads), kMaxHistRows);
   }
 
-  template <bool PAIR>
-  void LaunchHist(const RowBuffers &cur, unsigned grid) {
+  void Plan(int state, int L, int select, unsigned rows_per_item, WorkItem *work, unsigned *n_work,
+            bool count_rows, const SplitRec *split, unsigned max_items) {
+    hipLaunchKernelGGL(k_plan, dim3(1), dim3(1024), 0, stream_, d_tot_[state], d_seg_[state], L, select,
+                       rows_per_item, work, n_work, d_node_first_, d_node_items_,
+                       count_rows ? d_rows_scanned_ : (unsigned long long *)nullptr, split, max_items);
+  }
+
+  // Histograms of contiguous node ranges in `cur` (level order), feature group by group.
+  void HistOfNodes(const RowBuffers &cur, int state, int L, bool select_smaller, size_t rows_max, bool root) {
+    const unsigned per_item = HistRowsPerItem(rows_max);
+    const unsigned grid = (unsigned)std::min<size_t>(rows_max / per_item + L + 1, max_hist_items_);
+    Mark(kPlan);
+    Plan(state, L, select_smaller ? 1 : 0, per_item, d_hwork_, d_nwork_, true, nullptr, grid);
+    Mark(root ? kHistRoot : kHistDeep);
     for (int q0 = 0; q0 < Q_; q0 += quads_per_group_) {
       const int nq = std::min(quads_per_group_, Q_ - q0);
-      const size_t lds = (size_t)nq * 4 * kSlots * 8 * (PAIR ? 2 : 1);
-      hipLaunchKernelGGL(k_hist<PAIR>, dim3(grid), dim3(kHistThreads), lds, stream_, cur.bins, stride_,
-                         q0, nq, F_, cur.g, cur.h, d_shifts_, d_hwork_, d_nwork_, d_slab_, nbin_total_);
+      if (pair_)
+        LaunchHist<true>(nq, stream_, grid, cur.bins, stride_, q0, F_, cur.g, cur.h, d_shifts_, d_hwork_, d_nwork_, d_slab_, nbin_total_);
+      else
+        LaunchHist<false>(nq, stream_, grid, cur.bins, stride_, q0, F_, cur.g, cur.h, d_shifts_, d_hwork_, d_nwork_, d_slab_, nbin_total_);
+      if (timing_) ++(root ? timings_.hist_root_launches : timings_.hist_deep_launches);
     }
+    if (timing_ && root) timings_.hist_root_rows += n_;
+  }
+
+  void Reduce(int L, int hb, bool by_parent, int parent_state, bool trick) {
+    Mark(kReduce);
+    dim3 grid(nbin_total_ / 64, L);
+    if (pair_)
+      hipLaunchKernelGGL(k_hist_reduce<true>, grid, dim3(1024), 0, stream_, d_slab_, nbin_total_, d_node_first_,
+                         d_node_items_, by_parent ? 1 : 0, d_split_, d_tot_[parent_state], d_hg_[hb], d_hh_[hb],
+                         d_hc_[hb], d_hg_[hb ^ 1], d_hh_[hb ^ 1], d_hc_[hb ^ 1], trick ? 1 : 0);
+    else
+      hipLaunchKernelGGL(k_hist_reduce<false>, grid, dim3(1024), 0, stream_, d_slab_, nbin_total_, d_node_first_,
+                         d_node_items_, by_parent ? 1 : 0, d_split_, d_tot_[parent_state], d_hg_[hb], d_hh_[hb],
+                         d_hc_[hb], d_hg_[hb ^ 1], d_hh_[hb ^ 1], d_hc_[hb ^ 1], trick ? 1 : 0);
   }
 
   void GrowOne(int label, RegTree *tree) {
@@ -1117,54 +1419,66 @@ class HipTreeBuilder : public TreeBuilder {
     orig.bins = dm_->bins;
     orig.g = d_g_ + (size_t)label * n_;
     orig.h = d_h_ + (size_t)label * n_;
-    orig.rowid = nullptr;
     if (inspect_) kept_hist_.assign(D_ - 1, {});
 
-    Mark(kGrad);
-    if (cfg_.objective != kLinearRegression || label > 0)
-      hipLaunchKernelGGL(k_init_root, dim3(1), dim3(64), 0, stream_, d_tot_[0], d_seg_[0],
-                         (unsigned long long)n_, (unsigned *)nullptr);
-    if (pair_)
-      hipLaunchKernelGGL(k_root_total<true>, dim3(GridFor(n_, 256, 1024)), dim3(256), 0, stream_, orig.g, orig.h, d_shifts_, n_, d_tot_[0]);
-    else
-      hipLaunchKernelGGL(k_root_total<false>, dim3(GridFor(n_, 256, 1024)), dim3(256), 0, stream_, orig.g, orig.h, d_shifts_, n_, d_tot_[0]);
-
-    int cur_state = 0;  // index into d_tot_/d_seg_
+    hipLaunchKernelGGL(k_init_root, dim3(1), dim3(64), 0, stream_, d_tot_[0], d_seg_[0],
+                       (unsigned long long)n_, (unsigned *)nullptr);
+    int state = 0;  // d_tot_/d_seg_[state] describe the nodes of the current level
     for (int level = 0; level + 1 < D_; ++level) {
       const int L = 1 << level;
-      const RowBuffers &cur = level == 0 ? orig : buf_[(level - 1) & 1];
-      const bool trick = trick_ && level > 0;
-      const int hb = level & 1;  // histogram buffer of this level; parent is hb ^ 1
-      // ---- histogram of the level
-      const size_t rows_max = trick ? n_ / 2 : n_;
-      const unsigned per_item = HistRowsPerItem(rows_max);
-      const unsigned grid_bound = (unsigned)std::min<size_t>(rows_max / per_item + L + 1, max_hist_items_);
-      Mark(kPlan);
-      hipLaunchKernelGGL(k_plan, dim3(1), dim3(1024), 0, stream_, d_tot_[cur_state], d_seg_[cur_state], L,
-                         trick ? 1 : 0, per_item, d_hwork_, d_nwork_, d_node_first_, d_node_items_,
-                         d_rows_scanned_, grid_bound);
-      Mark(level == 0 ? kHistRoot : kHistDeep);
-      if (timing_) {
-        if (level == 0) {
-          timings_.hist_root_launches += (Q_ + quads_per_group_ - 1) / quads_per_group_;
-          timings_.hist_root_rows += n_;
+      const int hb = level & 1;  // histogram buffer of this level; the parent level is hb ^ 1
+      const bool last = level + 2 >= D_;
+      if (level == 0) {
+        HistOfNodes(orig, state, 1, false, n_, true);
+        Reduce(1, hb, false, state, false);
+        hipLaunchKernelGGL(k_root_from_hist, dim3(1), dim3(64), 0, stream_, d_hg_[hb], d_hh_[hb], d_tot_[state]);
+      } else {
+        // rows are in the order of level-1; the parents' state is state ^ 1
+        const int ps = state ^ 1, PL = L >> 1;
+        const RowBuffers &src = level == 1 ? orig : buf_[level & 1];
+        const RowBuffers &dst = buf_[(level & 1) ^ 1];
+        if (fused_) {
+          const unsigned per_item = HistRowsPerItem(n_);
+          const unsigned grid = (unsigned)std::min<size_t>(n_ / per_item + PL + 1, max_part_items_);
+          Mark(kPlan);
+          Plan(ps, PL, 0, per_item, d_pwork_, d_nwork_ + 1, true, d_split_, grid);
+          if (!last) {  // destination offsets; the last level moves no rows
+            Mark(kPartition);
+            hipLaunchKernelGGL(k_part_count, dim3(grid), dim3(kHistThreads), 0, stream_, src.bins, stride_, d_split_,
+                               d_pwork_, d_nwork_ + 1, d_wave_left_);
+            hipLaunchKernelGGL(k_part_scan, dim3(1), dim3(1024), 0, stream_, d_wave_left_, d_nwork_ + 1, d_excl_);
+          }
+          Mark(last ? kFusedLast : kHistDeep);
+          FusedArgs a{src.bins, dst.bins, stride_, F_, src.g, dst.g, src.h, dst.h, d_shifts_, d_split_,
+                      d_tot_[ps], d_seg_[ps], d_pwork_, d_nwork_ + 1, d_excl_, d_slab_, nbin_total_};
+          if (pair_) {
+            if (last) LaunchFused<true, false>(Q_, stream_, grid, a);
+            else LaunchFused<true, true>(Q_, stream_, grid, a);
+          } else {
+            if (last) LaunchFused<false, false>(Q_, stream_, grid, a);
+            else LaunchFused<false, true>(Q_, stream_, grid, a);
+          }
+          if (timing_) ++(last ? timings_.fused_last_launches : timings_.hist_deep_launches);
+          Reduce(L, hb, true, ps, true);
         } else {
-          timings_.hist_deep_launches += (Q_ + quads_per_group_ - 1) / quads_per_group_;
+          const unsigned grid = (unsigned)std::min<size_t>(n_ / kPartRows + PL + 1, max_part_items_);
+          Mark(kPlan);
+          Plan(ps, PL, 0, kPartRows, d_pwork_, d_nwork_ + 1, false, nullptr, grid);
+          Mark(kPartition);
+          hipLaunchKernelGGL(k_part_count, dim3(grid), dim3(kHistThreads), 0, stream_, src.bins, stride_, d_split_,
+                             d_pwork_, d_nwork_ + 1, d_wave_left_);
+          hipLaunchKernelGGL(k_part_scan, dim3(1), dim3(1024), 0, stream_, d_wave_left_, d_nwork_ + 1, d_excl_);
+          if (pair_)
+            hipLaunchKernelGGL(k_partition<true>, dim3(grid), dim3(kHistThreads), 0, stream_, src.bins, dst.bins,
+                               stride_, Q_, src.g, dst.g, src.h, dst.h, d_split_, d_seg_[ps], d_pwork_,
+                               d_nwork_ + 1, d_excl_);
+          else
+            hipLaunchKernelGGL(k_partition<false>, dim3(grid), dim3(kHistThreads), 0, stream_, src.bins, dst.bins,
+                               stride_, Q_, src.g, dst.g, src.h, dst.h, d_split_, d_seg_[ps], d_pwork_,
+                               d_nwork_ + 1, d_excl_);
+          HistOfNodes(dst, state, L, trick_, trick_ ? n_ / 2 : n_, false);
+          Reduce(L, hb, false, ps, trick_);
         }
-      }
-      if (pair_)
-        LaunchHist<true>(cur, grid_bound);
-      else
-        LaunchHist<false>(cur, grid_bound);
-      Mark(kReduce);
-      {
-        dim3 grid(nbin_total_ / 64, L);
-        if (pair_)
-          hipLaunchKernelGGL(k_hist_reduce<true>, grid, dim3(1024), 0, stream_, d_slab_, nbin_total_, d_node_first_,
-                             d_node_items_, d_hg_[hb], d_hh_[hb], d_hc_[hb], d_hg_[hb ^ 1], d_hh_[hb ^ 1], d_hc_[hb ^ 1], trick ? 1 : 0);
-        else
-          hipLaunchKernelGGL(k_hist_reduce<false>, grid, dim3(1024), 0, stream_, d_slab_, nbin_total_, d_node_first_,
-                             d_node_items_, d_hg_[hb], d_hh_[hb], d_hc_[hb], d_hg_[hb ^ 1], d_hh_[hb ^ 1], d_hc_[hb ^ 1], trick ? 1 : 0);
       }
       if (inspect_) KeepHist(level, L, hb);
       // ---- split scan and selection
@@ -1174,52 +1488,51 @@ class HipTreeBuilder : public TreeBuilder {
         const int hs = std::min(cfg_.internal.hist_size, kSlots);
 #define ARB_SCAN(P, D) \
   hipLaunchKernelGGL((k_split_scan<P, D>), grid, dim3(64), 0, stream_, d_hg_[hb], d_hh_[hb], d_hc_[hb], \
-                     nbin_total_, F_, d_tot_[cur_state], d_shifts_, gp, hs, d_cand_)
+                     nbin_total_, F_, d_tot_[state], d_shifts_, gp, hs, d_cand_)
         if (pair_ && f64_) ARB_SCAN(true, true);
         else if (pair_) ARB_SCAN(true, false);
         else if (f64_) ARB_SCAN(false, true);
         else ARB_SCAN(false, false);
 #undef ARB_SCAN
         hipLaunchKernelGGL(k_split_select, dim3((L + 127) / 128), dim3(128), 0, stream_, d_cand_, F_, L,
-                           d_tot_[cur_state], d_seg_[cur_state], d_tot_[cur_state ^ 1], d_seg_[cur_state ^ 1],
-                           d_split_, d_tfid_, d_tbin_, d_tgain_, L - 1);
+                           d_tot_[state], d_seg_[state], d_tot_[state ^ 1], d_seg_[state ^ 1], d_split_,
+                           d_tfid_, d_tbin_, d_tgain_, L - 1);
       }
-      // ---- move rows to the children order, or assign leaves at the last level
-      const unsigned pgrid = (unsigned)std::min<size_t>(n_ / kPartRows + L + 1, max_part_items_);
-      Mark(kPlan);
-      hipLaunchKernelGGL(k_plan, dim3(1), dim3(1024), 0, stream_, d_tot_[cur_state], d_seg_[cur_state], L, 0,
-                         kPartRows, d_pwork_, d_nwork_ + 1, d_node_first_, d_node_items_,
-                         (unsigned long long *)nullptr, pgrid);
-      Mark(level + 2 < D_ ? kPartition : kLeaf);
-      if (level + 2 < D_) {
-        const RowBuffers &nxt = buf_[level & 1];
-        hipLaunchKernelGGL(k_part_count, dim3(pgrid), dim3(kPartThreads), 0, stream_, cur.bins, stride_, d_split_,
-                           d_pwork_, d_nwork_ + 1, d_item_left_);
-        hipLaunchKernelGGL(k_part_scan, dim3(1), dim3(1024), 0, stream_, d_item_left_, d_nwork_ + 1, d_excl_);
-        if (pair_)
-          hipLaunchKernelGGL(k_partition<true>, dim3(pgrid), dim3(kPartThreads), 0, stream_, cur.bins, nxt.bins,
-                             stride_, Q_, cur.g, nxt.g, cur.h, nxt.h, cur.rowid, nxt.rowid, d_split_,
-                             d_seg_[cur_state], d_pwork_, d_nwork_ + 1, d_excl_);
-        else
-          hipLaunchKernelGGL(k_partition<false>, dim3(pgrid), dim3(kPartThreads), 0, stream_, cur.bins, nxt.bins,
-                             stride_, Q_, cur.g, nxt.g, cur.h, nxt.h, cur.rowid, nxt.rowid, d_split_,
-                             d_seg_[cur_state], d_pwork_, d_nwork_ + 1, d_excl_);
-      } else {
+      if (last) {
+        Mark(kLeaf);
         const int blocks = (L + 127) / 128;
 #define ARB_LEAF(P, D) \
-  hipLaunchKernelGGL((k_leaf_weights<P, D>), dim3(blocks), dim3(128), 0, stream_, d_split_, d_tot_[cur_state], L, \
+  hipLaunchKernelGGL((k_leaf_weights<P, D>), dim3(blocks), dim3(128), 0, stream_, d_split_, d_tot_[state], L, \
                      d_shifts_, gp, cfg_.tree.eta, d_weights_)
         if (pair_ && f64_) ARB_LEAF(true, true);
         else if (pair_) ARB_LEAF(true, false);
         else if (f64_) ARB_LEAF(false, true);
         else ARB_LEAF(false, false);
 #undef ARB_LEAF
-        hipLaunchKernelGGL(k_leaf_assign, dim3(pgrid), dim3(kPartThreads), 0, stream_, cur.bins, stride_, cur.rowid,
-                           d_split_, d_pwork_, d_nwork_ + 1, d_leaf_);
-        hipLaunchKernelGGL(k_update_yhat, dim3(GridFor(n_, 256)), dim3(256), 0, stream_,
-                           d_yhat_ + (size_t)label * n_, d_leaf_, d_weights_, n_);
       }
-      cur_state ^= 1;
+      state ^= 1;
+    }
+    // ---- leaf of every row, y_hat update, gradients of the next round
+    Mark(kLeaf);
+    {
+      const int internal = (1 << (D_ - 1)) - 1;
+      const size_t lds = (size_t)internal * 2 * sizeof(int);
+      float *yh = d_yhat_ + (size_t)label * n_;
+      const int grid = GridFor(n_, 256, 8192);
+      const bool next_grad = !inspect_ && K_ == 1;
+      if (next_grad && cfg_.objective == kLinearRegression) {
+        HIP_OK(hipMemsetAsync(d_gmax_, 0, sizeof(unsigned), stream_));
+        hipLaunchKernelGGL(k_final<1>, dim3(grid), dim3(256), lds, stream_, dm_->bins, stride_, d_tfid_, d_tbin_, D_,
+                           d_weights_, yh, d_y_, d_leaf_, d_g_, d_h_, d_gmax_, n_);
+      } else if (next_grad && cfg_.objective == kLogisticRegression) {
+        hipLaunchKernelGGL(k_final<2>, dim3(grid), dim3(256), lds, stream_, dm_->bins, stride_, d_tfid_, d_tbin_, D_,
+                           d_weights_, yh, d_y_, d_leaf_, d_g_, d_h_, d_gmax_, n_);
+      } else {
+        if (cfg_.objective == kLinearRegression) HIP_OK(hipMemsetAsync(d_gmax_, 0, sizeof(unsigned), stream_));
+        hipLaunchKernelGGL(k_final<0>, dim3(grid), dim3(256), lds, stream_, dm_->bins, stride_, d_tfid_, d_tbin_, D_,
+                           d_weights_, yh, d_y_, d_leaf_, d_g_, d_h_, d_gmax_, n_);
+      }
+      grad_ready_ = next_grad;
     }
     Mark(kNone);
     HIP_OK(hipGetLastError());
@@ -1268,14 +1581,14 @@ class HipTreeBuilder : public TreeBuilder {
   DeviceMatrix *dm_;
   size_t n_ = 0, stride_ = 0;
   int F_ = 0, Q_ = 0, K_ = 1, D_ = 2, nbin_total_ = 0;
-  bool pair_ = false, f64_ = false, trick_ = true, inspect_ = false, timing_ = false;
+  bool pair_ = false, f64_ = false, trick_ = true, fused_ = false, inspect_ = false, timing_ = false;
+  bool grad_ready_ = false;
   int quads_per_group_ = 1;
-  size_t lds_bytes_ = 0;
   hipStream_t stream_ = nullptr;
   float *d_y_ = nullptr, *d_yhat_ = nullptr, *d_g_ = nullptr, *d_h_ = nullptr, *d_weights_ = nullptr, *d_tgain_ = nullptr;
   uint8_t *d_labels_ = nullptr;
   unsigned *d_leaf_ = nullptr, *d_node_first_ = nullptr, *d_node_items_ = nullptr, *d_nwork_ = nullptr,
-           *d_item_left_ = nullptr, *d_excl_ = nullptr, *d_gmax_ = nullptr;
+           *d_wave_left_ = nullptr, *d_excl_ = nullptr, *d_gmax_ = nullptr;
   RowBuffers buf_[2];
   NodeSum *d_tot_[2] = {nullptr, nullptr};
   unsigned *d_seg_[2] = {nullptr, nullptr};

@@ -272,6 +272,8 @@ const char *AGardenGetTimings(VoidPointer garden, double *out) {
     out[8] = (double)t.hist_root_launches;
     out[9] = (double)t.hist_root_rows;
     out[10] = (double)t.hist_deep_launches;
+    out[11] = t.fused_last;
+    out[12] = (double)t.fused_last_launches;
   });
 }
 const char *AGardenRowsScanned(VoidPointer garden, unsigned long long *out) {

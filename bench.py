@@ -8,9 +8,9 @@ matrix.  Prints ONE JSON line.
   value        row*feature histogram updates per second over the whole step
                (rows actually accumulated into histograms x 28 / step time)
   ms_per_step  milliseconds per tree
-  roofline     the histogram kernel (k_hist): algorithmic bytes of all its
-               launches / their summed duration (HIP events on the builder's
-               stream), against 8 TB/s
+  roofline     the dominant kernel (fused partition + histogram pass):
+               algorithmic bytes of its launches / their summed duration (HIP
+               events on the builder's stream), against 8 TB/s
   cpu_baseline the CPU checker (oracle/, OpenMP) on a bounded row sample of the
                same workload, timed on this host
 """
@@ -86,8 +86,8 @@ def main():
     ap.add_argument("--features", type=int, default=28)
     ap.add_argument("--max-depth", type=int, default=8)
     ap.add_argument("--hist-size", type=int, default=256)
-    ap.add_argument("--cpu-rows", type=int, default=2_000_000)
-    ap.add_argument("--cpu-trees", type=int, default=2)
+    ap.add_argument("--cpu-rows", type=int, default=10_500_000)
+    ap.add_argument("--cpu-trees", type=int, default=8)
     ap.add_argument("--no-cpu", action="store_true")
     args = ap.parse_args()
     if args.gpus != 1:
@@ -121,16 +121,26 @@ def main():
 
     F = args.features
     updates = scanned * F
-    launches = tm["hist_root_launches"] + tm["hist_deep_launches"]
-    hist_ms = tm["hist_root_ms"] + tm["hist_deep_ms"]
-    # algorithmic bytes of the histogram kernel: every scanned row reads F bin
-    # bytes and one (g,h) pair; every level writes its nodes' histograms once
-    # (16 B per (feature, bin) cell of the nodes built directly).
-    nodes_built = args.steps * (1 + sum(1 << (l - 1) for l in range(1, args.max_depth)))
-    hist_bytes = scanned * (F + 8) + nodes_built * F * 256 * 16
-    achieved = hist_bytes / (hist_ms * 1e-3)
-    root_bytes = tm["hist_root_rows"] * (F + 8) + args.steps * F * 256 * 16
-    root_achieved = root_bytes / (tm["hist_root_ms"] * 1e-3) if tm["hist_root_ms"] > 0 else 0.0
+    row_bytes = F + 8  # uint8 bins of all features + one (g, h) pair
+    cell_bytes = 16    # one histogram cell as written by a workgroup (two 64-bit words)
+    # Dominant kernel: the fused partition + histogram pass of levels 1..max_depth-2
+    # (k_part_hist<true, 7, true>).  Algorithmic bytes of one launch: every row is
+    # read once and written once in the children order, and the smaller child of
+    # each parent gets one histogram written.
+    fl = max(tm["hist_deep_launches"], 1)
+    parents = sum(1 << (l - 1) for l in range(1, args.max_depth - 1)) * args.steps
+    fused_bytes = fl * args.rows * 2 * row_bytes + parents * F * 256 * cell_bytes
+    fused_s = tm["hist_deep_ms"] * 1e-3
+    achieved = fused_bytes / fused_s if fused_s > 0 else 0.0
+    # root level (k_hist<true, 7>): reads every row, writes one histogram
+    root_bytes = tm["hist_root_rows"] * row_bytes + args.steps * F * 256 * cell_bytes
+    root_s = tm["hist_root_ms"] * 1e-3
+    # last level (k_part_hist<true, 7, false>): reads every row, moves none
+    last_bytes = tm["fused_last_launches"] * args.rows * row_bytes
+    last_s = tm["fused_last_ms"] * 1e-3
+
+    def frac(b, t):
+        return (b / t) / HBM_PEAK if t > 0 else 0.0
 
     out = {
         "metric": "row*feature hist updates/s + sec/tree at 10M x 28 depth 8; % of HBM peak",
@@ -152,13 +162,20 @@ def main():
                    "rows": args.rows, "features": F, "bins": args.hist_size, "max_depth": args.max_depth},
         "roofline": {"bound": "hbm", "achieved": achieved / 1e9, "peak": HBM_PEAK / 1e9, "unit": "GB/s",
                      "frac": achieved / HBM_PEAK, "traffic": None,
-                     "kernel": "k_hist<true>", "launches": int(launches),
-                     "avg_launch_us": hist_ms * 1e3 / max(launches, 1),
-                     "root_level": {"achieved": root_achieved / 1e9, "frac": root_achieved / HBM_PEAK,
-                                    "avg_launch_us": tm["hist_root_ms"] * 1e3 / max(tm["hist_root_launches"], 1),
-                                    "updates_per_s": tm["hist_root_rows"] * F / (tm["hist_root_ms"] * 1e-3)
-                                    if tm["hist_root_ms"] > 0 else 0.0}},
-        "tree_floor_frac_of_hbm": (2.9e9 / (dt / args.steps)) / HBM_PEAK,
+                     "kernel": "k_part_hist<true,7,true> (fused partition + histogram, levels 1..%d)"
+                               % (args.max_depth - 2),
+                     "launches": int(tm["hist_deep_launches"]),
+                     "avg_launch_us": tm["hist_deep_ms"] * 1e3 / fl,
+                     "bytes_per_launch": fused_bytes / fl},
+        "other_kernels": {
+            "k_hist<true,7> (root level)": {
+                "frac_of_hbm": frac(root_bytes, root_s),
+                "avg_launch_us": tm["hist_root_ms"] * 1e3 / max(tm["hist_root_launches"], 1),
+                "updates_per_s": tm["hist_root_rows"] * F / root_s if root_s > 0 else 0.0},
+            "k_part_hist<true,7,false> (last level)": {
+                "frac_of_hbm": frac(last_bytes, last_s),
+                "avg_launch_us": tm["fused_last_ms"] * 1e3 / max(tm["fused_last_launches"], 1)}},
+        "tree_algorithmic_floor_frac_of_hbm": (2.9e9 / (dt / args.steps)) / HBM_PEAK,
         "phase_ms_per_tree": {k: v / args.steps for k, v in tm.items() if k.endswith("_ms")},
         "quantise_s": t_quant,
     }

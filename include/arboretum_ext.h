@@ -55,10 +55,14 @@ const char *AGardenGetLevelHist(VoidPointer garden, int level, long long *out, i
 const char *AGardenGetShifts(VoidPointer garden, int *shift_g, int *shift_h);
 
 /* Device timings (HIP events on the builder's stream), accumulated since the
- * call that enabled them.  out[0..8] = milliseconds in: gradients, root
- * histogram kernel, deeper histogram kernels, slab reduce, split scan,
- * partition, leaf update, planning; out[8] = root histogram launches,
- * out[9] = rows read by them, out[10] = deeper histogram launches. */
+ * call that enabled them; `out` holds 16 doubles.  out[0..7] = milliseconds
+ * in: gradients, root histogram kernel, deeper-level histogram kernels (the
+ * fused partition + histogram kernel where it applies), slab reduce, split
+ * scan, partition bookkeeping (left counts, offset scan, stand-alone
+ * partition), leaf pass, planning; out[8] = root histogram launches, out[9] =
+ * rows read by them, out[10] = deeper-level histogram launches, out[11] =
+ * milliseconds in the fused kernel of the last level (it moves no rows),
+ * out[12] = its launches. */
 const char *AGardenEnableTiming(VoidPointer garden, int on);
 const char *AGardenGetTimings(VoidPointer garden, double *out);
 /* Rows accumulated into histograms so far (x ncol = histogram updates). */
