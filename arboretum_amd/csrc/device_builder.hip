@@ -484,10 +484,87 @@ __device__ __forceinline__ void WaveOffsets(const WorkItem &it, const SplitRec &
   *ro = start + (unsigned)s.left.c + (wb - start) - lefts_before;
 }
 
+__device__ __forceinline__ unsigned RankBelow(unsigned long long m) {
+  // number of set bits of m below this lane
+  return __builtin_amdgcn_mbcnt_hi((unsigned)(m >> 32), __builtin_amdgcn_mbcnt_lo((unsigned)m, 0u));
+}
+
+// Position of the k-th (0-based) set bit of the wave-uniform mask m; k < popcount(m).
+__device__ __forceinline__ int SelectBit(unsigned long long m, unsigned k) {
+  const unsigned lo = (unsigned)m, hi = (unsigned)(m >> 32);
+  unsigned c = (unsigned)__popc(lo);
+  const bool up = k >= c;
+  unsigned word = up ? hi : lo;
+  int pos = up ? 32 : 0;
+  k = up ? k - c : k;
+#pragma unroll
+  for (int width = 16; width >= 1; width >>= 1) {
+    const unsigned low = word & ((1u << width) - 1u);
+    c = (unsigned)__popc(low);
+    const bool u = k >= c;
+    word = u ? (word >> width) : low;
+    pos += u ? width : 0;
+    k = u ? k - c : k;
+  }
+  return pos;
+}
+
+// A wave's register-resident queue of rows waiting to be accumulated: one row
+// per lane.  LDS atomic instructions cost the same with one active lane as
+// with 64, so the rows selected for the histogram are first packed into full
+// waves with lane permutes.
+template <int NQ>
+struct Pending {
+  uint32_t b[NQ];
+  float g, h;
+};
+
+// Moves the rows of X flagged in xm (wave-uniform mask) into free lanes of P
+// (occupied lanes: pmask); when P is full it is accumulated and the rest of X
+// becomes the new P.
+template <bool PAIR, int NQ>
+__device__ __forceinline__ void MergePending(unsigned long long *__restrict__ lds, Pending<NQ> &P,
+                                             unsigned long long &pmask, const uint32_t (&xb)[NQ], float xg,
+                                             float xh, unsigned long long xm, int lane, int sg, int sh,
+                                             int F) {
+  const unsigned nx = (unsigned)__popcll(xm);
+  if (nx == 0) return;  // wave-uniform
+  const unsigned np = (unsigned)__popcll(pmask);
+  const unsigned moved = min(nx, 64u - np);
+  const unsigned long long holes = ~pmask;
+  const unsigned hr = RankBelow(holes);  // rank of this lane among the free lanes of P
+  const bool take = ((holes >> lane) & 1ull) && hr < moved;
+  const int src = take ? SelectBit(xm, hr) : lane;  // the hr-th row of X
+#pragma unroll
+  for (int q = 0; q < NQ; ++q) {
+    const uint32_t v = (uint32_t)__shfl((int)xb[q], src);
+    P.b[q] = take ? v : P.b[q];
+  }
+  {
+    const float v = __shfl(xg, src);
+    P.g = take ? v : P.g;
+  }
+  if (PAIR) {
+    const float v = __shfl(xh, src);
+    P.h = take ? v : P.h;
+  }
+  pmask |= __ballot(take);
+  if (np + moved == 64u) {  // wave-uniform: P is full
+    AccumulateRow<PAIR, NQ>(lds, P.b, P.g, P.h, sg, sh, 0, F);
+    const bool keep = ((xm >> lane) & 1ull) && RankBelow(xm) >= moved;
+#pragma unroll
+    for (int q = 0; q < NQ; ++q) P.b[q] = xb[q];
+    P.g = xg;
+    P.h = xh;
+    pmask = __ballot(keep);
+  }
+}
+
 // Fused pass over the rows of the parent nodes of a level: stable partition
 // into the children order (WRITE) and histogram of the smaller child of every
 // split in LDS.  Each wave owns a contiguous row range and runs without
-// workgroup barriers.  NQ = all quads of the matrix.
+// workgroup barriers; the rows of the next iteration are requested before the
+// current ones are processed.  NQ = all quads of the matrix.
 template <bool PAIR, int NQ, bool WRITE>
 __global__ void __launch_bounds__(kHistThreads)
 k_part_hist(const uint32_t *__restrict__ bins, uint32_t *__restrict__ bins_out, size_t stride, int F,
@@ -514,19 +591,49 @@ k_part_hist(const uint32_t *__restrict__ bins, uint32_t *__restrict__ bins_out, 
   unsigned lo = 0, ro = 0;
   if (WRITE) WaveOffsets(it, s, seg_start[it.node], excl, w, wave, wb, &lo, &ro);
   const int fq = s.fid >> 2, fs = 8 * (s.fid & 3);
-  const unsigned long long below = (1ull << lane) - 1ull;
-  for (unsigned base = wb; base < we; base += 128) {
-    const unsigned r0 = base + lane, r1 = r0 + 64;
-    const bool v0 = r0 < we, v1 = r1 < we;
-    const unsigned a0 = v0 ? r0 : wb, a1 = v1 ? r1 : wb;
-    uint32_t b0[NQ], b1[NQ];
+  Pending<NQ> P;
+#pragma unroll
+  for (int q = 0; q < NQ; ++q) P.b[q] = 0;
+  P.g = P.h = 0.0f;
+  unsigned long long pmask = 0;
+
+  uint32_t b0[NQ], b1[NQ];
+  float g0 = 0, g1 = 0, h0 = 0, h1 = 0;
+  if (wb < we) {
+    const unsigned a0 = min(wb + lane, we - 1), a1 = min(wb + 64 + lane, we - 1);
 #pragma unroll
     for (int q = 0; q < NQ; ++q) {
       b0[q] = bins[(size_t)q * stride + a0];
       b1[q] = bins[(size_t)q * stride + a1];
     }
-    const float g0 = g[a0], g1 = g[a1];
-    const float h0 = PAIR ? h[a0] : 0.0f, h1 = PAIR ? h[a1] : 0.0f;
+    g0 = g[a0];
+    g1 = g[a1];
+    if (PAIR) {
+      h0 = h[a0];
+      h1 = h[a1];
+    }
+  }
+  for (unsigned base = wb; base < we; base += 128) {
+    // rows of the next iteration
+    uint32_t nb0[NQ], nb1[NQ];
+    float ng0 = 0, ng1 = 0, nh0 = 0, nh1 = 0;
+    const unsigned next = base + 128;
+    if (next < we) {
+      const unsigned a0 = min(next + lane, we - 1), a1 = min(next + 64 + lane, we - 1);
+#pragma unroll
+      for (int q = 0; q < NQ; ++q) {
+        nb0[q] = bins[(size_t)q * stride + a0];
+        nb1[q] = bins[(size_t)q * stride + a1];
+      }
+      ng0 = g[a0];
+      ng1 = g[a1];
+      if (PAIR) {
+        nh0 = h[a0];
+        nh1 = h[a1];
+      }
+    }
+    const unsigned r0 = base + lane, r1 = r0 + 64;
+    const bool v0 = r0 < we, v1 = r1 < we;
     uint32_t s0 = 0, s1 = 0;
 #pragma unroll
     for (int q = 0; q < NQ; ++q) {
@@ -540,15 +647,14 @@ k_part_hist(const uint32_t *__restrict__ bins, uint32_t *__restrict__ bins_out, 
       const unsigned long long lm1 = __ballot(v1 && !right1), rm1 = __ballot(right1);
       const unsigned nl0 = (unsigned)__popcll(lm0), nr0 = (unsigned)__popcll(rm0);
       if (v0) {
-        const unsigned d = right0 ? ro + (unsigned)__popcll(rm0 & below) : lo + (unsigned)__popcll(lm0 & below);
+        const unsigned d = right0 ? ro + RankBelow(rm0) : lo + RankBelow(lm0);
 #pragma unroll
         for (int q = 0; q < NQ; ++q) bins_out[(size_t)q * stride + d] = b0[q];
         g_out[d] = g0;
         if (PAIR) h_out[d] = h0;
       }
       if (v1) {
-        const unsigned d = right1 ? ro + nr0 + (unsigned)__popcll(rm1 & below)
-                                  : lo + nl0 + (unsigned)__popcll(lm1 & below);
+        const unsigned d = right1 ? ro + nr0 + RankBelow(rm1) : lo + nl0 + RankBelow(lm1);
 #pragma unroll
         for (int q = 0; q < NQ; ++q) bins_out[(size_t)q * stride + d] = b1[q];
         g_out[d] = g1;
@@ -557,9 +663,19 @@ k_part_hist(const uint32_t *__restrict__ bins, uint32_t *__restrict__ bins_out, 
       lo += nl0 + (unsigned)__popcll(lm1);
       ro += nr0 + (unsigned)__popcll(rm1);
     }
-    if (v0 && right0 == build_right) AccumulateRow<PAIR, NQ>(lds, b0, g0, h0, sg, sh, 0, F);
-    if (v1 && right1 == build_right) AccumulateRow<PAIR, NQ>(lds, b1, g1, h1, sg, sh, 0, F);
+    MergePending<PAIR, NQ>(lds, P, pmask, b0, g0, h0, __ballot(v0 && right0 == build_right), lane, sg, sh, F);
+    MergePending<PAIR, NQ>(lds, P, pmask, b1, g1, h1, __ballot(v1 && right1 == build_right), lane, sg, sh, F);
+#pragma unroll
+    for (int q = 0; q < NQ; ++q) {
+      b0[q] = nb0[q];
+      b1[q] = nb1[q];
+    }
+    g0 = ng0;
+    g1 = ng1;
+    h0 = nh0;
+    h1 = nh1;
   }
+  if ((pmask >> lane) & 1ull) AccumulateRow<PAIR, NQ>(lds, P.b, P.g, P.h, sg, sh, 0, F);
   __syncthreads();
   FlushSlab<PAIR, NQ>(lds, slab, w, nbin_total, 0);
 }
@@ -1200,8 +1316,7 @@ class HipTreeBuilder : public TreeBuilder {
 
     // ping-pong row buffers in node order (not needed for a single split level)
     if (D_ > 2) {
-      const int nbuf = (fused_ && D_ == 3) ? 0 : 2;  // fused: the last level writes nothing
-      for (int b = 0; b < nbuf; ++b) {
+      for (int b = 0; b < 2; ++b) {
         buf_[b].bins = DevAlloc<uint32_t>((size_t)Q_ * stride_);
         buf_[b].g = DevAlloc<float>(n_);
         buf_[b].h = DevAlloc<float>(n_);
