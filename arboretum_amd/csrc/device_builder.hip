@@ -412,7 +412,7 @@ __device__ __forceinline__ bool GoesRight(const uint32_t *__restrict__ bins, siz
 __global__ void __launch_bounds__(kHistThreads)
 k_part_count(const uint32_t *__restrict__ bins, size_t stride, const SplitRec *__restrict__ split,
              const WorkItem *__restrict__ work, const unsigned *__restrict__ n_work,
-             unsigned *__restrict__ wave_left) {
+             unsigned *__restrict__ wave_left, unsigned *__restrict__ item_left) {
   const unsigned w = blockIdx.x;
   if (w >= *n_work) return;
   const WorkItem it = work[w];
@@ -430,56 +430,41 @@ k_part_count(const uint32_t *__restrict__ bins, size_t stride, const SplitRec *_
   }
   for (int off = 32; off > 0; off >>= 1) cnt += __shfl_down(cnt, off);
   if (lane == 0) wave_left[(size_t)w * kItemWaves + wave] = cnt;
+  // per-item total for the offset computation of later items of the node
+  __shared__ unsigned s_cnt[kItemWaves];
+  if (lane == 0) s_cnt[wave] = cnt;
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    unsigned t = 0;
+    for (int k = 0; k < kItemWaves; ++k) t += s_cnt[k];
+    item_left[w] = t;
+  }
 }
 
-// Exclusive scan of wave_left over all (item, wave) pairs.  One workgroup.
-__global__ void __launch_bounds__(1024)
-k_part_scan(const unsigned *__restrict__ wave_left, const unsigned *__restrict__ n_work,
-            unsigned *__restrict__ excl) {
-  __shared__ unsigned s_part[1024];
-  const unsigned n = *n_work * kItemWaves;
-  const unsigned per = (n + 1023) / 1024;
-  const unsigned b = min(n, threadIdx.x * per), e = min(n, b + per);
-  unsigned sum = 0;
-  for (unsigned i = b; i < e; ++i) sum += wave_left[i];
-  s_part[threadIdx.x] = sum;
+// Rows going left in the earlier work items of the same node and in the
+// earlier waves of this item.  Called by the whole workgroup; s_tmp holds
+// kItemWaves + 1 words.
+__device__ __forceinline__ unsigned LeftsBefore(const WorkItem &it, unsigned w, int wave,
+                                                const unsigned *__restrict__ wave_left,
+                                                const unsigned *__restrict__ item_left,
+                                                unsigned *s_tmp) {
+  unsigned part = 0;
+  for (unsigned k = it.first + threadIdx.x; k < w; k += blockDim.x) part += item_left[k];
+  for (int off = 32; off > 0; off >>= 1) part += __shfl_down(part, off);
+  if ((threadIdx.x & 63) == 0) s_tmp[threadIdx.x >> 6] = part;
   __syncthreads();
-  // exclusive scan of the 1024 partial sums by the first wave
-  if (threadIdx.x < 64) {
-    const int lane = threadIdx.x;
-    unsigned v[16], t = 0;
-#pragma unroll
-    for (int k = 0; k < 16; ++k) {
-      v[k] = s_part[lane * 16 + k];
-      t += v[k];
-    }
-    unsigned incl = t;
-    for (int off = 1; off < 64; off <<= 1) {
-      const unsigned o = __shfl_up(incl, off);
-      if (lane >= off) incl += o;
-    }
-    unsigned run = incl - t;
-#pragma unroll
-    for (int k = 0; k < 16; ++k) {
-      s_part[lane * 16 + k] = run;
-      run += v[k];
-    }
-  }
+  unsigned before = 0;
+  for (int k = 0; k < kItemWaves; ++k) before += s_tmp[k];
+  for (int k = 0; k < wave; ++k) before += wave_left[(size_t)w * kItemWaves + k];
   __syncthreads();
-  unsigned run = s_part[threadIdx.x];
-  for (unsigned i = b; i < e; ++i) {
-    excl[i] = run;
-    run += wave_left[i];
-  }
+  return before;
 }
 
 // Destination offsets of one wave range: rows going left are packed in order
 // from the start of the parent's range, rows going right from the start of
 // the right child's range (stable on both sides).
-__device__ __forceinline__ void WaveOffsets(const WorkItem &it, const SplitRec &s, unsigned start,
-                                            const unsigned *__restrict__ excl, unsigned w, int wave,
+__device__ __forceinline__ void WaveOffsets(const SplitRec &s, unsigned start, unsigned lefts_before,
                                             unsigned wb, unsigned *lo, unsigned *ro) {
-  const unsigned lefts_before = excl[(size_t)w * kItemWaves + wave] - excl[(size_t)it.first * kItemWaves];
   *lo = start + lefts_before;
   *ro = start + (unsigned)s.left.c + (wb - start) - lefts_before;
 }
@@ -572,9 +557,11 @@ k_part_hist(const uint32_t *__restrict__ bins, uint32_t *__restrict__ bins_out, 
             float *__restrict__ h_out, const int *__restrict__ shifts,
             const SplitRec *__restrict__ split, const NodeSum *__restrict__ tot,
             const unsigned *__restrict__ seg_start, const WorkItem *__restrict__ work,
-            const unsigned *__restrict__ n_work, const unsigned *__restrict__ excl,
-            unsigned long long *__restrict__ slab, int nbin_total) {
+            const unsigned *__restrict__ n_work, const unsigned *__restrict__ wave_left,
+            const unsigned *__restrict__ item_left, unsigned long long *__restrict__ slab,
+            int nbin_total) {
   extern __shared__ unsigned long long lds[];
+  __shared__ unsigned s_tmp[kItemWaves + 1];
   const unsigned w = blockIdx.x;
   if (w >= *n_work) return;
   const WorkItem it = work[w];
@@ -583,13 +570,16 @@ k_part_hist(const uint32_t *__restrict__ bins, uint32_t *__restrict__ bins_out, 
   const bool build_right = cl > cr;  // ties -> left (hist_grad_sum.cu:288-290)
   constexpr int words = NQ * 4 * kSlots * (PAIR ? 2 : 1);
   for (int i = threadIdx.x; i < words; i += kHistThreads) lds[i] = 0ull;
-  __syncthreads();
   const int sg = shifts[0], sh = shifts[1];
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   unsigned wb, we;
   WaveRange(it, wave, &wb, &we);
   unsigned lo = 0, ro = 0;
-  if (WRITE) WaveOffsets(it, s, seg_start[it.node], excl, w, wave, wb, &lo, &ro);
+  if (WRITE) {
+    const unsigned before = LeftsBefore(it, w, wave, wave_left, item_left, s_tmp);
+    WaveOffsets(s, seg_start[it.node], before, wb, &lo, &ro);
+  }
+  __syncthreads();
   const int fq = s.fid >> 2, fs = 8 * (s.fid & 3);
   Pending<NQ> P;
 #pragma unroll
@@ -688,7 +678,9 @@ k_partition(const uint32_t *__restrict__ bins, uint32_t *__restrict__ bins_out, 
             const float *__restrict__ g, float *__restrict__ g_out, const float *__restrict__ h,
             float *__restrict__ h_out, const SplitRec *__restrict__ split,
             const unsigned *__restrict__ seg_start, const WorkItem *__restrict__ work,
-            const unsigned *__restrict__ n_work, const unsigned *__restrict__ excl) {
+            const unsigned *__restrict__ n_work, const unsigned *__restrict__ wave_left,
+            const unsigned *__restrict__ item_left) {
+  __shared__ unsigned s_tmp[kItemWaves + 1];
   const unsigned w = blockIdx.x;
   if (w >= *n_work) return;
   const WorkItem it = work[w];
@@ -697,7 +689,8 @@ k_partition(const uint32_t *__restrict__ bins, uint32_t *__restrict__ bins_out, 
   unsigned wb, we;
   WaveRange(it, wave, &wb, &we);
   unsigned lo, ro;
-  WaveOffsets(it, s, seg_start[it.node], excl, w, wave, wb, &lo, &ro);
+  const unsigned before = LeftsBefore(it, w, wave, wave_left, item_left, s_tmp);
+  WaveOffsets(s, seg_start[it.node], before, wb, &lo, &ro);
   const unsigned long long below = (1ull << lane) - 1ull;
   for (unsigned base = wb; base < we; base += 64) {
     const unsigned r = base + lane;
@@ -978,7 +971,10 @@ __global__ void k_leaf_weights(const SplitRec *__restrict__ split, const NodeSum
 // to y_hat (update_by_last_tree, garden.cu:45-76) and, when NEXT_GRAD is not
 // 0, write the gradients of the next round (objective.cu:28-56):
 // 1 = squared (also max |g|), 2 = logistic.
-template <int NEXT_GRAD>
+// NQ > 0: the matrix has NQ quads, all loaded up front (coalesced, independent
+// loads) and selected in registers; NQ == 0: any width, one dependent 4-byte
+// load per level.
+template <int NEXT_GRAD, int NQ>
 __global__ void __launch_bounds__(256)
 k_final(const uint32_t *__restrict__ bins, size_t stride, const int *__restrict__ t_fid,
         const int *__restrict__ t_bin, int depth, const float *__restrict__ weights,
@@ -994,28 +990,40 @@ k_final(const uint32_t *__restrict__ bins, size_t stride, const int *__restrict_
   float m = 0.0f;
   for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < n;
        i += (size_t)gridDim.x * blockDim.x) {
+    uint32_t b[NQ > 0 ? NQ : 1];
+#pragma unroll
+    for (int q = 0; q < NQ; ++q) b[q] = bins[(size_t)q * stride + i];
+    const float yh0 = yhat[i];
+    const float yv = NEXT_GRAD != 0 ? y[i] : 0.0f;
     unsigned node = 0;
     for (int level = 0; level + 1 < depth; ++level) {
       const int id = (1 << level) - 1 + (int)node;
       const int fid = s_nodes[id], bin = s_nodes[internal + id];
       unsigned right = 0;
       if (bin >= 0) {
-        const uint32_t b4 = bins[(size_t)(fid >> 2) * stride + i];
+        uint32_t b4 = 0;
+        if (NQ > 0) {
+          const int fq = fid >> 2;
+#pragma unroll
+          for (int q = 0; q < NQ; ++q) b4 = q == fq ? b[q] : b4;
+        } else {
+          b4 = bins[(size_t)(fid >> 2) * stride + i];
+        }
         right = (int)((b4 >> (8 * (fid & 3))) & 255u) > bin ? 1u : 0u;
       }
       node = node * 2 + right;
     }
     leaf_of[i] = node;
-    const float yh = yhat[i] + weights[node];
+    const float yh = yh0 + weights[node];
     yhat[i] = yh;
     if (NEXT_GRAD == 1) {
-      const float v = y[i] - yh;
+      const float v = yv - yh;
       g[i] = v;
       const float a = fabsf(v);
       if (a > m) m = a;
     } else if (NEXT_GRAD == 2) {
       const float s = SigmoidF(yh);
-      g[i] = y[i] - s;
+      g[i] = yv - s;
       h[i] = s * (1.0f - s);
     }
   }
@@ -1244,7 +1252,8 @@ struct FusedArgs {
   const unsigned *seg_start;
   const WorkItem *work;
   const unsigned *n_work;
-  const unsigned *excl;
+  const unsigned *wave_left;
+  const unsigned *item_left;
   unsigned long long *slab;
   int nbin_total;
 };
@@ -1259,7 +1268,7 @@ void LaunchFusedNQ(hipStream_t st, unsigned grid, const FusedArgs &a) {
   }
   hipLaunchKernelGGL((k_part_hist<PAIR, NQ, WRITE>), dim3(grid), dim3(kHistThreads), lds, st, a.bins, a.bins_out,
                      a.stride, a.F, a.g, a.g_out, a.h, a.h_out, a.shifts, a.split, a.tot, a.seg_start, a.work,
-                     a.n_work, a.excl, a.slab, a.nbin_total);
+                     a.n_work, a.wave_left, a.item_left, a.slab, a.nbin_total);
 }
 
 template <bool PAIR, bool WRITE>
@@ -1341,7 +1350,7 @@ class HipTreeBuilder : public TreeBuilder {
     d_pwork_ = DevAlloc<WorkItem>(max_part_items_);
     d_nwork_ = DevAlloc<unsigned>(2);
     d_wave_left_ = DevAlloc<unsigned>((size_t)max_part_items_ * kItemWaves);
-    d_excl_ = DevAlloc<unsigned>((size_t)max_part_items_ * kItemWaves);
+    d_item_left_ = DevAlloc<unsigned>(max_part_items_);
     d_slab_ = DevAlloc<unsigned long long>((size_t)std::max(max_hist_items_, max_part_items_) * nbin_total_ * (pair_ ? 2 : 1));
     d_shifts_ = DevAlloc<int>(2);
     d_gmax_ = DevAlloc<unsigned>(1);
@@ -1363,7 +1372,7 @@ class HipTreeBuilder : public TreeBuilder {
   ~HipTreeBuilder() override {
     (void)hipStreamSynchronize(stream_);
     void *ptrs[] = {d_y_, d_labels_, d_yhat_, d_g_, d_h_, d_leaf_, d_split_, d_cand_, d_node_first_,
-                    d_node_items_, d_hwork_, d_pwork_, d_nwork_, d_wave_left_, d_excl_, d_slab_,
+                    d_node_items_, d_hwork_, d_pwork_, d_nwork_, d_wave_left_, d_item_left_, d_slab_,
                     d_shifts_, d_gmax_, d_rows_scanned_, d_tfid_, d_tbin_, d_tgain_, d_weights_};
     for (void *p : ptrs)
       if (p) (void)hipFree(p);
@@ -1560,12 +1569,11 @@ class HipTreeBuilder : public TreeBuilder {
           if (!last) {  // destination offsets; the last level moves no rows
             Mark(kPartition);
             hipLaunchKernelGGL(k_part_count, dim3(grid), dim3(kHistThreads), 0, stream_, src.bins, stride_, d_split_,
-                               d_pwork_, d_nwork_ + 1, d_wave_left_);
-            hipLaunchKernelGGL(k_part_scan, dim3(1), dim3(1024), 0, stream_, d_wave_left_, d_nwork_ + 1, d_excl_);
+                               d_pwork_, d_nwork_ + 1, d_wave_left_, d_item_left_);
           }
           Mark(last ? kFusedLast : kHistDeep);
           FusedArgs a{src.bins, dst.bins, stride_, F_, src.g, dst.g, src.h, dst.h, d_shifts_, d_split_,
-                      d_tot_[ps], d_seg_[ps], d_pwork_, d_nwork_ + 1, d_excl_, d_slab_, nbin_total_};
+                      d_tot_[ps], d_seg_[ps], d_pwork_, d_nwork_ + 1, d_wave_left_, d_item_left_, d_slab_, nbin_total_};
           if (pair_) {
             if (last) LaunchFused<true, false>(Q_, stream_, grid, a);
             else LaunchFused<true, true>(Q_, stream_, grid, a);
@@ -1581,16 +1589,15 @@ class HipTreeBuilder : public TreeBuilder {
           Plan(ps, PL, 0, kPartRows, d_pwork_, d_nwork_ + 1, false, nullptr, grid);
           Mark(kPartition);
           hipLaunchKernelGGL(k_part_count, dim3(grid), dim3(kHistThreads), 0, stream_, src.bins, stride_, d_split_,
-                             d_pwork_, d_nwork_ + 1, d_wave_left_);
-          hipLaunchKernelGGL(k_part_scan, dim3(1), dim3(1024), 0, stream_, d_wave_left_, d_nwork_ + 1, d_excl_);
+                             d_pwork_, d_nwork_ + 1, d_wave_left_, d_item_left_);
           if (pair_)
             hipLaunchKernelGGL(k_partition<true>, dim3(grid), dim3(kHistThreads), 0, stream_, src.bins, dst.bins,
                                stride_, Q_, src.g, dst.g, src.h, dst.h, d_split_, d_seg_[ps], d_pwork_,
-                               d_nwork_ + 1, d_excl_);
+                               d_nwork_ + 1, d_wave_left_, d_item_left_);
           else
             hipLaunchKernelGGL(k_partition<false>, dim3(grid), dim3(kHistThreads), 0, stream_, src.bins, dst.bins,
                                stride_, Q_, src.g, dst.g, src.h, dst.h, d_split_, d_seg_[ps], d_pwork_,
-                               d_nwork_ + 1, d_excl_);
+                               d_nwork_ + 1, d_wave_left_, d_item_left_);
           HistOfNodes(dst, state, L, trick_, trick_ ? n_ / 2 : n_, false);
           Reduce(L, hb, false, ps, trick_);
         }
@@ -1635,18 +1642,28 @@ class HipTreeBuilder : public TreeBuilder {
       float *yh = d_yhat_ + (size_t)label * n_;
       const int grid = GridFor(n_, 256, 8192);
       const bool next_grad = !inspect_ && K_ == 1;
-      if (next_grad && cfg_.objective == kLinearRegression) {
-        HIP_OK(hipMemsetAsync(d_gmax_, 0, sizeof(unsigned), stream_));
-        hipLaunchKernelGGL(k_final<1>, dim3(grid), dim3(256), lds, stream_, dm_->bins, stride_, d_tfid_, d_tbin_, D_,
-                           d_weights_, yh, d_y_, d_leaf_, d_g_, d_h_, d_gmax_, n_);
-      } else if (next_grad && cfg_.objective == kLogisticRegression) {
-        hipLaunchKernelGGL(k_final<2>, dim3(grid), dim3(256), lds, stream_, dm_->bins, stride_, d_tfid_, d_tbin_, D_,
-                           d_weights_, yh, d_y_, d_leaf_, d_g_, d_h_, d_gmax_, n_);
-      } else {
-        if (cfg_.objective == kLinearRegression) HIP_OK(hipMemsetAsync(d_gmax_, 0, sizeof(unsigned), stream_));
-        hipLaunchKernelGGL(k_final<0>, dim3(grid), dim3(256), lds, stream_, dm_->bins, stride_, d_tfid_, d_tbin_, D_,
-                           d_weights_, yh, d_y_, d_leaf_, d_g_, d_h_, d_gmax_, n_);
+      int mode = 0;
+      if (next_grad && cfg_.objective == kLinearRegression) mode = 1;
+      if (next_grad && cfg_.objective == kLogisticRegression) mode = 2;
+      if (cfg_.objective == kLinearRegression) HIP_OK(hipMemsetAsync(d_gmax_, 0, sizeof(unsigned), stream_));
+#define ARB_FINAL(M, N) \
+  hipLaunchKernelGGL((k_final<M, N>), dim3(grid), dim3(256), lds, stream_, dm_->bins, stride_, d_tfid_, d_tbin_, D_, \
+                     d_weights_, yh, d_y_, d_leaf_, d_g_, d_h_, d_gmax_, n_)
+#define ARB_FINAL_Q(N) \
+  do { if (mode == 1) ARB_FINAL(1, N); else if (mode == 2) ARB_FINAL(2, N); else ARB_FINAL(0, N); } while (0)
+      switch (Q_ <= 8 ? Q_ : 0) {
+        case 1: ARB_FINAL_Q(1); break;
+        case 2: ARB_FINAL_Q(2); break;
+        case 3: ARB_FINAL_Q(3); break;
+        case 4: ARB_FINAL_Q(4); break;
+        case 5: ARB_FINAL_Q(5); break;
+        case 6: ARB_FINAL_Q(6); break;
+        case 7: ARB_FINAL_Q(7); break;
+        case 8: ARB_FINAL_Q(8); break;
+        default: ARB_FINAL_Q(0); break;
       }
+#undef ARB_FINAL_Q
+#undef ARB_FINAL
       grad_ready_ = next_grad;
     }
     Mark(kNone);
@@ -1703,7 +1720,7 @@ class HipTreeBuilder : public TreeBuilder {
   float *d_y_ = nullptr, *d_yhat_ = nullptr, *d_g_ = nullptr, *d_h_ = nullptr, *d_weights_ = nullptr, *d_tgain_ = nullptr;
   uint8_t *d_labels_ = nullptr;
   unsigned *d_leaf_ = nullptr, *d_node_first_ = nullptr, *d_node_items_ = nullptr, *d_nwork_ = nullptr,
-           *d_wave_left_ = nullptr, *d_excl_ = nullptr, *d_gmax_ = nullptr;
+           *d_wave_left_ = nullptr, *d_item_left_ = nullptr, *d_gmax_ = nullptr;
   RowBuffers buf_[2];
   NodeSum *d_tot_[2] = {nullptr, nullptr};
   unsigned *d_seg_[2] = {nullptr, nullptr};
