@@ -1492,9 +1492,10 @@ class HipTreeBuilder : public TreeBuilder {
     event_used_ = 0;
   }
 
-  static unsigned HistRowsPerItem(size_t rows_max) {
-    // about 512 work items per level, whole 1024-row tiles, at most kMaxHistRows rows
-    size_t t = (rows_max + 511) / 512;
+  static unsigned HistRowsPerItem(size_t rows_max, size_t items = 512) {
+    // about `items` work items per level (512 = two per CU measured best for
+    // the fused pass), whole 1024-row tiles, at most kMaxHistRows rows
+    size_t t = (rows_max + items - 1) / items;
     t = (t + kHistThreads - 1) / kHistThreads * kHistThreads;
     return (unsigned)std::min<size_t>(std::max<size_t>(t, kHistThreads), kMaxHistRows);
   }
@@ -1508,7 +1509,8 @@ class HipTreeBuilder : public TreeBuilder {
 
   // Histograms of contiguous node ranges in `cur` (level order), feature group by group.
   void HistOfNodes(const RowBuffers &cur, int state, int L, bool select_smaller, size_t rows_max, bool root) {
-    const unsigned per_item = HistRowsPerItem(rows_max);
+    // the root level is one node: one item per CU avoids a second, partial round
+    const unsigned per_item = HistRowsPerItem(rows_max, root ? 256 : 512);
     const unsigned grid = (unsigned)std::min<size_t>(rows_max / per_item + L + 1, max_hist_items_);
     Mark(kPlan);
     Plan(state, L, select_smaller ? 1 : 0, per_item, d_hwork_, d_nwork_, true, nullptr, grid);

@@ -1,0 +1,170 @@
+"""CPU-side tests of the C-ABI library: it loads without a GPU, exports every
+symbol the headers declare, and its host-only entry points (configuration,
+model JSON, prediction) behave like the reference's."""
+import ctypes
+import json
+import os
+import re
+
+import numpy as np
+import pytest
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+LIB = os.path.join(ROOT, "arboretum_amd", "libarboretum.so")
+
+
+def declared_symbols():
+    names = []
+    for header in ("arboretum_wrapper.h", "arboretum_ext.h"):
+        text = open(os.path.join(ROOT, "include", header)).read()
+        text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+        names += re.findall(r"const char \*(A\w+)\(", text)
+    return names
+
+
+def test_library_exports_every_declared_symbol():
+    assert os.path.exists(LIB), "libarboretum.so is not built (python -m arboretum_amd.build)"
+    lib = ctypes.CDLL(LIB)
+    names = declared_symbols()
+    # the 14 entry points of python-wrapper/arboretum_wrapper.h:6-39
+    for ref in ["ACreateFromDenseMatrix", "ASetY", "ASetLabel", "ASetWeights", "AInitGarden", "AGrowTree",
+                "AAppendLastTree", "AGetY", "APredict", "ADumpModel", "ALoadModel", "AFreeDMatrix",
+                "AFreeGarden", "ADeleteArray"]:
+        assert ref in names
+    for n in names:
+        assert hasattr(lib, n), n
+
+
+@pytest.fixture(scope="module")
+def arb():
+    import arboretum_amd
+    return arboretum_amd
+
+
+def test_import_alias(arb):
+    import arboretum
+    assert arboretum.DMatrix is arb.DMatrix and arboretum.Garden is arb.Garden
+
+
+def test_configuration_round_trip(arb):
+    cfg = {"objective": 1, "method": 1,
+           "internals": {"double_precision": True, "compute_overlap": 3, "hist_size": 12, "seed": 7,
+                         "use_hist_subtraction_trick": False, "upload_features": False},
+           "tree": {"eta": 0.99999, "max_depth": 3, "gamma": 0.0, "min_child_weight": 2, "min_leaf_size": 2,
+                    "lambda": 0.0, "alpha": 0.5, "max_leaf_weight": 1.5, "gamma_absolute": 0.25},
+           "verbose": {"gpu": True}}
+    g = arb.Garden(cfg)
+    conf = json.loads(g.dump())["configuration"]
+    # float32 values print as the shortest double that round-trips (json_conversion.h / nlohmann)
+    assert conf["tree"]["eta"] == 0.9999899864196777
+    assert conf["tree"]["max_depth"] == 3 and conf["tree"]["min_leaf_size"] == 2
+    assert conf["tree"]["min_child_weight"] == 2.0 and conf["tree"]["alpha"] == 0.5
+    assert conf["tree"]["lambda"] == 0.0 and conf["tree"]["initial_y"] == 0.5 and conf["tree"]["labels_count"] == 1
+    assert conf["internals"] == {"compute_overlap": 3, "double_precision": True, "hist_size": 12, "seed": 7,
+                                 "upload_features": False, "use_hist_subtraction_trick": False}
+    assert conf["verbose"] == {"booster": False, "data": False, "gpu": True}
+    assert conf["method"] == 1 and conf["objective"] == 1
+    assert json.loads(g.dump())["model"] == []
+
+
+def test_defaults_follow_reference(arb):
+    conf = json.loads(arb.Garden({"objective": 0, "method": 1}).dump())["configuration"]
+    t, it = conf["tree"], conf["internals"]      # src/core/param.h:21-27,54-57
+    assert t["max_depth"] == 7 and t["min_child_weight"] == 1.0 and t["min_leaf_size"] == 1
+    assert t["lambda"] == 1.0 and t["alpha"] == 0.0 and t["initial_y"] == 0.5
+    assert abs(t["eta"] - 0.3) < 1e-7 and t["colsample_bytree"] == 1.0
+    assert it["hist_size"] == 255 and it["use_hist_subtraction_trick"] and it["upload_features"]
+    assert it["compute_overlap"] == 2 and it["seed"] == 0 and not it["double_precision"]
+
+
+@pytest.mark.parametrize("bad", ["{", "[1,2]", '{"tree": {"max_depth": "x"}}', '{"objective": 7}',
+                                 '{"tree": {"max_depth": 0}}', '{"tree": {"max_depth": 40}}'])
+def test_bad_configuration_is_an_error_string(arb, bad):
+    lib = ctypes.CDLL(LIB)
+    lib.AInitGarden.restype = ctypes.c_char_p
+    h = ctypes.c_void_p()
+    msg = lib.AInitGarden(bad.encode(), ctypes.byref(h))
+    assert msg is not None and len(msg) > 0
+
+
+def _golden(name):
+    with open(os.path.join(ROOT, "tests", "golden", name)) as f:
+        return json.load(f)
+
+
+def test_load_golden_model_and_predict_on_host(arb):
+    # model JSON of tests/py/test_hist_regregression.py; prediction is host code
+    fx = _golden("hist_regression_boston10.json")
+    X = np.array(fx["X"], np.float32)
+    data = arb.DMatrix(X, y=np.array(fx["y"], np.float32))
+    for name, case in fx["cases"].items():
+        true = case["true_model"]
+        for tree in true["model"]:
+            tree.setdefault("depth", case["max_depth"] + 1)   # the goldens predate the "depth" key
+        model = arb.load(json.dumps(true))
+        for i in range(case["trees"]):
+            assert np.allclose(model.predict(data, i + 1), case["true_values"][i]), name
+        again = json.loads(model.dump())
+        for tt, ct in zip(true["model"], again["model"]):
+            assert tt["nodes"] == ct["nodes"]
+            assert np.allclose(tt["weights"], ct["weights"], rtol=1e-6)
+        # n_rounds counts trees; 0 trees gives the initial value
+        assert np.allclose(model.predict(data, 0), 0.5)
+
+
+def test_load_golden_logistic_model(arb):
+    fx = _golden("hist_logistic_iris.json")
+    X = np.array(fx["X"], np.float32)
+    data = arb.DMatrix(X, y=(np.array(fx["target"]) != 2).astype(np.float32))
+    for name, case in fx["cases"].items():
+        true = case["true_model"]
+        for tree in true["model"]:
+            tree.setdefault("depth", case["max_depth"] + 1)
+        model = arb.load(json.dumps(true))
+        for i in range(case["trees"]):
+            assert np.allclose(model.predict(data, i + 1), case["true_values"][i]), name
+
+
+def test_append_last_tree_and_get_y(arb):
+    fx = _golden("hist_regression_boston10.json")
+    case = fx["cases"]["test_2trees_depth_2"]
+    true = case["true_model"]
+    for tree in true["model"]:
+        tree.setdefault("depth", 3)
+    model = arb.load(json.dumps(true))
+    ev = arb.DMatrix(np.array(fx["X"], np.float32))
+    model.append_last_tree(ev)       # adds the LAST tree to y_hat (starts from initial_y)
+    want = model.predict(ev, 2) - model.predict(ev, 1) + 0.5
+    assert np.allclose(model.get_y(ev), want, atol=1e-5)
+
+
+def test_null_threshold_loads_as_infinity(arb):
+    model = {"configuration": {"objective": 0, "method": 1, "tree": {"max_depth": 1}},
+             "model": [{"depth": 2, "weights": [1.5, -2.5],
+                        "nodes": [{"id": 0, "leaf": False, "left": 1, "right": 2, "threshold": None, "fid": 0},
+                                  {"id": 1, "leaf": True, "idx": 0}, {"id": 2, "leaf": True, "idx": 1}]}]}
+    g = arb.load(json.dumps(model))
+    X = np.array([[1.0], [np.nan], [np.inf]], np.float32)
+    # x < +INF is left; NaN and +INF go right (garden.h:79-86)
+    assert g.predict(arb.DMatrix(X)).tolist() == [2.0, -2.0, -2.0]
+    assert json.loads(g.dump())["model"][0]["nodes"][0]["threshold"] is None
+
+
+def test_training_without_gpu_fails_loudly(arb):
+    if arb.device_count() > 0:
+        pytest.skip("a GPU is present")
+    X = np.random.default_rng(0).normal(size=(20, 3)).astype(np.float32)
+    g = arb.Garden({"objective": 0, "method": 1, "tree": {"max_depth": 2}}, arb.DMatrix(X, y=X[:, 0]))
+    with pytest.raises(arb.ArboretumError, match="no HIP device"):
+        g.grow_tree()
+
+
+def test_errors(arb):
+    X = np.zeros((4, 2), np.float32)
+    with pytest.raises(ValueError):
+        arb.DMatrix(X, y=np.zeros(4), labels=np.zeros(4, np.uint8))
+    with pytest.raises(ValueError):
+        arb.DMatrix(np.zeros(4, np.float32))
+    g = arb.Garden({"objective": 0, "method": 1})
+    with pytest.raises(arb.ArboretumError):
+        g.load('{"no_model": 1}')
