@@ -41,6 +41,7 @@ def _load_lib():
         "ADeleteArray": [P(c_float)],
         # extensions (include/arboretum_ext.h)
         "ADeviceCount": [P(c_int)],
+        "ADeviceCopyProbe": [ctypes.c_ulonglong],
         "ACreateFromQuantized": [c_void_p, ctypes.c_longlong, c_int, P(c_void_p)],
         "AQuantize": [c_void_p, c_int],
         "AGetBins": [c_void_p, c_void_p],
@@ -77,6 +78,11 @@ def device_count():
     n = ctypes.c_int(0)
     _check(_LIB.ADeviceCount(ctypes.byref(n)))
     return n.value
+
+
+def copy_probe(nbytes):
+    """One device-to-device copy kernel of known size (profile calibration)."""
+    _check(_LIB.ADeviceCopyProbe(int(nbytes)))
 
 
 def _fptr(a):

@@ -110,6 +110,7 @@ void FreeDeviceMatrix(DeviceMatrix *m);
 void GetDeviceBins(const DataMatrix &data, uint8_t *out);  // row-major [rows][F]
 TreeBuilder *CreateTreeBuilder(const Configuration &cfg, DataMatrix *data);
 int DeviceCount();
+void CopyProbe(size_t bytes);
 
 class Garden {
  public:

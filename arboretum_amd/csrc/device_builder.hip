@@ -316,15 +316,12 @@ k_plan(const NodeSum *__restrict__ tot, const unsigned *__restrict__ seg_start, 
   }
 }
 
-// Row sub-range of one wave inside a work item: kItemWaves equal contiguous
-// pieces, each a multiple of 64 rows.
-__device__ __forceinline__ void WaveRange(const WorkItem &it, int wave, unsigned *b, unsigned *e) {
-  const unsigned rows = it.end - it.begin;
-  const unsigned per = ((rows + kItemWaves - 1) / kItemWaves + 63u) & ~63u;
-  const unsigned wb = min(it.begin + (unsigned)wave * per, it.end);
-  *b = wb;
-  *e = min(wb + per, it.end);
-}
+// Rows of a work item are dealt to its waves in chunks of kChunkRows
+// consecutive rows, round-robin: wave v takes chunks v, v + kItemWaves, ...  A
+// workgroup therefore streams one contiguous block of the item per step (good
+// DRAM page locality) while every wave still owns a fixed, countable row set.
+constexpr unsigned kChunkRows = 128;
+constexpr unsigned kChunkStep = kChunkRows * kItemWaves;
 
 // ---------------------------------------------------------------- histogram
 // Adds the four features of quad q (bins packed in b4) of one row.
@@ -418,15 +415,18 @@ k_part_count(const uint32_t *__restrict__ bins, size_t stride, const SplitRec *_
   const WorkItem it = work[w];
   const SplitRec s = split[it.node];
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-  unsigned wb, we;
-  WaveRange(it, wave, &wb, &we);
   unsigned cnt = 0;
   if (s.fid < 0) {
-    cnt = lane == 0 ? we - wb : 0;
+    for (unsigned base = it.begin + wave * kChunkRows; base < it.end; base += kChunkStep)
+      cnt += lane == 0 ? min(kChunkRows, it.end - base) : 0u;
   } else {
     const uint32_t *col = bins + (size_t)(s.fid >> 2) * stride;
     const int sh = 8 * (s.fid & 3);
-    for (unsigned r = wb + lane; r < we; r += 64) cnt += ((int)((col[r] >> sh) & 255u) > s.bin) ? 0u : 1u;
+    for (unsigned base = it.begin + wave * kChunkRows; base < it.end; base += kChunkStep) {
+      const unsigned r0 = base + lane, r1 = r0 + 64;
+      if (r0 < it.end) cnt += ((int)((col[r0] >> sh) & 255u) > s.bin) ? 0u : 1u;
+      if (r1 < it.end) cnt += ((int)((col[r1] >> sh) & 255u) > s.bin) ? 0u : 1u;
+    }
   }
   for (int off = 32; off > 0; off >>= 1) cnt += __shfl_down(cnt, off);
   if (lane == 0) wave_left[(size_t)w * kItemWaves + wave] = cnt;
@@ -460,13 +460,21 @@ __device__ __forceinline__ unsigned LeftsBefore(const WorkItem &it, unsigned w, 
   return before;
 }
 
-// Destination offsets of one wave range: rows going left are packed in order
-// from the start of the parent's range, rows going right from the start of
-// the right child's range (stable on both sides).
-__device__ __forceinline__ void WaveOffsets(const SplitRec &s, unsigned start, unsigned lefts_before,
-                                            unsigned wb, unsigned *lo, unsigned *ro) {
+// Number of rows of a work item dealt to the waves before `wave`.
+__device__ __forceinline__ unsigned RowsOfEarlierWaves(const WorkItem &it, int wave) {
+  const unsigned rows = it.end - it.begin;
+  const unsigned full = rows / kChunkStep, rem = rows % kChunkStep;  // full rounds, rows of the last partial round
+  return full * kChunkRows * (unsigned)wave + min(rem, kChunkRows * (unsigned)wave);
+}
+
+// Destination offsets of one wave: its rows going left are packed in order
+// from the start of the parent's range (after those of earlier items and
+// waves), its rows going right from the start of the right child's range.
+__device__ __forceinline__ void WaveOffsets(const WorkItem &it, const SplitRec &s, unsigned start,
+                                            unsigned lefts_before, int wave, unsigned *lo, unsigned *ro) {
+  const unsigned rows_before = (it.begin - start) + RowsOfEarlierWaves(it, wave);
   *lo = start + lefts_before;
-  *ro = start + (unsigned)s.left.c + (wb - start) - lefts_before;
+  *ro = start + (unsigned)s.left.c + rows_before - lefts_before;
 }
 
 __device__ __forceinline__ unsigned RankBelow(unsigned long long m) {
@@ -572,12 +580,11 @@ k_part_hist(const uint32_t *__restrict__ bins, uint32_t *__restrict__ bins_out, 
   for (int i = threadIdx.x; i < words; i += kHistThreads) lds[i] = 0ull;
   const int sg = shifts[0], sh = shifts[1];
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-  unsigned wb, we;
-  WaveRange(it, wave, &wb, &we);
+  const unsigned wb = it.begin + wave * kChunkRows, we = it.end;
   unsigned lo = 0, ro = 0;
   if (WRITE) {
     const unsigned before = LeftsBefore(it, w, wave, wave_left, item_left, s_tmp);
-    WaveOffsets(s, seg_start[it.node], before, wb, &lo, &ro);
+    WaveOffsets(it, s, seg_start[it.node], before, wave, &lo, &ro);
   }
   __syncthreads();
   const int fq = s.fid >> 2, fs = 8 * (s.fid & 3);
@@ -603,11 +610,11 @@ k_part_hist(const uint32_t *__restrict__ bins, uint32_t *__restrict__ bins_out, 
       h1 = h[a1];
     }
   }
-  for (unsigned base = wb; base < we; base += 128) {
+  for (unsigned base = wb; base < we; base += kChunkStep) {
     // rows of the next iteration
     uint32_t nb0[NQ], nb1[NQ];
     float ng0 = 0, ng1 = 0, nh0 = 0, nh1 = 0;
-    const unsigned next = base + 128;
+    const unsigned next = base + kChunkStep;
     if (next < we) {
       const unsigned a0 = min(next + lane, we - 1), a1 = min(next + 64 + lane, we - 1);
 #pragma unroll
@@ -686,15 +693,14 @@ k_partition(const uint32_t *__restrict__ bins, uint32_t *__restrict__ bins_out, 
   const WorkItem it = work[w];
   const SplitRec s = split[it.node];
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-  unsigned wb, we;
-  WaveRange(it, wave, &wb, &we);
   unsigned lo, ro;
   const unsigned before = LeftsBefore(it, w, wave, wave_left, item_left, s_tmp);
-  WaveOffsets(s, seg_start[it.node], before, wb, &lo, &ro);
+  WaveOffsets(it, s, seg_start[it.node], before, wave, &lo, &ro);
   const unsigned long long below = (1ull << lane) - 1ull;
-  for (unsigned base = wb; base < we; base += 64) {
+  for (unsigned chunk = it.begin + wave * kChunkRows; chunk < it.end; chunk += kChunkStep)
+  for (unsigned base = chunk; base < min(chunk + kChunkRows, it.end); base += 64) {
     const unsigned r = base + lane;
-    const bool valid = r < we;
+    const bool valid = r < it.end;
     const bool right = valid && GoesRight(bins, stride, s, r);
     const unsigned long long lm = __ballot(valid && !right), rm = __ballot(right);
     if (valid) {
@@ -1058,6 +1064,26 @@ struct DeviceMatrix {
   int F = 0, Q = 0;
   uint32_t *bins = nullptr;  // [Q][stride]
 };
+
+// Plain device-to-device copy of `bytes` bytes: a kernel of exactly known HBM
+// traffic, used to scale hardware traffic counters in profiles.
+__global__ void k_copy_probe(const uint4 *__restrict__ src, uint4 *__restrict__ dst, size_t n16) {
+  for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < n16; i += (size_t)gridDim.x * blockDim.x)
+    dst[i] = src[i];
+}
+
+void CopyProbe(size_t bytes) {
+  const size_t n16 = bytes / 16;
+  uint4 *src = nullptr, *dst = nullptr;
+  HIP_OK(hipMalloc((void **)&src, n16 * 16));
+  HIP_OK(hipMalloc((void **)&dst, n16 * 16));
+  HIP_OK(hipMemset(src, 1, n16 * 16));
+  HIP_OK(hipDeviceSynchronize());
+  hipLaunchKernelGGL(k_copy_probe, dim3(4096), dim3(256), 0, 0, src, dst, n16);
+  HIP_OK(hipDeviceSynchronize());
+  HIP_OK(hipFree(src));
+  HIP_OK(hipFree(dst));
+}
 
 int DeviceCount() {
   int n = 0;

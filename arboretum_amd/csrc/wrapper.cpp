@@ -177,6 +177,13 @@ const char *ADeviceCount(int *out) {
   return Guard([&] { *out = DeviceCount(); });
 }
 
+const char *ADeviceCopyProbe(unsigned long long bytes) {
+  return Guard([&] {
+    if (DeviceCount() <= 0) throw std::runtime_error("no HIP device available");
+    CopyProbe((size_t)bytes);
+  });
+}
+
 const char *ACreateFromQuantized(const unsigned char *bins, long long nrow, int ncol, VoidPointer *out) {
   return Guard([&] {
     if (!bins || !out || nrow <= 0 || ncol <= 0) throw std::runtime_error("bad arguments");

@@ -89,6 +89,9 @@ def main():
     ap.add_argument("--cpu-rows", type=int, default=10_500_000)
     ap.add_argument("--cpu-trees", type=int, default=8)
     ap.add_argument("--no-cpu", action="store_true")
+    ap.add_argument("--copy-probe", type=int, default=0, metavar="MiB",
+                    help="also run one device-to-device copy of this many MiB (a kernel of known traffic, "
+                         "used to scale the FETCH_SIZE / WRITE_SIZE counters of a rocprofv3 --pmc run)")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this build runs on one GPU only (no collectives, no sharding); use --gpus 1")
@@ -96,6 +99,9 @@ def main():
     import arboretum_amd as arb
     if arb.device_count() < 1:
         sys.exit("bench.py: no HIP device; the benchmark needs an MI355X")
+
+    if args.copy_probe:
+        arb.copy_probe(args.copy_probe << 20)
 
     X, y = make_workload(args.rows, args.features)
     cfg = config(args.max_depth, args.hist_size)

@@ -18,6 +18,11 @@ extern "C" {
 /* Number of HIP devices visible (0 on a CPU-only host). */
 const char *ADeviceCount(int *out);
 
+/* Runs one plain device-to-device copy kernel (k_copy_probe) of `bytes` bytes:
+ * a dispatch of exactly known HBM traffic, against which the FETCH_SIZE /
+ * WRITE_SIZE counters of a profile are scaled. */
+const char *ADeviceCopyProbe(unsigned long long bytes);
+
 /* Data matrix from bin ids: `bins` row-major uint8 [nrow][ncol], copied.
  * Thresholds are reported as bin + 0.5 and prediction walks the bin ids.
  * Counterpart of the reference's quantised columns (src/io/io.h:65-76), which
