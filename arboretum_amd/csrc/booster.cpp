@@ -114,13 +114,11 @@ void Garden::GrowTree(DataMatrix *data, const float *grad) {
     throw std::runtime_error("y is not set");
   }
   // colsample checks of InitGrowingTree, garden.cu:126-140
-  const size_t columns = data->columns_dense;
+  const size_t columns = data->columns_dense + data->columns_category;
   if ((int)(cfg.tree.colsample_bytree * columns) == 0)
     throw std::runtime_error("colsample_bytree is too small");
   if ((int)(cfg.tree.colsample_bytree * cfg.tree.colsample_bylevel * columns) == 0)
     throw std::runtime_error("colsample_bytree and colsample_bylevel are too small");
-  if ((size_t)(cfg.tree.colsample_bytree * cfg.tree.colsample_bylevel * columns) != columns)
-    throw std::runtime_error("column sampling below 1.0 is not implemented");
   if (DeviceCount() <= 0) throw std::runtime_error("no HIP device available: training needs an MI355X");
   if (!builder_) {
     QuantiseOnDevice(data, cfg.internal.hist_size, cfg.verbose.data);

@@ -43,6 +43,7 @@
 #include <cstdio>
 #include <cstring>
 #include <limits>
+#include <random>
 #include <stdexcept>
 #include <string>
 #include <thread>
@@ -902,15 +903,17 @@ k_split_scan(const long long *__restrict__ hg, const long long *__restrict__ hh,
   if (lane == 0) cand[(size_t)nd * F + f] = best;
 }
 
-// One thread per node: best candidate over features (higher gain, then lower
-// feature id: hist_tree_grower.cu:59-60), children totals and row ranges,
-// node record.  A node without a candidate keeps every row left.
+// One thread per node: best candidate over the features active at this level
+// (higher gain, then lower feature id: hist_tree_grower.cu:59-60), children
+// totals and row ranges, node record.  A node without a candidate keeps every
+// row left.
 __global__ void k_split_select(const Cand *__restrict__ cand, int F, int L,
                                const NodeSum *__restrict__ tot,
                                const unsigned *__restrict__ seg_start,
                                NodeSum *__restrict__ tot_next, unsigned *__restrict__ seg_next,
                                SplitRec *__restrict__ split, int *__restrict__ t_fid,
-                               int *__restrict__ t_bin, float *__restrict__ t_gain, int heap_off) {
+                               int *__restrict__ t_bin, float *__restrict__ t_gain, int heap_off,
+                               const unsigned char *__restrict__ active) {
   const int nd = blockIdx.x * blockDim.x + threadIdx.x;
   if (nd >= L) return;
   const NodeSum t = tot[nd];
@@ -922,6 +925,7 @@ __global__ void k_split_select(const Cand *__restrict__ cand, int F, int L,
   rec.left = t;
   if (t.c != 0) {
     for (int f = 0; f < F; ++f) {
+      if (active && !active[f]) continue;  // feature not sampled at this level
       const Cand c = cand[(size_t)nd * F + f];
       if (c.bin >= 0 && (rec.fid < 0 || rec.gain < c.gain)) {
         rec.gain = c.gain;
@@ -1388,6 +1392,8 @@ class HipTreeBuilder : public TreeBuilder {
     d_tbin_ = DevAlloc<int>(internal);
     d_tgain_ = DevAlloc<float>(internal);
     d_weights_ = DevAlloc<float>(max_nodes);
+    d_active_ = DevAlloc<unsigned char>((size_t)(D_ - 1) * F_);
+    rnd_.seed(cfg.internal.seed);  // garden.cu:87
     int shifts[2] = {30, 0};
     if (cfg.objective == kLogisticRegression) shifts[1] = 32;  // 0 <= h <= 1/4
     if (cfg.objective >= kSoftMaxOneVsAll) shifts[1] = 31;     // 0 <= h <= 1/2
@@ -1399,7 +1405,7 @@ class HipTreeBuilder : public TreeBuilder {
     (void)hipStreamSynchronize(stream_);
     void *ptrs[] = {d_y_, d_labels_, d_yhat_, d_g_, d_h_, d_leaf_, d_split_, d_cand_, d_node_first_,
                     d_node_items_, d_hwork_, d_pwork_, d_nwork_, d_wave_left_, d_item_left_, d_slab_,
-                    d_shifts_, d_gmax_, d_rows_scanned_, d_tfid_, d_tbin_, d_tgain_, d_weights_};
+                    d_shifts_, d_gmax_, d_rows_scanned_, d_tfid_, d_tbin_, d_tgain_, d_weights_, d_active_};
     for (void *p : ptrs)
       if (p) (void)hipFree(p);
     for (int b = 0; b < 2; ++b) {
@@ -1572,6 +1578,7 @@ class HipTreeBuilder : public TreeBuilder {
     orig.g = d_g_ + (size_t)label * n_;
     orig.h = d_h_ + (size_t)label * n_;
     if (inspect_) kept_hist_.assign(D_ - 1, {});
+    SampleColumns();
 
     hipLaunchKernelGGL(k_init_root, dim3(1), dim3(64), 0, stream_, d_tot_[0], d_seg_[0],
                        (unsigned long long)n_, (unsigned *)nullptr);
@@ -1646,7 +1653,8 @@ class HipTreeBuilder : public TreeBuilder {
 #undef ARB_SCAN
         hipLaunchKernelGGL(k_split_select, dim3((L + 127) / 128), dim3(128), 0, stream_, d_cand_, F_, L,
                            d_tot_[state], d_seg_[state], d_tot_[state ^ 1], d_seg_[state ^ 1], d_split_,
-                           d_tfid_, d_tbin_, d_tgain_, L - 1);
+                           d_tfid_, d_tbin_, d_tgain_, L - 1,
+                           sampling_ ? d_active_ + (size_t)level * F_ : (const unsigned char *)nullptr);
       }
       if (last) {
         Mark(kLeaf);
@@ -1714,6 +1722,30 @@ class HipTreeBuilder : public TreeBuilder {
     }
   }
 
+  // Column sampling of one tree (InitGrowingTree / InitTreeLevel,
+  // garden.cu:126-165, and the `take` prefix of FindBestSplits, :249-253): the
+  // ids are shuffled per tree, the first floor(bytree * columns) of them again
+  // per level, and the first floor(bylevel * bytree * columns) are active.
+  void SampleColumns() {
+    const size_t columns = data_->columns_dense + data_->columns_category;
+    const int take_tree = (int)(cfg_.tree.colsample_bytree * columns);
+    const unsigned take_level = (unsigned)(cfg_.tree.colsample_bylevel * cfg_.tree.colsample_bytree * columns);
+    sampling_ = take_level < columns;
+    if (!sampling_) return;
+    std::vector<unsigned> ids(columns);
+    for (size_t i = 0; i < columns; ++i) ids[i] = (unsigned)i;
+    std::shuffle(ids.begin(), ids.end(), rnd_);
+    active_host_.assign((size_t)(D_ - 1) * F_, 0);
+    for (int level = 0; level + 1 < D_; ++level) {
+      std::shuffle(ids.begin(), ids.begin() + take_tree, rnd_);
+      for (unsigned j = 0; j < take_level; ++j)
+        if (ids[j] < (unsigned)F_) active_host_[(size_t)level * F_ + ids[j]] = 1;
+    }
+    // the previous tree's kernels may still read the mask
+    HIP_OK(hipStreamSynchronize(stream_));
+    HIP_OK(hipMemcpy(d_active_, active_host_.data(), active_host_.size(), hipMemcpyHostToDevice));
+  }
+
   void KeepHist(int level, int L, int hb) {
     const size_t cells = (size_t)L * nbin_total_;
     std::vector<long long> g(cells), h(cells);
@@ -1747,6 +1779,10 @@ class HipTreeBuilder : public TreeBuilder {
   hipStream_t stream_ = nullptr;
   float *d_y_ = nullptr, *d_yhat_ = nullptr, *d_g_ = nullptr, *d_h_ = nullptr, *d_weights_ = nullptr, *d_tgain_ = nullptr;
   uint8_t *d_labels_ = nullptr;
+  unsigned char *d_active_ = nullptr;  // [level][feature] 1 = sampled at that level
+  std::vector<unsigned char> active_host_;
+  std::default_random_engine rnd_;
+  bool sampling_ = false;
   unsigned *d_leaf_ = nullptr, *d_node_first_ = nullptr, *d_node_items_ = nullptr, *d_nwork_ = nullptr,
            *d_wave_left_ = nullptr, *d_item_left_ = nullptr, *d_gmax_ = nullptr;
   RowBuffers buf_[2];

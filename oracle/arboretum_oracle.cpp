@@ -43,6 +43,7 @@
 #include <cstdio>
 #include <cstring>
 #include <limits>
+#include <random>
 #include <vector>
 #ifdef _OPENMP
 #include <omp.h>
@@ -69,6 +70,9 @@ struct OrcParams {
   int use_trick;          // sibling subtraction (param.h:55)
   int labels_count;
   int threads;            // OpenMP threads for the histogram loop (0 = default)
+  float colsample_bytree;
+  float colsample_bylevel;
+  unsigned seed;
 };
 
 // ------------------------------------------------------------------- exp
@@ -358,6 +362,7 @@ struct Booster {
   std::vector<std::vector<Acc>> lvl_hist;  // [level][node*F*slots + f*slots + b]
   std::vector<std::vector<Acc>> lvl_tot;   // [level][node]
   int shift_g = 30, shift_h = 32;
+  std::default_random_engine rnd;  // garden.cu:87, seeded with internals.seed
   uint64_t updates = 0;  // rows*features actually accumulated (work counter)
   int kind() const { return (p.objective == 0 ? 0 : 2) + (p.double_precision ? 1 : 0); }
 };
@@ -505,6 +510,18 @@ static void grow_tree(Booster &b, int label) {
   t.gain.assign(n_internal, 0.0f);
   t.weights.assign((size_t)1 << (D - 1), 0.0f);
 
+  // column sampling: InitGrowingTree (garden.cu:142-146) shuffles all ids once
+  // per tree, InitTreeLevel (:162-165) reshuffles the first
+  // int(colsample_bytree * columns) per level, and FindBestSplits (:252-253,
+  // 309-310) takes the first unsigned(bylevel * bytree * columns) as active.
+  // Parity with the reference's random stream is unpinned (it depends on the
+  // standard library's shuffle); with both ratios 1.0 every feature is active.
+  std::vector<unsigned> active_fids(F);
+  for (int f = 0; f < F; ++f) active_fids[f] = f;
+  std::shuffle(active_fids.begin(), active_fids.end(), b.rnd);
+  const int take_tree = (int)(b.p.colsample_bytree * (size_t)F);
+  const unsigned take_level = (unsigned)(b.p.colsample_bylevel * b.p.colsample_bytree * (size_t)F);
+
   std::vector<uint32_t> node(n, 0);
   b.lvl_hist.assign(D - 1, {});
   b.lvl_tot.assign(D - 1, {});
@@ -523,6 +540,9 @@ static void grow_tree(Booster &b, int label) {
 
   for (int level = 0; level + 1 < D; ++level) {
     const int L = 1 << level;
+    std::shuffle(active_fids.begin(), active_fids.begin() + take_tree, b.rnd);
+    std::vector<uint8_t> is_active(F, 0);
+    for (unsigned j = 0; j < take_level && j < (unsigned)F; ++j) is_active[active_fids[j]] = 1;
     std::vector<Acc> &hist = b.lvl_hist[level];
     hist.assign((size_t)L * F * SL, Acc());
     b.lvl_tot[level] = tot;
@@ -606,6 +626,7 @@ static void grow_tree(Booster &b, int label) {
       double GT, HT;
       acc_value(b, tot[nd], GT, HT);
       for (int f = 0; f < F; ++f) {
+        if (!is_active[f]) continue;
         const Acc *hf = &hist[((size_t)nd * F + f) * SL];
         Acc run;
         float cg = 0.0f;
@@ -793,6 +814,7 @@ void *orc_create(const float *X, int64_t n, int F, const float *y, const uint8_t
       b->bins[(size_t)i * F + f] = (uint16_t)bin_of(q.thr.data(), q.size, col[i]);
   }
   b->yhat.assign((size_t)n * p->labels_count, into_internal(p->objective, p->initial_y));
+  b->rnd.seed(p->seed);
   return b;
 }
 
@@ -813,6 +835,7 @@ void *orc_create_binned(const uint8_t *bins, int64_t n, int F, const float *y,
   b->bins.resize((size_t)n * F);
   for (size_t k = 0; k < (size_t)n * F; ++k) b->bins[k] = bins[k];
   b->yhat.assign((size_t)n * p->labels_count, into_internal(p->objective, p->initial_y));
+  b->rnd.seed(p->seed);
   return b;
 }
 

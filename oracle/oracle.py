@@ -29,6 +29,9 @@ class OrcParams(ctypes.Structure):
         ("use_trick", ctypes.c_int),
         ("labels_count", ctypes.c_int),
         ("threads", ctypes.c_int),
+        ("colsample_bytree", ctypes.c_float),
+        ("colsample_bylevel", ctypes.c_float),
+        ("seed", ctypes.c_uint),
     ]
 
 
@@ -125,6 +128,9 @@ def params_from_config(config, accum=0, threads=0):
         use_trick=int(bool(it.get("use_hist_subtraction_trick", True))),
         labels_count=int(t.get("labels_count", 1)),
         threads=threads,
+        colsample_bytree=float(t.get("colsample_bytree", 1.0)),
+        colsample_bylevel=float(t.get("colsample_bylevel", 1.0)),
+        seed=int(it.get("seed", 0)),
     )
 
 

@@ -150,6 +150,30 @@ def test_constant_features_give_unsplit_nodes(arb, oracle):
     assert all(n["threshold"] is None for n in model["model"][0]["nodes"] if not n["leaf"])
 
 
+@pytest.mark.parametrize("bytree,bylevel,seed", [(0.5, 1.0, 0), (1.0, 0.6, 3), (0.7, 0.7, 11)])
+def test_column_sampling(arb, oracle, bytree, bylevel, seed):
+    # same shuffle stream on both sides (std::shuffle + std::default_random_engine(seed),
+    # src/core/garden.cu:87,126-165); parity with the reference's stream is unpinned
+    X, y = make_data(8000, 12, 1, seed=6)
+    cfg = {"objective": 1, "method": 1, "internals": {"hist_size": 32, "double_precision": True, "seed": seed},
+           "tree": {"max_depth": 4, "eta": 0.3, "lambda": 1.0, "colsample_bytree": bytree,
+                    "colsample_bylevel": bylevel}}
+    ob, g = assert_same_training(arb, oracle, X, y, cfg, rounds=4, check_hist=False)
+    used = set()
+    for t in range(4):
+        tr = g.tree(t)
+        used |= set(tr["fid"][tr["quantized"] >= 0].tolist())
+    assert len(used) > 1
+
+
+def test_column_sampling_too_small_is_an_error(arb):
+    X, y = make_data(100, 3, 0, seed=1)
+    for tree in ({"colsample_bytree": 0.1}, {"colsample_bytree": 0.5, "colsample_bylevel": 0.5}):
+        g = arb.Garden({"objective": 0, "method": 1, "tree": dict(tree, max_depth=2)}, arb.DMatrix(X, y=y))
+        with pytest.raises(arb.ArboretumError, match="too small"):
+            g.grow_tree()
+
+
 def test_softmax_matches_oracle(arb, oracle):
     # Parity unpinned against the reference (its soft-max kernel is empty,
     # src/core/objective.cu:91-100); the oracle restates the formula left in the
