@@ -104,6 +104,12 @@ class TreeBuilder {
   virtual void Synchronize() = 0;
 };
 
+// quantiser.hip: thresholds of one column by a device radix sort
+struct SortWorkspace;
+SortWorkspace *CreateSortWorkspace(size_t n, int hist_size);
+void FreeSortWorkspace(SortWorkspace *ws);
+void DeviceThresholds(SortWorkspace *ws, const float *d_col, std::vector<float> *thr, int *size, bool *has_nan);
+
 // device_builder.hip
 void QuantiseOnDevice(DataMatrix *data, int hist_size, bool verbose);
 void FreeDeviceMatrix(DeviceMatrix *m);

@@ -22,6 +22,7 @@
 //
 // What replaces what (reference file:line):
 //   k_bin_assign      build_histogram              src/io/io.cu:293-312
+//                     (thresholds: quantiser.hip)
 //   k_grad_*          update_grad                  src/core/objective.cu:15-56
 //   k_root_from_hist  cub::DeviceReduce::Sum       src/core/garden.cu:432-435
 //   k_hist            hist_sum_node / hist_sum_multi_node
@@ -1101,30 +1102,6 @@ void FreeDeviceMatrix(DeviceMatrix *m) {
   delete m;
 }
 
-// Thresholds of one column, from the sorted column: the k-th change of value
-// at sorted position i writes its midpoint to slot min(k+1, i/seg+1) - 2,
-// lowest midpoint wins (src/io/io.cu:349-410, 255-270, 27-153).
-static void ThresholdsFromSorted(const std::vector<float> &s, int hist_size, std::vector<float> *thr,
-                                 int *size) {
-  const size_t n = s.size();
-  thr->assign(hist_size, std::numeric_limits<float>::infinity());
-  unsigned seg = (unsigned)(n / (size_t)hist_size);
-  if (seg < 1) seg = 1;
-  unsigned k = 0;
-  for (size_t i = 1; i < n; ++i) {
-    if (s[i] != s[i - 1]) {
-      ++k;
-      const float mid = (float)((double)(float)(s[i] + s[i - 1]) * 0.5);
-      const long long slot = (long long)std::min<unsigned long long>(k + 1ull, i / seg + 1ull) - 2;
-      if (slot >= 0 && slot < hist_size && mid < (*thr)[slot]) (*thr)[slot] = mid;
-    }
-  }
-  int unique = 0;
-  while (unique < hist_size && !std::isinf((*thr)[unique])) ++unique;
-  ++unique;
-  *size = std::min(unique, hist_size);
-}
-
 void QuantiseOnDevice(DataMatrix *data, int hist_size, bool verbose) {
   if (data->quantised) {
     if (data->hist_size != hist_size) throw std::runtime_error("data matrix was quantised with another hist_size");
@@ -1157,35 +1134,8 @@ void QuantiseOnDevice(DataMatrix *data, int hist_size, bool verbose) {
     HIP_OK(hipDeviceSynchronize());
     HIP_OK(hipFree(d_in));
   } else {
-    // thresholds: host sort per column (NaN last), columns in parallel
-    std::vector<char> has_nan(F, 0);
-    {
-      std::vector<std::thread> th;
-      unsigned hw = std::thread::hardware_concurrency();
-      const int nt = std::max(1, std::min<int>(hw ? hw : 1, std::min(F, 16)));
-      std::atomic<int> next{0};
-      for (int t = 0; t < nt; ++t)
-        th.emplace_back([&] {
-          std::vector<float> s;
-          for (;;) {
-            const int f = next.fetch_add(1);
-            if (f >= F) break;
-            s = data->data[f];
-            auto mid = std::partition(s.begin(), s.end(), [](float v) { return v == v; });
-            has_nan[f] = mid != s.end();
-            std::sort(s.begin(), mid);
-            ThresholdsFromSorted(s, hist_size, &data->thresholds[f], &data->reduced_size[f]);
-          }
-        });
-      for (auto &t : th) t.join();
-    }
-    for (int f = 0; f < F; ++f) {
-      if (data->reduced_size[f] + (has_nan[f] ? 1 : 0) > kSlots)
-        throw std::runtime_error("a feature needs more than 256 bin ids: 16-bit bins are not implemented");
-      if (verbose)
-        printf("feature %d has been reduced to %d bits \n", f,
-               32 - __builtin_clz((unsigned)data->reduced_size[f]));
-    }
+    // per quad: upload four columns, thresholds by device sort, bin assignment
+    std::unique_ptr<SortWorkspace, void (*)(SortWorkspace *)> ws(CreateSortWorkspace(n, hist_size), FreeSortWorkspace);
     float *d_x = DevAlloc<float>(4 * n);
     float *d_thr = DevAlloc<float>(4 * (size_t)hist_size);
     int *d_size = DevAlloc<int>(4);
@@ -1195,6 +1145,13 @@ void QuantiseOnDevice(DataMatrix *data, int hist_size, bool verbose) {
       for (int c = 0; c < nc; ++c) {
         const int f = q * 4 + c;
         HIP_OK(hipMemcpy(d_x + (size_t)c * n, data->data[f].data(), n * sizeof(float), hipMemcpyHostToDevice));
+        bool has_nan = false;
+        DeviceThresholds(ws.get(), d_x + (size_t)c * n, &data->thresholds[f], &data->reduced_size[f], &has_nan);
+        if (data->reduced_size[f] + (has_nan ? 1 : 0) > kSlots)
+          throw std::runtime_error("a feature needs more than 256 bin ids: 16-bit bins are not implemented");
+        if (verbose)
+          printf("feature %d has been reduced to %d bits \n", f,
+                 32 - __builtin_clz((unsigned)data->reduced_size[f]));
         HIP_OK(hipMemcpy(d_thr + (size_t)c * hist_size, data->thresholds[f].data(),
                          hist_size * sizeof(float), hipMemcpyHostToDevice));
         sizes[c] = data->reduced_size[f];

@@ -79,6 +79,49 @@ def assert_same_training(arb, oracle, X, y, cfg, rounds, check_hist=True):
     return ob, g
 
 
+# ---------------------------------------------------------------- quantiser
+@pytest.mark.parametrize("case", load_golden("quantiser.json"), ids=lambda c: c["name"])
+def test_quantiser_reference_goldens(arb, case):
+    # tests/cpp/test_datamatrix.cu:25-197 through the device sort + bin assignment
+    x = np.array(case["x"], np.float32).reshape(-1, 1)
+    data = arb.DMatrix(x)
+    data.quantize(case["hist_size"])
+    assert data.bins()[:, 0].tolist() == case["bins"]
+    thr, size = data.thresholds(0, case["hist_size"])
+    assert int(size).bit_length() == case["bits"]
+    if case.get("first_threshold_inf"):
+        assert np.isinf(thr[0])
+
+
+def _columns_for_quantiser(n, rng):
+    cols = [
+        rng.normal(size=n),                                   # continuous
+        np.exp(rng.normal(size=n)),                           # skewed
+        rng.integers(0, 7, size=n).astype(np.float64),        # few distinct values
+        np.round(rng.normal(size=n) * 20) / 20,               # many ties
+        np.where(rng.random(n) < 0.3, np.nan, rng.random(n)), # 30 % NaN
+        np.concatenate([np.arange(n // 20), np.full(n - n // 20 - n // 2, n // 20), n // 20 + 1 + np.arange(n // 2)]),  # gap rule
+        rng.choice([-np.inf, -1.5, -0.0, 0.0, 2.0, np.inf], size=n),  # infinities and signed zeros
+        np.full(n, 3.25),                                     # constant
+        -np.abs(rng.normal(size=n)) * 1e-30,                  # tiny negatives
+    ]
+    return np.stack(cols, axis=1).astype(np.float32)
+
+
+@pytest.mark.parametrize("n,hist_size", [(5000, 16), (70000, 255), (4097, 64), (300, 256), (9000, 3)])
+def test_quantiser_matches_oracle(arb, oracle, n, hist_size):
+    X = _columns_for_quantiser(n, np.random.default_rng(n))
+    data = arb.DMatrix(X)
+    data.quantize(hist_size)
+    bins = data.bins()
+    for f in range(X.shape[1]):
+        thr_o, bins_o, size_o = oracle.quantize_column(X[:, f], hist_size)
+        thr_g, size_g = data.thresholds(f, hist_size)
+        assert size_g == size_o, f
+        assert np.array_equal(thr_g, thr_o), f
+        assert np.array_equal(bins[:, f], bins_o.astype(np.uint8)), f
+
+
 @pytest.mark.parametrize("objective", [0, 1])
 @pytest.mark.parametrize("dp", [True, False])
 @pytest.mark.parametrize("trick", [True, False])
