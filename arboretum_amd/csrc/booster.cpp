@@ -121,7 +121,10 @@ void Garden::GrowTree(DataMatrix *data, const float *grad) {
     throw std::runtime_error("colsample_bytree and colsample_bylevel are too small");
   if (DeviceCount() <= 0) throw std::runtime_error("no HIP device available: training needs an MI355X");
   if (!builder_) {
-    QuantiseOnDevice(data, cfg.internal.hist_size, cfg.verbose.data);
+    // upload_features = false keeps the bins in pinned host memory and streams
+    // them (src/core/garden.cu:603-604, hist_tree_grower.cu:335-366)
+    QuantiseOnDevice(data, cfg.internal.hist_size, cfg.verbose.data, !cfg.internal.upload_features,
+                     cfg.internal.stream_block_rows);
     builder_.reset(CreateTreeBuilder(cfg, data));
     builder_->SetInspect(inspect_);
     builder_->EnableTiming(timing_);

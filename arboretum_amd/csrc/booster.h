@@ -49,10 +49,17 @@ class DataMatrix {
   std::vector<std::vector<float>> thresholds;
   std::vector<int> reduced_size;
   DeviceMatrix *device = nullptr;
+  // Streamed matrices (bins in pinned host blocks instead of HBM): block b
+  // holds rows [b * stream_block_rows, ...) as quads [Q][stream_block_rows].
+  std::vector<uint32_t *> stream_blocks;
+  size_t stream_block_rows = 0;
 
   // Feature value as seen by host prediction.
   inline float value(size_t f, size_t i) const {
-    return is_prebinned ? (float)prebinned[i * columns_dense + f] : data[f][i];
+    if (!is_prebinned) return data[f][i];
+    if (!prebinned.empty()) return (float)prebinned[i * columns_dense + f];
+    const uint32_t q = stream_blocks[i / stream_block_rows][(f >> 2) * stream_block_rows + i % stream_block_rows];
+    return (float)((q >> (8 * (f & 3))) & 255u);
   }
 };
 
@@ -111,7 +118,10 @@ void FreeSortWorkspace(SortWorkspace *ws);
 void DeviceThresholds(SortWorkspace *ws, const float *d_col, std::vector<float> *thr, int *size, bool *has_nan);
 
 // device_builder.hip
-void QuantiseOnDevice(DataMatrix *data, int hist_size, bool verbose);
+// streamed = false: bins resident in HBM; true: bins in pinned host blocks of
+// block_rows rows, copied to the GPU block by block at every tree level.
+void QuantiseOnDevice(DataMatrix *data, int hist_size, bool verbose, bool streamed = false,
+                      size_t block_rows = 0);
 void FreeDeviceMatrix(DeviceMatrix *m);
 void GetDeviceBins(const DataMatrix &data, uint8_t *out);  // row-major [rows][F]
 TreeBuilder *CreateTreeBuilder(const Configuration &cfg, DataMatrix *data);

@@ -51,6 +51,7 @@ Configuration Configuration::Parse(const char *text) {
     GetBool(*v, "use_hist_subtraction_trick", &cfg.internal.use_hist_subtraction_trick);
     GetBool(*v, "upload_features", &cfg.internal.upload_features);
     GetNum(*v, "hist_size", &cfg.internal.hist_size);
+    GetNum(*v, "stream_block_rows", &cfg.internal.stream_block_rows);
   }
   return cfg;
 }

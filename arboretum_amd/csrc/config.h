@@ -48,6 +48,9 @@ struct InternalConfiguration {  // param.h:54-64
   bool use_hist_subtraction_trick = true;
   bool upload_features = true;
   int hist_size = 255;
+  // Extension (not a reference key): rows per pinned-host block when the bins
+  // are streamed (upload_features = false).
+  unsigned stream_block_rows = 1u << 22;
 };
 
 struct Configuration {  // param.h:66-74

@@ -238,7 +238,7 @@ k_plan(const NodeSum *__restrict__ tot, const unsigned *__restrict__ seg_start, 
        unsigned rows_per_item, WorkItem *__restrict__ work, unsigned *__restrict__ n_work,
        unsigned *__restrict__ node_first, unsigned *__restrict__ node_items,
        unsigned long long *__restrict__ rows_scanned, const SplitRec *__restrict__ split,
-       unsigned max_items) {
+       unsigned max_items, unsigned *__restrict__ overflow) {
   __shared__ unsigned s_base[kMaxPlanNodes + 1];
   __shared__ unsigned s_wave[16];
   __shared__ unsigned s_carry;
@@ -293,6 +293,7 @@ k_plan(const NodeSum *__restrict__ tot, const unsigned *__restrict__ seg_start, 
   if (tid == 0) {
     s_base[L] = total;
     *n_work = total <= max_items ? total : 0;  // never exceed the launch bound
+    if (total > max_items) *overflow = 1;      // reported as an error at the end of the tree
     if (rows_scanned) *rows_scanned += s_rows;
   }
   __syncthreads();
@@ -724,8 +725,9 @@ k_partition(const uint32_t *__restrict__ bins, uint32_t *__restrict__ bins_out, 
   }
 }
 
-// Adds the slabs of every directly built node of a level and, with `trick`,
-// derives its sibling as parent - node.  grid (nbin_total/64, L), 1024
+// Adds the slabs of every directly built node of a level (on top of the stored
+// histogram when `accumulate`) and, with `trick`, derives its sibling as
+// parent - node.  grid (nbin_total/64, L), 1024
 // threads = 64 entries x 16 slab lanes.
 //   by_parent = 0: slabs belong to work items of the node itself
 //               (node_items == 0xffffffff marks a derived node);
@@ -739,7 +741,7 @@ k_hist_reduce(const unsigned long long *__restrict__ slab, int nbin_total,
               const NodeSum *__restrict__ parent_tot, long long *__restrict__ hg,
               long long *__restrict__ hh, unsigned *__restrict__ hc,
               const long long *__restrict__ pg, const long long *__restrict__ ph,
-              const unsigned *__restrict__ pc, int trick) {
+              const unsigned *__restrict__ pc, int trick, int accumulate) {
   __shared__ long long s_g[16][64];
   __shared__ long long s_h[16][64];
   __shared__ unsigned s_c[16][64];
@@ -780,6 +782,11 @@ k_hist_reduce(const unsigned long long *__restrict__ slab, int nbin_total,
       ac += s_c[k][e];
     }
     const size_t o = (size_t)nd * nbin_total + entry;
+    if (accumulate) {  // streamed matrices: one call per row block
+      ag += hg[o];
+      ah += hh[o];
+      ac += hc[o];
+    }
     hg[o] = ag;
     hh[o] = ah;
     hc[o] = ac;
@@ -810,6 +817,119 @@ k_root_from_hist(const long long *__restrict__ hg, const long long *__restrict__
     tot[0].g = a;
     tot[0].h = b;
   }
+}
+
+// ----------------------------------------------------- streamed row blocks
+// When the bins do not live in HBM (pinned host blocks copied in at every
+// level; the reference streams whole columns, hist_tree_grower.cu:335-366),
+// rows are never re-ordered.  A resident node id per row is advanced with the
+// parents' splits while its block is on the GPU, the rows of the nodes built
+// at this level are gathered node by node into a staging buffer, and the
+// ordinary histogram kernel runs on that buffer.
+
+// Is node nd accumulated directly at this level?  With sibling subtraction
+// only the smaller child of each pair, ties -> left (hist_grad_sum.cu:279-294).
+__device__ __forceinline__ bool NodeIsBuilt(const NodeSum *__restrict__ tot, unsigned nd, int level, int trick) {
+  if (level == 0 || !trick) return true;
+  const unsigned long long c = tot[nd].c, sib = tot[nd ^ 1u].c;
+  return (nd & 1u) ? (c < sib) : (c <= sib);
+}
+
+// Advances the node id of every row of the block by the parents' splits and
+// counts the rows of every built node (blk_cnt, zero on entry).
+__global__ void __launch_bounds__(256)
+k_stream_route(const uint32_t *__restrict__ bins, size_t bstride, unsigned rows, int level, int trick,
+               const SplitRec *__restrict__ split, const NodeSum *__restrict__ tot,
+               unsigned *__restrict__ node_of, unsigned *__restrict__ blk_cnt) {
+  __shared__ unsigned s_cnt[kMaxPlanNodes];
+  const int L = 1 << level;
+  for (int i = threadIdx.x; i < L; i += blockDim.x) s_cnt[i] = 0;
+  __syncthreads();
+  for (unsigned r = blockIdx.x * blockDim.x + threadIdx.x; r < rows; r += gridDim.x * blockDim.x) {
+    unsigned nd = 0;
+    if (level > 0) {
+      const unsigned parent = node_of[r];
+      nd = parent * 2u + (GoesRight(bins, bstride, split[parent], r) ? 1u : 0u);
+    }
+    node_of[r] = nd;
+    if (NodeIsBuilt(tot, nd, level, trick)) atomicAdd(&s_cnt[nd], 1u);
+  }
+  __syncthreads();
+  for (int i = threadIdx.x; i < L; i += blockDim.x)
+    if (s_cnt[i]) atomicAdd(&blk_cnt[i], s_cnt[i]);
+}
+
+// Row ranges of the built nodes inside the staging buffer: exclusive scan of
+// blk_cnt; also the cursors of the gather and the totals the planner reads.
+// Clears blk_cnt for the next block.  One workgroup.
+__global__ void __launch_bounds__(1024)
+k_stream_segments(unsigned *__restrict__ blk_cnt, int L, NodeSum *__restrict__ blk_tot,
+                  unsigned *__restrict__ blk_seg, unsigned *__restrict__ cursor) {
+  __shared__ unsigned s_wave[16];
+  __shared__ unsigned s_carry;
+  if (threadIdx.x == 0) s_carry = 0;
+  __syncthreads();
+  for (int base = 0; base < L; base += 1024) {
+    const int nd = base + threadIdx.x;
+    const unsigned c = nd < L ? blk_cnt[nd] : 0u;
+    unsigned incl = c;
+    for (int off = 1; off < 64; off <<= 1) {
+      const unsigned o = __shfl_up(incl, off);
+      if ((threadIdx.x & 63) >= off) incl += o;
+    }
+    if ((threadIdx.x & 63) == 63) s_wave[threadIdx.x >> 6] = incl;
+    __syncthreads();
+    unsigned off = s_carry;
+    for (int w = 0; w < (int)(threadIdx.x >> 6); ++w) off += s_wave[w];
+    const unsigned excl = off + incl - c;
+    if (nd < L) {
+      blk_seg[nd] = excl;
+      cursor[nd] = excl;
+      blk_tot[nd].g = 0;
+      blk_tot[nd].h = 0;
+      blk_tot[nd].c = c;
+      blk_cnt[nd] = 0;
+    }
+    __syncthreads();
+    if (threadIdx.x == 1023) s_carry = excl + c;
+    __syncthreads();
+  }
+}
+
+// Copies the rows of the built nodes into the staging buffer, node by node.
+// The order inside a node is whatever the atomics give; sums are integers.
+template <bool PAIR>
+__global__ void __launch_bounds__(256)
+k_stream_gather(const uint32_t *__restrict__ bins, size_t bstride, int Q, unsigned rows,
+                const float *__restrict__ g, const float *__restrict__ h,
+                const unsigned *__restrict__ node_of, int level, int trick,
+                const NodeSum *__restrict__ tot, unsigned *__restrict__ cursor,
+                uint32_t *__restrict__ st_bins, size_t sstride, float *__restrict__ st_g,
+                float *__restrict__ st_h) {
+  for (unsigned r = blockIdx.x * blockDim.x + threadIdx.x; r < rows; r += gridDim.x * blockDim.x) {
+    const unsigned nd = node_of[r];
+    if (!NodeIsBuilt(tot, nd, level, trick)) continue;
+    const unsigned d = atomicAdd(&cursor[nd], 1u);
+    for (int q = 0; q < Q; ++q) st_bins[(size_t)q * sstride + d] = bins[(size_t)q * bstride + r];
+    st_g[d] = g[r];
+    if (PAIR) st_h[d] = h[r];
+  }
+}
+
+// sibling = parent - built child for every node that was not built directly
+__global__ void k_sibling(long long *__restrict__ hg, long long *__restrict__ hh, unsigned *__restrict__ hc,
+                          const long long *__restrict__ pg, const long long *__restrict__ ph,
+                          const unsigned *__restrict__ pc, const NodeSum *__restrict__ tot, int level,
+                          int nbin_total) {
+  const unsigned nd = blockIdx.y;
+  if (NodeIsBuilt(tot, nd, level, 1)) return;
+  const int e = blockIdx.x * blockDim.x + threadIdx.x;
+  if (e >= nbin_total) return;
+  const size_t o = (size_t)nd * nbin_total + e, so = (size_t)(nd ^ 1u) * nbin_total + e,
+               po = (size_t)(nd >> 1) * nbin_total + e;
+  hg[o] = pg[po] - hg[so];
+  hh[o] = ph[po] - hh[so];
+  hc[o] = pc[po] - hc[so];
 }
 
 // --------------------------------------------------------------- split scan
@@ -1067,7 +1187,11 @@ inline int GridFor(size_t n, int block, int cap = 4096) {
 struct DeviceMatrix {
   size_t rows = 0, stride = 0;
   int F = 0, Q = 0;
-  uint32_t *bins = nullptr;  // [Q][stride]
+  uint32_t *bins = nullptr;  // resident: [Q][stride] in HBM
+  // streamed: pinned host blocks [Q][block_rows], block b = rows [b*block_rows, ...)
+  bool streamed = false;
+  size_t block_rows = 0;
+  std::vector<uint32_t *> host_blocks;
 };
 
 // Plain device-to-device copy of `bytes` bytes: a kernel of exactly known HBM
@@ -1099,10 +1223,12 @@ int DeviceCount() {
 void FreeDeviceMatrix(DeviceMatrix *m) {
   if (!m) return;
   if (m->bins) (void)hipFree(m->bins);
+  for (uint32_t *b : m->host_blocks)
+    if (b) (void)hipHostFree(b);
   delete m;
 }
 
-void QuantiseOnDevice(DataMatrix *data, int hist_size, bool verbose) {
+void QuantiseOnDevice(DataMatrix *data, int hist_size, bool verbose, bool streamed, size_t block_rows) {
   if (data->quantised) {
     if (data->hist_size != hist_size) throw std::runtime_error("data matrix was quantised with another hist_size");
     return;
@@ -1111,13 +1237,35 @@ void QuantiseOnDevice(DataMatrix *data, int hist_size, bool verbose) {
   const size_t n = data->rows;
   const int F = (int)data->columns_dense;
   if (n == 0 || F == 0) throw std::runtime_error("empty data matrix");
-  if (n >= 0xffffffffull) throw std::runtime_error("too many rows");
+  if (n >= (1ull << 31)) throw std::runtime_error("too many rows");
   std::unique_ptr<DeviceMatrix, void (*)(DeviceMatrix *)> dm(new DeviceMatrix(), FreeDeviceMatrix);
   dm->rows = n;
   dm->F = F;
   dm->Q = (F + 3) / 4;
   dm->stride = (n + 63) / 64 * 64;
-  dm->bins = DevAlloc<uint32_t>((size_t)dm->Q * dm->stride);
+  dm->streamed = streamed;
+  uint32_t *d_col = nullptr;  // streamed: one quad column at a time on the device
+  size_t nblocks = 0;
+  if (streamed) {
+    if (block_rows < 64) block_rows = 64;
+    block_rows = (block_rows + 63) / 64 * 64;
+    dm->block_rows = block_rows;
+    nblocks = (n + block_rows - 1) / block_rows;
+    dm->host_blocks.assign(nblocks, nullptr);
+    for (size_t b = 0; b < nblocks; ++b)
+      HIP_OK(hipHostMalloc((void **)&dm->host_blocks[b], (size_t)dm->Q * block_rows * sizeof(uint32_t), hipHostMallocDefault));
+    d_col = DevAlloc<uint32_t>(dm->stride);
+  } else {
+    dm->bins = DevAlloc<uint32_t>((size_t)dm->Q * dm->stride);
+  }
+  // streamed: quad q of all rows (in d_col) -> its slice of every host block
+  auto store_quad = [&](int q) {
+    for (size_t b = 0; b < nblocks; ++b) {
+      const size_t r0 = b * block_rows, rows = std::min(block_rows, n - r0);
+      HIP_OK(hipMemcpy(dm->host_blocks[b] + (size_t)q * block_rows, d_col + r0, rows * sizeof(uint32_t),
+                       hipMemcpyDeviceToHost));
+    }
+  };
   data->thresholds.assign(F, {});
   data->reduced_size.assign(F, 0);
 
@@ -1127,12 +1275,28 @@ void QuantiseOnDevice(DataMatrix *data, int hist_size, bool verbose) {
       for (int k = 0; k < hist_size; ++k) data->thresholds[f][k] = (float)k + 0.5f;
       data->reduced_size[f] = std::min(hist_size, kSlots);
     }
-    uint8_t *d_in = DevAlloc<uint8_t>(n * F);
-    HIP_OK(hipMemcpy(d_in, data->prebinned.data(), n * F, hipMemcpyHostToDevice));
-    hipLaunchKernelGGL(k_pack_prebinned, dim3(GridFor(n, 256)), dim3(256), 0, 0, d_in, F, dm->Q,
-                       dm->bins, dm->stride, n);
-    HIP_OK(hipDeviceSynchronize());
-    HIP_OK(hipFree(d_in));
+    if (!streamed) {
+      uint8_t *d_in = DevAlloc<uint8_t>(n * F);
+      HIP_OK(hipMemcpy(d_in, data->prebinned.data(), n * F, hipMemcpyHostToDevice));
+      hipLaunchKernelGGL(k_pack_prebinned, dim3(GridFor(n, 256)), dim3(256), 0, 0, d_in, F, dm->Q,
+                         dm->bins, dm->stride, n);
+      HIP_OK(hipDeviceSynchronize());
+      HIP_OK(hipFree(d_in));
+    } else {
+      // pack block by block: row-major bytes up, quads down into the pinned block
+      uint8_t *d_in = DevAlloc<uint8_t>(block_rows * F);
+      uint32_t *d_out = DevAlloc<uint32_t>((size_t)dm->Q * block_rows);
+      for (size_t b = 0; b < nblocks; ++b) {
+        const size_t r0 = b * block_rows, rows = std::min(block_rows, n - r0);
+        HIP_OK(hipMemcpy(d_in, data->prebinned.data() + r0 * F, rows * F, hipMemcpyHostToDevice));
+        hipLaunchKernelGGL(k_pack_prebinned, dim3(GridFor(rows, 256)), dim3(256), 0, 0, d_in, F, dm->Q, d_out,
+                           block_rows, rows);
+        HIP_OK(hipMemcpy(dm->host_blocks[b], d_out, (size_t)dm->Q * block_rows * sizeof(uint32_t), hipMemcpyDeviceToHost));
+      }
+      HIP_OK(hipFree(d_in));
+      HIP_OK(hipFree(d_out));
+      std::vector<uint8_t>().swap(data->prebinned);  // the pinned blocks are the only copy from here on
+    }
   } else {
     // per quad: upload four columns, thresholds by device sort, bin assignment
     std::unique_ptr<SortWorkspace, void (*)(SortWorkspace *)> ws(CreateSortWorkspace(n, hist_size), FreeSortWorkspace);
@@ -1158,13 +1322,19 @@ void QuantiseOnDevice(DataMatrix *data, int hist_size, bool verbose) {
       }
       HIP_OK(hipMemcpy(d_size, sizes, sizeof(sizes), hipMemcpyHostToDevice));
       hipLaunchKernelGGL(k_bin_assign, dim3(GridFor(n, 256)), dim3(256), 0, 0, d_x, nc, d_thr,
-                         hist_size, d_size, dm->bins + (size_t)q * dm->stride, n);
+                         hist_size, d_size, streamed ? d_col : dm->bins + (size_t)q * dm->stride, n);
       HIP_OK(hipGetLastError());
       HIP_OK(hipDeviceSynchronize());
+      if (streamed) store_quad(q);
     }
     HIP_OK(hipFree(d_x));
     HIP_OK(hipFree(d_thr));
     HIP_OK(hipFree(d_size));
+  }
+  if (d_col) HIP_OK(hipFree(d_col));
+  if (streamed) {
+    data->stream_blocks = dm->host_blocks;
+    data->stream_block_rows = block_rows;
   }
   data->device = dm.release();
   data->hist_size = hist_size;
@@ -1174,6 +1344,14 @@ void QuantiseOnDevice(DataMatrix *data, int hist_size, bool verbose) {
 void GetDeviceBins(const DataMatrix &data, uint8_t *out) {
   const DeviceMatrix *dm = data.device;
   if (!dm) throw std::runtime_error("data matrix is not quantised");
+  if (dm->streamed) {
+    for (size_t r = 0; r < dm->rows; ++r) {
+      const uint32_t *blk = dm->host_blocks[r / dm->block_rows];
+      for (int f = 0; f < dm->F; ++f)
+        out[r * dm->F + f] = (uint8_t)(blk[(size_t)(f >> 2) * dm->block_rows + r % dm->block_rows] >> (8 * (f & 3)));
+    }
+    return;
+  }
   std::vector<uint32_t> q((size_t)dm->Q * dm->stride);
   HIP_OK(hipMemcpy(q.data(), dm->bins, q.size() * sizeof(uint32_t), hipMemcpyDeviceToHost));
   for (size_t r = 0; r < dm->rows; ++r)
@@ -1310,8 +1488,27 @@ class HipTreeBuilder : public TreeBuilder {
     hipLaunchKernelGGL(k_fill_f32, dim3(GridFor(n_ * K_, 256)), dim3(256), 0, stream_, d_yhat_, init, n_ * K_);
     data->y_hat.assign(n_ * K_, init);  // garden.cu:104
 
+    streamed_ = dm_->streamed;
+    if (streamed_) {
+      const size_t br = dm_->block_rows;
+      HIP_OK(hipStreamCreateWithFlags(&copy_stream_, hipStreamNonBlocking));
+      for (int b = 0; b < 2; ++b) {
+        blk_[b] = DevAlloc<uint32_t>((size_t)Q_ * br);
+        HIP_OK(hipEventCreateWithFlags(&ev_ready_[b], hipEventDisableTiming));
+        HIP_OK(hipEventCreateWithFlags(&ev_free_[b], hipEventDisableTiming));
+      }
+      stage_.bins = DevAlloc<uint32_t>((size_t)Q_ * br);
+      stage_.g = DevAlloc<float>(br);
+      stage_.h = DevAlloc<float>(br);
+      d_node_of_ = DevAlloc<unsigned>(n_);
+      d_blk_cnt_ = DevAlloc<unsigned>(last_nodes);
+      d_blk_seg_ = DevAlloc<unsigned>(last_nodes);
+      d_cursor_ = DevAlloc<unsigned>(last_nodes);
+      d_blk_tot_ = DevAlloc<NodeSum>(last_nodes);
+      HIP_OK(hipMemsetAsync(d_blk_cnt_, 0, (size_t)last_nodes * sizeof(unsigned), stream_));
+    }
     // ping-pong row buffers in node order (not needed for a single split level)
-    if (D_ > 2) {
+    if (D_ > 2 && !streamed_) {
       for (int b = 0; b < 2; ++b) {
         buf_[b].bins = DevAlloc<uint32_t>((size_t)Q_ * stride_);
         buf_[b].g = DevAlloc<float>(n_);
@@ -1332,6 +1529,7 @@ class HipTreeBuilder : public TreeBuilder {
     d_node_first_ = DevAlloc<unsigned>(last_nodes);
     d_node_items_ = DevAlloc<unsigned>(last_nodes);
     max_hist_items_ = (unsigned)(n_ / HistRowsPerItem(n_)) + last_nodes + 2;
+    max_hist_items_ = std::max<unsigned>(max_hist_items_, 1024 + last_nodes + 2);
     max_part_items_ = std::max<unsigned>((unsigned)(n_ / kPartRows + 1) + last_nodes, max_hist_items_);
     d_hwork_ = DevAlloc<WorkItem>(max_hist_items_);
     d_pwork_ = DevAlloc<WorkItem>(max_part_items_);
@@ -1342,6 +1540,8 @@ class HipTreeBuilder : public TreeBuilder {
     d_shifts_ = DevAlloc<int>(2);
     d_gmax_ = DevAlloc<unsigned>(1);
     d_rows_scanned_ = DevAlloc<unsigned long long>(1);
+    d_overflow_ = DevAlloc<unsigned>(1);
+    HIP_OK(hipMemsetAsync(d_overflow_, 0, sizeof(unsigned), stream_));
     HIP_OK(hipMemsetAsync(d_rows_scanned_, 0, sizeof(unsigned long long), stream_));
     HIP_OK(hipMemsetAsync(d_gmax_, 0, sizeof(unsigned), stream_));
     const int internal = (1 << (D_ - 1)) - 1;
@@ -1362,7 +1562,7 @@ class HipTreeBuilder : public TreeBuilder {
     (void)hipStreamSynchronize(stream_);
     void *ptrs[] = {d_y_, d_labels_, d_yhat_, d_g_, d_h_, d_leaf_, d_split_, d_cand_, d_node_first_,
                     d_node_items_, d_hwork_, d_pwork_, d_nwork_, d_wave_left_, d_item_left_, d_slab_,
-                    d_shifts_, d_gmax_, d_rows_scanned_, d_tfid_, d_tbin_, d_tgain_, d_weights_, d_active_};
+                    d_shifts_, d_gmax_, d_rows_scanned_, d_tfid_, d_tbin_, d_tgain_, d_weights_, d_active_, d_overflow_};
     for (void *p : ptrs)
       if (p) (void)hipFree(p);
     for (int b = 0; b < 2; ++b) {
@@ -1371,6 +1571,18 @@ class HipTreeBuilder : public TreeBuilder {
         if (p) (void)hipFree(p);
     }
     for (hipEvent_t e : event_pool_) (void)hipEventDestroy(e);
+    if (streamed_) {
+      (void)hipStreamSynchronize(copy_stream_);
+      void *sp[] = {blk_[0], blk_[1], stage_.bins, stage_.g, stage_.h, d_node_of_, d_blk_cnt_, d_blk_seg_,
+                    d_cursor_, d_blk_tot_};
+      for (void *p : sp)
+        if (p) (void)hipFree(p);
+      for (int b = 0; b < 2; ++b) {
+        (void)hipEventDestroy(ev_ready_[b]);
+        (void)hipEventDestroy(ev_free_[b]);
+      }
+      (void)hipStreamDestroy(copy_stream_);
+    }
     (void)hipStreamDestroy(stream_);
   }
 
@@ -1491,9 +1703,13 @@ class HipTreeBuilder : public TreeBuilder {
 
   void Plan(int state, int L, int select, unsigned rows_per_item, WorkItem *work, unsigned *n_work,
             bool count_rows, const SplitRec *split, unsigned max_items) {
-    hipLaunchKernelGGL(k_plan, dim3(1), dim3(1024), 0, stream_, d_tot_[state], d_seg_[state], L, select,
+    PlanOn(d_tot_[state], d_seg_[state], L, select, rows_per_item, work, n_work, count_rows, split, max_items);
+  }
+  void PlanOn(const NodeSum *tot, const unsigned *seg, int L, int select, unsigned rows_per_item, WorkItem *work,
+              unsigned *n_work, bool count_rows, const SplitRec *split, unsigned max_items) {
+    hipLaunchKernelGGL(k_plan, dim3(1), dim3(1024), 0, stream_, tot, seg, L, select,
                        rows_per_item, work, n_work, d_node_first_, d_node_items_,
-                       count_rows ? d_rows_scanned_ : (unsigned long long *)nullptr, split, max_items);
+                       count_rows ? d_rows_scanned_ : (unsigned long long *)nullptr, split, max_items, d_overflow_);
   }
 
   // Histograms of contiguous node ranges in `cur` (level order), feature group by group.
@@ -1515,17 +1731,17 @@ class HipTreeBuilder : public TreeBuilder {
     if (timing_ && root) timings_.hist_root_rows += n_;
   }
 
-  void Reduce(int L, int hb, bool by_parent, int parent_state, bool trick) {
+  void Reduce(int L, int hb, bool by_parent, int parent_state, bool trick, bool accumulate = false) {
     Mark(kReduce);
     dim3 grid(nbin_total_ / 64, L);
     if (pair_)
       hipLaunchKernelGGL(k_hist_reduce<true>, grid, dim3(1024), 0, stream_, d_slab_, nbin_total_, d_node_first_,
                          d_node_items_, by_parent ? 1 : 0, d_split_, d_tot_[parent_state], d_hg_[hb], d_hh_[hb],
-                         d_hc_[hb], d_hg_[hb ^ 1], d_hh_[hb ^ 1], d_hc_[hb ^ 1], trick ? 1 : 0);
+                         d_hc_[hb], d_hg_[hb ^ 1], d_hh_[hb ^ 1], d_hc_[hb ^ 1], trick ? 1 : 0, accumulate ? 1 : 0);
     else
       hipLaunchKernelGGL(k_hist_reduce<false>, grid, dim3(1024), 0, stream_, d_slab_, nbin_total_, d_node_first_,
                          d_node_items_, by_parent ? 1 : 0, d_split_, d_tot_[parent_state], d_hg_[hb], d_hh_[hb],
-                         d_hc_[hb], d_hg_[hb ^ 1], d_hh_[hb ^ 1], d_hc_[hb ^ 1], trick ? 1 : 0);
+                         d_hc_[hb], d_hg_[hb ^ 1], d_hh_[hb ^ 1], d_hc_[hb ^ 1], trick ? 1 : 0, accumulate ? 1 : 0);
   }
 
   void GrowOne(int label, RegTree *tree) {
@@ -1536,6 +1752,10 @@ class HipTreeBuilder : public TreeBuilder {
     orig.h = d_h_ + (size_t)label * n_;
     if (inspect_) kept_hist_.assign(D_ - 1, {});
     SampleColumns();
+    if (streamed_) {
+      GrowOneStreamed(label, tree, orig, gp);
+      return;
+    }
 
     hipLaunchKernelGGL(k_init_root, dim3(1), dim3(64), 0, stream_, d_tot_[0], d_seg_[0],
                        (unsigned long long)n_, (unsigned *)nullptr);
@@ -1595,73 +1815,25 @@ class HipTreeBuilder : public TreeBuilder {
         }
       }
       if (inspect_) KeepHist(level, L, hb);
-      // ---- split scan and selection
-      Mark(kSplit);
-      {
-        dim3 grid(F_, L);
-        const int hs = std::min(cfg_.internal.hist_size, kSlots);
-#define ARB_SCAN(P, D) \
-  hipLaunchKernelGGL((k_split_scan<P, D>), grid, dim3(64), 0, stream_, d_hg_[hb], d_hh_[hb], d_hc_[hb], \
-                     nbin_total_, F_, d_tot_[state], d_shifts_, gp, hs, d_cand_)
-        if (pair_ && f64_) ARB_SCAN(true, true);
-        else if (pair_) ARB_SCAN(true, false);
-        else if (f64_) ARB_SCAN(false, true);
-        else ARB_SCAN(false, false);
-#undef ARB_SCAN
-        hipLaunchKernelGGL(k_split_select, dim3((L + 127) / 128), dim3(128), 0, stream_, d_cand_, F_, L,
-                           d_tot_[state], d_seg_[state], d_tot_[state ^ 1], d_seg_[state ^ 1], d_split_,
-                           d_tfid_, d_tbin_, d_tgain_, L - 1,
-                           sampling_ ? d_active_ + (size_t)level * F_ : (const unsigned char *)nullptr);
-      }
-      if (last) {
-        Mark(kLeaf);
-        const int blocks = (L + 127) / 128;
-#define ARB_LEAF(P, D) \
-  hipLaunchKernelGGL((k_leaf_weights<P, D>), dim3(blocks), dim3(128), 0, stream_, d_split_, d_tot_[state], L, \
-                     d_shifts_, gp, cfg_.tree.eta, d_weights_)
-        if (pair_ && f64_) ARB_LEAF(true, true);
-        else if (pair_) ARB_LEAF(true, false);
-        else if (f64_) ARB_LEAF(false, true);
-        else ARB_LEAF(false, false);
-#undef ARB_LEAF
-      }
+      LaunchSplit(level, L, hb, state, gp);
+      if (last) LaunchLeafWeights(L, state, gp);
       state ^= 1;
     }
     // ---- leaf of every row, y_hat update, gradients of the next round
     Mark(kLeaf);
     {
-      const int internal = (1 << (D_ - 1)) - 1;
-      const size_t lds = (size_t)internal * 2 * sizeof(int);
-      float *yh = d_yhat_ + (size_t)label * n_;
-      const int grid = GridFor(n_, 256, 8192);
       const bool next_grad = !inspect_ && K_ == 1;
-      int mode = 0;
-      if (next_grad && cfg_.objective == kLinearRegression) mode = 1;
-      if (next_grad && cfg_.objective == kLogisticRegression) mode = 2;
       if (cfg_.objective == kLinearRegression) HIP_OK(hipMemsetAsync(d_gmax_, 0, sizeof(unsigned), stream_));
-#define ARB_FINAL(M, N) \
-  hipLaunchKernelGGL((k_final<M, N>), dim3(grid), dim3(256), lds, stream_, dm_->bins, stride_, d_tfid_, d_tbin_, D_, \
-                     d_weights_, yh, d_y_, d_leaf_, d_g_, d_h_, d_gmax_, n_)
-#define ARB_FINAL_Q(N) \
-  do { if (mode == 1) ARB_FINAL(1, N); else if (mode == 2) ARB_FINAL(2, N); else ARB_FINAL(0, N); } while (0)
-      switch (Q_ <= 8 ? Q_ : 0) {
-        case 1: ARB_FINAL_Q(1); break;
-        case 2: ARB_FINAL_Q(2); break;
-        case 3: ARB_FINAL_Q(3); break;
-        case 4: ARB_FINAL_Q(4); break;
-        case 5: ARB_FINAL_Q(5); break;
-        case 6: ARB_FINAL_Q(6); break;
-        case 7: ARB_FINAL_Q(7); break;
-        case 8: ARB_FINAL_Q(8); break;
-        default: ARB_FINAL_Q(0); break;
-      }
-#undef ARB_FINAL_Q
-#undef ARB_FINAL
+      LaunchFinal(dm_->bins, stride_, 0, n_, label, next_grad);
       grad_ready_ = next_grad;
     }
+    FetchTree(tree);
+  }
+
+  // Tree record to the host (garden.cu:447-503): node arrays and leaf weights.
+  void FetchTree(RegTree *tree) {
     Mark(kNone);
     HIP_OK(hipGetLastError());
-    // ---- tree record to the host (garden.cu:447-503)
     const int internal = (1 << (D_ - 1)) - 1;
     std::vector<int> fid(internal), bin(internal);
     HIP_OK(hipMemcpyAsync(fid.data(), d_tfid_, internal * sizeof(int), hipMemcpyDeviceToHost, stream_));
@@ -1669,7 +1841,10 @@ class HipTreeBuilder : public TreeBuilder {
     HIP_OK(hipMemcpyAsync(tree->gain.data(), d_tgain_, internal * sizeof(float), hipMemcpyDeviceToHost, stream_));
     HIP_OK(hipMemcpyAsync(tree->weights.data(), d_weights_, tree->weights.size() * sizeof(float),
                           hipMemcpyDeviceToHost, stream_));
+    unsigned overflow = 0;
+    HIP_OK(hipMemcpyAsync(&overflow, d_overflow_, sizeof(unsigned), hipMemcpyDeviceToHost, stream_));
     HIP_OK(hipStreamSynchronize(stream_));
+    if (overflow) throw std::runtime_error("internal: work plan exceeded its launch bound");
     for (int i = 0; i < internal; ++i) {
       tree->fid[i] = (unsigned)fid[i];
       tree->quantized[i] = bin[i];
@@ -1677,6 +1852,154 @@ class HipTreeBuilder : public TreeBuilder {
       if (bin[i] >= 0 && bin[i] < (int)data_->thresholds[fid[i]].size()) thr = data_->thresholds[fid[i]][bin[i]];
       tree->threshold[i] = thr;
     }
+  }
+
+  // ---- streamed matrices -------------------------------------------------
+  // Block `b` of the matrix into one of the two device buffers, on the copy
+  // stream; returns the buffer index.  The compute stream waits for ev_ready_
+  // before reading and records ev_free_ when it is done with the buffer.
+  int CopyBlockIn(size_t b) {
+    const int buf = (int)(next_copy_++ & 1);
+    if (buf_used_[buf]) HIP_OK(hipStreamWaitEvent(copy_stream_, ev_free_[buf], 0));
+    HIP_OK(hipMemcpyAsync(blk_[buf], dm_->host_blocks[b], (size_t)Q_ * dm_->block_rows * sizeof(uint32_t),
+                          hipMemcpyHostToDevice, copy_stream_));
+    HIP_OK(hipEventRecord(ev_ready_[buf], copy_stream_));
+    buf_used_[buf] = true;
+    return buf;
+  }
+
+  void LaunchSplit(int level, int L, int hb, int state, const GainParams &gp) {
+    Mark(kSplit);
+    dim3 grid(F_, L);
+    const int hs = std::min(cfg_.internal.hist_size, kSlots);
+#define ARB_SCAN(P, D) \
+  hipLaunchKernelGGL((k_split_scan<P, D>), grid, dim3(64), 0, stream_, d_hg_[hb], d_hh_[hb], d_hc_[hb], \
+                     nbin_total_, F_, d_tot_[state], d_shifts_, gp, hs, d_cand_)
+    if (pair_ && f64_) ARB_SCAN(true, true);
+    else if (pair_) ARB_SCAN(true, false);
+    else if (f64_) ARB_SCAN(false, true);
+    else ARB_SCAN(false, false);
+#undef ARB_SCAN
+    hipLaunchKernelGGL(k_split_select, dim3((L + 127) / 128), dim3(128), 0, stream_, d_cand_, F_, L,
+                       d_tot_[state], d_seg_[state], d_tot_[state ^ 1], d_seg_[state ^ 1], d_split_,
+                       d_tfid_, d_tbin_, d_tgain_, L - 1,
+                       sampling_ ? d_active_ + (size_t)level * F_ : (const unsigned char *)nullptr);
+  }
+
+  void LaunchLeafWeights(int L, int state, const GainParams &gp) {
+    Mark(kLeaf);
+    const int blocks = (L + 127) / 128;
+#define ARB_LEAF(P, D) \
+  hipLaunchKernelGGL((k_leaf_weights<P, D>), dim3(blocks), dim3(128), 0, stream_, d_split_, d_tot_[state], L, \
+                     d_shifts_, gp, cfg_.tree.eta, d_weights_)
+    if (pair_ && f64_) ARB_LEAF(true, true);
+    else if (pair_) ARB_LEAF(true, false);
+    else if (f64_) ARB_LEAF(false, true);
+    else ARB_LEAF(false, false);
+#undef ARB_LEAF
+  }
+
+  void LaunchFinal(const uint32_t *bins, size_t stride, size_t row0, size_t rows, int label, bool next_grad) {
+    const int internal = (1 << (D_ - 1)) - 1;
+    const size_t lds = (size_t)internal * 2 * sizeof(int);
+    float *yh = d_yhat_ + (size_t)label * n_ + row0;
+    const int grid = GridFor(rows, 256, 8192);
+    int mode = 0;
+    if (next_grad && cfg_.objective == kLinearRegression) mode = 1;
+    if (next_grad && cfg_.objective == kLogisticRegression) mode = 2;
+#define ARB_FINAL(M, N) \
+  hipLaunchKernelGGL((k_final<M, N>), dim3(grid), dim3(256), lds, stream_, bins, stride, d_tfid_, d_tbin_, D_, \
+                     d_weights_, yh, d_y_ + row0, d_leaf_ + row0, d_g_ + row0, d_h_ + row0, d_gmax_, rows)
+#define ARB_FINAL_Q(N) \
+  do { if (mode == 1) ARB_FINAL(1, N); else if (mode == 2) ARB_FINAL(2, N); else ARB_FINAL(0, N); } while (0)
+    switch (Q_ <= 8 ? Q_ : 0) {
+      case 1: ARB_FINAL_Q(1); break;
+      case 2: ARB_FINAL_Q(2); break;
+      case 3: ARB_FINAL_Q(3); break;
+      case 4: ARB_FINAL_Q(4); break;
+      case 5: ARB_FINAL_Q(5); break;
+      case 6: ARB_FINAL_Q(6); break;
+      case 7: ARB_FINAL_Q(7); break;
+      case 8: ARB_FINAL_Q(8); break;
+      default: ARB_FINAL_Q(0); break;
+    }
+#undef ARB_FINAL_Q
+#undef ARB_FINAL
+  }
+
+  // One tree over a streamed matrix: every level copies every block in once
+  // (double buffered against the kernels of the previous block), one more pass
+  // assigns the leaves.
+  void GrowOneStreamed(int label, RegTree *tree, const RowBuffers &orig, const GainParams &gp) {
+    const size_t br = dm_->block_rows;
+    const size_t nblocks = dm_->host_blocks.size();
+    hipLaunchKernelGGL(k_init_root, dim3(1), dim3(64), 0, stream_, d_tot_[0], d_seg_[0],
+                       (unsigned long long)n_, (unsigned *)nullptr);
+    int state = 0;
+    for (int level = 0; level + 1 < D_; ++level) {
+      const int L = 1 << level;
+      const int hb = level & 1;
+      const bool trick = trick_ && level > 0;
+      for (size_t b = 0; b < nblocks; ++b) {
+        const size_t row0 = b * br;
+        const unsigned rows = (unsigned)std::min(br, n_ - row0);
+        const int buf = CopyBlockIn(b);
+        HIP_OK(hipStreamWaitEvent(stream_, ev_ready_[buf], 0));
+        Mark(kPartition);
+        hipLaunchKernelGGL(k_stream_route, dim3(GridFor(rows, 256, 1024)), dim3(256), 0, stream_, blk_[buf], br, rows,
+                           level, trick ? 1 : 0, d_split_, d_tot_[state], d_node_of_ + row0, d_blk_cnt_);
+        hipLaunchKernelGGL(k_stream_segments, dim3(1), dim3(1024), 0, stream_, d_blk_cnt_, L, d_blk_tot_, d_blk_seg_,
+                           d_cursor_);
+        if (pair_)
+          hipLaunchKernelGGL(k_stream_gather<true>, dim3(GridFor(rows, 256, 2048)), dim3(256), 0, stream_, blk_[buf],
+                             br, Q_, rows, orig.g + row0, orig.h + row0, d_node_of_ + row0, level, trick ? 1 : 0,
+                             d_tot_[state], d_cursor_, stage_.bins, br, stage_.g, stage_.h);
+        else
+          hipLaunchKernelGGL(k_stream_gather<false>, dim3(GridFor(rows, 256, 2048)), dim3(256), 0, stream_, blk_[buf],
+                             br, Q_, rows, orig.g + row0, orig.h + row0, d_node_of_ + row0, level, trick ? 1 : 0,
+                             d_tot_[state], d_cursor_, stage_.bins, br, stage_.g, stage_.h);
+        HIP_OK(hipEventRecord(ev_free_[buf], stream_));
+        // histograms of the gathered rows, added to the level's histograms
+        const unsigned per_item = HistRowsPerItem(rows);
+        const unsigned grid = (unsigned)std::min<size_t>(rows / per_item + L + 1, max_hist_items_);
+        Mark(kPlan);
+        PlanOn(d_blk_tot_, d_blk_seg_, L, 0, per_item, d_hwork_, d_nwork_, true, nullptr, grid);
+        Mark(level == 0 ? kHistRoot : kHistDeep);
+        for (int q0 = 0; q0 < Q_; q0 += quads_per_group_) {
+          const int nq = std::min(quads_per_group_, Q_ - q0);
+          if (pair_)
+            LaunchHist<true>(nq, stream_, grid, stage_.bins, br, q0, F_, stage_.g, stage_.h, d_shifts_, d_hwork_,
+                             d_nwork_, d_slab_, nbin_total_);
+          else
+            LaunchHist<false>(nq, stream_, grid, stage_.bins, br, q0, F_, stage_.g, stage_.h, d_shifts_, d_hwork_,
+                              d_nwork_, d_slab_, nbin_total_);
+        }
+        Reduce(L, hb, false, state, false, b > 0);
+      }
+      if (level == 0)
+        hipLaunchKernelGGL(k_root_from_hist, dim3(1), dim3(64), 0, stream_, d_hg_[hb], d_hh_[hb], d_tot_[state]);
+      if (trick)
+        hipLaunchKernelGGL(k_sibling, dim3((nbin_total_ + 255) / 256, L), dim3(256), 0, stream_, d_hg_[hb], d_hh_[hb],
+                           d_hc_[hb], d_hg_[hb ^ 1], d_hh_[hb ^ 1], d_hc_[hb ^ 1], d_tot_[state], level, nbin_total_);
+      if (inspect_) KeepHist(level, L, hb);
+      LaunchSplit(level, L, hb, state, gp);
+      if (level + 2 >= D_) LaunchLeafWeights(L, state, gp);
+      state ^= 1;
+    }
+    // leaves, y_hat, next gradients: one more pass over the blocks
+    Mark(kLeaf);
+    const bool next_grad = !inspect_ && K_ == 1;
+    if (cfg_.objective == kLinearRegression) HIP_OK(hipMemsetAsync(d_gmax_, 0, sizeof(unsigned), stream_));
+    for (size_t b = 0; b < nblocks; ++b) {
+      const size_t row0 = b * br;
+      const size_t rows = std::min(br, n_ - row0);
+      const int buf = CopyBlockIn(b);
+      HIP_OK(hipStreamWaitEvent(stream_, ev_ready_[buf], 0));
+      LaunchFinal(blk_[buf], br, row0, rows, label, next_grad);
+      HIP_OK(hipEventRecord(ev_free_[buf], stream_));
+    }
+    grad_ready_ = next_grad;
+    FetchTree(tree);
   }
 
   // Column sampling of one tree (InitGrowingTree / InitTreeLevel,
@@ -1736,6 +2059,7 @@ class HipTreeBuilder : public TreeBuilder {
   hipStream_t stream_ = nullptr;
   float *d_y_ = nullptr, *d_yhat_ = nullptr, *d_g_ = nullptr, *d_h_ = nullptr, *d_weights_ = nullptr, *d_tgain_ = nullptr;
   uint8_t *d_labels_ = nullptr;
+  unsigned *d_overflow_ = nullptr;     // set by the planner when a launch bound was too small
   unsigned char *d_active_ = nullptr;  // [level][feature] 1 = sampled at that level
   std::vector<unsigned char> active_host_;
   std::default_random_engine rnd_;
@@ -1743,6 +2067,17 @@ class HipTreeBuilder : public TreeBuilder {
   unsigned *d_leaf_ = nullptr, *d_node_first_ = nullptr, *d_node_items_ = nullptr, *d_nwork_ = nullptr,
            *d_wave_left_ = nullptr, *d_item_left_ = nullptr, *d_gmax_ = nullptr;
   RowBuffers buf_[2];
+  // streamed matrices: two block buffers filled by the copy stream, a staging
+  // buffer with the rows of the built nodes, a resident node id per row
+  bool streamed_ = false;
+  hipStream_t copy_stream_ = nullptr;
+  uint32_t *blk_[2] = {nullptr, nullptr};
+  hipEvent_t ev_ready_[2] = {nullptr, nullptr}, ev_free_[2] = {nullptr, nullptr};
+  bool buf_used_[2] = {false, false};
+  size_t next_copy_ = 0;  // running block-copy counter (selects the buffer)
+  RowBuffers stage_;
+  unsigned *d_node_of_ = nullptr, *d_blk_cnt_ = nullptr, *d_blk_seg_ = nullptr, *d_cursor_ = nullptr;
+  NodeSum *d_blk_tot_ = nullptr;
   NodeSum *d_tot_[2] = {nullptr, nullptr};
   unsigned *d_seg_[2] = {nullptr, nullptr};
   long long *d_hg_[2] = {nullptr, nullptr}, *d_hh_[2] = {nullptr, nullptr};

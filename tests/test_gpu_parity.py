@@ -142,6 +142,47 @@ def test_training_without_inspection(arb, oracle, objective):
     assert_same_training(arb, oracle, X, y, cfg, rounds=4, check_hist=False)
 
 
+# ----------------------------------------------- streamed (out-of-core) bins
+@pytest.mark.parametrize("objective", [0, 1])
+@pytest.mark.parametrize("trick", [True, False])
+@pytest.mark.parametrize("block_rows", [64, 1000, 4096, 1 << 20])
+def test_streamed_bins_match_oracle(arb, oracle, objective, trick, block_rows):
+    # upload_features = false: bins stay in pinned host blocks and are copied in
+    # block by block at every level (reference: garden.cu:603-604,
+    # hist_tree_grower.cu:335-366); results must not depend on it
+    X, y = make_data(9000, 11, objective, seed=13, nan_frac=0.02)
+    cfg = {"objective": objective, "method": 1,
+           "internals": {"hist_size": 63, "double_precision": True, "use_hist_subtraction_trick": trick,
+                         "upload_features": False, "stream_block_rows": block_rows},
+           "tree": {"max_depth": 5, "eta": 0.3, "lambda": 1.0}}
+    assert_same_training(arb, oracle, X, y, cfg, rounds=3)
+    assert_same_training(arb, oracle, X, y, cfg, rounds=3, check_hist=False)
+
+
+def test_streamed_wide_matrix_and_prequantised(arb, oracle):
+    rng = np.random.default_rng(3)
+    n, F = 20000, 50
+    bins = rng.integers(0, 256, size=(n, F), dtype=np.uint8)
+    y = (bins[:, 3].astype(np.int32) + bins[:, 40] > 250).astype(np.float32)
+    cfg = {"objective": 1, "method": 1,
+           "internals": {"hist_size": 256, "double_precision": False, "upload_features": False,
+                         "stream_block_rows": 6000},
+           "tree": {"max_depth": 4, "eta": 0.5, "lambda": 1.0}}
+    ob = oracle.Booster(bins, y=y, config=cfg, binned=True)
+    data = arb.DMatrix(bins, y=y, quantized=True)
+    g = arb.Garden(cfg, data)
+    for r in range(2):
+        ob.grow(1)
+        g.grow_tree()
+        to, tg = ob.tree(r), g.tree(r)
+        for key in ("fid", "quantized", "gain", "weights"):
+            assert np.array_equal(to[key], tg[key], equal_nan=True), (key, r)
+        assert np.array_equal(ob.leaf(), g.leaves())
+    assert np.array_equal(data.bins(), bins)
+    # host prediction walks the pinned blocks
+    assert np.allclose(g.predict(data), ob.predict(bins.astype(np.float32)), atol=1e-6)
+
+
 def test_training_255_bins_28_features(arb, oracle):
     X, y = make_data(60000, 28, 1, seed=11)
     cfg = {"objective": 1, "method": 1,
