@@ -49,8 +49,8 @@ struct InternalConfiguration {  // param.h:54-64
   bool upload_features = true;
   int hist_size = 255;
   // Extension (not a reference key): rows per pinned-host block when the bins
-  // are streamed (upload_features = false).
-  unsigned stream_block_rows = 1u << 22;
+  // are streamed (upload_features = false); 0 = chosen from the matrix size.
+  unsigned stream_block_rows = 0;
 };
 
 struct Configuration {  // param.h:66-74

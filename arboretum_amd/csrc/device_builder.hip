@@ -225,6 +225,11 @@ __global__ void k_init_root(NodeSum *tot, unsigned *seg_start, unsigned long lon
   }
 }
 
+__device__ __forceinline__ unsigned RankBelow(unsigned long long m) {
+  // number of set bits of m below this lane
+  return __builtin_amdgcn_mbcnt_hi((unsigned)(m >> 32), __builtin_amdgcn_mbcnt_lo((unsigned)m, 0u));
+}
+
 // ------------------------------------------------------------------ planner
 // Splits the row ranges of the selected nodes of a level into work items of
 // at most `rows_per_item` rows.  select: 0 = every node, 1 = the smaller
@@ -478,11 +483,6 @@ __device__ __forceinline__ void WaveOffsets(const WorkItem &it, const SplitRec &
   const unsigned rows_before = (it.begin - start) + RowsOfEarlierWaves(it, wave);
   *lo = start + lefts_before;
   *ro = start + (unsigned)s.left.c + rows_before - lefts_before;
-}
-
-__device__ __forceinline__ unsigned RankBelow(unsigned long long m) {
-  // number of set bits of m below this lane
-  return __builtin_amdgcn_mbcnt_hi((unsigned)(m >> 32), __builtin_amdgcn_mbcnt_lo((unsigned)m, 0u));
 }
 
 // Position of the k-th (0-based) set bit of the wave-uniform mask m; k < popcount(m).
@@ -845,14 +845,29 @@ k_stream_route(const uint32_t *__restrict__ bins, size_t bstride, unsigned rows,
   const int L = 1 << level;
   for (int i = threadIdx.x; i < L; i += blockDim.x) s_cnt[i] = 0;
   __syncthreads();
-  for (unsigned r = blockIdx.x * blockDim.x + threadIdx.x; r < rows; r += gridDim.x * blockDim.x) {
+  const int lane = threadIdx.x & 63;
+  const unsigned step = gridDim.x * blockDim.x;
+  for (unsigned r0 = blockIdx.x * blockDim.x; r0 < rows; r0 += step) {  // whole waves stay together
+    const unsigned r = r0 + threadIdx.x;
     unsigned nd = 0;
-    if (level > 0) {
-      const unsigned parent = node_of[r];
-      nd = parent * 2u + (GoesRight(bins, bstride, split[parent], r) ? 1u : 0u);
+    bool built = false;
+    if (r < rows) {
+      if (level > 0) {
+        const unsigned parent = node_of[r];
+        nd = parent * 2u + (GoesRight(bins, bstride, split[parent], r) ? 1u : 0u);
+      }
+      node_of[r] = nd;
+      built = NodeIsBuilt(tot, nd, level, trick);
     }
-    node_of[r] = nd;
-    if (NodeIsBuilt(tot, nd, level, trick)) atomicAdd(&s_cnt[nd], 1u);
+    // one LDS atomic per distinct node of the wave (64 lanes on one address serialise)
+    unsigned long long todo = __ballot(built);
+    while (todo) {
+      const int leader = __ffsll((long long)todo) - 1;
+      const unsigned lead_nd = (unsigned)__shfl((int)nd, leader);
+      const unsigned long long same = __ballot(built && nd == lead_nd);
+      if (lane == leader) atomicAdd(&s_cnt[lead_nd], (unsigned)__popcll(same));
+      todo &= ~same;
+    }
   }
   __syncthreads();
   for (int i = threadIdx.x; i < L; i += blockDim.x)
@@ -906,13 +921,34 @@ k_stream_gather(const uint32_t *__restrict__ bins, size_t bstride, int Q, unsign
                 const NodeSum *__restrict__ tot, unsigned *__restrict__ cursor,
                 uint32_t *__restrict__ st_bins, size_t sstride, float *__restrict__ st_g,
                 float *__restrict__ st_h) {
-  for (unsigned r = blockIdx.x * blockDim.x + threadIdx.x; r < rows; r += gridDim.x * blockDim.x) {
-    const unsigned nd = node_of[r];
-    if (!NodeIsBuilt(tot, nd, level, trick)) continue;
-    const unsigned d = atomicAdd(&cursor[nd], 1u);
-    for (int q = 0; q < Q; ++q) st_bins[(size_t)q * sstride + d] = bins[(size_t)q * bstride + r];
-    st_g[d] = g[r];
-    if (PAIR) st_h[d] = h[r];
+  const int lane = threadIdx.x & 63;
+  const unsigned step = gridDim.x * blockDim.x;
+  for (unsigned r0 = blockIdx.x * blockDim.x; r0 < rows; r0 += step) {  // whole waves stay together
+    const unsigned r = r0 + threadIdx.x;
+    unsigned nd = 0;
+    bool built = false;
+    if (r < rows) {
+      nd = node_of[r];
+      built = NodeIsBuilt(tot, nd, level, trick);
+    }
+    // one cursor atomic per distinct node of the wave
+    unsigned d = 0;
+    unsigned long long todo = __ballot(built);
+    while (todo) {
+      const int leader = __ffsll((long long)todo) - 1;
+      const unsigned lead_nd = (unsigned)__shfl((int)nd, leader);
+      const unsigned long long same = __ballot(built && nd == lead_nd);
+      unsigned base = 0;
+      if (lane == leader) base = atomicAdd(&cursor[lead_nd], (unsigned)__popcll(same));
+      base = (unsigned)__shfl((int)base, leader);
+      if (built && nd == lead_nd) d = base + RankBelow(same);
+      todo &= ~same;
+    }
+    if (built) {
+      for (int q = 0; q < Q; ++q) st_bins[(size_t)q * sstride + d] = bins[(size_t)q * bstride + r];
+      st_g[d] = g[r];
+      if (PAIR) st_h[d] = h[r];
+    }
   }
 }
 
@@ -1247,6 +1283,9 @@ void QuantiseOnDevice(DataMatrix *data, int hist_size, bool verbose, bool stream
   uint32_t *d_col = nullptr;  // streamed: one quad column at a time on the device
   size_t nblocks = 0;
   if (streamed) {
+    // default: 16M-row blocks (2 GB of bins at 128 features), large enough that
+    // the per-block fixed costs vanish against the PCIe copy
+    if (block_rows == 0) block_rows = std::min<size_t>(n, (size_t)1 << 24);
     if (block_rows < 64) block_rows = 64;
     block_rows = (block_rows + 63) / 64 * 64;
     dm->block_rows = block_rows;

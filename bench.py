@@ -57,6 +57,65 @@ def config(max_depth=8, hist_size=256):
                      "min_leaf_size": 1, "colsample_bytree": 1.0, "colsample_bylevel": 1.0}}
 
 
+def make_stream_workload(rows, features=128, seed=0):
+    """BASELINE config 5 shape: uint8 bins, per column either U{0..255} or a
+    Binomial(255, 0.3) look-alike (rounded normal), labels from a random depth-6
+    tree on the bins with 10 % flips.  A base tile of at most 4M rows is generated
+    and repeated (the content does not change what is measured: PCIe streaming)."""
+    rng = np.random.default_rng(seed)
+    base = min(rows, 1 << 22)
+    tile = rng.integers(0, 256, size=(base, features), dtype=np.uint8)
+    for f in range(0, features, 2):
+        tile[:, f] = np.clip(np.rint(rng.normal(76.5, 7.3, size=base)), 0, 255).astype(np.uint8)
+    reps = (rows + base - 1) // base
+    bins = np.tile(tile, (reps, 1))[:rows]
+    node = np.zeros(rows, dtype=np.int32)
+    for level in range(6):
+        nn = 1 << level
+        fid = rng.integers(0, features, size=nn)
+        thr = rng.integers(40, 200, size=nn)
+        node = 2 * node + (bins[np.arange(rows), fid[node]] > thr[node])
+    leaf_label = rng.integers(0, 2, size=64)
+    y = leaf_label[node].astype(np.float32)
+    flip = rng.random(rows) < 0.1
+    y[flip] = 1.0 - y[flip]
+    return bins, y
+
+
+def stream_mode(args, arb):
+    """Out-of-core leg: bins in pinned host memory, streamed block by block at
+    every level (not the headline metric; prints its own JSON line)."""
+    bins, y = make_stream_workload(args.stream_rows, args.stream_features)
+    cfg = config(args.max_depth, 256)
+    cfg["internals"]["upload_features"] = False
+    cfg["internals"]["stream_block_rows"] = args.stream_block_rows
+    data = arb.DMatrix(bins, y=y, quantized=True)
+    del bins
+    model = arb.Garden(cfg, data)
+    model.grow_tree()      # first call packs the blocks into pinned memory
+    model.synchronize()
+    if args.stream_timing:
+        model.enable_timing(True)
+    s0 = model.rows_scanned()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        model.grow_tree()
+    model.synchronize()
+    dt = time.perf_counter() - t0
+    scanned = model.rows_scanned() - s0
+    passes = args.max_depth + 1    # one copy of every block per level + the leaf pass
+    host_bytes = args.stream_rows * ((args.stream_features + 3) // 4 * 4)
+    print(json.dumps({
+        "metric": "streamed (out-of-core) tree growing, bins in pinned host memory",
+        "sec_per_tree": dt / args.steps, "steps": args.steps,
+        "rows": args.stream_rows, "features": args.stream_features, "block_rows": args.stream_block_rows,
+        "host_bin_bytes": host_bytes, "passes_per_tree": passes,
+        "h2d_GBps": host_bytes * passes * args.steps / dt / 1e9,
+        "hist_updates_per_s": scanned * args.stream_features / dt,
+        "phase_ms_per_tree": ({k: v / args.steps for k, v in model.timings().items() if k.endswith("_ms")}
+                              if args.stream_timing else None)}))
+
+
 def cpu_baseline(X, y, cfg, sample_rows, trees):
     """The CPU checker on the first `sample_rows` rows (same columns, same
     configuration), all host cores."""
@@ -89,6 +148,11 @@ def main():
     ap.add_argument("--cpu-rows", type=int, default=10_500_000)
     ap.add_argument("--cpu-trees", type=int, default=8)
     ap.add_argument("--no-cpu", action="store_true")
+    ap.add_argument("--mode", choices=["resident", "stream"], default="resident")
+    ap.add_argument("--stream-rows", type=int, default=64_000_000)
+    ap.add_argument("--stream-features", type=int, default=128)
+    ap.add_argument("--stream-block-rows", type=int, default=1 << 22)
+    ap.add_argument("--stream-timing", action="store_true")
     ap.add_argument("--copy-probe", type=int, default=0, metavar="MiB",
                     help="also run one device-to-device copy of this many MiB (a kernel of known traffic, "
                          "used to scale the FETCH_SIZE / WRITE_SIZE counters of a rocprofv3 --pmc run)")
@@ -102,6 +166,9 @@ def main():
 
     if args.copy_probe:
         arb.copy_probe(args.copy_probe << 20)
+    if args.mode == "stream":
+        stream_mode(args, arb)
+        return
 
     X, y = make_workload(args.rows, args.features)
     cfg = config(args.max_depth, args.hist_size)
