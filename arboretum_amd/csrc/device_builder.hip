@@ -72,6 +72,21 @@ constexpr unsigned kMaxHistRows = 64512;  // rows per histogram work item (< 2^1
 constexpr int kCountShift = 47;           // word0 = count << 47 | g
 constexpr int kMaxPlanNodes = 4096;       // nodes per level the planner handles
 constexpr size_t kLdsBudget = 160 * 1024;
+// Replicas of the most frequent bin of every feature in the LDS histogram.
+// LDS atomics of lanes that hit one address are serialised (a wave whose 64
+// lanes add to one word takes ~40x the time of a conflict-free one), and
+// real matrices concentrate rows in one bin per feature (missing values,
+// zeros, the top category).  Lanes that hit that bin add to replica
+// lane % kHotReplicas instead; the replicas are folded into the bin before
+// the histogram leaves LDS.  Integer sums: the result does not change.
+#ifndef ARB_HOT_REPLICAS
+#define ARB_HOT_REPLICAS 16
+#endif
+constexpr int kHotReplicas = ARB_HOT_REPLICAS;  // power of two, 0 = off
+// LDS bytes of a histogram of nq quads
+constexpr size_t HistLdsBytes(int nq, bool pair) {
+  return (size_t)nq * 4 * (kSlots + kHotReplicas) * 8 * (pair ? 2 : 1);
+}
 
 struct NodeSum {
   long long g;
@@ -332,39 +347,80 @@ constexpr unsigned kChunkRows = 128;
 constexpr unsigned kChunkStep = kChunkRows * kItemWaves;
 
 // ---------------------------------------------------------------- histogram
-// Adds the four features of quad q (bins packed in b4) of one row.
+// LDS layout of a histogram of NQ quads: word0[nbin], replicas of word0
+// [NQ*4*kHotReplicas], then (PAIR) word1 and its replicas in the same order.
+template <int NQ>
+struct HistLds {
+  static constexpr int nbin = NQ * 4 * kSlots;
+  static constexpr int nrep = NQ * 4 * kHotReplicas;
+  static constexpr int word1 = nbin + nrep;  // offset of word1 of the same entry
+};
+
+// Adds one row (bins of its NQ quads in b) to the LDS histogram.  hot[q] packs
+// the replicated bin of each feature of quad q (wave-uniform).
 template <bool PAIR, int NQ>
 __device__ __forceinline__ void AccumulateRow(unsigned long long *__restrict__ lds,
-                                              const uint32_t (&b)[NQ], float gv, float hv, int sg,
-                                              int sh, int q_first, int F) {
-  constexpr int nbin = NQ * 4 * kSlots;
+                                              const uint32_t (&b)[NQ], const uint32_t (&hot)[NQ],
+                                              float gv, float hv, int sg, int sh, int q_first, int F) {
+  using L = HistLds<NQ>;
   const unsigned long long w0 = (1ull << kCountShift) + (unsigned long long)ToFixed(gv, sg);
   unsigned long long w1 = 0;
   if (PAIR) w1 = (unsigned long long)ToFixed(hv, sh);
+  const unsigned rep = kHotReplicas > 0 ? (unsigned)L::nbin + (threadIdx.x & (unsigned)(kHotReplicas - 1)) : 0u;
 #pragma unroll
   for (int q = 0; q < NQ; ++q) {
 #pragma unroll
     for (int c = 0; c < 4; ++c) {
       // only the last quad can hold padding features
       if (q < NQ - 1 || (q_first + q) * 4 + c < F) {
-        const unsigned idx = (unsigned)(q * 4 + c) * kSlots + ((b[q] >> (8 * c)) & 255u);
+        const unsigned bin = (b[q] >> (8 * c)) & 255u;
+        unsigned idx = (unsigned)(q * 4 + c) * kSlots + bin;
+        if (kHotReplicas > 0) {
+          const unsigned hb = (hot[q] >> (8 * c)) & 255u;
+          idx = bin == hb ? rep + (unsigned)(q * 4 + c) * kHotReplicas : idx;
+        }
         atomicAdd(&lds[idx], w0);
-        if (PAIR) atomicAdd(&lds[nbin + idx], w1);
+        if (PAIR) atomicAdd(&lds[L::word1 + idx], w1);
       }
     }
   }
 }
 
+// Loads the replicated bins of quads [q_first, q_first + NQ).
+template <int NQ>
+__device__ __forceinline__ void LoadHot(const uint32_t *__restrict__ hot_bins, int q_first, uint32_t (&hot)[NQ]) {
+#pragma unroll
+  for (int q = 0; q < NQ; ++q) hot[q] = kHotReplicas > 0 ? hot_bins[q_first + q] : 0u;
+}
+
+// Folds the replicas into their bins and writes the histogram to the slab of
+// work item w.  Called by the whole workgroup after the last LDS update.
 template <bool PAIR, int NQ>
-__device__ __forceinline__ void FlushSlab(const unsigned long long *__restrict__ lds,
+__device__ __forceinline__ void FlushSlab(unsigned long long *__restrict__ lds, const uint32_t (&hot)[NQ],
                                           unsigned long long *__restrict__ slab, unsigned w,
                                           int nbin_total, int q_first) {
+  using L = HistLds<NQ>;
+  __syncthreads();
+  if (kHotReplicas > 0) {
+    // one thread per (feature, word)
+    const int f = threadIdx.x >> 1, second = threadIdx.x & 1;
+    if (f < NQ * 4 && (PAIR || !second)) {
+      uint32_t hq = 0;
+#pragma unroll
+      for (int q = 0; q < NQ; ++q) hq = q == (f >> 2) ? hot[q] : hq;
+      const unsigned hb = (hq >> (8 * (f & 3))) & 255u;
+      const int off = second ? L::word1 : 0;
+      unsigned long long acc = lds[off + f * kSlots + hb];
+      for (int k = 0; k < kHotReplicas; ++k) acc += lds[off + L::nbin + f * kHotReplicas + k];
+      lds[off + f * kSlots + hb] = acc;
+    }
+    __syncthreads();
+  }
   // slab layout per work item: word0[nbin_total], word1[nbin_total]
-  constexpr int nbin = NQ * 4 * kSlots;
   unsigned long long *out = slab + (size_t)w * nbin_total * (PAIR ? 2 : 1) + (size_t)q_first * 4 * kSlots;
-  for (int i = threadIdx.x; i < nbin; i += kHistThreads) {
+  for (int i = threadIdx.x; i < L::nbin; i += kHistThreads) {
     out[i] = lds[i];
-    if (PAIR) out[nbin_total + i] = lds[nbin + i];
+    if (PAIR) out[nbin_total + i] = lds[L::word1 + i];
   }
 }
 
@@ -375,14 +431,16 @@ __global__ void __launch_bounds__(kHistThreads)
 k_hist(const uint32_t *__restrict__ bins, size_t stride, int q0, int F,
        const float *__restrict__ g, const float *__restrict__ h, const int *__restrict__ shifts,
        const WorkItem *__restrict__ work, const unsigned *__restrict__ n_work,
-       unsigned long long *__restrict__ slab, int nbin_total) {
+       unsigned long long *__restrict__ slab, int nbin_total, const uint32_t *__restrict__ hot_bins) {
   extern __shared__ unsigned long long lds[];
   const unsigned w = blockIdx.x;
   if (w >= *n_work) return;
   const WorkItem it = work[w];
-  constexpr int words = NQ * 4 * kSlots * (PAIR ? 2 : 1);
+  constexpr int words = (int)(HistLdsBytes(NQ, PAIR) / 8);
   for (int i = threadIdx.x; i < words; i += kHistThreads) lds[i] = 0ull;
   __syncthreads();
+  uint32_t hot[NQ];
+  LoadHot<NQ>(hot_bins, q0, hot);
   const int sg = shifts[0], sh = shifts[1];
   const uint32_t *bq = bins + (size_t)q0 * stride;
   for (unsigned base = it.begin; base < it.end; base += 2 * kHistThreads) {
@@ -397,11 +455,10 @@ k_hist(const uint32_t *__restrict__ bins, size_t stride, int q0, int F,
     }
     const float g0 = g[a0], g1 = g[a1];
     const float h0 = PAIR ? h[a0] : 0.0f, h1 = PAIR ? h[a1] : 0.0f;
-    if (v0) AccumulateRow<PAIR, NQ>(lds, b0, g0, h0, sg, sh, q0, F);
-    if (v1) AccumulateRow<PAIR, NQ>(lds, b1, g1, h1, sg, sh, q0, F);
+    if (v0) AccumulateRow<PAIR, NQ>(lds, b0, hot, g0, h0, sg, sh, q0, F);
+    if (v1) AccumulateRow<PAIR, NQ>(lds, b1, hot, g1, h1, sg, sh, q0, F);
   }
-  __syncthreads();
-  FlushSlab<PAIR, NQ>(lds, slab, w, nbin_total, q0);
+  FlushSlab<PAIR, NQ>(lds, hot, slab, w, nbin_total, q0);
 }
 
 // ---------------------------------------------------------------- partition
@@ -520,9 +577,9 @@ struct Pending {
 // becomes the new P.
 template <bool PAIR, int NQ>
 __device__ __forceinline__ void MergePending(unsigned long long *__restrict__ lds, Pending<NQ> &P,
-                                             unsigned long long &pmask, const uint32_t (&xb)[NQ], float xg,
-                                             float xh, unsigned long long xm, int lane, int sg, int sh,
-                                             int F) {
+                                             unsigned long long &pmask, const uint32_t (&hot)[NQ],
+                                             const uint32_t (&xb)[NQ], float xg, float xh,
+                                             unsigned long long xm, int lane, int sg, int sh, int F) {
   const unsigned nx = (unsigned)__popcll(xm);
   if (nx == 0) return;  // wave-uniform
   const unsigned np = (unsigned)__popcll(pmask);
@@ -546,7 +603,7 @@ __device__ __forceinline__ void MergePending(unsigned long long *__restrict__ ld
   }
   pmask |= __ballot(take);
   if (np + moved == 64u) {  // wave-uniform: P is full
-    AccumulateRow<PAIR, NQ>(lds, P.b, P.g, P.h, sg, sh, 0, F);
+    AccumulateRow<PAIR, NQ>(lds, P.b, hot, P.g, P.h, sg, sh, 0, F);
     const bool keep = ((xm >> lane) & 1ull) && RankBelow(xm) >= moved;
 #pragma unroll
     for (int q = 0; q < NQ; ++q) P.b[q] = xb[q];
@@ -570,7 +627,7 @@ k_part_hist(const uint32_t *__restrict__ bins, uint32_t *__restrict__ bins_out, 
             const unsigned *__restrict__ seg_start, const WorkItem *__restrict__ work,
             const unsigned *__restrict__ n_work, const unsigned *__restrict__ wave_left,
             const unsigned *__restrict__ item_left, unsigned long long *__restrict__ slab,
-            int nbin_total) {
+            int nbin_total, const uint32_t *__restrict__ hot_bins) {
   extern __shared__ unsigned long long lds[];
   __shared__ unsigned s_tmp[kItemWaves + 1];
   const unsigned w = blockIdx.x;
@@ -579,8 +636,10 @@ k_part_hist(const uint32_t *__restrict__ bins, uint32_t *__restrict__ bins_out, 
   const SplitRec s = split[it.node];
   const unsigned long long cl = s.left.c, cr = tot[it.node].c - cl;
   const bool build_right = cl > cr;  // ties -> left (hist_grad_sum.cu:288-290)
-  constexpr int words = NQ * 4 * kSlots * (PAIR ? 2 : 1);
+  constexpr int words = (int)(HistLdsBytes(NQ, PAIR) / 8);
   for (int i = threadIdx.x; i < words; i += kHistThreads) lds[i] = 0ull;
+  uint32_t hot[NQ];
+  LoadHot<NQ>(hot_bins, 0, hot);
   const int sg = shifts[0], sh = shifts[1];
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const unsigned wb = it.begin + wave * kChunkRows, we = it.end;
@@ -663,8 +722,8 @@ k_part_hist(const uint32_t *__restrict__ bins, uint32_t *__restrict__ bins_out, 
       lo += nl0 + (unsigned)__popcll(lm1);
       ro += nr0 + (unsigned)__popcll(rm1);
     }
-    MergePending<PAIR, NQ>(lds, P, pmask, b0, g0, h0, __ballot(v0 && right0 == build_right), lane, sg, sh, F);
-    MergePending<PAIR, NQ>(lds, P, pmask, b1, g1, h1, __ballot(v1 && right1 == build_right), lane, sg, sh, F);
+    MergePending<PAIR, NQ>(lds, P, pmask, hot, b0, g0, h0, __ballot(v0 && right0 == build_right), lane, sg, sh, F);
+    MergePending<PAIR, NQ>(lds, P, pmask, hot, b1, g1, h1, __ballot(v1 && right1 == build_right), lane, sg, sh, F);
 #pragma unroll
     for (int q = 0; q < NQ; ++q) {
       b0[q] = nb0[q];
@@ -675,9 +734,8 @@ k_part_hist(const uint32_t *__restrict__ bins, uint32_t *__restrict__ bins_out, 
     h0 = nh0;
     h1 = nh1;
   }
-  if ((pmask >> lane) & 1ull) AccumulateRow<PAIR, NQ>(lds, P.b, P.g, P.h, sg, sh, 0, F);
-  __syncthreads();
-  FlushSlab<PAIR, NQ>(lds, slab, w, nbin_total, 0);
+  if ((pmask >> lane) & 1ull) AccumulateRow<PAIR, NQ>(lds, P.b, hot, P.g, P.h, sg, sh, 0, F);
+  FlushSlab<PAIR, NQ>(lds, hot, slab, w, nbin_total, 0);
 }
 
 // Stable partition alone (matrices too wide for the fused pass): any number
@@ -798,6 +856,26 @@ k_hist_reduce(const unsigned long long *__restrict__ slab, int nbin_total,
       hc[so] = pc[po] - ac;
     }
   }
+}
+
+// Picks the bin to replicate in LDS for every feature: the one holding most
+// rows of the root histogram.  Only the speed of later histograms depends on
+// the choice.  One thread per feature; hot[q] packs the four bins of quad q.
+__global__ void k_pick_hot(const unsigned *__restrict__ hc, int Q, uint32_t *__restrict__ hot) {
+  const int q = blockIdx.x * blockDim.x + threadIdx.x;
+  if (q >= Q) return;
+  uint32_t packed = 0;
+  for (int c = 0; c < 4; ++c) {
+    const unsigned *cnt = hc + (size_t)(q * 4 + c) * kSlots;
+    unsigned best = 0, best_cnt = cnt[0];
+    for (unsigned b = 1; b < (unsigned)kSlots; ++b)
+      if (cnt[b] > best_cnt) {
+        best_cnt = cnt[b];
+        best = b;
+      }
+    packed |= best << (8 * c);
+  }
+  hot[q] = packed;
 }
 
 // Root totals = sum over the slots of feature 0 of the root histogram (every
@@ -1417,23 +1495,23 @@ void AllowLds(K kernel, size_t bytes) {
 template <bool PAIR, int NQ>
 void LaunchHistNQ(hipStream_t st, unsigned grid, const uint32_t *bins, size_t stride, int q0, int F,
                   const float *g, const float *h, const int *shifts, const WorkItem *work,
-                  const unsigned *n_work, unsigned long long *slab, int nbin_total) {
-  const size_t lds = (size_t)NQ * 4 * kSlots * 8 * (PAIR ? 2 : 1);
+                  const unsigned *n_work, unsigned long long *slab, int nbin_total, const uint32_t *hot) {
+  const size_t lds = HistLdsBytes(NQ, PAIR);
   static bool configured = false;
   if (!configured) {
     AllowLds(k_hist<PAIR, NQ>, lds);
     configured = true;
   }
   hipLaunchKernelGGL((k_hist<PAIR, NQ>), dim3(grid), dim3(kHistThreads), lds, st, bins, stride, q0, F, g, h,
-                     shifts, work, n_work, slab, nbin_total);
+                     shifts, work, n_work, slab, nbin_total, hot);
 }
 
 template <bool PAIR>
 void LaunchHist(int nq, hipStream_t st, unsigned grid, const uint32_t *bins, size_t stride, int q0, int F,
                 const float *g, const float *h, const int *shifts, const WorkItem *work,
-                const unsigned *n_work, unsigned long long *slab, int nbin_total) {
+                const unsigned *n_work, unsigned long long *slab, int nbin_total, const uint32_t *hot) {
 #define ARB_CASE(N) \
-  case N: LaunchHistNQ<PAIR, N>(st, grid, bins, stride, q0, F, g, h, shifts, work, n_work, slab, nbin_total); break;
+  case N: LaunchHistNQ<PAIR, N>(st, grid, bins, stride, q0, F, g, h, shifts, work, n_work, slab, nbin_total, hot); break;
   switch (nq) {
     ARB_CASE(1) ARB_CASE(2) ARB_CASE(3) ARB_CASE(4) ARB_CASE(5) ARB_CASE(6) ARB_CASE(7) ARB_CASE(8) ARB_CASE(9)
     default: throw std::runtime_error("internal: bad quad count");
@@ -1460,11 +1538,12 @@ struct FusedArgs {
   const unsigned *item_left;
   unsigned long long *slab;
   int nbin_total;
+  const uint32_t *hot;
 };
 
 template <bool PAIR, int NQ, bool WRITE>
 void LaunchFusedNQ(hipStream_t st, unsigned grid, const FusedArgs &a) {
-  const size_t lds = (size_t)NQ * 4 * kSlots * 8 * (PAIR ? 2 : 1);
+  const size_t lds = HistLdsBytes(NQ, PAIR);
   static bool configured = false;
   if (!configured) {
     AllowLds(k_part_hist<PAIR, NQ, WRITE>, lds);
@@ -1472,7 +1551,7 @@ void LaunchFusedNQ(hipStream_t st, unsigned grid, const FusedArgs &a) {
   }
   hipLaunchKernelGGL((k_part_hist<PAIR, NQ, WRITE>), dim3(grid), dim3(kHistThreads), lds, st, a.bins, a.bins_out,
                      a.stride, a.F, a.g, a.g_out, a.h, a.h_out, a.shifts, a.split, a.tot, a.seg_start, a.work,
-                     a.n_work, a.wave_left, a.item_left, a.slab, a.nbin_total);
+                     a.n_work, a.wave_left, a.item_left, a.slab, a.nbin_total, a.hot);
 }
 
 template <bool PAIR, bool WRITE>
@@ -1507,7 +1586,7 @@ class HipTreeBuilder : public TreeBuilder {
     HIP_OK(hipStreamCreateWithFlags(&stream_, hipStreamNonBlocking));
 
     // quads per histogram launch, limited by LDS
-    const size_t per_quad = (size_t)4 * kSlots * 8 * (pair_ ? 2 : 1);
+    const size_t per_quad = HistLdsBytes(1, pair_);
     quads_per_group_ = (int)std::min<size_t>(std::min<size_t>((kLdsBudget - 1024) / per_quad, kMaxGroupQuads), Q_);
     // the fused partition + histogram pass holds one histogram of all
     // features and builds only the smaller child
@@ -1577,6 +1656,8 @@ class HipTreeBuilder : public TreeBuilder {
     d_item_left_ = DevAlloc<unsigned>(max_part_items_);
     d_slab_ = DevAlloc<unsigned long long>((size_t)std::max(max_hist_items_, max_part_items_) * nbin_total_ * (pair_ ? 2 : 1));
     d_shifts_ = DevAlloc<int>(2);
+    d_hot_ = DevAlloc<uint32_t>(Q_);
+    HIP_OK(hipMemsetAsync(d_hot_, 0, Q_ * sizeof(uint32_t), stream_));
     d_gmax_ = DevAlloc<unsigned>(1);
     d_rows_scanned_ = DevAlloc<unsigned long long>(1);
     d_overflow_ = DevAlloc<unsigned>(1);
@@ -1601,7 +1682,7 @@ class HipTreeBuilder : public TreeBuilder {
     (void)hipStreamSynchronize(stream_);
     void *ptrs[] = {d_y_, d_labels_, d_yhat_, d_g_, d_h_, d_leaf_, d_split_, d_cand_, d_node_first_,
                     d_node_items_, d_hwork_, d_pwork_, d_nwork_, d_wave_left_, d_item_left_, d_slab_,
-                    d_shifts_, d_gmax_, d_rows_scanned_, d_tfid_, d_tbin_, d_tgain_, d_weights_, d_active_, d_overflow_};
+                    d_shifts_, d_gmax_, d_rows_scanned_, d_tfid_, d_tbin_, d_tgain_, d_weights_, d_active_, d_overflow_, d_hot_};
     for (void *p : ptrs)
       if (p) (void)hipFree(p);
     for (int b = 0; b < 2; ++b) {
@@ -1762,9 +1843,9 @@ class HipTreeBuilder : public TreeBuilder {
     for (int q0 = 0; q0 < Q_; q0 += quads_per_group_) {
       const int nq = std::min(quads_per_group_, Q_ - q0);
       if (pair_)
-        LaunchHist<true>(nq, stream_, grid, cur.bins, stride_, q0, F_, cur.g, cur.h, d_shifts_, d_hwork_, d_nwork_, d_slab_, nbin_total_);
+        LaunchHist<true>(nq, stream_, grid, cur.bins, stride_, q0, F_, cur.g, cur.h, d_shifts_, d_hwork_, d_nwork_, d_slab_, nbin_total_, d_hot_);
       else
-        LaunchHist<false>(nq, stream_, grid, cur.bins, stride_, q0, F_, cur.g, cur.h, d_shifts_, d_hwork_, d_nwork_, d_slab_, nbin_total_);
+        LaunchHist<false>(nq, stream_, grid, cur.bins, stride_, q0, F_, cur.g, cur.h, d_shifts_, d_hwork_, d_nwork_, d_slab_, nbin_total_, d_hot_);
       if (timing_) ++(root ? timings_.hist_root_launches : timings_.hist_deep_launches);
     }
     if (timing_ && root) timings_.hist_root_rows += n_;
@@ -1807,6 +1888,7 @@ class HipTreeBuilder : public TreeBuilder {
         HistOfNodes(orig, state, 1, false, n_, true);
         Reduce(1, hb, false, state, false);
         hipLaunchKernelGGL(k_root_from_hist, dim3(1), dim3(64), 0, stream_, d_hg_[hb], d_hh_[hb], d_tot_[state]);
+        PickHotBins(hb);
       } else {
         // rows are in the order of level-1; the parents' state is state ^ 1
         const int ps = state ^ 1, PL = L >> 1;
@@ -1824,7 +1906,7 @@ class HipTreeBuilder : public TreeBuilder {
           }
           Mark(last ? kFusedLast : kHistDeep);
           FusedArgs a{src.bins, dst.bins, stride_, F_, src.g, dst.g, src.h, dst.h, d_shifts_, d_split_,
-                      d_tot_[ps], d_seg_[ps], d_pwork_, d_nwork_ + 1, d_wave_left_, d_item_left_, d_slab_, nbin_total_};
+                      d_tot_[ps], d_seg_[ps], d_pwork_, d_nwork_ + 1, d_wave_left_, d_item_left_, d_slab_, nbin_total_, d_hot_};
           if (pair_) {
             if (last) LaunchFused<true, false>(Q_, stream_, grid, a);
             else LaunchFused<true, true>(Q_, stream_, grid, a);
@@ -2008,15 +2090,17 @@ class HipTreeBuilder : public TreeBuilder {
           const int nq = std::min(quads_per_group_, Q_ - q0);
           if (pair_)
             LaunchHist<true>(nq, stream_, grid, stage_.bins, br, q0, F_, stage_.g, stage_.h, d_shifts_, d_hwork_,
-                             d_nwork_, d_slab_, nbin_total_);
+                             d_nwork_, d_slab_, nbin_total_, d_hot_);
           else
             LaunchHist<false>(nq, stream_, grid, stage_.bins, br, q0, F_, stage_.g, stage_.h, d_shifts_, d_hwork_,
-                              d_nwork_, d_slab_, nbin_total_);
+                              d_nwork_, d_slab_, nbin_total_, d_hot_);
         }
         Reduce(L, hb, false, state, false, b > 0);
       }
-      if (level == 0)
+      if (level == 0) {
         hipLaunchKernelGGL(k_root_from_hist, dim3(1), dim3(64), 0, stream_, d_hg_[hb], d_hh_[hb], d_tot_[state]);
+        PickHotBins(hb);
+      }
       if (trick)
         hipLaunchKernelGGL(k_sibling, dim3((nbin_total_ + 255) / 256, L), dim3(256), 0, stream_, d_hg_[hb], d_hh_[hb],
                            d_hc_[hb], d_hg_[hb ^ 1], d_hh_[hb ^ 1], d_hc_[hb ^ 1], d_tot_[state], level, nbin_total_);
@@ -2063,6 +2147,14 @@ class HipTreeBuilder : public TreeBuilder {
     // the previous tree's kernels may still read the mask
     HIP_OK(hipStreamSynchronize(stream_));
     HIP_OK(hipMemcpy(d_active_, active_host_.data(), active_host_.size(), hipMemcpyHostToDevice));
+  }
+
+  // After the first root histogram of this builder: choose the bins that get
+  // LDS replicas from its counts.
+  void PickHotBins(int hb) {
+    if (hot_ready_ || kHotReplicas == 0) return;
+    hipLaunchKernelGGL(k_pick_hot, dim3((Q_ + 63) / 64), dim3(64), 0, stream_, d_hc_[hb], Q_, d_hot_);
+    hot_ready_ = true;
   }
 
   void KeepHist(int level, int L, int hb) {
@@ -2127,6 +2219,8 @@ class HipTreeBuilder : public TreeBuilder {
   unsigned max_hist_items_ = 0, max_part_items_ = 0;
   unsigned long long *d_slab_ = nullptr, *d_rows_scanned_ = nullptr;
   int *d_shifts_ = nullptr, *d_tfid_ = nullptr, *d_tbin_ = nullptr;
+  uint32_t *d_hot_ = nullptr;  // per quad: the replicated bin of each of its features
+  bool hot_ready_ = false;
   std::vector<std::vector<int64_t>> kept_hist_;
   std::vector<hipEvent_t> event_pool_;
   size_t event_used_ = 0;

@@ -148,6 +148,9 @@ def main():
     ap.add_argument("--cpu-rows", type=int, default=10_500_000)
     ap.add_argument("--cpu-trees", type=int, default=8)
     ap.add_argument("--no-cpu", action="store_true")
+    ap.add_argument("--nan-frac", type=float, default=0.0,
+                    help="stress variant: this fraction of the feature values is replaced by NaN (all land in "
+                         "one bin per feature; needs --hist-size <= 255)")
     ap.add_argument("--mode", choices=["resident", "stream"], default="resident")
     ap.add_argument("--stream-rows", type=int, default=64_000_000)
     ap.add_argument("--stream-features", type=int, default=128)
@@ -171,6 +174,10 @@ def main():
         return
 
     X, y = make_workload(args.rows, args.features)
+    if args.nan_frac > 0:
+        rng = np.random.default_rng(1)
+        for f in range(args.features):
+            X[rng.random(args.rows, dtype=np.float32) < args.nan_frac, f] = np.nan
     cfg = config(args.max_depth, args.hist_size)
     data = arb.DMatrix(X, y=y)
     t0 = time.perf_counter()

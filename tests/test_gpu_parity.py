@@ -223,6 +223,33 @@ def test_max_depth_1(arb, oracle):
     assert_same_training(arb, oracle, X, y, cfg, rounds=2)
 
 
+def _skewed_matrix(n, seed):
+    """Columns whose rows pile up in one bin: 30 % missing, Zipf categories, a binary flag, zeros, a constant."""
+    rng = np.random.default_rng(seed)
+    X = rng.normal(size=(n, 13)).astype(np.float32)
+    X[:, :4][rng.random((n, 4)) < 0.3] = np.nan
+    X[:, 4:7] = np.minimum(rng.zipf(1.3, size=(n, 3)), 200).astype(np.float32)
+    X[:, 7] = (rng.random(n) < 0.05).astype(np.float32)
+    X[:, 8] = np.where(rng.random(n) < 0.9, 0.0, X[:, 8])
+    X[:, 9] = 3.5
+    X[:, 10] = np.nan
+    s = np.nan_to_num(X[:, 0]) + (X[:, 4] > 2) - X[:, 7] + 0.5 * X[:, 11]
+    y = (rng.random(n) < 1 / (1 + np.exp(-s))).astype(np.float32)
+    return X, y
+
+
+@pytest.mark.parametrize("upload", [True, False])
+@pytest.mark.parametrize("objective", [0, 1])
+def test_rows_concentrated_in_one_bin(arb, oracle, upload, objective):
+    # exercises the LDS replicas of the most frequent bin of every feature
+    X, y = _skewed_matrix(40000, seed=21)
+    cfg = {"objective": objective, "method": 1,
+           "internals": {"hist_size": 255, "double_precision": True, "upload_features": upload,
+                         "stream_block_rows": 9000},
+           "tree": {"max_depth": 6, "eta": 0.3, "lambda": 1.0, "min_child_weight": 1.0}}
+    assert_same_training(arb, oracle, X, y, cfg, rounds=3)
+
+
 def test_constant_features_give_unsplit_nodes(arb, oracle):
     X = np.ones((500, 3), np.float32)
     y = np.arange(500, dtype=np.float32)
