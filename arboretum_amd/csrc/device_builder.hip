@@ -67,25 +67,26 @@ constexpr int kSlots = 256;               // histogram slots per feature (uint8 
 constexpr int kHistThreads = 1024;        // one workgroup per CU, 16 waves
 constexpr int kItemWaves = kHistThreads / 64;  // waves per work item in row passes
 constexpr unsigned kPartRows = 16384;     // rows per work item of the stand-alone partition
-constexpr int kMaxGroupQuads = 9;         // quads per histogram launch (compile-time variants)
+constexpr int kMaxGroupQuads = 8;         // quads per histogram launch (compile-time variants, whole blocks)
 constexpr unsigned kMaxHistRows = 64512;  // rows per histogram work item (< 2^16)
 constexpr int kCountShift = 47;           // word0 = count << 47 | g
 constexpr int kMaxPlanNodes = 4096;       // nodes per level the planner handles
 constexpr size_t kLdsBudget = 160 * 1024;
-// Replicas of the most frequent bin of every feature in the LDS histogram.
-// LDS atomics of lanes that hit one address are serialised (a wave whose 64
-// lanes add to one word takes ~40x the time of a conflict-free one), and
-// real matrices concentrate rows in one bin per feature (missing values,
-// zeros, the top category).  Lanes that hit that bin add to replica
-// lane % kHotReplicas instead; the replicas are folded into the bin before
-// the histogram leaves LDS.  Integer sums: the result does not change.
-#ifndef ARB_HOT_REPLICAS
-#define ARB_HOT_REPLICAS 16
-#endif
-constexpr int kHotReplicas = ARB_HOT_REPLICAS;  // power of two, 0 = off
+// LDS histograms are laid out in blocks of 16 features (4 quads):
+//   entry(f, bin) = (f / 16) * 4096 + bin * 16 + f % 16.
+// A 64-bit LDS atomic is executed 16 lanes per pass, and two of those lanes
+// collide when their addresses share a bank pair (entry % 16).  With this
+// layout the bank pair is the feature, and the kernels let the 16 lanes of a
+// pass work on 16 different features of their rows, so a pass never has a
+// bank conflict and never two lanes on one address, whatever the bin
+// distribution is (missing values, zeros, a dominant category).
+constexpr int kBlockFeatures = 16;
+constexpr int kBlockQuads = 4;
+constexpr int kBlockEntries = kBlockFeatures * kSlots;  // 4096
+constexpr int HistBlocks(int nq) { return (nq + kBlockQuads - 1) / kBlockQuads; }
 // LDS bytes of a histogram of nq quads
 constexpr size_t HistLdsBytes(int nq, bool pair) {
-  return (size_t)nq * 4 * (kSlots + kHotReplicas) * 8 * (pair ? 2 : 1);
+  return (size_t)HistBlocks(nq) * kBlockEntries * 8 * (pair ? 2 : 1);
 }
 
 struct NodeSum {
@@ -347,80 +348,75 @@ constexpr unsigned kChunkRows = 128;
 constexpr unsigned kChunkStep = kChunkRows * kItemWaves;
 
 // ---------------------------------------------------------------- histogram
-// LDS layout of a histogram of NQ quads: word0[nbin], replicas of word0
-// [NQ*4*kHotReplicas], then (PAIR) word1 and its replicas in the same order.
+// LDS layout of a histogram of NQ quads: word0 of every entry, then (PAIR)
+// word1 in the same order.
 template <int NQ>
 struct HistLds {
-  static constexpr int nbin = NQ * 4 * kSlots;
-  static constexpr int nrep = NQ * 4 * kHotReplicas;
-  static constexpr int word1 = nbin + nrep;  // offset of word1 of the same entry
+  static constexpr int blocks = HistBlocks(NQ);
+  static constexpr int entries = blocks * kBlockEntries;
+  static constexpr int word1 = entries;  // offset of word1 of the same entry
 };
 
-// Adds one row (bins of its NQ quads in b) to the LDS histogram.  hot[q] packs
-// the replicated bin of each feature of quad q (wave-uniform).
+// Adds one row per lane (bins of its NQ quads in b) to the LDS histogram.  The
+// 28 (or 4*NQ) updates of a row are issued in an order that depends on the
+// lane: in step (s, t) of a block, lane l works on quad (s + (l>>2)) % 4 and
+// byte (t + l) % 4 of that quad, so the 16 lanes of a pass of the LDS atomic
+// touch 16 different features = 16 different bank pairs.  q_first: first quad
+// of this launch (a multiple of 4).
 template <bool PAIR, int NQ>
 __device__ __forceinline__ void AccumulateRow(unsigned long long *__restrict__ lds,
-                                              const uint32_t (&b)[NQ], const uint32_t (&hot)[NQ],
-                                              float gv, float hv, int sg, int sh, int q_first, int F) {
+                                              const uint32_t (&b)[NQ], float gv, float hv, int sg,
+                                              int sh, int q_first, int F) {
   using L = HistLds<NQ>;
   const unsigned long long w0 = (1ull << kCountShift) + (unsigned long long)ToFixed(gv, sg);
   unsigned long long w1 = 0;
   if (PAIR) w1 = (unsigned long long)ToFixed(hv, sh);
-  const unsigned rep = kHotReplicas > 0 ? (unsigned)L::nbin + (threadIdx.x & (unsigned)(kHotReplicas - 1)) : 0u;
+  const unsigned j = (threadIdx.x >> 2) & 3u, i = threadIdx.x & 3u;
 #pragma unroll
-  for (int q = 0; q < NQ; ++q) {
+  for (int k = 0; k < L::blocks; ++k) {
+    // quads of this block; the ones past NQ do not exist
+    uint32_t r[4];
 #pragma unroll
-    for (int c = 0; c < 4; ++c) {
-      // only the last quad can hold padding features
-      if (q < NQ - 1 || (q_first + q) * 4 + c < F) {
-        const unsigned bin = (b[q] >> (8 * c)) & 255u;
-        unsigned idx = (unsigned)(q * 4 + c) * kSlots + bin;
-        if (kHotReplicas > 0) {
-          const unsigned hb = (hot[q] >> (8 * c)) & 255u;
-          idx = bin == hb ? rep + (unsigned)(q * 4 + c) * kHotReplicas : idx;
+    for (int x = 0; x < 4; ++x) r[x] = 4 * k + x < NQ ? b[4 * k + x < NQ ? 4 * k + x : 0] : 0u;
+#pragma unroll
+    for (int s_ = 0; s_ < 4; ++s_) {
+      const unsigned qi = ((unsigned)s_ + j) & 3u;  // quad of the block this lane works on
+      const uint32_t lo = (j & 1u) ? r[(s_ + 1) & 3] : r[s_];
+      const uint32_t hi = (j & 1u) ? r[(s_ + 3) & 3] : r[(s_ + 2) & 3];
+      const uint32_t sel = (j & 2u) ? hi : lo;
+#pragma unroll
+      for (int t = 0; t < 4; ++t) {
+        const unsigned bi = ((unsigned)t + i) & 3u;  // byte of the quad
+        const unsigned bin = (sel >> (8u * bi)) & 255u;
+        const unsigned f16 = 4u * qi + bi;
+        bool on = true;
+        if (4 * k + 3 >= NQ) on = 4u * k + qi < (unsigned)NQ;  // block with missing quads
+        // only the last quad of the matrix can hold padding features
+        if (4 * k + 3 >= NQ - 1) on = on && (int)((q_first + 4 * k) * 4 + f16) < F;
+        if (on) {
+          const unsigned idx = (unsigned)(k * kBlockEntries) + bin * kBlockFeatures + f16;
+          atomicAdd(&lds[idx], w0);
+          if (PAIR) atomicAdd(&lds[L::word1 + idx], w1);
         }
-        atomicAdd(&lds[idx], w0);
-        if (PAIR) atomicAdd(&lds[L::word1 + idx], w1);
       }
     }
   }
 }
 
-// Loads the replicated bins of quads [q_first, q_first + NQ).
-template <int NQ>
-__device__ __forceinline__ void LoadHot(const uint32_t *__restrict__ hot_bins, int q_first, uint32_t (&hot)[NQ]) {
-#pragma unroll
-  for (int q = 0; q < NQ; ++q) hot[q] = kHotReplicas > 0 ? hot_bins[q_first + q] : 0u;
-}
-
-// Folds the replicas into their bins and writes the histogram to the slab of
-// work item w.  Called by the whole workgroup after the last LDS update.
+// Writes the LDS histogram to the slab of work item w in LDS order.  Called by
+// the whole workgroup after its last LDS update.  Slab layout per work item:
+// word0[slab_entries], word1[slab_entries]; q_first is a multiple of 4.
 template <bool PAIR, int NQ>
-__device__ __forceinline__ void FlushSlab(unsigned long long *__restrict__ lds, const uint32_t (&hot)[NQ],
+__device__ __forceinline__ void FlushSlab(const unsigned long long *__restrict__ lds,
                                           unsigned long long *__restrict__ slab, unsigned w,
-                                          int nbin_total, int q_first) {
+                                          int slab_entries, int q_first) {
   using L = HistLds<NQ>;
   __syncthreads();
-  if (kHotReplicas > 0) {
-    // one thread per (feature, word)
-    const int f = threadIdx.x >> 1, second = threadIdx.x & 1;
-    if (f < NQ * 4 && (PAIR || !second)) {
-      uint32_t hq = 0;
-#pragma unroll
-      for (int q = 0; q < NQ; ++q) hq = q == (f >> 2) ? hot[q] : hq;
-      const unsigned hb = (hq >> (8 * (f & 3))) & 255u;
-      const int off = second ? L::word1 : 0;
-      unsigned long long acc = lds[off + f * kSlots + hb];
-      for (int k = 0; k < kHotReplicas; ++k) acc += lds[off + L::nbin + f * kHotReplicas + k];
-      lds[off + f * kSlots + hb] = acc;
-    }
-    __syncthreads();
-  }
-  // slab layout per work item: word0[nbin_total], word1[nbin_total]
-  unsigned long long *out = slab + (size_t)w * nbin_total * (PAIR ? 2 : 1) + (size_t)q_first * 4 * kSlots;
-  for (int i = threadIdx.x; i < L::nbin; i += kHistThreads) {
-    out[i] = lds[i];
-    if (PAIR) out[nbin_total + i] = lds[L::word1 + i];
+  unsigned long long *out =
+      slab + (size_t)w * slab_entries * (PAIR ? 2 : 1) + (size_t)(q_first / kBlockQuads) * kBlockEntries;
+  for (int e = threadIdx.x; e < L::entries; e += kHistThreads) {
+    out[e] = lds[e];
+    if (PAIR) out[slab_entries + e] = lds[L::word1 + e];
   }
 }
 
@@ -431,7 +427,7 @@ __global__ void __launch_bounds__(kHistThreads)
 k_hist(const uint32_t *__restrict__ bins, size_t stride, int q0, int F,
        const float *__restrict__ g, const float *__restrict__ h, const int *__restrict__ shifts,
        const WorkItem *__restrict__ work, const unsigned *__restrict__ n_work,
-       unsigned long long *__restrict__ slab, int nbin_total, const uint32_t *__restrict__ hot_bins) {
+       unsigned long long *__restrict__ slab, int slab_entries) {
   extern __shared__ unsigned long long lds[];
   const unsigned w = blockIdx.x;
   if (w >= *n_work) return;
@@ -439,8 +435,6 @@ k_hist(const uint32_t *__restrict__ bins, size_t stride, int q0, int F,
   constexpr int words = (int)(HistLdsBytes(NQ, PAIR) / 8);
   for (int i = threadIdx.x; i < words; i += kHistThreads) lds[i] = 0ull;
   __syncthreads();
-  uint32_t hot[NQ];
-  LoadHot<NQ>(hot_bins, q0, hot);
   const int sg = shifts[0], sh = shifts[1];
   const uint32_t *bq = bins + (size_t)q0 * stride;
   for (unsigned base = it.begin; base < it.end; base += 2 * kHistThreads) {
@@ -455,10 +449,10 @@ k_hist(const uint32_t *__restrict__ bins, size_t stride, int q0, int F,
     }
     const float g0 = g[a0], g1 = g[a1];
     const float h0 = PAIR ? h[a0] : 0.0f, h1 = PAIR ? h[a1] : 0.0f;
-    if (v0) AccumulateRow<PAIR, NQ>(lds, b0, hot, g0, h0, sg, sh, q0, F);
-    if (v1) AccumulateRow<PAIR, NQ>(lds, b1, hot, g1, h1, sg, sh, q0, F);
+    if (v0) AccumulateRow<PAIR, NQ>(lds, b0, g0, h0, sg, sh, q0, F);
+    if (v1) AccumulateRow<PAIR, NQ>(lds, b1, g1, h1, sg, sh, q0, F);
   }
-  FlushSlab<PAIR, NQ>(lds, hot, slab, w, nbin_total, q0);
+  FlushSlab<PAIR, NQ>(lds, slab, w, slab_entries, q0);
 }
 
 // ---------------------------------------------------------------- partition
@@ -577,9 +571,9 @@ struct Pending {
 // becomes the new P.
 template <bool PAIR, int NQ>
 __device__ __forceinline__ void MergePending(unsigned long long *__restrict__ lds, Pending<NQ> &P,
-                                             unsigned long long &pmask, const uint32_t (&hot)[NQ],
-                                             const uint32_t (&xb)[NQ], float xg, float xh,
-                                             unsigned long long xm, int lane, int sg, int sh, int F) {
+                                             unsigned long long &pmask, const uint32_t (&xb)[NQ], float xg,
+                                             float xh, unsigned long long xm, int lane, int sg, int sh,
+                                             int F) {
   const unsigned nx = (unsigned)__popcll(xm);
   if (nx == 0) return;  // wave-uniform
   const unsigned np = (unsigned)__popcll(pmask);
@@ -603,7 +597,7 @@ __device__ __forceinline__ void MergePending(unsigned long long *__restrict__ ld
   }
   pmask |= __ballot(take);
   if (np + moved == 64u) {  // wave-uniform: P is full
-    AccumulateRow<PAIR, NQ>(lds, P.b, hot, P.g, P.h, sg, sh, 0, F);
+    AccumulateRow<PAIR, NQ>(lds, P.b, P.g, P.h, sg, sh, 0, F);
     const bool keep = ((xm >> lane) & 1ull) && RankBelow(xm) >= moved;
 #pragma unroll
     for (int q = 0; q < NQ; ++q) P.b[q] = xb[q];
@@ -627,7 +621,7 @@ k_part_hist(const uint32_t *__restrict__ bins, uint32_t *__restrict__ bins_out, 
             const unsigned *__restrict__ seg_start, const WorkItem *__restrict__ work,
             const unsigned *__restrict__ n_work, const unsigned *__restrict__ wave_left,
             const unsigned *__restrict__ item_left, unsigned long long *__restrict__ slab,
-            int nbin_total, const uint32_t *__restrict__ hot_bins) {
+            int slab_entries) {
   extern __shared__ unsigned long long lds[];
   __shared__ unsigned s_tmp[kItemWaves + 1];
   const unsigned w = blockIdx.x;
@@ -638,8 +632,6 @@ k_part_hist(const uint32_t *__restrict__ bins, uint32_t *__restrict__ bins_out, 
   const bool build_right = cl > cr;  // ties -> left (hist_grad_sum.cu:288-290)
   constexpr int words = (int)(HistLdsBytes(NQ, PAIR) / 8);
   for (int i = threadIdx.x; i < words; i += kHistThreads) lds[i] = 0ull;
-  uint32_t hot[NQ];
-  LoadHot<NQ>(hot_bins, 0, hot);
   const int sg = shifts[0], sh = shifts[1];
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const unsigned wb = it.begin + wave * kChunkRows, we = it.end;
@@ -722,8 +714,8 @@ k_part_hist(const uint32_t *__restrict__ bins, uint32_t *__restrict__ bins_out, 
       lo += nl0 + (unsigned)__popcll(lm1);
       ro += nr0 + (unsigned)__popcll(rm1);
     }
-    MergePending<PAIR, NQ>(lds, P, pmask, hot, b0, g0, h0, __ballot(v0 && right0 == build_right), lane, sg, sh, F);
-    MergePending<PAIR, NQ>(lds, P, pmask, hot, b1, g1, h1, __ballot(v1 && right1 == build_right), lane, sg, sh, F);
+    MergePending<PAIR, NQ>(lds, P, pmask, b0, g0, h0, __ballot(v0 && right0 == build_right), lane, sg, sh, F);
+    MergePending<PAIR, NQ>(lds, P, pmask, b1, g1, h1, __ballot(v1 && right1 == build_right), lane, sg, sh, F);
 #pragma unroll
     for (int q = 0; q < NQ; ++q) {
       b0[q] = nb0[q];
@@ -734,8 +726,8 @@ k_part_hist(const uint32_t *__restrict__ bins, uint32_t *__restrict__ bins_out, 
     h0 = nh0;
     h1 = nh1;
   }
-  if ((pmask >> lane) & 1ull) AccumulateRow<PAIR, NQ>(lds, P.b, hot, P.g, P.h, sg, sh, 0, F);
-  FlushSlab<PAIR, NQ>(lds, hot, slab, w, nbin_total, 0);
+  if ((pmask >> lane) & 1ull) AccumulateRow<PAIR, NQ>(lds, P.b, P.g, P.h, sg, sh, 0, F);
+  FlushSlab<PAIR, NQ>(lds, slab, w, slab_entries, 0);
 }
 
 // Stable partition alone (matrices too wide for the fused pass): any number
@@ -785,15 +777,16 @@ k_partition(const uint32_t *__restrict__ bins, uint32_t *__restrict__ bins_out, 
 
 // Adds the slabs of every directly built node of a level (on top of the stored
 // histogram when `accumulate`) and, with `trick`, derives its sibling as
-// parent - node.  grid (nbin_total/64, L), 1024
-// threads = 64 entries x 16 slab lanes.
+// parent - node.  Slabs are in LDS order (16-feature blocks, bin-major); the
+// histograms written here are feature-major: hist[node][f * 256 + bin].
+// grid (slab_entries/64, L), 1024 threads = 64 entries x 16 slab lanes.
 //   by_parent = 0: slabs belong to work items of the node itself
 //               (node_items == 0xffffffff marks a derived node);
 //   by_parent = 1: slabs belong to work items of the parent (fused pass); the
 //               built child is the smaller one, ties -> left.
 template <bool PAIR>
 __global__ void __launch_bounds__(1024)
-k_hist_reduce(const unsigned long long *__restrict__ slab, int nbin_total,
+k_hist_reduce(const unsigned long long *__restrict__ slab, int slab_entries, int nbin_total,
               const unsigned *__restrict__ node_first, const unsigned *__restrict__ node_items,
               int by_parent, const SplitRec *__restrict__ parent_split,
               const NodeSum *__restrict__ parent_tot, long long *__restrict__ hg,
@@ -818,28 +811,34 @@ k_hist_reduce(const unsigned long long *__restrict__ slab, int nbin_total,
     if (items == 0xffffffffu) return;  // derived from its sibling
   }
   const int e = threadIdx.x & 63, lane = threadIdx.x >> 6;
-  const int entry = blockIdx.x * 64 + e;
+  const int entry = blockIdx.x * 64 + e;  // slab order
+  const int f = (entry / kBlockEntries) * kBlockFeatures + (entry & (kBlockFeatures - 1));
+  const int bin = (entry / kBlockFeatures) & (kSlots - 1);
+  const bool live = f * kSlots < nbin_total;  // the last block may have fewer than 16 features
   long long ag = 0, ah = 0;
   unsigned ac = 0;
-  for (unsigned s = lane; s < items; s += 16) {
-    const unsigned long long *p = slab + (size_t)(first + s) * nbin_total * (PAIR ? 2 : 1);
-    const unsigned long long w0 = p[entry];
-    const long long gq = ((long long)(w0 << (64 - kCountShift))) >> (64 - kCountShift);
-    ag += gq;
-    ac += (unsigned)((w0 - (unsigned long long)gq) >> kCountShift);
-    if (PAIR) ah += (long long)p[nbin_total + entry];
+  if (live) {
+    for (unsigned s = lane; s < items; s += 16) {
+      const unsigned long long *p = slab + (size_t)(first + s) * slab_entries * (PAIR ? 2 : 1);
+      const unsigned long long w0 = p[entry];
+      const long long gq = ((long long)(w0 << (64 - kCountShift))) >> (64 - kCountShift);
+      ag += gq;
+      ac += (unsigned)((w0 - (unsigned long long)gq) >> kCountShift);
+      if (PAIR) ah += (long long)p[slab_entries + entry];
+    }
   }
   s_g[lane][e] = ag;
   s_h[lane][e] = ah;
   s_c[lane][e] = ac;
   __syncthreads();
-  if (lane == 0) {
+  if (lane == 0 && live) {
     for (int k = 1; k < 16; ++k) {
       ag += s_g[k][e];
       ah += s_h[k][e];
       ac += s_c[k][e];
     }
-    const size_t o = (size_t)nd * nbin_total + entry;
+    const size_t cell = (size_t)f * kSlots + bin;
+    const size_t o = (size_t)nd * nbin_total + cell;
     if (accumulate) {  // streamed matrices: one call per row block
       ag += hg[o];
       ah += hh[o];
@@ -849,33 +848,13 @@ k_hist_reduce(const unsigned long long *__restrict__ slab, int nbin_total,
     hh[o] = ah;
     hc[o] = ac;
     if (trick) {
-      const size_t po = (size_t)(nd >> 1) * nbin_total + entry;
-      const size_t so = (size_t)(nd ^ 1) * nbin_total + entry;
+      const size_t po = (size_t)(nd >> 1) * nbin_total + cell;
+      const size_t so = (size_t)(nd ^ 1) * nbin_total + cell;
       hg[so] = pg[po] - ag;
       hh[so] = ph[po] - ah;
       hc[so] = pc[po] - ac;
     }
   }
-}
-
-// Picks the bin to replicate in LDS for every feature: the one holding most
-// rows of the root histogram.  Only the speed of later histograms depends on
-// the choice.  One thread per feature; hot[q] packs the four bins of quad q.
-__global__ void k_pick_hot(const unsigned *__restrict__ hc, int Q, uint32_t *__restrict__ hot) {
-  const int q = blockIdx.x * blockDim.x + threadIdx.x;
-  if (q >= Q) return;
-  uint32_t packed = 0;
-  for (int c = 0; c < 4; ++c) {
-    const unsigned *cnt = hc + (size_t)(q * 4 + c) * kSlots;
-    unsigned best = 0, best_cnt = cnt[0];
-    for (unsigned b = 1; b < (unsigned)kSlots; ++b)
-      if (cnt[b] > best_cnt) {
-        best_cnt = cnt[b];
-        best = b;
-      }
-    packed |= best << (8 * c);
-  }
-  hot[q] = packed;
 }
 
 // Root totals = sum over the slots of feature 0 of the root histogram (every
@@ -1495,7 +1474,7 @@ void AllowLds(K kernel, size_t bytes) {
 template <bool PAIR, int NQ>
 void LaunchHistNQ(hipStream_t st, unsigned grid, const uint32_t *bins, size_t stride, int q0, int F,
                   const float *g, const float *h, const int *shifts, const WorkItem *work,
-                  const unsigned *n_work, unsigned long long *slab, int nbin_total, const uint32_t *hot) {
+                  const unsigned *n_work, unsigned long long *slab, int slab_entries) {
   const size_t lds = HistLdsBytes(NQ, PAIR);
   static bool configured = false;
   if (!configured) {
@@ -1503,17 +1482,17 @@ void LaunchHistNQ(hipStream_t st, unsigned grid, const uint32_t *bins, size_t st
     configured = true;
   }
   hipLaunchKernelGGL((k_hist<PAIR, NQ>), dim3(grid), dim3(kHistThreads), lds, st, bins, stride, q0, F, g, h,
-                     shifts, work, n_work, slab, nbin_total, hot);
+                     shifts, work, n_work, slab, slab_entries);
 }
 
 template <bool PAIR>
 void LaunchHist(int nq, hipStream_t st, unsigned grid, const uint32_t *bins, size_t stride, int q0, int F,
                 const float *g, const float *h, const int *shifts, const WorkItem *work,
-                const unsigned *n_work, unsigned long long *slab, int nbin_total, const uint32_t *hot) {
+                const unsigned *n_work, unsigned long long *slab, int slab_entries) {
 #define ARB_CASE(N) \
-  case N: LaunchHistNQ<PAIR, N>(st, grid, bins, stride, q0, F, g, h, shifts, work, n_work, slab, nbin_total, hot); break;
+  case N: LaunchHistNQ<PAIR, N>(st, grid, bins, stride, q0, F, g, h, shifts, work, n_work, slab, slab_entries); break;
   switch (nq) {
-    ARB_CASE(1) ARB_CASE(2) ARB_CASE(3) ARB_CASE(4) ARB_CASE(5) ARB_CASE(6) ARB_CASE(7) ARB_CASE(8) ARB_CASE(9)
+    ARB_CASE(1) ARB_CASE(2) ARB_CASE(3) ARB_CASE(4) ARB_CASE(5) ARB_CASE(6) ARB_CASE(7) ARB_CASE(8)
     default: throw std::runtime_error("internal: bad quad count");
   }
 #undef ARB_CASE
@@ -1537,8 +1516,7 @@ struct FusedArgs {
   const unsigned *wave_left;
   const unsigned *item_left;
   unsigned long long *slab;
-  int nbin_total;
-  const uint32_t *hot;
+  int slab_entries;
 };
 
 template <bool PAIR, int NQ, bool WRITE>
@@ -1551,7 +1529,7 @@ void LaunchFusedNQ(hipStream_t st, unsigned grid, const FusedArgs &a) {
   }
   hipLaunchKernelGGL((k_part_hist<PAIR, NQ, WRITE>), dim3(grid), dim3(kHistThreads), lds, st, a.bins, a.bins_out,
                      a.stride, a.F, a.g, a.g_out, a.h, a.h_out, a.shifts, a.split, a.tot, a.seg_start, a.work,
-                     a.n_work, a.wave_left, a.item_left, a.slab, a.nbin_total, a.hot);
+                     a.n_work, a.wave_left, a.item_left, a.slab, a.slab_entries);
 }
 
 template <bool PAIR, bool WRITE>
@@ -1559,7 +1537,7 @@ void LaunchFused(int nq, hipStream_t st, unsigned grid, const FusedArgs &a) {
 #define ARB_CASE(N) \
   case N: LaunchFusedNQ<PAIR, N, WRITE>(st, grid, a); break;
   switch (nq) {
-    ARB_CASE(1) ARB_CASE(2) ARB_CASE(3) ARB_CASE(4) ARB_CASE(5) ARB_CASE(6) ARB_CASE(7) ARB_CASE(8) ARB_CASE(9)
+    ARB_CASE(1) ARB_CASE(2) ARB_CASE(3) ARB_CASE(4) ARB_CASE(5) ARB_CASE(6) ARB_CASE(7) ARB_CASE(8)
     default: throw std::runtime_error("internal: bad quad count");
   }
 #undef ARB_CASE
@@ -1579,6 +1557,7 @@ class HipTreeBuilder : public TreeBuilder {
     f64_ = cfg.internal.double_precision;
     trick_ = cfg.internal.use_hist_subtraction_trick;
     nbin_total_ = Q_ * 4 * kSlots;
+    slab_entries_ = HistBlocks(Q_) * kBlockEntries;
     if (cfg.objective >= kSoftMaxOneVsAll && K_ < 2) throw std::runtime_error("soft-max needs labels_count >= 2");
     if (cfg.objective < kSoftMaxOneVsAll && K_ != 1) throw std::runtime_error("labels_count must be 1 for this objective");
     const int last_nodes = 1 << (D_ - 2);
@@ -1586,8 +1565,10 @@ class HipTreeBuilder : public TreeBuilder {
     HIP_OK(hipStreamCreateWithFlags(&stream_, hipStreamNonBlocking));
 
     // quads per histogram launch, limited by LDS
-    const size_t per_quad = HistLdsBytes(1, pair_);
-    quads_per_group_ = (int)std::min<size_t>(std::min<size_t>((kLdsBudget - 1024) / per_quad, kMaxGroupQuads), Q_);
+    // whole 16-feature blocks per launch
+    const size_t per_block = HistLdsBytes(kBlockQuads, pair_);
+    quads_per_group_ = (int)std::min<size_t>((kLdsBudget - 1024) / per_block * kBlockQuads, kMaxGroupQuads);
+    quads_per_group_ = std::min(quads_per_group_, Q_);
     // the fused partition + histogram pass holds one histogram of all
     // features and builds only the smaller child
     fused_ = trick_ && Q_ <= quads_per_group_;
@@ -1654,10 +1635,8 @@ class HipTreeBuilder : public TreeBuilder {
     d_nwork_ = DevAlloc<unsigned>(2);
     d_wave_left_ = DevAlloc<unsigned>((size_t)max_part_items_ * kItemWaves);
     d_item_left_ = DevAlloc<unsigned>(max_part_items_);
-    d_slab_ = DevAlloc<unsigned long long>((size_t)std::max(max_hist_items_, max_part_items_) * nbin_total_ * (pair_ ? 2 : 1));
+    d_slab_ = DevAlloc<unsigned long long>((size_t)std::max(max_hist_items_, max_part_items_) * slab_entries_ * (pair_ ? 2 : 1));
     d_shifts_ = DevAlloc<int>(2);
-    d_hot_ = DevAlloc<uint32_t>(Q_);
-    HIP_OK(hipMemsetAsync(d_hot_, 0, Q_ * sizeof(uint32_t), stream_));
     d_gmax_ = DevAlloc<unsigned>(1);
     d_rows_scanned_ = DevAlloc<unsigned long long>(1);
     d_overflow_ = DevAlloc<unsigned>(1);
@@ -1682,7 +1661,7 @@ class HipTreeBuilder : public TreeBuilder {
     (void)hipStreamSynchronize(stream_);
     void *ptrs[] = {d_y_, d_labels_, d_yhat_, d_g_, d_h_, d_leaf_, d_split_, d_cand_, d_node_first_,
                     d_node_items_, d_hwork_, d_pwork_, d_nwork_, d_wave_left_, d_item_left_, d_slab_,
-                    d_shifts_, d_gmax_, d_rows_scanned_, d_tfid_, d_tbin_, d_tgain_, d_weights_, d_active_, d_overflow_, d_hot_};
+                    d_shifts_, d_gmax_, d_rows_scanned_, d_tfid_, d_tbin_, d_tgain_, d_weights_, d_active_, d_overflow_};
     for (void *p : ptrs)
       if (p) (void)hipFree(p);
     for (int b = 0; b < 2; ++b) {
@@ -1843,9 +1822,9 @@ class HipTreeBuilder : public TreeBuilder {
     for (int q0 = 0; q0 < Q_; q0 += quads_per_group_) {
       const int nq = std::min(quads_per_group_, Q_ - q0);
       if (pair_)
-        LaunchHist<true>(nq, stream_, grid, cur.bins, stride_, q0, F_, cur.g, cur.h, d_shifts_, d_hwork_, d_nwork_, d_slab_, nbin_total_, d_hot_);
+        LaunchHist<true>(nq, stream_, grid, cur.bins, stride_, q0, F_, cur.g, cur.h, d_shifts_, d_hwork_, d_nwork_, d_slab_, slab_entries_);
       else
-        LaunchHist<false>(nq, stream_, grid, cur.bins, stride_, q0, F_, cur.g, cur.h, d_shifts_, d_hwork_, d_nwork_, d_slab_, nbin_total_, d_hot_);
+        LaunchHist<false>(nq, stream_, grid, cur.bins, stride_, q0, F_, cur.g, cur.h, d_shifts_, d_hwork_, d_nwork_, d_slab_, slab_entries_);
       if (timing_) ++(root ? timings_.hist_root_launches : timings_.hist_deep_launches);
     }
     if (timing_ && root) timings_.hist_root_rows += n_;
@@ -1853,13 +1832,13 @@ class HipTreeBuilder : public TreeBuilder {
 
   void Reduce(int L, int hb, bool by_parent, int parent_state, bool trick, bool accumulate = false) {
     Mark(kReduce);
-    dim3 grid(nbin_total_ / 64, L);
+    dim3 grid(slab_entries_ / 64, L);
     if (pair_)
-      hipLaunchKernelGGL(k_hist_reduce<true>, grid, dim3(1024), 0, stream_, d_slab_, nbin_total_, d_node_first_,
+      hipLaunchKernelGGL(k_hist_reduce<true>, grid, dim3(1024), 0, stream_, d_slab_, slab_entries_, nbin_total_, d_node_first_,
                          d_node_items_, by_parent ? 1 : 0, d_split_, d_tot_[parent_state], d_hg_[hb], d_hh_[hb],
                          d_hc_[hb], d_hg_[hb ^ 1], d_hh_[hb ^ 1], d_hc_[hb ^ 1], trick ? 1 : 0, accumulate ? 1 : 0);
     else
-      hipLaunchKernelGGL(k_hist_reduce<false>, grid, dim3(1024), 0, stream_, d_slab_, nbin_total_, d_node_first_,
+      hipLaunchKernelGGL(k_hist_reduce<false>, grid, dim3(1024), 0, stream_, d_slab_, slab_entries_, nbin_total_, d_node_first_,
                          d_node_items_, by_parent ? 1 : 0, d_split_, d_tot_[parent_state], d_hg_[hb], d_hh_[hb],
                          d_hc_[hb], d_hg_[hb ^ 1], d_hh_[hb ^ 1], d_hc_[hb ^ 1], trick ? 1 : 0, accumulate ? 1 : 0);
   }
@@ -1888,7 +1867,6 @@ class HipTreeBuilder : public TreeBuilder {
         HistOfNodes(orig, state, 1, false, n_, true);
         Reduce(1, hb, false, state, false);
         hipLaunchKernelGGL(k_root_from_hist, dim3(1), dim3(64), 0, stream_, d_hg_[hb], d_hh_[hb], d_tot_[state]);
-        PickHotBins(hb);
       } else {
         // rows are in the order of level-1; the parents' state is state ^ 1
         const int ps = state ^ 1, PL = L >> 1;
@@ -1906,7 +1884,7 @@ class HipTreeBuilder : public TreeBuilder {
           }
           Mark(last ? kFusedLast : kHistDeep);
           FusedArgs a{src.bins, dst.bins, stride_, F_, src.g, dst.g, src.h, dst.h, d_shifts_, d_split_,
-                      d_tot_[ps], d_seg_[ps], d_pwork_, d_nwork_ + 1, d_wave_left_, d_item_left_, d_slab_, nbin_total_, d_hot_};
+                      d_tot_[ps], d_seg_[ps], d_pwork_, d_nwork_ + 1, d_wave_left_, d_item_left_, d_slab_, slab_entries_};
           if (pair_) {
             if (last) LaunchFused<true, false>(Q_, stream_, grid, a);
             else LaunchFused<true, true>(Q_, stream_, grid, a);
@@ -2090,17 +2068,15 @@ class HipTreeBuilder : public TreeBuilder {
           const int nq = std::min(quads_per_group_, Q_ - q0);
           if (pair_)
             LaunchHist<true>(nq, stream_, grid, stage_.bins, br, q0, F_, stage_.g, stage_.h, d_shifts_, d_hwork_,
-                             d_nwork_, d_slab_, nbin_total_, d_hot_);
+                             d_nwork_, d_slab_, slab_entries_);
           else
             LaunchHist<false>(nq, stream_, grid, stage_.bins, br, q0, F_, stage_.g, stage_.h, d_shifts_, d_hwork_,
-                              d_nwork_, d_slab_, nbin_total_, d_hot_);
+                              d_nwork_, d_slab_, slab_entries_);
         }
         Reduce(L, hb, false, state, false, b > 0);
       }
-      if (level == 0) {
+      if (level == 0)
         hipLaunchKernelGGL(k_root_from_hist, dim3(1), dim3(64), 0, stream_, d_hg_[hb], d_hh_[hb], d_tot_[state]);
-        PickHotBins(hb);
-      }
       if (trick)
         hipLaunchKernelGGL(k_sibling, dim3((nbin_total_ + 255) / 256, L), dim3(256), 0, stream_, d_hg_[hb], d_hh_[hb],
                            d_hc_[hb], d_hg_[hb ^ 1], d_hh_[hb ^ 1], d_hc_[hb ^ 1], d_tot_[state], level, nbin_total_);
@@ -2149,14 +2125,6 @@ class HipTreeBuilder : public TreeBuilder {
     HIP_OK(hipMemcpy(d_active_, active_host_.data(), active_host_.size(), hipMemcpyHostToDevice));
   }
 
-  // After the first root histogram of this builder: choose the bins that get
-  // LDS replicas from its counts.
-  void PickHotBins(int hb) {
-    if (hot_ready_ || kHotReplicas == 0) return;
-    hipLaunchKernelGGL(k_pick_hot, dim3((Q_ + 63) / 64), dim3(64), 0, stream_, d_hc_[hb], Q_, d_hot_);
-    hot_ready_ = true;
-  }
-
   void KeepHist(int level, int L, int hb) {
     const size_t cells = (size_t)L * nbin_total_;
     std::vector<long long> g(cells), h(cells);
@@ -2184,6 +2152,7 @@ class HipTreeBuilder : public TreeBuilder {
   DeviceMatrix *dm_;
   size_t n_ = 0, stride_ = 0;
   int F_ = 0, Q_ = 0, K_ = 1, D_ = 2, nbin_total_ = 0;
+  int slab_entries_ = 0;  // histogram entries of one work item's slab (whole 16-feature blocks)
   bool pair_ = false, f64_ = false, trick_ = true, fused_ = false, inspect_ = false, timing_ = false;
   bool grad_ready_ = false;
   int quads_per_group_ = 1;
@@ -2219,8 +2188,6 @@ class HipTreeBuilder : public TreeBuilder {
   unsigned max_hist_items_ = 0, max_part_items_ = 0;
   unsigned long long *d_slab_ = nullptr, *d_rows_scanned_ = nullptr;
   int *d_shifts_ = nullptr, *d_tfid_ = nullptr, *d_tbin_ = nullptr;
-  uint32_t *d_hot_ = nullptr;  // per quad: the replicated bin of each of its features
-  bool hot_ready_ = false;
   std::vector<std::vector<int64_t>> kept_hist_;
   std::vector<hipEvent_t> event_pool_;
   size_t event_used_ = 0;
