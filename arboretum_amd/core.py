@@ -19,7 +19,7 @@ def _load_lib():
     path = os.path.join(here, "libarboretum.so")
     if not os.path.exists(path):
         raise ArboretumError(
-            "libarboretum.so is not built: run `python -m arboretum_amd.build` (needs hipcc)")
+            "libarboretum.so is not built: run `python arboretum_amd/build.py` (needs hipcc)")
     lib = ctypes.cdll.LoadLibrary(path)
     c_char_p, c_void_p, c_int, c_float = ctypes.c_char_p, ctypes.c_void_p, ctypes.c_int, ctypes.c_float
     P = ctypes.POINTER

@@ -15,10 +15,14 @@
 //   word0 = count << 47 | sum of g_q   (g_q fixed point, |g_q| <= 2^30)
 //   word1 = sum of h_q
 // so one update costs two ds_add_u64 (one for the squared objective).  A range
-// holds at most 64512 rows, which keeps both fields exact.  Each workgroup
-// writes its LDS histogram to a private slab in HBM; a reduce kernel adds the
-// slabs of a node, and derives the larger sibling as parent - smaller child.
-// All sums are integers: the result does not depend on scheduling.
+// holds at most 64512 rows, which keeps both fields exact.  The LDS histogram
+// is laid out in blocks of 16 features, bin-major inside a block, and every
+// lane of a wave updates a different feature of its own row at a time: the 16
+// lanes that one pass of the LDS atomic unit serves never share a bank pair or
+// an address, whatever the bins are.  Each workgroup writes its LDS histogram
+// to a private slab in HBM; a reduce kernel adds the slabs of a node, turns
+// them feature-major, and derives the larger sibling as parent - smaller
+// child.  All sums are integers: the result does not depend on scheduling.
 //
 // What replaces what (reference file:line):
 //   k_bin_assign      build_histogram              src/io/io.cu:293-312
@@ -481,10 +485,22 @@ k_part_count(const uint32_t *__restrict__ bins, size_t stride, const SplitRec *_
   } else {
     const uint32_t *col = bins + (size_t)(s.fid >> 2) * stride;
     const int sh = 8 * (s.fid & 3);
-    for (unsigned base = it.begin + wave * kChunkRows; base < it.end; base += kChunkStep) {
-      const unsigned r0 = base + lane, r1 = r0 + 64;
-      if (r0 < it.end) cnt += ((int)((col[r0] >> sh) & 255u) > s.bin) ? 0u : 1u;
-      if (r1 < it.end) cnt += ((int)((col[r1] >> sh) & 255u) > s.bin) ? 0u : 1u;
+    // eight chunks (16 loads) in flight per wave: the pass is latency-bound
+    constexpr int kBatch = 8;
+    for (unsigned base = it.begin + wave * kChunkRows; base < it.end; base += kBatch * kChunkStep) {
+      uint32_t v0[kBatch], v1[kBatch];
+#pragma unroll
+      for (int k = 0; k < kBatch; ++k) {
+        const unsigned r0 = base + k * kChunkStep + lane, r1 = r0 + 64;
+        v0[k] = col[min(r0, it.end - 1)];
+        v1[k] = col[min(r1, it.end - 1)];
+      }
+#pragma unroll
+      for (int k = 0; k < kBatch; ++k) {
+        const unsigned r0 = base + k * kChunkStep + lane, r1 = r0 + 64;
+        if (r0 < it.end) cnt += ((int)((v0[k] >> sh) & 255u) > s.bin) ? 0u : 1u;
+        if (r1 < it.end) cnt += ((int)((v1[k] >> sh) & 255u) > s.bin) ? 0u : 1u;
+      }
     }
   }
   for (int off = 32; off > 0; off >>= 1) cnt += __shfl_down(cnt, off);
@@ -566,6 +582,13 @@ struct Pending {
   float g, h;
 };
 
+// Two rows per lane of a wave's 128-row chunk, as loaded.
+template <int NQ>
+struct RowSet {
+  uint32_t b0[NQ], b1[NQ];
+  float g0, g1, h0, h1;
+};
+
 // Moves the rows of X flagged in xm (wave-uniform mask) into free lanes of P
 // (occupied lanes: pmask); when P is full it is accumulated and the rest of X
 // becomes the new P.
@@ -609,9 +632,13 @@ __device__ __forceinline__ void MergePending(unsigned long long *__restrict__ ld
 
 // Fused pass over the rows of the parent nodes of a level: stable partition
 // into the children order (WRITE) and histogram of the smaller child of every
-// split in LDS.  Each wave owns a contiguous row range and runs without
-// workgroup barriers; the rows of the next iteration are requested before the
-// current ones are processed.  NQ = all quads of the matrix.
+// split in LDS.  Each wave owns the 128-row chunks v, v + 16, ... of the item
+// and runs without workgroup barriers.  LDS atomic instructions cost the same
+// with one active lane as with 64, so the rows of the built child are packed
+// into full waves first: with WRITE the rows are in registers anyway and are
+// packed with lane permutes (Pending); on the last level only the quad of the
+// split feature is read for every row, the selected rows are queued by row id
+// and read 64 at a time.  NQ = all quads of the matrix.
 template <bool PAIR, int NQ, bool WRITE>
 __global__ void __launch_bounds__(kHistThreads)
 k_part_hist(const uint32_t *__restrict__ bins, uint32_t *__restrict__ bins_out, size_t stride, int F,
@@ -642,91 +669,152 @@ k_part_hist(const uint32_t *__restrict__ bins, uint32_t *__restrict__ bins_out, 
   }
   __syncthreads();
   const int fq = s.fid >> 2, fs = 8 * (s.fid & 3);
-  Pending<NQ> P;
+  if constexpr (WRITE) {
+    Pending<NQ> P;
 #pragma unroll
-  for (int q = 0; q < NQ; ++q) P.b[q] = 0;
-  P.g = P.h = 0.0f;
-  unsigned long long pmask = 0;
+    for (int q = 0; q < NQ; ++q) P.b[q] = 0;
+    P.g = P.h = 0.0f;
+    unsigned long long pmask = 0;
 
-  uint32_t b0[NQ], b1[NQ];
-  float g0 = 0, g1 = 0, h0 = 0, h1 = 0;
-  if (wb < we) {
-    const unsigned a0 = min(wb + lane, we - 1), a1 = min(wb + 64 + lane, we - 1);
-#pragma unroll
-    for (int q = 0; q < NQ; ++q) {
-      b0[q] = bins[(size_t)q * stride + a0];
-      b1[q] = bins[(size_t)q * stride + a1];
-    }
-    g0 = g[a0];
-    g1 = g[a1];
-    if (PAIR) {
-      h0 = h[a0];
-      h1 = h[a1];
-    }
-  }
-  for (unsigned base = wb; base < we; base += kChunkStep) {
-    // rows of the next iteration
-    uint32_t nb0[NQ], nb1[NQ];
-    float ng0 = 0, ng1 = 0, nh0 = 0, nh1 = 0;
-    const unsigned next = base + kChunkStep;
-    if (next < we) {
-      const unsigned a0 = min(next + lane, we - 1), a1 = min(next + 64 + lane, we - 1);
+    // Two register sets of 128 rows each: while one is processed the other is
+    // in flight.  The loads are unconditional (addresses clamped to the last
+    // row of the item) and the sets are never copied, so every wait in the loop
+    // is for exactly the set that is needed next.
+    auto load = [&](RowSet<NQ> &R, unsigned base) {
+      const unsigned a0 = min(base + lane, we - 1), a1 = min(base + 64 + lane, we - 1);
 #pragma unroll
       for (int q = 0; q < NQ; ++q) {
-        nb0[q] = bins[(size_t)q * stride + a0];
-        nb1[q] = bins[(size_t)q * stride + a1];
+        R.b0[q] = bins[(size_t)q * stride + a0];
+        R.b1[q] = bins[(size_t)q * stride + a1];
       }
-      ng0 = g[a0];
-      ng1 = g[a1];
-      if (PAIR) {
-        nh0 = h[a0];
-        nh1 = h[a1];
+      R.g0 = g[a0];
+      R.g1 = g[a1];
+      R.h0 = PAIR ? h[a0] : 0.0f;
+      R.h1 = PAIR ? h[a1] : 0.0f;
+    };
+    auto process = [&](const RowSet<NQ> &R, unsigned base) {
+      const unsigned r0 = base + lane, r1 = r0 + 64;
+      const bool v0 = r0 < we, v1 = r1 < we;
+      uint32_t s0 = 0, s1 = 0;
+#pragma unroll
+      for (int q = 0; q < NQ; ++q) {
+        s0 = q == fq ? R.b0[q] : s0;
+        s1 = q == fq ? R.b1[q] : s1;
+      }
+      const bool right0 = v0 && s.fid >= 0 && (int)((s0 >> fs) & 255u) > s.bin;
+      const bool right1 = v1 && s.fid >= 0 && (int)((s1 >> fs) & 255u) > s.bin;
+      {
+        const unsigned long long lm0 = __ballot(v0 && !right0), rm0 = __ballot(right0);
+        const unsigned long long lm1 = __ballot(v1 && !right1), rm1 = __ballot(right1);
+        const unsigned nl0 = (unsigned)__popcll(lm0), nr0 = (unsigned)__popcll(rm0);
+        if (v0) {
+          const unsigned d = right0 ? ro + RankBelow(rm0) : lo + RankBelow(lm0);
+#pragma unroll
+          for (int q = 0; q < NQ; ++q) bins_out[(size_t)q * stride + d] = R.b0[q];
+          g_out[d] = R.g0;
+          if (PAIR) h_out[d] = R.h0;
+        }
+        if (v1) {
+          const unsigned d = right1 ? ro + nr0 + RankBelow(rm1) : lo + nl0 + RankBelow(lm1);
+#pragma unroll
+          for (int q = 0; q < NQ; ++q) bins_out[(size_t)q * stride + d] = R.b1[q];
+          g_out[d] = R.g1;
+          if (PAIR) h_out[d] = R.h1;
+        }
+        lo += nl0 + (unsigned)__popcll(lm1);
+        ro += nr0 + (unsigned)__popcll(rm1);
+      }
+      MergePending<PAIR, NQ>(lds, P, pmask, R.b0, R.g0, R.h0, __ballot(v0 && right0 == build_right), lane, sg, sh, F);
+      MergePending<PAIR, NQ>(lds, P, pmask, R.b1, R.g1, R.h1, __ballot(v1 && right1 == build_right), lane, sg, sh, F);
+    };
+    if (wb < we) {
+      RowSet<NQ> A, B;
+      load(A, wb);
+      for (unsigned base = wb;; base += 2 * kChunkStep) {
+        load(B, base + kChunkStep);
+        process(A, base);
+        if (base + kChunkStep >= we) break;  // wave-uniform
+        load(A, base + 2 * kChunkStep);
+        process(B, base + kChunkStep);
+        if (base + 2 * kChunkStep >= we) break;
       }
     }
-    const unsigned r0 = base + lane, r1 = r0 + 64;
-    const bool v0 = r0 < we, v1 = r1 < we;
-    uint32_t s0 = 0, s1 = 0;
+    if ((pmask >> lane) & 1ull) AccumulateRow<PAIR, NQ>(lds, P.b, P.g, P.h, sg, sh, 0, F);
+  } else {
+    // Rows selected for the histogram are queued by row id (slot 64 * j + lane
+    // of the queue is lane `lane` of q[j]; slots [0, np) are occupied) and read
+    // again 64 at a time: LDS atomic instructions cost the same with one active
+    // lane as with 64, so only full waves are accumulated.  The second read
+    // hits the cache, is requested at the start of a chunk and used at its end,
+    // and the wave never waits for its LDS atomics.
+    unsigned q0 = it.begin, q1 = it.begin, q2 = it.begin;
+    unsigned np = 0;
+    uint32_t gb[NQ];
+    float gg = 0.0f, gh = 0.0f;
+    auto gather = [&](bool valid) {  // requests the rows of queue slots [0, 64)
+      const unsigned a = valid ? q0 : it.begin;
 #pragma unroll
-    for (int q = 0; q < NQ; ++q) {
-      s0 = q == fq ? b0[q] : s0;
-      s1 = q == fq ? b1[q] : s1;
-    }
-    const bool right0 = v0 && s.fid >= 0 && (int)((s0 >> fs) & 255u) > s.bin;
-    const bool right1 = v1 && s.fid >= 0 && (int)((s1 >> fs) & 255u) > s.bin;
-    if (WRITE) {
-      const unsigned long long lm0 = __ballot(v0 && !right0), rm0 = __ballot(right0);
-      const unsigned long long lm1 = __ballot(v1 && !right1), rm1 = __ballot(right1);
-      const unsigned nl0 = (unsigned)__popcll(lm0), nr0 = (unsigned)__popcll(rm0);
-      if (v0) {
-        const unsigned d = right0 ? ro + RankBelow(rm0) : lo + RankBelow(lm0);
-#pragma unroll
-        for (int q = 0; q < NQ; ++q) bins_out[(size_t)q * stride + d] = b0[q];
-        g_out[d] = g0;
-        if (PAIR) h_out[d] = h0;
+      for (int q = 0; q < NQ; ++q) gb[q] = bins[(size_t)q * stride + a];
+      gg = g[a];
+      gh = PAIR ? h[a] : 0.0f;
+      q0 = q1;
+      q1 = q2;
+    };
+    // m: wave-uniform mask of the selected rows among base + [0, 64); np < 128
+    auto enqueue = [&](unsigned base, unsigned long long m) {
+      const unsigned nx = (unsigned)__popcll(m);
+      if (nx == 0) return;
+      const unsigned r = np & 63u, j = np >> 6;
+      const unsigned k = ((unsigned)lane - r) & 63u;  // slot np + k
+      const unsigned id = base + (unsigned)SelectBit(m, k < nx ? k : 0u);
+      const bool here = (unsigned)lane >= r && k < nx;   // lands in q[j]
+      const bool next = (unsigned)lane < r && k < nx;    // lands in q[j + 1]
+      q0 = (j == 0 && here) ? id : q0;
+      q1 = ((j == 1 && here) || (j == 0 && next)) ? id : q1;
+      q2 = (j == 1 && next) ? id : q2;
+      np += nx;
+    };
+    // after a chunk: at most 127 rows stay queued
+    auto drain = [&](unsigned limit) {
+      while (np > limit) {
+        const unsigned take = min(np, 64u);
+        const bool valid = (unsigned)lane < take;
+        gather(valid);
+        if (valid) AccumulateRow<PAIR, NQ>(lds, gb, gg, gh, sg, sh, 0, F);
+        np -= take;
       }
-      if (v1) {
-        const unsigned d = right1 ? ro + nr0 + RankBelow(rm1) : lo + nl0 + RankBelow(lm1);
-#pragma unroll
-        for (int q = 0; q < NQ; ++q) bins_out[(size_t)q * stride + d] = b1[q];
-        g_out[d] = g1;
-        if (PAIR) h_out[d] = h1;
+    };
+    if (wb < we) {
+      // last level: only the quad of the split feature decides; the selected
+      // rows are read when they are accumulated
+      const uint32_t *col = bins + (size_t)(s.fid < 0 ? 0 : fq) * stride;
+      auto step = [&](uint32_t s0, uint32_t s1, uint32_t &n0, uint32_t &n1, unsigned base) {
+        const bool full = np >= 64u;  // wave-uniform
+        if (full) {
+          gather(true);
+          np -= 64u;
+        }
+        n0 = col[min(base + kChunkStep + lane, we - 1)];
+        n1 = col[min(base + kChunkStep + 64 + lane, we - 1)];
+        const unsigned r0 = base + lane, r1 = r0 + 64;
+        const bool v0 = r0 < we, v1 = r1 < we;
+        const bool right0 = v0 && s.fid >= 0 && (int)((s0 >> fs) & 255u) > s.bin;
+        const bool right1 = v1 && s.fid >= 0 && (int)((s1 >> fs) & 255u) > s.bin;
+        enqueue(base, __ballot(v0 && right0 == build_right));
+        enqueue(base + 64, __ballot(v1 && right1 == build_right));
+        if (full) AccumulateRow<PAIR, NQ>(lds, gb, gg, gh, sg, sh, 0, F);
+        drain(127u);
+      };
+      uint32_t a0 = col[min(wb + lane, we - 1)], a1 = col[min(wb + 64 + lane, we - 1)], b0, b1;
+      for (unsigned base = wb;; base += 2 * kChunkStep) {
+        step(a0, a1, b0, b1, base);
+        if (base + kChunkStep >= we) break;  // wave-uniform
+        step(b0, b1, a0, a1, base + kChunkStep);
+        if (base + 2 * kChunkStep >= we) break;
       }
-      lo += nl0 + (unsigned)__popcll(lm1);
-      ro += nr0 + (unsigned)__popcll(rm1);
     }
-    MergePending<PAIR, NQ>(lds, P, pmask, b0, g0, h0, __ballot(v0 && right0 == build_right), lane, sg, sh, F);
-    MergePending<PAIR, NQ>(lds, P, pmask, b1, g1, h1, __ballot(v1 && right1 == build_right), lane, sg, sh, F);
-#pragma unroll
-    for (int q = 0; q < NQ; ++q) {
-      b0[q] = nb0[q];
-      b1[q] = nb1[q];
-    }
-    g0 = ng0;
-    g1 = ng1;
-    h0 = nh0;
-    h1 = nh1;
+    drain(0u);
   }
-  if ((pmask >> lane) & 1ull) AccumulateRow<PAIR, NQ>(lds, P.b, P.g, P.h, sg, sh, 0, F);
   FlushSlab<PAIR, NQ>(lds, slab, w, slab_entries, 0);
 }
 

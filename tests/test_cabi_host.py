@@ -23,7 +23,7 @@ def declared_symbols():
 
 
 def test_library_exports_every_declared_symbol():
-    assert os.path.exists(LIB), "libarboretum.so is not built (python -m arboretum_amd.build)"
+    assert os.path.exists(LIB), "libarboretum.so is not built (python arboretum_amd/build.py)"
     lib = ctypes.CDLL(LIB)
     names = declared_symbols()
     # the 14 entry points of python-wrapper/arboretum_wrapper.h:6-39
