@@ -572,16 +572,6 @@ __device__ __forceinline__ int SelectBit(unsigned long long m, unsigned k) {
   return pos;
 }
 
-// A wave's register-resident queue of rows waiting to be accumulated: one row
-// per lane.  LDS atomic instructions cost the same with one active lane as
-// with 64, so the rows selected for the histogram are first packed into full
-// waves with lane permutes.
-template <int NQ>
-struct Pending {
-  uint32_t b[NQ];
-  float g, h;
-};
-
 // Two rows per lane of a wave's 128-row chunk, as loaded.
 template <int NQ>
 struct RowSet {
@@ -589,56 +579,100 @@ struct RowSet {
   float g0, g1, h0, h1;
 };
 
-// Moves the rows of X flagged in xm (wave-uniform mask) into free lanes of P
-// (occupied lanes: pmask); when P is full it is accumulated and the rest of X
-// becomes the new P.
+// A wave's register-resident queue of rows on their way to one child's row
+// range: lane l holds the row whose destination is base + l, lanes [0, n) are
+// occupied, and on a wave's first batch lanes [0, skip) stand for the rows
+// before the wave's own range (base is a multiple of 64 rows, so every batch
+// is written as one aligned, fully coalesced 256-byte store per array).
+template <int NQ>
+struct RowQueue {
+  uint32_t b[NQ];
+  float g, h;
+  unsigned n, skip, base;
+  __device__ __forceinline__ void Init(unsigned first_row) {
+#pragma unroll
+    for (int q = 0; q < NQ; ++q) b[q] = 0;
+    g = h = 0.0f;
+    n = skip = first_row & 63u;
+    base = first_row - n;
+  }
+};
+
+// Writes lanes [from, to) of Q to their destination and, for the child whose
+// histogram is built, adds them to the LDS histogram.
 template <bool PAIR, int NQ>
-__device__ __forceinline__ void MergePending(unsigned long long *__restrict__ lds, Pending<NQ> &P,
-                                             unsigned long long &pmask, const uint32_t (&xb)[NQ], float xg,
-                                             float xh, unsigned long long xm, int lane, int sg, int sh,
-                                             int F) {
+__device__ __forceinline__ void EmitRows(unsigned long long *__restrict__ lds, const RowQueue<NQ> &Q,
+                                         unsigned from, unsigned to, bool built,
+                                         uint32_t *__restrict__ bins_out, size_t stride,
+                                         float *__restrict__ g_out, float *__restrict__ h_out, int lane,
+                                         int sg, int sh, int F) {
+  if ((unsigned)lane >= from && (unsigned)lane < to) {
+    const unsigned d = Q.base + (unsigned)lane;
+#pragma unroll
+    for (int q = 0; q < NQ; ++q) bins_out[(size_t)q * stride + d] = Q.b[q];
+    g_out[d] = Q.g;
+    if (PAIR) h_out[d] = Q.h;
+    if (built) AccumulateRow<PAIR, NQ>(lds, Q.b, Q.g, Q.h, sg, sh, 0, F);
+  }
+}
+
+// Appends the rows of X flagged in xm (wave-uniform mask, one row per lane) to
+// Q in row order with one lane permute per register; a full queue is emitted
+// and the rest of X starts the next batch.
+template <bool PAIR, int NQ>
+__device__ __forceinline__ void MergeRows(unsigned long long *__restrict__ lds, RowQueue<NQ> &Q,
+                                          const uint32_t (&xb)[NQ], float xg, float xh,
+                                          unsigned long long xm, bool built,
+                                          uint32_t *__restrict__ bins_out, size_t stride,
+                                          float *__restrict__ g_out, float *__restrict__ h_out, int lane,
+                                          int sg, int sh, int F) {
   const unsigned nx = (unsigned)__popcll(xm);
   if (nx == 0) return;  // wave-uniform
-  const unsigned np = (unsigned)__popcll(pmask);
-  const unsigned moved = min(nx, 64u - np);
-  const unsigned long long holes = ~pmask;
-  const unsigned hr = RankBelow(holes);  // rank of this lane among the free lanes of P
-  const bool take = ((holes >> lane) & 1ull) && hr < moved;
-  const int src = take ? SelectBit(xm, hr) : lane;  // the hr-th row of X
+  // lane l receives the k-th flagged row, k = (l - n) mod 64: lanes >= n fill
+  // the current batch, lanes < n hold what overflows into the next one
+  const unsigned k = ((unsigned)lane - Q.n) & 63u;
+  const int src = SelectBit(xm, k < nx ? k : 0u);
+  uint32_t vb[NQ];
 #pragma unroll
-  for (int q = 0; q < NQ; ++q) {
-    const uint32_t v = (uint32_t)__shfl((int)xb[q], src);
-    P.b[q] = take ? v : P.b[q];
-  }
-  {
-    const float v = __shfl(xg, src);
-    P.g = take ? v : P.g;
-  }
-  if (PAIR) {
-    const float v = __shfl(xh, src);
-    P.h = take ? v : P.h;
-  }
-  pmask |= __ballot(take);
-  if (np + moved == 64u) {  // wave-uniform: P is full
-    AccumulateRow<PAIR, NQ>(lds, P.b, P.g, P.h, sg, sh, 0, F);
-    const bool keep = ((xm >> lane) & 1ull) && RankBelow(xm) >= moved;
+  for (int q = 0; q < NQ; ++q) vb[q] = (uint32_t)__shfl((int)xb[q], src);
+  const float vg = __shfl(xg, src);
+  const float vh = PAIR ? __shfl(xh, src) : 0.0f;
+  if (Q.n + nx >= 64u) {  // wave-uniform: the batch is complete
+    const bool fill = (unsigned)lane >= Q.n;
 #pragma unroll
-    for (int q = 0; q < NQ; ++q) P.b[q] = xb[q];
-    P.g = xg;
-    P.h = xh;
-    pmask = __ballot(keep);
+    for (int q = 0; q < NQ; ++q) Q.b[q] = fill ? vb[q] : Q.b[q];
+    Q.g = fill ? vg : Q.g;
+    Q.h = fill ? vh : Q.h;
+    EmitRows<PAIR, NQ>(lds, Q, Q.skip, 64u, built, bins_out, stride, g_out, h_out, lane, sg, sh, F);
+    Q.base += 64u;
+    Q.skip = 0u;
+#pragma unroll
+    for (int q = 0; q < NQ; ++q) Q.b[q] = vb[q];
+    Q.g = vg;
+    Q.h = vh;
+    Q.n = Q.n + nx - 64u;
+  } else {
+    const bool fill = (unsigned)lane >= Q.n && k < nx;
+#pragma unroll
+    for (int q = 0; q < NQ; ++q) Q.b[q] = fill ? vb[q] : Q.b[q];
+    Q.g = fill ? vg : Q.g;
+    Q.h = fill ? vh : Q.h;
+    Q.n += nx;
   }
 }
 
 // Fused pass over the rows of the parent nodes of a level: stable partition
 // into the children order (WRITE) and histogram of the smaller child of every
 // split in LDS.  Each wave owns the 128-row chunks v, v + 16, ... of the item
-// and runs without workgroup barriers.  LDS atomic instructions cost the same
-// with one active lane as with 64, so the rows of the built child are packed
-// into full waves first: with WRITE the rows are in registers anyway and are
-// packed with lane permutes (Pending); on the last level only the quad of the
-// split feature is read for every row, the selected rows are queued by row id
-// and read 64 at a time.  NQ = all quads of the matrix.
+// and runs without workgroup barriers.  With WRITE the rows of a chunk are
+// sorted into two register queues (one per child) with lane permutes; a full
+// queue is one aligned 64-row store per array, and the queue of the built
+// child is added to the histogram as a full wave (LDS atomic instructions
+// cost the same with one active lane as with 64).  Writing each chunk's rows
+// directly, as two short unaligned runs per store, costs 40 % more time than
+// the copy itself.  On the last level only the quad of the split feature is
+// read for every row; the selected rows are queued by row id and read 64 at a
+// time.  NQ = all quads of the matrix.
 template <bool PAIR, int NQ, bool WRITE>
 __global__ void __launch_bounds__(kHistThreads)
 k_part_hist(const uint32_t *__restrict__ bins, uint32_t *__restrict__ bins_out, size_t stride, int F,
@@ -670,12 +704,10 @@ k_part_hist(const uint32_t *__restrict__ bins, uint32_t *__restrict__ bins_out, 
   __syncthreads();
   const int fq = s.fid >> 2, fs = 8 * (s.fid & 3);
   if constexpr (WRITE) {
-    Pending<NQ> P;
-#pragma unroll
-    for (int q = 0; q < NQ; ++q) P.b[q] = 0;
-    P.g = P.h = 0.0f;
-    unsigned long long pmask = 0;
-
+    // QB: rows of the child whose histogram is built, QO: the other child
+    RowQueue<NQ> QB, QO;
+    QB.Init(build_right ? ro : lo);
+    QO.Init(build_right ? lo : ro);
     // Two register sets of 128 rows each: while one is processed the other is
     // in flight.  The loads are unconditional (addresses clamped to the last
     // row of the item) and the sets are never copied, so every wait in the loop
@@ -703,29 +735,12 @@ k_part_hist(const uint32_t *__restrict__ bins, uint32_t *__restrict__ bins_out, 
       }
       const bool right0 = v0 && s.fid >= 0 && (int)((s0 >> fs) & 255u) > s.bin;
       const bool right1 = v1 && s.fid >= 0 && (int)((s1 >> fs) & 255u) > s.bin;
-      {
-        const unsigned long long lm0 = __ballot(v0 && !right0), rm0 = __ballot(right0);
-        const unsigned long long lm1 = __ballot(v1 && !right1), rm1 = __ballot(right1);
-        const unsigned nl0 = (unsigned)__popcll(lm0), nr0 = (unsigned)__popcll(rm0);
-        if (v0) {
-          const unsigned d = right0 ? ro + RankBelow(rm0) : lo + RankBelow(lm0);
-#pragma unroll
-          for (int q = 0; q < NQ; ++q) bins_out[(size_t)q * stride + d] = R.b0[q];
-          g_out[d] = R.g0;
-          if (PAIR) h_out[d] = R.h0;
-        }
-        if (v1) {
-          const unsigned d = right1 ? ro + nr0 + RankBelow(rm1) : lo + nl0 + RankBelow(lm1);
-#pragma unroll
-          for (int q = 0; q < NQ; ++q) bins_out[(size_t)q * stride + d] = R.b1[q];
-          g_out[d] = R.g1;
-          if (PAIR) h_out[d] = R.h1;
-        }
-        lo += nl0 + (unsigned)__popcll(lm1);
-        ro += nr0 + (unsigned)__popcll(rm1);
-      }
-      MergePending<PAIR, NQ>(lds, P, pmask, R.b0, R.g0, R.h0, __ballot(v0 && right0 == build_right), lane, sg, sh, F);
-      MergePending<PAIR, NQ>(lds, P, pmask, R.b1, R.g1, R.h1, __ballot(v1 && right1 == build_right), lane, sg, sh, F);
+      const unsigned long long b0 = __ballot(v0 && right0 == build_right), o0 = __ballot(v0 && right0 != build_right);
+      const unsigned long long b1 = __ballot(v1 && right1 == build_right), o1 = __ballot(v1 && right1 != build_right);
+      MergeRows<PAIR, NQ>(lds, QO, R.b0, R.g0, R.h0, o0, false, bins_out, stride, g_out, h_out, lane, sg, sh, F);
+      MergeRows<PAIR, NQ>(lds, QB, R.b0, R.g0, R.h0, b0, true, bins_out, stride, g_out, h_out, lane, sg, sh, F);
+      MergeRows<PAIR, NQ>(lds, QO, R.b1, R.g1, R.h1, o1, false, bins_out, stride, g_out, h_out, lane, sg, sh, F);
+      MergeRows<PAIR, NQ>(lds, QB, R.b1, R.g1, R.h1, b1, true, bins_out, stride, g_out, h_out, lane, sg, sh, F);
     };
     if (wb < we) {
       RowSet<NQ> A, B;
@@ -739,7 +754,8 @@ k_part_hist(const uint32_t *__restrict__ bins, uint32_t *__restrict__ bins_out, 
         if (base + 2 * kChunkStep >= we) break;
       }
     }
-    if ((pmask >> lane) & 1ull) AccumulateRow<PAIR, NQ>(lds, P.b, P.g, P.h, sg, sh, 0, F);
+    EmitRows<PAIR, NQ>(lds, QO, QO.skip, QO.n, false, bins_out, stride, g_out, h_out, lane, sg, sh, F);
+    EmitRows<PAIR, NQ>(lds, QB, QB.skip, QB.n, true, bins_out, stride, g_out, h_out, lane, sg, sh, F);
   } else {
     // Rows selected for the histogram are queued by row id (slot 64 * j + lane
     // of the queue is lane `lane` of q[j]; slots [0, np) are occupied) and read
