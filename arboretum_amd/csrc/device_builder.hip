@@ -607,11 +607,12 @@ __device__ __forceinline__ void EmitRows(unsigned long long *__restrict__ lds, c
                                          float *__restrict__ g_out, float *__restrict__ h_out, int lane,
                                          int sg, int sh, int F) {
   if ((unsigned)lane >= from && (unsigned)lane < to) {
+    // streaming stores and loads: the pass touches every byte once
     const unsigned d = Q.base + (unsigned)lane;
 #pragma unroll
-    for (int q = 0; q < NQ; ++q) bins_out[(size_t)q * stride + d] = Q.b[q];
-    g_out[d] = Q.g;
-    if (PAIR) h_out[d] = Q.h;
+    for (int q = 0; q < NQ; ++q) __builtin_nontemporal_store(Q.b[q], &bins_out[(size_t)q * stride + d]);
+    __builtin_nontemporal_store(Q.g, &g_out[d]);
+    if (PAIR) __builtin_nontemporal_store(Q.h, &h_out[d]);
     if (built) AccumulateRow<PAIR, NQ>(lds, Q.b, Q.g, Q.h, sg, sh, 0, F);
   }
 }
@@ -716,13 +717,13 @@ k_part_hist(const uint32_t *__restrict__ bins, uint32_t *__restrict__ bins_out, 
       const unsigned a0 = min(base + lane, we - 1), a1 = min(base + 64 + lane, we - 1);
 #pragma unroll
       for (int q = 0; q < NQ; ++q) {
-        R.b0[q] = bins[(size_t)q * stride + a0];
-        R.b1[q] = bins[(size_t)q * stride + a1];
+        R.b0[q] = __builtin_nontemporal_load(&bins[(size_t)q * stride + a0]);
+        R.b1[q] = __builtin_nontemporal_load(&bins[(size_t)q * stride + a1]);
       }
-      R.g0 = g[a0];
-      R.g1 = g[a1];
-      R.h0 = PAIR ? h[a0] : 0.0f;
-      R.h1 = PAIR ? h[a1] : 0.0f;
+      R.g0 = __builtin_nontemporal_load(&g[a0]);
+      R.g1 = __builtin_nontemporal_load(&g[a1]);
+      R.h0 = PAIR ? __builtin_nontemporal_load(&h[a0]) : 0.0f;
+      R.h1 = PAIR ? __builtin_nontemporal_load(&h[a1]) : 0.0f;
     };
     auto process = [&](const RowSet<NQ> &R, unsigned base) {
       const unsigned r0 = base + lane, r1 = r0 + 64;
