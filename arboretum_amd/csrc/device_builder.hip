@@ -448,8 +448,8 @@ k_hist(const uint32_t *__restrict__ bins, size_t stride, int q0, int F,
     uint32_t b0[NQ], b1[NQ];
 #pragma unroll
     for (int q = 0; q < NQ; ++q) {
-      b0[q] = bq[(size_t)q * stride + a0];
-      b1[q] = bq[(size_t)q * stride + a1];
+      b0[q] = __builtin_nontemporal_load(&bq[(size_t)q * stride + a0]);
+      b1[q] = __builtin_nontemporal_load(&bq[(size_t)q * stride + a1]);
     }
     const float g0 = g[a0], g1 = g[a1];
     const float h0 = PAIR ? h[a0] : 0.0f, h1 = PAIR ? h[a1] : 0.0f;
@@ -1321,9 +1321,9 @@ k_final(const uint32_t *__restrict__ bins, size_t stride, const int *__restrict_
        i += (size_t)gridDim.x * blockDim.x) {
     uint32_t b[NQ > 0 ? NQ : 1];
 #pragma unroll
-    for (int q = 0; q < NQ; ++q) b[q] = bins[(size_t)q * stride + i];
+    for (int q = 0; q < NQ; ++q) b[q] = __builtin_nontemporal_load(&bins[(size_t)q * stride + i]);
     const float yh0 = yhat[i];
-    const float yv = NEXT_GRAD != 0 ? y[i] : 0.0f;
+    const float yv = NEXT_GRAD != 0 ? __builtin_nontemporal_load(&y[i]) : 0.0f;
     unsigned node = 0;
     for (int level = 0; level + 1 < depth; ++level) {
       const int id = (1 << level) - 1 + (int)node;
@@ -1342,7 +1342,7 @@ k_final(const uint32_t *__restrict__ bins, size_t stride, const int *__restrict_
       }
       node = node * 2 + right;
     }
-    leaf_of[i] = node;
+    __builtin_nontemporal_store(node, &leaf_of[i]);
     const float yh = yh0 + weights[node];
     yhat[i] = yh;
     if (NEXT_GRAD == 1) {
@@ -1360,6 +1360,75 @@ k_final(const uint32_t *__restrict__ bins, size_t stride, const int *__restrict_
     m = WaveMaxF(m);
     if ((threadIdx.x & 63) == 0) atomicMax(gmax_bits, __float_as_uint(m));
   }
+}
+
+// Last pass of a tree fused with the root histogram of the next one
+// (logistic objective, resident matrix, all quads in one LDS histogram): the
+// rows are read once; the leaf walk, the prediction update and the new
+// gradients are bound by HBM, the histogram by LDS atomics, and they overlap.
+// One workgroup per root work item; LDS: histogram, then the node arrays.
+template <int NQ>
+__global__ void __launch_bounds__(kHistThreads)
+k_final_hist(const uint32_t *__restrict__ bins, size_t stride, int F, const int *__restrict__ t_fid,
+             const int *__restrict__ t_bin, int depth, const float *__restrict__ weights,
+             float *__restrict__ yhat, const float *__restrict__ y, unsigned *__restrict__ leaf_of,
+             float *__restrict__ g, float *__restrict__ h, const int *__restrict__ shifts,
+             const WorkItem *__restrict__ work, const unsigned *__restrict__ n_work,
+             unsigned long long *__restrict__ slab, int slab_entries) {
+  extern __shared__ unsigned long long lds[];
+  const unsigned w = blockIdx.x;
+  if (w >= *n_work) return;
+  const WorkItem it = work[w];
+  constexpr int words = (int)(HistLdsBytes(NQ, true) / 8);
+  int *s_nodes = reinterpret_cast<int *>(lds + words);  // fid[internal], bin[internal]
+  const int internal = (1 << (depth - 1)) - 1;
+  for (int i = threadIdx.x; i < words; i += kHistThreads) lds[i] = 0ull;
+  for (int i = threadIdx.x; i < internal; i += kHistThreads) {
+    s_nodes[i] = t_fid[i];
+    s_nodes[internal + i] = t_bin[i];
+  }
+  __syncthreads();
+  const int sg = shifts[0], sh = shifts[1];
+  auto row = [&](const uint32_t (&b)[NQ], float p, float yv, unsigned r) {
+    unsigned node = 0;
+    for (int level = 0; level + 1 < depth; ++level) {
+      const int id = (1 << level) - 1 + (int)node;
+      const int fid = s_nodes[id], bin = s_nodes[internal + id];
+      unsigned right = 0;
+      if (bin >= 0) {
+        uint32_t b4 = 0;
+        const int fq = fid >> 2;
+#pragma unroll
+        for (int q = 0; q < NQ; ++q) b4 = q == fq ? b[q] : b4;
+        right = (int)((b4 >> (8 * (fid & 3))) & 255u) > bin ? 1u : 0u;
+      }
+      node = node * 2 + right;
+    }
+    __builtin_nontemporal_store(node, &leaf_of[r]);
+    const float yh = p + weights[node];
+    yhat[r] = yh;
+    const float s = SigmoidF(yh);
+    const float gv = yv - s, hv = s * (1.0f - s);
+    g[r] = gv;
+    h[r] = hv;
+    AccumulateRow<true, NQ>(lds, b, gv, hv, sg, sh, 0, F);
+  };
+  for (unsigned base = it.begin; base < it.end; base += 2 * kHistThreads) {
+    const unsigned r0 = base + threadIdx.x, r1 = r0 + kHistThreads;
+    const bool v0 = r0 < it.end, v1 = r1 < it.end;
+    const unsigned a0 = v0 ? r0 : it.begin, a1 = v1 ? r1 : it.begin;
+    uint32_t b0[NQ], b1[NQ];
+#pragma unroll
+    for (int q = 0; q < NQ; ++q) {
+      b0[q] = __builtin_nontemporal_load(&bins[(size_t)q * stride + a0]);
+      b1[q] = __builtin_nontemporal_load(&bins[(size_t)q * stride + a1]);
+    }
+    const float p0 = yhat[a0], p1 = yhat[a1];
+    const float y0 = __builtin_nontemporal_load(&y[a0]), y1 = __builtin_nontemporal_load(&y[a1]);
+    if (v0) row(b0, p0, y0, r0);
+    if (v1) row(b1, p1, y1, r1);
+  }
+  FlushSlab<true, NQ>(lds, slab, w, slab_entries, 0);
 }
 
 __global__ void k_fill_f32(float *p, float v, size_t n) {
@@ -1969,7 +2038,9 @@ class HipTreeBuilder : public TreeBuilder {
       const int hb = level & 1;  // histogram buffer of this level; the parent level is hb ^ 1
       const bool last = level + 2 >= D_;
       if (level == 0) {
-        HistOfNodes(orig, state, 1, false, n_, true);
+        // the slabs of the root may have been written by the last pass of the previous tree
+        if (!root_hist_ready_) HistOfNodes(orig, state, 1, false, n_, true);
+        root_hist_ready_ = false;
         Reduce(1, hb, false, state, false);
         hipLaunchKernelGGL(k_root_from_hist, dim3(1), dim3(64), 0, stream_, d_hg_[hb], d_hh_[hb], d_tot_[state]);
       } else {
@@ -2028,7 +2099,21 @@ class HipTreeBuilder : public TreeBuilder {
     {
       const bool next_grad = !inspect_ && K_ == 1;
       if (cfg_.objective == kLinearRegression) HIP_OK(hipMemsetAsync(d_gmax_, 0, sizeof(unsigned), stream_));
-      LaunchFinal(dm_->bins, stride_, 0, n_, label, next_grad);
+      const int internal = (1 << (D_ - 1)) - 1;
+      const size_t lds = HistLdsBytes(Q_, true) + (size_t)internal * 2 * sizeof(int);
+      if (next_grad && cfg_.objective == kLogisticRegression && Q_ <= quads_per_group_ && lds <= kLdsBudget) {
+        // plan of the next tree's root, then one pass: leaves, predictions,
+        // gradients and the root histogram of the next tree
+        hipLaunchKernelGGL(k_init_root, dim3(1), dim3(64), 0, stream_, d_tot_[0], d_seg_[0],
+                           (unsigned long long)n_, (unsigned *)nullptr);
+        const unsigned per_item = HistRowsPerItem(n_, 256);
+        const unsigned grid = (unsigned)std::min<size_t>(n_ / per_item + 2, max_hist_items_);
+        Plan(0, 1, 0, per_item, d_hwork_, d_nwork_, true, nullptr, grid);
+        LaunchFinalHist(grid, label, lds);
+        root_hist_ready_ = true;
+      } else {
+        LaunchFinal(dm_->bins, stride_, 0, n_, label, next_grad);
+      }
       grad_ready_ = next_grad;
     }
     FetchTree(tree);
@@ -2129,6 +2214,26 @@ class HipTreeBuilder : public TreeBuilder {
     }
 #undef ARB_FINAL_Q
 #undef ARB_FINAL
+  }
+
+  void LaunchFinalHist(unsigned grid, int label, size_t lds) {
+    float *yh = d_yhat_ + (size_t)label * n_;
+#define ARB_CASE(N)                                                                                              \
+  case N: {                                                                                                      \
+    static bool configured = false;                                                                              \
+    if (!configured) {                                                                                           \
+      AllowLds(k_final_hist<N>, kLdsBudget);                                                                     \
+      configured = true;                                                                                         \
+    }                                                                                                            \
+    hipLaunchKernelGGL((k_final_hist<N>), dim3(grid), dim3(kHistThreads), lds, stream_, dm_->bins, stride_, F_, \
+                       d_tfid_, d_tbin_, D_, d_weights_, yh, d_y_, d_leaf_, d_g_, d_h_, d_shifts_, d_hwork_,     \
+                       d_nwork_, d_slab_, slab_entries_);                                                        \
+  } break;
+    switch (Q_) {
+      ARB_CASE(1) ARB_CASE(2) ARB_CASE(3) ARB_CASE(4) ARB_CASE(5) ARB_CASE(6) ARB_CASE(7) ARB_CASE(8)
+      default: throw std::runtime_error("internal: bad quad count");
+    }
+#undef ARB_CASE
   }
 
   // One tree over a streamed matrix: every level copies every block in once
@@ -2258,6 +2363,7 @@ class HipTreeBuilder : public TreeBuilder {
   size_t n_ = 0, stride_ = 0;
   int F_ = 0, Q_ = 0, K_ = 1, D_ = 2, nbin_total_ = 0;
   int slab_entries_ = 0;  // histogram entries of one work item's slab (whole 16-feature blocks)
+  bool root_hist_ready_ = false;  // the slabs hold the root histogram of the tree grown next
   bool pair_ = false, f64_ = false, trick_ = true, fused_ = false, inspect_ = false, timing_ = false;
   bool grad_ready_ = false;
   int quads_per_group_ = 1;

@@ -222,6 +222,24 @@ def main():
     def frac(b, t):
         return (b / t) / HBM_PEAK if t > 0 else 0.0
 
+    other = {"k_part_hist<true,7,false> (last level)": {
+        "frac_of_hbm": frac(last_bytes, last_s),
+        "avg_launch_us": tm["fused_last_ms"] * 1e3 / max(tm["fused_last_launches"], 1)}}
+    if tm["hist_root_launches"] > 0:
+        other["k_hist<true,7> (root level)"] = {
+            "frac_of_hbm": frac(root_bytes, root_s),
+            "avg_launch_us": tm["hist_root_ms"] * 1e3 / tm["hist_root_launches"],
+            "updates_per_s": tm["hist_root_rows"] * F / root_s if root_s > 0 else 0.0}
+    else:
+        # the last pass of a tree (leaf of every row, prediction update, next gradients)
+        # also builds the root histogram of the next tree: rows read once (bins, y_hat, y),
+        # leaf id, y_hat, g, h written
+        final_bytes = args.steps * (args.rows * (F + 8 + 16) + F * 256 * cell_bytes * 256)
+        other["k_final_hist<7> (last pass of a tree + root histogram of the next)"] = {
+            "frac_of_hbm": frac(final_bytes, tm["leaf_ms"] * 1e-3),
+            "avg_launch_us": tm["leaf_ms"] * 1e3 / args.steps,
+            "updates_per_s": args.steps * args.rows * F / (tm["leaf_ms"] * 1e-3) if tm["leaf_ms"] > 0 else 0.0}
+
     out = {
         "metric": "row*feature hist updates/s + sec/tree at 10M x 28 depth 8; % of HBM peak",
         "value": updates / dt,
@@ -247,14 +265,7 @@ def main():
                      "launches": int(tm["hist_deep_launches"]),
                      "avg_launch_us": tm["hist_deep_ms"] * 1e3 / fl,
                      "bytes_per_launch": fused_bytes / fl},
-        "other_kernels": {
-            "k_hist<true,7> (root level)": {
-                "frac_of_hbm": frac(root_bytes, root_s),
-                "avg_launch_us": tm["hist_root_ms"] * 1e3 / max(tm["hist_root_launches"], 1),
-                "updates_per_s": tm["hist_root_rows"] * F / root_s if root_s > 0 else 0.0},
-            "k_part_hist<true,7,false> (last level)": {
-                "frac_of_hbm": frac(last_bytes, last_s),
-                "avg_launch_us": tm["fused_last_ms"] * 1e3 / max(tm["fused_last_launches"], 1)}},
+        "other_kernels": other,
         "tree_algorithmic_floor_frac_of_hbm": (2.9e9 / (dt / args.steps)) / HBM_PEAK,
         "phase_ms_per_tree": {k: v / args.steps for k, v in tm.items() if k.endswith("_ms")},
         "quantise_s": t_quant,

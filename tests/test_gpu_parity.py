@@ -142,6 +142,37 @@ def test_training_without_inspection(arb, oracle, objective):
     assert_same_training(arb, oracle, X, y, cfg, rounds=4, check_hist=False)
 
 
+@pytest.mark.parametrize("n,F,depth", [(1, 3, 2), (65, 1, 1), (2049, 5, 3), (70000, 8, 4), (5000, 32, 5)])
+def test_last_pass_feeds_next_root_histogram(arb, oracle, n, F, depth):
+    # logistic, inspection off: the pass that assigns the leaves of a tree also
+    # builds the root histogram of the next tree
+    X, y = make_data(n, F, 1, seed=n + F)
+    cfg = {"objective": 1, "method": 1, "internals": {"hist_size": 64, "double_precision": False},
+           "tree": {"max_depth": depth, "eta": 0.5, "lambda": 1.0, "min_child_weight": 0.0}}
+    assert_same_training(arb, oracle, X, y, cfg, rounds=5, check_hist=False)
+
+
+def test_inspection_switched_on_between_rounds(arb, oracle):
+    X, y = make_data(20000, 12, 1, seed=77)
+    cfg = {"objective": 1, "method": 1, "internals": {"hist_size": 255, "double_precision": True},
+           "tree": {"max_depth": 5, "eta": 0.4, "lambda": 1.0}}
+    ob = oracle.Booster(X, y=y, config=cfg)
+    data = arb.DMatrix(X, y=y)
+    g = arb.Garden(cfg, data)
+    for r in range(6):
+        g.set_inspect(r in (2, 3))  # off, off, on, on, off, off
+        ob.grow(1)
+        g.grow_tree()
+        to, tg = ob.tree(r), g.tree(r)
+        for key in ("fid", "quantized", "threshold", "gain"):
+            assert np.array_equal(to[key], tg[key]), "%s round %d" % (key, r)
+        assert np.array_equal(to["weights"], tg["weights"], equal_nan=True)
+        assert np.array_equal(ob.yhat(), g.train_yhat()), "y_hat round %d" % r
+        if r in (2, 3):
+            for level in range(5):
+                assert np.array_equal(g.level_hist(level)[:, :, :256, :], ob.level_hist(level)[:, :, :256, :])
+
+
 # ----------------------------------------------- streamed (out-of-core) bins
 @pytest.mark.parametrize("objective", [0, 1])
 @pytest.mark.parametrize("trick", [True, False])
