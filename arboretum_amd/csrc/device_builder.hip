@@ -258,12 +258,13 @@ __device__ __forceinline__ unsigned RankBelow(unsigned long long m) {
 // into histograms: the selected rows, or, when `split` is given (fused
 // partition + histogram over parent nodes), the smaller side of every split.
 // One workgroup.
-__global__ void __launch_bounds__(1024)
-k_plan(const NodeSum *__restrict__ tot, const unsigned *__restrict__ seg_start, int L, int select,
-       unsigned rows_per_item, WorkItem *__restrict__ work, unsigned *__restrict__ n_work,
-       unsigned *__restrict__ node_first, unsigned *__restrict__ node_items,
-       unsigned long long *__restrict__ rows_scanned, const SplitRec *__restrict__ split,
-       unsigned max_items, unsigned *__restrict__ overflow) {
+__device__ __forceinline__ void PlanBody(const NodeSum *__restrict__ tot, const unsigned *__restrict__ seg_start,
+                                         int L, int select, unsigned rows_per_item,
+                                         WorkItem *__restrict__ work, unsigned *__restrict__ n_work,
+                                         unsigned *__restrict__ node_first, unsigned *__restrict__ node_items,
+                                         unsigned long long *__restrict__ rows_scanned,
+                                         const SplitRec *__restrict__ split, unsigned max_items,
+                                         unsigned *__restrict__ overflow) {
   __shared__ unsigned s_base[kMaxPlanNodes + 1];
   __shared__ unsigned s_wave[16];
   __shared__ unsigned s_carry;
@@ -342,6 +343,16 @@ k_plan(const NodeSum *__restrict__ tot, const unsigned *__restrict__ seg_start, 
     it.first = s_base[lo];
     work[w] = it;
   }
+}
+
+__global__ void __launch_bounds__(1024)
+k_plan(const NodeSum *__restrict__ tot, const unsigned *__restrict__ seg_start, int L, int select,
+       unsigned rows_per_item, WorkItem *__restrict__ work, unsigned *__restrict__ n_work,
+       unsigned *__restrict__ node_first, unsigned *__restrict__ node_items,
+       unsigned long long *__restrict__ rows_scanned, const SplitRec *__restrict__ split,
+       unsigned max_items, unsigned *__restrict__ overflow) {
+  PlanBody(tot, seg_start, L, select, rows_per_item, work, n_work, node_first, node_items, rows_scanned, split,
+           max_items, overflow);
 }
 
 // Rows of a work item are dealt to its waves in chunks of kChunkRows
@@ -1226,15 +1237,13 @@ k_split_scan(const long long *__restrict__ hg, const long long *__restrict__ hh,
 // (higher gain, then lower feature id: hist_tree_grower.cu:59-60), children
 // totals and row ranges, node record.  A node without a candidate keeps every
 // row left.
-__global__ void k_split_select(const Cand *__restrict__ cand, int F, int L,
-                               const NodeSum *__restrict__ tot,
-                               const unsigned *__restrict__ seg_start,
-                               NodeSum *__restrict__ tot_next, unsigned *__restrict__ seg_next,
-                               SplitRec *__restrict__ split, int *__restrict__ t_fid,
-                               int *__restrict__ t_bin, float *__restrict__ t_gain, int heap_off,
-                               const unsigned char *__restrict__ active) {
-  const int nd = blockIdx.x * blockDim.x + threadIdx.x;
-  if (nd >= L) return;
+__device__ __forceinline__ void SelectNode(int nd, const Cand *__restrict__ cand, int F,
+                                           const NodeSum *__restrict__ tot,
+                                           const unsigned *__restrict__ seg_start,
+                                           NodeSum *__restrict__ tot_next, unsigned *__restrict__ seg_next,
+                                           SplitRec *__restrict__ split, int *__restrict__ t_fid,
+                                           int *__restrict__ t_bin, float *__restrict__ t_gain, int heap_off,
+                                           const unsigned char *__restrict__ active) {
   const NodeSum t = tot[nd];
   SplitRec rec;
   rec.gain = 0.0f;
@@ -1267,6 +1276,38 @@ __global__ void k_split_select(const Cand *__restrict__ cand, int F, int L,
   t_fid[heap_off + nd] = rec.fid < 0 ? 0 : rec.fid;  // garden.cu:471-481
   t_bin[heap_off + nd] = rec.fid < 0 ? -1 : rec.bin;
   t_gain[heap_off + nd] = rec.gain;
+}
+
+__global__ void k_split_select(const Cand *__restrict__ cand, int F, int L,
+                               const NodeSum *__restrict__ tot,
+                               const unsigned *__restrict__ seg_start,
+                               NodeSum *__restrict__ tot_next, unsigned *__restrict__ seg_next,
+                               SplitRec *__restrict__ split, int *__restrict__ t_fid,
+                               int *__restrict__ t_bin, float *__restrict__ t_gain, int heap_off,
+                               const unsigned char *__restrict__ active) {
+  const int nd = blockIdx.x * blockDim.x + threadIdx.x;
+  if (nd < L)
+    SelectNode(nd, cand, F, tot, seg_start, tot_next, seg_next, split, t_fid, t_bin, t_gain, heap_off, active);
+}
+
+// k_split_select followed, in the same workgroup, by the work plan of the
+// fused pass over these nodes' rows (the plan needs the splits only for the
+// row statistics).  One workgroup of 1024 threads.
+__global__ void __launch_bounds__(1024)
+k_select_plan(const Cand *__restrict__ cand, int F, int L, const NodeSum *__restrict__ tot,
+              const unsigned *__restrict__ seg_start, NodeSum *__restrict__ tot_next,
+              unsigned *__restrict__ seg_next, SplitRec *__restrict__ split, int *__restrict__ t_fid,
+              int *__restrict__ t_bin, float *__restrict__ t_gain, int heap_off,
+              const unsigned char *__restrict__ active, unsigned rows_per_item,
+              WorkItem *__restrict__ work, unsigned *__restrict__ n_work,
+              unsigned *__restrict__ node_first, unsigned *__restrict__ node_items,
+              unsigned long long *__restrict__ rows_scanned, unsigned max_items,
+              unsigned *__restrict__ overflow) {
+  for (int nd = threadIdx.x; nd < L; nd += 1024)
+    SelectNode(nd, cand, F, tot, seg_start, tot_next, seg_next, split, t_fid, t_bin, t_gain, heap_off, active);
+  __syncthreads();  // the splits written above are read by the plan
+  PlanBody(tot, seg_start, L, 0, rows_per_item, work, n_work, node_first, node_items, rows_scanned, split,
+           max_items, overflow);
 }
 
 // --------------------------------------------------------------- leaves
@@ -2049,10 +2090,8 @@ class HipTreeBuilder : public TreeBuilder {
         const RowBuffers &src = level == 1 ? orig : buf_[level & 1];
         const RowBuffers &dst = buf_[(level & 1) ^ 1];
         if (fused_) {
-          const unsigned per_item = HistRowsPerItem(n_);
-          const unsigned grid = (unsigned)std::min<size_t>(n_ / per_item + PL + 1, max_part_items_);
-          Mark(kPlan);
-          Plan(ps, PL, 0, per_item, d_pwork_, d_nwork_ + 1, true, d_split_, grid);
+          // the work plan was written together with the splits of the parents
+          const unsigned grid = FusedGrid(PL);
           if (!last) {  // destination offsets; the last level moves no rows
             Mark(kPartition);
             hipLaunchKernelGGL(k_part_count, dim3(grid), dim3(kHistThreads), 0, stream_, src.bins, stride_, d_split_,
@@ -2090,7 +2129,7 @@ class HipTreeBuilder : public TreeBuilder {
         }
       }
       if (inspect_) KeepHist(level, L, hb);
-      LaunchSplit(level, L, hb, state, gp);
+      LaunchSplit(level, L, hb, state, gp, fused_ && !last);
       if (last) LaunchLeafWeights(L, state, gp);
       state ^= 1;
     }
@@ -2157,7 +2196,8 @@ class HipTreeBuilder : public TreeBuilder {
     return buf;
   }
 
-  void LaunchSplit(int level, int L, int hb, int state, const GainParams &gp) {
+  // plan_next: also plan the fused pass of the next level over these nodes
+  void LaunchSplit(int level, int L, int hb, int state, const GainParams &gp, bool plan_next = false) {
     Mark(kSplit);
     dim3 grid(F_, L);
     const int hs = std::min(cfg_.internal.hist_size, kSlots);
@@ -2169,10 +2209,23 @@ class HipTreeBuilder : public TreeBuilder {
     else if (f64_) ARB_SCAN(false, true);
     else ARB_SCAN(false, false);
 #undef ARB_SCAN
-    hipLaunchKernelGGL(k_split_select, dim3((L + 127) / 128), dim3(128), 0, stream_, d_cand_, F_, L,
-                       d_tot_[state], d_seg_[state], d_tot_[state ^ 1], d_seg_[state ^ 1], d_split_,
-                       d_tfid_, d_tbin_, d_tgain_, L - 1,
-                       sampling_ ? d_active_ + (size_t)level * F_ : (const unsigned char *)nullptr);
+    const unsigned char *active = sampling_ ? d_active_ + (size_t)level * F_ : (const unsigned char *)nullptr;
+    if (plan_next) {
+      const unsigned per_item = HistRowsPerItem(n_);
+      hipLaunchKernelGGL(k_select_plan, dim3(1), dim3(1024), 0, stream_, d_cand_, F_, L, d_tot_[state],
+                         d_seg_[state], d_tot_[state ^ 1], d_seg_[state ^ 1], d_split_, d_tfid_, d_tbin_, d_tgain_,
+                         L - 1, active, per_item, d_pwork_, d_nwork_ + 1, d_node_first_, d_node_items_,
+                         d_rows_scanned_, FusedGrid(L), d_overflow_);
+    } else {
+      hipLaunchKernelGGL(k_split_select, dim3((L + 127) / 128), dim3(128), 0, stream_, d_cand_, F_, L,
+                         d_tot_[state], d_seg_[state], d_tot_[state ^ 1], d_seg_[state ^ 1], d_split_,
+                         d_tfid_, d_tbin_, d_tgain_, L - 1, active);
+    }
+  }
+
+  // launch bound of the fused pass over PL parent nodes
+  unsigned FusedGrid(int PL) const {
+    return (unsigned)std::min<size_t>(n_ / HistRowsPerItem(n_) + PL + 1, max_part_items_);
   }
 
   void LaunchLeafWeights(int L, int state, const GainParams &gp) {
