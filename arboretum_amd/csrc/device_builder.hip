@@ -1614,12 +1614,29 @@ void QuantiseOnDevice(DataMatrix *data, int hist_size, bool verbose, bool stream
     float *d_x = DevAlloc<float>(4 * n);
     float *d_thr = DevAlloc<float>(4 * (size_t)hist_size);
     int *d_size = DevAlloc<int>(4);
+    // Columns go through two pinned staging buffers: the next column is copied
+    // there by host threads while the GPU sorts the current one, and the copy
+    // to the device runs at the full host-to-device rate.
+    float *stage[2] = {nullptr, nullptr};
+    for (int k = 0; k < 2; ++k) HIP_OK(hipHostMalloc((void **)&stage[k], n * sizeof(float), hipHostMallocDefault));
+    auto stage_column = [&](int f, int slot) {
+      const float *src = data->data[f].data();
+      float *dst = stage[slot];
+      ParallelFor(n, [&](size_t b, size_t e) { std::memcpy(dst + b, src + b, (e - b) * sizeof(float)); });
+    };
+    stage_column(0, 0);
     for (int q = 0; q < dm->Q; ++q) {
       const int nc = std::min(4, F - q * 4);
       int sizes[4] = {0, 0, 0, 0};
       for (int c = 0; c < nc; ++c) {
         const int f = q * 4 + c;
-        HIP_OK(hipMemcpy(d_x + (size_t)c * n, data->data[f].data(), n * sizeof(float), hipMemcpyHostToDevice));
+        std::thread next;
+        if (f + 1 < F) next = std::thread(stage_column, f + 1, (f + 1) & 1);
+        struct Joiner {
+          std::thread &t;
+          ~Joiner() { if (t.joinable()) t.join(); }
+        } joiner{next};
+        HIP_OK(hipMemcpy(d_x + (size_t)c * n, stage[f & 1], n * sizeof(float), hipMemcpyHostToDevice));
         bool has_nan = false;
         DeviceThresholds(ws.get(), d_x + (size_t)c * n, &data->thresholds[f], &data->reduced_size[f], &has_nan);
         if (data->reduced_size[f] + (has_nan ? 1 : 0) > kSlots)
@@ -1641,6 +1658,7 @@ void QuantiseOnDevice(DataMatrix *data, int hist_size, bool verbose, bool stream
     HIP_OK(hipFree(d_x));
     HIP_OK(hipFree(d_thr));
     HIP_OK(hipFree(d_size));
+    for (int k = 0; k < 2; ++k) HIP_OK(hipHostFree(stage[k]));
   }
   if (d_col) HIP_OK(hipFree(d_col));
   if (streamed) {

@@ -102,6 +102,36 @@ __global__ void __launch_bounds__(1024) k_rs_scan(unsigned *__restrict__ v, size
   }
 }
 
+// Exclusive scan of the tile counts of every digit: workgroup d scans
+// counts[d * nblk .. (d + 1) * nblk) in place and writes the digit's total.
+__global__ void __launch_bounds__(1024)
+k_rs_scan_digits(unsigned *__restrict__ counts, unsigned nblk, unsigned *__restrict__ digit_total) {
+  __shared__ unsigned s_wave[16];
+  __shared__ unsigned s_carry;
+  unsigned *v = counts + (size_t)blockIdx.x * nblk;
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  if (threadIdx.x == 0) s_carry = 0;
+  __syncthreads();
+  for (unsigned base = 0; base < nblk; base += 1024) {
+    const unsigned i = base + threadIdx.x;
+    const unsigned c = i < nblk ? v[i] : 0u;
+    unsigned incl = c;
+    for (int off = 1; off < 64; off <<= 1) {
+      const unsigned o = __shfl_up(incl, off);
+      if (lane >= off) incl += o;
+    }
+    if (lane == 63) s_wave[wave] = incl;
+    __syncthreads();
+    unsigned before = s_carry;
+    for (int w = 0; w < wave; ++w) before += s_wave[w];
+    if (i < nblk) v[i] = before + incl - c;
+    __syncthreads();
+    if (threadIdx.x == 1023) s_carry = before + incl;
+    __syncthreads();
+  }
+  if (threadIdx.x == 0) digit_total[blockIdx.x] = s_carry;
+}
+
 // Lanes of the wave holding the same 8-bit digit as this lane.
 __device__ __forceinline__ unsigned long long DigitPeers(unsigned d, bool valid) {
   unsigned long long peers = __ballot(valid);
@@ -117,11 +147,26 @@ __device__ __forceinline__ unsigned long long DigitPeers(unsigned d, bool valid)
 // first output position of the tile's keys with that digit.
 __global__ void __launch_bounds__(kSortThreads)
 k_rs_scatter(const unsigned *__restrict__ keys, unsigned *__restrict__ out, size_t n, int shift,
-             const unsigned *__restrict__ offsets, unsigned nblk) {
+             const unsigned *__restrict__ offsets, unsigned nblk,
+             const unsigned *__restrict__ digit_total) {
   __shared__ unsigned s_run[256];                       // keys of each digit already placed
   __shared__ unsigned s_wave[kSortThreads / 64][256];   // per wave counts of the current round
+  __shared__ unsigned s_tot[kSortThreads / 64];
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-  s_run[threadIdx.x] = offsets[(size_t)threadIdx.x * nblk + blockIdx.x];
+  {
+    // keys with a smaller digit: exclusive scan of the 256 digit totals (thread = digit)
+    const unsigned c = digit_total[threadIdx.x];
+    unsigned incl = c;
+    for (int off = 1; off < 64; off <<= 1) {
+      const unsigned o = __shfl_up(incl, off);
+      if (lane >= off) incl += o;
+    }
+    if (lane == 63) s_tot[wave] = incl;
+    __syncthreads();
+    unsigned before = 0;
+    for (int w = 0; w < wave; ++w) before += s_tot[w];
+    s_run[threadIdx.x] = before + incl - c + offsets[(size_t)threadIdx.x * nblk + blockIdx.x];
+  }
   for (int w = 0; w < kSortThreads / 64; ++w) s_wave[w][threadIdx.x] = 0;
   __syncthreads();
   const size_t base = (size_t)blockIdx.x * kSortTile;
@@ -179,28 +224,31 @@ k_thr_count(const unsigned *__restrict__ keys, size_t n, unsigned *__restrict__ 
 }
 
 // Thresholds as ordered keys: thr[slot] = min over the changes mapped to slot.
+// Every wave owns a contiguous quarter of the tile: it counts its changes,
+// the workgroup synchronises once, then the wave numbers its changes alone.
 __global__ void __launch_bounds__(kSortThreads)
 k_thr_emit(const unsigned *__restrict__ keys, size_t n, const unsigned *__restrict__ before, unsigned seg,
            int hist_size, unsigned *__restrict__ thr) {
-  __shared__ unsigned s_wave[kSortThreads / 64];
-  __shared__ unsigned s_run;
+  constexpr int kWaves = kSortThreads / 64;
+  constexpr int kWaveKeys = kSortTile / kWaves;
+  __shared__ unsigned s_wave[kWaves];
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-  if (threadIdx.x == 0) s_run = before[blockIdx.x];
+  const size_t wbase = (size_t)blockIdx.x * kSortTile + (size_t)wave * kWaveKeys;
+  unsigned mine = 0;
+  for (int j = 0; j < kWaveKeys; j += 64) {
+    const size_t i = wbase + j + lane;
+    mine += (unsigned)__popcll(__ballot(i < n && IsBorder(keys, i)));
+  }
+  if (lane == 0) s_wave[wave] = mine;
   __syncthreads();
-  const size_t base = (size_t)blockIdx.x * kSortTile;
-  for (int j = 0; j < kSortRounds; ++j) {
-    const size_t i = base + (size_t)j * kSortThreads + threadIdx.x;
+  unsigned run = before[blockIdx.x];  // changes before this wave's keys
+  for (int w = 0; w < wave; ++w) run += s_wave[w];
+  for (int j = 0; j < kWaveKeys; j += 64) {
+    const size_t i = wbase + j + lane;
     const bool border = i < n && IsBorder(keys, i);
     const unsigned long long m = __ballot(border);
-    if (lane == 0) s_wave[wave] = (unsigned)__popcll(m);
-    __syncthreads();
-    unsigned k = s_run + (unsigned)__popcll(m & ((1ull << lane) - 1ull)) + 1u;  // inclusive count
-    unsigned round_total = 0;
-    for (int w = 0; w < kSortThreads / 64; ++w) {
-      if (w < wave) k += s_wave[w];
-      round_total += s_wave[w];
-    }
     if (border) {
+      const unsigned k = run + (unsigned)__popcll(m & ((1ull << lane) - 1ull)) + 1u;  // inclusive count
       const float a = ValueOf(keys[i]), b = ValueOf(keys[i - 1]);
       const float mid = (float)((double)(float)(a + b) * 0.5);
       const unsigned long long pos_slot = (unsigned long long)(i / seg) + 1ull;
@@ -210,9 +258,7 @@ k_thr_emit(const unsigned *__restrict__ keys, size_t n, const unsigned *__restri
         if (mk < thr[slot]) atomicMin(&thr[slot], mk);
       }
     }
-    __syncthreads();
-    if (threadIdx.x == 0) s_run += round_total;
-    __syncthreads();
+    run += (unsigned)__popcll(m);
   }
 }
 
@@ -235,7 +281,7 @@ struct SortWorkspace {
   unsigned nblk = 0;
   int hist_size = 0;
   unsigned *keys[2] = {nullptr, nullptr};
-  unsigned *counts = nullptr, *thr = nullptr, *has_nan = nullptr;
+  unsigned *counts = nullptr, *digit_total = nullptr, *thr = nullptr, *has_nan = nullptr;
   float *thr_f = nullptr;
 };
 
@@ -247,6 +293,7 @@ SortWorkspace *CreateSortWorkspace(size_t n, int hist_size) {
   HIP_OK(hipMalloc((void **)&ws->keys[0], n * sizeof(unsigned)));
   HIP_OK(hipMalloc((void **)&ws->keys[1], n * sizeof(unsigned)));
   HIP_OK(hipMalloc((void **)&ws->counts, (size_t)256 * ws->nblk * sizeof(unsigned)));
+  HIP_OK(hipMalloc((void **)&ws->digit_total, 256 * sizeof(unsigned)));
   HIP_OK(hipMalloc((void **)&ws->thr, (size_t)hist_size * sizeof(unsigned)));
   HIP_OK(hipMalloc((void **)&ws->thr_f, (size_t)hist_size * sizeof(float)));
   HIP_OK(hipMalloc((void **)&ws->has_nan, sizeof(unsigned)));
@@ -255,7 +302,7 @@ SortWorkspace *CreateSortWorkspace(size_t n, int hist_size) {
 
 void FreeSortWorkspace(SortWorkspace *ws) {
   if (!ws) return;
-  void *p[] = {ws->keys[0], ws->keys[1], ws->counts, ws->thr, ws->thr_f, ws->has_nan};
+  void *p[] = {ws->keys[0], ws->keys[1], ws->counts, ws->digit_total, ws->thr, ws->thr_f, ws->has_nan};
   for (void *q : p)
     if (q) (void)hipFree(q);
   delete ws;
@@ -274,9 +321,9 @@ void DeviceThresholds(SortWorkspace *ws, const float *d_col, std::vector<float> 
   int cur = 0;
   for (int shift = 0; shift < 32; shift += 8) {
     hipLaunchKernelGGL(k_rs_count, dim3(nblk), dim3(kSortThreads), 0, 0, ws->keys[cur], n, shift, ws->counts, nblk);
-    hipLaunchKernelGGL(k_rs_scan, dim3(1), dim3(1024), 0, 0, ws->counts, (size_t)256 * nblk);
+    hipLaunchKernelGGL(k_rs_scan_digits, dim3(256), dim3(1024), 0, 0, ws->counts, nblk, ws->digit_total);
     hipLaunchKernelGGL(k_rs_scatter, dim3(nblk), dim3(kSortThreads), 0, 0, ws->keys[cur], ws->keys[cur ^ 1], n,
-                       shift, ws->counts, nblk);
+                       shift, ws->counts, nblk, ws->digit_total);
     cur ^= 1;
   }
   unsigned seg = (unsigned)(n / (size_t)hs);

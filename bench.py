@@ -25,6 +25,7 @@ import numpy as np
 ROOT = os.path.dirname(os.path.abspath(__file__))
 sys.path.insert(0, ROOT)
 
+MEASURED_FUSED_TRAFFIC_BYTES = 870.2e6  # 403.5 MiB fetched + 426.4 MiB written per launch
 HBM_PEAK = 8.0e12  # bytes/s, MI355X
 
 
@@ -219,6 +220,13 @@ def main():
     last_bytes = tm["fused_last_launches"] * args.rows * row_bytes
     last_s = tm["fused_last_ms"] * 1e-3
 
+    # HBM bytes per launch of the dominant kernel from hardware counters: two rocprofv3 --pmc
+    # runs of this file (FETCH_SIZE, WRITE_SIZE), scaled by the same counters over a copy of
+    # known size (--copy-probe); summary and commands in profiles/hbm_traffic_config2_*.txt.
+    # Only known for the default workload.
+    default_workload = (args.rows, F, args.hist_size, args.max_depth) == (10500000, 28, 256, 8)
+    traffic = MEASURED_FUSED_TRAFFIC_BYTES if default_workload else None
+
     def frac(b, t):
         return (b / t) / HBM_PEAK if t > 0 else 0.0
 
@@ -259,7 +267,7 @@ def main():
                                % (args.rows, F, args.hist_size, args.max_depth),
                    "rows": args.rows, "features": F, "bins": args.hist_size, "max_depth": args.max_depth},
         "roofline": {"bound": "hbm", "achieved": achieved / 1e9, "peak": HBM_PEAK / 1e9, "unit": "GB/s",
-                     "frac": achieved / HBM_PEAK, "traffic": None,
+                     "frac": achieved / HBM_PEAK, "traffic": traffic,
                      "kernel": "k_part_hist<true,7,true> (fused partition + histogram, levels 1..%d)"
                                % (args.max_depth - 2),
                      "launches": int(tm["hist_deep_launches"]),
