@@ -45,6 +45,8 @@ def _load_lib():
         "ACreateFromQuantized": [c_void_p, ctypes.c_longlong, c_int, P(c_void_p)],
         "AQuantize": [c_void_p, c_int],
         "AGetBins": [c_void_p, c_void_p],
+        "AGetBins16": [c_void_p, c_void_p],
+        "AGetBinLayout": [c_void_p, P(c_int), P(c_int)],
         "AGetThresholds": [c_void_p, c_int, c_void_p, P(c_int)],
         "AGardenSetInspect": [c_void_p, c_int],
         "AGardenNumTrees": [c_void_p, P(c_int)],
@@ -144,7 +146,17 @@ class DMatrix(object):
     def quantize(self, hist_size):
         _check(_LIB.AQuantize(self.handle, int(hist_size)))
 
+    def bin_layout(self):
+        """(bits per bin id, histogram slots per feature) of the quantised matrix."""
+        bits, slots = ctypes.c_int(), ctypes.c_int()
+        _check(_LIB.AGetBinLayout(self.handle, ctypes.byref(bits), ctypes.byref(slots)))
+        return bits.value, slots.value
+
     def bins(self):
+        if self.bin_layout()[0] == 16:
+            out = np.empty((self.rows, self.columns), dtype=np.uint16)
+            _check(_LIB.AGetBins16(self.handle, out.ctypes.data_as(ctypes.c_void_p)))
+            return out
         out = np.empty((self.rows, self.columns), dtype=np.uint8)
         _check(_LIB.AGetBins(self.handle, out.ctypes.data_as(ctypes.c_void_p)))
         return out
@@ -283,10 +295,11 @@ class Garden(object):
 
     def level_hist(self, level):
         nodes = 1 << level
-        out = np.empty((nodes, self.data.columns, 256, 3), dtype=np.int64)
+        slots = self.data.bin_layout()[1]
+        out = np.empty((nodes, self.data.columns, slots, 3), dtype=np.int64)
         cells = ctypes.c_int()
         _check(_LIB.AGardenGetLevelHist(self.handle, level, out.ctypes.data_as(ctypes.c_void_p), ctypes.byref(cells)))
-        assert cells.value == nodes * self.data.columns * 256
+        assert cells.value == nodes * self.data.columns * slots
         return out
 
     def shifts(self):

@@ -123,7 +123,9 @@ void DeviceThresholds(SortWorkspace *ws, const float *d_col, std::vector<float> 
 void QuantiseOnDevice(DataMatrix *data, int hist_size, bool verbose, bool streamed = false,
                       size_t block_rows = 0);
 void FreeDeviceMatrix(DeviceMatrix *m);
-void GetDeviceBins(const DataMatrix &data, uint8_t *out);  // row-major [rows][F]
+void GetDeviceBins(const DataMatrix &data, uint8_t *out);  // row-major [rows][F], 8-bit bins
+void GetDeviceBins16(const DataMatrix &data, uint16_t *out);  // row-major [rows][F], 16-bit bins
+void GetBinLayout(const DataMatrix &data, int *bits, int *slots);  // bits per bin id, histogram slots per feature
 TreeBuilder *CreateTreeBuilder(const Configuration &cfg, DataMatrix *data);
 int DeviceCount();
 void CopyProbe(size_t bytes);

@@ -68,6 +68,7 @@ namespace {
   } while (0)
 
 constexpr int kSlots = 256;               // histogram slots per feature (uint8 bins)
+constexpr int kMaxWideSlots = 4096;       // histogram slots per feature with 16-bit bins (power of two)
 constexpr int kHistThreads = 1024;        // one workgroup per CU, 16 waves
 constexpr int kItemWaves = kHistThreads / 64;  // waves per work item in row passes
 constexpr unsigned kPartRows = 16384;     // rows per work item of the stand-alone partition
@@ -148,6 +149,38 @@ __global__ void k_bin_assign(const float *__restrict__ x, int ncols, const float
         }
         packed |= l << (8 * c);
       }
+    }
+    out[r] = packed;
+  }
+}
+
+// The same with 16-bit bins: two features per word, thresholds of both in
+// dynamic LDS (2 * thr_stride floats).
+__global__ void k_bin_assign_wide(const float *__restrict__ x, int ncols, const float *__restrict__ thr,
+                                  int thr_stride, const int *__restrict__ sizes,
+                                  uint32_t *__restrict__ out, size_t n) {
+  extern __shared__ float s_thr_wide[];
+  for (int i = threadIdx.x; i < 2 * thr_stride; i += blockDim.x) {
+    const int c = i / thr_stride, t = i % thr_stride;
+    float v = INFINITY;
+    if (c < ncols && t < sizes[c] - 1) v = thr[(size_t)c * thr_stride + t];
+    s_thr_wide[i] = v;
+  }
+  __syncthreads();
+  for (size_t r = (size_t)blockIdx.x * blockDim.x + threadIdx.x; r < n;
+       r += (size_t)gridDim.x * blockDim.x) {
+    uint32_t packed = 0;
+    for (int c = 0; c < ncols; ++c) {
+      const float v = x[(size_t)c * n + r];
+      unsigned l = 0, h = (unsigned)sizes[c];
+      while (l < h) {
+        const unsigned mid = (l + h) >> 1;
+        if (v <= s_thr_wide[c * thr_stride + mid])
+          h = mid;
+        else
+          l = mid + 1;
+      }
+      packed |= l << (16 * c);
     }
     out[r] = packed;
   }
@@ -470,20 +503,75 @@ k_hist(const uint32_t *__restrict__ bins, size_t stride, int q0, int F,
   FlushSlab<PAIR, NQ>(lds, slab, w, slab_entries, q0);
 }
 
+// Histogram of contiguous row ranges with 16-bit bins: features [f0, f0 + nf)
+// (f0 even), `slots` histogram slots per feature, LDS layout f * slots + bin,
+// word0 of every entry first, then (PAIR) word1.  The slab of a work item has
+// the same feature-major order: word0[slab_entries], word1[slab_entries].
+template <bool PAIR>
+__global__ void __launch_bounds__(kHistThreads)
+k_hist_wide(const uint32_t *__restrict__ bins, size_t stride, int f0, int nf, int slots,
+            const float *__restrict__ g, const float *__restrict__ h, const int *__restrict__ shifts,
+            const WorkItem *__restrict__ work, const unsigned *__restrict__ n_work,
+            unsigned long long *__restrict__ slab, int slab_entries) {
+  extern __shared__ unsigned long long lds[];
+  const unsigned w = blockIdx.x;
+  if (w >= *n_work) return;
+  const WorkItem it = work[w];
+  const int entries = nf * slots;
+  for (int i = threadIdx.x; i < entries * (PAIR ? 2 : 1); i += kHistThreads) lds[i] = 0ull;
+  __syncthreads();
+  const int sg = shifts[0], sh = shifts[1];
+  const int words = (nf + 1) / 2;
+  for (unsigned r = it.begin + threadIdx.x; r < it.end; r += kHistThreads) {
+    const unsigned long long w0 = (1ull << kCountShift) + (unsigned long long)ToFixed(g[r], sg);
+    unsigned long long w1 = 0;
+    if (PAIR) w1 = (unsigned long long)ToFixed(h[r], sh);
+    for (int k = 0; k < words; ++k) {
+      const uint32_t word = bins[(size_t)(f0 / 2 + k) * stride + r];
+      const unsigned lo = (unsigned)(2 * k) * slots + (word & 0xffffu);
+      atomicAdd(&lds[lo], w0);
+      if (PAIR) atomicAdd(&lds[entries + lo], w1);
+      if (2 * k + 1 < nf) {
+        const unsigned hi = (unsigned)(2 * k + 1) * slots + (word >> 16);
+        atomicAdd(&lds[hi], w0);
+        if (PAIR) atomicAdd(&lds[entries + hi], w1);
+      }
+    }
+  }
+  __syncthreads();
+  unsigned long long *out = slab + (size_t)w * slab_entries * (PAIR ? 2 : 1) + (size_t)f0 * slots;
+  for (int e = threadIdx.x; e < entries; e += kHistThreads) {
+    out[e] = lds[e];
+    if (PAIR) out[slab_entries + e] = lds[entries + e];
+  }
+}
+
 // ---------------------------------------------------------------- partition
+// How bin ids are packed in the 32-bit words of a row: 8 bits (four features
+// per word) or 16 bits (two features per word).
+struct BinCode {
+  int wshift;  // feature -> word: fid >> wshift
+  int bits;
+  __host__ __device__ static BinCode Of(int bits) { return BinCode{bits == 8 ? 2 : 1, bits}; }
+  __device__ __forceinline__ int Word(int fid) const { return fid >> wshift; }
+  __device__ __forceinline__ unsigned Bin(uint32_t word, int fid) const {
+    return (word >> (bits * (fid & ((1 << wshift) - 1)))) & ((1u << bits) - 1u);
+  }
+};
+
 __device__ __forceinline__ bool GoesRight(const uint32_t *__restrict__ bins, size_t stride,
-                                          const SplitRec &s, unsigned r) {
+                                          const SplitRec &s, unsigned r, BinCode code = BinCode{2, 8}) {
   // builder.h:107-123: bin >= q + 1 goes right
   if (s.fid < 0) return false;
-  const uint32_t b4 = bins[(size_t)(s.fid >> 2) * stride + r];
-  return (int)((b4 >> (8 * (s.fid & 3))) & 255u) > s.bin;
+  const uint32_t word = bins[(size_t)code.Word(s.fid) * stride + r];
+  return (int)code.Bin(word, s.fid) > s.bin;
 }
 
 // Rows going left, per (work item, wave range).
 __global__ void __launch_bounds__(kHistThreads)
 k_part_count(const uint32_t *__restrict__ bins, size_t stride, const SplitRec *__restrict__ split,
              const WorkItem *__restrict__ work, const unsigned *__restrict__ n_work,
-             unsigned *__restrict__ wave_left, unsigned *__restrict__ item_left) {
+             unsigned *__restrict__ wave_left, unsigned *__restrict__ item_left, BinCode code) {
   const unsigned w = blockIdx.x;
   if (w >= *n_work) return;
   const WorkItem it = work[w];
@@ -494,8 +582,7 @@ k_part_count(const uint32_t *__restrict__ bins, size_t stride, const SplitRec *_
     for (unsigned base = it.begin + wave * kChunkRows; base < it.end; base += kChunkStep)
       cnt += lane == 0 ? min(kChunkRows, it.end - base) : 0u;
   } else {
-    const uint32_t *col = bins + (size_t)(s.fid >> 2) * stride;
-    const int sh = 8 * (s.fid & 3);
+    const uint32_t *col = bins + (size_t)code.Word(s.fid) * stride;
     // eight chunks (16 loads) in flight per wave: the pass is latency-bound
     constexpr int kBatch = 8;
     for (unsigned base = it.begin + wave * kChunkRows; base < it.end; base += kBatch * kChunkStep) {
@@ -509,8 +596,8 @@ k_part_count(const uint32_t *__restrict__ bins, size_t stride, const SplitRec *_
 #pragma unroll
       for (int k = 0; k < kBatch; ++k) {
         const unsigned r0 = base + k * kChunkStep + lane, r1 = r0 + 64;
-        if (r0 < it.end) cnt += ((int)((v0[k] >> sh) & 255u) > s.bin) ? 0u : 1u;
-        if (r1 < it.end) cnt += ((int)((v1[k] >> sh) & 255u) > s.bin) ? 0u : 1u;
+        if (r0 < it.end) cnt += ((int)code.Bin(v0[k], s.fid) > s.bin) ? 0u : 1u;
+        if (r1 < it.end) cnt += ((int)code.Bin(v1[k], s.fid) > s.bin) ? 0u : 1u;
       }
     }
   }
@@ -855,7 +942,7 @@ k_partition(const uint32_t *__restrict__ bins, uint32_t *__restrict__ bins_out, 
             float *__restrict__ h_out, const SplitRec *__restrict__ split,
             const unsigned *__restrict__ seg_start, const WorkItem *__restrict__ work,
             const unsigned *__restrict__ n_work, const unsigned *__restrict__ wave_left,
-            const unsigned *__restrict__ item_left) {
+            const unsigned *__restrict__ item_left, BinCode code) {
   __shared__ unsigned s_tmp[kItemWaves + 1];
   const unsigned w = blockIdx.x;
   if (w >= *n_work) return;
@@ -870,7 +957,7 @@ k_partition(const uint32_t *__restrict__ bins, uint32_t *__restrict__ bins_out, 
   for (unsigned base = chunk; base < min(chunk + kChunkRows, it.end); base += 64) {
     const unsigned r = base + lane;
     const bool valid = r < it.end;
-    const bool right = valid && GoesRight(bins, stride, s, r);
+    const bool right = valid && GoesRight(bins, stride, s, r, code);
     const unsigned long long lm = __ballot(valid && !right), rm = __ballot(right);
     if (valid) {
       const unsigned d = right ? ro + (unsigned)__popcll(rm & below) : lo + (unsigned)__popcll(lm & below);
@@ -908,7 +995,7 @@ k_hist_reduce(const unsigned long long *__restrict__ slab, int slab_entries, int
               const NodeSum *__restrict__ parent_tot, long long *__restrict__ hg,
               long long *__restrict__ hh, unsigned *__restrict__ hc,
               const long long *__restrict__ pg, const long long *__restrict__ ph,
-              const unsigned *__restrict__ pc, int trick, int accumulate) {
+              const unsigned *__restrict__ pc, int trick, int accumulate, int plain) {
   __shared__ long long s_g[16][64];
   __shared__ long long s_h[16][64];
   __shared__ unsigned s_c[16][64];
@@ -928,9 +1015,11 @@ k_hist_reduce(const unsigned long long *__restrict__ slab, int slab_entries, int
   }
   const int e = threadIdx.x & 63, lane = threadIdx.x >> 6;
   const int entry = blockIdx.x * 64 + e;  // slab order
+  // plain: the slabs are feature-major already (16-bit bins)
   const int f = (entry / kBlockEntries) * kBlockFeatures + (entry & (kBlockFeatures - 1));
   const int bin = (entry / kBlockFeatures) & (kSlots - 1);
-  const bool live = f * kSlots < nbin_total;  // the last block may have fewer than 16 features
+  // the last 16-feature block may have fewer than 16 features
+  const bool live = plain ? entry < nbin_total : f * kSlots < nbin_total;
   long long ag = 0, ah = 0;
   unsigned ac = 0;
   if (live) {
@@ -953,7 +1042,7 @@ k_hist_reduce(const unsigned long long *__restrict__ slab, int slab_entries, int
       ah += s_h[k][e];
       ac += s_c[k][e];
     }
-    const size_t cell = (size_t)f * kSlots + bin;
+    const size_t cell = plain ? (size_t)entry : (size_t)f * kSlots + bin;
     const size_t o = (size_t)nd * nbin_total + cell;
     if (accumulate) {  // streamed matrices: one call per row block
       ag += hg[o];
@@ -978,9 +1067,9 @@ k_hist_reduce(const unsigned long long *__restrict__ slab, int slab_entries, int
 // the gradient array of garden.cu:432-435.  One wave.
 __global__ void __launch_bounds__(64)
 k_root_from_hist(const long long *__restrict__ hg, const long long *__restrict__ hh,
-                 NodeSum *__restrict__ tot) {
+                 NodeSum *__restrict__ tot, int slots) {
   long long a = 0, b = 0;
-  for (int i = threadIdx.x; i < kSlots; i += 64) {
+  for (int i = threadIdx.x; i < slots; i += 64) {
     a += hg[i];
     b += hh[i];
   }
@@ -1154,7 +1243,7 @@ struct Cand {
 template <bool PAIR, bool F64>
 __global__ void __launch_bounds__(64)
 k_split_scan(const long long *__restrict__ hg, const long long *__restrict__ hh,
-             const unsigned *__restrict__ hc, int nbin_total, int F,
+             const unsigned *__restrict__ hc, int nbin_total, int F, int slots,
              const NodeSum *__restrict__ tot, const int *__restrict__ shifts, GainParams gp,
              int hist_size, Cand *__restrict__ cand) {
   const int f = blockIdx.x, nd = blockIdx.y, lane = threadIdx.x;
@@ -1166,54 +1255,62 @@ k_split_scan(const long long *__restrict__ hg, const long long *__restrict__ hh,
   best.left.c = 0;
   if (t.c != 0) {
     const int sg = shifts[0], sh = shifts[1];
-    const size_t base = (size_t)nd * nbin_total + (size_t)f * kSlots + lane * 4;
-    long long g4[4], h4[4];
-    unsigned long long c4[4];
-#pragma unroll
-    for (int j = 0; j < 4; ++j) {
-      g4[j] = hg[base + j];
-      h4[j] = PAIR ? hh[base + j] : 0;
-      c4[j] = hc[base + j];
-    }
-#pragma unroll
-    for (int j = 1; j < 4; ++j) {
-      g4[j] += g4[j - 1];
-      h4[j] += h4[j - 1];
-      c4[j] += c4[j - 1];
-    }
-    long long ig = g4[3], ih = h4[3];
-    unsigned long long ic = c4[3];
-    for (int off = 1; off < 64; off <<= 1) {
-      const long long og = __shfl_up(ig, off);
-      const long long oh = __shfl_up(ih, off);
-      const unsigned long long oc = __shfl_up(ic, off);
-      if (lane >= off) {
-        ig += og;
-        ih += oh;
-        ic += oc;
-      }
-    }
-    const long long eg = ig - g4[3], eh = ih - h4[3];
-    const unsigned long long ec = ic - c4[3];
     const double GT = FromFixed<F64>(t.g, sg);
     const double HT = PAIR ? FromFixed<F64>(t.h, sh) : 0.0;
+    // sums of the slots below the current chunk of 256
+    long long carry_g = 0, carry_h = 0;
+    unsigned long long carry_c = 0;
+    for (int chunk = 0; chunk < slots && chunk < hist_size; chunk += 256) {
+      const size_t base = (size_t)nd * nbin_total + (size_t)f * slots + chunk + lane * 4;
+      long long g4[4], h4[4];
+      unsigned long long c4[4];
 #pragma unroll
-    for (int j = 0; j < 4; ++j) {
-      const int bin = lane * 4 + j;
-      if (bin < hist_size) {
-        const long long lg = eg + g4[j], lh = eh + h4[j];
-        const unsigned long long lc = ec + c4[j];
-        const double GL = FromFixed<F64>(lg, sg);
-        const double HL = PAIR ? FromFixed<F64>(lh, sh) : 0.0;
-        const float gn = SplitGain<PAIR, F64>(GL, HL, lc, GT, HT, t.c, gp);
-        if (gn > 0.0f && gn >= best.gain) {
-          best.gain = gn;
-          best.bin = bin;
-          best.left.g = lg;
-          best.left.h = lh;
-          best.left.c = lc;
+      for (int j = 0; j < 4; ++j) {
+        g4[j] = hg[base + j];
+        h4[j] = PAIR ? hh[base + j] : 0;
+        c4[j] = hc[base + j];
+      }
+#pragma unroll
+      for (int j = 1; j < 4; ++j) {
+        g4[j] += g4[j - 1];
+        h4[j] += h4[j - 1];
+        c4[j] += c4[j - 1];
+      }
+      long long ig = g4[3], ih = h4[3];
+      unsigned long long ic = c4[3];
+      for (int off = 1; off < 64; off <<= 1) {
+        const long long og = __shfl_up(ig, off);
+        const long long oh = __shfl_up(ih, off);
+        const unsigned long long oc = __shfl_up(ic, off);
+        if (lane >= off) {
+          ig += og;
+          ih += oh;
+          ic += oc;
         }
       }
+      const long long eg = carry_g + ig - g4[3], eh = carry_h + ih - h4[3];
+      const unsigned long long ec = carry_c + ic - c4[3];
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        const int bin = chunk + lane * 4 + j;
+        if (bin < hist_size) {
+          const long long lg = eg + g4[j], lh = eh + h4[j];
+          const unsigned long long lc = ec + c4[j];
+          const double GL = FromFixed<F64>(lg, sg);
+          const double HL = PAIR ? FromFixed<F64>(lh, sh) : 0.0;
+          const float gn = SplitGain<PAIR, F64>(GL, HL, lc, GT, HT, t.c, gp);
+          if (gn > 0.0f && gn >= best.gain) {
+            best.gain = gn;
+            best.bin = bin;
+            best.left.g = lg;
+            best.left.h = lh;
+            best.left.c = lc;
+          }
+        }
+      }
+      carry_g += __shfl(ig, 63);
+      carry_h += __shfl(ih, 63);
+      carry_c += __shfl(ic, 63);
     }
     for (int off = 32; off > 0; off >>= 1) {
       const float og = __shfl_down(best.gain, off);
@@ -1349,7 +1446,8 @@ __global__ void __launch_bounds__(256)
 k_final(const uint32_t *__restrict__ bins, size_t stride, const int *__restrict__ t_fid,
         const int *__restrict__ t_bin, int depth, const float *__restrict__ weights,
         float *__restrict__ yhat, const float *__restrict__ y, unsigned *__restrict__ leaf_of,
-        float *__restrict__ g, float *__restrict__ h, unsigned *__restrict__ gmax_bits, size_t n) {
+        float *__restrict__ g, float *__restrict__ h, unsigned *__restrict__ gmax_bits, size_t n,
+        BinCode code) {
   extern __shared__ int s_nodes[];  // fid[internal], bin[internal]
   const int internal = (1 << (depth - 1)) - 1;
   for (int i = threadIdx.x; i < internal; i += blockDim.x) {
@@ -1371,15 +1469,15 @@ k_final(const uint32_t *__restrict__ bins, size_t stride, const int *__restrict_
       const int fid = s_nodes[id], bin = s_nodes[internal + id];
       unsigned right = 0;
       if (bin >= 0) {
-        uint32_t b4 = 0;
-        if (NQ > 0) {
+        if (NQ > 0) {  // 8-bit bins, all quads in registers
+          uint32_t b4 = 0;
           const int fq = fid >> 2;
 #pragma unroll
           for (int q = 0; q < NQ; ++q) b4 = q == fq ? b[q] : b4;
+          right = (int)((b4 >> (8 * (fid & 3))) & 255u) > bin ? 1u : 0u;
         } else {
-          b4 = bins[(size_t)(fid >> 2) * stride + i];
+          right = (int)code.Bin(bins[(size_t)code.Word(fid) * stride + i], fid) > bin ? 1u : 0u;
         }
-        right = (int)((b4 >> (8 * (fid & 3))) & 255u) > bin ? 1u : 0u;
       }
       node = node * 2 + right;
     }
@@ -1494,7 +1592,9 @@ inline int GridFor(size_t n, int block, int cap = 4096) {
 
 struct DeviceMatrix {
   size_t rows = 0, stride = 0;
-  int F = 0, Q = 0;
+  int F = 0, Q = 0;          // Q words of 32 bits per row
+  int bits = 8;              // bits per bin id: 8 (four features per word) or 16 (two)
+  int slots = kSlots;        // histogram slots per feature
   uint32_t *bins = nullptr;  // resident: [Q][stride] in HBM
   // streamed: pinned host blocks [Q][block_rows], block b = rows [b*block_rows, ...)
   bool streamed = false;
@@ -1624,36 +1724,61 @@ void QuantiseOnDevice(DataMatrix *data, int hist_size, bool verbose, bool stream
       float *dst = stage[slot];
       ParallelFor(n, [&](size_t b, size_t e) { std::memcpy(dst + b, src + b, (e - b) * sizeof(float)); });
     };
-    stage_column(0, 0);
-    for (int q = 0; q < dm->Q; ++q) {
-      const int nc = std::min(4, F - q * 4);
-      int sizes[4] = {0, 0, 0, 0};
-      for (int c = 0; c < nc; ++c) {
-        const int f = q * 4 + c;
-        std::thread next;
-        if (f + 1 < F) next = std::thread(stage_column, f + 1, (f + 1) & 1);
-        struct Joiner {
-          std::thread &t;
-          ~Joiner() { if (t.joinable()) t.join(); }
-        } joiner{next};
-        HIP_OK(hipMemcpy(d_x + (size_t)c * n, stage[f & 1], n * sizeof(float), hipMemcpyHostToDevice));
-        bool has_nan = false;
-        DeviceThresholds(ws.get(), d_x + (size_t)c * n, &data->thresholds[f], &data->reduced_size[f], &has_nan);
-        if (data->reduced_size[f] + (has_nan ? 1 : 0) > kSlots)
-          throw std::runtime_error("a feature needs more than 256 bin ids: 16-bit bins are not implemented");
-        if (verbose)
-          printf("feature %d has been reduced to %d bits \n", f,
-                 32 - __builtin_clz((unsigned)data->reduced_size[f]));
-        HIP_OK(hipMemcpy(d_thr + (size_t)c * hist_size, data->thresholds[f].data(),
-                         hist_size * sizeof(float), hipMemcpyHostToDevice));
-        sizes[c] = data->reduced_size[f];
+    // One pass over the columns with `bits` bits per bin id; false when a
+    // feature needs more ids than 8 bits hold.
+    auto quantise_columns = [&](int bits) -> bool {
+      const int W = 32 / bits;  // features per word
+      stage_column(0, 0);
+      for (int q = 0; q < dm->Q; ++q) {
+        const int nc = std::min(W, F - q * W);
+        int sizes[4] = {0, 0, 0, 0};
+        for (int c = 0; c < nc; ++c) {
+          const int f = q * W + c;
+          std::thread next;
+          if (f + 1 < F) next = std::thread(stage_column, f + 1, (f + 1) & 1);
+          struct Joiner {
+            std::thread &t;
+            ~Joiner() { if (t.joinable()) t.join(); }
+          } joiner{next};
+          HIP_OK(hipMemcpy(d_x + (size_t)c * n, stage[f & 1], n * sizeof(float), hipMemcpyHostToDevice));
+          bool has_nan = false;
+          DeviceThresholds(ws.get(), d_x + (size_t)c * n, &data->thresholds[f], &data->reduced_size[f], &has_nan);
+          if (bits == 8 && data->reduced_size[f] + (has_nan ? 1 : 0) > kSlots) return false;
+          if (verbose)
+            printf("feature %d has been reduced to %d bits \n", f,
+                   32 - __builtin_clz((unsigned)data->reduced_size[f]));
+          HIP_OK(hipMemcpy(d_thr + (size_t)c * hist_size, data->thresholds[f].data(),
+                           hist_size * sizeof(float), hipMemcpyHostToDevice));
+          sizes[c] = data->reduced_size[f];
+        }
+        HIP_OK(hipMemcpy(d_size, sizes, sizeof(sizes), hipMemcpyHostToDevice));
+        uint32_t *out = streamed ? d_col : dm->bins + (size_t)q * dm->stride;
+        if (bits == 8)
+          hipLaunchKernelGGL(k_bin_assign, dim3(GridFor(n, 256)), dim3(256), 0, 0, d_x, nc, d_thr, hist_size, d_size,
+                             out, n);
+        else
+          hipLaunchKernelGGL(k_bin_assign_wide, dim3(GridFor(n, 256)), dim3(256),
+                             2 * (size_t)hist_size * sizeof(float), 0, d_x, nc, d_thr, hist_size, d_size, out, n);
+        HIP_OK(hipGetLastError());
+        HIP_OK(hipDeviceSynchronize());
+        if (streamed) store_quad(q);
       }
-      HIP_OK(hipMemcpy(d_size, sizes, sizeof(sizes), hipMemcpyHostToDevice));
-      hipLaunchKernelGGL(k_bin_assign, dim3(GridFor(n, 256)), dim3(256), 0, 0, d_x, nc, d_thr,
-                         hist_size, d_size, streamed ? d_col : dm->bins + (size_t)q * dm->stride, n);
-      HIP_OK(hipGetLastError());
-      HIP_OK(hipDeviceSynchronize());
-      if (streamed) store_quad(q);
+      return true;
+    };
+    if (!quantise_columns(8)) {
+      // Some feature has more than 256 bin ids: 16-bit bins, two features per
+      // word, hist_size + 1 slots per feature rounded up to a power of two.
+      if (streamed) throw std::runtime_error("a feature needs more than 256 bin ids: 16-bit bins are not built for streamed matrices");
+      int slots = kSlots;
+      while (slots < hist_size + 1) slots *= 2;
+      if (slots > kMaxWideSlots) throw std::runtime_error("hist_size above 4095 is not supported");
+      HIP_OK(hipFree(dm->bins));
+      dm->bins = nullptr;
+      dm->bits = 16;
+      dm->slots = slots;
+      dm->Q = (F + 1) / 2;
+      dm->bins = DevAlloc<uint32_t>((size_t)dm->Q * dm->stride);
+      if (!quantise_columns(16)) throw std::runtime_error("internal: 16-bit quantisation failed");
     }
     HIP_OK(hipFree(d_x));
     HIP_OK(hipFree(d_thr));
@@ -1670,9 +1795,28 @@ void QuantiseOnDevice(DataMatrix *data, int hist_size, bool verbose, bool stream
   data->quantised = true;
 }
 
+void GetBinLayout(const DataMatrix &data, int *bits, int *slots) {
+  const DeviceMatrix *dm = data.device;
+  if (!dm) throw std::runtime_error("data matrix is not quantised");
+  *bits = dm->bits;
+  *slots = dm->slots;
+}
+
+void GetDeviceBins16(const DataMatrix &data, uint16_t *out) {
+  const DeviceMatrix *dm = data.device;
+  if (!dm) throw std::runtime_error("data matrix is not quantised");
+  if (dm->bits != 16) throw std::runtime_error("the matrix has 8-bit bins");
+  std::vector<uint32_t> q((size_t)dm->Q * dm->stride);
+  HIP_OK(hipMemcpy(q.data(), dm->bins, q.size() * sizeof(uint32_t), hipMemcpyDeviceToHost));
+  for (size_t r = 0; r < dm->rows; ++r)
+    for (int f = 0; f < dm->F; ++f)
+      out[r * dm->F + f] = (uint16_t)(q[(size_t)(f >> 1) * dm->stride + r] >> (16 * (f & 1)));
+}
+
 void GetDeviceBins(const DataMatrix &data, uint8_t *out) {
   const DeviceMatrix *dm = data.device;
   if (!dm) throw std::runtime_error("data matrix is not quantised");
+  if (dm->bits != 8) throw std::runtime_error("the matrix has 16-bit bins");
   if (dm->streamed) {
     for (size_t r = 0; r < dm->rows; ++r) {
       const uint32_t *blk = dm->host_blocks[r / dm->block_rows];
@@ -1789,8 +1933,17 @@ class HipTreeBuilder : public TreeBuilder {
     pair_ = cfg.objective != kLinearRegression;
     f64_ = cfg.internal.double_precision;
     trick_ = cfg.internal.use_hist_subtraction_trick;
-    nbin_total_ = Q_ * 4 * kSlots;
-    slab_entries_ = HistBlocks(Q_) * kBlockEntries;
+    wide_ = dm_->bits == 16;
+    slots_ = dm_->slots;
+    code_ = BinCode::Of(dm_->bits);
+    if (wide_) {
+      if (dm_->streamed) throw std::runtime_error("16-bit bins are not built for streamed matrices");
+      nbin_total_ = F_ * slots_;
+      slab_entries_ = nbin_total_;  // slabs are feature-major
+    } else {
+      nbin_total_ = Q_ * 4 * kSlots;
+      slab_entries_ = HistBlocks(Q_) * kBlockEntries;
+    }
     if (cfg.objective >= kSoftMaxOneVsAll && K_ < 2) throw std::runtime_error("soft-max needs labels_count >= 2");
     if (cfg.objective < kSoftMaxOneVsAll && K_ != 1) throw std::runtime_error("labels_count must be 1 for this objective");
     const int last_nodes = 1 << (D_ - 2);
@@ -1804,7 +1957,12 @@ class HipTreeBuilder : public TreeBuilder {
     quads_per_group_ = std::min(quads_per_group_, Q_);
     // the fused partition + histogram pass holds one histogram of all
     // features and builds only the smaller child
-    fused_ = trick_ && Q_ <= quads_per_group_;
+    fused_ = trick_ && Q_ <= quads_per_group_ && !wide_;
+    if (wide_) {
+      // features per histogram launch (an even number, two per word)
+      const size_t per_feature = (size_t)slots_ * 8 * (pair_ ? 2 : 1);
+      wide_group_ = (int)std::max<size_t>(2, (kLdsBudget - 1024) / per_feature / 2 * 2);
+    }
 
     // per-row state in original order
     d_y_ = DevAlloc<float>(n_);
@@ -2052,6 +2210,24 @@ class HipTreeBuilder : public TreeBuilder {
     Mark(kPlan);
     Plan(state, L, select_smaller ? 1 : 0, per_item, d_hwork_, d_nwork_, true, nullptr, grid);
     Mark(root ? kHistRoot : kHistDeep);
+    if (wide_) {
+      for (int f0 = 0; f0 < F_; f0 += wide_group_) {
+        const int nf = std::min(wide_group_, F_ - f0);
+        const size_t lds = (size_t)nf * slots_ * 8 * (pair_ ? 2 : 1);
+        if (pair_) {
+          AllowLds(k_hist_wide<true>, kLdsBudget);
+          hipLaunchKernelGGL(k_hist_wide<true>, dim3(grid), dim3(kHistThreads), lds, stream_, cur.bins, stride_, f0, nf,
+                             slots_, cur.g, cur.h, d_shifts_, d_hwork_, d_nwork_, d_slab_, slab_entries_);
+        } else {
+          AllowLds(k_hist_wide<false>, kLdsBudget);
+          hipLaunchKernelGGL(k_hist_wide<false>, dim3(grid), dim3(kHistThreads), lds, stream_, cur.bins, stride_, f0, nf,
+                             slots_, cur.g, cur.h, d_shifts_, d_hwork_, d_nwork_, d_slab_, slab_entries_);
+        }
+        if (timing_) ++(root ? timings_.hist_root_launches : timings_.hist_deep_launches);
+      }
+      if (timing_ && root) timings_.hist_root_rows += n_;
+      return;
+    }
     for (int q0 = 0; q0 < Q_; q0 += quads_per_group_) {
       const int nq = std::min(quads_per_group_, Q_ - q0);
       if (pair_)
@@ -2065,15 +2241,17 @@ class HipTreeBuilder : public TreeBuilder {
 
   void Reduce(int L, int hb, bool by_parent, int parent_state, bool trick, bool accumulate = false) {
     Mark(kReduce);
-    dim3 grid(slab_entries_ / 64, L);
+    dim3 grid((slab_entries_ + 63) / 64, L);
     if (pair_)
       hipLaunchKernelGGL(k_hist_reduce<true>, grid, dim3(1024), 0, stream_, d_slab_, slab_entries_, nbin_total_, d_node_first_,
                          d_node_items_, by_parent ? 1 : 0, d_split_, d_tot_[parent_state], d_hg_[hb], d_hh_[hb],
-                         d_hc_[hb], d_hg_[hb ^ 1], d_hh_[hb ^ 1], d_hc_[hb ^ 1], trick ? 1 : 0, accumulate ? 1 : 0);
+                         d_hc_[hb], d_hg_[hb ^ 1], d_hh_[hb ^ 1], d_hc_[hb ^ 1], trick ? 1 : 0, accumulate ? 1 : 0,
+                         wide_ ? 1 : 0);
     else
       hipLaunchKernelGGL(k_hist_reduce<false>, grid, dim3(1024), 0, stream_, d_slab_, slab_entries_, nbin_total_, d_node_first_,
                          d_node_items_, by_parent ? 1 : 0, d_split_, d_tot_[parent_state], d_hg_[hb], d_hh_[hb],
-                         d_hc_[hb], d_hg_[hb ^ 1], d_hh_[hb ^ 1], d_hc_[hb ^ 1], trick ? 1 : 0, accumulate ? 1 : 0);
+                         d_hc_[hb], d_hg_[hb ^ 1], d_hh_[hb ^ 1], d_hc_[hb ^ 1], trick ? 1 : 0, accumulate ? 1 : 0,
+                         wide_ ? 1 : 0);
   }
 
   void GrowOne(int label, RegTree *tree) {
@@ -2101,7 +2279,7 @@ class HipTreeBuilder : public TreeBuilder {
         if (!root_hist_ready_) HistOfNodes(orig, state, 1, false, n_, true);
         root_hist_ready_ = false;
         Reduce(1, hb, false, state, false);
-        hipLaunchKernelGGL(k_root_from_hist, dim3(1), dim3(64), 0, stream_, d_hg_[hb], d_hh_[hb], d_tot_[state]);
+        hipLaunchKernelGGL(k_root_from_hist, dim3(1), dim3(64), 0, stream_, d_hg_[hb], d_hh_[hb], d_tot_[state], slots_);
       } else {
         // rows are in the order of level-1; the parents' state is state ^ 1
         const int ps = state ^ 1, PL = L >> 1;
@@ -2113,7 +2291,7 @@ class HipTreeBuilder : public TreeBuilder {
           if (!last) {  // destination offsets; the last level moves no rows
             Mark(kPartition);
             hipLaunchKernelGGL(k_part_count, dim3(grid), dim3(kHistThreads), 0, stream_, src.bins, stride_, d_split_,
-                               d_pwork_, d_nwork_ + 1, d_wave_left_, d_item_left_);
+                               d_pwork_, d_nwork_ + 1, d_wave_left_, d_item_left_, code_);
           }
           Mark(last ? kFusedLast : kHistDeep);
           FusedArgs a{src.bins, dst.bins, stride_, F_, src.g, dst.g, src.h, dst.h, d_shifts_, d_split_,
@@ -2133,15 +2311,15 @@ class HipTreeBuilder : public TreeBuilder {
           Plan(ps, PL, 0, kPartRows, d_pwork_, d_nwork_ + 1, false, nullptr, grid);
           Mark(kPartition);
           hipLaunchKernelGGL(k_part_count, dim3(grid), dim3(kHistThreads), 0, stream_, src.bins, stride_, d_split_,
-                             d_pwork_, d_nwork_ + 1, d_wave_left_, d_item_left_);
+                             d_pwork_, d_nwork_ + 1, d_wave_left_, d_item_left_, code_);
           if (pair_)
             hipLaunchKernelGGL(k_partition<true>, dim3(grid), dim3(kHistThreads), 0, stream_, src.bins, dst.bins,
                                stride_, Q_, src.g, dst.g, src.h, dst.h, d_split_, d_seg_[ps], d_pwork_,
-                               d_nwork_ + 1, d_wave_left_, d_item_left_);
+                               d_nwork_ + 1, d_wave_left_, d_item_left_, code_);
           else
             hipLaunchKernelGGL(k_partition<false>, dim3(grid), dim3(kHistThreads), 0, stream_, src.bins, dst.bins,
                                stride_, Q_, src.g, dst.g, src.h, dst.h, d_split_, d_seg_[ps], d_pwork_,
-                               d_nwork_ + 1, d_wave_left_, d_item_left_);
+                               d_nwork_ + 1, d_wave_left_, d_item_left_, code_);
           HistOfNodes(dst, state, L, trick_, trick_ ? n_ / 2 : n_, false);
           Reduce(L, hb, false, ps, trick_);
         }
@@ -2158,7 +2336,8 @@ class HipTreeBuilder : public TreeBuilder {
       if (cfg_.objective == kLinearRegression) HIP_OK(hipMemsetAsync(d_gmax_, 0, sizeof(unsigned), stream_));
       const int internal = (1 << (D_ - 1)) - 1;
       const size_t lds = HistLdsBytes(Q_, true) + (size_t)internal * 2 * sizeof(int);
-      if (next_grad && cfg_.objective == kLogisticRegression && Q_ <= quads_per_group_ && lds <= kLdsBudget) {
+      if (next_grad && cfg_.objective == kLogisticRegression && Q_ <= quads_per_group_ && !wide_ &&
+          lds <= kLdsBudget) {
         // plan of the next tree's root, then one pass: leaves, predictions,
         // gradients and the root histogram of the next tree
         hipLaunchKernelGGL(k_init_root, dim3(1), dim3(64), 0, stream_, d_tot_[0], d_seg_[0],
@@ -2218,10 +2397,10 @@ class HipTreeBuilder : public TreeBuilder {
   void LaunchSplit(int level, int L, int hb, int state, const GainParams &gp, bool plan_next = false) {
     Mark(kSplit);
     dim3 grid(F_, L);
-    const int hs = std::min(cfg_.internal.hist_size, kSlots);
+    const int hs = std::min(cfg_.internal.hist_size, slots_);
 #define ARB_SCAN(P, D) \
   hipLaunchKernelGGL((k_split_scan<P, D>), grid, dim3(64), 0, stream_, d_hg_[hb], d_hh_[hb], d_hc_[hb], \
-                     nbin_total_, F_, d_tot_[state], d_shifts_, gp, hs, d_cand_)
+                     nbin_total_, F_, slots_, d_tot_[state], d_shifts_, gp, hs, d_cand_)
     if (pair_ && f64_) ARB_SCAN(true, true);
     else if (pair_) ARB_SCAN(true, false);
     else if (f64_) ARB_SCAN(false, true);
@@ -2269,10 +2448,10 @@ class HipTreeBuilder : public TreeBuilder {
     if (next_grad && cfg_.objective == kLogisticRegression) mode = 2;
 #define ARB_FINAL(M, N) \
   hipLaunchKernelGGL((k_final<M, N>), dim3(grid), dim3(256), lds, stream_, bins, stride, d_tfid_, d_tbin_, D_, \
-                     d_weights_, yh, d_y_ + row0, d_leaf_ + row0, d_g_ + row0, d_h_ + row0, d_gmax_, rows)
+                     d_weights_, yh, d_y_ + row0, d_leaf_ + row0, d_g_ + row0, d_h_ + row0, d_gmax_, rows, code_)
 #define ARB_FINAL_Q(N) \
   do { if (mode == 1) ARB_FINAL(1, N); else if (mode == 2) ARB_FINAL(2, N); else ARB_FINAL(0, N); } while (0)
-    switch (Q_ <= 8 ? Q_ : 0) {
+    switch (Q_ <= 8 && !wide_ ? Q_ : 0) {
       case 1: ARB_FINAL_Q(1); break;
       case 2: ARB_FINAL_Q(2); break;
       case 3: ARB_FINAL_Q(3); break;
@@ -2357,7 +2536,7 @@ class HipTreeBuilder : public TreeBuilder {
         Reduce(L, hb, false, state, false, b > 0);
       }
       if (level == 0)
-        hipLaunchKernelGGL(k_root_from_hist, dim3(1), dim3(64), 0, stream_, d_hg_[hb], d_hh_[hb], d_tot_[state]);
+        hipLaunchKernelGGL(k_root_from_hist, dim3(1), dim3(64), 0, stream_, d_hg_[hb], d_hh_[hb], d_tot_[state], slots_);
       if (trick)
         hipLaunchKernelGGL(k_sibling, dim3((nbin_total_ + 255) / 256, L), dim3(256), 0, stream_, d_hg_[hb], d_hh_[hb],
                            d_hc_[hb], d_hg_[hb ^ 1], d_hh_[hb ^ 1], d_hc_[hb ^ 1], d_tot_[state], level, nbin_total_);
@@ -2414,14 +2593,14 @@ class HipTreeBuilder : public TreeBuilder {
     HIP_OK(hipMemcpy(g.data(), d_hg_[hb], cells * sizeof(long long), hipMemcpyDeviceToHost));
     HIP_OK(hipMemcpy(h.data(), d_hh_[hb], cells * sizeof(long long), hipMemcpyDeviceToHost));
     HIP_OK(hipMemcpy(c.data(), d_hc_[hb], cells * sizeof(unsigned), hipMemcpyDeviceToHost));
-    // keep [node][F][256][3] (padding features of the last quad dropped)
+    // keep [node][F][slots][3] (padding features of the last quad dropped)
     std::vector<int64_t> &out = kept_hist_[level];
-    out.resize((size_t)L * F_ * kSlots * 3);
+    out.resize((size_t)L * F_ * slots_ * 3);
     for (int nd = 0; nd < L; ++nd)
       for (int f = 0; f < F_; ++f)
-        for (int b = 0; b < kSlots; ++b) {
-          const size_t s = (size_t)nd * nbin_total_ + (size_t)f * kSlots + b;
-          const size_t d = (((size_t)nd * F_ + f) * kSlots + b) * 3;
+        for (int b = 0; b < slots_; ++b) {
+          const size_t s = (size_t)nd * nbin_total_ + (size_t)f * slots_ + b;
+          const size_t d = (((size_t)nd * F_ + f) * slots_ + b) * 3;
           out[d] = g[s];
           out[d + 1] = pair_ ? h[s] : 0;
           out[d + 2] = c[s];
@@ -2434,6 +2613,10 @@ class HipTreeBuilder : public TreeBuilder {
   size_t n_ = 0, stride_ = 0;
   int F_ = 0, Q_ = 0, K_ = 1, D_ = 2, nbin_total_ = 0;
   int slab_entries_ = 0;  // histogram entries of one work item's slab (whole 16-feature blocks)
+  bool wide_ = false;     // 16-bit bins: two features per word, slots_ histogram slots per feature
+  int slots_ = kSlots;
+  int wide_group_ = 2;    // features per histogram launch with 16-bit bins
+  BinCode code_ = BinCode{2, 8};
   bool root_hist_ready_ = false;  // the slabs hold the root histogram of the tree grown next
   bool pair_ = false, f64_ = false, trick_ = true, fused_ = false, inspect_ = false, timing_ = false;
   bool grad_ready_ = false;

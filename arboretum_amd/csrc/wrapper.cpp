@@ -205,6 +205,14 @@ const char *AGetBins(VoidPointer data, unsigned char *out) {
   return Guard([&] { GetDeviceBins(*AsData(data), out); });
 }
 
+const char *AGetBins16(VoidPointer data, unsigned short *out) {
+  return Guard([&] { GetDeviceBins16(*AsData(data), out); });
+}
+
+const char *AGetBinLayout(VoidPointer data, int *bits, int *slots) {
+  return Guard([&] { GetBinLayout(*AsData(data), bits, slots); });
+}
+
 const char *AGetThresholds(VoidPointer data, int fid, float *thr, int *size) {
   return Guard([&] {
     DataMatrix *d = AsData(data);

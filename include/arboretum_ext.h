@@ -39,6 +39,13 @@ const char *AQuantize(VoidPointer data, int hist_size);
  * (DataMatrix::data_reduced_mapping / reduced_size, src/io/io.h:24,32). */
 const char *AGetBins(VoidPointer data, unsigned char *out);
 const char *AGetThresholds(VoidPointer data, int fid, float *thr, int *size);
+/* Bin ids take 8 bits unless a feature has more than 256 of them (hist_size
+ * above 255 on a column with that many distinct values): then 16 bits, as the
+ * reference switches BIN_T by hist_size (src/core/garden.cu:506-569).
+ * AGetBinLayout: bits per bin id (8 or 16) and histogram slots per feature;
+ * AGetBins16: the bins as row-major uint16 [nrow][ncol] (AGetBins is for 8). */
+const char *AGetBinLayout(VoidPointer data, int *bits, int *slots);
+const char *AGetBins16(VoidPointer data, unsigned short *out);
 
 /* Inspection of the booster; valid after AGrowTree. */
 const char *AGardenSetInspect(VoidPointer garden, int on);      /* keep per-level histograms */

@@ -46,7 +46,8 @@ def assert_same_training(arb, oracle, X, y, cfg, rounds, check_hist=True):
         ob.grow(1)
         g.grow_tree()
         if r == 0:
-            assert np.array_equal(data.bins(), ob.bins().astype(np.uint8)), "bins"
+            gb = data.bins()
+            assert np.array_equal(gb, ob.bins().astype(gb.dtype)), "bins"
             for f in range(X.shape[1]):
                 t0, s0 = ob.thresholds(f)
                 t1, s1 = data.thresholds(f, hs)
@@ -61,11 +62,12 @@ def assert_same_training(arb, oracle, X, y, cfg, rounds, check_hist=True):
             for level in range(D - 1):
                 ho = ob.level_hist(level)[:, :, :hs + 1, :]
                 hg = g.level_hist(level)
-                if hs + 1 <= 256:
+                slots = hg.shape[2]
+                if hs + 1 <= slots:
                     assert np.array_equal(hg[:, :, :hs + 1, :], ho), "hist level %d round %d" % (level, r)
                     assert not hg[:, :, hs + 1:, :].any()
-                else:
-                    assert np.array_equal(hg, ho[:, :, :256, :])
+                else:  # hist_size above 255 on columns with few distinct values: 8-bit bins
+                    assert np.array_equal(hg, ho[:, :, :slots, :])
         to, tg = ob.tree(r), g.tree(r)
         assert np.array_equal(to["fid"], tg["fid"]), "fid round %d" % r
         assert np.array_equal(to["quantized"], tg["quantized"]), "bin round %d" % r
@@ -252,6 +254,36 @@ def test_max_depth_1(arb, oracle):
     cfg = {"objective": 0, "method": 1, "internals": {"hist_size": 255},
            "tree": {"max_depth": 1, "eta": 0.5, "lambda": 1.0}}
     assert_same_training(arb, oracle, X, y, cfg, rounds=2)
+
+
+# ------------------------------------------------------------ 16-bit bins
+@pytest.mark.parametrize("objective", [0, 1])
+@pytest.mark.parametrize("trick", [True, False])
+@pytest.mark.parametrize("hist_size,F", [(1000, 5), (300, 3), (4095, 2)])
+def test_sixteen_bit_bins(arb, oracle, objective, trick, hist_size, F):
+    # continuous columns with hist_size above 255 need more than 256 bin ids per feature
+    X, y = make_data(30000, F, objective, seed=hist_size, nan_frac=0.02)
+    X[:, : (F + 1) // 2] = np.random.default_rng(1).normal(size=(30000, (F + 1) // 2)).astype(np.float32)
+    cfg = {"objective": objective, "method": 1,
+           "internals": {"hist_size": hist_size, "double_precision": True, "use_hist_subtraction_trick": trick},
+           "tree": {"max_depth": 5, "eta": 0.4, "lambda": 1.0, "min_child_weight": 0.5}}
+    ob, g = assert_same_training(arb, oracle, X, y, cfg, rounds=2)
+    bits, slots = g.data.bin_layout()
+    assert bits == 16 and slots >= hist_size + 1
+
+
+def test_sixteen_bit_bins_without_inspection_and_limits(arb, oracle):
+    X, y = make_data(9000, 4, 1, seed=5)
+    X[:, 0] = np.random.default_rng(2).normal(size=9000).astype(np.float32)
+    cfg = {"objective": 1, "method": 1, "internals": {"hist_size": 600, "double_precision": False},
+           "tree": {"max_depth": 4, "eta": 0.3, "lambda": 1.0}}
+    assert_same_training(arb, oracle, X, y, cfg, rounds=3, check_hist=False)
+    too_many = dict(cfg, internals={"hist_size": 5000})
+    with pytest.raises(Exception, match="hist_size above 4095"):
+        arb.Garden(too_many, arb.DMatrix(X, y=y)).grow_tree()
+    streamed = dict(cfg, internals={"hist_size": 600, "upload_features": False})
+    with pytest.raises(Exception, match="16-bit bins are not built for streamed"):
+        arb.Garden(streamed, arb.DMatrix(X, y=y)).grow_tree()
 
 
 def _skewed_matrix(n, seed):
