@@ -698,7 +698,8 @@ struct RowQueue {
 
 // Writes lanes [from, to) of Q to their destination and, for the child whose
 // histogram is built, adds them to the LDS histogram.
-template <bool PAIR, int NQ>
+// HIST: the kernel builds a histogram; GH: the gradients move with the rows.
+template <bool PAIR, int NQ, bool HIST = true, bool GH = true>
 __device__ __forceinline__ void EmitRows(unsigned long long *__restrict__ lds, const RowQueue<NQ> &Q,
                                          unsigned from, unsigned to, bool built,
                                          uint32_t *__restrict__ bins_out, size_t stride,
@@ -709,16 +710,18 @@ __device__ __forceinline__ void EmitRows(unsigned long long *__restrict__ lds, c
     const unsigned d = Q.base + (unsigned)lane;
 #pragma unroll
     for (int q = 0; q < NQ; ++q) __builtin_nontemporal_store(Q.b[q], &bins_out[(size_t)q * stride + d]);
-    __builtin_nontemporal_store(Q.g, &g_out[d]);
-    if (PAIR) __builtin_nontemporal_store(Q.h, &h_out[d]);
-    if (built) AccumulateRow<PAIR, NQ>(lds, Q.b, Q.g, Q.h, sg, sh, 0, F);
+    if (GH) {
+      __builtin_nontemporal_store(Q.g, &g_out[d]);
+      if (PAIR) __builtin_nontemporal_store(Q.h, &h_out[d]);
+    }
+    if (HIST && built) AccumulateRow<PAIR, NQ>(lds, Q.b, Q.g, Q.h, sg, sh, 0, F);
   }
 }
 
 // Appends the rows of X flagged in xm (wave-uniform mask, one row per lane) to
 // Q in row order with one lane permute per register; a full queue is emitted
 // and the rest of X starts the next batch.
-template <bool PAIR, int NQ>
+template <bool PAIR, int NQ, bool HIST = true, bool GH = true>
 __device__ __forceinline__ void MergeRows(unsigned long long *__restrict__ lds, RowQueue<NQ> &Q,
                                           const uint32_t (&xb)[NQ], float xg, float xh,
                                           unsigned long long xm, bool built,
@@ -734,15 +737,15 @@ __device__ __forceinline__ void MergeRows(unsigned long long *__restrict__ lds, 
   uint32_t vb[NQ];
 #pragma unroll
   for (int q = 0; q < NQ; ++q) vb[q] = (uint32_t)__shfl((int)xb[q], src);
-  const float vg = __shfl(xg, src);
-  const float vh = PAIR ? __shfl(xh, src) : 0.0f;
+  const float vg = GH ? __shfl(xg, src) : 0.0f;
+  const float vh = GH && PAIR ? __shfl(xh, src) : 0.0f;
   if (Q.n + nx >= 64u) {  // wave-uniform: the batch is complete
     const bool fill = (unsigned)lane >= Q.n;
 #pragma unroll
     for (int q = 0; q < NQ; ++q) Q.b[q] = fill ? vb[q] : Q.b[q];
     Q.g = fill ? vg : Q.g;
     Q.h = fill ? vh : Q.h;
-    EmitRows<PAIR, NQ>(lds, Q, Q.skip, 64u, built, bins_out, stride, g_out, h_out, lane, sg, sh, F);
+    EmitRows<PAIR, NQ, HIST, GH>(lds, Q, Q.skip, 64u, built, bins_out, stride, g_out, h_out, lane, sg, sh, F);
     Q.base += 64u;
     Q.skip = 0u;
 #pragma unroll
@@ -933,11 +936,13 @@ k_part_hist(const uint32_t *__restrict__ bins, uint32_t *__restrict__ bins_out, 
   FlushSlab<PAIR, NQ>(lds, slab, w, slab_entries, 0);
 }
 
-// Stable partition alone (matrices too wide for the fused pass): any number
-// of quads, moved eight at a time.
-template <bool PAIR>
+// Stable partition alone (matrices too wide for the fused pass, 16-bit bins):
+// words [q0, q0 + NQ) of every row, and with GH the gradients, go to the
+// children order through the two register queues of the fused pass.  One launch
+// per group of words; every launch reads the word of the split feature again.
+template <bool PAIR, int NQ, bool GH>
 __global__ void __launch_bounds__(kHistThreads)
-k_partition(const uint32_t *__restrict__ bins, uint32_t *__restrict__ bins_out, size_t stride, int Q,
+k_part_rows(const uint32_t *__restrict__ bins, uint32_t *__restrict__ bins_out, size_t stride, int q0,
             const float *__restrict__ g, float *__restrict__ g_out, const float *__restrict__ h,
             float *__restrict__ h_out, const SplitRec *__restrict__ split,
             const unsigned *__restrict__ seg_start, const WorkItem *__restrict__ work,
@@ -949,33 +954,59 @@ k_partition(const uint32_t *__restrict__ bins, uint32_t *__restrict__ bins_out, 
   const WorkItem it = work[w];
   const SplitRec s = split[it.node];
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const unsigned wb = it.begin + wave * kChunkRows, we = it.end;
   unsigned lo, ro;
   const unsigned before = LeftsBefore(it, w, wave, wave_left, item_left, s_tmp);
   WaveOffsets(it, s, seg_start[it.node], before, wave, &lo, &ro);
-  const unsigned long long below = (1ull << lane) - 1ull;
-  for (unsigned chunk = it.begin + wave * kChunkRows; chunk < it.end; chunk += kChunkStep)
-  for (unsigned base = chunk; base < min(chunk + kChunkRows, it.end); base += 64) {
-    const unsigned r = base + lane;
-    const bool valid = r < it.end;
-    const bool right = valid && GoesRight(bins, stride, s, r, code);
-    const unsigned long long lm = __ballot(valid && !right), rm = __ballot(right);
-    if (valid) {
-      const unsigned d = right ? ro + (unsigned)__popcll(rm & below) : lo + (unsigned)__popcll(lm & below);
-      for (int q0 = 0; q0 < Q; q0 += 8) {
-        uint32_t v[8];
+  if (wb >= we) return;
+  const uint32_t *group = bins + (size_t)q0 * stride;
+  uint32_t *group_out = bins_out + (size_t)q0 * stride;
+  const uint32_t *split_col = bins + (size_t)(s.fid < 0 ? 0 : code.Word(s.fid)) * stride;
+  RowQueue<NQ> QL, QR;
+  QL.Init(lo);
+  QR.Init(ro);
+  struct Rows {
+    RowSet<NQ> r;
+    uint32_t s0, s1;  // word of the split feature
+  };
+  auto load = [&](Rows &R, unsigned base) {
+    const unsigned a0 = min(base + lane, we - 1), a1 = min(base + 64 + lane, we - 1);
 #pragma unroll
-        for (int k = 0; k < 8; ++k)
-          if (q0 + k < Q) v[k] = bins[(size_t)(q0 + k) * stride + r];
-#pragma unroll
-        for (int k = 0; k < 8; ++k)
-          if (q0 + k < Q) bins_out[(size_t)(q0 + k) * stride + d] = v[k];
-      }
-      g_out[d] = g[r];
-      if (PAIR) h_out[d] = h[r];
+    for (int q = 0; q < NQ; ++q) {
+      R.r.b0[q] = __builtin_nontemporal_load(&group[(size_t)q * stride + a0]);
+      R.r.b1[q] = __builtin_nontemporal_load(&group[(size_t)q * stride + a1]);
     }
-    lo += (unsigned)__popcll(lm);
-    ro += (unsigned)__popcll(rm);
+    R.s0 = split_col[a0];
+    R.s1 = split_col[a1];
+    R.r.g0 = GH ? __builtin_nontemporal_load(&g[a0]) : 0.0f;
+    R.r.g1 = GH ? __builtin_nontemporal_load(&g[a1]) : 0.0f;
+    R.r.h0 = GH && PAIR ? __builtin_nontemporal_load(&h[a0]) : 0.0f;
+    R.r.h1 = GH && PAIR ? __builtin_nontemporal_load(&h[a1]) : 0.0f;
+  };
+  auto process = [&](const Rows &R, unsigned base) {
+    const unsigned r0 = base + lane, r1 = r0 + 64;
+    const bool v0 = r0 < we, v1 = r1 < we;
+    const bool right0 = v0 && s.fid >= 0 && (int)code.Bin(R.s0, s.fid) > s.bin;
+    const bool right1 = v1 && s.fid >= 0 && (int)code.Bin(R.s1, s.fid) > s.bin;
+    const unsigned long long lm0 = __ballot(v0 && !right0), rm0 = __ballot(right0);
+    const unsigned long long lm1 = __ballot(v1 && !right1), rm1 = __ballot(right1);
+    MergeRows<PAIR, NQ, false, GH>(nullptr, QL, R.r.b0, R.r.g0, R.r.h0, lm0, false, group_out, stride, g_out, h_out, lane, 0, 0, 0);
+    MergeRows<PAIR, NQ, false, GH>(nullptr, QR, R.r.b0, R.r.g0, R.r.h0, rm0, false, group_out, stride, g_out, h_out, lane, 0, 0, 0);
+    MergeRows<PAIR, NQ, false, GH>(nullptr, QL, R.r.b1, R.r.g1, R.r.h1, lm1, false, group_out, stride, g_out, h_out, lane, 0, 0, 0);
+    MergeRows<PAIR, NQ, false, GH>(nullptr, QR, R.r.b1, R.r.g1, R.r.h1, rm1, false, group_out, stride, g_out, h_out, lane, 0, 0, 0);
+  };
+  Rows A, B;
+  load(A, wb);
+  for (unsigned base = wb;; base += 2 * kChunkStep) {
+    load(B, base + kChunkStep);
+    process(A, base);
+    if (base + kChunkStep >= we) break;  // wave-uniform
+    load(A, base + 2 * kChunkStep);
+    process(B, base + kChunkStep);
+    if (base + 2 * kChunkStep >= we) break;
   }
+  EmitRows<PAIR, NQ, false, GH>(nullptr, QL, QL.skip, QL.n, false, group_out, stride, g_out, h_out, lane, 0, 0, 0);
+  EmitRows<PAIR, NQ, false, GH>(nullptr, QR, QR.skip, QR.n, false, group_out, stride, g_out, h_out, lane, 0, 0, 0);
 }
 
 // Adds the slabs of every directly built node of a level (on top of the stored
@@ -2312,14 +2343,7 @@ class HipTreeBuilder : public TreeBuilder {
           Mark(kPartition);
           hipLaunchKernelGGL(k_part_count, dim3(grid), dim3(kHistThreads), 0, stream_, src.bins, stride_, d_split_,
                              d_pwork_, d_nwork_ + 1, d_wave_left_, d_item_left_, code_);
-          if (pair_)
-            hipLaunchKernelGGL(k_partition<true>, dim3(grid), dim3(kHistThreads), 0, stream_, src.bins, dst.bins,
-                               stride_, Q_, src.g, dst.g, src.h, dst.h, d_split_, d_seg_[ps], d_pwork_,
-                               d_nwork_ + 1, d_wave_left_, d_item_left_, code_);
-          else
-            hipLaunchKernelGGL(k_partition<false>, dim3(grid), dim3(kHistThreads), 0, stream_, src.bins, dst.bins,
-                               stride_, Q_, src.g, dst.g, src.h, dst.h, d_split_, d_seg_[ps], d_pwork_,
-                               d_nwork_ + 1, d_wave_left_, d_item_left_, code_);
+          LaunchPartRows(grid, src, dst, ps);
           HistOfNodes(dst, state, L, trick_, trick_ ? n_ / 2 : n_, false);
           Reduce(L, hb, false, ps, trick_);
         }
@@ -2417,6 +2441,32 @@ class HipTreeBuilder : public TreeBuilder {
       hipLaunchKernelGGL(k_split_select, dim3((L + 127) / 128), dim3(128), 0, stream_, d_cand_, F_, L,
                          d_tot_[state], d_seg_[state], d_tot_[state ^ 1], d_seg_[state ^ 1], d_split_,
                          d_tfid_, d_tbin_, d_tgain_, L - 1, active);
+    }
+  }
+
+  // Stand-alone partition: groups of up to eight words per launch; the first
+  // launch also moves the gradients.
+  void LaunchPartRows(unsigned grid, const RowBuffers &src, const RowBuffers &dst, int ps) {
+    for (int q0 = 0; q0 < Q_; q0 += 8) {
+      const int nq = std::min(8, Q_ - q0);
+#define ARB_PART(P, N, G)                                                                                        \
+  hipLaunchKernelGGL((k_part_rows<P, N, G>), dim3(grid), dim3(kHistThreads), 0, stream_, src.bins, dst.bins,    \
+                     stride_, q0, src.g, dst.g, src.h, dst.h, d_split_, d_seg_[ps], d_pwork_, d_nwork_ + 1,      \
+                     d_wave_left_, d_item_left_, code_)
+#define ARB_PART_N(N)                                          \
+  case N:                                                      \
+    if (q0 == 0) {                                             \
+      if (pair_) ARB_PART(true, N, true);                      \
+      else ARB_PART(false, N, true);                           \
+    } else {                                                   \
+      ARB_PART(false, N, false);                               \
+    }                                                          \
+    break;
+      switch (nq) {
+        ARB_PART_N(1) ARB_PART_N(2) ARB_PART_N(3) ARB_PART_N(4) ARB_PART_N(5) ARB_PART_N(6) ARB_PART_N(7) ARB_PART_N(8)
+      }
+#undef ARB_PART_N
+#undef ARB_PART
     }
   }
 
