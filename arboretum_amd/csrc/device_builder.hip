@@ -437,10 +437,11 @@ __device__ __forceinline__ void AccumulateRow(unsigned long long *__restrict__ l
         const unsigned bi = ((unsigned)t + i) & 3u;  // byte of the quad
         const unsigned bin = (sel >> (8u * bi)) & 255u;
         const unsigned f16 = 4u * qi + bi;
+        // Quads past NQ do not exist.  Padding features of the last quad of
+        // the matrix (bin 0 in every row) are accumulated like real ones into
+        // slots nobody reads: cheaper than a per-update test.
         bool on = true;
-        if (4 * k + 3 >= NQ) on = 4u * k + qi < (unsigned)NQ;  // block with missing quads
-        // only the last quad of the matrix can hold padding features
-        if (4 * k + 3 >= NQ - 1) on = on && (int)((q_first + 4 * k) * 4 + f16) < F;
+        if (4 * k + 3 >= NQ) on = 4u * k + qi < (unsigned)NQ;
         if (on) {
           const unsigned idx = (unsigned)(k * kBlockEntries) + bin * kBlockFeatures + f16;
           atomicAdd(&lds[idx], w0);
