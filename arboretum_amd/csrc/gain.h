@@ -48,9 +48,13 @@ ARB_HD int FixShiftFromMax(float vmax) {
 }
 
 ARB_HD long long ToFixed(float v, int shift) {
-  double s = ldexp((double)v, shift);
-  if (!(fabs(s) <= 1073741824.0)) return 0;  // NaN, Inf or out of range
-  return (long long)(int)rint(s);  // |s| <= 2^30 fits 32 bits
+  // Scaling by a power of two is exact in fp32, and so is rounding the result
+  // to an integer (at or above 2^23 it is one already): the value is
+  // rint(v * 2^shift) of the real numbers, with no double arithmetic.  A
+  // result below the normal range rounds to 0 either way.
+  const float s = ldexpf(v, shift);
+  if (!(fabsf(s) <= 1073741824.0f)) return 0;  // NaN, Inf or out of range
+  return (long long)(int)rintf(s);  // |s| <= 2^30 fits 32 bits
 }
 
 // Integer sum -> value in the sum type (float results are float-representable).
