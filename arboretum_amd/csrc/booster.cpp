@@ -137,6 +137,7 @@ void Garden::GrowTree(DataMatrix *data, const float *grad) {
 
 void Garden::Predict(const DataMatrix *data, std::vector<float> *out, int n_rounds) const {
   const size_t K = cfg.tree.labels_count;
+  SyncTrees();
   std::vector<float> tmp(data->rows * K, IntoInternal(cfg.tree.initial_y));
   const long long use = std::min<long long>(n_rounds, (long long)trees_.size());
   for (long long t = 0; t < use; ++t) trees_[t].Predict(*data, tmp.data());
@@ -147,6 +148,7 @@ void Garden::UpdateByLastTree(DataMatrix *data) {
   const size_t K = cfg.tree.labels_count;
   if (data->y_hat.empty()) data->y_hat.assign(data->rows * K, IntoInternal(cfg.tree.initial_y));
   if (trees_.size() < K) return;
+  SyncTrees();
   for (size_t t = trees_.size() - K; t < trees_.size(); ++t) trees_[t].Predict(*data, data->y_hat.data());
 }
 
@@ -160,6 +162,7 @@ const char *Garden::GetModel() {
   Value root = Value::MakeObject();
   root["configuration"] = cfg.ToJson();
   Value model = Value::MakeArray();
+  SyncTrees();
   for (const RegTree &t : trees_) {
     Value jt = Value::MakeObject();
     Value nodes = Value::MakeArray();
@@ -222,6 +225,7 @@ void Garden::Restore(const char *json_model) {
     }
     loaded.push_back(std::move(t));
   }
+  SyncTrees();
   for (RegTree &t : loaded) trees_.push_back(std::move(t));
 }
 

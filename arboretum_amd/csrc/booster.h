@@ -97,7 +97,10 @@ class TreeBuilder {
  public:
   virtual ~TreeBuilder() {}
   // One boosting round: gradients, labels_count trees, prediction update.
+  // The trees are appended to `trees` at once, but their contents may stay on
+  // the device until FlushTrees() is called.
   virtual void GrowRound(std::vector<RegTree> *trees) = 0;
+  virtual void FlushTrees() = 0;
   // Inspection (tests, benchmark).
   virtual void SetInspect(bool on) = 0;
   virtual void GetLeaves(uint32_t *out) = 0;               // leaf of every row, last tree
@@ -152,12 +155,17 @@ class Garden {
 
   TreeBuilder *builder() { return builder_.get(); }
   size_t num_trees() const { return trees_.size(); }
-  const RegTree &tree(size_t i) const { return trees_[i]; }
+  const RegTree &tree(size_t i) const {
+    SyncTrees();
+    return trees_[i];
+  }
 
  private:
   std::unique_ptr<TreeBuilder> builder_;
   DataMatrix *bound_ = nullptr;
-  std::vector<RegTree> trees_;
+  // Records of freshly grown trees are fetched from the GPU on first use.
+  void SyncTrees() const { if (builder_) builder_->FlushTrees(); }
+  mutable std::vector<RegTree> trees_;
   std::string model_;
   bool inspect_ = false, timing_ = false;
 };

@@ -1602,6 +1602,22 @@ k_final_hist(const uint32_t *__restrict__ bins, size_t stride, int F, const int 
   FlushSlab<true, NQ>(lds, slab, w, slab_entries, 0);
 }
 
+// Tree record of the tree just grown into one slot of the record ring:
+// fid[internal], bin[internal], gain[internal], weights[leaves], overflow flag.
+__global__ void k_pack_record(const int *__restrict__ t_fid, const int *__restrict__ t_bin,
+                              const float *__restrict__ t_gain, const float *__restrict__ weights,
+                              const unsigned *__restrict__ overflow, int internal, int leaves,
+                              uint32_t *__restrict__ out) {
+  const int i = blockIdx.x * blockDim.x + threadIdx.x;
+  if (i < internal) {
+    out[i] = (uint32_t)t_fid[i];
+    out[internal + i] = (uint32_t)t_bin[i];
+    out[2 * internal + i] = __float_as_uint(t_gain[i]);
+  }
+  if (i < leaves) out[3 * internal + i] = __float_as_uint(weights[i]);
+  if (i == 0) out[3 * internal + leaves] = *overflow;
+}
+
 __global__ void k_fill_f32(float *p, float v, size_t n) {
   for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < n;
        i += (size_t)gridDim.x * blockDim.x)
@@ -2060,6 +2076,7 @@ class HipTreeBuilder : public TreeBuilder {
     d_item_left_ = DevAlloc<unsigned>(max_part_items_);
     d_slab_ = DevAlloc<unsigned long long>((size_t)std::max(max_hist_items_, max_part_items_) * slab_entries_ * (pair_ ? 2 : 1));
     d_shifts_ = DevAlloc<int>(2);
+    d_records_ = DevAlloc<uint32_t>(kRecordRing * RecordWords());
     d_gmax_ = DevAlloc<unsigned>(1);
     d_rows_scanned_ = DevAlloc<unsigned long long>(1);
     d_overflow_ = DevAlloc<unsigned>(1);
@@ -2084,7 +2101,7 @@ class HipTreeBuilder : public TreeBuilder {
     (void)hipStreamSynchronize(stream_);
     void *ptrs[] = {d_y_, d_labels_, d_yhat_, d_g_, d_h_, d_leaf_, d_split_, d_cand_, d_node_first_,
                     d_node_items_, d_hwork_, d_pwork_, d_nwork_, d_wave_left_, d_item_left_, d_slab_,
-                    d_shifts_, d_gmax_, d_rows_scanned_, d_tfid_, d_tbin_, d_tgain_, d_weights_, d_active_, d_overflow_};
+                    d_shifts_, d_gmax_, d_rows_scanned_, d_tfid_, d_tbin_, d_tgain_, d_weights_, d_active_, d_overflow_, d_records_};
     for (void *p : ptrs)
       if (p) (void)hipFree(p);
     for (int b = 0; b < 2; ++b) {
@@ -2125,12 +2142,46 @@ class HipTreeBuilder : public TreeBuilder {
       hipLaunchKernelGGL(k_set_shift, dim3(1), dim3(64), 0, stream_, d_gmax_, d_shifts_);
     grad_ready_ = false;
     Mark(kNone);
+    owner_ = trees;
     for (int k = 0; k < K_; ++k) {
-      RegTree tree((unsigned)D_, (unsigned)k);
-      GrowOne(k, &tree);
-      trees->push_back(std::move(tree));
+      // the record stays on the device until somebody needs it: no host
+      // synchronisation between trees
+      trees->emplace_back((unsigned)D_, (unsigned)k);
+      GrowOne(k);
+      pending_.push_back(trees->size() - 1);
+      if (inspect_ || pending_.size() == kRecordRing) FlushTrees();
     }
-    ResolveTimings();
+    // phase times are read back lazily as well (GetTimings), or when many events are waiting
+    if (!timing_ || marks_.size() > 8192) ResolveTimings();
+  }
+
+  // Copies the records of the trees grown since the last call to the host and
+  // completes their RegTree entries (garden.cu:447-503).
+  void FlushTrees() override {
+    if (pending_.empty()) return;
+    const int internal = (1 << (D_ - 1)) - 1, leaves = 1 << (D_ - 1);
+    const size_t words = RecordWords();
+    std::vector<uint32_t> rec(words * pending_.size());
+    HIP_OK(hipStreamSynchronize(stream_));
+    HIP_OK(hipMemcpy(rec.data(), d_records_, rec.size() * sizeof(uint32_t), hipMemcpyDeviceToHost));
+    bool overflow = false;
+    for (size_t k = 0; k < pending_.size(); ++k) {
+      RegTree &tree = (*owner_)[pending_[k]];
+      const uint32_t *r = rec.data() + k * words;
+      for (int i = 0; i < internal; ++i) {
+        const int fid = (int)r[i], bin = (int)r[internal + i];
+        tree.fid[i] = (unsigned)fid;
+        tree.quantized[i] = bin;
+        std::memcpy(&tree.gain[i], &r[2 * internal + i], sizeof(float));
+        float thr = std::numeric_limits<float>::infinity();
+        if (bin >= 0 && bin < (int)data_->thresholds[fid].size()) thr = data_->thresholds[fid][bin];
+        tree.threshold[i] = thr;
+      }
+      std::memcpy(tree.weights.data(), r + 3 * internal, (size_t)leaves * sizeof(float));
+      overflow = overflow || r[3 * internal + leaves] != 0;
+    }
+    pending_.clear();
+    if (overflow) throw std::runtime_error("internal: work plan exceeded its launch bound");
   }
 
   void SetInspect(bool on) override { inspect_ = on; }
@@ -2168,15 +2219,24 @@ class HipTreeBuilder : public TreeBuilder {
     *sg = s[0];
     *sh = s[1];
   }
-  void EnableTiming(bool on) override { timing_ = on; }
-  BuilderTimings GetTimings() override { return timings_; }
+  void EnableTiming(bool on) override {
+    ResolveTimings();
+    timing_ = on;
+  }
+  BuilderTimings GetTimings() override {
+    ResolveTimings();
+    return timings_;
+  }
   unsigned long long RowsScanned() override {
     unsigned long long v = 0;
     HIP_OK(hipStreamSynchronize(stream_));
     HIP_OK(hipMemcpy(&v, d_rows_scanned_, sizeof(v), hipMemcpyDeviceToHost));
     return v;
   }
-  void Synchronize() override { HIP_OK(hipStreamSynchronize(stream_)); }
+  void Synchronize() override {
+    HIP_OK(hipStreamSynchronize(stream_));
+    FlushTrees();
+  }
 
  private:
   enum Phase { kNone = -1, kGrad = 0, kHistRoot, kHistDeep, kReduce, kSplit, kPartition, kLeaf, kPlan, kFusedLast, kPhases };
@@ -2286,7 +2346,7 @@ class HipTreeBuilder : public TreeBuilder {
                          wide_ ? 1 : 0);
   }
 
-  void GrowOne(int label, RegTree *tree) {
+  void GrowOne(int label) {
     const GainParams gp = cfg_.gain_params();
     RowBuffers orig;
     orig.bins = dm_->bins;
@@ -2295,7 +2355,7 @@ class HipTreeBuilder : public TreeBuilder {
     if (inspect_) kept_hist_.assign(D_ - 1, {});
     SampleColumns();
     if (streamed_) {
-      GrowOneStreamed(label, tree, orig, gp);
+      GrowOneStreamed(label, orig, gp);
       return;
     }
 
@@ -2377,31 +2437,17 @@ class HipTreeBuilder : public TreeBuilder {
       }
       grad_ready_ = next_grad;
     }
-    FetchTree(tree);
+    EnqueueRecord();
   }
 
-  // Tree record to the host (garden.cu:447-503): node arrays and leaf weights.
-  void FetchTree(RegTree *tree) {
+  // Tree record into the next slot of the device ring; FlushTrees reads it.
+  size_t RecordWords() const { return (size_t)3 * ((1 << (D_ - 1)) - 1) + (size_t)(1 << (D_ - 1)) + 1; }
+  void EnqueueRecord() {
     Mark(kNone);
+    const int internal = (1 << (D_ - 1)) - 1, leaves = 1 << (D_ - 1);
+    hipLaunchKernelGGL(k_pack_record, dim3((leaves + 255) / 256), dim3(256), 0, stream_, d_tfid_, d_tbin_, d_tgain_,
+                       d_weights_, d_overflow_, internal, leaves, d_records_ + pending_.size() * RecordWords());
     HIP_OK(hipGetLastError());
-    const int internal = (1 << (D_ - 1)) - 1;
-    std::vector<int> fid(internal), bin(internal);
-    HIP_OK(hipMemcpyAsync(fid.data(), d_tfid_, internal * sizeof(int), hipMemcpyDeviceToHost, stream_));
-    HIP_OK(hipMemcpyAsync(bin.data(), d_tbin_, internal * sizeof(int), hipMemcpyDeviceToHost, stream_));
-    HIP_OK(hipMemcpyAsync(tree->gain.data(), d_tgain_, internal * sizeof(float), hipMemcpyDeviceToHost, stream_));
-    HIP_OK(hipMemcpyAsync(tree->weights.data(), d_weights_, tree->weights.size() * sizeof(float),
-                          hipMemcpyDeviceToHost, stream_));
-    unsigned overflow = 0;
-    HIP_OK(hipMemcpyAsync(&overflow, d_overflow_, sizeof(unsigned), hipMemcpyDeviceToHost, stream_));
-    HIP_OK(hipStreamSynchronize(stream_));
-    if (overflow) throw std::runtime_error("internal: work plan exceeded its launch bound");
-    for (int i = 0; i < internal; ++i) {
-      tree->fid[i] = (unsigned)fid[i];
-      tree->quantized[i] = bin[i];
-      float thr = std::numeric_limits<float>::infinity();
-      if (bin[i] >= 0 && bin[i] < (int)data_->thresholds[fid[i]].size()) thr = data_->thresholds[fid[i]][bin[i]];
-      tree->threshold[i] = thr;
-    }
   }
 
   // ---- streamed matrices -------------------------------------------------
@@ -2540,7 +2586,7 @@ class HipTreeBuilder : public TreeBuilder {
   // One tree over a streamed matrix: every level copies every block in once
   // (double buffered against the kernels of the previous block), one more pass
   // assigns the leaves.
-  void GrowOneStreamed(int label, RegTree *tree, const RowBuffers &orig, const GainParams &gp) {
+  void GrowOneStreamed(int label, const RowBuffers &orig, const GainParams &gp) {
     const size_t br = dm_->block_rows;
     const size_t nblocks = dm_->host_blocks.size();
     hipLaunchKernelGGL(k_init_root, dim3(1), dim3(64), 0, stream_, d_tot_[0], d_seg_[0],
@@ -2609,7 +2655,7 @@ class HipTreeBuilder : public TreeBuilder {
       HIP_OK(hipEventRecord(ev_free_[buf], stream_));
     }
     grad_ready_ = next_grad;
-    FetchTree(tree);
+    EnqueueRecord();
   }
 
   // Column sampling of one tree (InitGrowingTree / InitTreeLevel,
@@ -2669,6 +2715,10 @@ class HipTreeBuilder : public TreeBuilder {
   int wide_group_ = 2;    // features per histogram launch with 16-bit bins
   BinCode code_ = BinCode{2, 8};
   bool root_hist_ready_ = false;  // the slabs hold the root histogram of the tree grown next
+  static constexpr size_t kRecordRing = 64;  // trees whose records may wait on the device
+  uint32_t *d_records_ = nullptr;
+  std::vector<size_t> pending_;              // indices into *owner_ of the trees not fetched yet
+  std::vector<RegTree> *owner_ = nullptr;
   bool pair_ = false, f64_ = false, trick_ = true, fused_ = false, inspect_ = false, timing_ = false;
   bool grad_ready_ = false;
   int quads_per_group_ = 1;
