@@ -1019,7 +1019,7 @@ k_part_rows(const uint32_t *__restrict__ bins, uint32_t *__restrict__ bins_out, 
 //               (node_items == 0xffffffff marks a derived node);
 //   by_parent = 1: slabs belong to work items of the parent (fused pass); the
 //               built child is the smaller one, ties -> left.
-template <bool PAIR>
+template <bool PAIR, int LANES>
 __global__ void __launch_bounds__(1024)
 k_hist_reduce(const unsigned long long *__restrict__ slab, int slab_entries, int nbin_total,
               const unsigned *__restrict__ node_first, const unsigned *__restrict__ node_items,
@@ -1028,9 +1028,13 @@ k_hist_reduce(const unsigned long long *__restrict__ slab, int slab_entries, int
               long long *__restrict__ hh, unsigned *__restrict__ hc,
               const long long *__restrict__ pg, const long long *__restrict__ ph,
               const unsigned *__restrict__ pc, int trick, int accumulate, int plain) {
-  __shared__ long long s_g[16][64];
-  __shared__ long long s_h[16][64];
-  __shared__ unsigned s_c[16][64];
+  // LANES threads share the slabs of one entry; a block covers 1024 / LANES
+  // consecutive entries (with 4 lanes: 16 bins x 16 features, so the
+  // feature-major output is written in runs of 16 bins)
+  constexpr int kEntries = 1024 / LANES;
+  __shared__ long long s_g[LANES][kEntries];
+  __shared__ long long s_h[LANES][kEntries];
+  __shared__ unsigned s_c[LANES][kEntries];
   const int nd = blockIdx.y;
   unsigned items, first;
   if (by_parent) {
@@ -1045,8 +1049,8 @@ k_hist_reduce(const unsigned long long *__restrict__ slab, int slab_entries, int
     first = node_first[nd];
     if (items == 0xffffffffu) return;  // derived from its sibling
   }
-  const int e = threadIdx.x & 63, lane = threadIdx.x >> 6;
-  const int entry = blockIdx.x * 64 + e;  // slab order
+  const int e = threadIdx.x % kEntries, lane = threadIdx.x / kEntries;
+  const int entry = blockIdx.x * kEntries + e;  // slab order
   // plain: the slabs are feature-major already (16-bit bins)
   const int f = (entry / kBlockEntries) * kBlockFeatures + (entry & (kBlockFeatures - 1));
   const int bin = (entry / kBlockFeatures) & (kSlots - 1);
@@ -1055,7 +1059,7 @@ k_hist_reduce(const unsigned long long *__restrict__ slab, int slab_entries, int
   long long ag = 0, ah = 0;
   unsigned ac = 0;
   if (live) {
-    for (unsigned s = lane; s < items; s += 16) {
+    for (unsigned s = lane; s < items; s += LANES) {
       const unsigned long long *p = slab + (size_t)(first + s) * slab_entries * (PAIR ? 2 : 1);
       const unsigned long long w0 = p[entry];
       const long long gq = ((long long)(w0 << (64 - kCountShift))) >> (64 - kCountShift);
@@ -1069,7 +1073,7 @@ k_hist_reduce(const unsigned long long *__restrict__ slab, int slab_entries, int
   s_c[lane][e] = ac;
   __syncthreads();
   if (lane == 0 && live) {
-    for (int k = 1; k < 16; ++k) {
+    for (int k = 1; k < LANES; ++k) {
       ag += s_g[k][e];
       ah += s_h[k][e];
       ac += s_c[k][e];
@@ -2333,17 +2337,23 @@ class HipTreeBuilder : public TreeBuilder {
 
   void Reduce(int L, int hb, bool by_parent, int parent_state, bool trick, bool accumulate = false) {
     Mark(kReduce);
-    dim3 grid((slab_entries_ + 63) / 64, L);
-    if (pair_)
-      hipLaunchKernelGGL(k_hist_reduce<true>, grid, dim3(1024), 0, stream_, d_slab_, slab_entries_, nbin_total_, d_node_first_,
-                         d_node_items_, by_parent ? 1 : 0, d_split_, d_tot_[parent_state], d_hg_[hb], d_hh_[hb],
-                         d_hc_[hb], d_hg_[hb ^ 1], d_hh_[hb ^ 1], d_hc_[hb ^ 1], trick ? 1 : 0, accumulate ? 1 : 0,
-                         wide_ ? 1 : 0);
-    else
-      hipLaunchKernelGGL(k_hist_reduce<false>, grid, dim3(1024), 0, stream_, d_slab_, slab_entries_, nbin_total_, d_node_first_,
-                         d_node_items_, by_parent ? 1 : 0, d_split_, d_tot_[parent_state], d_hg_[hb], d_hh_[hb],
-                         d_hc_[hb], d_hg_[hb ^ 1], d_hh_[hb ^ 1], d_hc_[hb ^ 1], trick ? 1 : 0, accumulate ? 1 : 0,
-                         wide_ ? 1 : 0);
+    // many nodes: few slabs per node and the output dominates -> longer output runs per block
+    const bool wide_blocks = L >= 32;
+    const int entries = wide_blocks ? 256 : 64;
+    dim3 grid((slab_entries_ + entries - 1) / entries, L);
+#define ARB_REDUCE(P, LN)                                                                                          \
+  hipLaunchKernelGGL((k_hist_reduce<P, LN>), grid, dim3(1024), 0, stream_, d_slab_, slab_entries_, nbin_total_,   \
+                     d_node_first_, d_node_items_, by_parent ? 1 : 0, d_split_, d_tot_[parent_state], d_hg_[hb], \
+                     d_hh_[hb], d_hc_[hb], d_hg_[hb ^ 1], d_hh_[hb ^ 1], d_hc_[hb ^ 1], trick ? 1 : 0,           \
+                     accumulate ? 1 : 0, wide_ ? 1 : 0)
+    if (pair_) {
+      if (wide_blocks) ARB_REDUCE(true, 4);
+      else ARB_REDUCE(true, 16);
+    } else {
+      if (wide_blocks) ARB_REDUCE(false, 4);
+      else ARB_REDUCE(false, 16);
+    }
+#undef ARB_REDUCE
   }
 
   void GrowOne(int label) {
