@@ -1370,7 +1370,9 @@ k_split_scan(const long long *__restrict__ hg, const long long *__restrict__ hh,
 // (higher gain, then lower feature id: hist_tree_grower.cu:59-60), children
 // totals and row ranges, node record.  A node without a candidate keeps every
 // row left.
-__device__ __forceinline__ void SelectNode(int nd, const Cand *__restrict__ cand, int F,
+// One wave per node: lane l looks at features l, l + 64, ...; the wave keeps
+// the candidate with the highest gain, ties to the lowest feature id.
+__device__ __forceinline__ void SelectNode(int nd, int lane, const Cand *__restrict__ cand, int F,
                                            const NodeSum *__restrict__ tot,
                                            const unsigned *__restrict__ seg_start,
                                            NodeSum *__restrict__ tot_next, unsigned *__restrict__ seg_next,
@@ -1378,23 +1380,51 @@ __device__ __forceinline__ void SelectNode(int nd, const Cand *__restrict__ cand
                                            int *__restrict__ t_bin, float *__restrict__ t_gain, int heap_off,
                                            const unsigned char *__restrict__ active) {
   const NodeSum t = tot[nd];
-  SplitRec rec;
-  rec.gain = 0.0f;
-  rec.fid = -1;
-  rec.bin = -1;
-  rec.pad = 0;
-  rec.left = t;
+  float gain = 0.0f;
+  int fid = -1, bin = -1;
+  long long lg = 0, lh = 0;
+  unsigned long long lc = 0;
   if (t.c != 0) {
-    for (int f = 0; f < F; ++f) {
+    for (int f = lane; f < F; f += 64) {
       if (active && !active[f]) continue;  // feature not sampled at this level
       const Cand c = cand[(size_t)nd * F + f];
-      if (c.bin >= 0 && (rec.fid < 0 || rec.gain < c.gain)) {
-        rec.gain = c.gain;
-        rec.fid = f;
-        rec.bin = c.bin;
-        rec.left = c.left;
+      if (c.bin >= 0 && (fid < 0 || gain < c.gain)) {
+        gain = c.gain;
+        fid = f;
+        bin = c.bin;
+        lg = c.left.g;
+        lh = c.left.h;
+        lc = c.left.c;
       }
     }
+  }
+  for (int off = 32; off > 0; off >>= 1) {
+    const float og = __shfl_down(gain, off);
+    const int of = __shfl_down(fid, off);
+    const int ob = __shfl_down(bin, off);
+    const long long olg = __shfl_down(lg, off);
+    const long long olh = __shfl_down(lh, off);
+    const unsigned long long olc = __shfl_down(lc, off);
+    if (of >= 0 && (fid < 0 || og > gain || (og == gain && of < fid))) {
+      gain = og;
+      fid = of;
+      bin = ob;
+      lg = olg;
+      lh = olh;
+      lc = olc;
+    }
+  }
+  if (lane != 0) return;
+  SplitRec rec;
+  rec.gain = fid < 0 ? 0.0f : gain;
+  rec.fid = fid;
+  rec.bin = fid < 0 ? -1 : bin;
+  rec.pad = 0;
+  rec.left = t;
+  if (fid >= 0) {
+    rec.left.g = lg;
+    rec.left.h = lh;
+    rec.left.c = lc;
   }
   split[nd] = rec;
   NodeSum r;
@@ -1411,16 +1441,17 @@ __device__ __forceinline__ void SelectNode(int nd, const Cand *__restrict__ cand
   t_gain[heap_off + nd] = rec.gain;
 }
 
-__global__ void k_split_select(const Cand *__restrict__ cand, int F, int L,
-                               const NodeSum *__restrict__ tot,
-                               const unsigned *__restrict__ seg_start,
-                               NodeSum *__restrict__ tot_next, unsigned *__restrict__ seg_next,
-                               SplitRec *__restrict__ split, int *__restrict__ t_fid,
-                               int *__restrict__ t_bin, float *__restrict__ t_gain, int heap_off,
-                               const unsigned char *__restrict__ active) {
-  const int nd = blockIdx.x * blockDim.x + threadIdx.x;
+// grid ceil(L / 16), 1024 threads: one wave per node
+__global__ void __launch_bounds__(1024)
+k_split_select(const Cand *__restrict__ cand, int F, int L, const NodeSum *__restrict__ tot,
+               const unsigned *__restrict__ seg_start, NodeSum *__restrict__ tot_next,
+               unsigned *__restrict__ seg_next, SplitRec *__restrict__ split, int *__restrict__ t_fid,
+               int *__restrict__ t_bin, float *__restrict__ t_gain, int heap_off,
+               const unsigned char *__restrict__ active) {
+  const int nd = blockIdx.x * 16 + (threadIdx.x >> 6);
   if (nd < L)
-    SelectNode(nd, cand, F, tot, seg_start, tot_next, seg_next, split, t_fid, t_bin, t_gain, heap_off, active);
+    SelectNode(nd, threadIdx.x & 63, cand, F, tot, seg_start, tot_next, seg_next, split, t_fid, t_bin, t_gain,
+               heap_off, active);
 }
 
 // k_split_select followed, in the same workgroup, by the work plan of the
@@ -1436,8 +1467,9 @@ k_select_plan(const Cand *__restrict__ cand, int F, int L, const NodeSum *__rest
               unsigned *__restrict__ node_first, unsigned *__restrict__ node_items,
               unsigned long long *__restrict__ rows_scanned, unsigned max_items,
               unsigned *__restrict__ overflow) {
-  for (int nd = threadIdx.x; nd < L; nd += 1024)
-    SelectNode(nd, cand, F, tot, seg_start, tot_next, seg_next, split, t_fid, t_bin, t_gain, heap_off, active);
+  for (int nd = threadIdx.x >> 6; nd < L; nd += 16)
+    SelectNode(nd, threadIdx.x & 63, cand, F, tot, seg_start, tot_next, seg_next, split, t_fid, t_bin, t_gain,
+               heap_off, active);
   __syncthreads();  // the splits written above are read by the plan
   PlanBody(tot, seg_start, L, 0, rows_per_item, work, n_work, node_first, node_items, rows_scanned, split,
            max_items, overflow);
@@ -2495,7 +2527,7 @@ class HipTreeBuilder : public TreeBuilder {
                          L - 1, active, per_item, d_pwork_, d_nwork_ + 1, d_node_first_, d_node_items_,
                          d_rows_scanned_, FusedGrid(L), d_overflow_);
     } else {
-      hipLaunchKernelGGL(k_split_select, dim3((L + 127) / 128), dim3(128), 0, stream_, d_cand_, F_, L,
+      hipLaunchKernelGGL(k_split_select, dim3((L + 15) / 16), dim3(1024), 0, stream_, d_cand_, F_, L,
                          d_tot_[state], d_seg_[state], d_tot_[state ^ 1], d_seg_[state ^ 1], d_split_,
                          d_tfid_, d_tbin_, d_tgain_, L - 1, active);
     }
