@@ -675,6 +675,7 @@ __device__ __forceinline__ int SelectBit(unsigned long long m, unsigned k) {
 template <int NQ>
 struct RowSet {
   uint32_t b0[NQ], b1[NQ];
+  uint32_t s0, s1;  // word of the split feature when it is not among b0/b1
   float g0, g1, h0, h1;
 };
 
@@ -711,7 +712,7 @@ __device__ __forceinline__ void EmitRows(unsigned long long *__restrict__ lds, c
     const unsigned d = Q.base + (unsigned)lane;
 #pragma unroll
     for (int q = 0; q < NQ; ++q) __builtin_nontemporal_store(Q.b[q], &bins_out[(size_t)q * stride + d]);
-    if (GH) {
+    if (GH && g_out != nullptr) {  // a group pass after the first leaves the gradients alone
       __builtin_nontemporal_store(Q.g, &g_out[d]);
       if (PAIR) __builtin_nontemporal_store(Q.h, &h_out[d]);
     }
@@ -776,7 +777,11 @@ __device__ __forceinline__ void MergeRows(unsigned long long *__restrict__ lds, 
 // the copy itself.  On the last level only the quad of the split feature is
 // read for every row; the selected rows are queued by row id and read 64 at a
 // time.  NQ = all quads of the matrix.
-template <bool PAIR, int NQ, bool WRITE>
+// GROUP: `bins` / `bins_out` point at quad q0 of a wider matrix (q0 a multiple
+// of 4); the quad of the split feature is read from `split_bins`, the start of
+// the whole matrix, and g_out may be null (the gradients moved with an
+// earlier group of the same level).
+template <bool PAIR, int NQ, bool WRITE, bool GROUP = false>
 __global__ void __launch_bounds__(kHistThreads)
 k_part_hist(const uint32_t *__restrict__ bins, uint32_t *__restrict__ bins_out, size_t stride, int F,
             const float *__restrict__ g, float *__restrict__ g_out, const float *__restrict__ h,
@@ -785,7 +790,7 @@ k_part_hist(const uint32_t *__restrict__ bins, uint32_t *__restrict__ bins_out, 
             const unsigned *__restrict__ seg_start, const WorkItem *__restrict__ work,
             const unsigned *__restrict__ n_work, const unsigned *__restrict__ wave_left,
             const unsigned *__restrict__ item_left, unsigned long long *__restrict__ slab,
-            int slab_entries) {
+            int slab_entries, const uint32_t *__restrict__ split_bins, int q0) {
   extern __shared__ unsigned long long lds[];
   __shared__ unsigned s_tmp[kItemWaves + 1];
   const unsigned w = blockIdx.x;
@@ -815,12 +820,17 @@ k_part_hist(const uint32_t *__restrict__ bins, uint32_t *__restrict__ bins_out, 
     // in flight.  The loads are unconditional (addresses clamped to the last
     // row of the item) and the sets are never copied, so every wait in the loop
     // is for exactly the set that is needed next.
+    const uint32_t *split_col = split_bins + (size_t)(s.fid < 0 ? 0 : fq) * stride;
     auto load = [&](RowSet<NQ> &R, unsigned base) {
       const unsigned a0 = min(base + lane, we - 1), a1 = min(base + 64 + lane, we - 1);
 #pragma unroll
       for (int q = 0; q < NQ; ++q) {
         R.b0[q] = __builtin_nontemporal_load(&bins[(size_t)q * stride + a0]);
         R.b1[q] = __builtin_nontemporal_load(&bins[(size_t)q * stride + a1]);
+      }
+      if (GROUP) {  // the quad of the split feature, wherever it lives
+        R.s0 = split_col[a0];
+        R.s1 = split_col[a1];
       }
       R.g0 = __builtin_nontemporal_load(&g[a0]);
       R.g1 = __builtin_nontemporal_load(&g[a1]);
@@ -831,10 +841,15 @@ k_part_hist(const uint32_t *__restrict__ bins, uint32_t *__restrict__ bins_out, 
       const unsigned r0 = base + lane, r1 = r0 + 64;
       const bool v0 = r0 < we, v1 = r1 < we;
       uint32_t s0 = 0, s1 = 0;
+      if (GROUP) {
+        s0 = R.s0;
+        s1 = R.s1;
+      } else {
 #pragma unroll
-      for (int q = 0; q < NQ; ++q) {
-        s0 = q == fq ? R.b0[q] : s0;
-        s1 = q == fq ? R.b1[q] : s1;
+        for (int q = 0; q < NQ; ++q) {
+          s0 = q == fq ? R.b0[q] : s0;
+          s1 = q == fq ? R.b1[q] : s1;
+        }
       }
       const bool right0 = v0 && s.fid >= 0 && (int)((s0 >> fs) & 255u) > s.bin;
       const bool right1 = v1 && s.fid >= 0 && (int)((s1 >> fs) & 255u) > s.bin;
@@ -906,7 +921,7 @@ k_part_hist(const uint32_t *__restrict__ bins, uint32_t *__restrict__ bins_out, 
     if (wb < we) {
       // last level: only the quad of the split feature decides; the selected
       // rows are read when they are accumulated
-      const uint32_t *col = bins + (size_t)(s.fid < 0 ? 0 : fq) * stride;
+      const uint32_t *col = split_bins + (size_t)(s.fid < 0 ? 0 : fq) * stride;
       auto step = [&](uint32_t s0, uint32_t s1, uint32_t &n0, uint32_t &n1, unsigned base) {
         const bool full = np >= 64u;  // wave-uniform
         if (full) {
@@ -934,7 +949,7 @@ k_part_hist(const uint32_t *__restrict__ bins, uint32_t *__restrict__ bins_out, 
     }
     drain(0u);
   }
-  FlushSlab<PAIR, NQ>(lds, slab, w, slab_entries, 0);
+  FlushSlab<PAIR, NQ>(lds, slab, w, slab_entries, q0);
 }
 
 // Stable partition alone (matrices too wide for the fused pass, 16-bit bins):
@@ -1978,25 +1993,28 @@ struct FusedArgs {
   const unsigned *item_left;
   unsigned long long *slab;
   int slab_entries;
+  const uint32_t *split_bins;  // start of the whole matrix
+  int q0;                      // first quad of this launch
 };
 
-template <bool PAIR, int NQ, bool WRITE>
+template <bool PAIR, int NQ, bool WRITE, bool GROUP>
 void LaunchFusedNQ(hipStream_t st, unsigned grid, const FusedArgs &a) {
   const size_t lds = HistLdsBytes(NQ, PAIR);
   static bool configured = false;
   if (!configured) {
-    AllowLds(k_part_hist<PAIR, NQ, WRITE>, lds);
+    AllowLds(k_part_hist<PAIR, NQ, WRITE, GROUP>, lds);
     configured = true;
   }
-  hipLaunchKernelGGL((k_part_hist<PAIR, NQ, WRITE>), dim3(grid), dim3(kHistThreads), lds, st, a.bins, a.bins_out,
+  hipLaunchKernelGGL((k_part_hist<PAIR, NQ, WRITE, GROUP>), dim3(grid), dim3(kHistThreads), lds, st,
+                     a.bins + (size_t)a.q0 * a.stride, a.bins_out ? a.bins_out + (size_t)a.q0 * a.stride : nullptr,
                      a.stride, a.F, a.g, a.g_out, a.h, a.h_out, a.shifts, a.split, a.tot, a.seg_start, a.work,
-                     a.n_work, a.wave_left, a.item_left, a.slab, a.slab_entries);
+                     a.n_work, a.wave_left, a.item_left, a.slab, a.slab_entries, a.split_bins, a.q0);
 }
 
-template <bool PAIR, bool WRITE>
+template <bool PAIR, bool WRITE, bool GROUP>
 void LaunchFused(int nq, hipStream_t st, unsigned grid, const FusedArgs &a) {
 #define ARB_CASE(N) \
-  case N: LaunchFusedNQ<PAIR, N, WRITE>(st, grid, a); break;
+  case N: LaunchFusedNQ<PAIR, N, WRITE, GROUP>(st, grid, a); break;
   switch (nq) {
     ARB_CASE(1) ARB_CASE(2) ARB_CASE(3) ARB_CASE(4) ARB_CASE(5) ARB_CASE(6) ARB_CASE(7) ARB_CASE(8)
     default: throw std::runtime_error("internal: bad quad count");
@@ -2041,7 +2059,8 @@ class HipTreeBuilder : public TreeBuilder {
     quads_per_group_ = std::min(quads_per_group_, Q_);
     // the fused partition + histogram pass holds one histogram of all
     // features and builds only the smaller child
-    fused_ = trick_ && Q_ <= quads_per_group_ && !wide_;
+    fused_ = trick_ && !wide_;
+    single_group_ = Q_ <= quads_per_group_;
     if (wide_) {
       // features per histogram launch (an even number, two per word)
       const size_t per_feature = (size_t)slots_ * 8 * (pair_ ? 2 : 1);
@@ -2428,16 +2447,28 @@ class HipTreeBuilder : public TreeBuilder {
                                d_pwork_, d_nwork_ + 1, d_wave_left_, d_item_left_, code_);
           }
           Mark(last ? kFusedLast : kHistDeep);
-          FusedArgs a{src.bins, dst.bins, stride_, F_, src.g, dst.g, src.h, dst.h, d_shifts_, d_split_,
-                      d_tot_[ps], d_seg_[ps], d_pwork_, d_nwork_ + 1, d_wave_left_, d_item_left_, d_slab_, slab_entries_};
-          if (pair_) {
-            if (last) LaunchFused<true, false>(Q_, stream_, grid, a);
-            else LaunchFused<true, true>(Q_, stream_, grid, a);
-          } else {
-            if (last) LaunchFused<false, false>(Q_, stream_, grid, a);
-            else LaunchFused<false, true>(Q_, stream_, grid, a);
+          // matrices wider than one LDS histogram: one launch per group of
+          // quads; the first one moves the gradients
+          for (int q0 = 0; q0 < Q_; q0 += quads_per_group_) {
+            const int nq = std::min(quads_per_group_, Q_ - q0);
+            FusedArgs a{src.bins, last ? nullptr : dst.bins, stride_, F_, src.g, q0 == 0 ? dst.g : nullptr, src.h,
+                        q0 == 0 ? dst.h : nullptr, d_shifts_, d_split_, d_tot_[ps], d_seg_[ps], d_pwork_,
+                        d_nwork_ + 1, d_wave_left_, d_item_left_, d_slab_, slab_entries_, src.bins, q0};
+#define ARB_FUSED(P, W)                                        \
+  do {                                                         \
+    if (single_group_) LaunchFused<P, W, false>(nq, stream_, grid, a); \
+    else LaunchFused<P, W, true>(nq, stream_, grid, a);        \
+  } while (0)
+            if (pair_) {
+              if (last) ARB_FUSED(true, false);
+              else ARB_FUSED(true, true);
+            } else {
+              if (last) ARB_FUSED(false, false);
+              else ARB_FUSED(false, true);
+            }
+#undef ARB_FUSED
+            if (timing_) ++(last ? timings_.fused_last_launches : timings_.hist_deep_launches);
           }
-          if (timing_) ++(last ? timings_.fused_last_launches : timings_.hist_deep_launches);
           Reduce(L, hb, true, ps, true);
         } else {
           const unsigned grid = (unsigned)std::min<size_t>(n_ / kPartRows + PL + 1, max_part_items_);
@@ -2463,7 +2494,7 @@ class HipTreeBuilder : public TreeBuilder {
       if (cfg_.objective == kLinearRegression) HIP_OK(hipMemsetAsync(d_gmax_, 0, sizeof(unsigned), stream_));
       const int internal = (1 << (D_ - 1)) - 1;
       const size_t lds = HistLdsBytes(Q_, true) + (size_t)internal * 2 * sizeof(int);
-      if (next_grad && cfg_.objective == kLogisticRegression && Q_ <= quads_per_group_ && !wide_ &&
+      if (next_grad && cfg_.objective == kLogisticRegression && single_group_ && !wide_ &&
           lds <= kLdsBudget) {
         // plan of the next tree's root, then one pass: leaves, predictions,
         // gradients and the root histogram of the next tree
@@ -2752,6 +2783,7 @@ class HipTreeBuilder : public TreeBuilder {
   size_t n_ = 0, stride_ = 0;
   int F_ = 0, Q_ = 0, K_ = 1, D_ = 2, nbin_total_ = 0;
   int slab_entries_ = 0;  // histogram entries of one work item's slab (whole 16-feature blocks)
+  bool single_group_ = true;  // all quads fit one LDS histogram
   bool wide_ = false;     // 16-bit bins: two features per word, slots_ histogram slots per feature
   int slots_ = kSlots;
   int wide_group_ = 2;    // features per histogram launch with 16-bit bins
