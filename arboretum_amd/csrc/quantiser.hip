@@ -247,16 +247,25 @@ k_thr_emit(const unsigned *__restrict__ keys, size_t n, const unsigned *__restri
     const size_t i = wbase + j + lane;
     const bool border = i < n && IsBorder(keys, i);
     const unsigned long long m = __ballot(border);
+    const unsigned long long below = m & ((1ull << lane) - 1ull);
+    int slot = -3;
+    float mid = 0.0f;
     if (border) {
-      const unsigned k = run + (unsigned)__popcll(m & ((1ull << lane) - 1ull)) + 1u;  // inclusive count
+      const unsigned k = run + (unsigned)__popcll(below) + 1u;  // inclusive count
       const float a = ValueOf(keys[i]), b = ValueOf(keys[i - 1]);
-      const float mid = (float)((double)(float)(a + b) * 0.5);
+      mid = (float)((double)(float)(a + b) * 0.5);
       const unsigned long long pos_slot = (unsigned long long)(i / seg) + 1ull;
-      const long long slot = (long long)min((unsigned long long)k + 1ull, pos_slot) - 2;
-      if (mid == mid && slot >= 0 && slot < hist_size) {
-        const unsigned mk = KeyOf(mid);
-        if (mk < thr[slot]) atomicMin(&thr[slot], mk);
-      }
+      slot = (int)((long long)min((unsigned long long)k + 1ull, pos_slot) - 2);
+    }
+    // Slots and midpoints grow with the position (NaN midpoints come last), so
+    // the minimum of a slot is at its first change: only the first change of
+    // each slot within the wave goes to memory.
+    const int prev = below ? 63 - __clzll((long long)below) : lane;
+    const int prev_slot = __shfl(slot, prev);
+    const bool first = border && (below == 0ull || prev_slot != slot);
+    if (first && mid == mid && slot >= 0 && slot < hist_size) {
+      const unsigned mk = KeyOf(mid);
+      if (mk < thr[slot]) atomicMin(&thr[slot], mk);
     }
     run += (unsigned)__popcll(m);
   }
