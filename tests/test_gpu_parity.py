@@ -232,6 +232,35 @@ def test_training_many_features_uses_feature_groups(arb, oracle):
     assert_same_training(arb, oracle, X, y, cfg, rounds=2)
 
 
+@pytest.mark.parametrize("objective,F", [(0, 36), (1, 33), (0, 70)])
+def test_quad_groups_of_the_fused_pass(arb, oracle, objective, F):
+    # 33 and 36 features: a group of eight quads and a group of one; 70: three groups
+    X, y = make_data(20000, F, objective, seed=F, nan_frac=0.05)
+    cfg = {"objective": objective, "method": 1, "internals": {"hist_size": 100, "double_precision": True},
+           "tree": {"max_depth": 6, "eta": 0.3, "lambda": 1.0}}
+    assert_same_training(arb, oracle, X, y, cfg, rounds=2)
+
+
+def test_many_trees_without_reading_the_model(arb, oracle):
+    # tree records wait on the device (a ring of 64) until the model is read
+    X, y = make_data(3000, 6, 1, seed=64)
+    cfg = {"objective": 1, "method": 1, "internals": {"hist_size": 32, "double_precision": True},
+           "tree": {"max_depth": 3, "eta": 0.2, "lambda": 1.0}}
+    rounds = 150
+    ob = oracle.Booster(X, y=y, config=cfg)
+    ob.grow(rounds)
+    data = arb.DMatrix(X, y=y)
+    g = arb.Garden(cfg, data)
+    for _ in range(rounds):
+        g.grow_tree()
+    for r in range(rounds):
+        to, tg = ob.tree(r), g.tree(r)
+        for key in ("fid", "quantized", "threshold", "gain", "weights"):
+            assert np.array_equal(to[key], tg[key], equal_nan=True), "%s of tree %d" % (key, r)
+    assert np.array_equal(ob.yhat(), g.train_yhat())
+    assert np.allclose(ob.predict(X), g.predict(data), rtol=0, atol=1e-6)
+
+
 @pytest.mark.parametrize("n", [1, 2, 63, 64, 65, 1023, 1025, 4097])
 def test_ragged_row_counts(arb, oracle, n):
     X, y = make_data(n, 5, 0, seed=n)
