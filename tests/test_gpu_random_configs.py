@@ -23,11 +23,12 @@ def _draw(seed):
     n = int(rng.choice([37, 300, 2049, 9000, 33000, 70000]))
     F = int(rng.choice([1, 2, 3, 5, 8, 13, 28, 31, 33, 40]))
     depth = int(rng.integers(1, 8))
-    hist_size = int(rng.choice([2, 7, 16, 63, 64, 100, 255, 256]))
+    hist_size = int(rng.choice([2, 7, 16, 63, 64, 100, 255, 256, 300, 1000]))
     cfg = {"objective": objective, "method": 1,
            "internals": {"hist_size": hist_size, "double_precision": bool(rng.integers(0, 2)),
                          "use_hist_subtraction_trick": bool(rng.integers(0, 2)),
-                         "upload_features": bool(rng.random() < 0.75),
+                         # 16-bit bins (more than 256 ids per feature) are resident only
+                         "upload_features": bool(rng.random() < 0.75) or hist_size > 256,
                          "stream_block_rows": int(rng.choice([64, 1000, 5000, 1 << 20])),
                          "seed": int(rng.integers(0, 100))},
            "tree": {"max_depth": depth, "eta": float(rng.choice([0.1, 0.3, 1.0])),
@@ -43,7 +44,7 @@ def _draw(seed):
     return n, F, objective, cfg, nan_frac, inspect
 
 
-@pytest.mark.parametrize("seed", range(48))
+@pytest.mark.parametrize("seed", range(64))
 def test_random_configuration(arb, oracle, seed):
     n, F, objective, cfg, nan_frac, inspect = _draw(seed)
     columns = F
