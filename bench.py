@@ -205,7 +205,7 @@ def main():
     row_bytes = F + 8  # uint8 bins of all features + one (g, h) pair
     cell_bytes = 16    # one histogram cell as written by a workgroup (two 64-bit words)
     # Dominant kernel: the fused partition + histogram pass of levels 1..max_depth-2
-    # (k_part_hist<true, 7, true>).  Algorithmic bytes of one launch: every row is
+    # (k_part_hist<true, 7, true, false>).  Algorithmic bytes of one launch: every row is
     # read once and written once in the children order, and the smaller child of
     # each parent gets one histogram written.
     fl = max(tm["hist_deep_launches"], 1)
@@ -216,7 +216,7 @@ def main():
     # root level (k_hist<true, 7>): reads every row, writes one histogram
     root_bytes = tm["hist_root_rows"] * row_bytes + args.steps * F * 256 * cell_bytes
     root_s = tm["hist_root_ms"] * 1e-3
-    # last level (k_part_hist<true, 7, false>): reads every row, moves none
+    # last level (k_part_hist<true, 7, false, false>): reads every row, moves none
     last_bytes = tm["fused_last_launches"] * args.rows * row_bytes
     last_s = tm["fused_last_ms"] * 1e-3
 
@@ -230,7 +230,7 @@ def main():
     def frac(b, t):
         return (b / t) / HBM_PEAK if t > 0 else 0.0
 
-    other = {"k_part_hist<true,7,false> (last level)": {
+    other = {"k_part_hist<true,7,false,false> (last level)": {
         "frac_of_hbm": frac(last_bytes, last_s),
         "avg_launch_us": tm["fused_last_ms"] * 1e3 / max(tm["fused_last_launches"], 1)}}
     if tm["hist_root_launches"] > 0:
@@ -268,7 +268,7 @@ def main():
                    "rows": args.rows, "features": F, "bins": args.hist_size, "max_depth": args.max_depth},
         "roofline": {"bound": "hbm", "achieved": achieved / 1e9, "peak": HBM_PEAK / 1e9, "unit": "GB/s",
                      "frac": achieved / HBM_PEAK, "traffic": traffic,
-                     "kernel": "k_part_hist<true,7,true> (fused partition + histogram, levels 1..%d)"
+                     "kernel": "k_part_hist<true,7,true,false> (fused partition + histogram, levels 1..%d)"
                                % (args.max_depth - 2),
                      "launches": int(tm["hist_deep_launches"]),
                      "avg_launch_us": tm["hist_deep_ms"] * 1e3 / fl,
