@@ -262,6 +262,26 @@ def test_many_trees_without_reading_the_model(arb, oracle):
     assert np.allclose(ob.predict(X), g.predict(data), rtol=0, atol=1e-6)
 
 
+@pytest.mark.parametrize("depth,objective,trick,upload",
+                         [(11, 1, True, True), (12, 0, True, True), (12, 1, False, True), (13, 1, True, True),
+                          (11, 0, True, False)])
+def test_deep_trees(arb, oracle, depth, objective, trick, upload):
+    # up to 4096 nodes on the last level, most of them empty
+    X, y = make_data(120000, 9, objective, seed=depth, nan_frac=0.01)
+    cfg = {"objective": objective, "method": 1,
+           "internals": {"hist_size": 64, "double_precision": True, "use_hist_subtraction_trick": trick,
+                         "upload_features": upload, "stream_block_rows": 50000},
+           "tree": {"max_depth": depth, "eta": 0.3, "lambda": 1.0, "min_child_weight": 0.0, "min_leaf_size": 0}}
+    assert_same_training(arb, oracle, X, y, cfg, rounds=2, check_hist=(depth <= 11))
+
+
+def test_depth_limit_is_an_error(arb):
+    X, y = make_data(1000, 3, 0, seed=1)
+    cfg = {"objective": 0, "method": 1, "internals": {"hist_size": 16}, "tree": {"max_depth": 14}}
+    with pytest.raises(Exception, match="unsupported depth"):
+        arb.Garden(cfg, arb.DMatrix(X, y=y)).grow_tree()
+
+
 @pytest.mark.parametrize("n", [1, 2, 63, 64, 65, 1023, 1025, 4097])
 def test_ragged_row_counts(arb, oracle, n):
     X, y = make_data(n, 5, 0, seed=n)
