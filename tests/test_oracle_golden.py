@@ -240,3 +240,23 @@ def test_invariants_random(oracle, objective):
     tracked = b.yhat() if objective == 0 else 1 / (1 + np.exp(-b.yhat().astype(np.float64)))
     clean = ~np.isnan(X).any(axis=1)
     assert np.allclose(b.predict(X)[clean], tracked[clean], atol=1e-5)
+
+
+def test_baseline_config_0_on_the_oracle(oracle):
+    # The CPU-runnable benchmark configuration: 10,000 x 28 ~ N(0,1), y = X.w + 0.1 N(0,1), squared
+    # error, 256 bins, max_depth 6, eta 0.3, lambda 1, 10 trees.  The training error must fall with
+    # every tree, and predicting the training rows must reproduce the kept y_hat.
+    rng = np.random.default_rng(0)
+    X = rng.standard_normal(size=(10000, 28), dtype=np.float32)
+    w = rng.standard_normal(28)
+    y = (X @ w + 0.1 * rng.standard_normal(10000)).astype(np.float32)
+    cfg = {"objective": 0, "method": 1, "internals": {"hist_size": 256, "double_precision": True},
+           "tree": {"max_depth": 6, "eta": 0.3, "lambda": 1.0}}
+    ob = oracle.Booster(X, y=y, config=cfg)
+    errors = []
+    for _ in range(10):
+        ob.grow(1)
+        errors.append(float(np.mean((ob.yhat() - y) ** 2)))
+    assert all(b < a for a, b in zip(errors, errors[1:]))
+    assert errors[-1] < 0.25 * np.var(y)
+    assert np.allclose(ob.predict(X), ob.yhat(), atol=1e-5)
