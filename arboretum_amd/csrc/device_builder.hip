@@ -2420,8 +2420,10 @@ class HipTreeBuilder : public TreeBuilder {
       return;
     }
 
-    hipLaunchKernelGGL(k_init_root, dim3(1), dim3(64), 0, stream_, d_tot_[0], d_seg_[0],
-                       (unsigned long long)n_, (unsigned *)nullptr);
+    // (the last pass of the previous tree has done this when it built the root histogram)
+    if (!root_hist_ready_)
+      hipLaunchKernelGGL(k_init_root, dim3(1), dim3(64), 0, stream_, d_tot_[0], d_seg_[0],
+                         (unsigned long long)n_, (unsigned *)nullptr);
     int state = 0;  // d_tot_/d_seg_[state] describe the nodes of the current level
     for (int level = 0; level + 1 < D_; ++level) {
       const int L = 1 << level;
