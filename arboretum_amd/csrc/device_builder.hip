@@ -24,7 +24,8 @@
 // them feature-major, and derives the larger sibling as parent - smaller
 // child.  All sums are integers: the result does not depend on scheduling.
 //
-// What replaces what (reference file:line):
+// The kernels live in kernels_*.h (one header per stage), shared constants
+// and records in device_common.h.  What replaces what (reference file:line):
 //   k_bin_assign      build_histogram              src/io/io.cu:293-312
 //                     (thresholds: quantiser.hip)
 //   k_grad_*          update_grad                  src/core/objective.cu:15-56
@@ -55,1639 +56,18 @@
 #include <vector>
 
 #include "booster.h"
+#include "device_common.h"
 #include "gain.h"
+#include "kernels_final.h"
+#include "kernels_hist.h"
+#include "kernels_objective.h"
+#include "kernels_partition.h"
+#include "kernels_plan.h"
+#include "kernels_quantise.h"
+#include "kernels_split.h"
+#include "kernels_stream.h"
 
 namespace arb {
-namespace {
-
-#define HIP_OK(expr)                                                                        \
-  do {                                                                                      \
-    hipError_t e_ = (expr);                                                                 \
-    if (e_ != hipSuccess)                                                                   \
-      throw std::runtime_error(std::string("HIP error: ") + hipGetErrorString(e_) + " in " #expr); \
-  } while (0)
-
-constexpr int kSlots = 256;               // histogram slots per feature (uint8 bins)
-constexpr int kMaxWideSlots = 4096;       // histogram slots per feature with 16-bit bins (power of two)
-constexpr int kHistThreads = 1024;        // one workgroup per CU, 16 waves
-constexpr int kItemWaves = kHistThreads / 64;  // waves per work item in row passes
-constexpr unsigned kPartRows = 16384;     // rows per work item of the stand-alone partition
-constexpr int kMaxGroupQuads = 8;         // quads per histogram launch (compile-time variants, whole blocks)
-constexpr unsigned kMaxHistRows = 64512;  // rows per histogram work item (< 2^16)
-constexpr int kCountShift = 47;           // word0 = count << 47 | g
-constexpr int kMaxPlanNodes = 4096;       // nodes per level the planner handles
-constexpr size_t kLdsBudget = 160 * 1024;
-// LDS histograms are laid out in blocks of 16 features (4 quads):
-//   entry(f, bin) = (f / 16) * 4096 + bin * 16 + f % 16.
-// A 64-bit LDS atomic is executed 16 lanes per pass, and two of those lanes
-// collide when their addresses share a bank pair (entry % 16).  With this
-// layout the bank pair is the feature, and the kernels let the 16 lanes of a
-// pass work on 16 different features of their rows, so a pass never has a
-// bank conflict and never two lanes on one address, whatever the bin
-// distribution is (missing values, zeros, a dominant category).
-constexpr int kBlockFeatures = 16;
-constexpr int kBlockQuads = 4;
-constexpr int kBlockEntries = kBlockFeatures * kSlots;  // 4096
-constexpr int HistBlocks(int nq) { return (nq + kBlockQuads - 1) / kBlockQuads; }
-// LDS bytes of a histogram of nq quads
-constexpr size_t HistLdsBytes(int nq, bool pair) {
-  return (size_t)HistBlocks(nq) * kBlockEntries * 8 * (pair ? 2 : 1);
-}
-
-struct NodeSum {
-  long long g;
-  long long h;
-  unsigned long long c;
-};
-
-struct SplitRec {
-  float gain;
-  int fid;   // -1: not split (every row stays left)
-  int bin;
-  unsigned pad;
-  NodeSum left;
-};
-
-struct WorkItem {
-  unsigned node;
-  unsigned begin;  // row range in the current order
-  unsigned end;
-  unsigned first;  // index of the first work item of this node
-};
-
-// --------------------------------------------------------------- quantiser
-// bin(x) = first l in [0,size] with x <= v[l], v[t] = thr[t] for t < size-1,
-// +INF above (src/core/cuda_helpers.h:207-222, src/io/io.cu:297-302); NaN
-// compares false everywhere and lands in bin `size`.
-__global__ void k_bin_assign(const float *__restrict__ x, int ncols, const float *__restrict__ thr,
-                             int thr_stride, const int *__restrict__ sizes,
-                             uint32_t *__restrict__ out, size_t n) {
-  __shared__ float s_thr[4][kSlots];
-  __shared__ int s_size[4];
-  for (int i = threadIdx.x; i < 4 * kSlots; i += blockDim.x) {
-    const int c = i >> 8, t = i & 255;
-    float v = INFINITY;
-    if (c < ncols && t < sizes[c] - 1) v = thr[(size_t)c * thr_stride + t];
-    s_thr[c][t] = v;
-  }
-  if (threadIdx.x < 4) s_size[threadIdx.x] = threadIdx.x < ncols ? sizes[threadIdx.x] : 0;
-  __syncthreads();
-  for (size_t r = (size_t)blockIdx.x * blockDim.x + threadIdx.x; r < n;
-       r += (size_t)gridDim.x * blockDim.x) {
-    uint32_t packed = 0;
-#pragma unroll
-    for (int c = 0; c < 4; ++c) {
-      if (c < ncols) {
-        const float v = x[(size_t)c * n + r];
-        unsigned l = 0, h = (unsigned)s_size[c];
-        while (l < h) {
-          const unsigned mid = (l + h) >> 1;
-          if (v <= s_thr[c][mid])
-            h = mid;
-          else
-            l = mid + 1;
-        }
-        packed |= l << (8 * c);
-      }
-    }
-    out[r] = packed;
-  }
-}
-
-// The same with 16-bit bins: two features per word, thresholds of both in
-// dynamic LDS (2 * thr_stride floats).
-__global__ void k_bin_assign_wide(const float *__restrict__ x, int ncols, const float *__restrict__ thr,
-                                  int thr_stride, const int *__restrict__ sizes,
-                                  uint32_t *__restrict__ out, size_t n) {
-  extern __shared__ float s_thr_wide[];
-  for (int i = threadIdx.x; i < 2 * thr_stride; i += blockDim.x) {
-    const int c = i / thr_stride, t = i % thr_stride;
-    float v = INFINITY;
-    if (c < ncols && t < sizes[c] - 1) v = thr[(size_t)c * thr_stride + t];
-    s_thr_wide[i] = v;
-  }
-  __syncthreads();
-  for (size_t r = (size_t)blockIdx.x * blockDim.x + threadIdx.x; r < n;
-       r += (size_t)gridDim.x * blockDim.x) {
-    uint32_t packed = 0;
-    for (int c = 0; c < ncols; ++c) {
-      const float v = x[(size_t)c * n + r];
-      unsigned l = 0, h = (unsigned)sizes[c];
-      while (l < h) {
-        const unsigned mid = (l + h) >> 1;
-        if (v <= s_thr_wide[c * thr_stride + mid])
-          h = mid;
-        else
-          l = mid + 1;
-      }
-      packed |= l << (16 * c);
-    }
-    out[r] = packed;
-  }
-}
-
-// row-major uint8 [n][F] -> quads
-__global__ void k_pack_prebinned(const uint8_t *__restrict__ in, int F, int Q,
-                                 uint32_t *__restrict__ out, size_t stride, size_t n) {
-  for (size_t r = (size_t)blockIdx.x * blockDim.x + threadIdx.x; r < n;
-       r += (size_t)gridDim.x * blockDim.x) {
-    for (int q = 0; q < Q; ++q) {
-      uint32_t packed = 0;
-      for (int c = 0; c < 4; ++c) {
-        const int f = q * 4 + c;
-        if (f < F) packed |= (uint32_t)in[r * F + f] << (8 * c);
-      }
-      out[(size_t)q * stride + r] = packed;
-    }
-  }
-}
-
-// ------------------------------------------------------------- objectives
-__device__ __forceinline__ float WaveMaxF(float v) {
-  for (int off = 32; off > 0; off >>= 1) v = fmaxf(v, __shfl_down(v, off));
-  return v;
-}
-__device__ __forceinline__ long long WaveSumLL(long long v) {
-  for (int off = 32; off > 0; off >>= 1) v += __shfl_down(v, off);
-  return v;
-}
-
-// squared error: g = y - y_hat (objective.cu:28-38); also max |g| for the
-// fixed-point scale
-__global__ void k_grad_squared(const float *__restrict__ y, const float *__restrict__ yhat,
-                               float *__restrict__ g, size_t n, unsigned *__restrict__ gmax_bits) {
-  float m = 0.0f;
-  for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < n;
-       i += (size_t)gridDim.x * blockDim.x) {
-    const float v = y[i] - yhat[i];
-    g[i] = v;
-    const float a = fabsf(v);
-    if (a > m) m = a;  // NaN never raises the maximum
-  }
-  m = WaveMaxF(m);
-  if ((threadIdx.x & 63) == 0) atomicMax(gmax_bits, __float_as_uint(m));
-}
-
-__global__ void k_set_shift(const unsigned *__restrict__ gmax_bits, int *__restrict__ shifts) {
-  if (threadIdx.x == 0 && blockIdx.x == 0) {
-    shifts[0] = FixShiftFromMax(__uint_as_float(*gmax_bits));
-    shifts[1] = 0;
-  }
-}
-
-// logistic: s = sigmoid(y_hat), g = y - s, h = s(1-s) (objective.cu:43-56)
-__global__ void k_grad_logistic(const float *__restrict__ y, const float *__restrict__ yhat,
-                                float *__restrict__ g, float *__restrict__ h, size_t n) {
-  for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < n;
-       i += (size_t)gridDim.x * blockDim.x) {
-    const float s = SigmoidF(yhat[i]);
-    g[i] = y[i] - s;
-    h[i] = s * (1.0f - s);
-  }
-}
-
-// soft-max: p = softmax(y_hat[., row]), g_k = [label == k] - p_k,
-// h_k = 2 p_k (1 - p_k) (formula in the comment at objective.cu:60-89).
-// y_hat, g, h are class-major [K][n].
-__global__ void k_grad_softmax(const uint8_t *__restrict__ labels, const float *__restrict__ yhat,
-                               float *__restrict__ g, float *__restrict__ h, size_t n, int K) {
-  for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < n;
-       i += (size_t)gridDim.x * blockDim.x) {
-    double mx = -1e300;
-    for (int k = 0; k < K; ++k) mx = fmax(mx, (double)yhat[i + (size_t)k * n]);
-    double sum = 0.0;
-    for (int k = 0; k < K; ++k) sum += (double)ExpF((float)((double)yhat[i + (size_t)k * n] - mx));
-    const int lab = labels[i];
-    for (int k = 0; k < K; ++k) {
-      const double e = (double)ExpF((float)((double)yhat[i + (size_t)k * n] - mx));
-      const float pk = (float)(e / sum);
-      g[i + (size_t)k * n] = (lab == k ? 1.0f : 0.0f) - pk;
-      h[i + (size_t)k * n] = 2.0f * pk * (1.0f - pk);
-    }
-  }
-}
-
-__global__ void k_init_root(NodeSum *tot, unsigned *seg_start, unsigned long long n,
-                            unsigned *gmax_bits) {  // gmax_bits may be NULL
-  if (threadIdx.x == 0 && blockIdx.x == 0) {
-    tot[0].g = 0;
-    tot[0].h = 0;
-    tot[0].c = n;
-    seg_start[0] = 0;
-    if (gmax_bits) *gmax_bits = 0;
-  }
-}
-
-__device__ __forceinline__ unsigned RankBelow(unsigned long long m) {
-  // number of set bits of m below this lane
-  return __builtin_amdgcn_mbcnt_hi((unsigned)(m >> 32), __builtin_amdgcn_mbcnt_lo((unsigned)m, 0u));
-}
-
-// ------------------------------------------------------------------ planner
-// Splits the row ranges of the selected nodes of a level into work items of
-// at most `rows_per_item` rows.  select: 0 = every node, 1 = the smaller
-// child of each sibling pair, ties -> left (hist_grad_sum.cu:279-294).
-// rows_scanned (optional) is advanced by the rows that will be accumulated
-// into histograms: the selected rows, or, when `split` is given (fused
-// partition + histogram over parent nodes), the smaller side of every split.
-// One workgroup.
-__device__ __forceinline__ void PlanBody(const NodeSum *__restrict__ tot, const unsigned *__restrict__ seg_start,
-                                         int L, int select, unsigned rows_per_item,
-                                         WorkItem *__restrict__ work, unsigned *__restrict__ n_work,
-                                         unsigned *__restrict__ node_first, unsigned *__restrict__ node_items,
-                                         unsigned long long *__restrict__ rows_scanned,
-                                         const SplitRec *__restrict__ split, unsigned max_items,
-                                         unsigned *__restrict__ overflow) {
-  __shared__ unsigned s_base[kMaxPlanNodes + 1];
-  __shared__ unsigned s_wave[16];
-  __shared__ unsigned s_carry;
-  __shared__ unsigned long long s_rows;
-  const int tid = threadIdx.x;
-  if (tid == 0) {
-    s_carry = 0;
-    s_rows = 0;
-  }
-  __syncthreads();
-  for (int base = 0; base < L; base += 1024) {
-    const int nd = base + tid;
-    unsigned cnt = 0;
-    if (nd < L) {
-      const unsigned long long len = tot[nd].c;
-      bool sel = true;
-      if (select == 1) {
-        const unsigned long long sib = tot[nd ^ 1].c;
-        sel = (nd & 1) ? (len < sib) : (len <= sib);
-      }
-      if (sel && len > 0) {
-        cnt = (unsigned)((len + rows_per_item - 1) / rows_per_item);
-        unsigned long long acc = len;
-        if (split) {
-          const unsigned long long cl = split[nd].left.c;
-          acc = min(cl, len - cl);
-        }
-        atomicAdd(&s_rows, acc);
-      }
-      node_items[nd] = sel ? cnt : 0xffffffffu;  // 0xffffffff marks "not selected"
-    }
-    // block exclusive scan of cnt
-    unsigned incl = cnt;
-    for (int off = 1; off < 64; off <<= 1) {
-      const unsigned o = __shfl_up(incl, off);
-      if ((tid & 63) >= off) incl += o;
-    }
-    if ((tid & 63) == 63) s_wave[tid >> 6] = incl;
-    __syncthreads();
-    unsigned wave_off = 0;
-    for (int w = 0; w < (tid >> 6); ++w) wave_off += s_wave[w];
-    const unsigned excl = s_carry + wave_off + incl - cnt;
-    if (nd < L) {
-      s_base[nd] = excl;
-      node_first[nd] = excl;
-    }
-    __syncthreads();
-    if (tid == 1023) s_carry = excl + cnt;
-    __syncthreads();
-  }
-  const unsigned total = s_carry;
-  if (tid == 0) {
-    s_base[L] = total;
-    *n_work = total <= max_items ? total : 0;  // never exceed the launch bound
-    if (total > max_items) *overflow = 1;      // reported as an error at the end of the tree
-    if (rows_scanned) *rows_scanned += s_rows;
-  }
-  __syncthreads();
-  if (total > max_items) return;
-  for (unsigned w = tid; w < total; w += 1024) {
-    int lo = 0, hi = L;  // last node whose first item is <= w
-    while (hi - lo > 1) {
-      const int mid = (lo + hi) >> 1;
-      if (s_base[mid] <= w)
-        lo = mid;
-      else
-        hi = mid;
-    }
-    const unsigned start = seg_start[lo];
-    const unsigned len = (unsigned)tot[lo].c;
-    const unsigned k = w - s_base[lo];
-    WorkItem it;
-    it.node = lo;
-    it.begin = start + k * rows_per_item;
-    it.end = min(start + len, it.begin + rows_per_item);
-    it.first = s_base[lo];
-    work[w] = it;
-  }
-}
-
-__global__ void __launch_bounds__(1024)
-k_plan(const NodeSum *__restrict__ tot, const unsigned *__restrict__ seg_start, int L, int select,
-       unsigned rows_per_item, WorkItem *__restrict__ work, unsigned *__restrict__ n_work,
-       unsigned *__restrict__ node_first, unsigned *__restrict__ node_items,
-       unsigned long long *__restrict__ rows_scanned, const SplitRec *__restrict__ split,
-       unsigned max_items, unsigned *__restrict__ overflow) {
-  PlanBody(tot, seg_start, L, select, rows_per_item, work, n_work, node_first, node_items, rows_scanned, split,
-           max_items, overflow);
-}
-
-// Rows of a work item are dealt to its waves in chunks of kChunkRows
-// consecutive rows, round-robin: wave v takes chunks v, v + kItemWaves, ...  A
-// workgroup therefore streams one contiguous block of the item per step (good
-// DRAM page locality) while every wave still owns a fixed, countable row set.
-constexpr unsigned kChunkRows = 128;
-constexpr unsigned kChunkStep = kChunkRows * kItemWaves;
-
-// ---------------------------------------------------------------- histogram
-// LDS layout of a histogram of NQ quads: word0 of every entry, then (PAIR)
-// word1 in the same order.
-template <int NQ>
-struct HistLds {
-  static constexpr int blocks = HistBlocks(NQ);
-  static constexpr int entries = blocks * kBlockEntries;
-  static constexpr int word1 = entries;  // offset of word1 of the same entry
-};
-
-// Adds one row per lane (bins of its NQ quads in b) to the LDS histogram.  The
-// 28 (or 4*NQ) updates of a row are issued in an order that depends on the
-// lane: in step (s, t) of a block, lane l works on quad (s + (l>>2)) % 4 and
-// byte (t + l) % 4 of that quad, so the 16 lanes of a pass of the LDS atomic
-// touch 16 different features = 16 different bank pairs.  q_first: first quad
-// of this launch (a multiple of 4).
-template <bool PAIR, int NQ>
-__device__ __forceinline__ void AccumulateRow(unsigned long long *__restrict__ lds,
-                                              const uint32_t (&b)[NQ], float gv, float hv, int sg,
-                                              int sh, int q_first, int F) {
-  using L = HistLds<NQ>;
-  const unsigned long long w0 = (1ull << kCountShift) + (unsigned long long)ToFixed(gv, sg);
-  unsigned long long w1 = 0;
-  if (PAIR) w1 = (unsigned long long)ToFixed(hv, sh);
-  const unsigned j = (threadIdx.x >> 2) & 3u, i = threadIdx.x & 3u;
-#pragma unroll
-  for (int k = 0; k < L::blocks; ++k) {
-    // quads of this block; the ones past NQ do not exist
-    uint32_t r[4];
-#pragma unroll
-    for (int x = 0; x < 4; ++x) r[x] = 4 * k + x < NQ ? b[4 * k + x < NQ ? 4 * k + x : 0] : 0u;
-#pragma unroll
-    for (int s_ = 0; s_ < 4; ++s_) {
-      const unsigned qi = ((unsigned)s_ + j) & 3u;  // quad of the block this lane works on
-      const uint32_t lo = (j & 1u) ? r[(s_ + 1) & 3] : r[s_];
-      const uint32_t hi = (j & 1u) ? r[(s_ + 3) & 3] : r[(s_ + 2) & 3];
-      const uint32_t sel = (j & 2u) ? hi : lo;
-#pragma unroll
-      for (int t = 0; t < 4; ++t) {
-        const unsigned bi = ((unsigned)t + i) & 3u;  // byte of the quad
-        const unsigned bin = (sel >> (8u * bi)) & 255u;
-        const unsigned f16 = 4u * qi + bi;
-        // Quads past NQ do not exist.  Padding features of the last quad of
-        // the matrix (bin 0 in every row) are accumulated like real ones into
-        // slots nobody reads: cheaper than a per-update test.
-        bool on = true;
-        if (4 * k + 3 >= NQ) on = 4u * k + qi < (unsigned)NQ;
-        if (on) {
-          const unsigned idx = (unsigned)(k * kBlockEntries) + bin * kBlockFeatures + f16;
-          atomicAdd(&lds[idx], w0);
-          if (PAIR) atomicAdd(&lds[L::word1 + idx], w1);
-        }
-      }
-    }
-  }
-}
-
-// Writes the LDS histogram to the slab of work item w in LDS order.  Called by
-// the whole workgroup after its last LDS update.  Slab layout per work item:
-// word0[slab_entries], word1[slab_entries]; q_first is a multiple of 4.
-template <bool PAIR, int NQ>
-__device__ __forceinline__ void FlushSlab(const unsigned long long *__restrict__ lds,
-                                          unsigned long long *__restrict__ slab, unsigned w,
-                                          int slab_entries, int q_first) {
-  using L = HistLds<NQ>;
-  __syncthreads();
-  unsigned long long *out =
-      slab + (size_t)w * slab_entries * (PAIR ? 2 : 1) + (size_t)(q_first / kBlockQuads) * kBlockEntries;
-  for (int e = threadIdx.x; e < L::entries; e += kHistThreads) {
-    out[e] = lds[e];
-    if (PAIR) out[slab_entries + e] = lds[L::word1 + e];
-  }
-}
-
-// Histogram of contiguous row ranges: one workgroup per work item, quads
-// [q0, q0+NQ).  LDS: NQ*1024 word0 entries, then (PAIR) as many word1 entries.
-template <bool PAIR, int NQ>
-__global__ void __launch_bounds__(kHistThreads)
-k_hist(const uint32_t *__restrict__ bins, size_t stride, int q0, int F,
-       const float *__restrict__ g, const float *__restrict__ h, const int *__restrict__ shifts,
-       const WorkItem *__restrict__ work, const unsigned *__restrict__ n_work,
-       unsigned long long *__restrict__ slab, int slab_entries) {
-  extern __shared__ unsigned long long lds[];
-  const unsigned w = blockIdx.x;
-  if (w >= *n_work) return;
-  const WorkItem it = work[w];
-  constexpr int words = (int)(HistLdsBytes(NQ, PAIR) / 8);
-  for (int i = threadIdx.x; i < words; i += kHistThreads) lds[i] = 0ull;
-  __syncthreads();
-  const int sg = shifts[0], sh = shifts[1];
-  const uint32_t *bq = bins + (size_t)q0 * stride;
-  for (unsigned base = it.begin; base < it.end; base += 2 * kHistThreads) {
-    const unsigned r0 = base + threadIdx.x, r1 = r0 + kHistThreads;
-    const bool v0 = r0 < it.end, v1 = r1 < it.end;
-    const unsigned a0 = v0 ? r0 : it.begin, a1 = v1 ? r1 : it.begin;
-    uint32_t b0[NQ], b1[NQ];
-#pragma unroll
-    for (int q = 0; q < NQ; ++q) {
-      b0[q] = __builtin_nontemporal_load(&bq[(size_t)q * stride + a0]);
-      b1[q] = __builtin_nontemporal_load(&bq[(size_t)q * stride + a1]);
-    }
-    const float g0 = g[a0], g1 = g[a1];
-    const float h0 = PAIR ? h[a0] : 0.0f, h1 = PAIR ? h[a1] : 0.0f;
-    if (v0) AccumulateRow<PAIR, NQ>(lds, b0, g0, h0, sg, sh, q0, F);
-    if (v1) AccumulateRow<PAIR, NQ>(lds, b1, g1, h1, sg, sh, q0, F);
-  }
-  FlushSlab<PAIR, NQ>(lds, slab, w, slab_entries, q0);
-}
-
-// Histogram of contiguous row ranges with 16-bit bins: features [f0, f0 + nf)
-// (f0 even), `slots` histogram slots per feature, LDS layout f * slots + bin,
-// word0 of every entry first, then (PAIR) word1.  The slab of a work item has
-// the same feature-major order: word0[slab_entries], word1[slab_entries].
-template <bool PAIR>
-__global__ void __launch_bounds__(kHistThreads)
-k_hist_wide(const uint32_t *__restrict__ bins, size_t stride, int f0, int nf, int slots,
-            const float *__restrict__ g, const float *__restrict__ h, const int *__restrict__ shifts,
-            const WorkItem *__restrict__ work, const unsigned *__restrict__ n_work,
-            unsigned long long *__restrict__ slab, int slab_entries) {
-  extern __shared__ unsigned long long lds[];
-  const unsigned w = blockIdx.x;
-  if (w >= *n_work) return;
-  const WorkItem it = work[w];
-  const int entries = nf * slots;
-  for (int i = threadIdx.x; i < entries * (PAIR ? 2 : 1); i += kHistThreads) lds[i] = 0ull;
-  __syncthreads();
-  const int sg = shifts[0], sh = shifts[1];
-  const int words = (nf + 1) / 2;
-  for (unsigned r = it.begin + threadIdx.x; r < it.end; r += kHistThreads) {
-    const unsigned long long w0 = (1ull << kCountShift) + (unsigned long long)ToFixed(g[r], sg);
-    unsigned long long w1 = 0;
-    if (PAIR) w1 = (unsigned long long)ToFixed(h[r], sh);
-    for (int k = 0; k < words; ++k) {
-      const uint32_t word = bins[(size_t)(f0 / 2 + k) * stride + r];
-      const unsigned lo = (unsigned)(2 * k) * slots + (word & 0xffffu);
-      atomicAdd(&lds[lo], w0);
-      if (PAIR) atomicAdd(&lds[entries + lo], w1);
-      if (2 * k + 1 < nf) {
-        const unsigned hi = (unsigned)(2 * k + 1) * slots + (word >> 16);
-        atomicAdd(&lds[hi], w0);
-        if (PAIR) atomicAdd(&lds[entries + hi], w1);
-      }
-    }
-  }
-  __syncthreads();
-  unsigned long long *out = slab + (size_t)w * slab_entries * (PAIR ? 2 : 1) + (size_t)f0 * slots;
-  for (int e = threadIdx.x; e < entries; e += kHistThreads) {
-    out[e] = lds[e];
-    if (PAIR) out[slab_entries + e] = lds[entries + e];
-  }
-}
-
-// ---------------------------------------------------------------- partition
-// How bin ids are packed in the 32-bit words of a row: 8 bits (four features
-// per word) or 16 bits (two features per word).
-struct BinCode {
-  int wshift;  // feature -> word: fid >> wshift
-  int bits;
-  __host__ __device__ static BinCode Of(int bits) { return BinCode{bits == 8 ? 2 : 1, bits}; }
-  __device__ __forceinline__ int Word(int fid) const { return fid >> wshift; }
-  __device__ __forceinline__ unsigned Bin(uint32_t word, int fid) const {
-    return (word >> (bits * (fid & ((1 << wshift) - 1)))) & ((1u << bits) - 1u);
-  }
-};
-
-__device__ __forceinline__ bool GoesRight(const uint32_t *__restrict__ bins, size_t stride,
-                                          const SplitRec &s, unsigned r, BinCode code = BinCode{2, 8}) {
-  // builder.h:107-123: bin >= q + 1 goes right
-  if (s.fid < 0) return false;
-  const uint32_t word = bins[(size_t)code.Word(s.fid) * stride + r];
-  return (int)code.Bin(word, s.fid) > s.bin;
-}
-
-// Rows going left, per (work item, wave range).
-__global__ void __launch_bounds__(kHistThreads)
-k_part_count(const uint32_t *__restrict__ bins, size_t stride, const SplitRec *__restrict__ split,
-             const WorkItem *__restrict__ work, const unsigned *__restrict__ n_work,
-             unsigned *__restrict__ wave_left, unsigned *__restrict__ item_left, BinCode code) {
-  const unsigned w = blockIdx.x;
-  if (w >= *n_work) return;
-  const WorkItem it = work[w];
-  const SplitRec s = split[it.node];
-  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-  unsigned cnt = 0;
-  if (s.fid < 0) {
-    for (unsigned base = it.begin + wave * kChunkRows; base < it.end; base += kChunkStep)
-      cnt += lane == 0 ? min(kChunkRows, it.end - base) : 0u;
-  } else {
-    const uint32_t *col = bins + (size_t)code.Word(s.fid) * stride;
-    // eight chunks (16 loads) in flight per wave: the pass is latency-bound
-    constexpr int kBatch = 8;
-    for (unsigned base = it.begin + wave * kChunkRows; base < it.end; base += kBatch * kChunkStep) {
-      uint32_t v0[kBatch], v1[kBatch];
-#pragma unroll
-      for (int k = 0; k < kBatch; ++k) {
-        const unsigned r0 = base + k * kChunkStep + lane, r1 = r0 + 64;
-        v0[k] = col[min(r0, it.end - 1)];
-        v1[k] = col[min(r1, it.end - 1)];
-      }
-#pragma unroll
-      for (int k = 0; k < kBatch; ++k) {
-        const unsigned r0 = base + k * kChunkStep + lane, r1 = r0 + 64;
-        if (r0 < it.end) cnt += ((int)code.Bin(v0[k], s.fid) > s.bin) ? 0u : 1u;
-        if (r1 < it.end) cnt += ((int)code.Bin(v1[k], s.fid) > s.bin) ? 0u : 1u;
-      }
-    }
-  }
-  for (int off = 32; off > 0; off >>= 1) cnt += __shfl_down(cnt, off);
-  if (lane == 0) wave_left[(size_t)w * kItemWaves + wave] = cnt;
-  // per-item total for the offset computation of later items of the node
-  __shared__ unsigned s_cnt[kItemWaves];
-  if (lane == 0) s_cnt[wave] = cnt;
-  __syncthreads();
-  if (threadIdx.x == 0) {
-    unsigned t = 0;
-    for (int k = 0; k < kItemWaves; ++k) t += s_cnt[k];
-    item_left[w] = t;
-  }
-}
-
-// Rows going left in the earlier work items of the same node and in the
-// earlier waves of this item.  Called by the whole workgroup; s_tmp holds
-// kItemWaves + 1 words.
-__device__ __forceinline__ unsigned LeftsBefore(const WorkItem &it, unsigned w, int wave,
-                                                const unsigned *__restrict__ wave_left,
-                                                const unsigned *__restrict__ item_left,
-                                                unsigned *s_tmp) {
-  unsigned part = 0;
-  for (unsigned k = it.first + threadIdx.x; k < w; k += blockDim.x) part += item_left[k];
-  for (int off = 32; off > 0; off >>= 1) part += __shfl_down(part, off);
-  if ((threadIdx.x & 63) == 0) s_tmp[threadIdx.x >> 6] = part;
-  __syncthreads();
-  unsigned before = 0;
-  for (int k = 0; k < kItemWaves; ++k) before += s_tmp[k];
-  for (int k = 0; k < wave; ++k) before += wave_left[(size_t)w * kItemWaves + k];
-  __syncthreads();
-  return before;
-}
-
-// Number of rows of a work item dealt to the waves before `wave`.
-__device__ __forceinline__ unsigned RowsOfEarlierWaves(const WorkItem &it, int wave) {
-  const unsigned rows = it.end - it.begin;
-  const unsigned full = rows / kChunkStep, rem = rows % kChunkStep;  // full rounds, rows of the last partial round
-  return full * kChunkRows * (unsigned)wave + min(rem, kChunkRows * (unsigned)wave);
-}
-
-// Destination offsets of one wave: its rows going left are packed in order
-// from the start of the parent's range (after those of earlier items and
-// waves), its rows going right from the start of the right child's range.
-__device__ __forceinline__ void WaveOffsets(const WorkItem &it, const SplitRec &s, unsigned start,
-                                            unsigned lefts_before, int wave, unsigned *lo, unsigned *ro) {
-  const unsigned rows_before = (it.begin - start) + RowsOfEarlierWaves(it, wave);
-  *lo = start + lefts_before;
-  *ro = start + (unsigned)s.left.c + rows_before - lefts_before;
-}
-
-// Position of the k-th (0-based) set bit of the wave-uniform mask m; k < popcount(m).
-__device__ __forceinline__ int SelectBit(unsigned long long m, unsigned k) {
-  const unsigned lo = (unsigned)m, hi = (unsigned)(m >> 32);
-  unsigned c = (unsigned)__popc(lo);
-  const bool up = k >= c;
-  unsigned word = up ? hi : lo;
-  int pos = up ? 32 : 0;
-  k = up ? k - c : k;
-#pragma unroll
-  for (int width = 16; width >= 1; width >>= 1) {
-    const unsigned low = word & ((1u << width) - 1u);
-    c = (unsigned)__popc(low);
-    const bool u = k >= c;
-    word = u ? (word >> width) : low;
-    pos += u ? width : 0;
-    k = u ? k - c : k;
-  }
-  return pos;
-}
-
-// Two rows per lane of a wave's 128-row chunk, as loaded.
-template <int NQ>
-struct RowSet {
-  uint32_t b0[NQ], b1[NQ];
-  uint32_t s0, s1;  // word of the split feature when it is not among b0/b1
-  float g0, g1, h0, h1;
-};
-
-// A wave's register-resident queue of rows on their way to one child's row
-// range: lane l holds the row whose destination is base + l, lanes [0, n) are
-// occupied, and on a wave's first batch lanes [0, skip) stand for the rows
-// before the wave's own range (base is a multiple of 64 rows, so every batch
-// is written as one aligned, fully coalesced 256-byte store per array).
-template <int NQ>
-struct RowQueue {
-  uint32_t b[NQ];
-  float g, h;
-  unsigned n, skip, base;
-  __device__ __forceinline__ void Init(unsigned first_row) {
-#pragma unroll
-    for (int q = 0; q < NQ; ++q) b[q] = 0;
-    g = h = 0.0f;
-    n = skip = first_row & 63u;
-    base = first_row - n;
-  }
-};
-
-// Writes lanes [from, to) of Q to their destination and, for the child whose
-// histogram is built, adds them to the LDS histogram.
-// HIST: the kernel builds a histogram; GH: the gradients move with the rows.
-template <bool PAIR, int NQ, bool HIST = true, bool GH = true>
-__device__ __forceinline__ void EmitRows(unsigned long long *__restrict__ lds, const RowQueue<NQ> &Q,
-                                         unsigned from, unsigned to, bool built,
-                                         uint32_t *__restrict__ bins_out, size_t stride,
-                                         float *__restrict__ g_out, float *__restrict__ h_out, int lane,
-                                         int sg, int sh, int F) {
-  if ((unsigned)lane >= from && (unsigned)lane < to) {
-    // streaming stores and loads: the pass touches every byte once
-    const unsigned d = Q.base + (unsigned)lane;
-#pragma unroll
-    for (int q = 0; q < NQ; ++q) __builtin_nontemporal_store(Q.b[q], &bins_out[(size_t)q * stride + d]);
-    if (GH && g_out != nullptr) {  // a group pass after the first leaves the gradients alone
-      __builtin_nontemporal_store(Q.g, &g_out[d]);
-      if (PAIR) __builtin_nontemporal_store(Q.h, &h_out[d]);
-    }
-    if (HIST && built) AccumulateRow<PAIR, NQ>(lds, Q.b, Q.g, Q.h, sg, sh, 0, F);
-  }
-}
-
-// Appends the rows of X flagged in xm (wave-uniform mask, one row per lane) to
-// Q in row order with one lane permute per register; a full queue is emitted
-// and the rest of X starts the next batch.
-template <bool PAIR, int NQ, bool HIST = true, bool GH = true>
-__device__ __forceinline__ void MergeRows(unsigned long long *__restrict__ lds, RowQueue<NQ> &Q,
-                                          const uint32_t (&xb)[NQ], float xg, float xh,
-                                          unsigned long long xm, bool built,
-                                          uint32_t *__restrict__ bins_out, size_t stride,
-                                          float *__restrict__ g_out, float *__restrict__ h_out, int lane,
-                                          int sg, int sh, int F) {
-  const unsigned nx = (unsigned)__popcll(xm);
-  if (nx == 0) return;  // wave-uniform
-  // lane l receives the k-th flagged row, k = (l - n) mod 64: lanes >= n fill
-  // the current batch, lanes < n hold what overflows into the next one
-  const unsigned k = ((unsigned)lane - Q.n) & 63u;
-  const int src = SelectBit(xm, k < nx ? k : 0u);
-  uint32_t vb[NQ];
-#pragma unroll
-  for (int q = 0; q < NQ; ++q) vb[q] = (uint32_t)__shfl((int)xb[q], src);
-  const float vg = GH ? __shfl(xg, src) : 0.0f;
-  const float vh = GH && PAIR ? __shfl(xh, src) : 0.0f;
-  if (Q.n + nx >= 64u) {  // wave-uniform: the batch is complete
-    const bool fill = (unsigned)lane >= Q.n;
-#pragma unroll
-    for (int q = 0; q < NQ; ++q) Q.b[q] = fill ? vb[q] : Q.b[q];
-    Q.g = fill ? vg : Q.g;
-    Q.h = fill ? vh : Q.h;
-    EmitRows<PAIR, NQ, HIST, GH>(lds, Q, Q.skip, 64u, built, bins_out, stride, g_out, h_out, lane, sg, sh, F);
-    Q.base += 64u;
-    Q.skip = 0u;
-#pragma unroll
-    for (int q = 0; q < NQ; ++q) Q.b[q] = vb[q];
-    Q.g = vg;
-    Q.h = vh;
-    Q.n = Q.n + nx - 64u;
-  } else {
-    const bool fill = (unsigned)lane >= Q.n && k < nx;
-#pragma unroll
-    for (int q = 0; q < NQ; ++q) Q.b[q] = fill ? vb[q] : Q.b[q];
-    Q.g = fill ? vg : Q.g;
-    Q.h = fill ? vh : Q.h;
-    Q.n += nx;
-  }
-}
-
-// Fused pass over the rows of the parent nodes of a level: stable partition
-// into the children order (WRITE) and histogram of the smaller child of every
-// split in LDS.  Each wave owns the 128-row chunks v, v + 16, ... of the item
-// and runs without workgroup barriers.  With WRITE the rows of a chunk are
-// sorted into two register queues (one per child) with lane permutes; a full
-// queue is one aligned 64-row store per array, and the queue of the built
-// child is added to the histogram as a full wave (LDS atomic instructions
-// cost the same with one active lane as with 64).  Writing each chunk's rows
-// directly, as two short unaligned runs per store, costs 40 % more time than
-// the copy itself.  On the last level only the quad of the split feature is
-// read for every row; the selected rows are queued by row id and read 64 at a
-// time.  NQ = all quads of the matrix.
-// GROUP: `bins` / `bins_out` point at quad q0 of a wider matrix (q0 a multiple
-// of 4); the quad of the split feature is read from `split_bins`, the start of
-// the whole matrix, and g_out may be null (the gradients moved with an
-// earlier group of the same level).
-template <bool PAIR, int NQ, bool WRITE, bool GROUP = false>
-__global__ void __launch_bounds__(kHistThreads)
-k_part_hist(const uint32_t *__restrict__ bins, uint32_t *__restrict__ bins_out, size_t stride, int F,
-            const float *__restrict__ g, float *__restrict__ g_out, const float *__restrict__ h,
-            float *__restrict__ h_out, const int *__restrict__ shifts,
-            const SplitRec *__restrict__ split, const NodeSum *__restrict__ tot,
-            const unsigned *__restrict__ seg_start, const WorkItem *__restrict__ work,
-            const unsigned *__restrict__ n_work, const unsigned *__restrict__ wave_left,
-            const unsigned *__restrict__ item_left, unsigned long long *__restrict__ slab,
-            int slab_entries, const uint32_t *__restrict__ split_bins, int q0) {
-  extern __shared__ unsigned long long lds[];
-  __shared__ unsigned s_tmp[kItemWaves + 1];
-  const unsigned w = blockIdx.x;
-  if (w >= *n_work) return;
-  const WorkItem it = work[w];
-  const SplitRec s = split[it.node];
-  const unsigned long long cl = s.left.c, cr = tot[it.node].c - cl;
-  const bool build_right = cl > cr;  // ties -> left (hist_grad_sum.cu:288-290)
-  constexpr int words = (int)(HistLdsBytes(NQ, PAIR) / 8);
-  for (int i = threadIdx.x; i < words; i += kHistThreads) lds[i] = 0ull;
-  const int sg = shifts[0], sh = shifts[1];
-  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-  const unsigned wb = it.begin + wave * kChunkRows, we = it.end;
-  unsigned lo = 0, ro = 0;
-  if (WRITE) {
-    const unsigned before = LeftsBefore(it, w, wave, wave_left, item_left, s_tmp);
-    WaveOffsets(it, s, seg_start[it.node], before, wave, &lo, &ro);
-  }
-  __syncthreads();
-  const int fq = s.fid >> 2, fs = 8 * (s.fid & 3);
-  if constexpr (WRITE) {
-    // QB: rows of the child whose histogram is built, QO: the other child
-    RowQueue<NQ> QB, QO;
-    QB.Init(build_right ? ro : lo);
-    QO.Init(build_right ? lo : ro);
-    // Two register sets of 128 rows each: while one is processed the other is
-    // in flight.  The loads are unconditional (addresses clamped to the last
-    // row of the item) and the sets are never copied, so every wait in the loop
-    // is for exactly the set that is needed next.
-    const uint32_t *split_col = split_bins + (size_t)(s.fid < 0 ? 0 : fq) * stride;
-    auto load = [&](RowSet<NQ> &R, unsigned base) {
-      const unsigned a0 = min(base + lane, we - 1), a1 = min(base + 64 + lane, we - 1);
-#pragma unroll
-      for (int q = 0; q < NQ; ++q) {
-        R.b0[q] = __builtin_nontemporal_load(&bins[(size_t)q * stride + a0]);
-        R.b1[q] = __builtin_nontemporal_load(&bins[(size_t)q * stride + a1]);
-      }
-      if (GROUP) {  // the quad of the split feature, wherever it lives
-        R.s0 = split_col[a0];
-        R.s1 = split_col[a1];
-      }
-      R.g0 = __builtin_nontemporal_load(&g[a0]);
-      R.g1 = __builtin_nontemporal_load(&g[a1]);
-      R.h0 = PAIR ? __builtin_nontemporal_load(&h[a0]) : 0.0f;
-      R.h1 = PAIR ? __builtin_nontemporal_load(&h[a1]) : 0.0f;
-    };
-    auto process = [&](const RowSet<NQ> &R, unsigned base) {
-      const unsigned r0 = base + lane, r1 = r0 + 64;
-      const bool v0 = r0 < we, v1 = r1 < we;
-      uint32_t s0 = 0, s1 = 0;
-      if (GROUP) {
-        s0 = R.s0;
-        s1 = R.s1;
-      } else {
-#pragma unroll
-        for (int q = 0; q < NQ; ++q) {
-          s0 = q == fq ? R.b0[q] : s0;
-          s1 = q == fq ? R.b1[q] : s1;
-        }
-      }
-      const bool right0 = v0 && s.fid >= 0 && (int)((s0 >> fs) & 255u) > s.bin;
-      const bool right1 = v1 && s.fid >= 0 && (int)((s1 >> fs) & 255u) > s.bin;
-      const unsigned long long b0 = __ballot(v0 && right0 == build_right), o0 = __ballot(v0 && right0 != build_right);
-      const unsigned long long b1 = __ballot(v1 && right1 == build_right), o1 = __ballot(v1 && right1 != build_right);
-      MergeRows<PAIR, NQ>(lds, QO, R.b0, R.g0, R.h0, o0, false, bins_out, stride, g_out, h_out, lane, sg, sh, F);
-      MergeRows<PAIR, NQ>(lds, QB, R.b0, R.g0, R.h0, b0, true, bins_out, stride, g_out, h_out, lane, sg, sh, F);
-      MergeRows<PAIR, NQ>(lds, QO, R.b1, R.g1, R.h1, o1, false, bins_out, stride, g_out, h_out, lane, sg, sh, F);
-      MergeRows<PAIR, NQ>(lds, QB, R.b1, R.g1, R.h1, b1, true, bins_out, stride, g_out, h_out, lane, sg, sh, F);
-    };
-    if (wb < we) {
-      RowSet<NQ> A, B;
-      load(A, wb);
-      for (unsigned base = wb;; base += 2 * kChunkStep) {
-        load(B, base + kChunkStep);
-        process(A, base);
-        if (base + kChunkStep >= we) break;  // wave-uniform
-        load(A, base + 2 * kChunkStep);
-        process(B, base + kChunkStep);
-        if (base + 2 * kChunkStep >= we) break;
-      }
-    }
-    EmitRows<PAIR, NQ>(lds, QO, QO.skip, QO.n, false, bins_out, stride, g_out, h_out, lane, sg, sh, F);
-    EmitRows<PAIR, NQ>(lds, QB, QB.skip, QB.n, true, bins_out, stride, g_out, h_out, lane, sg, sh, F);
-  } else {
-    // Rows selected for the histogram are queued by row id (slot 64 * j + lane
-    // of the queue is lane `lane` of q[j]; slots [0, np) are occupied) and read
-    // again 64 at a time: LDS atomic instructions cost the same with one active
-    // lane as with 64, so only full waves are accumulated.  The second read
-    // hits the cache, is requested at the start of a chunk and used at its end,
-    // and the wave never waits for its LDS atomics.
-    unsigned q0 = it.begin, q1 = it.begin, q2 = it.begin;
-    unsigned np = 0;
-    uint32_t gb[NQ];
-    float gg = 0.0f, gh = 0.0f;
-    auto gather = [&](bool valid) {  // requests the rows of queue slots [0, 64)
-      const unsigned a = valid ? q0 : it.begin;
-#pragma unroll
-      for (int q = 0; q < NQ; ++q) gb[q] = bins[(size_t)q * stride + a];
-      gg = g[a];
-      gh = PAIR ? h[a] : 0.0f;
-      q0 = q1;
-      q1 = q2;
-    };
-    // m: wave-uniform mask of the selected rows among base + [0, 64); np < 128
-    auto enqueue = [&](unsigned base, unsigned long long m) {
-      const unsigned nx = (unsigned)__popcll(m);
-      if (nx == 0) return;
-      const unsigned r = np & 63u, j = np >> 6;
-      const unsigned k = ((unsigned)lane - r) & 63u;  // slot np + k
-      const unsigned id = base + (unsigned)SelectBit(m, k < nx ? k : 0u);
-      const bool here = (unsigned)lane >= r && k < nx;   // lands in q[j]
-      const bool next = (unsigned)lane < r && k < nx;    // lands in q[j + 1]
-      q0 = (j == 0 && here) ? id : q0;
-      q1 = ((j == 1 && here) || (j == 0 && next)) ? id : q1;
-      q2 = (j == 1 && next) ? id : q2;
-      np += nx;
-    };
-    // after a chunk: at most 127 rows stay queued
-    auto drain = [&](unsigned limit) {
-      while (np > limit) {
-        const unsigned take = min(np, 64u);
-        const bool valid = (unsigned)lane < take;
-        gather(valid);
-        if (valid) AccumulateRow<PAIR, NQ>(lds, gb, gg, gh, sg, sh, 0, F);
-        np -= take;
-      }
-    };
-    if (wb < we) {
-      // last level: only the quad of the split feature decides; the selected
-      // rows are read when they are accumulated
-      const uint32_t *col = split_bins + (size_t)(s.fid < 0 ? 0 : fq) * stride;
-      auto step = [&](uint32_t s0, uint32_t s1, uint32_t &n0, uint32_t &n1, unsigned base) {
-        const bool full = np >= 64u;  // wave-uniform
-        if (full) {
-          gather(true);
-          np -= 64u;
-        }
-        n0 = col[min(base + kChunkStep + lane, we - 1)];
-        n1 = col[min(base + kChunkStep + 64 + lane, we - 1)];
-        const unsigned r0 = base + lane, r1 = r0 + 64;
-        const bool v0 = r0 < we, v1 = r1 < we;
-        const bool right0 = v0 && s.fid >= 0 && (int)((s0 >> fs) & 255u) > s.bin;
-        const bool right1 = v1 && s.fid >= 0 && (int)((s1 >> fs) & 255u) > s.bin;
-        enqueue(base, __ballot(v0 && right0 == build_right));
-        enqueue(base + 64, __ballot(v1 && right1 == build_right));
-        if (full) AccumulateRow<PAIR, NQ>(lds, gb, gg, gh, sg, sh, 0, F);
-        drain(127u);
-      };
-      uint32_t a0 = col[min(wb + lane, we - 1)], a1 = col[min(wb + 64 + lane, we - 1)], b0, b1;
-      for (unsigned base = wb;; base += 2 * kChunkStep) {
-        step(a0, a1, b0, b1, base);
-        if (base + kChunkStep >= we) break;  // wave-uniform
-        step(b0, b1, a0, a1, base + kChunkStep);
-        if (base + 2 * kChunkStep >= we) break;
-      }
-    }
-    drain(0u);
-  }
-  FlushSlab<PAIR, NQ>(lds, slab, w, slab_entries, q0);
-}
-
-// Stable partition alone (matrices too wide for the fused pass, 16-bit bins):
-// words [q0, q0 + NQ) of every row, and with GH the gradients, go to the
-// children order through the two register queues of the fused pass.  One launch
-// per group of words; every launch reads the word of the split feature again.
-template <bool PAIR, int NQ, bool GH>
-__global__ void __launch_bounds__(kHistThreads)
-k_part_rows(const uint32_t *__restrict__ bins, uint32_t *__restrict__ bins_out, size_t stride, int q0,
-            const float *__restrict__ g, float *__restrict__ g_out, const float *__restrict__ h,
-            float *__restrict__ h_out, const SplitRec *__restrict__ split,
-            const unsigned *__restrict__ seg_start, const WorkItem *__restrict__ work,
-            const unsigned *__restrict__ n_work, const unsigned *__restrict__ wave_left,
-            const unsigned *__restrict__ item_left, BinCode code) {
-  __shared__ unsigned s_tmp[kItemWaves + 1];
-  const unsigned w = blockIdx.x;
-  if (w >= *n_work) return;
-  const WorkItem it = work[w];
-  const SplitRec s = split[it.node];
-  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-  const unsigned wb = it.begin + wave * kChunkRows, we = it.end;
-  unsigned lo, ro;
-  const unsigned before = LeftsBefore(it, w, wave, wave_left, item_left, s_tmp);
-  WaveOffsets(it, s, seg_start[it.node], before, wave, &lo, &ro);
-  if (wb >= we) return;
-  const uint32_t *group = bins + (size_t)q0 * stride;
-  uint32_t *group_out = bins_out + (size_t)q0 * stride;
-  const uint32_t *split_col = bins + (size_t)(s.fid < 0 ? 0 : code.Word(s.fid)) * stride;
-  RowQueue<NQ> QL, QR;
-  QL.Init(lo);
-  QR.Init(ro);
-  struct Rows {
-    RowSet<NQ> r;
-    uint32_t s0, s1;  // word of the split feature
-  };
-  auto load = [&](Rows &R, unsigned base) {
-    const unsigned a0 = min(base + lane, we - 1), a1 = min(base + 64 + lane, we - 1);
-#pragma unroll
-    for (int q = 0; q < NQ; ++q) {
-      R.r.b0[q] = __builtin_nontemporal_load(&group[(size_t)q * stride + a0]);
-      R.r.b1[q] = __builtin_nontemporal_load(&group[(size_t)q * stride + a1]);
-    }
-    R.s0 = split_col[a0];
-    R.s1 = split_col[a1];
-    R.r.g0 = GH ? __builtin_nontemporal_load(&g[a0]) : 0.0f;
-    R.r.g1 = GH ? __builtin_nontemporal_load(&g[a1]) : 0.0f;
-    R.r.h0 = GH && PAIR ? __builtin_nontemporal_load(&h[a0]) : 0.0f;
-    R.r.h1 = GH && PAIR ? __builtin_nontemporal_load(&h[a1]) : 0.0f;
-  };
-  auto process = [&](const Rows &R, unsigned base) {
-    const unsigned r0 = base + lane, r1 = r0 + 64;
-    const bool v0 = r0 < we, v1 = r1 < we;
-    const bool right0 = v0 && s.fid >= 0 && (int)code.Bin(R.s0, s.fid) > s.bin;
-    const bool right1 = v1 && s.fid >= 0 && (int)code.Bin(R.s1, s.fid) > s.bin;
-    const unsigned long long lm0 = __ballot(v0 && !right0), rm0 = __ballot(right0);
-    const unsigned long long lm1 = __ballot(v1 && !right1), rm1 = __ballot(right1);
-    MergeRows<PAIR, NQ, false, GH>(nullptr, QL, R.r.b0, R.r.g0, R.r.h0, lm0, false, group_out, stride, g_out, h_out, lane, 0, 0, 0);
-    MergeRows<PAIR, NQ, false, GH>(nullptr, QR, R.r.b0, R.r.g0, R.r.h0, rm0, false, group_out, stride, g_out, h_out, lane, 0, 0, 0);
-    MergeRows<PAIR, NQ, false, GH>(nullptr, QL, R.r.b1, R.r.g1, R.r.h1, lm1, false, group_out, stride, g_out, h_out, lane, 0, 0, 0);
-    MergeRows<PAIR, NQ, false, GH>(nullptr, QR, R.r.b1, R.r.g1, R.r.h1, rm1, false, group_out, stride, g_out, h_out, lane, 0, 0, 0);
-  };
-  Rows A, B;
-  load(A, wb);
-  for (unsigned base = wb;; base += 2 * kChunkStep) {
-    load(B, base + kChunkStep);
-    process(A, base);
-    if (base + kChunkStep >= we) break;  // wave-uniform
-    load(A, base + 2 * kChunkStep);
-    process(B, base + kChunkStep);
-    if (base + 2 * kChunkStep >= we) break;
-  }
-  EmitRows<PAIR, NQ, false, GH>(nullptr, QL, QL.skip, QL.n, false, group_out, stride, g_out, h_out, lane, 0, 0, 0);
-  EmitRows<PAIR, NQ, false, GH>(nullptr, QR, QR.skip, QR.n, false, group_out, stride, g_out, h_out, lane, 0, 0, 0);
-}
-
-// Adds the slabs of every directly built node of a level (on top of the stored
-// histogram when `accumulate`) and, with `trick`, derives its sibling as
-// parent - node.  Slabs are in LDS order (16-feature blocks, bin-major); the
-// histograms written here are feature-major: hist[node][f * 256 + bin].
-// grid (slab_entries/64, L), 1024 threads = 64 entries x 16 slab lanes.
-//   by_parent = 0: slabs belong to work items of the node itself
-//               (node_items == 0xffffffff marks a derived node);
-//   by_parent = 1: slabs belong to work items of the parent (fused pass); the
-//               built child is the smaller one, ties -> left.
-template <bool PAIR, int LANES>
-__global__ void __launch_bounds__(1024)
-k_hist_reduce(const unsigned long long *__restrict__ slab, int slab_entries, int nbin_total,
-              const unsigned *__restrict__ node_first, const unsigned *__restrict__ node_items,
-              int by_parent, const SplitRec *__restrict__ parent_split,
-              const NodeSum *__restrict__ parent_tot, long long *__restrict__ hg,
-              long long *__restrict__ hh, unsigned *__restrict__ hc,
-              const long long *__restrict__ pg, const long long *__restrict__ ph,
-              const unsigned *__restrict__ pc, int trick, int accumulate, int plain) {
-  // LANES threads share the slabs of one entry; a block covers 1024 / LANES
-  // consecutive entries (with 4 lanes: 16 bins x 16 features, so the
-  // feature-major output is written in runs of 16 bins)
-  constexpr int kEntries = 1024 / LANES;
-  __shared__ long long s_g[LANES][kEntries];
-  __shared__ long long s_h[LANES][kEntries];
-  __shared__ unsigned s_c[LANES][kEntries];
-  const int nd = blockIdx.y;
-  unsigned items, first;
-  if (by_parent) {
-    const int p = nd >> 1;
-    const unsigned long long cl = parent_split[p].left.c, cr = parent_tot[p].c - cl;
-    const bool build_right = cl > cr;
-    if (((nd & 1) != 0) != build_right) return;  // derived from its sibling
-    items = node_items[p];
-    first = node_first[p];
-  } else {
-    items = node_items[nd];
-    first = node_first[nd];
-    if (items == 0xffffffffu) return;  // derived from its sibling
-  }
-  const int e = threadIdx.x % kEntries, lane = threadIdx.x / kEntries;
-  const int entry = blockIdx.x * kEntries + e;  // slab order
-  // plain: the slabs are feature-major already (16-bit bins)
-  const int f = (entry / kBlockEntries) * kBlockFeatures + (entry & (kBlockFeatures - 1));
-  const int bin = (entry / kBlockFeatures) & (kSlots - 1);
-  // the last 16-feature block may have fewer than 16 features
-  const bool live = plain ? entry < nbin_total : f * kSlots < nbin_total;
-  long long ag = 0, ah = 0;
-  unsigned ac = 0;
-  if (live) {
-    for (unsigned s = lane; s < items; s += LANES) {
-      const unsigned long long *p = slab + (size_t)(first + s) * slab_entries * (PAIR ? 2 : 1);
-      const unsigned long long w0 = p[entry];
-      const long long gq = ((long long)(w0 << (64 - kCountShift))) >> (64 - kCountShift);
-      ag += gq;
-      ac += (unsigned)((w0 - (unsigned long long)gq) >> kCountShift);
-      if (PAIR) ah += (long long)p[slab_entries + entry];
-    }
-  }
-  s_g[lane][e] = ag;
-  s_h[lane][e] = ah;
-  s_c[lane][e] = ac;
-  __syncthreads();
-  if (lane == 0 && live) {
-    for (int k = 1; k < LANES; ++k) {
-      ag += s_g[k][e];
-      ah += s_h[k][e];
-      ac += s_c[k][e];
-    }
-    const size_t cell = plain ? (size_t)entry : (size_t)f * kSlots + bin;
-    const size_t o = (size_t)nd * nbin_total + cell;
-    if (accumulate) {  // streamed matrices: one call per row block
-      ag += hg[o];
-      ah += hh[o];
-      ac += hc[o];
-    }
-    hg[o] = ag;
-    hh[o] = ah;
-    hc[o] = ac;
-    if (trick) {
-      const size_t po = (size_t)(nd >> 1) * nbin_total + cell;
-      const size_t so = (size_t)(nd ^ 1) * nbin_total + cell;
-      hg[so] = pg[po] - ag;
-      hh[so] = ph[po] - ah;
-      hc[so] = pc[po] - ac;
-    }
-  }
-}
-
-// Root totals = sum over the slots of feature 0 of the root histogram (every
-// row, NaN included, sits in exactly one slot).  Replaces the reduction over
-// the gradient array of garden.cu:432-435.  One wave.
-__global__ void __launch_bounds__(64)
-k_root_from_hist(const long long *__restrict__ hg, const long long *__restrict__ hh,
-                 NodeSum *__restrict__ tot, int slots) {
-  long long a = 0, b = 0;
-  for (int i = threadIdx.x; i < slots; i += 64) {
-    a += hg[i];
-    b += hh[i];
-  }
-  a = WaveSumLL(a);
-  b = WaveSumLL(b);
-  if (threadIdx.x == 0) {
-    tot[0].g = a;
-    tot[0].h = b;
-  }
-}
-
-// ----------------------------------------------------- streamed row blocks
-// When the bins do not live in HBM (pinned host blocks copied in at every
-// level; the reference streams whole columns, hist_tree_grower.cu:335-366),
-// rows are never re-ordered.  A resident node id per row is advanced with the
-// parents' splits while its block is on the GPU, the rows of the nodes built
-// at this level are gathered node by node into a staging buffer, and the
-// ordinary histogram kernel runs on that buffer.
-
-// Is node nd accumulated directly at this level?  With sibling subtraction
-// only the smaller child of each pair, ties -> left (hist_grad_sum.cu:279-294).
-__device__ __forceinline__ bool NodeIsBuilt(const NodeSum *__restrict__ tot, unsigned nd, int level, int trick) {
-  if (level == 0 || !trick) return true;
-  const unsigned long long c = tot[nd].c, sib = tot[nd ^ 1u].c;
-  return (nd & 1u) ? (c < sib) : (c <= sib);
-}
-
-// Advances the node id of every row of the block by the parents' splits and
-// counts the rows of every built node (blk_cnt, zero on entry).
-__global__ void __launch_bounds__(256)
-k_stream_route(const uint32_t *__restrict__ bins, size_t bstride, unsigned rows, int level, int trick,
-               const SplitRec *__restrict__ split, const NodeSum *__restrict__ tot,
-               unsigned *__restrict__ node_of, unsigned *__restrict__ blk_cnt) {
-  __shared__ unsigned s_cnt[kMaxPlanNodes];
-  const int L = 1 << level;
-  for (int i = threadIdx.x; i < L; i += blockDim.x) s_cnt[i] = 0;
-  __syncthreads();
-  const int lane = threadIdx.x & 63;
-  const unsigned step = gridDim.x * blockDim.x;
-  for (unsigned r0 = blockIdx.x * blockDim.x; r0 < rows; r0 += step) {  // whole waves stay together
-    const unsigned r = r0 + threadIdx.x;
-    unsigned nd = 0;
-    bool built = false;
-    if (r < rows) {
-      if (level > 0) {
-        const unsigned parent = node_of[r];
-        nd = parent * 2u + (GoesRight(bins, bstride, split[parent], r) ? 1u : 0u);
-      }
-      node_of[r] = nd;
-      built = NodeIsBuilt(tot, nd, level, trick);
-    }
-    // one LDS atomic per distinct node of the wave (64 lanes on one address serialise)
-    unsigned long long todo = __ballot(built);
-    while (todo) {
-      const int leader = __ffsll((long long)todo) - 1;
-      const unsigned lead_nd = (unsigned)__shfl((int)nd, leader);
-      const unsigned long long same = __ballot(built && nd == lead_nd);
-      if (lane == leader) atomicAdd(&s_cnt[lead_nd], (unsigned)__popcll(same));
-      todo &= ~same;
-    }
-  }
-  __syncthreads();
-  for (int i = threadIdx.x; i < L; i += blockDim.x)
-    if (s_cnt[i]) atomicAdd(&blk_cnt[i], s_cnt[i]);
-}
-
-// Row ranges of the built nodes inside the staging buffer: exclusive scan of
-// blk_cnt; also the cursors of the gather and the totals the planner reads.
-// Clears blk_cnt for the next block.  One workgroup.
-__global__ void __launch_bounds__(1024)
-k_stream_segments(unsigned *__restrict__ blk_cnt, int L, NodeSum *__restrict__ blk_tot,
-                  unsigned *__restrict__ blk_seg, unsigned *__restrict__ cursor) {
-  __shared__ unsigned s_wave[16];
-  __shared__ unsigned s_carry;
-  if (threadIdx.x == 0) s_carry = 0;
-  __syncthreads();
-  for (int base = 0; base < L; base += 1024) {
-    const int nd = base + threadIdx.x;
-    const unsigned c = nd < L ? blk_cnt[nd] : 0u;
-    unsigned incl = c;
-    for (int off = 1; off < 64; off <<= 1) {
-      const unsigned o = __shfl_up(incl, off);
-      if ((threadIdx.x & 63) >= off) incl += o;
-    }
-    if ((threadIdx.x & 63) == 63) s_wave[threadIdx.x >> 6] = incl;
-    __syncthreads();
-    unsigned off = s_carry;
-    for (int w = 0; w < (int)(threadIdx.x >> 6); ++w) off += s_wave[w];
-    const unsigned excl = off + incl - c;
-    if (nd < L) {
-      blk_seg[nd] = excl;
-      cursor[nd] = excl;
-      blk_tot[nd].g = 0;
-      blk_tot[nd].h = 0;
-      blk_tot[nd].c = c;
-      blk_cnt[nd] = 0;
-    }
-    __syncthreads();
-    if (threadIdx.x == 1023) s_carry = excl + c;
-    __syncthreads();
-  }
-}
-
-// Copies the rows of the built nodes into the staging buffer, node by node.
-// The order inside a node is whatever the atomics give; sums are integers.
-template <bool PAIR>
-__global__ void __launch_bounds__(256)
-k_stream_gather(const uint32_t *__restrict__ bins, size_t bstride, int Q, unsigned rows,
-                const float *__restrict__ g, const float *__restrict__ h,
-                const unsigned *__restrict__ node_of, int level, int trick,
-                const NodeSum *__restrict__ tot, unsigned *__restrict__ cursor,
-                uint32_t *__restrict__ st_bins, size_t sstride, float *__restrict__ st_g,
-                float *__restrict__ st_h) {
-  const int lane = threadIdx.x & 63;
-  const unsigned step = gridDim.x * blockDim.x;
-  for (unsigned r0 = blockIdx.x * blockDim.x; r0 < rows; r0 += step) {  // whole waves stay together
-    const unsigned r = r0 + threadIdx.x;
-    unsigned nd = 0;
-    bool built = false;
-    if (r < rows) {
-      nd = node_of[r];
-      built = NodeIsBuilt(tot, nd, level, trick);
-    }
-    // one cursor atomic per distinct node of the wave
-    unsigned d = 0;
-    unsigned long long todo = __ballot(built);
-    while (todo) {
-      const int leader = __ffsll((long long)todo) - 1;
-      const unsigned lead_nd = (unsigned)__shfl((int)nd, leader);
-      const unsigned long long same = __ballot(built && nd == lead_nd);
-      unsigned base = 0;
-      if (lane == leader) base = atomicAdd(&cursor[lead_nd], (unsigned)__popcll(same));
-      base = (unsigned)__shfl((int)base, leader);
-      if (built && nd == lead_nd) d = base + RankBelow(same);
-      todo &= ~same;
-    }
-    if (built) {
-      for (int q = 0; q < Q; ++q) st_bins[(size_t)q * sstride + d] = bins[(size_t)q * bstride + r];
-      st_g[d] = g[r];
-      if (PAIR) st_h[d] = h[r];
-    }
-  }
-}
-
-// sibling = parent - built child for every node that was not built directly
-__global__ void k_sibling(long long *__restrict__ hg, long long *__restrict__ hh, unsigned *__restrict__ hc,
-                          const long long *__restrict__ pg, const long long *__restrict__ ph,
-                          const unsigned *__restrict__ pc, const NodeSum *__restrict__ tot, int level,
-                          int nbin_total) {
-  const unsigned nd = blockIdx.y;
-  if (NodeIsBuilt(tot, nd, level, 1)) return;
-  const int e = blockIdx.x * blockDim.x + threadIdx.x;
-  if (e >= nbin_total) return;
-  const size_t o = (size_t)nd * nbin_total + e, so = (size_t)(nd ^ 1u) * nbin_total + e,
-               po = (size_t)(nd >> 1) * nbin_total + e;
-  hg[o] = pg[po] - hg[so];
-  hh[o] = ph[po] - hh[so];
-  hc[o] = pc[po] - hc[so];
-}
-
-// --------------------------------------------------------------- split scan
-struct Cand {
-  float gain;
-  int bin;
-  NodeSum left;
-};
-
-// One wave per (feature, node): inclusive prefix over the 256 slots, gain per
-// bin < hist_size, arg-max with ties to the HIGHEST bin (builder.h:39-49),
-// only gains > 0 (hist_tree_grower.cu:31).
-template <bool PAIR, bool F64>
-__global__ void __launch_bounds__(64)
-k_split_scan(const long long *__restrict__ hg, const long long *__restrict__ hh,
-             const unsigned *__restrict__ hc, int nbin_total, int F, int slots,
-             const NodeSum *__restrict__ tot, const int *__restrict__ shifts, GainParams gp,
-             int hist_size, Cand *__restrict__ cand) {
-  const int f = blockIdx.x, nd = blockIdx.y, lane = threadIdx.x;
-  const NodeSum t = tot[nd];
-  Cand best;
-  best.gain = 0.0f;
-  best.bin = -1;
-  best.left.g = best.left.h = 0;
-  best.left.c = 0;
-  if (t.c != 0) {
-    const int sg = shifts[0], sh = shifts[1];
-    const double GT = FromFixed<F64>(t.g, sg);
-    const double HT = PAIR ? FromFixed<F64>(t.h, sh) : 0.0;
-    // sums of the slots below the current chunk of 256
-    long long carry_g = 0, carry_h = 0;
-    unsigned long long carry_c = 0;
-    for (int chunk = 0; chunk < slots && chunk < hist_size; chunk += 256) {
-      const size_t base = (size_t)nd * nbin_total + (size_t)f * slots + chunk + lane * 4;
-      long long g4[4], h4[4];
-      unsigned long long c4[4];
-#pragma unroll
-      for (int j = 0; j < 4; ++j) {
-        g4[j] = hg[base + j];
-        h4[j] = PAIR ? hh[base + j] : 0;
-        c4[j] = hc[base + j];
-      }
-#pragma unroll
-      for (int j = 1; j < 4; ++j) {
-        g4[j] += g4[j - 1];
-        h4[j] += h4[j - 1];
-        c4[j] += c4[j - 1];
-      }
-      long long ig = g4[3], ih = h4[3];
-      unsigned long long ic = c4[3];
-      for (int off = 1; off < 64; off <<= 1) {
-        const long long og = __shfl_up(ig, off);
-        const long long oh = __shfl_up(ih, off);
-        const unsigned long long oc = __shfl_up(ic, off);
-        if (lane >= off) {
-          ig += og;
-          ih += oh;
-          ic += oc;
-        }
-      }
-      const long long eg = carry_g + ig - g4[3], eh = carry_h + ih - h4[3];
-      const unsigned long long ec = carry_c + ic - c4[3];
-#pragma unroll
-      for (int j = 0; j < 4; ++j) {
-        const int bin = chunk + lane * 4 + j;
-        if (bin < hist_size) {
-          const long long lg = eg + g4[j], lh = eh + h4[j];
-          const unsigned long long lc = ec + c4[j];
-          const double GL = FromFixed<F64>(lg, sg);
-          const double HL = PAIR ? FromFixed<F64>(lh, sh) : 0.0;
-          const float gn = SplitGain<PAIR, F64>(GL, HL, lc, GT, HT, t.c, gp);
-          if (gn > 0.0f && gn >= best.gain) {
-            best.gain = gn;
-            best.bin = bin;
-            best.left.g = lg;
-            best.left.h = lh;
-            best.left.c = lc;
-          }
-        }
-      }
-      carry_g += __shfl(ig, 63);
-      carry_h += __shfl(ih, 63);
-      carry_c += __shfl(ic, 63);
-    }
-    for (int off = 32; off > 0; off >>= 1) {
-      const float og = __shfl_down(best.gain, off);
-      const int ob = __shfl_down(best.bin, off);
-      const long long olg = __shfl_down(best.left.g, off);
-      const long long olh = __shfl_down(best.left.h, off);
-      const unsigned long long olc = __shfl_down(best.left.c, off);
-      if (ob >= 0 && (best.bin < 0 || og > best.gain || (og == best.gain && ob > best.bin))) {
-        best.gain = og;
-        best.bin = ob;
-        best.left.g = olg;
-        best.left.h = olh;
-        best.left.c = olc;
-      }
-    }
-  }
-  if (lane == 0) cand[(size_t)nd * F + f] = best;
-}
-
-// One thread per node: best candidate over the features active at this level
-// (higher gain, then lower feature id: hist_tree_grower.cu:59-60), children
-// totals and row ranges, node record.  A node without a candidate keeps every
-// row left.
-// One wave per node: lane l looks at features l, l + 64, ...; the wave keeps
-// the candidate with the highest gain, ties to the lowest feature id.
-__device__ __forceinline__ void SelectNode(int nd, int lane, const Cand *__restrict__ cand, int F,
-                                           const NodeSum *__restrict__ tot,
-                                           const unsigned *__restrict__ seg_start,
-                                           NodeSum *__restrict__ tot_next, unsigned *__restrict__ seg_next,
-                                           SplitRec *__restrict__ split, int *__restrict__ t_fid,
-                                           int *__restrict__ t_bin, float *__restrict__ t_gain, int heap_off,
-                                           const unsigned char *__restrict__ active) {
-  const NodeSum t = tot[nd];
-  float gain = 0.0f;
-  int fid = -1, bin = -1;
-  long long lg = 0, lh = 0;
-  unsigned long long lc = 0;
-  if (t.c != 0) {
-    for (int f = lane; f < F; f += 64) {
-      if (active && !active[f]) continue;  // feature not sampled at this level
-      const Cand c = cand[(size_t)nd * F + f];
-      if (c.bin >= 0 && (fid < 0 || gain < c.gain)) {
-        gain = c.gain;
-        fid = f;
-        bin = c.bin;
-        lg = c.left.g;
-        lh = c.left.h;
-        lc = c.left.c;
-      }
-    }
-  }
-  for (int off = 32; off > 0; off >>= 1) {
-    const float og = __shfl_down(gain, off);
-    const int of = __shfl_down(fid, off);
-    const int ob = __shfl_down(bin, off);
-    const long long olg = __shfl_down(lg, off);
-    const long long olh = __shfl_down(lh, off);
-    const unsigned long long olc = __shfl_down(lc, off);
-    if (of >= 0 && (fid < 0 || og > gain || (og == gain && of < fid))) {
-      gain = og;
-      fid = of;
-      bin = ob;
-      lg = olg;
-      lh = olh;
-      lc = olc;
-    }
-  }
-  if (lane != 0) return;
-  SplitRec rec;
-  rec.gain = fid < 0 ? 0.0f : gain;
-  rec.fid = fid;
-  rec.bin = fid < 0 ? -1 : bin;
-  rec.pad = 0;
-  rec.left = t;
-  if (fid >= 0) {
-    rec.left.g = lg;
-    rec.left.h = lh;
-    rec.left.c = lc;
-  }
-  split[nd] = rec;
-  NodeSum r;
-  r.g = t.g - rec.left.g;
-  r.h = t.h - rec.left.h;
-  r.c = t.c - rec.left.c;
-  tot_next[2 * nd] = rec.left;
-  tot_next[2 * nd + 1] = r;
-  const unsigned start = seg_start[nd];
-  seg_next[2 * nd] = start;
-  seg_next[2 * nd + 1] = start + (unsigned)rec.left.c;
-  t_fid[heap_off + nd] = rec.fid < 0 ? 0 : rec.fid;  // garden.cu:471-481
-  t_bin[heap_off + nd] = rec.fid < 0 ? -1 : rec.bin;
-  t_gain[heap_off + nd] = rec.gain;
-}
-
-// grid ceil(L / 16), 1024 threads: one wave per node
-__global__ void __launch_bounds__(1024)
-k_split_select(const Cand *__restrict__ cand, int F, int L, const NodeSum *__restrict__ tot,
-               const unsigned *__restrict__ seg_start, NodeSum *__restrict__ tot_next,
-               unsigned *__restrict__ seg_next, SplitRec *__restrict__ split, int *__restrict__ t_fid,
-               int *__restrict__ t_bin, float *__restrict__ t_gain, int heap_off,
-               const unsigned char *__restrict__ active) {
-  const int nd = blockIdx.x * 16 + (threadIdx.x >> 6);
-  if (nd < L)
-    SelectNode(nd, threadIdx.x & 63, cand, F, tot, seg_start, tot_next, seg_next, split, t_fid, t_bin, t_gain,
-               heap_off, active);
-}
-
-// k_split_select followed, in the same workgroup, by the work plan of the
-// fused pass over these nodes' rows (the plan needs the splits only for the
-// row statistics).  One workgroup of 1024 threads.
-__global__ void __launch_bounds__(1024)
-k_select_plan(const Cand *__restrict__ cand, int F, int L, const NodeSum *__restrict__ tot,
-              const unsigned *__restrict__ seg_start, NodeSum *__restrict__ tot_next,
-              unsigned *__restrict__ seg_next, SplitRec *__restrict__ split, int *__restrict__ t_fid,
-              int *__restrict__ t_bin, float *__restrict__ t_gain, int heap_off,
-              const unsigned char *__restrict__ active, unsigned rows_per_item,
-              WorkItem *__restrict__ work, unsigned *__restrict__ n_work,
-              unsigned *__restrict__ node_first, unsigned *__restrict__ node_items,
-              unsigned long long *__restrict__ rows_scanned, unsigned max_items,
-              unsigned *__restrict__ overflow) {
-  for (int nd = threadIdx.x >> 6; nd < L; nd += 16)
-    SelectNode(nd, threadIdx.x & 63, cand, F, tot, seg_start, tot_next, seg_next, split, t_fid, t_bin, t_gain,
-               heap_off, active);
-  __syncthreads();  // the splits written above are read by the plan
-  PlanBody(tot, seg_start, L, 0, rows_per_item, work, n_work, node_first, node_items, rows_scanned, split,
-           max_items, overflow);
-}
-
-// --------------------------------------------------------------- leaves
-// UpdateLeafWeight (garden.cu:487-503, split.cu:25-35): left = Weight(left
-// sum), right = Weight(parent - left) with the subtraction in the sum type.
-template <bool PAIR, bool F64>
-__global__ void k_leaf_weights(const SplitRec *__restrict__ split, const NodeSum *__restrict__ tot,
-                               int L, const int *__restrict__ shifts, GainParams gp, float eta,
-                               float *__restrict__ weights) {
-  const int nd = blockIdx.x * blockDim.x + threadIdx.x;
-  if (nd >= L) return;
-  const int sg = shifts[0], sh = shifts[1];
-  const SplitRec s = split[nd];
-  const NodeSum t = tot[nd];
-  const double GL = FromFixed<F64>(s.left.g, sg), HL = PAIR ? FromFixed<F64>(s.left.h, sh) : 0.0;
-  const double GP = FromFixed<F64>(t.g, sg), HP = PAIR ? FromFixed<F64>(t.h, sh) : 0.0;
-  double GR, HR;
-  if (F64) {
-    GR = GP - GL;
-    HR = HP - HL;
-  } else {
-    GR = (double)((float)GP - (float)GL);
-    HR = (double)((float)HP - (float)HL);
-  }
-  weights[2 * nd] = LeafWeight<PAIR, F64>(GL, HL, (unsigned)s.left.c, gp) * eta;
-  weights[2 * nd + 1] = LeafWeight<PAIR, F64>(GR, HR, (unsigned)(t.c - s.left.c), gp) * eta;
-}
-
-// End of a tree, rows in original order: walk the tree on the row's bins
-// (bin >= q+1 goes right, builder.h:107-123), record the leaf, add its weight
-// to y_hat (update_by_last_tree, garden.cu:45-76) and, when NEXT_GRAD is not
-// 0, write the gradients of the next round (objective.cu:28-56):
-// 1 = squared (also max |g|), 2 = logistic.
-// NQ > 0: the matrix has NQ quads, all loaded up front (coalesced, independent
-// loads) and selected in registers; NQ == 0: any width, one dependent 4-byte
-// load per level.
-template <int NEXT_GRAD, int NQ>
-__global__ void __launch_bounds__(256)
-k_final(const uint32_t *__restrict__ bins, size_t stride, const int *__restrict__ t_fid,
-        const int *__restrict__ t_bin, int depth, const float *__restrict__ weights,
-        float *__restrict__ yhat, const float *__restrict__ y, unsigned *__restrict__ leaf_of,
-        float *__restrict__ g, float *__restrict__ h, unsigned *__restrict__ gmax_bits, size_t n,
-        BinCode code) {
-  extern __shared__ int s_nodes[];  // fid[internal], bin[internal]
-  const int internal = (1 << (depth - 1)) - 1;
-  for (int i = threadIdx.x; i < internal; i += blockDim.x) {
-    s_nodes[i] = t_fid[i];
-    s_nodes[internal + i] = t_bin[i];
-  }
-  __syncthreads();
-  float m = 0.0f;
-  for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < n;
-       i += (size_t)gridDim.x * blockDim.x) {
-    uint32_t b[NQ > 0 ? NQ : 1];
-#pragma unroll
-    for (int q = 0; q < NQ; ++q) b[q] = __builtin_nontemporal_load(&bins[(size_t)q * stride + i]);
-    const float yh0 = yhat[i];
-    const float yv = NEXT_GRAD != 0 ? __builtin_nontemporal_load(&y[i]) : 0.0f;
-    unsigned node = 0;
-    for (int level = 0; level + 1 < depth; ++level) {
-      const int id = (1 << level) - 1 + (int)node;
-      const int fid = s_nodes[id], bin = s_nodes[internal + id];
-      unsigned right = 0;
-      if (bin >= 0) {
-        if (NQ > 0) {  // 8-bit bins, all quads in registers
-          uint32_t b4 = 0;
-          const int fq = fid >> 2;
-#pragma unroll
-          for (int q = 0; q < NQ; ++q) b4 = q == fq ? b[q] : b4;
-          right = (int)((b4 >> (8 * (fid & 3))) & 255u) > bin ? 1u : 0u;
-        } else {
-          right = (int)code.Bin(bins[(size_t)code.Word(fid) * stride + i], fid) > bin ? 1u : 0u;
-        }
-      }
-      node = node * 2 + right;
-    }
-    __builtin_nontemporal_store(node, &leaf_of[i]);
-    const float yh = yh0 + weights[node];
-    yhat[i] = yh;
-    if (NEXT_GRAD == 1) {
-      const float v = yv - yh;
-      g[i] = v;
-      const float a = fabsf(v);
-      if (a > m) m = a;
-    } else if (NEXT_GRAD == 2) {
-      const float s = SigmoidF(yh);
-      g[i] = yv - s;
-      h[i] = s * (1.0f - s);
-    }
-  }
-  if (NEXT_GRAD == 1) {
-    m = WaveMaxF(m);
-    if ((threadIdx.x & 63) == 0) atomicMax(gmax_bits, __float_as_uint(m));
-  }
-}
-
-// Last pass of a tree fused with the root histogram of the next one
-// (logistic objective, resident matrix, all quads in one LDS histogram): the
-// rows are read once; the leaf walk, the prediction update and the new
-// gradients are bound by HBM, the histogram by LDS atomics, and they overlap.
-// One workgroup per root work item; LDS: histogram, then the node arrays.
-template <int NQ>
-__global__ void __launch_bounds__(kHistThreads)
-k_final_hist(const uint32_t *__restrict__ bins, size_t stride, int F, const int *__restrict__ t_fid,
-             const int *__restrict__ t_bin, int depth, const float *__restrict__ weights,
-             float *__restrict__ yhat, const float *__restrict__ y, unsigned *__restrict__ leaf_of,
-             float *__restrict__ g, float *__restrict__ h, const int *__restrict__ shifts,
-             const WorkItem *__restrict__ work, const unsigned *__restrict__ n_work,
-             unsigned long long *__restrict__ slab, int slab_entries) {
-  extern __shared__ unsigned long long lds[];
-  const unsigned w = blockIdx.x;
-  if (w >= *n_work) return;
-  const WorkItem it = work[w];
-  constexpr int words = (int)(HistLdsBytes(NQ, true) / 8);
-  int *s_nodes = reinterpret_cast<int *>(lds + words);  // fid[internal], bin[internal]
-  const int internal = (1 << (depth - 1)) - 1;
-  for (int i = threadIdx.x; i < words; i += kHistThreads) lds[i] = 0ull;
-  for (int i = threadIdx.x; i < internal; i += kHistThreads) {
-    s_nodes[i] = t_fid[i];
-    s_nodes[internal + i] = t_bin[i];
-  }
-  __syncthreads();
-  const int sg = shifts[0], sh = shifts[1];
-  auto row = [&](const uint32_t (&b)[NQ], float p, float yv, unsigned r) {
-    unsigned node = 0;
-    for (int level = 0; level + 1 < depth; ++level) {
-      const int id = (1 << level) - 1 + (int)node;
-      const int fid = s_nodes[id], bin = s_nodes[internal + id];
-      unsigned right = 0;
-      if (bin >= 0) {
-        uint32_t b4 = 0;
-        const int fq = fid >> 2;
-#pragma unroll
-        for (int q = 0; q < NQ; ++q) b4 = q == fq ? b[q] : b4;
-        right = (int)((b4 >> (8 * (fid & 3))) & 255u) > bin ? 1u : 0u;
-      }
-      node = node * 2 + right;
-    }
-    __builtin_nontemporal_store(node, &leaf_of[r]);
-    const float yh = p + weights[node];
-    yhat[r] = yh;
-    const float s = SigmoidF(yh);
-    const float gv = yv - s, hv = s * (1.0f - s);
-    g[r] = gv;
-    h[r] = hv;
-    AccumulateRow<true, NQ>(lds, b, gv, hv, sg, sh, 0, F);
-  };
-  for (unsigned base = it.begin; base < it.end; base += 2 * kHistThreads) {
-    const unsigned r0 = base + threadIdx.x, r1 = r0 + kHistThreads;
-    const bool v0 = r0 < it.end, v1 = r1 < it.end;
-    const unsigned a0 = v0 ? r0 : it.begin, a1 = v1 ? r1 : it.begin;
-    uint32_t b0[NQ], b1[NQ];
-#pragma unroll
-    for (int q = 0; q < NQ; ++q) {
-      b0[q] = __builtin_nontemporal_load(&bins[(size_t)q * stride + a0]);
-      b1[q] = __builtin_nontemporal_load(&bins[(size_t)q * stride + a1]);
-    }
-    const float p0 = yhat[a0], p1 = yhat[a1];
-    const float y0 = __builtin_nontemporal_load(&y[a0]), y1 = __builtin_nontemporal_load(&y[a1]);
-    if (v0) row(b0, p0, y0, r0);
-    if (v1) row(b1, p1, y1, r1);
-  }
-  FlushSlab<true, NQ>(lds, slab, w, slab_entries, 0);
-}
-
-// Tree record of the tree just grown into one slot of the record ring:
-// fid[internal], bin[internal], gain[internal], weights[leaves], overflow flag.
-__global__ void k_pack_record(const int *__restrict__ t_fid, const int *__restrict__ t_bin,
-                              const float *__restrict__ t_gain, const float *__restrict__ weights,
-                              const unsigned *__restrict__ overflow, int internal, int leaves,
-                              uint32_t *__restrict__ out) {
-  const int i = blockIdx.x * blockDim.x + threadIdx.x;
-  if (i < internal) {
-    out[i] = (uint32_t)t_fid[i];
-    out[internal + i] = (uint32_t)t_bin[i];
-    out[2 * internal + i] = __float_as_uint(t_gain[i]);
-  }
-  if (i < leaves) out[3 * internal + i] = __float_as_uint(weights[i]);
-  if (i == 0) out[3 * internal + leaves] = *overflow;
-}
-
-__global__ void k_fill_f32(float *p, float v, size_t n) {
-  for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < n;
-       i += (size_t)gridDim.x * blockDim.x)
-    p[i] = v;
-}
-
-template <typename T>
-T *DevAlloc(size_t n) {
-  void *p = nullptr;
-  HIP_OK(hipMalloc(&p, std::max<size_t>(n, 1) * sizeof(T)));
-  return static_cast<T *>(p);
-}
-
-inline int GridFor(size_t n, int block, int cap = 4096) {
-  size_t g = (n + block - 1) / block;
-  return (int)std::max<size_t>(1, std::min<size_t>(g, cap));
-}
-
-}  // namespace
 
 struct DeviceMatrix {
   size_t rows = 0, stride = 0;

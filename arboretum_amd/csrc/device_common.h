@@ -1,0 +1,116 @@
+// Constants, records and helpers shared by the device kernels of the tree builder.
+#ifndef ARBORETUM_AMD_DEVICE_COMMON_H_
+#define ARBORETUM_AMD_DEVICE_COMMON_H_
+#include <hip/hip_runtime.h>
+
+#include <cstdint>
+#include <stdexcept>
+#include <string>
+
+#include "gain.h"
+
+namespace arb {
+namespace {
+
+#define HIP_OK(expr)                                                                        \
+  do {                                                                                      \
+    hipError_t e_ = (expr);                                                                 \
+    if (e_ != hipSuccess)                                                                   \
+      throw std::runtime_error(std::string("HIP error: ") + hipGetErrorString(e_) + " in " #expr); \
+  } while (0)
+
+constexpr int kSlots = 256;               // histogram slots per feature (uint8 bins)
+constexpr int kMaxWideSlots = 4096;       // histogram slots per feature with 16-bit bins (power of two)
+constexpr int kHistThreads = 1024;        // one workgroup per CU, 16 waves
+constexpr int kItemWaves = kHistThreads / 64;  // waves per work item in row passes
+constexpr unsigned kPartRows = 16384;     // rows per work item of the stand-alone partition
+constexpr int kMaxGroupQuads = 8;         // quads per histogram launch (compile-time variants, whole blocks)
+constexpr unsigned kMaxHistRows = 64512;  // rows per histogram work item (< 2^16)
+constexpr int kCountShift = 47;           // word0 = count << 47 | g
+constexpr int kMaxPlanNodes = 4096;       // nodes per level the planner handles
+constexpr size_t kLdsBudget = 160 * 1024;
+// LDS histograms are laid out in blocks of 16 features (4 quads):
+//   entry(f, bin) = (f / 16) * 4096 + bin * 16 + f % 16.
+// A 64-bit LDS atomic is executed 16 lanes per pass, and two of those lanes
+// collide when their addresses share a bank pair (entry % 16).  With this
+// layout the bank pair is the feature, and the kernels let the 16 lanes of a
+// pass work on 16 different features of their rows, so a pass never has a
+// bank conflict and never two lanes on one address, whatever the bin
+// distribution is (missing values, zeros, a dominant category).
+constexpr int kBlockFeatures = 16;
+constexpr int kBlockQuads = 4;
+constexpr int kBlockEntries = kBlockFeatures * kSlots;  // 4096
+constexpr int HistBlocks(int nq) { return (nq + kBlockQuads - 1) / kBlockQuads; }
+// LDS bytes of a histogram of nq quads
+constexpr size_t HistLdsBytes(int nq, bool pair) {
+  return (size_t)HistBlocks(nq) * kBlockEntries * 8 * (pair ? 2 : 1);
+}
+
+struct NodeSum {
+  long long g;
+  long long h;
+  unsigned long long c;
+};
+
+struct SplitRec {
+  float gain;
+  int fid;   // -1: not split (every row stays left)
+  int bin;
+  unsigned pad;
+  NodeSum left;
+};
+
+struct WorkItem {
+  unsigned node;
+  unsigned begin;  // row range in the current order
+  unsigned end;
+  unsigned first;  // index of the first work item of this node
+};
+
+// How bin ids are packed in the 32-bit words of a row: 8 bits (four features
+// per word) or 16 bits (two features per word).
+struct BinCode {
+  int wshift;  // feature -> word: fid >> wshift
+  int bits;
+  __host__ __device__ static BinCode Of(int bits) { return BinCode{bits == 8 ? 2 : 1, bits}; }
+  __device__ __forceinline__ int Word(int fid) const { return fid >> wshift; }
+  __device__ __forceinline__ unsigned Bin(uint32_t word, int fid) const {
+    return (word >> (bits * (fid & ((1 << wshift) - 1)))) & ((1u << bits) - 1u);
+  }
+};
+
+__device__ __forceinline__ float WaveMaxF(float v) {
+  for (int off = 32; off > 0; off >>= 1) v = fmaxf(v, __shfl_down(v, off));
+  return v;
+}
+__device__ __forceinline__ long long WaveSumLL(long long v) {
+  for (int off = 32; off > 0; off >>= 1) v += __shfl_down(v, off);
+  return v;
+}
+
+__global__ void k_init_root(NodeSum *tot, unsigned *seg_start, unsigned long long n,
+                            unsigned *gmax_bits) {  // gmax_bits may be NULL
+  if (threadIdx.x == 0 && blockIdx.x == 0) {
+    tot[0].g = 0;
+    tot[0].h = 0;
+    tot[0].c = n;
+    seg_start[0] = 0;
+    if (gmax_bits) *gmax_bits = 0;
+  }
+}
+
+__device__ __forceinline__ unsigned RankBelow(unsigned long long m) {
+  // number of set bits of m below this lane
+  return __builtin_amdgcn_mbcnt_hi((unsigned)(m >> 32), __builtin_amdgcn_mbcnt_lo((unsigned)m, 0u));
+}
+
+// Rows of a work item are dealt to its waves in chunks of kChunkRows
+// consecutive rows, round-robin: wave v takes chunks v, v + kItemWaves, ...  A
+// workgroup therefore streams one contiguous block of the item per step (good
+// DRAM page locality) while every wave still owns a fixed, countable row set.
+constexpr unsigned kChunkRows = 128;
+constexpr unsigned kChunkStep = kChunkRows * kItemWaves;
+
+}  // namespace
+}  // namespace arb
+#endif  // ARBORETUM_AMD_DEVICE_COMMON_H_

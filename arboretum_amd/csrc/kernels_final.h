@@ -1,0 +1,209 @@
+// Leaf weights, last pass of a tree (leaf ids, predictions, next gradients), probes.
+#ifndef ARBORETUM_AMD_KERNELS_FINAL_H_
+#define ARBORETUM_AMD_KERNELS_FINAL_H_
+#include "device_common.h"
+#include "kernels_hist.h"
+
+namespace arb {
+namespace {
+
+// --------------------------------------------------------------- leaves
+// UpdateLeafWeight (garden.cu:487-503, split.cu:25-35): left = Weight(left
+// sum), right = Weight(parent - left) with the subtraction in the sum type.
+template <bool PAIR, bool F64>
+__global__ void k_leaf_weights(const SplitRec *__restrict__ split, const NodeSum *__restrict__ tot,
+                               int L, const int *__restrict__ shifts, GainParams gp, float eta,
+                               float *__restrict__ weights) {
+  const int nd = blockIdx.x * blockDim.x + threadIdx.x;
+  if (nd >= L) return;
+  const int sg = shifts[0], sh = shifts[1];
+  const SplitRec s = split[nd];
+  const NodeSum t = tot[nd];
+  const double GL = FromFixed<F64>(s.left.g, sg), HL = PAIR ? FromFixed<F64>(s.left.h, sh) : 0.0;
+  const double GP = FromFixed<F64>(t.g, sg), HP = PAIR ? FromFixed<F64>(t.h, sh) : 0.0;
+  double GR, HR;
+  if (F64) {
+    GR = GP - GL;
+    HR = HP - HL;
+  } else {
+    GR = (double)((float)GP - (float)GL);
+    HR = (double)((float)HP - (float)HL);
+  }
+  weights[2 * nd] = LeafWeight<PAIR, F64>(GL, HL, (unsigned)s.left.c, gp) * eta;
+  weights[2 * nd + 1] = LeafWeight<PAIR, F64>(GR, HR, (unsigned)(t.c - s.left.c), gp) * eta;
+}
+
+// End of a tree, rows in original order: walk the tree on the row's bins
+// (bin >= q+1 goes right, builder.h:107-123), record the leaf, add its weight
+// to y_hat (update_by_last_tree, garden.cu:45-76) and, when NEXT_GRAD is not
+// 0, write the gradients of the next round (objective.cu:28-56):
+// 1 = squared (also max |g|), 2 = logistic.
+// NQ > 0: the matrix has NQ quads, all loaded up front (coalesced, independent
+// loads) and selected in registers; NQ == 0: any width, one dependent 4-byte
+// load per level.
+template <int NEXT_GRAD, int NQ>
+__global__ void __launch_bounds__(256)
+k_final(const uint32_t *__restrict__ bins, size_t stride, const int *__restrict__ t_fid,
+        const int *__restrict__ t_bin, int depth, const float *__restrict__ weights,
+        float *__restrict__ yhat, const float *__restrict__ y, unsigned *__restrict__ leaf_of,
+        float *__restrict__ g, float *__restrict__ h, unsigned *__restrict__ gmax_bits, size_t n,
+        BinCode code) {
+  extern __shared__ int s_nodes[];  // fid[internal], bin[internal]
+  const int internal = (1 << (depth - 1)) - 1;
+  for (int i = threadIdx.x; i < internal; i += blockDim.x) {
+    s_nodes[i] = t_fid[i];
+    s_nodes[internal + i] = t_bin[i];
+  }
+  __syncthreads();
+  float m = 0.0f;
+  for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < n;
+       i += (size_t)gridDim.x * blockDim.x) {
+    uint32_t b[NQ > 0 ? NQ : 1];
+#pragma unroll
+    for (int q = 0; q < NQ; ++q) b[q] = __builtin_nontemporal_load(&bins[(size_t)q * stride + i]);
+    const float yh0 = yhat[i];
+    const float yv = NEXT_GRAD != 0 ? __builtin_nontemporal_load(&y[i]) : 0.0f;
+    unsigned node = 0;
+    for (int level = 0; level + 1 < depth; ++level) {
+      const int id = (1 << level) - 1 + (int)node;
+      const int fid = s_nodes[id], bin = s_nodes[internal + id];
+      unsigned right = 0;
+      if (bin >= 0) {
+        if (NQ > 0) {  // 8-bit bins, all quads in registers
+          uint32_t b4 = 0;
+          const int fq = fid >> 2;
+#pragma unroll
+          for (int q = 0; q < NQ; ++q) b4 = q == fq ? b[q] : b4;
+          right = (int)((b4 >> (8 * (fid & 3))) & 255u) > bin ? 1u : 0u;
+        } else {
+          right = (int)code.Bin(bins[(size_t)code.Word(fid) * stride + i], fid) > bin ? 1u : 0u;
+        }
+      }
+      node = node * 2 + right;
+    }
+    __builtin_nontemporal_store(node, &leaf_of[i]);
+    const float yh = yh0 + weights[node];
+    yhat[i] = yh;
+    if (NEXT_GRAD == 1) {
+      const float v = yv - yh;
+      g[i] = v;
+      const float a = fabsf(v);
+      if (a > m) m = a;
+    } else if (NEXT_GRAD == 2) {
+      const float s = SigmoidF(yh);
+      g[i] = yv - s;
+      h[i] = s * (1.0f - s);
+    }
+  }
+  if (NEXT_GRAD == 1) {
+    m = WaveMaxF(m);
+    if ((threadIdx.x & 63) == 0) atomicMax(gmax_bits, __float_as_uint(m));
+  }
+}
+
+// Last pass of a tree fused with the root histogram of the next one
+// (logistic objective, resident matrix, all quads in one LDS histogram): the
+// rows are read once; the leaf walk, the prediction update and the new
+// gradients are bound by HBM, the histogram by LDS atomics, and they overlap.
+// One workgroup per root work item; LDS: histogram, then the node arrays.
+template <int NQ>
+__global__ void __launch_bounds__(kHistThreads)
+k_final_hist(const uint32_t *__restrict__ bins, size_t stride, int F, const int *__restrict__ t_fid,
+             const int *__restrict__ t_bin, int depth, const float *__restrict__ weights,
+             float *__restrict__ yhat, const float *__restrict__ y, unsigned *__restrict__ leaf_of,
+             float *__restrict__ g, float *__restrict__ h, const int *__restrict__ shifts,
+             const WorkItem *__restrict__ work, const unsigned *__restrict__ n_work,
+             unsigned long long *__restrict__ slab, int slab_entries) {
+  extern __shared__ unsigned long long lds[];
+  const unsigned w = blockIdx.x;
+  if (w >= *n_work) return;
+  const WorkItem it = work[w];
+  constexpr int words = (int)(HistLdsBytes(NQ, true) / 8);
+  int *s_nodes = reinterpret_cast<int *>(lds + words);  // fid[internal], bin[internal]
+  const int internal = (1 << (depth - 1)) - 1;
+  for (int i = threadIdx.x; i < words; i += kHistThreads) lds[i] = 0ull;
+  for (int i = threadIdx.x; i < internal; i += kHistThreads) {
+    s_nodes[i] = t_fid[i];
+    s_nodes[internal + i] = t_bin[i];
+  }
+  __syncthreads();
+  const int sg = shifts[0], sh = shifts[1];
+  auto row = [&](const uint32_t (&b)[NQ], float p, float yv, unsigned r) {
+    unsigned node = 0;
+    for (int level = 0; level + 1 < depth; ++level) {
+      const int id = (1 << level) - 1 + (int)node;
+      const int fid = s_nodes[id], bin = s_nodes[internal + id];
+      unsigned right = 0;
+      if (bin >= 0) {
+        uint32_t b4 = 0;
+        const int fq = fid >> 2;
+#pragma unroll
+        for (int q = 0; q < NQ; ++q) b4 = q == fq ? b[q] : b4;
+        right = (int)((b4 >> (8 * (fid & 3))) & 255u) > bin ? 1u : 0u;
+      }
+      node = node * 2 + right;
+    }
+    __builtin_nontemporal_store(node, &leaf_of[r]);
+    const float yh = p + weights[node];
+    yhat[r] = yh;
+    const float s = SigmoidF(yh);
+    const float gv = yv - s, hv = s * (1.0f - s);
+    g[r] = gv;
+    h[r] = hv;
+    AccumulateRow<true, NQ>(lds, b, gv, hv, sg, sh, 0, F);
+  };
+  for (unsigned base = it.begin; base < it.end; base += 2 * kHistThreads) {
+    const unsigned r0 = base + threadIdx.x, r1 = r0 + kHistThreads;
+    const bool v0 = r0 < it.end, v1 = r1 < it.end;
+    const unsigned a0 = v0 ? r0 : it.begin, a1 = v1 ? r1 : it.begin;
+    uint32_t b0[NQ], b1[NQ];
+#pragma unroll
+    for (int q = 0; q < NQ; ++q) {
+      b0[q] = __builtin_nontemporal_load(&bins[(size_t)q * stride + a0]);
+      b1[q] = __builtin_nontemporal_load(&bins[(size_t)q * stride + a1]);
+    }
+    const float p0 = yhat[a0], p1 = yhat[a1];
+    const float y0 = __builtin_nontemporal_load(&y[a0]), y1 = __builtin_nontemporal_load(&y[a1]);
+    if (v0) row(b0, p0, y0, r0);
+    if (v1) row(b1, p1, y1, r1);
+  }
+  FlushSlab<true, NQ>(lds, slab, w, slab_entries, 0);
+}
+
+// Tree record of the tree just grown into one slot of the record ring:
+// fid[internal], bin[internal], gain[internal], weights[leaves], overflow flag.
+__global__ void k_pack_record(const int *__restrict__ t_fid, const int *__restrict__ t_bin,
+                              const float *__restrict__ t_gain, const float *__restrict__ weights,
+                              const unsigned *__restrict__ overflow, int internal, int leaves,
+                              uint32_t *__restrict__ out) {
+  const int i = blockIdx.x * blockDim.x + threadIdx.x;
+  if (i < internal) {
+    out[i] = (uint32_t)t_fid[i];
+    out[internal + i] = (uint32_t)t_bin[i];
+    out[2 * internal + i] = __float_as_uint(t_gain[i]);
+  }
+  if (i < leaves) out[3 * internal + i] = __float_as_uint(weights[i]);
+  if (i == 0) out[3 * internal + leaves] = *overflow;
+}
+
+__global__ void k_fill_f32(float *p, float v, size_t n) {
+  for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < n;
+       i += (size_t)gridDim.x * blockDim.x)
+    p[i] = v;
+}
+
+template <typename T>
+T *DevAlloc(size_t n) {
+  void *p = nullptr;
+  HIP_OK(hipMalloc(&p, std::max<size_t>(n, 1) * sizeof(T)));
+  return static_cast<T *>(p);
+}
+
+inline int GridFor(size_t n, int block, int cap = 4096) {
+  size_t g = (n + block - 1) / block;
+  return (int)std::max<size_t>(1, std::min<size_t>(g, cap));
+}
+
+}  // namespace
+}  // namespace arb
+#endif  // ARBORETUM_AMD_KERNELS_FINAL_H_

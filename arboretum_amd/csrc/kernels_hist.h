@@ -1,0 +1,163 @@
+// LDS histograms: update order and layout, stand-alone histogram kernels.
+#ifndef ARBORETUM_AMD_KERNELS_HIST_H_
+#define ARBORETUM_AMD_KERNELS_HIST_H_
+#include "device_common.h"
+
+namespace arb {
+namespace {
+
+// ---------------------------------------------------------------- histogram
+// LDS layout of a histogram of NQ quads: word0 of every entry, then (PAIR)
+// word1 in the same order.
+template <int NQ>
+struct HistLds {
+  static constexpr int blocks = HistBlocks(NQ);
+  static constexpr int entries = blocks * kBlockEntries;
+  static constexpr int word1 = entries;  // offset of word1 of the same entry
+};
+
+// Adds one row per lane (bins of its NQ quads in b) to the LDS histogram.  The
+// 28 (or 4*NQ) updates of a row are issued in an order that depends on the
+// lane: in step (s, t) of a block, lane l works on quad (s + (l>>2)) % 4 and
+// byte (t + l) % 4 of that quad, so the 16 lanes of a pass of the LDS atomic
+// touch 16 different features = 16 different bank pairs.  q_first: first quad
+// of this launch (a multiple of 4).
+template <bool PAIR, int NQ>
+__device__ __forceinline__ void AccumulateRow(unsigned long long *__restrict__ lds,
+                                              const uint32_t (&b)[NQ], float gv, float hv, int sg,
+                                              int sh, int q_first, int F) {
+  using L = HistLds<NQ>;
+  const unsigned long long w0 = (1ull << kCountShift) + (unsigned long long)ToFixed(gv, sg);
+  unsigned long long w1 = 0;
+  if (PAIR) w1 = (unsigned long long)ToFixed(hv, sh);
+  const unsigned j = (threadIdx.x >> 2) & 3u, i = threadIdx.x & 3u;
+#pragma unroll
+  for (int k = 0; k < L::blocks; ++k) {
+    // quads of this block; the ones past NQ do not exist
+    uint32_t r[4];
+#pragma unroll
+    for (int x = 0; x < 4; ++x) r[x] = 4 * k + x < NQ ? b[4 * k + x < NQ ? 4 * k + x : 0] : 0u;
+#pragma unroll
+    for (int s_ = 0; s_ < 4; ++s_) {
+      const unsigned qi = ((unsigned)s_ + j) & 3u;  // quad of the block this lane works on
+      const uint32_t lo = (j & 1u) ? r[(s_ + 1) & 3] : r[s_];
+      const uint32_t hi = (j & 1u) ? r[(s_ + 3) & 3] : r[(s_ + 2) & 3];
+      const uint32_t sel = (j & 2u) ? hi : lo;
+#pragma unroll
+      for (int t = 0; t < 4; ++t) {
+        const unsigned bi = ((unsigned)t + i) & 3u;  // byte of the quad
+        const unsigned bin = (sel >> (8u * bi)) & 255u;
+        const unsigned f16 = 4u * qi + bi;
+        // Quads past NQ do not exist.  Padding features of the last quad of
+        // the matrix (bin 0 in every row) are accumulated like real ones into
+        // slots nobody reads: cheaper than a per-update test.
+        bool on = true;
+        if (4 * k + 3 >= NQ) on = 4u * k + qi < (unsigned)NQ;
+        if (on) {
+          const unsigned idx = (unsigned)(k * kBlockEntries) + bin * kBlockFeatures + f16;
+          atomicAdd(&lds[idx], w0);
+          if (PAIR) atomicAdd(&lds[L::word1 + idx], w1);
+        }
+      }
+    }
+  }
+}
+
+// Writes the LDS histogram to the slab of work item w in LDS order.  Called by
+// the whole workgroup after its last LDS update.  Slab layout per work item:
+// word0[slab_entries], word1[slab_entries]; q_first is a multiple of 4.
+template <bool PAIR, int NQ>
+__device__ __forceinline__ void FlushSlab(const unsigned long long *__restrict__ lds,
+                                          unsigned long long *__restrict__ slab, unsigned w,
+                                          int slab_entries, int q_first) {
+  using L = HistLds<NQ>;
+  __syncthreads();
+  unsigned long long *out =
+      slab + (size_t)w * slab_entries * (PAIR ? 2 : 1) + (size_t)(q_first / kBlockQuads) * kBlockEntries;
+  for (int e = threadIdx.x; e < L::entries; e += kHistThreads) {
+    out[e] = lds[e];
+    if (PAIR) out[slab_entries + e] = lds[L::word1 + e];
+  }
+}
+
+// Histogram of contiguous row ranges: one workgroup per work item, quads
+// [q0, q0+NQ).  LDS: NQ*1024 word0 entries, then (PAIR) as many word1 entries.
+template <bool PAIR, int NQ>
+__global__ void __launch_bounds__(kHistThreads)
+k_hist(const uint32_t *__restrict__ bins, size_t stride, int q0, int F,
+       const float *__restrict__ g, const float *__restrict__ h, const int *__restrict__ shifts,
+       const WorkItem *__restrict__ work, const unsigned *__restrict__ n_work,
+       unsigned long long *__restrict__ slab, int slab_entries) {
+  extern __shared__ unsigned long long lds[];
+  const unsigned w = blockIdx.x;
+  if (w >= *n_work) return;
+  const WorkItem it = work[w];
+  constexpr int words = (int)(HistLdsBytes(NQ, PAIR) / 8);
+  for (int i = threadIdx.x; i < words; i += kHistThreads) lds[i] = 0ull;
+  __syncthreads();
+  const int sg = shifts[0], sh = shifts[1];
+  const uint32_t *bq = bins + (size_t)q0 * stride;
+  for (unsigned base = it.begin; base < it.end; base += 2 * kHistThreads) {
+    const unsigned r0 = base + threadIdx.x, r1 = r0 + kHistThreads;
+    const bool v0 = r0 < it.end, v1 = r1 < it.end;
+    const unsigned a0 = v0 ? r0 : it.begin, a1 = v1 ? r1 : it.begin;
+    uint32_t b0[NQ], b1[NQ];
+#pragma unroll
+    for (int q = 0; q < NQ; ++q) {
+      b0[q] = __builtin_nontemporal_load(&bq[(size_t)q * stride + a0]);
+      b1[q] = __builtin_nontemporal_load(&bq[(size_t)q * stride + a1]);
+    }
+    const float g0 = g[a0], g1 = g[a1];
+    const float h0 = PAIR ? h[a0] : 0.0f, h1 = PAIR ? h[a1] : 0.0f;
+    if (v0) AccumulateRow<PAIR, NQ>(lds, b0, g0, h0, sg, sh, q0, F);
+    if (v1) AccumulateRow<PAIR, NQ>(lds, b1, g1, h1, sg, sh, q0, F);
+  }
+  FlushSlab<PAIR, NQ>(lds, slab, w, slab_entries, q0);
+}
+
+// Histogram of contiguous row ranges with 16-bit bins: features [f0, f0 + nf)
+// (f0 even), `slots` histogram slots per feature, LDS layout f * slots + bin,
+// word0 of every entry first, then (PAIR) word1.  The slab of a work item has
+// the same feature-major order: word0[slab_entries], word1[slab_entries].
+template <bool PAIR>
+__global__ void __launch_bounds__(kHistThreads)
+k_hist_wide(const uint32_t *__restrict__ bins, size_t stride, int f0, int nf, int slots,
+            const float *__restrict__ g, const float *__restrict__ h, const int *__restrict__ shifts,
+            const WorkItem *__restrict__ work, const unsigned *__restrict__ n_work,
+            unsigned long long *__restrict__ slab, int slab_entries) {
+  extern __shared__ unsigned long long lds[];
+  const unsigned w = blockIdx.x;
+  if (w >= *n_work) return;
+  const WorkItem it = work[w];
+  const int entries = nf * slots;
+  for (int i = threadIdx.x; i < entries * (PAIR ? 2 : 1); i += kHistThreads) lds[i] = 0ull;
+  __syncthreads();
+  const int sg = shifts[0], sh = shifts[1];
+  const int words = (nf + 1) / 2;
+  for (unsigned r = it.begin + threadIdx.x; r < it.end; r += kHistThreads) {
+    const unsigned long long w0 = (1ull << kCountShift) + (unsigned long long)ToFixed(g[r], sg);
+    unsigned long long w1 = 0;
+    if (PAIR) w1 = (unsigned long long)ToFixed(h[r], sh);
+    for (int k = 0; k < words; ++k) {
+      const uint32_t word = bins[(size_t)(f0 / 2 + k) * stride + r];
+      const unsigned lo = (unsigned)(2 * k) * slots + (word & 0xffffu);
+      atomicAdd(&lds[lo], w0);
+      if (PAIR) atomicAdd(&lds[entries + lo], w1);
+      if (2 * k + 1 < nf) {
+        const unsigned hi = (unsigned)(2 * k + 1) * slots + (word >> 16);
+        atomicAdd(&lds[hi], w0);
+        if (PAIR) atomicAdd(&lds[entries + hi], w1);
+      }
+    }
+  }
+  __syncthreads();
+  unsigned long long *out = slab + (size_t)w * slab_entries * (PAIR ? 2 : 1) + (size_t)f0 * slots;
+  for (int e = threadIdx.x; e < entries; e += kHistThreads) {
+    out[e] = lds[e];
+    if (PAIR) out[slab_entries + e] = lds[entries + e];
+  }
+}
+
+}  // namespace
+}  // namespace arb
+#endif  // ARBORETUM_AMD_KERNELS_HIST_H_

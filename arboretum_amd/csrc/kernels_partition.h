@@ -1,0 +1,586 @@
+// Row partition, the fused partition + histogram pass, slab reduction.
+#ifndef ARBORETUM_AMD_KERNELS_PARTITION_H_
+#define ARBORETUM_AMD_KERNELS_PARTITION_H_
+#include "device_common.h"
+#include "kernels_hist.h"
+#include "kernels_plan.h"
+
+namespace arb {
+namespace {
+
+// ---------------------------------------------------------------- partition
+__device__ __forceinline__ bool GoesRight(const uint32_t *__restrict__ bins, size_t stride,
+                                          const SplitRec &s, unsigned r, BinCode code = BinCode{2, 8}) {
+  // builder.h:107-123: bin >= q + 1 goes right
+  if (s.fid < 0) return false;
+  const uint32_t word = bins[(size_t)code.Word(s.fid) * stride + r];
+  return (int)code.Bin(word, s.fid) > s.bin;
+}
+
+// Rows going left, per (work item, wave range).
+__global__ void __launch_bounds__(kHistThreads)
+k_part_count(const uint32_t *__restrict__ bins, size_t stride, const SplitRec *__restrict__ split,
+             const WorkItem *__restrict__ work, const unsigned *__restrict__ n_work,
+             unsigned *__restrict__ wave_left, unsigned *__restrict__ item_left, BinCode code) {
+  const unsigned w = blockIdx.x;
+  if (w >= *n_work) return;
+  const WorkItem it = work[w];
+  const SplitRec s = split[it.node];
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  unsigned cnt = 0;
+  if (s.fid < 0) {
+    for (unsigned base = it.begin + wave * kChunkRows; base < it.end; base += kChunkStep)
+      cnt += lane == 0 ? min(kChunkRows, it.end - base) : 0u;
+  } else {
+    const uint32_t *col = bins + (size_t)code.Word(s.fid) * stride;
+    // eight chunks (16 loads) in flight per wave: the pass is latency-bound
+    constexpr int kBatch = 8;
+    for (unsigned base = it.begin + wave * kChunkRows; base < it.end; base += kBatch * kChunkStep) {
+      uint32_t v0[kBatch], v1[kBatch];
+#pragma unroll
+      for (int k = 0; k < kBatch; ++k) {
+        const unsigned r0 = base + k * kChunkStep + lane, r1 = r0 + 64;
+        v0[k] = col[min(r0, it.end - 1)];
+        v1[k] = col[min(r1, it.end - 1)];
+      }
+#pragma unroll
+      for (int k = 0; k < kBatch; ++k) {
+        const unsigned r0 = base + k * kChunkStep + lane, r1 = r0 + 64;
+        if (r0 < it.end) cnt += ((int)code.Bin(v0[k], s.fid) > s.bin) ? 0u : 1u;
+        if (r1 < it.end) cnt += ((int)code.Bin(v1[k], s.fid) > s.bin) ? 0u : 1u;
+      }
+    }
+  }
+  for (int off = 32; off > 0; off >>= 1) cnt += __shfl_down(cnt, off);
+  if (lane == 0) wave_left[(size_t)w * kItemWaves + wave] = cnt;
+  // per-item total for the offset computation of later items of the node
+  __shared__ unsigned s_cnt[kItemWaves];
+  if (lane == 0) s_cnt[wave] = cnt;
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    unsigned t = 0;
+    for (int k = 0; k < kItemWaves; ++k) t += s_cnt[k];
+    item_left[w] = t;
+  }
+}
+
+// Rows going left in the earlier work items of the same node and in the
+// earlier waves of this item.  Called by the whole workgroup; s_tmp holds
+// kItemWaves + 1 words.
+__device__ __forceinline__ unsigned LeftsBefore(const WorkItem &it, unsigned w, int wave,
+                                                const unsigned *__restrict__ wave_left,
+                                                const unsigned *__restrict__ item_left,
+                                                unsigned *s_tmp) {
+  unsigned part = 0;
+  for (unsigned k = it.first + threadIdx.x; k < w; k += blockDim.x) part += item_left[k];
+  for (int off = 32; off > 0; off >>= 1) part += __shfl_down(part, off);
+  if ((threadIdx.x & 63) == 0) s_tmp[threadIdx.x >> 6] = part;
+  __syncthreads();
+  unsigned before = 0;
+  for (int k = 0; k < kItemWaves; ++k) before += s_tmp[k];
+  for (int k = 0; k < wave; ++k) before += wave_left[(size_t)w * kItemWaves + k];
+  __syncthreads();
+  return before;
+}
+
+// Number of rows of a work item dealt to the waves before `wave`.
+__device__ __forceinline__ unsigned RowsOfEarlierWaves(const WorkItem &it, int wave) {
+  const unsigned rows = it.end - it.begin;
+  const unsigned full = rows / kChunkStep, rem = rows % kChunkStep;  // full rounds, rows of the last partial round
+  return full * kChunkRows * (unsigned)wave + min(rem, kChunkRows * (unsigned)wave);
+}
+
+// Destination offsets of one wave: its rows going left are packed in order
+// from the start of the parent's range (after those of earlier items and
+// waves), its rows going right from the start of the right child's range.
+__device__ __forceinline__ void WaveOffsets(const WorkItem &it, const SplitRec &s, unsigned start,
+                                            unsigned lefts_before, int wave, unsigned *lo, unsigned *ro) {
+  const unsigned rows_before = (it.begin - start) + RowsOfEarlierWaves(it, wave);
+  *lo = start + lefts_before;
+  *ro = start + (unsigned)s.left.c + rows_before - lefts_before;
+}
+
+// Position of the k-th (0-based) set bit of the wave-uniform mask m; k < popcount(m).
+__device__ __forceinline__ int SelectBit(unsigned long long m, unsigned k) {
+  const unsigned lo = (unsigned)m, hi = (unsigned)(m >> 32);
+  unsigned c = (unsigned)__popc(lo);
+  const bool up = k >= c;
+  unsigned word = up ? hi : lo;
+  int pos = up ? 32 : 0;
+  k = up ? k - c : k;
+#pragma unroll
+  for (int width = 16; width >= 1; width >>= 1) {
+    const unsigned low = word & ((1u << width) - 1u);
+    c = (unsigned)__popc(low);
+    const bool u = k >= c;
+    word = u ? (word >> width) : low;
+    pos += u ? width : 0;
+    k = u ? k - c : k;
+  }
+  return pos;
+}
+
+// Two rows per lane of a wave's 128-row chunk, as loaded.
+template <int NQ>
+struct RowSet {
+  uint32_t b0[NQ], b1[NQ];
+  uint32_t s0, s1;  // word of the split feature when it is not among b0/b1
+  float g0, g1, h0, h1;
+};
+
+// A wave's register-resident queue of rows on their way to one child's row
+// range: lane l holds the row whose destination is base + l, lanes [0, n) are
+// occupied, and on a wave's first batch lanes [0, skip) stand for the rows
+// before the wave's own range (base is a multiple of 64 rows, so every batch
+// is written as one aligned, fully coalesced 256-byte store per array).
+template <int NQ>
+struct RowQueue {
+  uint32_t b[NQ];
+  float g, h;
+  unsigned n, skip, base;
+  __device__ __forceinline__ void Init(unsigned first_row) {
+#pragma unroll
+    for (int q = 0; q < NQ; ++q) b[q] = 0;
+    g = h = 0.0f;
+    n = skip = first_row & 63u;
+    base = first_row - n;
+  }
+};
+
+// Writes lanes [from, to) of Q to their destination and, for the child whose
+// histogram is built, adds them to the LDS histogram.
+// HIST: the kernel builds a histogram; GH: the gradients move with the rows.
+template <bool PAIR, int NQ, bool HIST = true, bool GH = true>
+__device__ __forceinline__ void EmitRows(unsigned long long *__restrict__ lds, const RowQueue<NQ> &Q,
+                                         unsigned from, unsigned to, bool built,
+                                         uint32_t *__restrict__ bins_out, size_t stride,
+                                         float *__restrict__ g_out, float *__restrict__ h_out, int lane,
+                                         int sg, int sh, int F) {
+  if ((unsigned)lane >= from && (unsigned)lane < to) {
+    // streaming stores and loads: the pass touches every byte once
+    const unsigned d = Q.base + (unsigned)lane;
+#pragma unroll
+    for (int q = 0; q < NQ; ++q) __builtin_nontemporal_store(Q.b[q], &bins_out[(size_t)q * stride + d]);
+    if (GH && g_out != nullptr) {  // a group pass after the first leaves the gradients alone
+      __builtin_nontemporal_store(Q.g, &g_out[d]);
+      if (PAIR) __builtin_nontemporal_store(Q.h, &h_out[d]);
+    }
+    if (HIST && built) AccumulateRow<PAIR, NQ>(lds, Q.b, Q.g, Q.h, sg, sh, 0, F);
+  }
+}
+
+// Appends the rows of X flagged in xm (wave-uniform mask, one row per lane) to
+// Q in row order with one lane permute per register; a full queue is emitted
+// and the rest of X starts the next batch.
+template <bool PAIR, int NQ, bool HIST = true, bool GH = true>
+__device__ __forceinline__ void MergeRows(unsigned long long *__restrict__ lds, RowQueue<NQ> &Q,
+                                          const uint32_t (&xb)[NQ], float xg, float xh,
+                                          unsigned long long xm, bool built,
+                                          uint32_t *__restrict__ bins_out, size_t stride,
+                                          float *__restrict__ g_out, float *__restrict__ h_out, int lane,
+                                          int sg, int sh, int F) {
+  const unsigned nx = (unsigned)__popcll(xm);
+  if (nx == 0) return;  // wave-uniform
+  // lane l receives the k-th flagged row, k = (l - n) mod 64: lanes >= n fill
+  // the current batch, lanes < n hold what overflows into the next one
+  const unsigned k = ((unsigned)lane - Q.n) & 63u;
+  const int src = SelectBit(xm, k < nx ? k : 0u);
+  uint32_t vb[NQ];
+#pragma unroll
+  for (int q = 0; q < NQ; ++q) vb[q] = (uint32_t)__shfl((int)xb[q], src);
+  const float vg = GH ? __shfl(xg, src) : 0.0f;
+  const float vh = GH && PAIR ? __shfl(xh, src) : 0.0f;
+  if (Q.n + nx >= 64u) {  // wave-uniform: the batch is complete
+    const bool fill = (unsigned)lane >= Q.n;
+#pragma unroll
+    for (int q = 0; q < NQ; ++q) Q.b[q] = fill ? vb[q] : Q.b[q];
+    Q.g = fill ? vg : Q.g;
+    Q.h = fill ? vh : Q.h;
+    EmitRows<PAIR, NQ, HIST, GH>(lds, Q, Q.skip, 64u, built, bins_out, stride, g_out, h_out, lane, sg, sh, F);
+    Q.base += 64u;
+    Q.skip = 0u;
+#pragma unroll
+    for (int q = 0; q < NQ; ++q) Q.b[q] = vb[q];
+    Q.g = vg;
+    Q.h = vh;
+    Q.n = Q.n + nx - 64u;
+  } else {
+    const bool fill = (unsigned)lane >= Q.n && k < nx;
+#pragma unroll
+    for (int q = 0; q < NQ; ++q) Q.b[q] = fill ? vb[q] : Q.b[q];
+    Q.g = fill ? vg : Q.g;
+    Q.h = fill ? vh : Q.h;
+    Q.n += nx;
+  }
+}
+
+// Fused pass over the rows of the parent nodes of a level: stable partition
+// into the children order (WRITE) and histogram of the smaller child of every
+// split in LDS.  Each wave owns the 128-row chunks v, v + 16, ... of the item
+// and runs without workgroup barriers.  With WRITE the rows of a chunk are
+// sorted into two register queues (one per child) with lane permutes; a full
+// queue is one aligned 64-row store per array, and the queue of the built
+// child is added to the histogram as a full wave (LDS atomic instructions
+// cost the same with one active lane as with 64).  Writing each chunk's rows
+// directly, as two short unaligned runs per store, costs 40 % more time than
+// the copy itself.  On the last level only the quad of the split feature is
+// read for every row; the selected rows are queued by row id and read 64 at a
+// time.  NQ = all quads of the matrix.
+// GROUP: `bins` / `bins_out` point at quad q0 of a wider matrix (q0 a multiple
+// of 4); the quad of the split feature is read from `split_bins`, the start of
+// the whole matrix, and g_out may be null (the gradients moved with an
+// earlier group of the same level).
+template <bool PAIR, int NQ, bool WRITE, bool GROUP = false>
+__global__ void __launch_bounds__(kHistThreads)
+k_part_hist(const uint32_t *__restrict__ bins, uint32_t *__restrict__ bins_out, size_t stride, int F,
+            const float *__restrict__ g, float *__restrict__ g_out, const float *__restrict__ h,
+            float *__restrict__ h_out, const int *__restrict__ shifts,
+            const SplitRec *__restrict__ split, const NodeSum *__restrict__ tot,
+            const unsigned *__restrict__ seg_start, const WorkItem *__restrict__ work,
+            const unsigned *__restrict__ n_work, const unsigned *__restrict__ wave_left,
+            const unsigned *__restrict__ item_left, unsigned long long *__restrict__ slab,
+            int slab_entries, const uint32_t *__restrict__ split_bins, int q0) {
+  extern __shared__ unsigned long long lds[];
+  __shared__ unsigned s_tmp[kItemWaves + 1];
+  const unsigned w = blockIdx.x;
+  if (w >= *n_work) return;
+  const WorkItem it = work[w];
+  const SplitRec s = split[it.node];
+  const unsigned long long cl = s.left.c, cr = tot[it.node].c - cl;
+  const bool build_right = cl > cr;  // ties -> left (hist_grad_sum.cu:288-290)
+  constexpr int words = (int)(HistLdsBytes(NQ, PAIR) / 8);
+  for (int i = threadIdx.x; i < words; i += kHistThreads) lds[i] = 0ull;
+  const int sg = shifts[0], sh = shifts[1];
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const unsigned wb = it.begin + wave * kChunkRows, we = it.end;
+  unsigned lo = 0, ro = 0;
+  if (WRITE) {
+    const unsigned before = LeftsBefore(it, w, wave, wave_left, item_left, s_tmp);
+    WaveOffsets(it, s, seg_start[it.node], before, wave, &lo, &ro);
+  }
+  __syncthreads();
+  const int fq = s.fid >> 2, fs = 8 * (s.fid & 3);
+  if constexpr (WRITE) {
+    // QB: rows of the child whose histogram is built, QO: the other child
+    RowQueue<NQ> QB, QO;
+    QB.Init(build_right ? ro : lo);
+    QO.Init(build_right ? lo : ro);
+    // Two register sets of 128 rows each: while one is processed the other is
+    // in flight.  The loads are unconditional (addresses clamped to the last
+    // row of the item) and the sets are never copied, so every wait in the loop
+    // is for exactly the set that is needed next.
+    const uint32_t *split_col = split_bins + (size_t)(s.fid < 0 ? 0 : fq) * stride;
+    auto load = [&](RowSet<NQ> &R, unsigned base) {
+      const unsigned a0 = min(base + lane, we - 1), a1 = min(base + 64 + lane, we - 1);
+#pragma unroll
+      for (int q = 0; q < NQ; ++q) {
+        R.b0[q] = __builtin_nontemporal_load(&bins[(size_t)q * stride + a0]);
+        R.b1[q] = __builtin_nontemporal_load(&bins[(size_t)q * stride + a1]);
+      }
+      if (GROUP) {  // the quad of the split feature, wherever it lives
+        R.s0 = split_col[a0];
+        R.s1 = split_col[a1];
+      }
+      R.g0 = __builtin_nontemporal_load(&g[a0]);
+      R.g1 = __builtin_nontemporal_load(&g[a1]);
+      R.h0 = PAIR ? __builtin_nontemporal_load(&h[a0]) : 0.0f;
+      R.h1 = PAIR ? __builtin_nontemporal_load(&h[a1]) : 0.0f;
+    };
+    auto process = [&](const RowSet<NQ> &R, unsigned base) {
+      const unsigned r0 = base + lane, r1 = r0 + 64;
+      const bool v0 = r0 < we, v1 = r1 < we;
+      uint32_t s0 = 0, s1 = 0;
+      if (GROUP) {
+        s0 = R.s0;
+        s1 = R.s1;
+      } else {
+#pragma unroll
+        for (int q = 0; q < NQ; ++q) {
+          s0 = q == fq ? R.b0[q] : s0;
+          s1 = q == fq ? R.b1[q] : s1;
+        }
+      }
+      const bool right0 = v0 && s.fid >= 0 && (int)((s0 >> fs) & 255u) > s.bin;
+      const bool right1 = v1 && s.fid >= 0 && (int)((s1 >> fs) & 255u) > s.bin;
+      const unsigned long long b0 = __ballot(v0 && right0 == build_right), o0 = __ballot(v0 && right0 != build_right);
+      const unsigned long long b1 = __ballot(v1 && right1 == build_right), o1 = __ballot(v1 && right1 != build_right);
+      MergeRows<PAIR, NQ>(lds, QO, R.b0, R.g0, R.h0, o0, false, bins_out, stride, g_out, h_out, lane, sg, sh, F);
+      MergeRows<PAIR, NQ>(lds, QB, R.b0, R.g0, R.h0, b0, true, bins_out, stride, g_out, h_out, lane, sg, sh, F);
+      MergeRows<PAIR, NQ>(lds, QO, R.b1, R.g1, R.h1, o1, false, bins_out, stride, g_out, h_out, lane, sg, sh, F);
+      MergeRows<PAIR, NQ>(lds, QB, R.b1, R.g1, R.h1, b1, true, bins_out, stride, g_out, h_out, lane, sg, sh, F);
+    };
+    if (wb < we) {
+      RowSet<NQ> A, B;
+      load(A, wb);
+      for (unsigned base = wb;; base += 2 * kChunkStep) {
+        load(B, base + kChunkStep);
+        process(A, base);
+        if (base + kChunkStep >= we) break;  // wave-uniform
+        load(A, base + 2 * kChunkStep);
+        process(B, base + kChunkStep);
+        if (base + 2 * kChunkStep >= we) break;
+      }
+    }
+    EmitRows<PAIR, NQ>(lds, QO, QO.skip, QO.n, false, bins_out, stride, g_out, h_out, lane, sg, sh, F);
+    EmitRows<PAIR, NQ>(lds, QB, QB.skip, QB.n, true, bins_out, stride, g_out, h_out, lane, sg, sh, F);
+  } else {
+    // Rows selected for the histogram are queued by row id (slot 64 * j + lane
+    // of the queue is lane `lane` of q[j]; slots [0, np) are occupied) and read
+    // again 64 at a time: LDS atomic instructions cost the same with one active
+    // lane as with 64, so only full waves are accumulated.  The second read
+    // hits the cache, is requested at the start of a chunk and used at its end,
+    // and the wave never waits for its LDS atomics.
+    unsigned q0 = it.begin, q1 = it.begin, q2 = it.begin;
+    unsigned np = 0;
+    uint32_t gb[NQ];
+    float gg = 0.0f, gh = 0.0f;
+    auto gather = [&](bool valid) {  // requests the rows of queue slots [0, 64)
+      const unsigned a = valid ? q0 : it.begin;
+#pragma unroll
+      for (int q = 0; q < NQ; ++q) gb[q] = bins[(size_t)q * stride + a];
+      gg = g[a];
+      gh = PAIR ? h[a] : 0.0f;
+      q0 = q1;
+      q1 = q2;
+    };
+    // m: wave-uniform mask of the selected rows among base + [0, 64); np < 128
+    auto enqueue = [&](unsigned base, unsigned long long m) {
+      const unsigned nx = (unsigned)__popcll(m);
+      if (nx == 0) return;
+      const unsigned r = np & 63u, j = np >> 6;
+      const unsigned k = ((unsigned)lane - r) & 63u;  // slot np + k
+      const unsigned id = base + (unsigned)SelectBit(m, k < nx ? k : 0u);
+      const bool here = (unsigned)lane >= r && k < nx;   // lands in q[j]
+      const bool next = (unsigned)lane < r && k < nx;    // lands in q[j + 1]
+      q0 = (j == 0 && here) ? id : q0;
+      q1 = ((j == 1 && here) || (j == 0 && next)) ? id : q1;
+      q2 = (j == 1 && next) ? id : q2;
+      np += nx;
+    };
+    // after a chunk: at most 127 rows stay queued
+    auto drain = [&](unsigned limit) {
+      while (np > limit) {
+        const unsigned take = min(np, 64u);
+        const bool valid = (unsigned)lane < take;
+        gather(valid);
+        if (valid) AccumulateRow<PAIR, NQ>(lds, gb, gg, gh, sg, sh, 0, F);
+        np -= take;
+      }
+    };
+    if (wb < we) {
+      // last level: only the quad of the split feature decides; the selected
+      // rows are read when they are accumulated
+      const uint32_t *col = split_bins + (size_t)(s.fid < 0 ? 0 : fq) * stride;
+      auto step = [&](uint32_t s0, uint32_t s1, uint32_t &n0, uint32_t &n1, unsigned base) {
+        const bool full = np >= 64u;  // wave-uniform
+        if (full) {
+          gather(true);
+          np -= 64u;
+        }
+        n0 = col[min(base + kChunkStep + lane, we - 1)];
+        n1 = col[min(base + kChunkStep + 64 + lane, we - 1)];
+        const unsigned r0 = base + lane, r1 = r0 + 64;
+        const bool v0 = r0 < we, v1 = r1 < we;
+        const bool right0 = v0 && s.fid >= 0 && (int)((s0 >> fs) & 255u) > s.bin;
+        const bool right1 = v1 && s.fid >= 0 && (int)((s1 >> fs) & 255u) > s.bin;
+        enqueue(base, __ballot(v0 && right0 == build_right));
+        enqueue(base + 64, __ballot(v1 && right1 == build_right));
+        if (full) AccumulateRow<PAIR, NQ>(lds, gb, gg, gh, sg, sh, 0, F);
+        drain(127u);
+      };
+      uint32_t a0 = col[min(wb + lane, we - 1)], a1 = col[min(wb + 64 + lane, we - 1)], b0, b1;
+      for (unsigned base = wb;; base += 2 * kChunkStep) {
+        step(a0, a1, b0, b1, base);
+        if (base + kChunkStep >= we) break;  // wave-uniform
+        step(b0, b1, a0, a1, base + kChunkStep);
+        if (base + 2 * kChunkStep >= we) break;
+      }
+    }
+    drain(0u);
+  }
+  FlushSlab<PAIR, NQ>(lds, slab, w, slab_entries, q0);
+}
+
+// Stable partition alone (matrices too wide for the fused pass, 16-bit bins):
+// words [q0, q0 + NQ) of every row, and with GH the gradients, go to the
+// children order through the two register queues of the fused pass.  One launch
+// per group of words; every launch reads the word of the split feature again.
+template <bool PAIR, int NQ, bool GH>
+__global__ void __launch_bounds__(kHistThreads)
+k_part_rows(const uint32_t *__restrict__ bins, uint32_t *__restrict__ bins_out, size_t stride, int q0,
+            const float *__restrict__ g, float *__restrict__ g_out, const float *__restrict__ h,
+            float *__restrict__ h_out, const SplitRec *__restrict__ split,
+            const unsigned *__restrict__ seg_start, const WorkItem *__restrict__ work,
+            const unsigned *__restrict__ n_work, const unsigned *__restrict__ wave_left,
+            const unsigned *__restrict__ item_left, BinCode code) {
+  __shared__ unsigned s_tmp[kItemWaves + 1];
+  const unsigned w = blockIdx.x;
+  if (w >= *n_work) return;
+  const WorkItem it = work[w];
+  const SplitRec s = split[it.node];
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const unsigned wb = it.begin + wave * kChunkRows, we = it.end;
+  unsigned lo, ro;
+  const unsigned before = LeftsBefore(it, w, wave, wave_left, item_left, s_tmp);
+  WaveOffsets(it, s, seg_start[it.node], before, wave, &lo, &ro);
+  if (wb >= we) return;
+  const uint32_t *group = bins + (size_t)q0 * stride;
+  uint32_t *group_out = bins_out + (size_t)q0 * stride;
+  const uint32_t *split_col = bins + (size_t)(s.fid < 0 ? 0 : code.Word(s.fid)) * stride;
+  RowQueue<NQ> QL, QR;
+  QL.Init(lo);
+  QR.Init(ro);
+  struct Rows {
+    RowSet<NQ> r;
+    uint32_t s0, s1;  // word of the split feature
+  };
+  auto load = [&](Rows &R, unsigned base) {
+    const unsigned a0 = min(base + lane, we - 1), a1 = min(base + 64 + lane, we - 1);
+#pragma unroll
+    for (int q = 0; q < NQ; ++q) {
+      R.r.b0[q] = __builtin_nontemporal_load(&group[(size_t)q * stride + a0]);
+      R.r.b1[q] = __builtin_nontemporal_load(&group[(size_t)q * stride + a1]);
+    }
+    R.s0 = split_col[a0];
+    R.s1 = split_col[a1];
+    R.r.g0 = GH ? __builtin_nontemporal_load(&g[a0]) : 0.0f;
+    R.r.g1 = GH ? __builtin_nontemporal_load(&g[a1]) : 0.0f;
+    R.r.h0 = GH && PAIR ? __builtin_nontemporal_load(&h[a0]) : 0.0f;
+    R.r.h1 = GH && PAIR ? __builtin_nontemporal_load(&h[a1]) : 0.0f;
+  };
+  auto process = [&](const Rows &R, unsigned base) {
+    const unsigned r0 = base + lane, r1 = r0 + 64;
+    const bool v0 = r0 < we, v1 = r1 < we;
+    const bool right0 = v0 && s.fid >= 0 && (int)code.Bin(R.s0, s.fid) > s.bin;
+    const bool right1 = v1 && s.fid >= 0 && (int)code.Bin(R.s1, s.fid) > s.bin;
+    const unsigned long long lm0 = __ballot(v0 && !right0), rm0 = __ballot(right0);
+    const unsigned long long lm1 = __ballot(v1 && !right1), rm1 = __ballot(right1);
+    MergeRows<PAIR, NQ, false, GH>(nullptr, QL, R.r.b0, R.r.g0, R.r.h0, lm0, false, group_out, stride, g_out, h_out, lane, 0, 0, 0);
+    MergeRows<PAIR, NQ, false, GH>(nullptr, QR, R.r.b0, R.r.g0, R.r.h0, rm0, false, group_out, stride, g_out, h_out, lane, 0, 0, 0);
+    MergeRows<PAIR, NQ, false, GH>(nullptr, QL, R.r.b1, R.r.g1, R.r.h1, lm1, false, group_out, stride, g_out, h_out, lane, 0, 0, 0);
+    MergeRows<PAIR, NQ, false, GH>(nullptr, QR, R.r.b1, R.r.g1, R.r.h1, rm1, false, group_out, stride, g_out, h_out, lane, 0, 0, 0);
+  };
+  Rows A, B;
+  load(A, wb);
+  for (unsigned base = wb;; base += 2 * kChunkStep) {
+    load(B, base + kChunkStep);
+    process(A, base);
+    if (base + kChunkStep >= we) break;  // wave-uniform
+    load(A, base + 2 * kChunkStep);
+    process(B, base + kChunkStep);
+    if (base + 2 * kChunkStep >= we) break;
+  }
+  EmitRows<PAIR, NQ, false, GH>(nullptr, QL, QL.skip, QL.n, false, group_out, stride, g_out, h_out, lane, 0, 0, 0);
+  EmitRows<PAIR, NQ, false, GH>(nullptr, QR, QR.skip, QR.n, false, group_out, stride, g_out, h_out, lane, 0, 0, 0);
+}
+
+// Adds the slabs of every directly built node of a level (on top of the stored
+// histogram when `accumulate`) and, with `trick`, derives its sibling as
+// parent - node.  Slabs are in LDS order (16-feature blocks, bin-major); the
+// histograms written here are feature-major: hist[node][f * 256 + bin].
+// grid (slab_entries/64, L), 1024 threads = 64 entries x 16 slab lanes.
+//   by_parent = 0: slabs belong to work items of the node itself
+//               (node_items == 0xffffffff marks a derived node);
+//   by_parent = 1: slabs belong to work items of the parent (fused pass); the
+//               built child is the smaller one, ties -> left.
+template <bool PAIR, int LANES>
+__global__ void __launch_bounds__(1024)
+k_hist_reduce(const unsigned long long *__restrict__ slab, int slab_entries, int nbin_total,
+              const unsigned *__restrict__ node_first, const unsigned *__restrict__ node_items,
+              int by_parent, const SplitRec *__restrict__ parent_split,
+              const NodeSum *__restrict__ parent_tot, long long *__restrict__ hg,
+              long long *__restrict__ hh, unsigned *__restrict__ hc,
+              const long long *__restrict__ pg, const long long *__restrict__ ph,
+              const unsigned *__restrict__ pc, int trick, int accumulate, int plain) {
+  // LANES threads share the slabs of one entry; a block covers 1024 / LANES
+  // consecutive entries (with 4 lanes: 16 bins x 16 features, so the
+  // feature-major output is written in runs of 16 bins)
+  constexpr int kEntries = 1024 / LANES;
+  __shared__ long long s_g[LANES][kEntries];
+  __shared__ long long s_h[LANES][kEntries];
+  __shared__ unsigned s_c[LANES][kEntries];
+  const int nd = blockIdx.y;
+  unsigned items, first;
+  if (by_parent) {
+    const int p = nd >> 1;
+    const unsigned long long cl = parent_split[p].left.c, cr = parent_tot[p].c - cl;
+    const bool build_right = cl > cr;
+    if (((nd & 1) != 0) != build_right) return;  // derived from its sibling
+    items = node_items[p];
+    first = node_first[p];
+  } else {
+    items = node_items[nd];
+    first = node_first[nd];
+    if (items == 0xffffffffu) return;  // derived from its sibling
+  }
+  const int e = threadIdx.x % kEntries, lane = threadIdx.x / kEntries;
+  const int entry = blockIdx.x * kEntries + e;  // slab order
+  // plain: the slabs are feature-major already (16-bit bins)
+  const int f = (entry / kBlockEntries) * kBlockFeatures + (entry & (kBlockFeatures - 1));
+  const int bin = (entry / kBlockFeatures) & (kSlots - 1);
+  // the last 16-feature block may have fewer than 16 features
+  const bool live = plain ? entry < nbin_total : f * kSlots < nbin_total;
+  long long ag = 0, ah = 0;
+  unsigned ac = 0;
+  if (live) {
+    for (unsigned s = lane; s < items; s += LANES) {
+      const unsigned long long *p = slab + (size_t)(first + s) * slab_entries * (PAIR ? 2 : 1);
+      const unsigned long long w0 = p[entry];
+      const long long gq = ((long long)(w0 << (64 - kCountShift))) >> (64 - kCountShift);
+      ag += gq;
+      ac += (unsigned)((w0 - (unsigned long long)gq) >> kCountShift);
+      if (PAIR) ah += (long long)p[slab_entries + entry];
+    }
+  }
+  s_g[lane][e] = ag;
+  s_h[lane][e] = ah;
+  s_c[lane][e] = ac;
+  __syncthreads();
+  if (lane == 0 && live) {
+    for (int k = 1; k < LANES; ++k) {
+      ag += s_g[k][e];
+      ah += s_h[k][e];
+      ac += s_c[k][e];
+    }
+    const size_t cell = plain ? (size_t)entry : (size_t)f * kSlots + bin;
+    const size_t o = (size_t)nd * nbin_total + cell;
+    if (accumulate) {  // streamed matrices: one call per row block
+      ag += hg[o];
+      ah += hh[o];
+      ac += hc[o];
+    }
+    hg[o] = ag;
+    hh[o] = ah;
+    hc[o] = ac;
+    if (trick) {
+      const size_t po = (size_t)(nd >> 1) * nbin_total + cell;
+      const size_t so = (size_t)(nd ^ 1) * nbin_total + cell;
+      hg[so] = pg[po] - ag;
+      hh[so] = ph[po] - ah;
+      hc[so] = pc[po] - ac;
+    }
+  }
+}
+
+// Root totals = sum over the slots of feature 0 of the root histogram (every
+// row, NaN included, sits in exactly one slot).  Replaces the reduction over
+// the gradient array of garden.cu:432-435.  One wave.
+__global__ void __launch_bounds__(64)
+k_root_from_hist(const long long *__restrict__ hg, const long long *__restrict__ hh,
+                 NodeSum *__restrict__ tot, int slots) {
+  long long a = 0, b = 0;
+  for (int i = threadIdx.x; i < slots; i += 64) {
+    a += hg[i];
+    b += hh[i];
+  }
+  a = WaveSumLL(a);
+  b = WaveSumLL(b);
+  if (threadIdx.x == 0) {
+    tot[0].g = a;
+    tot[0].h = b;
+  }
+}
+
+}  // namespace
+}  // namespace arb
+#endif  // ARBORETUM_AMD_KERNELS_PARTITION_H_

@@ -1,0 +1,117 @@
+// Work planning on the device: row ranges of nodes cut into work items.
+#ifndef ARBORETUM_AMD_KERNELS_PLAN_H_
+#define ARBORETUM_AMD_KERNELS_PLAN_H_
+#include "device_common.h"
+
+namespace arb {
+namespace {
+
+// ------------------------------------------------------------------ planner
+// Splits the row ranges of the selected nodes of a level into work items of
+// at most `rows_per_item` rows.  select: 0 = every node, 1 = the smaller
+// child of each sibling pair, ties -> left (hist_grad_sum.cu:279-294).
+// rows_scanned (optional) is advanced by the rows that will be accumulated
+// into histograms: the selected rows, or, when `split` is given (fused
+// partition + histogram over parent nodes), the smaller side of every split.
+// One workgroup.
+__device__ __forceinline__ void PlanBody(const NodeSum *__restrict__ tot, const unsigned *__restrict__ seg_start,
+                                         int L, int select, unsigned rows_per_item,
+                                         WorkItem *__restrict__ work, unsigned *__restrict__ n_work,
+                                         unsigned *__restrict__ node_first, unsigned *__restrict__ node_items,
+                                         unsigned long long *__restrict__ rows_scanned,
+                                         const SplitRec *__restrict__ split, unsigned max_items,
+                                         unsigned *__restrict__ overflow) {
+  __shared__ unsigned s_base[kMaxPlanNodes + 1];
+  __shared__ unsigned s_wave[16];
+  __shared__ unsigned s_carry;
+  __shared__ unsigned long long s_rows;
+  const int tid = threadIdx.x;
+  if (tid == 0) {
+    s_carry = 0;
+    s_rows = 0;
+  }
+  __syncthreads();
+  for (int base = 0; base < L; base += 1024) {
+    const int nd = base + tid;
+    unsigned cnt = 0;
+    if (nd < L) {
+      const unsigned long long len = tot[nd].c;
+      bool sel = true;
+      if (select == 1) {
+        const unsigned long long sib = tot[nd ^ 1].c;
+        sel = (nd & 1) ? (len < sib) : (len <= sib);
+      }
+      if (sel && len > 0) {
+        cnt = (unsigned)((len + rows_per_item - 1) / rows_per_item);
+        unsigned long long acc = len;
+        if (split) {
+          const unsigned long long cl = split[nd].left.c;
+          acc = min(cl, len - cl);
+        }
+        atomicAdd(&s_rows, acc);
+      }
+      node_items[nd] = sel ? cnt : 0xffffffffu;  // 0xffffffff marks "not selected"
+    }
+    // block exclusive scan of cnt
+    unsigned incl = cnt;
+    for (int off = 1; off < 64; off <<= 1) {
+      const unsigned o = __shfl_up(incl, off);
+      if ((tid & 63) >= off) incl += o;
+    }
+    if ((tid & 63) == 63) s_wave[tid >> 6] = incl;
+    __syncthreads();
+    unsigned wave_off = 0;
+    for (int w = 0; w < (tid >> 6); ++w) wave_off += s_wave[w];
+    const unsigned excl = s_carry + wave_off + incl - cnt;
+    if (nd < L) {
+      s_base[nd] = excl;
+      node_first[nd] = excl;
+    }
+    __syncthreads();
+    if (tid == 1023) s_carry = excl + cnt;
+    __syncthreads();
+  }
+  const unsigned total = s_carry;
+  if (tid == 0) {
+    s_base[L] = total;
+    *n_work = total <= max_items ? total : 0;  // never exceed the launch bound
+    if (total > max_items) *overflow = 1;      // reported as an error at the end of the tree
+    if (rows_scanned) *rows_scanned += s_rows;
+  }
+  __syncthreads();
+  if (total > max_items) return;
+  for (unsigned w = tid; w < total; w += 1024) {
+    int lo = 0, hi = L;  // last node whose first item is <= w
+    while (hi - lo > 1) {
+      const int mid = (lo + hi) >> 1;
+      if (s_base[mid] <= w)
+        lo = mid;
+      else
+        hi = mid;
+    }
+    const unsigned start = seg_start[lo];
+    const unsigned len = (unsigned)tot[lo].c;
+    const unsigned k = w - s_base[lo];
+    WorkItem it;
+    it.node = lo;
+    it.begin = start + k * rows_per_item;
+    it.end = min(start + len, it.begin + rows_per_item);
+    it.first = s_base[lo];
+    work[w] = it;
+  }
+}
+
+__global__ void __launch_bounds__(1024)
+k_plan(const NodeSum *__restrict__ tot, const unsigned *__restrict__ seg_start, int L, int select,
+       unsigned rows_per_item, WorkItem *__restrict__ work, unsigned *__restrict__ n_work,
+       unsigned *__restrict__ node_first, unsigned *__restrict__ node_items,
+       unsigned long long *__restrict__ rows_scanned, const SplitRec *__restrict__ split,
+       unsigned max_items, unsigned *__restrict__ overflow) {
+  PlanBody(tot, seg_start, L, select, rows_per_item, work, n_work, node_first, node_items, rows_scanned, split,
+           max_items, overflow);
+}
+
+
+}  // namespace
+}  // namespace arb
+#endif  // ARBORETUM_AMD_KERNELS_PLAN_H_

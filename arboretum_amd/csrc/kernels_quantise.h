@@ -1,0 +1,98 @@
+// Bin assignment from thresholds, packing of pre-quantised input.
+#ifndef ARBORETUM_AMD_KERNELS_QUANTISE_H_
+#define ARBORETUM_AMD_KERNELS_QUANTISE_H_
+#include "device_common.h"
+
+namespace arb {
+namespace {
+
+// --------------------------------------------------------------- quantiser
+// bin(x) = first l in [0,size] with x <= v[l], v[t] = thr[t] for t < size-1,
+// +INF above (src/core/cuda_helpers.h:207-222, src/io/io.cu:297-302); NaN
+// compares false everywhere and lands in bin `size`.
+__global__ void k_bin_assign(const float *__restrict__ x, int ncols, const float *__restrict__ thr,
+                             int thr_stride, const int *__restrict__ sizes,
+                             uint32_t *__restrict__ out, size_t n) {
+  __shared__ float s_thr[4][kSlots];
+  __shared__ int s_size[4];
+  for (int i = threadIdx.x; i < 4 * kSlots; i += blockDim.x) {
+    const int c = i >> 8, t = i & 255;
+    float v = INFINITY;
+    if (c < ncols && t < sizes[c] - 1) v = thr[(size_t)c * thr_stride + t];
+    s_thr[c][t] = v;
+  }
+  if (threadIdx.x < 4) s_size[threadIdx.x] = threadIdx.x < ncols ? sizes[threadIdx.x] : 0;
+  __syncthreads();
+  for (size_t r = (size_t)blockIdx.x * blockDim.x + threadIdx.x; r < n;
+       r += (size_t)gridDim.x * blockDim.x) {
+    uint32_t packed = 0;
+#pragma unroll
+    for (int c = 0; c < 4; ++c) {
+      if (c < ncols) {
+        const float v = x[(size_t)c * n + r];
+        unsigned l = 0, h = (unsigned)s_size[c];
+        while (l < h) {
+          const unsigned mid = (l + h) >> 1;
+          if (v <= s_thr[c][mid])
+            h = mid;
+          else
+            l = mid + 1;
+        }
+        packed |= l << (8 * c);
+      }
+    }
+    out[r] = packed;
+  }
+}
+
+// The same with 16-bit bins: two features per word, thresholds of both in
+// dynamic LDS (2 * thr_stride floats).
+__global__ void k_bin_assign_wide(const float *__restrict__ x, int ncols, const float *__restrict__ thr,
+                                  int thr_stride, const int *__restrict__ sizes,
+                                  uint32_t *__restrict__ out, size_t n) {
+  extern __shared__ float s_thr_wide[];
+  for (int i = threadIdx.x; i < 2 * thr_stride; i += blockDim.x) {
+    const int c = i / thr_stride, t = i % thr_stride;
+    float v = INFINITY;
+    if (c < ncols && t < sizes[c] - 1) v = thr[(size_t)c * thr_stride + t];
+    s_thr_wide[i] = v;
+  }
+  __syncthreads();
+  for (size_t r = (size_t)blockIdx.x * blockDim.x + threadIdx.x; r < n;
+       r += (size_t)gridDim.x * blockDim.x) {
+    uint32_t packed = 0;
+    for (int c = 0; c < ncols; ++c) {
+      const float v = x[(size_t)c * n + r];
+      unsigned l = 0, h = (unsigned)sizes[c];
+      while (l < h) {
+        const unsigned mid = (l + h) >> 1;
+        if (v <= s_thr_wide[c * thr_stride + mid])
+          h = mid;
+        else
+          l = mid + 1;
+      }
+      packed |= l << (16 * c);
+    }
+    out[r] = packed;
+  }
+}
+
+// row-major uint8 [n][F] -> quads
+__global__ void k_pack_prebinned(const uint8_t *__restrict__ in, int F, int Q,
+                                 uint32_t *__restrict__ out, size_t stride, size_t n) {
+  for (size_t r = (size_t)blockIdx.x * blockDim.x + threadIdx.x; r < n;
+       r += (size_t)gridDim.x * blockDim.x) {
+    for (int q = 0; q < Q; ++q) {
+      uint32_t packed = 0;
+      for (int c = 0; c < 4; ++c) {
+        const int f = q * 4 + c;
+        if (f < F) packed |= (uint32_t)in[r * F + f] << (8 * c);
+      }
+      out[(size_t)q * stride + r] = packed;
+    }
+  }
+}
+
+}  // namespace
+}  // namespace arb
+#endif  // ARBORETUM_AMD_KERNELS_QUANTISE_H_

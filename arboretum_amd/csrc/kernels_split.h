@@ -1,0 +1,221 @@
+// Split search: prefix scan and gain per feature, best feature per node.
+#ifndef ARBORETUM_AMD_KERNELS_SPLIT_H_
+#define ARBORETUM_AMD_KERNELS_SPLIT_H_
+#include "device_common.h"
+#include "kernels_plan.h"
+
+namespace arb {
+namespace {
+
+// --------------------------------------------------------------- split scan
+struct Cand {
+  float gain;
+  int bin;
+  NodeSum left;
+};
+
+// One wave per (feature, node): inclusive prefix over the 256 slots, gain per
+// bin < hist_size, arg-max with ties to the HIGHEST bin (builder.h:39-49),
+// only gains > 0 (hist_tree_grower.cu:31).
+template <bool PAIR, bool F64>
+__global__ void __launch_bounds__(64)
+k_split_scan(const long long *__restrict__ hg, const long long *__restrict__ hh,
+             const unsigned *__restrict__ hc, int nbin_total, int F, int slots,
+             const NodeSum *__restrict__ tot, const int *__restrict__ shifts, GainParams gp,
+             int hist_size, Cand *__restrict__ cand) {
+  const int f = blockIdx.x, nd = blockIdx.y, lane = threadIdx.x;
+  const NodeSum t = tot[nd];
+  Cand best;
+  best.gain = 0.0f;
+  best.bin = -1;
+  best.left.g = best.left.h = 0;
+  best.left.c = 0;
+  if (t.c != 0) {
+    const int sg = shifts[0], sh = shifts[1];
+    const double GT = FromFixed<F64>(t.g, sg);
+    const double HT = PAIR ? FromFixed<F64>(t.h, sh) : 0.0;
+    // sums of the slots below the current chunk of 256
+    long long carry_g = 0, carry_h = 0;
+    unsigned long long carry_c = 0;
+    for (int chunk = 0; chunk < slots && chunk < hist_size; chunk += 256) {
+      const size_t base = (size_t)nd * nbin_total + (size_t)f * slots + chunk + lane * 4;
+      long long g4[4], h4[4];
+      unsigned long long c4[4];
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        g4[j] = hg[base + j];
+        h4[j] = PAIR ? hh[base + j] : 0;
+        c4[j] = hc[base + j];
+      }
+#pragma unroll
+      for (int j = 1; j < 4; ++j) {
+        g4[j] += g4[j - 1];
+        h4[j] += h4[j - 1];
+        c4[j] += c4[j - 1];
+      }
+      long long ig = g4[3], ih = h4[3];
+      unsigned long long ic = c4[3];
+      for (int off = 1; off < 64; off <<= 1) {
+        const long long og = __shfl_up(ig, off);
+        const long long oh = __shfl_up(ih, off);
+        const unsigned long long oc = __shfl_up(ic, off);
+        if (lane >= off) {
+          ig += og;
+          ih += oh;
+          ic += oc;
+        }
+      }
+      const long long eg = carry_g + ig - g4[3], eh = carry_h + ih - h4[3];
+      const unsigned long long ec = carry_c + ic - c4[3];
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        const int bin = chunk + lane * 4 + j;
+        if (bin < hist_size) {
+          const long long lg = eg + g4[j], lh = eh + h4[j];
+          const unsigned long long lc = ec + c4[j];
+          const double GL = FromFixed<F64>(lg, sg);
+          const double HL = PAIR ? FromFixed<F64>(lh, sh) : 0.0;
+          const float gn = SplitGain<PAIR, F64>(GL, HL, lc, GT, HT, t.c, gp);
+          if (gn > 0.0f && gn >= best.gain) {
+            best.gain = gn;
+            best.bin = bin;
+            best.left.g = lg;
+            best.left.h = lh;
+            best.left.c = lc;
+          }
+        }
+      }
+      carry_g += __shfl(ig, 63);
+      carry_h += __shfl(ih, 63);
+      carry_c += __shfl(ic, 63);
+    }
+    for (int off = 32; off > 0; off >>= 1) {
+      const float og = __shfl_down(best.gain, off);
+      const int ob = __shfl_down(best.bin, off);
+      const long long olg = __shfl_down(best.left.g, off);
+      const long long olh = __shfl_down(best.left.h, off);
+      const unsigned long long olc = __shfl_down(best.left.c, off);
+      if (ob >= 0 && (best.bin < 0 || og > best.gain || (og == best.gain && ob > best.bin))) {
+        best.gain = og;
+        best.bin = ob;
+        best.left.g = olg;
+        best.left.h = olh;
+        best.left.c = olc;
+      }
+    }
+  }
+  if (lane == 0) cand[(size_t)nd * F + f] = best;
+}
+
+// One thread per node: best candidate over the features active at this level
+// (higher gain, then lower feature id: hist_tree_grower.cu:59-60), children
+// totals and row ranges, node record.  A node without a candidate keeps every
+// row left.
+// One wave per node: lane l looks at features l, l + 64, ...; the wave keeps
+// the candidate with the highest gain, ties to the lowest feature id.
+__device__ __forceinline__ void SelectNode(int nd, int lane, const Cand *__restrict__ cand, int F,
+                                           const NodeSum *__restrict__ tot,
+                                           const unsigned *__restrict__ seg_start,
+                                           NodeSum *__restrict__ tot_next, unsigned *__restrict__ seg_next,
+                                           SplitRec *__restrict__ split, int *__restrict__ t_fid,
+                                           int *__restrict__ t_bin, float *__restrict__ t_gain, int heap_off,
+                                           const unsigned char *__restrict__ active) {
+  const NodeSum t = tot[nd];
+  float gain = 0.0f;
+  int fid = -1, bin = -1;
+  long long lg = 0, lh = 0;
+  unsigned long long lc = 0;
+  if (t.c != 0) {
+    for (int f = lane; f < F; f += 64) {
+      if (active && !active[f]) continue;  // feature not sampled at this level
+      const Cand c = cand[(size_t)nd * F + f];
+      if (c.bin >= 0 && (fid < 0 || gain < c.gain)) {
+        gain = c.gain;
+        fid = f;
+        bin = c.bin;
+        lg = c.left.g;
+        lh = c.left.h;
+        lc = c.left.c;
+      }
+    }
+  }
+  for (int off = 32; off > 0; off >>= 1) {
+    const float og = __shfl_down(gain, off);
+    const int of = __shfl_down(fid, off);
+    const int ob = __shfl_down(bin, off);
+    const long long olg = __shfl_down(lg, off);
+    const long long olh = __shfl_down(lh, off);
+    const unsigned long long olc = __shfl_down(lc, off);
+    if (of >= 0 && (fid < 0 || og > gain || (og == gain && of < fid))) {
+      gain = og;
+      fid = of;
+      bin = ob;
+      lg = olg;
+      lh = olh;
+      lc = olc;
+    }
+  }
+  if (lane != 0) return;
+  SplitRec rec;
+  rec.gain = fid < 0 ? 0.0f : gain;
+  rec.fid = fid;
+  rec.bin = fid < 0 ? -1 : bin;
+  rec.pad = 0;
+  rec.left = t;
+  if (fid >= 0) {
+    rec.left.g = lg;
+    rec.left.h = lh;
+    rec.left.c = lc;
+  }
+  split[nd] = rec;
+  NodeSum r;
+  r.g = t.g - rec.left.g;
+  r.h = t.h - rec.left.h;
+  r.c = t.c - rec.left.c;
+  tot_next[2 * nd] = rec.left;
+  tot_next[2 * nd + 1] = r;
+  const unsigned start = seg_start[nd];
+  seg_next[2 * nd] = start;
+  seg_next[2 * nd + 1] = start + (unsigned)rec.left.c;
+  t_fid[heap_off + nd] = rec.fid < 0 ? 0 : rec.fid;  // garden.cu:471-481
+  t_bin[heap_off + nd] = rec.fid < 0 ? -1 : rec.bin;
+  t_gain[heap_off + nd] = rec.gain;
+}
+
+// grid ceil(L / 16), 1024 threads: one wave per node
+__global__ void __launch_bounds__(1024)
+k_split_select(const Cand *__restrict__ cand, int F, int L, const NodeSum *__restrict__ tot,
+               const unsigned *__restrict__ seg_start, NodeSum *__restrict__ tot_next,
+               unsigned *__restrict__ seg_next, SplitRec *__restrict__ split, int *__restrict__ t_fid,
+               int *__restrict__ t_bin, float *__restrict__ t_gain, int heap_off,
+               const unsigned char *__restrict__ active) {
+  const int nd = blockIdx.x * 16 + (threadIdx.x >> 6);
+  if (nd < L)
+    SelectNode(nd, threadIdx.x & 63, cand, F, tot, seg_start, tot_next, seg_next, split, t_fid, t_bin, t_gain,
+               heap_off, active);
+}
+
+// k_split_select followed, in the same workgroup, by the work plan of the
+// fused pass over these nodes' rows (the plan needs the splits only for the
+// row statistics).  One workgroup of 1024 threads.
+__global__ void __launch_bounds__(1024)
+k_select_plan(const Cand *__restrict__ cand, int F, int L, const NodeSum *__restrict__ tot,
+              const unsigned *__restrict__ seg_start, NodeSum *__restrict__ tot_next,
+              unsigned *__restrict__ seg_next, SplitRec *__restrict__ split, int *__restrict__ t_fid,
+              int *__restrict__ t_bin, float *__restrict__ t_gain, int heap_off,
+              const unsigned char *__restrict__ active, unsigned rows_per_item,
+              WorkItem *__restrict__ work, unsigned *__restrict__ n_work,
+              unsigned *__restrict__ node_first, unsigned *__restrict__ node_items,
+              unsigned long long *__restrict__ rows_scanned, unsigned max_items,
+              unsigned *__restrict__ overflow) {
+  for (int nd = threadIdx.x >> 6; nd < L; nd += 16)
+    SelectNode(nd, threadIdx.x & 63, cand, F, tot, seg_start, tot_next, seg_next, split, t_fid, t_bin, t_gain,
+               heap_off, active);
+  __syncthreads();  // the splits written above are read by the plan
+  PlanBody(tot, seg_start, L, 0, rows_per_item, work, n_work, node_first, node_items, rows_scanned, split,
+           max_items, overflow);
+}
+
+}  // namespace
+}  // namespace arb
+#endif  // ARBORETUM_AMD_KERNELS_SPLIT_H_
