@@ -243,9 +243,10 @@ class Garden(object):
         self._ensure()
         _check(_LIB.AGardenSetInspect(self.handle, int(on)))
 
-    def enable_timing(self, on=True):
+    def enable_timing(self, level=1):
+        """0: off; 1: every phase; 2: only the deeper-level histogram kernels (cheapest)."""
         self._ensure()
-        _check(_LIB.AGardenEnableTiming(self.handle, int(on)))
+        _check(_LIB.AGardenEnableTiming(self.handle, int(level)))
 
     def timings(self):
         out = np.zeros(16, dtype=np.float64)

@@ -42,21 +42,23 @@ RegTree::RegTree(unsigned depth, unsigned label) : depth(depth), label(label) {
   weights.assign((size_t)1 << (depth - 1), 0.0f);
 }
 
-void RegTree::Predict(const DataMatrix &data, float *out) const {
+void RegTree::PredictRows(const DataMatrix &data, size_t begin, size_t end, float *out) const {
   const size_t offset = ((size_t)1 << (depth - 1)) - 1;
   const size_t F = data.columns_dense;
-  ParallelFor(data.rows, [&](size_t b, size_t e) {
-    for (size_t i = b; i < e; ++i) {
-      size_t id = 0;
-      for (unsigned j = 1; j < depth; ++j) {
-        const unsigned f = fid[id];
-        // a feature id outside the matrix (foreign model) behaves like NaN: right
-        const bool left = f < F && data.value(f, i) < threshold[id];
-        id = left ? 2 * id + 1 : 2 * id + 2;
-      }
-      out[i + (size_t)label * data.rows] += weights[id - offset];
+  for (size_t i = begin; i < end; ++i) {
+    size_t id = 0;
+    for (unsigned j = 1; j < depth; ++j) {
+      const unsigned f = fid[id];
+      // a feature id outside the matrix (foreign model) behaves like NaN: right
+      const bool left = f < F && data.value(f, i) < threshold[id];
+      id = left ? 2 * id + 1 : 2 * id + 2;
     }
-  });
+    out[i + (size_t)label * data.rows] += weights[id - offset];
+  }
+}
+
+void RegTree::Predict(const DataMatrix &data, float *out) const {
+  ParallelFor(data.rows, [&](size_t b, size_t e) { PredictRows(data, b, e, out); });
 }
 
 Garden::Garden(const Configuration &c) : cfg(c) {
@@ -140,7 +142,17 @@ void Garden::Predict(const DataMatrix *data, std::vector<float> *out, int n_roun
   SyncTrees();
   std::vector<float> tmp(data->rows * K, IntoInternal(cfg.tree.initial_y));
   const long long use = std::min<long long>(n_rounds, (long long)trees_.size());
-  for (long long t = 0; t < use; ++t) trees_[t].Predict(*data, tmp.data());
+  // Every tree over one block of rows before the next block: the block's
+  // feature values (column-major, 4096 rows of every column) stay in cache, so
+  // the matrix is read once, not once per tree.  Sums per row are added in tree
+  // order either way.
+  constexpr size_t kBlock = 4096;
+  ParallelFor(data->rows, [&](size_t b, size_t e) {
+    for (size_t r0 = b; r0 < e; r0 += kBlock) {
+      const size_t r1 = std::min(e, r0 + kBlock);
+      for (long long t = 0; t < use; ++t) trees_[t].PredictRows(*data, r0, r1, tmp.data());
+    }
+  });
   FromInternal(tmp, out);
 }
 

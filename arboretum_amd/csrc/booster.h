@@ -78,6 +78,8 @@ struct RegTree {
   // RegTree::Predict, garden.h:70-90: x < threshold -> left; adds the leaf
   // weight to out[i + label * rows].
   void Predict(const DataMatrix &data, float *out) const;
+  // The same for rows [begin, end) only, on the calling thread.
+  void PredictRows(const DataMatrix &data, size_t begin, size_t end, float *out) const;
 };
 
 // Accumulated GPU milliseconds per kernel class.  hist_root: histogram kernel
@@ -108,7 +110,9 @@ class TreeBuilder {
   virtual void GetGrad(float *g, float *h) = 0;            // labels_count * rows each
   virtual int GetLevelHist(int level, int64_t *out) = 0;   // [node][F][256][3], needs inspect
   virtual void GetShifts(int *shift_g, int *shift_h) = 0;
-  virtual void EnableTiming(bool on) = 0;
+  // 0: off; 1: every phase; 2: only the dominant kernel (the fused pass), which
+  // costs a third of the event records
+  virtual void EnableTiming(int level) = 0;
   virtual BuilderTimings GetTimings() = 0;
   virtual unsigned long long RowsScanned() = 0;            // rows accumulated into histograms
   virtual void Synchronize() = 0;
@@ -151,7 +155,7 @@ class Garden {
 
   // Inspection / timing switches; they also apply to a builder created later.
   void SetInspect(bool on) { inspect_ = on; if (builder_) builder_->SetInspect(on); }
-  void SetTiming(bool on) { timing_ = on; if (builder_) builder_->EnableTiming(on); }
+  void SetTiming(int level) { timing_ = level; if (builder_) builder_->EnableTiming(level); }
 
   TreeBuilder *builder() { return builder_.get(); }
   size_t num_trees() const { return trees_.size(); }
@@ -167,7 +171,8 @@ class Garden {
   void SyncTrees() const { if (builder_) builder_->FlushTrees(); }
   mutable std::vector<RegTree> trees_;
   std::string model_;
-  bool inspect_ = false, timing_ = false;
+  bool inspect_ = false;
+  int timing_ = 0;
 };
 
 }  // namespace arb

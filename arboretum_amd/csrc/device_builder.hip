@@ -654,9 +654,11 @@ class HipTreeBuilder : public TreeBuilder {
     *sg = s[0];
     *sh = s[1];
   }
-  void EnableTiming(bool on) override {
+  void EnableTiming(int level) override {
     ResolveTimings();
-    timing_ = on;
+    timing_ = level != 0;
+    dominant_only_ = level == 2;
+    deep_open_ = false;
   }
   BuilderTimings GetTimings() override {
     ResolveTimings();
@@ -680,6 +682,12 @@ class HipTreeBuilder : public TreeBuilder {
   // consecutive events is charged to the phase that was open.
   void Mark(int phase) {
     if (!timing_) return;
+    if (dominant_only_) {
+      // only the fused pass is bracketed: an event where it starts, one where it ends
+      if (phase != kHistDeep && !deep_open_) return;
+      deep_open_ = phase == kHistDeep;
+      if (!deep_open_) phase = kNone;
+    }
     hipEvent_t e;
     if (event_used_ < event_pool_.size()) {
       e = event_pool_[event_used_];
@@ -1176,6 +1184,7 @@ class HipTreeBuilder : public TreeBuilder {
   std::vector<size_t> pending_;              // indices into *owner_ of the trees not fetched yet
   std::vector<RegTree> *owner_ = nullptr;
   bool pair_ = false, f64_ = false, trick_ = true, fused_ = false, inspect_ = false, timing_ = false;
+  bool dominant_only_ = false, deep_open_ = false;  // timing of the fused pass only
   bool grad_ready_ = false;
   int quads_per_group_ = 1;
   hipStream_t stream_ = nullptr;

@@ -270,7 +270,7 @@ const char *AGardenGetShifts(VoidPointer garden, int *shift_g, int *shift_h) {
 }
 const char *AGardenEnableTiming(VoidPointer garden, int on) {
   return Guard([&] {
-    AsGarden(garden)->garden.SetTiming(on != 0);
+    AsGarden(garden)->garden.SetTiming(on);
   });
 }
 const char *AGardenGetTimings(VoidPointer garden, double *out) {
