@@ -45,6 +45,24 @@ RegTree::RegTree(unsigned depth, unsigned label) : depth(depth), label(label) {
 void RegTree::PredictRows(const DataMatrix &data, size_t begin, size_t end, float *out) const {
   const size_t offset = ((size_t)1 << (depth - 1)) - 1;
   const size_t F = data.columns_dense;
+  if (!data.is_prebinned) {
+    // float columns: no per-value dispatch, no branch on the comparison
+    bool foreign = false;  // a feature id outside the matrix (foreign model) behaves like NaN: right
+    for (unsigned f : fid) foreign = foreign || f >= F;
+    if (!foreign) {
+      std::vector<const float *> cols(F);
+      for (size_t f = 0; f < F; ++f) cols[f] = data.data[f].data();
+      const unsigned *fids = fid.data();
+      const float *thr = threshold.data();
+      float *dst = out + (size_t)label * data.rows;
+      for (size_t i = begin; i < end; ++i) {
+        size_t id = 0;
+        for (unsigned j = 1; j < depth; ++j) id = 2 * id + 2 - (size_t)(cols[fids[id]][i] < thr[id]);
+        dst[i] += weights[id - offset];
+      }
+      return;
+    }
+  }
   for (size_t i = begin; i < end; ++i) {
     size_t id = 0;
     for (unsigned j = 1; j < depth; ++j) {
@@ -91,7 +109,9 @@ void Garden::FromInternal(const std::vector<float> &in, std::vector<float> *out)
   if (cfg.objective == kLinearRegression) {
     *out = in;
   } else if (cfg.objective == kLogisticRegression) {  // objective.h:58-69
-    for (size_t i = 0; i < in.size(); ++i) (*out)[i] = (float)(1.0 / (1.0 + (double)std::exp(-in[i])));
+    ParallelFor(in.size(), [&](size_t b, size_t e) {
+      for (size_t i = b; i < e; ++i) (*out)[i] = (float)(1.0 / (1.0 + (double)std::exp(-in[i])));
+    });
   } else {  // objective.h:80-113: class-major in, row-major out
     const size_t K = cfg.tree.labels_count;
     const size_t n = in.size() / K;
