@@ -6,6 +6,8 @@
 #include <new>
 #include <stdexcept>
 #include <string>
+#include <thread>
+#include <vector>
 
 #include "../../include/arboretum_ext.h"
 #include "booster.h"
@@ -71,11 +73,28 @@ const char *ACreateFromDenseMatrix(const float *data, const unsigned int *catego
   return Guard([&] {
     if (!data || !out || nrow < 0 || ncol < 0 || ccol < 0) throw std::runtime_error("bad arguments");
     DataMatrix *mat = new DataMatrix((size_t)nrow, (size_t)ncol, (size_t)ccol);
-    mat->data.assign(ncol, std::vector<float>((size_t)nrow));
     const size_t rows = (size_t)nrow, cols = (size_t)ncol;
+    // the columns are allocated (and their pages first touched) by several threads
+    mat->data.resize(cols);
+    {
+      const size_t nt = std::min<size_t>(cols, 16);
+      std::vector<std::thread> th;
+      for (size_t t = 0; t < nt; ++t)
+        th.emplace_back([&, t] {
+          for (size_t f = t; f < cols; f += nt) mat->data[f].resize(rows);
+        });
+      for (auto &x : th) x.join();
+    }
+    // row-major -> column-major in tiles of 256 rows, so that a tile's lines of every
+    // column stay in cache while its rows are read once
     ParallelFor(rows, [&](size_t b, size_t e) {
-      for (size_t i = b; i < e; ++i)
-        for (size_t f = 0; f < cols; ++f) mat->data[f][i] = data[i * cols + f];
+      for (size_t r0 = b; r0 < e; r0 += 256) {
+        const size_t r1 = std::min(e, r0 + 256);
+        for (size_t f = 0; f < cols; ++f) {
+          float *dst = mat->data[f].data();
+          for (size_t i = r0; i < r1; ++i) dst[i] = data[i * cols + f];
+        }
+      }
     });
     if (ccol > 0 && categories) {
       mat->data_categories.assign(ccol, std::vector<unsigned>(rows));
