@@ -244,7 +244,7 @@ class Garden(object):
         _check(_LIB.AGardenSetInspect(self.handle, int(on)))
 
     def enable_timing(self, level=1):
-        """0: off; 1: every phase; 2: only the deeper-level histogram kernels (cheapest)."""
+        """0: off; 1: every phase; 2: only the deeper-level histogram kernels; 3: those on every fourth tree."""
         self._ensure()
         _check(_LIB.AGardenEnableTiming(self.handle, int(level)))
 

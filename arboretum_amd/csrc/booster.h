@@ -111,7 +111,7 @@ class TreeBuilder {
   virtual int GetLevelHist(int level, int64_t *out) = 0;   // [node][F][256][3], needs inspect
   virtual void GetShifts(int *shift_g, int *shift_h) = 0;
   // 0: off; 1: every phase; 2: only the dominant kernel (the fused pass), which
-  // costs a third of the event records
+  // costs a third of the event records; 3: that on every fourth tree
   virtual void EnableTiming(int level) = 0;
   virtual BuilderTimings GetTimings() = 0;
   virtual unsigned long long RowsScanned() = 0;            // rows accumulated into histograms

@@ -583,6 +583,7 @@ class HipTreeBuilder : public TreeBuilder {
       // synchronisation between trees
       trees->emplace_back((unsigned)D_, (unsigned)k);
       GrowOne(k);
+      ++trees_grown_;
       pending_.push_back(trees->size() - 1);
       if (inspect_ || pending_.size() == kRecordRing) FlushTrees();
     }
@@ -657,7 +658,8 @@ class HipTreeBuilder : public TreeBuilder {
   void EnableTiming(int level) override {
     ResolveTimings();
     timing_ = level != 0;
-    dominant_only_ = level == 2;
+    dominant_only_ = level >= 2;
+    sample_every_ = level == 3 ? 4 : 1;
     deep_open_ = false;
   }
   BuilderTimings GetTimings() override {
@@ -683,7 +685,9 @@ class HipTreeBuilder : public TreeBuilder {
   void Mark(int phase) {
     if (!timing_) return;
     if (dominant_only_) {
-      // only the fused pass is bracketed: an event where it starts, one where it ends
+      // only the fused pass is bracketed: an event where it starts, one where it
+      // ends (level 3: on every fourth tree)
+      if (phase == kHistDeep && trees_grown_ % sample_every_ != 0) return;
       if (phase != kHistDeep && !deep_open_) return;
       deep_open_ = phase == kHistDeep;
       if (!deep_open_) phase = kNone;
@@ -857,7 +861,8 @@ class HipTreeBuilder : public TreeBuilder {
               else ARB_FUSED(false, true);
             }
 #undef ARB_FUSED
-            if (timing_) ++(last ? timings_.fused_last_launches : timings_.hist_deep_launches);
+            if (timing_ && (last || !dominant_only_ || trees_grown_ % sample_every_ == 0))
+            ++(last ? timings_.fused_last_launches : timings_.hist_deep_launches);
           }
           Reduce(L, hb, true, ps, true);
         } else {
@@ -1185,6 +1190,8 @@ class HipTreeBuilder : public TreeBuilder {
   std::vector<RegTree> *owner_ = nullptr;
   bool pair_ = false, f64_ = false, trick_ = true, fused_ = false, inspect_ = false, timing_ = false;
   bool dominant_only_ = false, deep_open_ = false;  // timing of the fused pass only
+  unsigned sample_every_ = 1;
+  unsigned long long trees_grown_ = 0;
   bool grad_ready_ = false;
   int quads_per_group_ = 1;
   hipStream_t stream_ = nullptr;

@@ -190,10 +190,10 @@ def main():
     for _ in range(args.warmup):
         model.grow_tree()
     model.synchronize()
-    # The timed region brackets only the dominant kernel with HIP events (two per launch);
-    # the phase breakdown comes from a few more trees grown afterwards with every phase
-    # bracketed (about 35 event records per tree, which costs 5 % of the tree time).
-    model.enable_timing(2)
+    # The timed region brackets only the dominant kernel with HIP events (two per launch), on
+    # every fourth tree; the phase breakdown comes from a few more trees grown afterwards with
+    # every phase bracketed (about 35 event records per tree, which costs 5 % of the tree time).
+    model.enable_timing(3)
     scanned0 = model.rows_scanned()
     t0 = time.perf_counter()
     for _ in range(args.steps):
@@ -222,7 +222,10 @@ def main():
     # read once and written once in the children order, and the smaller child of
     # each parent gets one histogram written.
     fl = max(fused_launches_timed, 1)
-    parents = sum(1 << (l - 1) for l in range(1, args.max_depth - 1)) * args.steps
+    # parents whose smaller child got a histogram in the measured launches (levels 1..max_depth-2
+    # of the sampled trees)
+    launches_per_tree = max(args.max_depth - 2, 1)
+    parents = sum(1 << (l - 1) for l in range(1, args.max_depth - 1)) * fl / launches_per_tree
     fused_bytes = fl * args.rows * 2 * row_bytes + parents * F * 256 * cell_bytes
     fused_s = fused_ms_timed * 1e-3
     achieved = fused_bytes / fused_s if fused_s > 0 else 0.0
@@ -291,7 +294,7 @@ def main():
         "other_kernels": other,
         "tree_algorithmic_floor_frac_of_hbm": (2.9e9 / (dt / args.steps)) / HBM_PEAK,
         "phase_ms_per_tree": dict({k: v / phase_trees for k, v in tm.items() if k.endswith("_ms")},
-                                  hist_deep_ms=fused_ms_timed / args.steps),
+                                  hist_deep_ms=fused_ms_timed / (fl / launches_per_tree)),
         "phase_trees": phase_trees,
         "quantise_s": t_quant,
     }

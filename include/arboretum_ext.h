@@ -76,7 +76,8 @@ const char *AGardenGetShifts(VoidPointer garden, int *shift_g, int *shift_h);
  * milliseconds in the fused kernel of the last level (it moves no rows),
  * out[12] = its launches.  `on`: 0 = off, 1 = every phase (about 35 event
  * records per tree), 2 = only the deeper-level histogram kernels (out[2] and
- * out[10]; a third of the records, for timed runs). */
+ * out[10]; a third of the records), 3 = those on every fourth tree only (for
+ * timed runs: the records themselves cost time). */
 const char *AGardenEnableTiming(VoidPointer garden, int on);
 const char *AGardenGetTimings(VoidPointer garden, double *out);
 /* Rows accumulated into histograms so far (x ncol = histogram updates). */
