@@ -363,6 +363,20 @@ def test_rows_concentrated_in_one_bin(arb, oracle, upload, objective):
     assert_same_training(arb, oracle, X, y, cfg, rounds=3)
 
 
+def test_duplicate_features_tie_to_the_lowest_feature_id(arb, oracle):
+    # equal gains across features: the lowest feature id wins (hist_tree_grower.cu:59-60)
+    X, y = make_data(8000, 6, 1, seed=12)
+    X[:, 4] = X[:, 1]
+    X[:, 5] = X[:, 0]
+    X = X[:, [5, 4, 2, 3, 1, 0]].copy()  # the duplicates come first
+    cfg = {"objective": 1, "method": 1, "internals": {"hist_size": 64, "double_precision": True},
+           "tree": {"max_depth": 5, "eta": 0.3, "lambda": 1.0}}
+    ob, g = assert_same_training(arb, oracle, X, y, cfg, rounds=3)
+    for r in range(3):
+        fid = g.tree(r)["fid"]
+        assert not np.isin(fid, [4, 5]).any(), "a duplicate with the higher id was chosen"
+
+
 def test_constant_features_give_unsplit_nodes(arb, oracle):
     X = np.ones((500, 3), np.float32)
     y = np.arange(500, dtype=np.float32)
