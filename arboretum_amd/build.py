@@ -6,7 +6,7 @@ import sys
 HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(HERE, "csrc")
 LIB = os.path.join(HERE, "libarboretum.so")
-SOURCES = ["device_builder.hip", "quantiser.hip", "booster.cpp", "config.cpp", "wrapper.cpp"]
+SOURCES = ["device_builder.hip", "quantiser.hip", "predictor.hip", "booster.cpp", "config.cpp", "wrapper.cpp"]
 # -ffp-contract=off: the gain arithmetic must round exactly like the host
 # restatement (no fused multiply-add).  packed-fp32-ops is switched off
 # because some packed forms have produced wrong results on this hardware.

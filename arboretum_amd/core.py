@@ -49,6 +49,7 @@ def _load_lib():
         "AGetBinLayout": [c_void_p, P(c_int), P(c_int)],
         "AGetThresholds": [c_void_p, c_int, c_void_p, P(c_int)],
         "AGardenSetInspect": [c_void_p, c_int],
+        "AGardenPredictOnDevice": [c_void_p, c_int],
         "AGardenNumTrees": [c_void_p, P(c_int)],
         "AGardenGetTree": [c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p],
         "AGardenGetLeaves": [c_void_p, c_void_p],
@@ -239,6 +240,11 @@ class Garden(object):
         return json_p.value.decode('utf-8')
 
     # ---- extensions (include/arboretum_ext.h)
+    def predict_on_device(self, on=True):
+        """Tree walks of predict() on the GPU (default) or on the host; the results are bit-identical."""
+        self._ensure()
+        _check(_LIB.AGardenPredictOnDevice(self.handle, int(on)))
+
     def set_inspect(self, on=True):
         self._ensure()
         _check(_LIB.AGardenSetInspect(self.handle, int(on)))

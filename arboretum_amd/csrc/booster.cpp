@@ -162,6 +162,12 @@ void Garden::Predict(const DataMatrix *data, std::vector<float> *out, int n_roun
   SyncTrees();
   std::vector<float> tmp(data->rows * K, IntoInternal(cfg.tree.initial_y));
   const long long use = std::min<long long>(n_rounds, (long long)trees_.size());
+  if (predict_on_device_ && use > 0 && !data->is_prebinned && data->rows > 0 && DeviceCount() > 0) {
+    if (!predictor_) predictor_.reset(CreateDevicePredictor());
+    PredictOnDevice(predictor_.get(), *data, trees_, (size_t)use, K, IntoInternal(cfg.tree.initial_y), tmp.data());
+    FromInternal(tmp, out);
+    return;
+  }
   // Every tree over one block of rows before the next block: the block's
   // feature values (column-major, 4096 rows of every column) stay in cache, so
   // the matrix is read once, not once per tree.  Sums per row are added in tree

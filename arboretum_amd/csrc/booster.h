@@ -137,6 +137,15 @@ TreeBuilder *CreateTreeBuilder(const Configuration &cfg, DataMatrix *data);
 int DeviceCount();
 void CopyProbe(size_t bytes);
 
+// predictor.hip: tree walks of a float matrix on the GPU.  out: [labels][rows]
+// sums of leaf weights of trees[0, use) on top of `init`, bit-identical to the
+// host walk (RegTree::Predict in tree order).
+struct DevicePredictor;
+DevicePredictor *CreateDevicePredictor();
+void FreeDevicePredictor(DevicePredictor *p);
+void PredictOnDevice(DevicePredictor *p, const DataMatrix &data, const std::vector<RegTree> &trees, size_t use,
+                     size_t labels, float init, float *out);
+
 class Garden {
  public:
   explicit Garden(const Configuration &cfg);
@@ -156,6 +165,9 @@ class Garden {
   // Inspection / timing switches; they also apply to a builder created later.
   void SetInspect(bool on) { inspect_ = on; if (builder_) builder_->SetInspect(on); }
   void SetTiming(int level) { timing_ = level; if (builder_) builder_->EnableTiming(level); }
+  // Predict walks the trees on the GPU when one is present and the matrix holds
+  // floats (default), or on the host as the reference does.
+  void SetPredictOnDevice(bool on) { predict_on_device_ = on; }
 
   TreeBuilder *builder() { return builder_.get(); }
   size_t num_trees() const { return trees_.size(); }
@@ -173,6 +185,8 @@ class Garden {
   std::string model_;
   bool inspect_ = false;
   int timing_ = 0;
+  bool predict_on_device_ = true;
+  mutable std::unique_ptr<DevicePredictor, void (*)(DevicePredictor *)> predictor_{nullptr, FreeDevicePredictor};
 };
 
 }  // namespace arb

@@ -248,6 +248,12 @@ const char *AGardenSetInspect(VoidPointer garden, int on) {
   });
 }
 
+const char *AGardenPredictOnDevice(VoidPointer garden, int on) {
+  return Guard([&] {
+    AsGarden(garden)->garden.SetPredictOnDevice(on != 0);
+  });
+}
+
 const char *AGardenNumTrees(VoidPointer garden, int *out) {
   return Guard([&] { *out = (int)AsGarden(garden)->garden.num_trees(); });
 }
