@@ -935,8 +935,28 @@ class HipTreeBuilder : public TreeBuilder {
   // plan_next: also plan the fused pass of the next level over these nodes
   void LaunchSplit(int level, int L, int hb, int state, const GainParams &gp, bool plan_next = false) {
     Mark(kSplit);
-    dim3 grid(F_, L);
     const int hs = std::min(cfg_.internal.hist_size, slots_);
+    const unsigned char *active = sampling_ ? d_active_ + (size_t)level * F_ : (const unsigned char *)nullptr;
+    const unsigned per_item = HistRowsPerItem(n_);
+    // From 32 nodes on, one launch: a workgroup per node scans its features and
+    // selects.  With fewer nodes that would leave the gain arithmetic (28
+    // features x 256 bins in double precision per node) on a few CUs, and the
+    // scan over (feature, node) waves followed by the selection is faster.
+    if (L >= 32) {
+#define ARB_SCAN_SELECT(P, D)                                                                                     \
+  hipLaunchKernelGGL((k_scan_select<P, D>), dim3(L + (plan_next ? 1 : 0)), dim3(1024), 0, stream_, d_hg_[hb],     \
+                     d_hh_[hb], d_hc_[hb], nbin_total_, F_, slots_, L, d_tot_[state], d_shifts_, gp, hs,          \
+                     d_seg_[state], d_tot_[state ^ 1], d_seg_[state ^ 1], d_split_, d_tfid_, d_tbin_, d_tgain_,   \
+                     L - 1, active, plan_next ? 1 : 0, per_item, d_pwork_, d_nwork_ + 1, d_node_first_,           \
+                     d_node_items_, d_rows_scanned_, FusedGrid(L), d_overflow_)
+      if (pair_ && f64_) ARB_SCAN_SELECT(true, true);
+      else if (pair_) ARB_SCAN_SELECT(true, false);
+      else if (f64_) ARB_SCAN_SELECT(false, true);
+      else ARB_SCAN_SELECT(false, false);
+#undef ARB_SCAN_SELECT
+      return;
+    }
+    dim3 grid(F_, L);
 #define ARB_SCAN(P, D) \
   hipLaunchKernelGGL((k_split_scan<P, D>), grid, dim3(64), 0, stream_, d_hg_[hb], d_hh_[hb], d_hc_[hb], \
                      nbin_total_, F_, slots_, d_tot_[state], d_shifts_, gp, hs, d_cand_)
@@ -945,9 +965,7 @@ class HipTreeBuilder : public TreeBuilder {
     else if (f64_) ARB_SCAN(false, true);
     else ARB_SCAN(false, false);
 #undef ARB_SCAN
-    const unsigned char *active = sampling_ ? d_active_ + (size_t)level * F_ : (const unsigned char *)nullptr;
     if (plan_next) {
-      const unsigned per_item = HistRowsPerItem(n_);
       hipLaunchKernelGGL(k_select_plan, dim3(1), dim3(1024), 0, stream_, d_cand_, F_, L, d_tot_[state],
                          d_seg_[state], d_tot_[state ^ 1], d_seg_[state ^ 1], d_split_, d_tfid_, d_tbin_, d_tgain_,
                          L - 1, active, per_item, d_pwork_, d_nwork_ + 1, d_node_first_, d_node_items_,

@@ -14,17 +14,15 @@ struct Cand {
   NodeSum left;
 };
 
-// One wave per (feature, node): inclusive prefix over the 256 slots, gain per
-// bin < hist_size, arg-max with ties to the HIGHEST bin (builder.h:39-49),
-// only gains > 0 (hist_tree_grower.cu:31).
+// One wave scans one (feature, node): inclusive prefix over the slots, gain
+// per bin < hist_size, arg-max with ties to the HIGHEST bin (builder.h:39-49),
+// only gains > 0 (hist_tree_grower.cu:31).  `first` is the index of the
+// feature's slot 0 in the histogram arrays.  The result is valid in lane 0.
 template <bool PAIR, bool F64>
-__global__ void __launch_bounds__(64)
-k_split_scan(const long long *__restrict__ hg, const long long *__restrict__ hh,
-             const unsigned *__restrict__ hc, int nbin_total, int F, int slots,
-             const NodeSum *__restrict__ tot, const int *__restrict__ shifts, GainParams gp,
-             int hist_size, Cand *__restrict__ cand) {
-  const int f = blockIdx.x, nd = blockIdx.y, lane = threadIdx.x;
-  const NodeSum t = tot[nd];
+__device__ __forceinline__ Cand ScanFeature(const long long *__restrict__ hg, const long long *__restrict__ hh,
+                                            const unsigned *__restrict__ hc, size_t first, int slots,
+                                            const NodeSum &t, const int *__restrict__ shifts,
+                                            const GainParams &gp, int hist_size, int lane) {
   Cand best;
   best.gain = 0.0f;
   best.bin = -1;
@@ -38,7 +36,7 @@ k_split_scan(const long long *__restrict__ hg, const long long *__restrict__ hh,
     long long carry_g = 0, carry_h = 0;
     unsigned long long carry_c = 0;
     for (int chunk = 0; chunk < slots && chunk < hist_size; chunk += 256) {
-      const size_t base = (size_t)nd * nbin_total + (size_t)f * slots + chunk + lane * 4;
+      const size_t base = first + chunk + lane * 4;
       long long g4[4], h4[4];
       unsigned long long c4[4];
 #pragma unroll
@@ -104,8 +102,57 @@ k_split_scan(const long long *__restrict__ hg, const long long *__restrict__ hh,
       }
     }
   }
+  return best;
+}
+
+// grid (F, L), 64 threads: one wave per (feature, node), candidates to `cand`.
+template <bool PAIR, bool F64>
+__global__ void __launch_bounds__(64)
+k_split_scan(const long long *__restrict__ hg, const long long *__restrict__ hh,
+             const unsigned *__restrict__ hc, int nbin_total, int F, int slots,
+             const NodeSum *__restrict__ tot, const int *__restrict__ shifts, GainParams gp,
+             int hist_size, Cand *__restrict__ cand) {
+  const int f = blockIdx.x, nd = blockIdx.y, lane = threadIdx.x;
+  const NodeSum t = tot[nd];
+  const Cand best = ScanFeature<PAIR, F64>(hg, hh, hc, (size_t)nd * nbin_total + (size_t)f * slots, slots, t, shifts,
+                                           gp, hist_size, lane);
   if (lane == 0) cand[(size_t)nd * F + f] = best;
 }
+
+// Record of one node from its best candidate (fid < 0: none, every row stays
+// left): split, totals and row ranges of the two children, tree arrays.
+__device__ __forceinline__ void WriteNode(int nd, const NodeSum &t, float gain, int fid, int bin, long long lg,
+                                          long long lh, unsigned long long lc,
+                                          const unsigned *__restrict__ seg_start, NodeSum *__restrict__ tot_next,
+                                          unsigned *__restrict__ seg_next, SplitRec *__restrict__ split,
+                                          int *__restrict__ t_fid, int *__restrict__ t_bin,
+                                          float *__restrict__ t_gain, int heap_off) {
+  SplitRec rec;
+  rec.gain = fid < 0 ? 0.0f : gain;
+  rec.fid = fid;
+  rec.bin = fid < 0 ? -1 : bin;
+  rec.pad = 0;
+  rec.left = t;
+  if (fid >= 0) {
+    rec.left.g = lg;
+    rec.left.h = lh;
+    rec.left.c = lc;
+  }
+  split[nd] = rec;
+  NodeSum r;
+  r.g = t.g - rec.left.g;
+  r.h = t.h - rec.left.h;
+  r.c = t.c - rec.left.c;
+  tot_next[2 * nd] = rec.left;
+  tot_next[2 * nd + 1] = r;
+  const unsigned start = seg_start[nd];
+  seg_next[2 * nd] = start;
+  seg_next[2 * nd + 1] = start + (unsigned)rec.left.c;
+  t_fid[heap_off + nd] = rec.fid < 0 ? 0 : rec.fid;  // garden.cu:471-481
+  t_bin[heap_off + nd] = rec.fid < 0 ? -1 : rec.bin;
+  t_gain[heap_off + nd] = rec.gain;
+}
+
 
 // One thread per node: best candidate over the features active at this level
 // (higher gain, then lower feature id: hist_tree_grower.cu:59-60), children
@@ -156,30 +203,7 @@ __device__ __forceinline__ void SelectNode(int nd, int lane, const Cand *__restr
     }
   }
   if (lane != 0) return;
-  SplitRec rec;
-  rec.gain = fid < 0 ? 0.0f : gain;
-  rec.fid = fid;
-  rec.bin = fid < 0 ? -1 : bin;
-  rec.pad = 0;
-  rec.left = t;
-  if (fid >= 0) {
-    rec.left.g = lg;
-    rec.left.h = lh;
-    rec.left.c = lc;
-  }
-  split[nd] = rec;
-  NodeSum r;
-  r.g = t.g - rec.left.g;
-  r.h = t.h - rec.left.h;
-  r.c = t.c - rec.left.c;
-  tot_next[2 * nd] = rec.left;
-  tot_next[2 * nd + 1] = r;
-  const unsigned start = seg_start[nd];
-  seg_next[2 * nd] = start;
-  seg_next[2 * nd + 1] = start + (unsigned)rec.left.c;
-  t_fid[heap_off + nd] = rec.fid < 0 ? 0 : rec.fid;  // garden.cu:471-481
-  t_bin[heap_off + nd] = rec.fid < 0 ? -1 : rec.bin;
-  t_gain[heap_off + nd] = rec.gain;
+  WriteNode(nd, t, gain, fid, bin, lg, lh, lc, seg_start, tot_next, seg_next, split, t_fid, t_bin, t_gain, heap_off);
 }
 
 // grid ceil(L / 16), 1024 threads: one wave per node
@@ -214,6 +238,91 @@ k_select_plan(const Cand *__restrict__ cand, int F, int L, const NodeSum *__rest
   __syncthreads();  // the splits written above are read by the plan
   PlanBody(tot, seg_start, L, 0, rows_per_item, work, n_work, node_first, node_items, rows_scanned, split,
            max_items, overflow);
+}
+
+// Split scan and selection in one launch: workgroup `nd` < L scans the
+// features of node nd (wave w takes features w, w + 16, ...), keeps the
+// candidate with the highest gain, ties to the lowest feature id, and writes
+// the node's record; with `plan` set, workgroup L cuts the row ranges of these
+// nodes into the work items of the fused pass that follows, and every node adds
+// the rows of its smaller side to rows_scanned.  grid L (+ 1), 1024 threads.
+template <bool PAIR, bool F64>
+__global__ void __launch_bounds__(1024)
+k_scan_select(const long long *__restrict__ hg, const long long *__restrict__ hh,
+              const unsigned *__restrict__ hc, int nbin_total, int F, int slots, int L,
+              const NodeSum *__restrict__ tot, const int *__restrict__ shifts, GainParams gp, int hist_size,
+              const unsigned *__restrict__ seg_start, NodeSum *__restrict__ tot_next,
+              unsigned *__restrict__ seg_next, SplitRec *__restrict__ split, int *__restrict__ t_fid,
+              int *__restrict__ t_bin, float *__restrict__ t_gain, int heap_off,
+              const unsigned char *__restrict__ active, int plan, unsigned rows_per_item,
+              WorkItem *__restrict__ work, unsigned *__restrict__ n_work, unsigned *__restrict__ node_first,
+              unsigned *__restrict__ node_items, unsigned long long *__restrict__ rows_scanned,
+              unsigned max_items, unsigned *__restrict__ overflow) {
+  if ((int)blockIdx.x >= L) {  // uniform per workgroup
+    PlanBody(tot, seg_start, L, 0, rows_per_item, work, n_work, node_first, node_items, nullptr, nullptr, max_items,
+             overflow);
+    return;
+  }
+  __shared__ Cand s_cand[16];
+  __shared__ int s_fid[16];
+  const int nd = blockIdx.x, wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  const NodeSum t = tot[nd];
+  Cand mine;
+  mine.gain = 0.0f;
+  mine.bin = -1;
+  mine.left.g = mine.left.h = 0;
+  mine.left.c = 0;
+  int mine_fid = -1;
+  for (int f = wave; f < F; f += 16) {
+    if (active && !active[f]) continue;  // feature not sampled at this level
+    const Cand c = ScanFeature<PAIR, F64>(hg, hh, hc, (size_t)nd * nbin_total + (size_t)f * slots, slots, t, shifts,
+                                          gp, hist_size, lane);
+    if (c.bin >= 0 && (mine_fid < 0 || mine.gain < c.gain)) {  // features ascend: ties keep the lower id
+      mine = c;
+      mine_fid = f;
+    }
+  }
+  if (lane == 0) {
+    s_cand[wave] = mine;
+    s_fid[wave] = mine_fid;
+  }
+  __syncthreads();
+  if (wave != 0) return;
+  float gain = 0.0f;
+  int fid = -1, bin = -1;
+  long long lg = 0, lh = 0;
+  unsigned long long lc = 0;
+  if (lane < 16 && s_fid[lane] >= 0) {
+    const Cand c = s_cand[lane];
+    gain = c.gain;
+    fid = s_fid[lane];
+    bin = c.bin;
+    lg = c.left.g;
+    lh = c.left.h;
+    lc = c.left.c;
+  }
+  for (int off = 8; off > 0; off >>= 1) {
+    const float og = __shfl_down(gain, off);
+    const int of = __shfl_down(fid, off);
+    const int ob = __shfl_down(bin, off);
+    const long long olg = __shfl_down(lg, off);
+    const long long olh = __shfl_down(lh, off);
+    const unsigned long long olc = __shfl_down(lc, off);
+    if (of >= 0 && (fid < 0 || og > gain || (og == gain && of < fid))) {
+      gain = og;
+      fid = of;
+      bin = ob;
+      lg = olg;
+      lh = olh;
+      lc = olc;
+    }
+  }
+  if (lane != 0) return;
+  WriteNode(nd, t, gain, fid, bin, lg, lh, lc, seg_start, tot_next, seg_next, split, t_fid, t_bin, t_gain, heap_off);
+  if (plan && rows_scanned && t.c != 0) {
+    const unsigned long long cl = fid < 0 ? t.c : lc;
+    atomicAdd(rows_scanned, min(cl, t.c - cl));
+  }
 }
 
 }  // namespace
