@@ -377,24 +377,24 @@ struct FusedArgs {
   int q0;                      // first quad of this launch
 };
 
-template <bool PAIR, int NQ, bool WRITE, bool GROUP>
+template <bool PAIR, int NQ, bool WRITE, bool GROUP, bool PACK>
 void LaunchFusedNQ(hipStream_t st, unsigned grid, const FusedArgs &a) {
   const size_t lds = HistLdsBytes(NQ, PAIR);
   static bool configured = false;
   if (!configured) {
-    AllowLds(k_part_hist<PAIR, NQ, WRITE, GROUP>, lds);
+    AllowLds(k_part_hist<PAIR, NQ, WRITE, GROUP, PACK>, lds);
     configured = true;
   }
-  hipLaunchKernelGGL((k_part_hist<PAIR, NQ, WRITE, GROUP>), dim3(grid), dim3(kHistThreads), lds, st,
+  hipLaunchKernelGGL((k_part_hist<PAIR, NQ, WRITE, GROUP, PACK>), dim3(grid), dim3(kHistThreads), lds, st,
                      a.bins + (size_t)a.q0 * a.stride, a.bins_out ? a.bins_out + (size_t)a.q0 * a.stride : nullptr,
                      a.stride, a.F, a.g, a.g_out, a.h, a.h_out, a.shifts, a.split, a.tot, a.seg_start, a.work,
                      a.n_work, a.wave_left, a.item_left, a.slab, a.slab_entries, a.split_bins, a.q0);
 }
 
-template <bool PAIR, bool WRITE, bool GROUP>
+template <bool PAIR, bool WRITE, bool GROUP, bool PACK>
 void LaunchFused(int nq, hipStream_t st, unsigned grid, const FusedArgs &a) {
 #define ARB_CASE(N) \
-  case N: LaunchFusedNQ<PAIR, N, WRITE, GROUP>(st, grid, a); break;
+  case N: LaunchFusedNQ<PAIR, N, WRITE, GROUP, PACK>(st, grid, a); break;
   switch (nq) {
     ARB_CASE(1) ARB_CASE(2) ARB_CASE(3) ARB_CASE(4) ARB_CASE(5) ARB_CASE(6) ARB_CASE(7) ARB_CASE(8)
     default: throw std::runtime_error("internal: bad quad count");
@@ -451,8 +451,14 @@ class HipTreeBuilder : public TreeBuilder {
     d_y_ = DevAlloc<float>(n_);
     d_labels_ = DevAlloc<uint8_t>(n_);
     d_yhat_ = DevAlloc<float>(n_ * K_);
+    streamed_ = dm_->streamed;
+    // Logistic gradients of 0/1 labels travel as one float per row (PackGrad):
+    // there is no h array then, and kernels given h == nullptr unpack g.
+    pack_ = cfg.objective == kLogisticRegression && !streamed_ && !wide_ && single_group_ &&
+            data->y.size() == n_ &&
+            std::all_of(data->y.begin(), data->y.end(), [](float v) { return v == 0.0f || v == 1.0f; });
     d_g_ = DevAlloc<float>(n_ * K_);
-    d_h_ = DevAlloc<float>(n_ * K_);
+    d_h_ = pack_ ? nullptr : DevAlloc<float>(n_ * K_);
     d_leaf_ = DevAlloc<unsigned>(n_);
     if (!data->y.empty()) HIP_OK(hipMemcpy(d_y_, data->y.data(), n_ * sizeof(float), hipMemcpyHostToDevice));
     if (!data->labels.empty()) HIP_OK(hipMemcpy(d_labels_, data->labels.data(), n_, hipMemcpyHostToDevice));
@@ -461,7 +467,6 @@ class HipTreeBuilder : public TreeBuilder {
     hipLaunchKernelGGL(k_fill_f32, dim3(GridFor(n_ * K_, 256)), dim3(256), 0, stream_, d_yhat_, init, n_ * K_);
     data->y_hat.assign(n_ * K_, init);  // garden.cu:104
 
-    streamed_ = dm_->streamed;
     if (streamed_) {
       const size_t br = dm_->block_rows;
       HIP_OK(hipStreamCreateWithFlags(&copy_stream_, hipStreamNonBlocking));
@@ -485,7 +490,7 @@ class HipTreeBuilder : public TreeBuilder {
       for (int b = 0; b < 2; ++b) {
         buf_[b].bins = DevAlloc<uint32_t>((size_t)Q_ * stride_);
         buf_[b].g = DevAlloc<float>(n_);
-        buf_[b].h = DevAlloc<float>(n_);
+        buf_[b].h = pack_ ? nullptr : DevAlloc<float>(n_);
       }
     }
     // level state
@@ -622,6 +627,12 @@ class HipTreeBuilder : public TreeBuilder {
 
   void SetInspect(bool on) override { inspect_ = on; }
   void GetLeaves(uint32_t *out) override {
+    if (!leaf_valid_) {  // the last pass did not record them: walk the last tree now
+      hipLaunchKernelGGL(k_leaf_ids, dim3(GridFor(n_, 256, 8192)), dim3(256), 0, stream_, dm_->bins, stride_, d_tfid_,
+                         d_tbin_, D_, d_leaf_, n_, code_);
+      HIP_OK(hipGetLastError());
+      leaf_valid_ = true;
+    }
     HIP_OK(hipStreamSynchronize(stream_));
     HIP_OK(hipMemcpy(out, d_leaf_, n_ * sizeof(unsigned), hipMemcpyDeviceToHost));
   }
@@ -633,7 +644,14 @@ class HipTreeBuilder : public TreeBuilder {
     if (!inspect_) throw std::runtime_error("gradients of the last round are only kept with inspection on");
     HIP_OK(hipStreamSynchronize(stream_));
     HIP_OK(hipMemcpy(g, d_g_, n_ * K_ * sizeof(float), hipMemcpyDeviceToHost));
-    if (h) {
+    if (pack_) {
+      for (size_t i = 0; i < n_; ++i) {
+        float gv, hv;
+        UnpackGrad(g[i], &gv, &hv);
+        g[i] = gv;
+        if (h) h[i] = hv;
+      }
+    } else if (h) {
       if (pair_)
         HIP_OK(hipMemcpy(h, d_h_, n_ * K_ * sizeof(float), hipMemcpyDeviceToHost));
       else
@@ -804,7 +822,7 @@ class HipTreeBuilder : public TreeBuilder {
     RowBuffers orig;
     orig.bins = dm_->bins;
     orig.g = d_g_ + (size_t)label * n_;
-    orig.h = d_h_ + (size_t)label * n_;
+    orig.h = d_h_ ? d_h_ + (size_t)label * n_ : nullptr;
     if (inspect_) kept_hist_.assign(D_ - 1, {});
     SampleColumns();
     if (streamed_) {
@@ -848,10 +866,11 @@ class HipTreeBuilder : public TreeBuilder {
             FusedArgs a{src.bins, last ? nullptr : dst.bins, stride_, F_, src.g, q0 == 0 ? dst.g : nullptr, src.h,
                         q0 == 0 ? dst.h : nullptr, d_shifts_, d_split_, d_tot_[ps], d_seg_[ps], d_pwork_,
                         d_nwork_ + 1, d_wave_left_, d_item_left_, d_slab_, slab_entries_, src.bins, q0};
-#define ARB_FUSED(P, W)                                        \
-  do {                                                         \
-    if (single_group_) LaunchFused<P, W, false>(nq, stream_, grid, a); \
-    else LaunchFused<P, W, true>(nq, stream_, grid, a);        \
+#define ARB_FUSED(P, W)                                                       \
+  do {                                                                        \
+    if (P && pack_) LaunchFused<P, W, false, P>(nq, stream_, grid, a);        \
+    else if (single_group_) LaunchFused<P, W, false, false>(nq, stream_, grid, a); \
+    else LaunchFused<P, W, true, false>(nq, stream_, grid, a);                \
   } while (0)
             if (pair_) {
               if (last) ARB_FUSED(true, false);
@@ -900,8 +919,10 @@ class HipTreeBuilder : public TreeBuilder {
         Plan(0, 1, 0, per_item, d_hwork_, d_nwork_, true, nullptr, grid);
         LaunchFinalHist(grid, label, lds);
         root_hist_ready_ = true;
+        leaf_valid_ = false;  // not recorded by this pass; GetLeaves walks the tree when asked
       } else {
         LaunchFinal(dm_->bins, stride_, 0, n_, label, next_grad);
+        leaf_valid_ = true;
       }
       grad_ready_ = next_grad;
     }
@@ -989,7 +1010,7 @@ class HipTreeBuilder : public TreeBuilder {
 #define ARB_PART_N(N)                                          \
   case N:                                                      \
     if (q0 == 0) {                                             \
-      if (pair_) ARB_PART(true, N, true);                      \
+      if (pair_ && !pack_) ARB_PART(true, N, true);            \
       else ARB_PART(false, N, true);                           \
     } else {                                                   \
       ARB_PART(false, N, false);                               \
@@ -1031,7 +1052,7 @@ class HipTreeBuilder : public TreeBuilder {
     if (next_grad && cfg_.objective == kLogisticRegression) mode = 2;
 #define ARB_FINAL(M, N) \
   hipLaunchKernelGGL((k_final<M, N>), dim3(grid), dim3(256), lds, stream_, bins, stride, d_tfid_, d_tbin_, D_, \
-                     d_weights_, yh, d_y_ + row0, d_leaf_ + row0, d_g_ + row0, d_h_ + row0, d_gmax_, rows, code_)
+                     d_weights_, yh, d_y_ + row0, d_leaf_ + row0, d_g_ + row0, d_h_ ? d_h_ + row0 : nullptr, d_gmax_, rows, code_)
 #define ARB_FINAL_Q(N) \
   do { if (mode == 1) ARB_FINAL(1, N); else if (mode == 2) ARB_FINAL(2, N); else ARB_FINAL(0, N); } while (0)
     switch (Q_ <= 8 && !wide_ ? Q_ : 0) {
@@ -1059,8 +1080,8 @@ class HipTreeBuilder : public TreeBuilder {
       configured = true;                                                                                         \
     }                                                                                                            \
     hipLaunchKernelGGL((k_final_hist<N>), dim3(grid), dim3(kHistThreads), lds, stream_, dm_->bins, stride_, F_, \
-                       d_tfid_, d_tbin_, D_, d_weights_, yh, d_y_, d_leaf_, d_g_, d_h_, d_shifts_, d_hwork_,     \
-                       d_nwork_, d_slab_, slab_entries_);                                                        \
+                       d_tfid_, d_tbin_, D_, d_weights_, yh, d_y_, (unsigned *)nullptr, d_g_, d_h_, d_shifts_,   \
+                       d_hwork_, d_nwork_, d_slab_, slab_entries_);                                              \
   } break;
     switch (Q_) {
       ARB_CASE(1) ARB_CASE(2) ARB_CASE(3) ARB_CASE(4) ARB_CASE(5) ARB_CASE(6) ARB_CASE(7) ARB_CASE(8)
@@ -1226,6 +1247,8 @@ class HipTreeBuilder : public TreeBuilder {
   // streamed matrices: two block buffers filled by the copy stream, a staging
   // buffer with the rows of the built nodes, a resident node id per row
   bool streamed_ = false;
+  bool leaf_valid_ = true;  // d_leaf_ holds the leaves of the last tree
+  bool pack_ = false;  // logistic gradients packed into one float per row, no h arrays
   hipStream_t copy_stream_ = nullptr;
   uint32_t *blk_[2] = {nullptr, nullptr};
   hipEvent_t ev_ready_[2] = {nullptr, nullptr}, ev_free_[2] = {nullptr, nullptr};

@@ -46,6 +46,27 @@ constexpr size_t HistLdsBytes(int nq, bool pair) {
   return (size_t)HistBlocks(nq) * kBlockEntries * 8 * (pair ? 2 : 1);
 }
 
+// Logistic gradients of 0/1 labels can travel as ONE float per row:
+// u = s with the sign bit set when y = 1, s = sigmoid(y_hat) >= 0.  The pair
+// (g, h) = (y - s, s (1 - s)) is recomputed where it is used, with the very
+// operations of the gradient kernel, so the values are bit-identical; the row
+// passes then move four bytes less per row and direction.
+__host__ __device__ __forceinline__ float PackGrad(float s, float y) {
+  union { float f; uint32_t u; } v;
+  v.f = s;
+  v.u |= (y != 0.0f) ? 0x80000000u : 0u;
+  return v.f;
+}
+__host__ __device__ __forceinline__ void UnpackGrad(float u, float *g, float *h) {
+  union { float f; uint32_t u; } v;
+  v.f = u;
+  const float y = (v.u >> 31) ? 1.0f : 0.0f;
+  v.u &= 0x7fffffffu;
+  const float s = v.f;
+  *g = y - s;
+  *h = s * (1.0f - s);
+}
+
 struct NodeSum {
   long long g;
   long long h;

@@ -37,7 +37,7 @@ __global__ void k_leaf_weights(const SplitRec *__restrict__ split, const NodeSum
 // (bin >= q+1 goes right, builder.h:107-123), record the leaf, add its weight
 // to y_hat (update_by_last_tree, garden.cu:45-76) and, when NEXT_GRAD is not
 // 0, write the gradients of the next round (objective.cu:28-56):
-// 1 = squared (also max |g|), 2 = logistic.
+// 1 = squared (also max |g|), 2 = logistic (h == nullptr: packed into g, PackGrad).
 // NQ > 0: the matrix has NQ quads, all loaded up front (coalesced, independent
 // loads) and selected in registers; NQ == 0: any width, one dependent 4-byte
 // load per level.
@@ -91,8 +91,12 @@ k_final(const uint32_t *__restrict__ bins, size_t stride, const int *__restrict_
       if (a > m) m = a;
     } else if (NEXT_GRAD == 2) {
       const float s = SigmoidF(yh);
-      g[i] = yv - s;
-      h[i] = s * (1.0f - s);
+      if (h != nullptr) {
+        g[i] = yv - s;
+        h[i] = s * (1.0f - s);
+      } else {
+        g[i] = PackGrad(s, yv);
+      }
     }
   }
   if (NEXT_GRAD == 1) {
@@ -106,6 +110,8 @@ k_final(const uint32_t *__restrict__ bins, size_t stride, const int *__restrict_
 // rows are read once; the leaf walk, the prediction update and the new
 // gradients are bound by HBM, the histogram by LDS atomics, and they overlap.
 // One workgroup per root work item; LDS: histogram, then the node arrays.
+// leaf_of may be null: the leaf ids are then not recorded (k_leaf_ids
+// computes them on demand).
 template <int NQ>
 __global__ void __launch_bounds__(kHistThreads)
 k_final_hist(const uint32_t *__restrict__ bins, size_t stride, int F, const int *__restrict__ t_fid,
@@ -143,13 +149,17 @@ k_final_hist(const uint32_t *__restrict__ bins, size_t stride, int F, const int 
       }
       node = node * 2 + right;
     }
-    __builtin_nontemporal_store(node, &leaf_of[r]);
+    if (leaf_of != nullptr) __builtin_nontemporal_store(node, &leaf_of[r]);  // uniform
     const float yh = p + weights[node];
     yhat[r] = yh;
     const float s = SigmoidF(yh);
     const float gv = yv - s, hv = s * (1.0f - s);
-    g[r] = gv;
-    h[r] = hv;
+    if (h != nullptr) {  // uniform
+      g[r] = gv;
+      h[r] = hv;
+    } else {
+      g[r] = PackGrad(s, yv);
+    }
     AccumulateRow<true, NQ>(lds, b, gv, hv, sg, sh, 0, F);
   };
   for (unsigned base = it.begin; base < it.end; base += 2 * kHistThreads) {
@@ -168,6 +178,25 @@ k_final_hist(const uint32_t *__restrict__ bins, size_t stride, int F, const int 
     if (v1) row(b1, p1, y1, r1);
   }
   FlushSlab<true, NQ>(lds, slab, w, slab_entries, 0);
+}
+
+// Leaf of every row under the tree in t_fid / t_bin (heap order), for a
+// caller that asks after a last pass that did not record the leaves.
+__global__ void __launch_bounds__(256)
+k_leaf_ids(const uint32_t *__restrict__ bins, size_t stride, const int *__restrict__ t_fid,
+           const int *__restrict__ t_bin, int depth, unsigned *__restrict__ leaf_of, size_t n, BinCode code) {
+  for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < n;
+       i += (size_t)gridDim.x * blockDim.x) {
+    unsigned node = 0;
+    for (int level = 0; level + 1 < depth; ++level) {
+      const int id = (1 << level) - 1 + (int)node;
+      const int fid = t_fid[id], bin = t_bin[id];
+      unsigned right = 0;
+      if (bin >= 0) right = (int)code.Bin(bins[(size_t)code.Word(fid) * stride + i], fid) > bin ? 1u : 0u;
+      node = node * 2 + right;
+    }
+    leaf_of[i] = node;
+  }
 }
 
 // Tree record of the tree just grown into one slot of the record ring:

@@ -82,6 +82,7 @@ __device__ __forceinline__ void FlushSlab(const unsigned long long *__restrict__
 
 // Histogram of contiguous row ranges: one workgroup per work item, quads
 // [q0, q0+NQ).  LDS: NQ*1024 word0 entries, then (PAIR) as many word1 entries.
+// PAIR with h == nullptr: g holds packed logistic gradients (PackGrad).
 template <bool PAIR, int NQ>
 __global__ void __launch_bounds__(kHistThreads)
 k_hist(const uint32_t *__restrict__ bins, size_t stride, int q0, int F,
@@ -107,8 +108,17 @@ k_hist(const uint32_t *__restrict__ bins, size_t stride, int q0, int F,
       b0[q] = __builtin_nontemporal_load(&bq[(size_t)q * stride + a0]);
       b1[q] = __builtin_nontemporal_load(&bq[(size_t)q * stride + a1]);
     }
-    const float g0 = g[a0], g1 = g[a1];
-    const float h0 = PAIR ? h[a0] : 0.0f, h1 = PAIR ? h[a1] : 0.0f;
+    float g0 = g[a0], g1 = g[a1];
+    float h0 = 0.0f, h1 = 0.0f;
+    if (PAIR) {
+      if (h != nullptr) {  // uniform
+        h0 = h[a0];
+        h1 = h[a1];
+      } else {  // packed logistic gradients
+        UnpackGrad(g0, &g0, &h0);
+        UnpackGrad(g1, &g1, &h1);
+      }
+    }
     if (v0) AccumulateRow<PAIR, NQ>(lds, b0, g0, h0, sg, sh, q0, F);
     if (v1) AccumulateRow<PAIR, NQ>(lds, b1, g1, h1, sg, sh, q0, F);
   }

@@ -31,14 +31,19 @@ __global__ void k_set_shift(const unsigned *__restrict__ gmax_bits, int *__restr
   }
 }
 
-// logistic: s = sigmoid(y_hat), g = y - s, h = s(1-s) (objective.cu:43-56)
+// logistic: s = sigmoid(y_hat), g = y - s, h = s(1-s) (objective.cu:43-56);
+// h == nullptr: packed into g (PackGrad)
 __global__ void k_grad_logistic(const float *__restrict__ y, const float *__restrict__ yhat,
                                 float *__restrict__ g, float *__restrict__ h, size_t n) {
   for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < n;
        i += (size_t)gridDim.x * blockDim.x) {
     const float s = SigmoidF(yhat[i]);
-    g[i] = y[i] - s;
-    h[i] = s * (1.0f - s);
+    if (h != nullptr) {
+      g[i] = y[i] - s;
+      h[i] = s * (1.0f - s);
+    } else {  // 0/1 labels: one float per row
+      g[i] = PackGrad(s, y[i]);
+    }
   }
 }
 

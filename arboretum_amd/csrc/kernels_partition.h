@@ -149,8 +149,9 @@ struct RowQueue {
 
 // Writes lanes [from, to) of Q to their destination and, for the child whose
 // histogram is built, adds them to the LDS histogram.
-// HIST: the kernel builds a histogram; GH: the gradients move with the rows.
-template <bool PAIR, int NQ, bool HIST = true, bool GH = true>
+// HIST: the kernel builds a histogram; GH: the gradients move with the rows;
+// PACK: Q.g holds packed logistic gradients (PackGrad), there is no h array.
+template <bool PAIR, int NQ, bool HIST = true, bool GH = true, bool PACK = false>
 __device__ __forceinline__ void EmitRows(unsigned long long *__restrict__ lds, const RowQueue<NQ> &Q,
                                          unsigned from, unsigned to, bool built,
                                          uint32_t *__restrict__ bins_out, size_t stride,
@@ -163,16 +164,20 @@ __device__ __forceinline__ void EmitRows(unsigned long long *__restrict__ lds, c
     for (int q = 0; q < NQ; ++q) __builtin_nontemporal_store(Q.b[q], &bins_out[(size_t)q * stride + d]);
     if (GH && g_out != nullptr) {  // a group pass after the first leaves the gradients alone
       __builtin_nontemporal_store(Q.g, &g_out[d]);
-      if (PAIR) __builtin_nontemporal_store(Q.h, &h_out[d]);
+      if (PAIR && !PACK) __builtin_nontemporal_store(Q.h, &h_out[d]);
     }
-    if (HIST && built) AccumulateRow<PAIR, NQ>(lds, Q.b, Q.g, Q.h, sg, sh, 0, F);
+    if (HIST && built) {
+      float gv = Q.g, hv = Q.h;
+      if (PACK) UnpackGrad(Q.g, &gv, &hv);
+      AccumulateRow<PAIR, NQ>(lds, Q.b, gv, hv, sg, sh, 0, F);
+    }
   }
 }
 
 // Appends the rows of X flagged in xm (wave-uniform mask, one row per lane) to
 // Q in row order with one lane permute per register; a full queue is emitted
 // and the rest of X starts the next batch.
-template <bool PAIR, int NQ, bool HIST = true, bool GH = true>
+template <bool PAIR, int NQ, bool HIST = true, bool GH = true, bool PACK = false>
 __device__ __forceinline__ void MergeRows(unsigned long long *__restrict__ lds, RowQueue<NQ> &Q,
                                           const uint32_t (&xb)[NQ], float xg, float xh,
                                           unsigned long long xm, bool built,
@@ -189,14 +194,14 @@ __device__ __forceinline__ void MergeRows(unsigned long long *__restrict__ lds, 
 #pragma unroll
   for (int q = 0; q < NQ; ++q) vb[q] = (uint32_t)__shfl((int)xb[q], src);
   const float vg = GH ? __shfl(xg, src) : 0.0f;
-  const float vh = GH && PAIR ? __shfl(xh, src) : 0.0f;
+  const float vh = GH && PAIR && !PACK ? __shfl(xh, src) : 0.0f;
   if (Q.n + nx >= 64u) {  // wave-uniform: the batch is complete
     const bool fill = (unsigned)lane >= Q.n;
 #pragma unroll
     for (int q = 0; q < NQ; ++q) Q.b[q] = fill ? vb[q] : Q.b[q];
     Q.g = fill ? vg : Q.g;
     Q.h = fill ? vh : Q.h;
-    EmitRows<PAIR, NQ, HIST, GH>(lds, Q, Q.skip, 64u, built, bins_out, stride, g_out, h_out, lane, sg, sh, F);
+    EmitRows<PAIR, NQ, HIST, GH, PACK>(lds, Q, Q.skip, 64u, built, bins_out, stride, g_out, h_out, lane, sg, sh, F);
     Q.base += 64u;
     Q.skip = 0u;
 #pragma unroll
@@ -230,7 +235,9 @@ __device__ __forceinline__ void MergeRows(unsigned long long *__restrict__ lds, 
 // of 4); the quad of the split feature is read from `split_bins`, the start of
 // the whole matrix, and g_out may be null (the gradients moved with an
 // earlier group of the same level).
-template <bool PAIR, int NQ, bool WRITE, bool GROUP = false>
+// PACK (with PAIR): g holds packed logistic gradients (PackGrad); h and h_out
+// are not touched.
+template <bool PAIR, int NQ, bool WRITE, bool GROUP = false, bool PACK = false>
 __global__ void __launch_bounds__(kHistThreads)
 k_part_hist(const uint32_t *__restrict__ bins, uint32_t *__restrict__ bins_out, size_t stride, int F,
             const float *__restrict__ g, float *__restrict__ g_out, const float *__restrict__ h,
@@ -283,8 +290,8 @@ k_part_hist(const uint32_t *__restrict__ bins, uint32_t *__restrict__ bins_out, 
       }
       R.g0 = __builtin_nontemporal_load(&g[a0]);
       R.g1 = __builtin_nontemporal_load(&g[a1]);
-      R.h0 = PAIR ? __builtin_nontemporal_load(&h[a0]) : 0.0f;
-      R.h1 = PAIR ? __builtin_nontemporal_load(&h[a1]) : 0.0f;
+      R.h0 = PAIR && !PACK ? __builtin_nontemporal_load(&h[a0]) : 0.0f;
+      R.h1 = PAIR && !PACK ? __builtin_nontemporal_load(&h[a1]) : 0.0f;
     };
     auto process = [&](const RowSet<NQ> &R, unsigned base) {
       const unsigned r0 = base + lane, r1 = r0 + 64;
@@ -304,10 +311,10 @@ k_part_hist(const uint32_t *__restrict__ bins, uint32_t *__restrict__ bins_out, 
       const bool right1 = v1 && s.fid >= 0 && (int)((s1 >> fs) & 255u) > s.bin;
       const unsigned long long b0 = __ballot(v0 && right0 == build_right), o0 = __ballot(v0 && right0 != build_right);
       const unsigned long long b1 = __ballot(v1 && right1 == build_right), o1 = __ballot(v1 && right1 != build_right);
-      MergeRows<PAIR, NQ>(lds, QO, R.b0, R.g0, R.h0, o0, false, bins_out, stride, g_out, h_out, lane, sg, sh, F);
-      MergeRows<PAIR, NQ>(lds, QB, R.b0, R.g0, R.h0, b0, true, bins_out, stride, g_out, h_out, lane, sg, sh, F);
-      MergeRows<PAIR, NQ>(lds, QO, R.b1, R.g1, R.h1, o1, false, bins_out, stride, g_out, h_out, lane, sg, sh, F);
-      MergeRows<PAIR, NQ>(lds, QB, R.b1, R.g1, R.h1, b1, true, bins_out, stride, g_out, h_out, lane, sg, sh, F);
+      MergeRows<PAIR, NQ, true, true, PACK>(lds, QO, R.b0, R.g0, R.h0, o0, false, bins_out, stride, g_out, h_out, lane, sg, sh, F);
+      MergeRows<PAIR, NQ, true, true, PACK>(lds, QB, R.b0, R.g0, R.h0, b0, true, bins_out, stride, g_out, h_out, lane, sg, sh, F);
+      MergeRows<PAIR, NQ, true, true, PACK>(lds, QO, R.b1, R.g1, R.h1, o1, false, bins_out, stride, g_out, h_out, lane, sg, sh, F);
+      MergeRows<PAIR, NQ, true, true, PACK>(lds, QB, R.b1, R.g1, R.h1, b1, true, bins_out, stride, g_out, h_out, lane, sg, sh, F);
     };
     if (wb < we) {
       RowSet<NQ> A, B;
@@ -321,8 +328,8 @@ k_part_hist(const uint32_t *__restrict__ bins, uint32_t *__restrict__ bins_out, 
         if (base + 2 * kChunkStep >= we) break;
       }
     }
-    EmitRows<PAIR, NQ>(lds, QO, QO.skip, QO.n, false, bins_out, stride, g_out, h_out, lane, sg, sh, F);
-    EmitRows<PAIR, NQ>(lds, QB, QB.skip, QB.n, true, bins_out, stride, g_out, h_out, lane, sg, sh, F);
+    EmitRows<PAIR, NQ, true, true, PACK>(lds, QO, QO.skip, QO.n, false, bins_out, stride, g_out, h_out, lane, sg, sh, F);
+    EmitRows<PAIR, NQ, true, true, PACK>(lds, QB, QB.skip, QB.n, true, bins_out, stride, g_out, h_out, lane, sg, sh, F);
   } else {
     // Rows selected for the histogram are queued by row id (slot 64 * j + lane
     // of the queue is lane `lane` of q[j]; slots [0, np) are occupied) and read
@@ -339,7 +346,7 @@ k_part_hist(const uint32_t *__restrict__ bins, uint32_t *__restrict__ bins_out, 
 #pragma unroll
       for (int q = 0; q < NQ; ++q) gb[q] = bins[(size_t)q * stride + a];
       gg = g[a];
-      gh = PAIR ? h[a] : 0.0f;
+      gh = PAIR && !PACK ? h[a] : 0.0f;
       q0 = q1;
       q1 = q2;
     };
@@ -363,6 +370,7 @@ k_part_hist(const uint32_t *__restrict__ bins, uint32_t *__restrict__ bins_out, 
         const unsigned take = min(np, 64u);
         const bool valid = (unsigned)lane < take;
         gather(valid);
+        if (PACK) UnpackGrad(gg, &gg, &gh);
         if (valid) AccumulateRow<PAIR, NQ>(lds, gb, gg, gh, sg, sh, 0, F);
         np -= take;
       }
@@ -385,7 +393,10 @@ k_part_hist(const uint32_t *__restrict__ bins, uint32_t *__restrict__ bins_out, 
         const bool right1 = v1 && s.fid >= 0 && (int)((s1 >> fs) & 255u) > s.bin;
         enqueue(base, __ballot(v0 && right0 == build_right));
         enqueue(base + 64, __ballot(v1 && right1 == build_right));
-        if (full) AccumulateRow<PAIR, NQ>(lds, gb, gg, gh, sg, sh, 0, F);
+        if (full) {
+          if (PACK) UnpackGrad(gg, &gg, &gh);
+          AccumulateRow<PAIR, NQ>(lds, gb, gg, gh, sg, sh, 0, F);
+        }
         drain(127u);
       };
       uint32_t a0 = col[min(wb + lane, we - 1)], a1 = col[min(wb + 64 + lane, we - 1)], b0, b1;

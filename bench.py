@@ -215,10 +215,12 @@ def main():
 
     F = args.features
     updates = scanned * F
-    row_bytes = F + 8  # uint8 bins of all features + one (g, h) pair
+    row_bytes = F + 8  # uint8 bins of all features + one (g, h) pair: the algorithmic figure
+    # what the kernels move: with 0/1 labels (this workload) the pair travels as one float
+    moved_row_bytes = F + 4
     cell_bytes = 16    # one histogram cell as written by a workgroup (two 64-bit words)
     # Dominant kernel: the fused partition + histogram pass of levels 1..max_depth-2
-    # (k_part_hist<true, 7, true, false>).  Algorithmic bytes of one launch: every row is
+    # (k_part_hist<true, 7, true, false, true>).  Algorithmic bytes of one launch: every row is
     # read once and written once in the children order, and the smaller child of
     # each parent gets one histogram written.
     fl = max(fused_launches_timed, 1)
@@ -232,7 +234,7 @@ def main():
     # root level (k_hist<true, 7>): reads every row, writes one histogram
     root_bytes = tm["hist_root_rows"] * row_bytes + phase_trees * F * 256 * cell_bytes
     root_s = tm["hist_root_ms"] * 1e-3
-    # last level (k_part_hist<true, 7, false, false>): moves no rows; reads the split feature's quad
+    # last level (k_part_hist<true, 7, false, false, true>): moves no rows; reads the split feature's quad
     # of every row and then the rows of the smaller children, which are spread over nearly every
     # 32-byte sector: counted as one full read of the rows (the counters show 387 MiB fetched)
     last_bytes = tm["fused_last_launches"] * args.rows * row_bytes
@@ -248,7 +250,7 @@ def main():
     def frac(b, t):
         return (b / t) / HBM_PEAK if t > 0 else 0.0
 
-    other = {"k_part_hist<true,7,false,false> (last level)": {
+    other = {"k_part_hist<true,7,false,false,true> (last level)": {
         "frac_of_hbm": frac(last_bytes, last_s),
         "avg_launch_us": tm["fused_last_ms"] * 1e3 / max(tm["fused_last_launches"], 1)}}
     if tm["hist_root_launches"] > 0:
@@ -286,11 +288,13 @@ def main():
                    "rows": args.rows, "features": F, "bins": args.hist_size, "max_depth": args.max_depth},
         "roofline": {"bound": "hbm", "achieved": achieved / 1e9, "peak": HBM_PEAK / 1e9, "unit": "GB/s",
                      "frac": achieved / HBM_PEAK, "traffic": traffic,
-                     "kernel": "k_part_hist<true,7,true,false> (fused partition + histogram, levels 1..%d)"
+                     "kernel": "k_part_hist<true,7,true,false,true> (fused partition + histogram, levels 1..%d)"
                                % (args.max_depth - 2),
                      "launches": int(fused_launches_timed),
                      "avg_launch_us": fused_ms_timed * 1e3 / fl,
-                     "bytes_per_launch": fused_bytes / fl},
+                     "bytes_per_launch": fused_bytes / fl,
+                     # (g, h) packed in 4 bytes: bytes the kernel needs to move per launch
+                     "bytes_moved_per_launch": (fused_bytes - fl * args.rows * 2 * (row_bytes - moved_row_bytes)) / fl},
         "other_kernels": other,
         "tree_algorithmic_floor_frac_of_hbm": (2.9e9 / (dt / args.steps)) / HBM_PEAK,
         "phase_ms_per_tree": dict({k: v / phase_trees for k, v in tm.items() if k.endswith("_ms")},

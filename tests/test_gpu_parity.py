@@ -145,6 +145,20 @@ def test_training_without_inspection(arb, oracle, objective):
     assert_same_training(arb, oracle, X, y, cfg, rounds=4, check_hist=False)
 
 
+@pytest.mark.parametrize("inspect", [True, False])
+@pytest.mark.parametrize("trick", [True, False])
+def test_logistic_with_fractional_labels(arb, oracle, inspect, trick):
+    # 0/1 labels let the builder carry (g, h) as one float per row; any other label value
+    # takes the two-array path, which must give the same bits as the checker too
+    X, y = make_data(30000, 13, 1, seed=31, nan_frac=0.01)
+    y[::3] = 0.25
+    y[1::7] = 0.5
+    cfg = {"objective": 1, "method": 1,
+           "internals": {"hist_size": 100, "double_precision": True, "use_hist_subtraction_trick": trick},
+           "tree": {"max_depth": 6, "eta": 0.3, "lambda": 1.0}}
+    assert_same_training(arb, oracle, X, y, cfg, rounds=4, check_hist=inspect)
+
+
 @pytest.mark.parametrize("n,F,depth", [(1, 3, 2), (65, 1, 1), (2049, 5, 3), (70000, 8, 4), (5000, 32, 5)])
 def test_last_pass_feeds_next_root_histogram(arb, oracle, n, F, depth):
     # logistic, inspection off: the pass that assigns the leaves of a tree also
