@@ -506,9 +506,9 @@ class HipTreeBuilder : public TreeBuilder {
     d_cand_ = DevAlloc<Cand>((size_t)last_nodes * F_);
     d_node_first_ = DevAlloc<unsigned>(last_nodes);
     d_node_items_ = DevAlloc<unsigned>(last_nodes);
-    max_hist_items_ = (unsigned)(n_ / HistRowsPerItem(n_)) + last_nodes + 2;
-    max_hist_items_ = std::max<unsigned>(max_hist_items_, 1024 + last_nodes + 2);
-    max_part_items_ = std::max<unsigned>((unsigned)(n_ / kPartRows + 1) + last_nodes, max_hist_items_);
+    max_hist_items_ = (unsigned)(n_ / HistRowsPerItem(n_)) + 2 * last_nodes + 2;
+    max_hist_items_ = std::max<unsigned>(max_hist_items_, 1024 + 2 * last_nodes + 2);
+    max_part_items_ = std::max<unsigned>((unsigned)(n_ / kPartRows + 1) + 2 * last_nodes, max_hist_items_);
     d_hwork_ = DevAlloc<WorkItem>(max_hist_items_);
     d_pwork_ = DevAlloc<WorkItem>(max_part_items_);
     d_nwork_ = DevAlloc<unsigned>(2);
@@ -763,7 +763,7 @@ class HipTreeBuilder : public TreeBuilder {
   void HistOfNodes(const RowBuffers &cur, int state, int L, bool select_smaller, size_t rows_max, bool root) {
     // the root level is one node: one item per CU avoids a second, partial round
     const unsigned per_item = HistRowsPerItem(rows_max, root ? 256 : 512);
-    const unsigned grid = (unsigned)std::min<size_t>(rows_max / per_item + L + 1, max_hist_items_);
+    const unsigned grid = (unsigned)std::min<size_t>(rows_max / per_item + 2 * L + 1, max_hist_items_);
     Mark(kPlan);
     Plan(state, L, select_smaller ? 1 : 0, per_item, d_hwork_, d_nwork_, true, nullptr, grid);
     Mark(root ? kHistRoot : kHistDeep);
@@ -885,7 +885,7 @@ class HipTreeBuilder : public TreeBuilder {
           }
           Reduce(L, hb, true, ps, true);
         } else {
-          const unsigned grid = (unsigned)std::min<size_t>(n_ / kPartRows + PL + 1, max_part_items_);
+          const unsigned grid = (unsigned)std::min<size_t>(n_ / kPartRows + 2 * PL + 1, max_part_items_);
           Mark(kPlan);
           Plan(ps, PL, 0, kPartRows, d_pwork_, d_nwork_ + 1, false, nullptr, grid);
           Mark(kPartition);
@@ -1026,7 +1026,7 @@ class HipTreeBuilder : public TreeBuilder {
 
   // launch bound of the fused pass over PL parent nodes
   unsigned FusedGrid(int PL) const {
-    return (unsigned)std::min<size_t>(n_ / HistRowsPerItem(n_) + PL + 1, max_part_items_);
+    return (unsigned)std::min<size_t>(n_ / HistRowsPerItem(n_) + 2 * PL + 1, max_part_items_);
   }
 
   void LaunchLeafWeights(int L, int state, const GainParams &gp) {
@@ -1124,7 +1124,7 @@ class HipTreeBuilder : public TreeBuilder {
         HIP_OK(hipEventRecord(ev_free_[buf], stream_));
         // histograms of the gathered rows, added to the level's histograms
         const unsigned per_item = HistRowsPerItem(rows);
-        const unsigned grid = (unsigned)std::min<size_t>(rows / per_item + L + 1, max_hist_items_);
+        const unsigned grid = (unsigned)std::min<size_t>(rows / per_item + 2 * L + 1, max_hist_items_);
         Mark(kPlan);
         PlanOn(d_blk_tot_, d_blk_seg_, L, 0, per_item, d_hwork_, d_nwork_, true, nullptr, grid);
         Mark(level == 0 ? kHistRoot : kHistDeep);

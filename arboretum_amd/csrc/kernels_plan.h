@@ -8,7 +8,8 @@ namespace {
 
 // ------------------------------------------------------------------ planner
 // Splits the row ranges of the selected nodes of a level into work items of
-// at most `rows_per_item` rows.  select: 0 = every node, 1 = the smaller
+// at most `rows_per_item` rows (a multiple of 64; at most len / rows_per_item
+// + 2 items per node).  select: 0 = every node, 1 = the smaller
 // child of each sibling pair, ties -> left (hist_grad_sum.cu:279-294).
 // rows_scanned (optional) is advanced by the rows that will be accumulated
 // into histograms: the selected rows, or, when `split` is given (fused
@@ -42,7 +43,10 @@ __device__ __forceinline__ void PlanBody(const NodeSum *__restrict__ tot, const 
         sel = (nd & 1) ? (len < sib) : (len <= sib);
       }
       if (sel && len > 0) {
-        cnt = (unsigned)((len + rows_per_item - 1) / rows_per_item);
+        // item boundaries sit at multiples of 64 rows from the node's start
+        // rounded down to one, so that every item but a node's first begins on
+        // a 256-byte boundary of the row arrays
+        cnt = (unsigned)(((seg_start[nd] & 63u) + len + rows_per_item - 1) / rows_per_item);
         unsigned long long acc = len;
         if (split) {
           const unsigned long long cl = split[nd].left.c;
@@ -92,10 +96,11 @@ __device__ __forceinline__ void PlanBody(const NodeSum *__restrict__ tot, const 
     const unsigned start = seg_start[lo];
     const unsigned len = (unsigned)tot[lo].c;
     const unsigned k = w - s_base[lo];
+    const unsigned origin = start - (start & 63u);
     WorkItem it;
     it.node = lo;
-    it.begin = start + k * rows_per_item;
-    it.end = min(start + len, it.begin + rows_per_item);
+    it.begin = max(start, origin + k * rows_per_item);
+    it.end = min(start + len, origin + (k + 1) * rows_per_item);
     it.first = s_base[lo];
     work[w] = it;
   }
