@@ -834,6 +834,13 @@ class HipTreeBuilder : public TreeBuilder {
     if (!root_hist_ready_)
       hipLaunchKernelGGL(k_init_root, dim3(1), dim3(64), 0, stream_, d_tot_[0], d_seg_[0],
                          (unsigned long long)n_, (unsigned *)nullptr);
+    // The last pass of the tree can also build the root histogram of the next
+    // one: logistic objective, gradients of the next round wanted, all quads in
+    // one LDS histogram next to the node arrays.
+    const bool next_grad = !inspect_ && K_ == 1;
+    const size_t final_lds = HistLdsBytes(Q_, true) + (size_t)((1 << (D_ - 1)) - 1) * 2 * sizeof(int);
+    const bool final_hist = next_grad && cfg_.objective == kLogisticRegression && single_group_ && !wide_ &&
+                            final_lds <= kLdsBudget;
     int state = 0;  // d_tot_/d_seg_[state] describe the nodes of the current level
     for (int level = 0; level + 1 < D_; ++level) {
       const int L = 1 << level;
@@ -898,26 +905,32 @@ class HipTreeBuilder : public TreeBuilder {
       }
       if (inspect_) KeepHist(level, L, hb);
       LaunchSplit(level, L, hb, state, gp, fused_ && !last);
-      if (last) LaunchLeafWeights(L, state, gp);
+      if (last && !final_hist) LaunchLeafWeights(L, state, gp);
       state ^= 1;
     }
     // ---- leaf of every row, y_hat update, gradients of the next round
     Mark(kLeaf);
+    bool record_written = false;
     {
-      const bool next_grad = !inspect_ && K_ == 1;
       if (cfg_.objective == kLinearRegression) HIP_OK(hipMemsetAsync(d_gmax_, 0, sizeof(unsigned), stream_));
-      const int internal = (1 << (D_ - 1)) - 1;
-      const size_t lds = HistLdsBytes(Q_, true) + (size_t)internal * 2 * sizeof(int);
-      if (next_grad && cfg_.objective == kLogisticRegression && single_group_ && !wide_ &&
-          lds <= kLdsBudget) {
-        // plan of the next tree's root, then one pass: leaves, predictions,
-        // gradients and the root histogram of the next tree
-        hipLaunchKernelGGL(k_init_root, dim3(1), dim3(64), 0, stream_, d_tot_[0], d_seg_[0],
-                           (unsigned long long)n_, (unsigned *)nullptr);
+      if (final_hist) {
+        // leaf weights, tree record, state and plan of the next tree's root in
+        // one launch, then one pass: leaves, predictions, gradients and the
+        // root histogram of the next tree
+        const int last_L = 1 << (D_ - 2), last_state = state ^ 1;
         const unsigned per_item = HistRowsPerItem(n_, 256);
         const unsigned grid = (unsigned)std::min<size_t>(n_ / per_item + 2, max_hist_items_);
-        Plan(0, 1, 0, per_item, d_hwork_, d_nwork_, true, nullptr, grid);
-        LaunchFinalHist(grid, label, lds);
+        if ((n_ + per_item - 1) / per_item > grid) throw std::runtime_error("internal: root plan exceeds its grid");
+#define ARB_END(D)                                                                                                \
+  hipLaunchKernelGGL((k_tree_end<true, D>), dim3((last_L + 127) / 128 + 1), dim3(128), 0, stream_, d_split_,      \
+                     d_tot_[last_state], last_L, d_shifts_, gp, cfg_.tree.eta, d_weights_, d_tfid_, d_tbin_,      \
+                     d_tgain_, d_overflow_, d_records_ + pending_.size() * RecordWords(), d_tot_[0], d_seg_[0],   \
+                     (unsigned)n_, per_item, d_hwork_, d_nwork_, d_node_first_, d_node_items_, d_rows_scanned_)
+        if (f64_) ARB_END(true);
+        else ARB_END(false);
+#undef ARB_END
+        record_written = true;
+        LaunchFinalHist(grid, label, final_lds);
         root_hist_ready_ = true;
         leaf_valid_ = false;  // not recorded by this pass; GetLeaves walks the tree when asked
       } else {
@@ -926,7 +939,9 @@ class HipTreeBuilder : public TreeBuilder {
       }
       grad_ready_ = next_grad;
     }
-    EnqueueRecord();
+    if (record_written) Mark(kNone);
+    else
+      EnqueueRecord();
   }
 
   // Tree record into the next slot of the device ring; FlushTrees reads it.

@@ -33,6 +33,77 @@ __global__ void k_leaf_weights(const SplitRec *__restrict__ split, const NodeSum
   weights[2 * nd + 1] = LeafWeight<PAIR, F64>(GR, HR, (unsigned)(t.c - s.left.c), gp) * eta;
 }
 
+// Leaf weights of a finished tree and, in the same launch, what would
+// otherwise be three more one-wave kernels in front of the last pass: the
+// tree's record into its slot of the record ring (layout of k_pack_record) and
+// the state and work plan of the next tree's root histogram over all n rows
+// (k_init_root + k_plan for one node starting at row 0).
+// grid ceil(L / 128) + 1, 128 threads: the last block writes the plan.
+template <bool PAIR, bool F64>
+__global__ void __launch_bounds__(128)
+k_tree_end(const SplitRec *__restrict__ split, const NodeSum *__restrict__ tot, int L,
+           const int *__restrict__ shifts, GainParams gp, float eta, float *__restrict__ weights,
+           const int *__restrict__ t_fid, const int *__restrict__ t_bin, const float *__restrict__ t_gain,
+           const unsigned *__restrict__ overflow, uint32_t *__restrict__ record,
+           NodeSum *__restrict__ root_tot, unsigned *__restrict__ root_seg, unsigned n, unsigned rows_per_item,
+           WorkItem *__restrict__ work, unsigned *__restrict__ n_work, unsigned *__restrict__ node_first,
+           unsigned *__restrict__ node_items, unsigned long long *__restrict__ rows_scanned) {
+  const int internal = 2 * L - 1, leaves = 2 * L;
+  const int node_blocks = (int)gridDim.x - 1;
+  if ((int)blockIdx.x == node_blocks) {
+    const unsigned items = (n + rows_per_item - 1) / rows_per_item;
+    for (unsigned w = threadIdx.x; w < items; w += blockDim.x) {
+      WorkItem it;
+      it.node = 0;
+      it.begin = w * rows_per_item;
+      it.end = min(n, it.begin + rows_per_item);
+      it.first = 0;
+      work[w] = it;
+    }
+    if (threadIdx.x == 0) {
+      node_first[0] = 0;
+      node_items[0] = items;
+      *n_work = items;
+      *rows_scanned += n;
+      record[3 * internal + leaves] = *overflow;
+    }
+    return;
+  }
+  const int nd = blockIdx.x * blockDim.x + threadIdx.x;
+  for (int i = nd; i < internal; i += node_blocks * (int)blockDim.x) {
+    record[i] = (uint32_t)t_fid[i];
+    record[internal + i] = (uint32_t)t_bin[i];
+    record[2 * internal + i] = __float_as_uint(t_gain[i]);
+  }
+  if (nd >= L) return;
+  const int sg = shifts[0], sh = shifts[1];
+  const SplitRec s = split[nd];
+  const NodeSum t = tot[nd];
+  const double GL = FromFixed<F64>(s.left.g, sg), HL = PAIR ? FromFixed<F64>(s.left.h, sh) : 0.0;
+  const double GP = FromFixed<F64>(t.g, sg), HP = PAIR ? FromFixed<F64>(t.h, sh) : 0.0;
+  double GR, HR;
+  if (F64) {
+    GR = GP - GL;
+    HR = HP - HL;
+  } else {
+    GR = (double)((float)GP - (float)GL);
+    HR = (double)((float)HP - (float)HL);
+  }
+  if (nd == 0) {
+    // root_tot may be the array `tot` of this level: entry 0 has been read above, by this thread
+    root_tot[0].g = 0;
+    root_tot[0].h = 0;
+    root_tot[0].c = n;
+    root_seg[0] = 0;
+  }
+  const float wl = LeafWeight<PAIR, F64>(GL, HL, (unsigned)s.left.c, gp) * eta;
+  const float wr = LeafWeight<PAIR, F64>(GR, HR, (unsigned)(t.c - s.left.c), gp) * eta;
+  weights[2 * nd] = wl;
+  weights[2 * nd + 1] = wr;
+  record[3 * internal + 2 * nd] = __float_as_uint(wl);
+  record[3 * internal + 2 * nd + 1] = __float_as_uint(wr);
+}
+
 // End of a tree, rows in original order: walk the tree on the row's bins
 // (bin >= q+1 goes right, builder.h:107-123), record the leaf, add its weight
 // to y_hat (update_by_last_tree, garden.cu:45-76) and, when NEXT_GRAD is not
