@@ -851,7 +851,10 @@ class HipTreeBuilder : public TreeBuilder {
         if (!root_hist_ready_) HistOfNodes(orig, state, 1, false, n_, true);
         root_hist_ready_ = false;
         Reduce(1, hb, false, state, false);
-        hipLaunchKernelGGL(k_root_from_hist, dim3(1), dim3(64), 0, stream_, d_hg_[hb], d_hh_[hb], d_tot_[state], slots_);
+        // (the last pass of the previous tree has also summed the root's totals)
+        if (!root_totals_ready_)
+          hipLaunchKernelGGL(k_root_from_hist, dim3(1), dim3(64), 0, stream_, d_hg_[hb], d_hh_[hb], d_tot_[state], slots_);
+        root_totals_ready_ = false;
       } else {
         // rows are in the order of level-1; the parents' state is state ^ 1
         const int ps = state ^ 1, PL = L >> 1;
@@ -932,6 +935,7 @@ class HipTreeBuilder : public TreeBuilder {
         record_written = true;
         LaunchFinalHist(grid, label, final_lds);
         root_hist_ready_ = true;
+        root_totals_ready_ = true;
         leaf_valid_ = false;  // not recorded by this pass; GetLeaves walks the tree when asked
       } else {
         LaunchFinal(dm_->bins, stride_, 0, n_, label, next_grad);
@@ -1096,7 +1100,7 @@ class HipTreeBuilder : public TreeBuilder {
     }                                                                                                            \
     hipLaunchKernelGGL((k_final_hist<N>), dim3(grid), dim3(kHistThreads), lds, stream_, dm_->bins, stride_, F_, \
                        d_tfid_, d_tbin_, D_, d_weights_, yh, d_y_, (unsigned *)nullptr, d_g_, d_h_, d_shifts_,   \
-                       d_hwork_, d_nwork_, d_slab_, slab_entries_);                                              \
+                       d_hwork_, d_nwork_, d_slab_, slab_entries_, d_tot_[0]);                                   \
   } break;
     switch (Q_) {
       ARB_CASE(1) ARB_CASE(2) ARB_CASE(3) ARB_CASE(4) ARB_CASE(5) ARB_CASE(6) ARB_CASE(7) ARB_CASE(8)
@@ -1262,6 +1266,7 @@ class HipTreeBuilder : public TreeBuilder {
   // streamed matrices: two block buffers filled by the copy stream, a staging
   // buffer with the rows of the built nodes, a resident node id per row
   bool streamed_ = false;
+  bool root_totals_ready_ = false;  // d_tot_[0][0] holds the gradient totals of the tree grown next
   bool leaf_valid_ = true;  // d_leaf_ holds the leaves of the last tree
   bool pack_ = false;  // logistic gradients packed into one float per row, no h arrays
   hipStream_t copy_stream_ = nullptr;

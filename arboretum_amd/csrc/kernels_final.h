@@ -182,7 +182,8 @@ k_final(const uint32_t *__restrict__ bins, size_t stride, const int *__restrict_
 // gradients are bound by HBM, the histogram by LDS atomics, and they overlap.
 // One workgroup per root work item; LDS: histogram, then the node arrays.
 // leaf_of may be null: the leaf ids are then not recorded (k_leaf_ids
-// computes them on demand).
+// computes them on demand).  root_tot (may be null): the gradient totals of
+// the next root are added to root_tot[0].g / .h, which the caller has zeroed.
 template <int NQ>
 __global__ void __launch_bounds__(kHistThreads)
 k_final_hist(const uint32_t *__restrict__ bins, size_t stride, int F, const int *__restrict__ t_fid,
@@ -190,7 +191,7 @@ k_final_hist(const uint32_t *__restrict__ bins, size_t stride, int F, const int 
              float *__restrict__ yhat, const float *__restrict__ y, unsigned *__restrict__ leaf_of,
              float *__restrict__ g, float *__restrict__ h, const int *__restrict__ shifts,
              const WorkItem *__restrict__ work, const unsigned *__restrict__ n_work,
-             unsigned long long *__restrict__ slab, int slab_entries) {
+             unsigned long long *__restrict__ slab, int slab_entries, NodeSum *__restrict__ root_tot) {
   extern __shared__ unsigned long long lds[];
   const unsigned w = blockIdx.x;
   if (w >= *n_work) return;
@@ -249,6 +250,24 @@ k_final_hist(const uint32_t *__restrict__ bins, size_t stride, int F, const int 
     if (v1) row(b1, p1, y1, r1);
   }
   FlushSlab<true, NQ>(lds, slab, w, slab_entries, 0);
+  // Totals of the next root (garden.cu:432-435 reduces the gradient array):
+  // every row sits in exactly one slot of feature 0, so this item's share is
+  // the sum of that feature's slots; integers, so the order of the adds over
+  // the work items does not matter.  root_tot starts at zero.
+  if (root_tot != nullptr && threadIdx.x < 64) {
+    long long a = 0, b = 0;
+    for (int bin = threadIdx.x; bin < kSlots; bin += 64) {
+      const unsigned long long w0 = lds[bin * kBlockFeatures];
+      a += ((long long)(w0 << (64 - kCountShift))) >> (64 - kCountShift);
+      b += (long long)lds[HistLds<NQ>::word1 + bin * kBlockFeatures];
+    }
+    a = WaveSumLL(a);
+    b = WaveSumLL(b);
+    if (threadIdx.x == 0) {
+      atomicAdd(reinterpret_cast<unsigned long long *>(&root_tot[0].g), (unsigned long long)a);
+      atomicAdd(reinterpret_cast<unsigned long long *>(&root_tot[0].h), (unsigned long long)b);
+    }
+  }
 }
 
 // Leaf of every row under the tree in t_fid / t_bin (heap order), for a
