@@ -118,9 +118,10 @@ struct DevBuf {
     HIP_OK(hipMalloc((void **)&p, want * sizeof(T)));
     n = want;
   }
-  void Upload(const std::vector<T> &v, hipStream_t s) {
+  // blocking: the vector may be gone when the call returns
+  void Upload(const std::vector<T> &v) {
     Reserve(std::max<size_t>(v.size(), 1));
-    if (!v.empty()) HIP_OK(hipMemcpyAsync(p, v.data(), v.size() * sizeof(T), hipMemcpyHostToDevice, s));
+    if (!v.empty()) HIP_OK(hipMemcpy(p, v.data(), v.size() * sizeof(T), hipMemcpyHostToDevice));
   }
 };
 
@@ -206,10 +207,10 @@ struct DevicePredictor {
         h_chunks.push_back(c);
       }
     }
-    nodes.Upload(h_nodes, stream);
-    leaves.Upload(h_leaves, stream);
-    refs.Upload(h_refs, stream);
-    chunks.Upload(h_chunks, stream);
+    nodes.Upload(h_nodes);
+    leaves.Upload(h_leaves);
+    refs.Upload(h_refs);
+    chunks.Upload(h_chunks);
     // ---- row blocks: [F][block_rows] floats, about kStageBytes each
     size_t block_rows = std::max<size_t>(kStageBytes / (F * sizeof(float)) / kPredictThreads, 1) * kPredictThreads;
     block_rows = std::min(block_rows, (n + 63) / 64 * 64);
