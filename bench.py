@@ -147,7 +147,7 @@ def main():
     ap.add_argument("--max-depth", type=int, default=8)
     ap.add_argument("--hist-size", type=int, default=256)
     ap.add_argument("--cpu-rows", type=int, default=10_500_000)
-    ap.add_argument("--cpu-trees", type=int, default=8)
+    ap.add_argument("--cpu-trees", type=int, default=16)
     ap.add_argument("--no-cpu", action="store_true")
     ap.add_argument("--nan-frac", type=float, default=0.0,
                     help="stress variant: this fraction of the feature values is replaced by NaN (all land in "
