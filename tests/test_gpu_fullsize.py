@@ -54,7 +54,7 @@ def _grow(arb, workload, cfg, inspect_first=False):
 
 @pytest.fixture(scope="module")
 def fused(arb, workload):
-    # sibling subtraction on: fused partition + histogram passes; round 0 with inspection
+    # sibling subtraction on: fused partition + histogram passes; the first boosting round with inspection
     return _grow(arb, workload, _config(), inspect_first=True)
 
 
