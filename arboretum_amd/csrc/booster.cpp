@@ -1,6 +1,7 @@
 #include "booster.h"
 
 #include <algorithm>
+#include <atomic>
 #include <cmath>
 #include <cstring>
 #include <limits>
@@ -26,8 +27,12 @@ void ParallelFor(size_t n, const std::function<void(size_t, size_t)> &fn) {
   for (auto &t : th) t.join();
 }
 
+namespace {
+std::atomic<uint64_t> g_next_matrix_uid{1};
+}
+
 DataMatrix::DataMatrix(size_t rows, size_t columns, size_t columns_category)
-    : rows(rows), columns_dense(columns), columns_category(columns_category) {}
+    : rows(rows), columns_dense(columns), columns_category(columns_category), uid(g_next_matrix_uid++) {}
 
 DataMatrix::~DataMatrix() {
   if (device) FreeDeviceMatrix(device);
@@ -106,24 +111,30 @@ float Garden::IntoInternal(float v) const {
 
 void Garden::FromInternal(const std::vector<float> &in, std::vector<float> *out) const {
   out->resize(in.size());
+  FromInternal(in.data(), in.size(), out->data());
+}
+
+void Garden::FromInternal(const float *in, size_t count, float *out) const {
   if (cfg.objective == kLinearRegression) {
-    *out = in;
+    ParallelFor(count, [&](size_t b, size_t e) { std::memcpy(out + b, in + b, (e - b) * sizeof(float)); });
   } else if (cfg.objective == kLogisticRegression) {  // objective.h:58-69
-    ParallelFor(in.size(), [&](size_t b, size_t e) {
-      for (size_t i = b; i < e; ++i) (*out)[i] = (float)(1.0 / (1.0 + (double)std::exp(-in[i])));
+    ParallelFor(count, [&](size_t b, size_t e) {
+      for (size_t i = b; i < e; ++i) out[i] = (float)(1.0 / (1.0 + (double)std::exp(-in[i])));
     });
   } else {  // objective.h:80-113: class-major in, row-major out
     const size_t K = cfg.tree.labels_count;
-    const size_t n = in.size() / K;
-    std::vector<double> v(K);
-    for (size_t i = 0; i < n; ++i) {
-      double sum = 0.0;
-      for (size_t k = 0; k < K; ++k) {
-        v[k] = std::exp((double)in[i + n * k]);
-        sum += v[k];
+    const size_t n = count / K;
+    ParallelFor(n, [&](size_t b, size_t e) {
+      std::vector<double> v(K);
+      for (size_t i = b; i < e; ++i) {
+        double sum = 0.0;
+        for (size_t k = 0; k < K; ++k) {
+          v[k] = std::exp((double)in[i + n * k]);
+          sum += v[k];
+        }
+        for (size_t k = 0; k < K; ++k) out[i * K + k] = (float)(v[k] / sum);
       }
-      for (size_t k = 0; k < K; ++k) (*out)[i * K + k] = (float)(v[k] / sum);
-    }
+    });
   }
 }
 
@@ -157,17 +168,18 @@ void Garden::GrowTree(DataMatrix *data, const float *grad) {
   builder_->GrowRound(&trees_);
 }
 
-void Garden::Predict(const DataMatrix *data, std::vector<float> *out, int n_rounds) const {
+void Garden::Predict(const DataMatrix *data, float *out, int n_rounds) const {
   const size_t K = cfg.tree.labels_count;
   SyncTrees();
-  std::vector<float> tmp(data->rows * K, IntoInternal(cfg.tree.initial_y));
   const long long use = std::min<long long>(n_rounds, (long long)trees_.size());
+  const float init = IntoInternal(cfg.tree.initial_y);
   if (predict_on_device_ && use > 0 && !data->is_prebinned && data->rows > 0 && DeviceCount() > 0) {
     if (!predictor_) predictor_.reset(CreateDevicePredictor());
-    PredictOnDevice(predictor_.get(), *data, trees_, (size_t)use, K, IntoInternal(cfg.tree.initial_y), tmp.data());
-    FromInternal(tmp, out);
+    const float *sums = PredictOnDevice(predictor_.get(), *data, trees_, (size_t)use, K, init);
+    FromInternal(sums, data->rows * K, out);
     return;
   }
+  std::vector<float> tmp(data->rows * K, init);
   // Every tree over one block of rows before the next block: the block's
   // feature values (column-major, 4096 rows of every column) stay in cache, so
   // the matrix is read once, not once per tree.  Sums per row are added in tree
@@ -179,7 +191,7 @@ void Garden::Predict(const DataMatrix *data, std::vector<float> *out, int n_roun
       for (long long t = 0; t < use; ++t) trees_[t].PredictRows(*data, r0, r1, tmp.data());
     }
   });
-  FromInternal(tmp, out);
+  FromInternal(tmp.data(), tmp.size(), out);
 }
 
 void Garden::UpdateByLastTree(DataMatrix *data) {

@@ -28,6 +28,9 @@ class DataMatrix {
   const size_t rows;
   const size_t columns_dense;
   const size_t columns_category;
+  // Distinguishes this matrix from any other, also from one created later at
+  // the same address (device-side caches are keyed by it).
+  const uint64_t uid;
 
   // Column-major host store, one contiguous vector per feature (io.h:22).
   std::vector<std::vector<float>> data;
@@ -137,14 +140,15 @@ TreeBuilder *CreateTreeBuilder(const Configuration &cfg, DataMatrix *data);
 int DeviceCount();
 void CopyProbe(size_t bytes);
 
-// predictor.hip: tree walks of a float matrix on the GPU.  out: [labels][rows]
+// predictor.hip: tree walks of a float matrix on the GPU.  Returns [labels][rows]
 // sums of leaf weights of trees[0, use) on top of `init`, bit-identical to the
-// host walk (RegTree::Predict in tree order).
+// host walk (RegTree::Predict in tree order), in pinned host memory that the
+// predictor owns and overwrites on its next call.
 struct DevicePredictor;
 DevicePredictor *CreateDevicePredictor();
 void FreeDevicePredictor(DevicePredictor *p);
-void PredictOnDevice(DevicePredictor *p, const DataMatrix &data, const std::vector<RegTree> &trees, size_t use,
-                     size_t labels, float init, float *out);
+const float *PredictOnDevice(DevicePredictor *p, const DataMatrix &data, const std::vector<RegTree> &trees,
+                             size_t use, size_t labels, float init);
 
 class Garden {
  public:
@@ -153,7 +157,8 @@ class Garden {
   const Configuration cfg;
 
   void GrowTree(DataMatrix *data, const float *grad);        // garden.cu:585-625
-  void Predict(const DataMatrix *data, std::vector<float> *out, int n_rounds) const;  // :643-657
+  // out: rows * labels_count floats
+  void Predict(const DataMatrix *data, float *out, int n_rounds) const;  // :643-657
   void UpdateByLastTree(DataMatrix *data);                   // :627-635
   void GetY(const DataMatrix *data, std::vector<float> *out) const;  // :637-641
   const char *GetModel();                                    // :659-665
@@ -161,6 +166,7 @@ class Garden {
 
   float IntoInternal(float v) const;                         // objective.h:20,55-57
   void FromInternal(const std::vector<float> &in, std::vector<float> *out) const;
+  void FromInternal(const float *in, size_t count, float *out) const;  // count = rows * labels_count
 
   // Inspection / timing switches; they also apply to a builder created later.
   void SetInspect(bool on) { inspect_ = on; if (builder_) builder_->SetInspect(on); }

@@ -29,6 +29,7 @@ namespace {
 constexpr int kPredictThreads = 1024;          // rows per workgroup, one row per thread
 constexpr size_t kTreeLdsBytes = 64 * 1024;    // trees staged in LDS at a time: two workgroups per CU
 constexpr size_t kStageBytes = 32u << 20;      // one pinned staging buffer
+constexpr size_t kCacheBytes = (size_t)8 << 30;  // largest float matrix kept on the device between calls
 
 struct TreeRef {
   unsigned node_off;  // first internal node in the flattened node array
@@ -127,13 +128,20 @@ struct DevBuf {
 
 }  // namespace
 
-// Buffers kept between calls: staging and device blocks are sized once.
+// Buffers kept between calls: staging and device blocks are sized once, and
+// the columns of the last matrix (up to kCacheBytes) stay on the device, so
+// that predicting on it again (an evaluation set, once per boosting round)
+// copies nothing.
 struct DevicePredictor {
   hipStream_t stream = nullptr;
   hipEvent_t copied[2] = {nullptr, nullptr};
   float *stage[2] = {nullptr, nullptr};
   size_t stage_floats = 0;
-  DevBuf<float> block, out, leaves;
+  DevBuf<float> block, out, leaves, cache;
+  float *result = nullptr;  // pinned; the sums of the last call
+  size_t result_floats = 0;
+  uint64_t cached_uid = 0;  // matrix whose columns `cache` holds as [F][cache_ld]
+  size_t cache_ld = 0;
   DevBuf<uint2> nodes;
   DevBuf<TreeRef> refs;
   DevBuf<Chunk> chunks;
@@ -143,11 +151,11 @@ struct DevicePredictor {
       if (stage[k]) (void)hipHostFree(stage[k]);
       if (copied[k]) (void)hipEventDestroy(copied[k]);
     }
+    if (result) (void)hipHostFree(result);
     if (stream) (void)hipStreamDestroy(stream);
   }
 
-  void Run(const DataMatrix &data, const std::vector<RegTree> &trees, size_t use, size_t labels, float init,
-           float *result) {
+  const float *Run(const DataMatrix &data, const std::vector<RegTree> &trees, size_t use, size_t labels, float init) {
     const size_t n = data.rows, F = data.columns_dense;
     if (data.is_prebinned) throw std::runtime_error("device prediction needs a float matrix");
     if (n == 0 || F == 0) throw std::runtime_error("empty data matrix");
@@ -211,53 +219,78 @@ struct DevicePredictor {
     leaves.Upload(h_leaves);
     refs.Upload(h_refs);
     chunks.Upload(h_chunks);
-    // ---- row blocks: [F][block_rows] floats, about kStageBytes each
-    size_t block_rows = std::max<size_t>(kStageBytes / (F * sizeof(float)) / kPredictThreads, 1) * kPredictThreads;
-    block_rows = std::min(block_rows, (n + 63) / 64 * 64);
-    const size_t floats = F * block_rows;
-    if (floats > stage_floats) {
-      for (int k = 0; k < 2; ++k) {
-        if (stage[k]) HIP_OK(hipHostFree(stage[k]));
-        stage[k] = nullptr;
-      }
-      stage_floats = 0;
-      for (int k = 0; k < 2; ++k) HIP_OK(hipHostMalloc((void **)&stage[k], floats * sizeof(float), hipHostMallocDefault));
-      stage_floats = floats;
-    }
-    block.Reserve(floats);
     out.Reserve(labels * n);
     hipLaunchKernelGGL(k_predict_fill, dim3((unsigned)((labels * n + 255) / 256)), dim3(256), 0, stream, out.p,
                        labels * n, init);
     HIP_OK(hipGetLastError());
-    const size_t nblocks = (n + block_rows - 1) / block_rows;
-    for (size_t b = 0; b < nblocks; ++b) {
-      const int buf = (int)(b & 1);
-      const size_t r0 = b * block_rows, rows = std::min(block_rows, n - r0);
-      if (b >= 2) HIP_OK(hipEventSynchronize(copied[buf]));  // the copy out of this staging buffer is done
-      float *dst = stage[buf];
-      ParallelFor(rows, [&](size_t lo, size_t hi) {
-        for (size_t f = 0; f < F; ++f)
-          std::memcpy(dst + f * block_rows + lo, data.data[f].data() + r0 + lo, (hi - lo) * sizeof(float));
-      });
-      HIP_OK(hipMemcpyAsync(block.p, dst, floats * sizeof(float), hipMemcpyHostToDevice, stream));
-      HIP_OK(hipEventRecord(copied[buf], stream));
-      if (use > 0) {
-        hipLaunchKernelGGL(k_predict, dim3((unsigned)((rows + kPredictThreads - 1) / kPredictThreads)),
-                           dim3(kPredictThreads), kTreeLdsBytes, stream, block.p, block_rows, (unsigned)rows,
-                           nodes.p, leaves.p, refs.p, chunks.p, (int)h_chunks.size(), out.p + r0, n);
-        HIP_OK(hipGetLastError());
+    auto walk = [&](const float *cols, size_t ld, size_t r0, size_t rows) {
+      if (use == 0) return;
+      hipLaunchKernelGGL(k_predict, dim3((unsigned)((rows + kPredictThreads - 1) / kPredictThreads)),
+                         dim3(kPredictThreads), kTreeLdsBytes, stream, cols, ld, (unsigned)rows, nodes.p, leaves.p,
+                         refs.p, chunks.p, (int)h_chunks.size(), out.p + r0, n);
+      HIP_OK(hipGetLastError());
+    };
+    const size_t ld_all = (n + 63) / 64 * 64;
+    const bool cacheable = F * ld_all * sizeof(float) <= kCacheBytes;
+    if (cacheable && cached_uid == data.uid && cache_ld == ld_all) {
+      walk(cache.p, cache_ld, 0, n);  // the columns are on the device already
+    } else {
+      // ---- row blocks: [F][block_rows] floats, about kStageBytes each
+      size_t block_rows = std::max<size_t>(kStageBytes / (F * sizeof(float)) / kPredictThreads, 1) * kPredictThreads;
+      block_rows = std::min(block_rows, ld_all);
+      const size_t floats = F * block_rows;
+      if (floats > stage_floats) {
+        for (int k = 0; k < 2; ++k) {
+          if (stage[k]) HIP_OK(hipHostFree(stage[k]));
+          stage[k] = nullptr;
+        }
+        stage_floats = 0;
+        for (int k = 0; k < 2; ++k) HIP_OK(hipHostMalloc((void **)&stage[k], floats * sizeof(float), hipHostMallocDefault));
+        stage_floats = floats;
       }
+      block.Reserve(floats);
+      cached_uid = 0;
+      if (cacheable) cache.Reserve(F * ld_all);
+      const size_t nblocks = (n + block_rows - 1) / block_rows;
+      for (size_t b = 0; b < nblocks; ++b) {
+        const int buf = (int)(b & 1);
+        const size_t r0 = b * block_rows, rows = std::min(block_rows, n - r0);
+        if (b >= 2) HIP_OK(hipEventSynchronize(copied[buf]));  // the copy out of this staging buffer is done
+        float *dst = stage[buf];
+        ParallelFor(rows, [&](size_t lo, size_t hi) {
+          for (size_t f = 0; f < F; ++f)
+            std::memcpy(dst + f * block_rows + lo, data.data[f].data() + r0 + lo, (hi - lo) * sizeof(float));
+        });
+        HIP_OK(hipMemcpyAsync(block.p, dst, floats * sizeof(float), hipMemcpyHostToDevice, stream));
+        HIP_OK(hipEventRecord(copied[buf], stream));
+        walk(block.p, block_rows, r0, rows);
+        if (cacheable)  // rows [r0, r0 + rows) of every column into their place in the whole matrix
+          HIP_OK(hipMemcpy2DAsync(cache.p + r0, ld_all * sizeof(float), block.p, block_rows * sizeof(float),
+                                  rows * sizeof(float), F, hipMemcpyDeviceToDevice, stream));
+      }
+      if (cacheable) {
+        cached_uid = data.uid;
+        cache_ld = ld_all;
+      }
+    }
+    if (labels * n > result_floats) {
+      if (result) HIP_OK(hipHostFree(result));
+      result = nullptr;
+      result_floats = 0;
+      HIP_OK(hipHostMalloc((void **)&result, labels * n * sizeof(float), hipHostMallocDefault));
+      result_floats = labels * n;
     }
     HIP_OK(hipMemcpyAsync(result, out.p, labels * n * sizeof(float), hipMemcpyDeviceToHost, stream));
     HIP_OK(hipStreamSynchronize(stream));
+    return result;
   }
 };
 
 DevicePredictor *CreateDevicePredictor() { return new DevicePredictor(); }
 void FreeDevicePredictor(DevicePredictor *p) { delete p; }
-void PredictOnDevice(DevicePredictor *p, const DataMatrix &data, const std::vector<RegTree> &trees, size_t use,
-                     size_t labels, float init, float *out) {
-  p->Run(data, trees, use, labels, init, out);
+const float *PredictOnDevice(DevicePredictor *p, const DataMatrix &data, const std::vector<RegTree> &trees,
+                             size_t use, size_t labels, float init) {
+  return p->Run(data, trees, use, labels, init);
 }
 
 }  // namespace arb

@@ -143,14 +143,22 @@ const char *AGrowTree(VoidPointer garden, VoidPointer data, const float *grad) {
 }
 
 const char *APredict(VoidPointer garden, VoidPointer data, const float **out, const int n_rounds) {
-  const char *err = nullptr;
-  std::vector<float> result;
-  err = Guard([&] {
+  float *result = nullptr;
+  const char *err = Guard([&] {
     if (!out) throw std::runtime_error("bad arguments");
-    AsGarden(garden)->garden.Predict(AsData(data), &result,
-                                     n_rounds == -1 ? std::numeric_limits<int>::max() : n_rounds);
+    Garden &g = AsGarden(garden)->garden;
+    const DataMatrix *d = AsData(data);
+    const size_t count = d->rows * g.cfg.tree.labels_count;
+    result = new (std::nothrow) float[count ? count : 1];
+    if (!result) throw std::runtime_error("unable to allocate array");
+    g.Predict(d, result, n_rounds == -1 ? std::numeric_limits<int>::max() : n_rounds);
   });
-  return err ? err : CopyOut(result, out);
+  if (err) {
+    delete[] result;
+    return err;
+  }
+  *out = result;
+  return nullptr;
 }
 
 const char *ADumpModel(const char **model, VoidPointer garden) {

@@ -86,6 +86,29 @@ def test_several_row_blocks(arb):
     assert (np.abs(p - dev) > 1e-6).mean() < 1e-4
 
 
+def test_repeated_prediction_on_the_same_matrix(arb):
+    # the columns of the last matrix stay on the device: a second call on it (with more trees, as
+    # an evaluation loop does), a call on another matrix, and the first one again
+    Xa, ya = make_data(50000, 7, 1, seed=3, nan_frac=0.05)
+    Xb, _ = make_data(1300, 7, 1, seed=4)
+    cfg = {"objective": 1, "method": 1, "internals": {"hist_size": 32, "double_precision": True},
+           "tree": {"max_depth": 4, "eta": 0.3, "lambda": 1.0}}
+    train = arb.DMatrix(Xa, y=ya)
+    a, b = arb.DMatrix(Xa), arb.DMatrix(Xb)
+    g = arb.Garden(cfg, train)
+    seen = []
+    for r in range(3):
+        g.grow_tree()
+        seen.append(both_ways(g, a))
+        if r == 1:
+            both_ways(g, b)
+    assert not np.array_equal(seen[0], seen[1]) and not np.array_equal(seen[1], seen[2])
+    both_ways(g, a, 1)
+    del a
+    c = arb.DMatrix(Xb[:700] * 2)      # possibly at the address of the matrix just freed
+    both_ways(g, c)
+
+
 def _random_model(rng, depths, F, fid_max):
     model = []
     for d in depths:           # d = internal depth: 2^(d-1) - 1 split nodes
