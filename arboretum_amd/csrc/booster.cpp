@@ -173,7 +173,7 @@ void Garden::Predict(const DataMatrix *data, float *out, int n_rounds) const {
   SyncTrees();
   const long long use = std::min<long long>(n_rounds, (long long)trees_.size());
   const float init = IntoInternal(cfg.tree.initial_y);
-  if (predict_on_device_ && use > 0 && !data->is_prebinned && data->rows > 0 && DeviceCount() > 0) {
+  if (predict_on_device_ && use > 0 && data->rows > 0 && DeviceCount() > 0) {
     if (!predictor_) predictor_.reset(CreateDevicePredictor());
     const float *sums = PredictOnDevice(predictor_.get(), *data, trees_, (size_t)use, K, init);
     FromInternal(sums, data->rows * K, out);

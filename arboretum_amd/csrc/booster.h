@@ -140,7 +140,7 @@ TreeBuilder *CreateTreeBuilder(const Configuration &cfg, DataMatrix *data);
 int DeviceCount();
 void CopyProbe(size_t bytes);
 
-// predictor.hip: tree walks of a float matrix on the GPU.  Returns [labels][rows]
+// predictor.hip: tree walks of a matrix (floats or bin ids) on the GPU.  Returns [labels][rows]
 // sums of leaf weights of trees[0, use) on top of `init`, bit-identical to the
 // host walk (RegTree::Predict in tree order), in pinned host memory that the
 // predictor owns and overwrites on its next call.
@@ -171,8 +171,8 @@ class Garden {
   // Inspection / timing switches; they also apply to a builder created later.
   void SetInspect(bool on) { inspect_ = on; if (builder_) builder_->SetInspect(on); }
   void SetTiming(int level) { timing_ = level; if (builder_) builder_->EnableTiming(level); }
-  // Predict walks the trees on the GPU when one is present and the matrix holds
-  // floats (default), or on the host as the reference does.
+  // Predict walks the trees on the GPU when one is present (default), or on
+  // the host as the reference does.
   void SetPredictOnDevice(bool on) { predict_on_device_ = on; }
 
   TreeBuilder *builder() { return builder_.get(); }

@@ -1,7 +1,8 @@
 // Batch prediction on the GPU: the tree walks of RegTree::Predict /
 // Garden::Predict (src/core/garden.h:70-90, src/core/garden.cu:643-657) for a
-// float matrix, every tree over a block of rows while the next block is
-// staged.  The arithmetic is the host walk's: `x < threshold` goes left (NaN
+// float matrix (or a pre-quantised one, whose bin ids are compared as floats
+// like the host walk does), every tree over a block of rows while the next
+// block is staged.  The arithmetic is the host walk's: `x < threshold` goes left (NaN
 // right), the leaf weights of one label are added in tree order in fp32, so
 // the sums are bit-identical to the host path.  The link function stays with
 // the caller.
@@ -44,12 +45,27 @@ struct Chunk {
   unsigned t0, t1, in_lds, n_nodes, n_leaves;
 };
 
-// Walks trees [t0, t1) for one row; x points at the row's value of feature 0,
-// features are ld floats apart.  acc holds the running sum of label *cur.
+// Where a row's feature values come from.
+enum Source {
+  kFloatCols = 0,  // float columns [F][ld]
+  kByteRows = 1,   // pre-quantised rows [rows][ld = F] of uint8 bin ids
+  kQuadCols = 2    // pre-quantised quad columns [Q][ld]: four uint8 bin ids per word
+};
+
+template <int SRC>
+__device__ __forceinline__ float Fetch(const void *__restrict__ base, size_t ld, unsigned r, unsigned f) {
+  if (SRC == kFloatCols) return static_cast<const float *>(base)[(size_t)f * ld + r];
+  if (SRC == kByteRows) return (float)static_cast<const uint8_t *>(base)[(size_t)r * ld + f];
+  return (float)((static_cast<const uint32_t *>(base)[(size_t)(f >> 2) * ld + r] >> (8u * (f & 3u))) & 255u);
+}
+
+// Walks trees [t0, t1) for row r of `base`.  acc holds the running sum of
+// label *cur.
+template <int SRC>
 __device__ __forceinline__ void WalkTrees(const uint2 *nd, const float *lf, unsigned node_base, unsigned leaf_base,
                                           const TreeRef *__restrict__ refs, unsigned t0, unsigned t1,
-                                          const float *__restrict__ x, size_t ld, float *__restrict__ out,
-                                          size_t out_ld, bool live, int *cur, float *acc) {
+                                          const void *__restrict__ base, size_t ld, unsigned r,
+                                          float *__restrict__ out, size_t out_ld, bool live, int *cur, float *acc) {
   for (unsigned t = t0; t < t1; ++t) {
     const TreeRef ref = refs[t];
     if ((int)ref.label != *cur) {
@@ -61,24 +77,24 @@ __device__ __forceinline__ void WalkTrees(const uint2 *nd, const float *lf, unsi
     unsigned id = 0;
     for (unsigned j = 1; j < ref.depth; ++j) {
       const uint2 n = tn[id];
-      const float v = x[(size_t)n.x * ld];
+      const float v = Fetch<SRC>(base, ld, r, n.x);
       id = 2 * id + 2 - (unsigned)(v < __uint_as_float(n.y));
     }
     *acc += lf[ref.leaf_off - leaf_base + (id - ((1u << (ref.depth - 1)) - 1))];
   }
 }
 
-// cols: [F][ld] floats of this block's rows; out: [labels][out_ld], already
-// offset to the block's first row.  grid ceil(rows / 1024).
+// base: this block's rows as SRC says; out: [labels][out_ld], already offset
+// to the block's first row.  grid ceil(rows / 1024).
+template <int SRC>
 __global__ void __launch_bounds__(kPredictThreads)
-k_predict(const float *__restrict__ cols, size_t ld, unsigned rows, const uint2 *__restrict__ nodes,
+k_predict(const void *__restrict__ base, size_t ld, unsigned rows, const uint2 *__restrict__ nodes,
           const float *__restrict__ leaves, const TreeRef *__restrict__ refs, const Chunk *__restrict__ chunks,
           int n_chunks, float *__restrict__ out, size_t out_ld) {
   extern __shared__ unsigned char smem[];
   const unsigned i = blockIdx.x * kPredictThreads + threadIdx.x;
   const bool live = i < rows;
   const unsigned r = live ? i : rows - 1;
-  const float *x = cols + r;
   float *o = out + r;
   int cur = -1;
   float acc = 0.0f;
@@ -92,10 +108,10 @@ k_predict(const float *__restrict__ cols, size_t ld, unsigned rows, const uint2 
       for (unsigned k = threadIdx.x; k < ch.n_nodes; k += kPredictThreads) s_nd[k] = nodes[node_base + k];
       for (unsigned k = threadIdx.x; k < ch.n_leaves; k += kPredictThreads) s_lf[k] = leaves[leaf_base + k];
       __syncthreads();
-      WalkTrees(s_nd, s_lf, node_base, leaf_base, refs, ch.t0, ch.t1, x, ld, o, out_ld, live, &cur, &acc);
+      WalkTrees<SRC>(s_nd, s_lf, node_base, leaf_base, refs, ch.t0, ch.t1, base, ld, r, o, out_ld, live, &cur, &acc);
     } else {
-      WalkTrees(nodes + node_base, leaves + leaf_base, node_base, leaf_base, refs, ch.t0, ch.t1, x, ld, o, out_ld,
-                live, &cur, &acc);
+      WalkTrees<SRC>(nodes + node_base, leaves + leaf_base, node_base, leaf_base, refs, ch.t0, ch.t1, base, ld, r, o,
+                     out_ld, live, &cur, &acc);
     }
   }
   if (cur >= 0 && live) o[(size_t)cur * out_ld] = acc;
@@ -157,7 +173,6 @@ struct DevicePredictor {
 
   const float *Run(const DataMatrix &data, const std::vector<RegTree> &trees, size_t use, size_t labels, float init) {
     const size_t n = data.rows, F = data.columns_dense;
-    if (data.is_prebinned) throw std::runtime_error("device prediction needs a float matrix");
     if (n == 0 || F == 0) throw std::runtime_error("empty data matrix");
     if (n >= (1ull << 31)) throw std::runtime_error("too many rows");
     if (!stream) {
@@ -223,54 +238,99 @@ struct DevicePredictor {
     hipLaunchKernelGGL(k_predict_fill, dim3((unsigned)((labels * n + 255) / 256)), dim3(256), 0, stream, out.p,
                        labels * n, init);
     HIP_OK(hipGetLastError());
-    auto walk = [&](const float *cols, size_t ld, size_t r0, size_t rows) {
+    auto walk = [&](int src, const void *base, size_t ld, size_t r0, size_t rows) {
       if (use == 0) return;
-      hipLaunchKernelGGL(k_predict, dim3((unsigned)((rows + kPredictThreads - 1) / kPredictThreads)),
-                         dim3(kPredictThreads), kTreeLdsBytes, stream, cols, ld, (unsigned)rows, nodes.p, leaves.p,
-                         refs.p, chunks.p, (int)h_chunks.size(), out.p + r0, n);
+      const dim3 grid((unsigned)((rows + kPredictThreads - 1) / kPredictThreads)), block_dim(kPredictThreads);
+#define ARB_WALK(S)                                                                                         \
+  hipLaunchKernelGGL((k_predict<S>), grid, block_dim, kTreeLdsBytes, stream, base, ld, (unsigned)rows, nodes.p, \
+                     leaves.p, refs.p, chunks.p, (int)h_chunks.size(), out.p + r0, n)
+      if (src == kFloatCols) ARB_WALK(kFloatCols);
+      else if (src == kByteRows) ARB_WALK(kByteRows);
+      else ARB_WALK(kQuadCols);
+#undef ARB_WALK
       HIP_OK(hipGetLastError());
     };
-    const size_t ld_all = (n + 63) / 64 * 64;
-    const bool cacheable = F * ld_all * sizeof(float) <= kCacheBytes;
-    if (cacheable && cached_uid == data.uid && cache_ld == ld_all) {
-      walk(cache.p, cache_ld, 0, n);  // the columns are on the device already
-    } else {
-      // ---- row blocks: [F][block_rows] floats, about kStageBytes each
-      size_t block_rows = std::max<size_t>(kStageBytes / (F * sizeof(float)) / kPredictThreads, 1) * kPredictThreads;
-      block_rows = std::min(block_rows, ld_all);
-      const size_t floats = F * block_rows;
-      if (floats > stage_floats) {
-        for (int k = 0; k < 2; ++k) {
-          if (stage[k]) HIP_OK(hipHostFree(stage[k]));
-          stage[k] = nullptr;
-        }
-        stage_floats = 0;
-        for (int k = 0; k < 2; ++k) HIP_OK(hipHostMalloc((void **)&stage[k], floats * sizeof(float), hipHostMallocDefault));
-        stage_floats = floats;
+    auto reserve_stage = [&](size_t floats) {
+      if (floats <= stage_floats) return;
+      for (int k = 0; k < 2; ++k) {
+        if (stage[k]) HIP_OK(hipHostFree(stage[k]));
+        stage[k] = nullptr;
       }
-      block.Reserve(floats);
+      stage_floats = 0;
+      for (int k = 0; k < 2; ++k) HIP_OK(hipHostMalloc((void **)&stage[k], floats * sizeof(float), hipHostMallocDefault));
+      stage_floats = floats;
+    };
+    if (data.is_prebinned) {
       cached_uid = 0;
-      if (cacheable) cache.Reserve(F * ld_all);
-      const size_t nblocks = (n + block_rows - 1) / block_rows;
-      for (size_t b = 0; b < nblocks; ++b) {
-        const int buf = (int)(b & 1);
-        const size_t r0 = b * block_rows, rows = std::min(block_rows, n - r0);
-        if (b >= 2) HIP_OK(hipEventSynchronize(copied[buf]));  // the copy out of this staging buffer is done
-        float *dst = stage[buf];
-        ParallelFor(rows, [&](size_t lo, size_t hi) {
-          for (size_t f = 0; f < F; ++f)
-            std::memcpy(dst + f * block_rows + lo, data.data[f].data() + r0 + lo, (hi - lo) * sizeof(float));
-        });
-        HIP_OK(hipMemcpyAsync(block.p, dst, floats * sizeof(float), hipMemcpyHostToDevice, stream));
-        HIP_OK(hipEventRecord(copied[buf], stream));
-        walk(block.p, block_rows, r0, rows);
-        if (cacheable)  // rows [r0, r0 + rows) of every column into their place in the whole matrix
-          HIP_OK(hipMemcpy2DAsync(cache.p + r0, ld_all * sizeof(float), block.p, block_rows * sizeof(float),
-                                  rows * sizeof(float), F, hipMemcpyDeviceToDevice, stream));
+      if (!data.prebinned.empty()) {
+        // row-major bytes on the host: blocks of whole rows through the staging buffers
+        const size_t block_rows =
+            std::min(std::max<size_t>(kStageBytes / F / kPredictThreads, 1) * kPredictThreads, (n + 63) / 64 * 64);
+        const size_t floats = (block_rows * F + 3) / 4;
+        reserve_stage(floats);
+        block.Reserve(floats);
+        const size_t nblocks = (n + block_rows - 1) / block_rows;
+        for (size_t b = 0; b < nblocks; ++b) {
+          const int buf = (int)(b & 1);
+          const size_t r0 = b * block_rows, rows = std::min(block_rows, n - r0);
+          if (b >= 2) HIP_OK(hipEventSynchronize(copied[buf]));
+          uint8_t *dst = reinterpret_cast<uint8_t *>(stage[buf]);
+          const uint8_t *src = data.prebinned.data() + r0 * F;
+          ParallelFor(rows * F, [&](size_t lo, size_t hi) { std::memcpy(dst + lo, src + lo, hi - lo); });
+          HIP_OK(hipMemcpyAsync(block.p, dst, rows * F, hipMemcpyHostToDevice, stream));
+          HIP_OK(hipEventRecord(copied[buf], stream));
+          walk(kByteRows, block.p, F, r0, rows);
+        }
+      } else if (!data.stream_blocks.empty()) {
+        // streamed matrix: its pinned blocks of quad columns go up as they are
+        const size_t br = data.stream_block_rows, Q = (F + 3) / 4;
+        block.Reserve(Q * br);
+        for (size_t b = 0; b < data.stream_blocks.size(); ++b) {
+          const size_t r0 = b * br;
+          if (r0 >= n) break;
+          const size_t rows = std::min(br, n - r0);
+          HIP_OK(hipMemcpyAsync(block.p, data.stream_blocks[b], Q * br * sizeof(uint32_t), hipMemcpyHostToDevice,
+                                stream));
+          walk(kQuadCols, block.p, br, r0, rows);
+        }
+      } else {
+        throw std::runtime_error("pre-quantised matrix without bins");
       }
-      if (cacheable) {
-        cached_uid = data.uid;
-        cache_ld = ld_all;
+    } else {
+      const size_t ld_all = (n + 63) / 64 * 64;
+      const bool cacheable = F * ld_all * sizeof(float) <= kCacheBytes;
+      if (cacheable && cached_uid == data.uid && cache_ld == ld_all) {
+        walk(kFloatCols, cache.p, cache_ld, 0, n);  // the columns are on the device already
+      } else {
+        // ---- row blocks: [F][block_rows] floats, about kStageBytes each
+        size_t block_rows = std::max<size_t>(kStageBytes / (F * sizeof(float)) / kPredictThreads, 1) * kPredictThreads;
+        block_rows = std::min(block_rows, ld_all);
+        const size_t floats = F * block_rows;
+        reserve_stage(floats);
+        block.Reserve(floats);
+        cached_uid = 0;
+        if (cacheable) cache.Reserve(F * ld_all);
+        const size_t nblocks = (n + block_rows - 1) / block_rows;
+        for (size_t b = 0; b < nblocks; ++b) {
+          const int buf = (int)(b & 1);
+          const size_t r0 = b * block_rows, rows = std::min(block_rows, n - r0);
+          if (b >= 2) HIP_OK(hipEventSynchronize(copied[buf]));  // the copy out of this staging buffer is done
+          float *dst = stage[buf];
+          ParallelFor(rows, [&](size_t lo, size_t hi) {
+            for (size_t f = 0; f < F; ++f)
+              std::memcpy(dst + f * block_rows + lo, data.data[f].data() + r0 + lo, (hi - lo) * sizeof(float));
+          });
+          HIP_OK(hipMemcpyAsync(block.p, dst, floats * sizeof(float), hipMemcpyHostToDevice, stream));
+          HIP_OK(hipEventRecord(copied[buf], stream));
+          walk(kFloatCols, block.p, block_rows, r0, rows);
+          if (cacheable)  // rows [r0, r0 + rows) of every column into their place in the whole matrix
+            HIP_OK(hipMemcpy2DAsync(cache.p + r0, ld_all * sizeof(float), block.p, block_rows * sizeof(float),
+                                    rows * sizeof(float), F, hipMemcpyDeviceToDevice, stream));
+        }
+        if (cacheable) {
+          cached_uid = data.uid;
+          cache_ld = ld_all;
+        }
       }
     }
     if (labels * n > result_floats) {

@@ -48,8 +48,8 @@ const char *AGetBinLayout(VoidPointer data, int *bits, int *slots);
 const char *AGetBins16(VoidPointer data, unsigned short *out);
 
 /* Where APredict walks the trees (src/core/garden.cu:643-657 does it on the
- * host): on != 0 (default) uses the GPU for float matrices when a device is
- * present, 0 the host walk.  Both give the same bits. */
+ * host): on != 0 (default) uses the GPU when a device is present, 0 the host
+ * walk.  Both give the same bits. */
 const char *AGardenPredictOnDevice(VoidPointer garden, int on);
 
 /* Inspection of the booster; valid after AGrowTree. */

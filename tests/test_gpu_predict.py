@@ -145,15 +145,23 @@ def test_loaded_model_mixed_depths_foreign_features_and_trees_beyond_lds(arb):
     both_ways(g, data, 5)
 
 
-def test_prebinned_matrix_uses_the_host_walk(arb):
+@pytest.mark.parametrize("upload", [True, False])
+def test_prequantised_matrices(arb, upload):
+    # bin ids are compared as floats against the thresholds, as the host walk does; the rows come from
+    # the row-major bytes on the host or, once a streamed matrix has given them up, from its pinned blocks
     rng = np.random.default_rng(2)
-    bins = rng.integers(0, 256, size=(3000, 8), dtype=np.uint8)
-    y = (bins[:, 0] > 100).astype(np.float32)
-    cfg = {"objective": 1, "method": 1, "internals": {"hist_size": 256, "double_precision": True},
-           "tree": {"max_depth": 3, "eta": 0.5, "lambda": 1.0}}
+    bins = rng.integers(0, 256, size=(70001, 9), dtype=np.uint8)
+    y = ((bins[:, 0] > 100) ^ (bins[:, 5] > 30)).astype(np.float32)
+    cfg = {"objective": 1, "method": 1,
+           "internals": {"hist_size": 256, "double_precision": True, "upload_features": upload,
+                         "stream_block_rows": 16384},
+           "tree": {"max_depth": 4, "eta": 0.5, "lambda": 1.0}}
     data = arb.DMatrix(bins, y=y, quantized=True)
+    fresh = arb.DMatrix(bins[::-1].copy(), quantized=True)   # never quantised: bytes on the host
     g = arb.Garden(cfg, data)
-    for _ in range(3):
+    for _ in range(5):
         g.grow_tree()
-    p = g.predict(data)
+    p = both_ways(g, data)
     assert ((p > 0.5) == (y > 0.5)).mean() > 0.95
+    assert np.array_equal(both_ways(g, fresh), p[::-1])
+    both_ways(g, data, 2)
