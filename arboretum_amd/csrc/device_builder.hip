@@ -454,8 +454,7 @@ class HipTreeBuilder : public TreeBuilder {
     streamed_ = dm_->streamed;
     // Logistic gradients of 0/1 labels travel as one float per row (PackGrad):
     // there is no h array then, and kernels given h == nullptr unpack g.
-    pack_ = cfg.objective == kLogisticRegression && !streamed_ && !wide_ && single_group_ &&
-            data->y.size() == n_ &&
+    pack_ = cfg.objective == kLogisticRegression && !streamed_ && !wide_ && data->y.size() == n_ &&
             std::all_of(data->y.begin(), data->y.end(), [](float v) { return v == 0.0f || v == 1.0f; });
     d_g_ = DevAlloc<float>(n_ * K_);
     d_h_ = pack_ ? nullptr : DevAlloc<float>(n_ * K_);
@@ -878,7 +877,8 @@ class HipTreeBuilder : public TreeBuilder {
                         d_nwork_ + 1, d_wave_left_, d_item_left_, d_slab_, slab_entries_, src.bins, q0};
 #define ARB_FUSED(P, W)                                                       \
   do {                                                                        \
-    if (P && pack_) LaunchFused<P, W, false, P>(nq, stream_, grid, a);        \
+    if (P && pack_ && single_group_) LaunchFused<P, W, false, P>(nq, stream_, grid, a); \
+    else if (P && pack_) LaunchFused<P, W, true, P>(nq, stream_, grid, a);    \
     else if (single_group_) LaunchFused<P, W, false, false>(nq, stream_, grid, a); \
     else LaunchFused<P, W, true, false>(nq, stream_, grid, a);                \
   } while (0)
