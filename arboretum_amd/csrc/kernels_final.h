@@ -197,29 +197,38 @@ k_final_hist(const uint32_t *__restrict__ bins, size_t stride, int F, const int 
   if (w >= *n_work) return;
   const WorkItem it = work[w];
   constexpr int words = (int)(HistLdsBytes(NQ, true) / 8);
-  int *s_nodes = reinterpret_cast<int *>(lds + words);  // fid[internal], bin[internal]
+  // Node table for the walk, two words per internal node: a byte selector for
+  // v_perm_b32 that picks byte fid % 8 out of a pair of quads (the other three
+  // result bytes are zero), and the split bin in bits 0-7 with the pair fid / 8
+  // in bits 8-9.  A node that was not split compares against 255: no bin id is
+  // larger, so every row stays left.
+  uint2 *s_tree = reinterpret_cast<uint2 *>(lds + words);
   const int internal = (1 << (depth - 1)) - 1;
   for (int i = threadIdx.x; i < words; i += kHistThreads) lds[i] = 0ull;
   for (int i = threadIdx.x; i < internal; i += kHistThreads) {
-    s_nodes[i] = t_fid[i];
-    s_nodes[internal + i] = t_bin[i];
+    const int fid = t_fid[i], bin = t_bin[i];
+    uint2 nd;
+    nd.x = 0x0c0c0c00u | (unsigned)(fid & 7);
+    nd.y = (bin < 0 ? 255u : (unsigned)bin) | ((unsigned)(fid >> 3) << 8);
+    s_tree[i] = nd;
   }
   __syncthreads();
   const int sg = shifts[0], sh = shifts[1];
+  // quad q of a row, zero past the last one
+  auto quad = [](const uint32_t (&b)[NQ], int q) { return q < NQ ? b[q < NQ ? q : 0] : 0u; };
   auto row = [&](const uint32_t (&b)[NQ], float p, float yv, unsigned r) {
     unsigned node = 0;
     for (int level = 0; level + 1 < depth; ++level) {
-      const int id = (1 << level) - 1 + (int)node;
-      const int fid = s_nodes[id], bin = s_nodes[internal + id];
-      unsigned right = 0;
-      if (bin >= 0) {
-        uint32_t b4 = 0;
-        const int fq = fid >> 2;
-#pragma unroll
-        for (int q = 0; q < NQ; ++q) b4 = q == fq ? b[q] : b4;
-        right = (int)((b4 >> (8 * (fid & 3))) & 255u) > bin ? 1u : 0u;
-      }
-      node = node * 2 + right;
+      const uint2 nd = s_tree[(1 << level) - 1 + (int)node];
+      // the row's bin of the split feature: byte fid % 8 of each pair of quads, then the pair
+      const uint32_t t0 = __builtin_amdgcn_perm(quad(b, 1), quad(b, 0), nd.x);
+      const uint32_t t1 = __builtin_amdgcn_perm(quad(b, 3), quad(b, 2), nd.x);
+      const uint32_t t2 = __builtin_amdgcn_perm(quad(b, 5), quad(b, 4), nd.x);
+      const uint32_t t3 = __builtin_amdgcn_perm(quad(b, 7), quad(b, 6), nd.x);
+      const unsigned pair = nd.y >> 8;
+      const uint32_t lo = pair == 1u ? t1 : t0, hi = pair == 3u ? t3 : t2;
+      const uint32_t v = pair >= 2u ? hi : lo;
+      node = node * 2 + (v > (nd.y & 255u) ? 1u : 0u);  // bin >= q + 1 goes right (builder.h:107-123)
     }
     if (leaf_of != nullptr) __builtin_nontemporal_store(node, &leaf_of[r]);  // uniform
     const float yh = p + weights[node];
