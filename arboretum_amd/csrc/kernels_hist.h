@@ -46,7 +46,7 @@ __device__ __forceinline__ void AccumulateRow(unsigned long long *__restrict__ l
 #pragma unroll
       for (int t = 0; t < 4; ++t) {
         const unsigned bi = ((unsigned)t + i) & 3u;  // byte of the quad
-        const unsigned bin = (sel >> (8u * bi)) & 255u;
+        const unsigned bin = __builtin_amdgcn_ubfe(sel, 8u * bi, 8u);  // one v_bfe_u32
         const unsigned f16 = 4u * qi + bi;
         // Quads past NQ do not exist.  Padding features of the last quad of
         // the matrix (bin 0 in every row) are accumulated like real ones into
