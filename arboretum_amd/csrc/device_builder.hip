@@ -16,7 +16,7 @@
 //   word1 = sum of h_q
 // so one update costs two ds_add_u64 (one for the squared objective).  A range
 // holds at most 64512 rows, which keeps both fields exact.  The LDS histogram
-// is laid out in blocks of 16 features, bin-major inside a block, and every
+// is laid out bin-major, the features of a bin in blocks of 16, and every
 // lane of a wave updates a different feature of its own row at a time: the 16
 // lanes that one pass of the LDS atomic unit serves never share a bank pair or
 // an address, whatever the bins are.  Each workgroup writes its LDS histogram
@@ -805,7 +805,7 @@ class HipTreeBuilder : public TreeBuilder {
   hipLaunchKernelGGL((k_hist_reduce<P, LN>), grid, dim3(1024), 0, stream_, d_slab_, slab_entries_, nbin_total_,   \
                      d_node_first_, d_node_items_, by_parent ? 1 : 0, d_split_, d_tot_[parent_state], d_hg_[hb], \
                      d_hh_[hb], d_hc_[hb], d_hg_[hb ^ 1], d_hh_[hb ^ 1], d_hc_[hb ^ 1], trick ? 1 : 0,           \
-                     accumulate ? 1 : 0, wide_ ? 1 : 0)
+                     accumulate ? 1 : 0, wide_ ? 1 : 0, HistBlocks(quads_per_group_))
     if (pair_) {
       if (wide_blocks) ARB_REDUCE(true, 4);
       else ARB_REDUCE(true, 16);

@@ -29,14 +29,18 @@ constexpr unsigned kMaxHistRows = 64512;  // rows per histogram work item (< 2^1
 constexpr int kCountShift = 47;           // word0 = count << 47 | g
 constexpr int kMaxPlanNodes = 4096;       // nodes per level the planner handles
 constexpr size_t kLdsBudget = 160 * 1024;
-// LDS histograms are laid out in blocks of 16 features (4 quads):
-//   entry(f, bin) = (f / 16) * 4096 + bin * 16 + f % 16.
-// A 64-bit LDS atomic is executed 16 lanes per pass, and two of those lanes
-// collide when their addresses share a bank pair (entry % 16).  With this
-// layout the bank pair is the feature, and the kernels let the 16 lanes of a
-// pass work on 16 different features of their rows, so a pass never has a
+// LDS histograms are laid out bin-major with the features of a bin in blocks
+// of 16 (4 quads): in 64-bit words, one word per entry,
+//   word(f, bin) = bin * 16 * blocks + (f / 16) * 16 + f % 16
+// (twice that with two words per entry, the second word 16 words further; see
+// HistLds).  A 64-bit LDS atomic is executed 16 lanes per pass, and two of
+// those lanes collide when their addresses share a bank pair (word % 16).
+// With this layout the bank pair is f % 16, and the kernels let the 16 lanes
+// of a pass work on 16 different features of their rows, so a pass never has a
 // bank conflict and never two lanes on one address, whatever the bin
-// distribution is (missing values, zeros, a dominant category).
+// distribution is (missing values, zeros, a dominant category).  Entries are
+// counted in "entry order", (f / 16) * 4096 + bin * 16 + f % 16, wherever a
+// histogram is addressed independently of its number of blocks.
 constexpr int kBlockFeatures = 16;
 constexpr int kBlockQuads = 4;
 constexpr int kBlockEntries = kBlockFeatures * kSlots;  // 4096

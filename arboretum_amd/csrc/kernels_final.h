@@ -266,9 +266,10 @@ k_final_hist(const uint32_t *__restrict__ bins, size_t stride, int F, const int 
   if (root_tot != nullptr && threadIdx.x < 64) {
     long long a = 0, b = 0;
     for (int bin = threadIdx.x; bin < kSlots; bin += 64) {
-      const unsigned long long w0 = lds[bin * kBlockFeatures];
+      const unsigned word = HistWord<true>(bin * kBlockFeatures, HistLds<NQ>::blocks);
+      const unsigned long long w0 = lds[word];
       a += ((long long)(w0 << (64 - kCountShift))) >> (64 - kCountShift);
-      b += (long long)lds[HistLds<NQ>::word1 + bin * kBlockFeatures];
+      b += (long long)lds[word + kWord1];
     }
     a = WaveSumLL(a);
     b = WaveSumLL(b);

@@ -7,14 +7,30 @@ namespace arb {
 namespace {
 
 // ---------------------------------------------------------------- histogram
-// LDS layout of a histogram of NQ quads: word0 of every entry, then (PAIR)
-// word1 in the same order.
+// LDS layout of a histogram of NQ quads (B = ceil(NQ / 4) blocks of 16
+// features), in 64-bit words.  Entry (f, bin) of block k = f / 16, f16 = f % 16:
+//   one word per entry (squared objective):  bin * 16 B + k * 16 + f16
+//   two words per entry (PAIR):              bin * 32 B + k * 32 + f16 for word0,
+//                                            16 words (128 bytes) further for word1.
+// The 16 lanes of one pass of an LDS atomic, which work on 16 different
+// features of their rows, fall on 16 different bank pairs (word % 16 = f16),
+// and every update of a row's bin of feature f16 in any block, first or second
+// word, uses ONE address register with an immediate offset.
 template <int NQ>
 struct HistLds {
   static constexpr int blocks = HistBlocks(NQ);
   static constexpr int entries = blocks * kBlockEntries;
-  static constexpr int word1 = entries;  // offset of word1 of the same entry
 };
+// Word of word0 of an entry of a histogram of `blocks` blocks, given the
+// entry's index in entry order (k * 4096 + bin * 16 + f16); word1 is kWord1
+// words further.
+constexpr int kWord1 = kBlockFeatures;
+template <bool PAIR>
+__host__ __device__ __forceinline__ unsigned HistWord(unsigned entry, int blocks) {
+  constexpr unsigned per = PAIR ? 2 : 1;
+  const unsigned k = entry / kBlockEntries, bin = (entry / kBlockFeatures) % kSlots, f16 = entry % kBlockFeatures;
+  return bin * (per * kBlockFeatures * (unsigned)blocks) + k * (per * kBlockFeatures) + f16;
+}
 
 // Adds one row per lane (bins of its NQ quads in b) to the LDS histogram.  The
 // 28 (or 4*NQ) updates of a row are issued in an order that depends on the
@@ -54,30 +70,31 @@ __device__ __forceinline__ void AccumulateRow(unsigned long long *__restrict__ l
         bool on = true;
         if (4 * k + 3 >= NQ) on = 4u * k + qi < (unsigned)NQ;
         if (on) {
-          const unsigned idx = (unsigned)(k * kBlockEntries) + bin * kBlockFeatures + f16;
-          atomicAdd(&lds[idx], w0);
-          if (PAIR) atomicAdd(&lds[L::word1 + idx], w1);
+          constexpr unsigned per = PAIR ? 2 : 1;
+          unsigned long long *cell = &lds[bin * (per * kBlockFeatures * L::blocks) + f16];
+          atomicAdd(cell + k * (per * kBlockFeatures), w0);
+          if (PAIR) atomicAdd(cell + k * (per * kBlockFeatures) + kWord1, w1);
         }
       }
     }
   }
 }
 
-// Writes the LDS histogram to the slab of work item w in LDS order.  Called by
-// the whole workgroup after its last LDS update.  Slab layout per work item:
-// word0[slab_entries], word1[slab_entries]; q_first is a multiple of 4.
+// Writes the LDS histogram to the slab of work item w as it lies in LDS.
+// Called by the whole workgroup after its last LDS update.  A slab holds
+// slab_entries entries (one or two words each): the histograms of the
+// launches (groups of quads) of a level one after the other, each in the
+// layout of HistLds for its own number of blocks; q_first is a multiple of 4.
 template <bool PAIR, int NQ>
 __device__ __forceinline__ void FlushSlab(const unsigned long long *__restrict__ lds,
                                           unsigned long long *__restrict__ slab, unsigned w,
                                           int slab_entries, int q_first) {
   using L = HistLds<NQ>;
+  constexpr int per = PAIR ? 2 : 1;
   __syncthreads();
   unsigned long long *out =
-      slab + (size_t)w * slab_entries * (PAIR ? 2 : 1) + (size_t)(q_first / kBlockQuads) * kBlockEntries;
-  for (int e = threadIdx.x; e < L::entries; e += kHistThreads) {
-    out[e] = lds[e];
-    if (PAIR) out[slab_entries + e] = lds[L::word1 + e];
-  }
+      slab + ((size_t)w * slab_entries + (size_t)(q_first / kBlockQuads) * kBlockEntries) * per;
+  for (int e = threadIdx.x; e < L::entries * per; e += kHistThreads) out[e] = lds[e];
 }
 
 // Histogram of contiguous row ranges: one workgroup per work item, quads

@@ -487,8 +487,9 @@ k_part_rows(const uint32_t *__restrict__ bins, uint32_t *__restrict__ bins_out, 
 
 // Adds the slabs of every directly built node of a level (on top of the stored
 // histogram when `accumulate`) and, with `trick`, derives its sibling as
-// parent - node.  Slabs are in LDS order (16-feature blocks, bin-major); the
-// histograms written here are feature-major: hist[node][f * 256 + bin].
+// parent - node.  Slabs are in LDS order (HistLds; `entry` below counts
+// k * 4096 + bin * 16 + f16 over all blocks of the matrix); the histograms
+// written here are feature-major: hist[node][f * 256 + bin].
 // grid (slab_entries/64, L), 1024 threads = 64 entries x 16 slab lanes.
 //   by_parent = 0: slabs belong to work items of the node itself
 //               (node_items == 0xffffffff marks a derived node);
@@ -502,7 +503,7 @@ k_hist_reduce(const unsigned long long *__restrict__ slab, int slab_entries, int
               const NodeSum *__restrict__ parent_tot, long long *__restrict__ hg,
               long long *__restrict__ hh, unsigned *__restrict__ hc,
               const long long *__restrict__ pg, const long long *__restrict__ ph,
-              const unsigned *__restrict__ pc, int trick, int accumulate, int plain) {
+              const unsigned *__restrict__ pc, int trick, int accumulate, int plain, int group_blocks) {
   // LANES threads share the slabs of one entry; a block covers 1024 / LANES
   // consecutive entries (with 4 lanes: 16 bins x 16 features, so the
   // feature-major output is written in runs of 16 bins)
@@ -534,13 +535,24 @@ k_hist_reduce(const unsigned long long *__restrict__ slab, int slab_entries, int
   long long ag = 0, ah = 0;
   unsigned ac = 0;
   if (live) {
+    // plain slabs: word0 of every entry, then word1 of every entry; others: the
+    // launches of the level (groups of group_blocks blocks, the last one maybe
+    // shorter) one after the other, each in its LDS layout
+    unsigned i0 = (unsigned)entry, i1 = (unsigned)(slab_entries + entry);
+    if (!plain) {
+      const int block = entry / kBlockEntries, group = block / group_blocks;
+      const int blocks_here = min(group_blocks, slab_entries / kBlockEntries - group * group_blocks);
+      const unsigned in_group = (unsigned)(entry - group * group_blocks * kBlockEntries);
+      i0 = (unsigned)(group * group_blocks * kBlockEntries) * (PAIR ? 2u : 1u) + HistWord<PAIR>(in_group, blocks_here);
+      i1 = i0 + kWord1;
+    }
     for (unsigned s = lane; s < items; s += LANES) {
       const unsigned long long *p = slab + (size_t)(first + s) * slab_entries * (PAIR ? 2 : 1);
-      const unsigned long long w0 = p[entry];
+      const unsigned long long w0 = p[i0];
       const long long gq = ((long long)(w0 << (64 - kCountShift))) >> (64 - kCountShift);
       ag += gq;
       ac += (unsigned)((w0 - (unsigned long long)gq) >> kCountShift);
-      if (PAIR) ah += (long long)p[slab_entries + entry];
+      if (PAIR) ah += (long long)p[i1];
     }
   }
   s_g[lane][e] = ag;
