@@ -216,32 +216,34 @@ k_final_hist(const uint32_t *__restrict__ bins, size_t stride, int F, const int 
   const int sg = shifts[0], sh = shifts[1];
   // quad q of a row, zero past the last one
   auto quad = [](const uint32_t (&b)[NQ], int q) { return q < NQ ? b[q < NQ ? q : 0] : 0u; };
-  auto row = [&](const uint32_t (&b)[NQ], float p, float yv, unsigned r) {
-    unsigned node = 0;
-    for (int level = 0; level + 1 < depth; ++level) {
-      const uint2 nd = s_tree[(1 << level) - 1 + (int)node];
-      // the row's bin of the split feature: byte fid % 8 of each pair of quads, then the pair
-      const uint32_t t0 = __builtin_amdgcn_perm(quad(b, 1), quad(b, 0), nd.x);
-      const uint32_t t1 = __builtin_amdgcn_perm(quad(b, 3), quad(b, 2), nd.x);
-      const uint32_t t2 = __builtin_amdgcn_perm(quad(b, 5), quad(b, 4), nd.x);
-      const uint32_t t3 = __builtin_amdgcn_perm(quad(b, 7), quad(b, 6), nd.x);
-      const unsigned pair = nd.y >> 8;
-      const uint32_t lo = pair == 1u ? t1 : t0, hi = pair == 3u ? t3 : t2;
-      const uint32_t v = pair >= 2u ? hi : lo;
-      node = node * 2 + (v > (nd.y & 255u) ? 1u : 0u);  // bin >= q + 1 goes right (builder.h:107-123)
-    }
-    if (leaf_of != nullptr) __builtin_nontemporal_store(node, &leaf_of[r]);  // uniform
+  // one step of the walk of a row from `node` at `level`
+  auto step = [&](const uint32_t (&b)[NQ], unsigned node, int level) {
+    const uint2 nd = s_tree[(1 << level) - 1 + (int)node];
+    // the row's bin of the split feature: byte fid % 8 of each pair of quads, then the pair
+    const uint32_t t0 = __builtin_amdgcn_perm(quad(b, 1), quad(b, 0), nd.x);
+    const uint32_t t1 = __builtin_amdgcn_perm(quad(b, 3), quad(b, 2), nd.x);
+    const uint32_t t2 = __builtin_amdgcn_perm(quad(b, 5), quad(b, 4), nd.x);
+    const uint32_t t3 = __builtin_amdgcn_perm(quad(b, 7), quad(b, 6), nd.x);
+    const unsigned pair = nd.y >> 8;
+    const uint32_t lo = pair == 1u ? t1 : t0, hi = pair == 3u ? t3 : t2;
+    const uint32_t v = pair >= 2u ? hi : lo;
+    return node * 2 + (v > (nd.y & 255u) ? 1u : 0u);  // bin >= q + 1 goes right (builder.h:107-123)
+  };
+  // leaf weight, prediction, gradients of a row; returns (g, h) for the histogram
+  auto finish = [&](unsigned node, float p, float yv, unsigned r, bool live, float *gv, float *hv) {
     const float yh = p + weights[node];
-    yhat[r] = yh;
     const float s = SigmoidF(yh);
-    const float gv = yv - s, hv = s * (1.0f - s);
+    *gv = yv - s;
+    *hv = s * (1.0f - s);
+    if (!live) return;
+    if (leaf_of != nullptr) __builtin_nontemporal_store(node, &leaf_of[r]);  // uniform
+    yhat[r] = yh;
     if (h != nullptr) {  // uniform
-      g[r] = gv;
-      h[r] = hv;
+      g[r] = *gv;
+      h[r] = *hv;
     } else {
       g[r] = PackGrad(s, yv);
     }
-    AccumulateRow<true, NQ>(lds, b, gv, hv, sg, sh, 0, F);
   };
   for (unsigned base = it.begin; base < it.end; base += 2 * kHistThreads) {
     const unsigned r0 = base + threadIdx.x, r1 = r0 + kHistThreads;
@@ -255,8 +257,17 @@ k_final_hist(const uint32_t *__restrict__ bins, size_t stride, int F, const int 
     }
     const float p0 = yhat[a0], p1 = yhat[a1];
     const float y0 = __builtin_nontemporal_load(&y[a0]), y1 = __builtin_nontemporal_load(&y[a1]);
-    if (v0) row(b0, p0, y0, r0);
-    if (v1) row(b1, p1, y1, r1);
+    // the two rows of a thread walk side by side: their table lookups overlap
+    unsigned n0 = 0, n1 = 0;
+    for (int level = 0; level + 1 < depth; ++level) {
+      n0 = step(b0, n0, level);
+      n1 = step(b1, n1, level);
+    }
+    float g0, h0, g1, h1;
+    finish(n0, p0, y0, r0, v0, &g0, &h0);
+    finish(n1, p1, y1, r1, v1, &g1, &h1);
+    if (v0) AccumulateRow<true, NQ>(lds, b0, g0, h0, sg, sh, 0, F);
+    if (v1) AccumulateRow<true, NQ>(lds, b1, g1, h1, sg, sh, 0, F);
   }
   FlushSlab<true, NQ>(lds, slab, w, slab_entries, 0);
   // Totals of the next root (garden.cu:432-435 reduces the gradient array):
