@@ -100,24 +100,20 @@ __device__ __forceinline__ void WaveOffsets(const WorkItem &it, const SplitRec &
   *ro = start + (unsigned)s.left.c + rows_before - lefts_before;
 }
 
-// Position of the k-th (0-based) set bit of the wave-uniform mask m; k < popcount(m).
-__device__ __forceinline__ int SelectBit(unsigned long long m, unsigned k) {
-  const unsigned lo = (unsigned)m, hi = (unsigned)(m >> 32);
-  unsigned c = (unsigned)__popc(lo);
-  const bool up = k >= c;
-  unsigned word = up ? hi : lo;
-  int pos = up ? 32 : 0;
-  k = up ? k - c : k;
-#pragma unroll
-  for (int width = 16; width >= 1; width >>= 1) {
-    const unsigned low = word & ((1u << width) - 1u);
-    c = (unsigned)__popc(low);
-    const bool u = k >= c;
-    word = u ? (word >> width) : low;
-    pos += u ? width : 0;
-    k = u ? k - c : k;
-  }
-  return pos;
+// Destination lane of this lane's row when the rows flagged in the
+// wave-uniform mask m are packed, in lane order, into lanes first, first + 1,
+// ... (mod 64) of a wave: the flagged rows first, the others behind them, so
+// the 64 destinations are a permutation and ds_permute_b32 (every lane sends
+// its value to its destination) moves a register in one instruction.
+__device__ __forceinline__ int PackedLane(unsigned long long m, unsigned first, int lane) {
+  const unsigned below = RankBelow(m);  // flagged rows in the lanes below this one
+  const bool mine = (m >> lane) & 1ull;
+  const unsigned pos = mine ? below : (unsigned)__popcll(m) + ((unsigned)lane - below);
+  return (int)((first + pos) & 63u);
+}
+// x of every lane to lane `dst` (a permutation of the lanes).
+__device__ __forceinline__ uint32_t SendTo(int dst, uint32_t x) {
+  return (uint32_t)__builtin_amdgcn_ds_permute(dst << 2, (int)x);
 }
 
 // Two rows per lane of a wave's 128-row chunk, as loaded.
@@ -175,7 +171,7 @@ __device__ __forceinline__ void EmitRows(unsigned long long *__restrict__ lds, c
 }
 
 // Appends the rows of X flagged in xm (wave-uniform mask, one row per lane) to
-// Q in row order with one lane permute per register; a full queue is emitted
+// Q in row order with one lane permute (ds_permute_b32) per register; a full queue is emitted
 // and the rest of X starts the next batch.
 template <bool PAIR, int NQ, bool HIST = true, bool GH = true, bool PACK = false>
 __device__ __forceinline__ void MergeRows(unsigned long long *__restrict__ lds, RowQueue<NQ> &Q,
@@ -189,12 +185,12 @@ __device__ __forceinline__ void MergeRows(unsigned long long *__restrict__ lds, 
   // lane l receives the k-th flagged row, k = (l - n) mod 64: lanes >= n fill
   // the current batch, lanes < n hold what overflows into the next one
   const unsigned k = ((unsigned)lane - Q.n) & 63u;
-  const int src = SelectBit(xm, k < nx ? k : 0u);
+  const int dst = PackedLane(xm, Q.n, lane);
   uint32_t vb[NQ];
 #pragma unroll
-  for (int q = 0; q < NQ; ++q) vb[q] = (uint32_t)__shfl((int)xb[q], src);
-  const float vg = GH ? __shfl(xg, src) : 0.0f;
-  const float vh = GH && PAIR && !PACK ? __shfl(xh, src) : 0.0f;
+  for (int q = 0; q < NQ; ++q) vb[q] = SendTo(dst, xb[q]);
+  const float vg = GH ? __uint_as_float(SendTo(dst, __float_as_uint(xg))) : 0.0f;
+  const float vh = GH && PAIR && !PACK ? __uint_as_float(SendTo(dst, __float_as_uint(xh))) : 0.0f;
   if (Q.n + nx >= 64u) {  // wave-uniform: the batch is complete
     const bool fill = (unsigned)lane >= Q.n;
 #pragma unroll
@@ -356,7 +352,7 @@ k_part_hist(const uint32_t *__restrict__ bins, uint32_t *__restrict__ bins_out, 
       if (nx == 0) return;
       const unsigned r = np & 63u, j = np >> 6;
       const unsigned k = ((unsigned)lane - r) & 63u;  // slot np + k
-      const unsigned id = base + (unsigned)SelectBit(m, k < nx ? k : 0u);
+      const unsigned id = SendTo(PackedLane(m, r, lane), base + (unsigned)lane);
       const bool here = (unsigned)lane >= r && k < nx;   // lands in q[j]
       const bool next = (unsigned)lane < r && k < nx;    // lands in q[j + 1]
       q0 = (j == 0 && here) ? id : q0;
