@@ -977,7 +977,7 @@ class HipTreeBuilder : public TreeBuilder {
     Mark(kSplit);
     const int hs = std::min(cfg_.internal.hist_size, slots_);
     const unsigned char *active = sampling_ ? d_active_ + (size_t)level * F_ : (const unsigned char *)nullptr;
-    const unsigned per_item = HistRowsPerItem(n_);
+    const unsigned per_item = FusedRowsPerItem(L);
     // From 32 nodes on, one launch: a workgroup per node scans its features and
     // selects.  With fewer nodes that would leave the gain arithmetic (28
     // features x 256 bins in double precision per node) on a few CUs, and the
@@ -1045,7 +1045,17 @@ class HipTreeBuilder : public TreeBuilder {
 
   // launch bound of the fused pass over PL parent nodes
   unsigned FusedGrid(int PL) const {
-    return (unsigned)std::min<size_t>(n_ / HistRowsPerItem(n_) + 2 * PL + 1, max_part_items_);
+    return (unsigned)std::min<size_t>(n_ / FusedRowsPerItem(PL) + 2 * PL + 1, max_part_items_);
+  }
+  // Rows per work item of the fused pass over PL parents.  A CU runs one
+  // workgroup at a time, so the pass takes as many rounds as items / CUs rounded
+  // up, and a round with a single item costs as much as a full one (measured:
+  // 513 items take 18 % longer than 489).  Every parent adds a short item or
+  // two at its ends; the items are sized to stay under one round for one or
+  // two parents and under two rounds otherwise.
+  unsigned FusedRowsPerItem(int PL) const {
+    const size_t target = PL <= 2 ? 246 : (size_t)std::max(256, 496 - PL);
+    return HistRowsPerItem(n_, target);
   }
 
   void LaunchLeafWeights(int L, int state, const GainParams &gp) {
