@@ -1051,10 +1051,10 @@ class HipTreeBuilder : public TreeBuilder {
   // workgroup at a time, so the pass takes as many rounds as items / CUs rounded
   // up, and a round with a single item costs as much as a full one (measured:
   // 513 items take 18 % longer than 489).  Every parent adds a short item or
-  // two at its ends; the items are sized to stay under one round for one or
-  // two parents and under two rounds otherwise.
+  // two at its ends; the items are sized so that all of them fit one round
+  // (fewer, larger slabs as well) up to 32 parents and two rounds beyond.
   unsigned FusedRowsPerItem(int PL) const {
-    const size_t target = PL <= 2 ? 246 : (size_t)std::max(256, 496 - PL);
+    const size_t target = PL <= 32 ? (size_t)(250 - 2 * PL) : (size_t)std::max(256, 496 - PL);
     return HistRowsPerItem(n_, target);
   }
 
