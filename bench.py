@@ -302,7 +302,7 @@ def main():
         "phase_trees": phase_trees,
         "quantise_s": t_quant,
     }
-    if not args.no_cpu:
+    if not args.no_cpu and args.cpu_trees > 0:
         out["cpu_baseline"] = cpu_baseline(X, y, cfg, min(args.cpu_rows, args.rows), args.cpu_trees)
     print(json.dumps(out))
 
