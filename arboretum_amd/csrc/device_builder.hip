@@ -837,7 +837,7 @@ class HipTreeBuilder : public TreeBuilder {
     // one: logistic objective, gradients of the next round wanted, all quads in
     // one LDS histogram next to the node arrays.
     const bool next_grad = !inspect_ && K_ == 1;
-    const size_t final_lds = HistLdsBytes(Q_, true) + (size_t)((1 << (D_ - 1)) - 1) * 2 * sizeof(int);
+    const size_t final_lds = FinalHistLdsBytes(Q_, D_);
     const bool final_hist = next_grad && cfg_.objective == kLogisticRegression && single_group_ && !wide_ &&
                             final_lds <= kLdsBudget;
     int state = 0;  // d_tot_/d_seg_[state] describe the nodes of the current level

@@ -189,34 +189,33 @@ ARB_HD float LeafWeightKind(int kind, double g, double h, unsigned c, const Gain
 // ------------------------------------------------------------------ exp
 // exp of a float evaluated in double with a fixed operation order (range
 // reduction by ln2/32, 32-entry table, degree-7 polynomial) so that host and
-// device give identical bits.  The sigmoid follows src/core/objective.h:67-69:
-// float exp, double 1/(1+e), rounded to float.
-ARB_HD double Exp2Table(int j) {
-  switch (j) {
-    case 0: return 0x1.0000000000000p+0; case 1: return 0x1.059b0d3158574p+0;
-    case 2: return 0x1.0b5586cf9890fp+0; case 3: return 0x1.11301d0125b51p+0;
-    case 4: return 0x1.172b83c7d517bp+0; case 5: return 0x1.1d4873168b9aap+0;
-    case 6: return 0x1.2387a6e756238p+0; case 7: return 0x1.29e9df51fdee1p+0;
-    case 8: return 0x1.306fe0a31b715p+0; case 9: return 0x1.371a7373aa9cbp+0;
-    case 10: return 0x1.3dea64c123422p+0; case 11: return 0x1.44e086061892dp+0;
-    case 12: return 0x1.4bfdad5362a27p+0; case 13: return 0x1.5342b569d4f82p+0;
-    case 14: return 0x1.5ab07dd485429p+0; case 15: return 0x1.6247eb03a5585p+0;
-    case 16: return 0x1.6a09e667f3bcdp+0; case 17: return 0x1.71f75e8ec5f74p+0;
-    case 18: return 0x1.7a11473eb0187p+0; case 19: return 0x1.82589994cce13p+0;
-    case 20: return 0x1.8ace5422aa0dbp+0; case 21: return 0x1.93737b0cdc5e5p+0;
-    case 22: return 0x1.9c49182a3f090p+0; case 23: return 0x1.a5503b23e255dp+0;
-    case 24: return 0x1.ae89f995ad3adp+0; case 25: return 0x1.b7f76f2fb5e47p+0;
-    case 26: return 0x1.c199bdd85529cp+0; case 27: return 0x1.cb720dcef9069p+0;
-    case 28: return 0x1.d5818dcfba487p+0; case 29: return 0x1.dfc97337b9b5fp+0;
-    case 30: return 0x1.ea4afa2a490dap+0; default: return 0x1.f50765b6e4540p+0;
-  }
+// device give identical bits.  The table is an array in constant memory: a
+// switch over its entries compiles, on the GPU, to a tree of divergent
+// branches that costs several times the rest of the function.  The sigmoid
+// follows src/core/objective.h:67-69: float exp, double 1/(1+e), rounded to
+// float.
+
+// 2^(j/32) rounded to double, j in [0, 32)
+ARB_HD const double *Exp2Table() {
+  static constexpr double kTable[32] = {
+      0x1.0000000000000p+0, 0x1.059b0d3158574p+0, 0x1.0b5586cf9890fp+0, 0x1.11301d0125b51p+0,
+      0x1.172b83c7d517bp+0, 0x1.1d4873168b9aap+0, 0x1.2387a6e756238p+0, 0x1.29e9df51fdee1p+0,
+      0x1.306fe0a31b715p+0, 0x1.371a7373aa9cbp+0, 0x1.3dea64c123422p+0, 0x1.44e086061892dp+0,
+      0x1.4bfdad5362a27p+0, 0x1.5342b569d4f82p+0, 0x1.5ab07dd485429p+0, 0x1.6247eb03a5585p+0,
+      0x1.6a09e667f3bcdp+0, 0x1.71f75e8ec5f74p+0, 0x1.7a11473eb0187p+0, 0x1.82589994cce13p+0,
+      0x1.8ace5422aa0dbp+0, 0x1.93737b0cdc5e5p+0, 0x1.9c49182a3f090p+0, 0x1.a5503b23e255dp+0,
+      0x1.ae89f995ad3adp+0, 0x1.b7f76f2fb5e47p+0, 0x1.c199bdd85529cp+0, 0x1.cb720dcef9069p+0,
+      0x1.d5818dcfba487p+0, 0x1.dfc97337b9b5fp+0, 0x1.ea4afa2a490dap+0, 0x1.f50765b6e4540p+0};
+  return kTable;
 }
 
-ARB_HD float ExpF(float xf) {
-  if (xf != xf) return xf;
-  if (xf > 88.8f) return INFINITY;
-  if (xf < -104.0f) return 0.0f;
-  const double x = (double)xf;
+// table: the 32 values of Exp2Table, wherever the caller keeps them
+ARB_HD float ExpFrom(float xf, const double *table) {
+  // Straight-line code: the polynomial runs on the clamped argument and the
+  // special cases are selected at the end, so that the evaluations of several
+  // rows of a GPU thread interleave (fmaxf drops a NaN: it is put back last).
+  const float xc = fminf(fmaxf(xf, -104.0f), 88.8f);
+  const double x = (double)xc;
   const double kd = rint(x * 0x1.71547652b82fep+5);   // 32 / ln 2
   const int k = (int)kd;
   const double r = x - kd * 0x1.62e42fefa39efp-6;     // ln 2 / 32
@@ -230,10 +229,19 @@ ARB_HD float ExpF(float xf) {
   p = p * r + 1.0;
   const int j = k & 31;
   const int m = (k - j) / 32;
-  return (float)ldexp(Exp2Table(j) * p, m);
+  float e = (float)ldexp(table[j] * p, m);
+  e = xf > 88.8f ? INFINITY : e;
+  e = xf < -104.0f ? 0.0f : e;
+  return xf != xf ? xf : e;
 }
 
+ARB_HD float ExpF(float xf) { return ExpFrom(xf, Exp2Table()); }
+
 ARB_HD float SigmoidF(float x) { return (float)(1.0 / (1.0 + (double)ExpF(-x))); }
+// the same with the caller's copy of the table (a kernel that keeps it in LDS)
+ARB_HD float SigmoidFrom(float x, const double *table) {
+  return (float)(1.0 / (1.0 + (double)ExpFrom(-x, table)));
+}
 
 }  // namespace arb
 #endif  // ARBORETUM_AMD_GAIN_H_

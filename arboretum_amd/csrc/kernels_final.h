@@ -184,6 +184,11 @@ k_final(const uint32_t *__restrict__ bins, size_t stride, const int *__restrict_
 // leaf_of may be null: the leaf ids are then not recorded (k_leaf_ids
 // computes them on demand).  root_tot (may be null): the gradient totals of
 // the next root are added to root_tot[0].g / .h, which the caller has zeroed.
+// LDS bytes of k_final_hist: histogram, node table, exp table, leaf weights
+constexpr size_t FinalHistLdsBytes(int nq, int depth) {
+  return HistLdsBytes(nq, true) + (size_t)((1 << (depth - 1)) - 1) * 8 + 32 * 8 + ((size_t)1 << (depth - 1)) * 4;
+}
+
 template <int NQ>
 __global__ void __launch_bounds__(kHistThreads)
 k_final_hist(const uint32_t *__restrict__ bins, size_t stride, int F, const int *__restrict__ t_fid,
@@ -203,8 +208,13 @@ k_final_hist(const uint32_t *__restrict__ bins, size_t stride, int F, const int 
   // in bits 8-9.  A node that was not split compares against 255: no bin id is
   // larger, so every row stays left.
   uint2 *s_tree = reinterpret_cast<uint2 *>(lds + words);
-  const int internal = (1 << (depth - 1)) - 1;
+  const int internal = (1 << (depth - 1)) - 1, leaves = internal + 1;
+  // the exp table and the leaf weights are read from LDS as well
+  double *s_exp = reinterpret_cast<double *>(s_tree + internal);
+  float *s_weight = reinterpret_cast<float *>(s_exp + 32);
   for (int i = threadIdx.x; i < words; i += kHistThreads) lds[i] = 0ull;
+  if (threadIdx.x < 32) s_exp[threadIdx.x] = Exp2Table()[threadIdx.x];
+  for (int i = threadIdx.x; i < leaves; i += kHistThreads) s_weight[i] = weights[i];
   for (int i = threadIdx.x; i < internal; i += kHistThreads) {
     const int fid = t_fid[i], bin = t_bin[i];
     uint2 nd;
@@ -216,9 +226,8 @@ k_final_hist(const uint32_t *__restrict__ bins, size_t stride, int F, const int 
   const int sg = shifts[0], sh = shifts[1];
   // quad q of a row, zero past the last one
   auto quad = [](const uint32_t (&b)[NQ], int q) { return q < NQ ? b[q < NQ ? q : 0] : 0u; };
-  // one step of the walk of a row from `node` at `level`
-  auto step = [&](const uint32_t (&b)[NQ], unsigned node, int level) {
-    const uint2 nd = s_tree[(1 << level) - 1 + (int)node];
+  // one step of the walk of a row from `node`, whose table entry is nd
+  auto step_at = [&](const uint32_t (&b)[NQ], unsigned node, uint2 nd) {
     // the row's bin of the split feature: byte fid % 8 of each pair of quads, then the pair
     const uint32_t t0 = __builtin_amdgcn_perm(quad(b, 1), quad(b, 0), nd.x);
     const uint32_t t1 = __builtin_amdgcn_perm(quad(b, 3), quad(b, 2), nd.x);
@@ -229,18 +238,21 @@ k_final_hist(const uint32_t *__restrict__ bins, size_t stride, int F, const int 
     const uint32_t v = pair >= 2u ? hi : lo;
     return node * 2 + (v > (nd.y & 255u) ? 1u : 0u);  // bin >= q + 1 goes right (builder.h:107-123)
   };
-  // leaf weight, prediction, gradients of a row; returns (g, h) for the histogram
-  auto finish = [&](unsigned node, float p, float yv, unsigned r, bool live, float *gv, float *hv) {
-    const float yh = p + weights[node];
-    const float s = SigmoidF(yh);
-    *gv = yv - s;
-    *hv = s * (1.0f - s);
-    if (!live) return;
+  auto step = [&](const uint32_t (&b)[NQ], unsigned node, int level) {
+    return step_at(b, node, s_tree[(1 << level) - 1 + (int)node]);
+  };
+  // The entries of the two top levels stay in registers: every row passes
+  // them, and a table read waits behind the histogram updates of the other
+  // waves in the LDS queue.
+  const uint2 top0 = s_tree[0];
+  const uint2 top1 = internal > 2 ? s_tree[1] : top0, top2 = internal > 2 ? s_tree[2] : top0;
+  // records leaf, prediction and gradients of row r
+  auto record = [&](unsigned node, float yh, float s, float yv, float gv, float hv, unsigned r) {
     if (leaf_of != nullptr) __builtin_nontemporal_store(node, &leaf_of[r]);  // uniform
     yhat[r] = yh;
     if (h != nullptr) {  // uniform
-      g[r] = *gv;
-      h[r] = *hv;
+      g[r] = gv;
+      h[r] = hv;
     } else {
       g[r] = PackGrad(s, yv);
     }
@@ -259,13 +271,31 @@ k_final_hist(const uint32_t *__restrict__ bins, size_t stride, int F, const int 
     const float y0 = __builtin_nontemporal_load(&y[a0]), y1 = __builtin_nontemporal_load(&y[a1]);
     // the two rows of a thread walk side by side: their table lookups overlap
     unsigned n0 = 0, n1 = 0;
-    for (int level = 0; level + 1 < depth; ++level) {
+    if (depth > 1) {
+      n0 = step_at(b0, 0u, top0);
+      n1 = step_at(b1, 0u, top0);
+    }
+    if (depth > 2) {
+      uint2 e0, e1;
+      e0.x = n0 ? top2.x : top1.x;
+      e0.y = n0 ? top2.y : top1.y;
+      e1.x = n1 ? top2.x : top1.x;
+      e1.y = n1 ? top2.y : top1.y;
+      n0 = step_at(b0, n0, e0);
+      n1 = step_at(b1, n1, e1);
+    }
+    for (int level = 2; level + 1 < depth; ++level) {
       n0 = step(b0, n0, level);
       n1 = step(b1, n1, level);
     }
-    float g0, h0, g1, h1;
-    finish(n0, p0, y0, r0, v0, &g0, &h0);
-    finish(n1, p1, y1, r1, v1, &g1, &h1);
+    // leaf weights, predictions and gradients of the two rows, side by side
+    // as well
+    const float yh0 = p0 + s_weight[n0], yh1 = p1 + s_weight[n1];
+    const float s0 = SigmoidFrom(yh0, s_exp), s1 = SigmoidFrom(yh1, s_exp);
+    const float g0 = y0 - s0, g1 = y1 - s1;
+    const float h0 = s0 * (1.0f - s0), h1 = s1 * (1.0f - s1);
+    if (v0) record(n0, yh0, s0, y0, g0, h0, r0);
+    if (v1) record(n1, yh1, s1, y1, g1, h1, r1);
     if (v0) AccumulateRow<true, NQ>(lds, b0, g0, h0, sg, sh, 0, F);
     if (v1) AccumulateRow<true, NQ>(lds, b1, g1, h1, sg, sh, 0, F);
   }
