@@ -1050,11 +1050,13 @@ class HipTreeBuilder : public TreeBuilder {
   // Rows per work item of the fused pass over PL parents.  A CU runs one
   // workgroup at a time, so the pass takes as many rounds as items / CUs rounded
   // up, and a round with a single item costs as much as a full one (measured:
-  // 513 items take 18 % longer than 489).  Every parent adds a short item or
-  // two at its ends; the items are sized so that all of them fit one round
-  // (fewer, larger slabs as well) up to 32 parents and two rounds beyond.
+  // 513 items take 18 % longer than 489).  Items are cut at multiples of the
+  // item size from a node's start, so every parent adds at most one item to
+  // rows / size (its last, short one); the size is chosen so that all items
+  // fit one round (fewer, larger slabs as well) up to 32 parents and two rounds
+  // beyond.
   unsigned FusedRowsPerItem(int PL) const {
-    const size_t target = PL <= 32 ? (size_t)(250 - 2 * PL) : (size_t)std::max(256, 496 - PL);
+    const size_t target = PL <= 32 ? (size_t)(254 - PL) : (size_t)std::max(256, 508 - PL);
     return HistRowsPerItem(n_, target);
   }
 
