@@ -159,6 +159,27 @@ def test_logistic_with_fractional_labels(arb, oracle, inspect, trick):
     assert_same_training(arb, oracle, X, y, cfg, rounds=4, check_hist=inspect)
 
 
+@pytest.mark.parametrize("inspect", [True, False])
+@pytest.mark.parametrize("eta", [30.0, 70.0, 1e4])
+def test_logistic_with_saturated_predictions(arb, oracle, inspect, eta):
+    # a huge learning rate drives the raw predictions past the range of exp (|x| > 88.8 and
+    # > 104): the sigmoid saturates to 0 and 1, hessians vanish, leaf weights blow up.  The
+    # device evaluates exp as straight-line code with the special cases selected at the end;
+    # the checker branches first.  Both must give the same bits, predictions included.
+    X, y = make_data(20000, 6, 1, seed=5)
+    cfg = {"objective": 1, "method": 1, "internals": {"hist_size": 32, "double_precision": True},
+           "tree": {"max_depth": 4, "eta": eta, "lambda": 1e-3, "min_child_weight": 0.0}}
+    assert_same_training(arb, oracle, X, y, cfg, rounds=4, check_hist=inspect)
+    data = arb.DMatrix(X, y=y)
+    g = arb.Garden(cfg, data)
+    for _ in range(4):
+        g.grow_tree()
+    raw = g.train_yhat()
+    assert np.abs(raw).max() > 104.0    # the case the test is about
+    p = g.predict(data)
+    assert np.isfinite(p).all() and p.min() == 0.0 and p.max() == 1.0
+
+
 @pytest.mark.parametrize("n,F,depth", [(1, 3, 2), (65, 1, 1), (2049, 5, 3), (70000, 8, 4), (5000, 32, 5)])
 def test_last_pass_feeds_next_root_histogram(arb, oracle, n, F, depth):
     # logistic, inspection off: the pass that assigns the leaves of a tree also
