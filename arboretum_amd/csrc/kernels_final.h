@@ -176,19 +176,20 @@ k_final(const uint32_t *__restrict__ bins, size_t stride, const int *__restrict_
   }
 }
 
-// Last pass of a tree fused with the root histogram of the next one
-// (logistic objective, resident matrix, all quads in one LDS histogram): the
-// rows are read once; the leaf walk, the prediction update and the new
-// gradients are bound by HBM, the histogram by LDS atomics, and they overlap.
-// One workgroup per root work item; LDS: histogram, then the node arrays.
-// leaf_of may be null: the leaf ids are then not recorded (k_leaf_ids
-// computes them on demand).  root_tot (may be null): the gradient totals of
-// the next root are added to root_tot[0].g / .h, which the caller has zeroed.
 // LDS bytes of k_final_hist: histogram, node table, exp table, leaf weights
 constexpr size_t FinalHistLdsBytes(int nq, int depth) {
   return HistLdsBytes(nq, true) + (size_t)((1 << (depth - 1)) - 1) * 8 + 32 * 8 + ((size_t)1 << (depth - 1)) * 4;
 }
 
+// Last pass of a tree fused with the root histogram of the next one
+// (logistic objective, resident matrix, all quads in one LDS histogram): the
+// rows are read once.  The histogram updates set the duration (the LDS is
+// busy 85 % of it); the leaf walk, the prediction update and the new
+// gradients run in their shadow as far as the waves of a CU interleave.
+// One workgroup per root work item; LDS: FinalHistLdsBytes.
+// leaf_of may be null: the leaf ids are then not recorded (k_leaf_ids
+// computes them on demand).  root_tot (may be null): the gradient totals of
+// the next root are added to root_tot[0].g / .h, which the caller has zeroed.
 template <int NQ>
 __global__ void __launch_bounds__(kHistThreads)
 k_final_hist(const uint32_t *__restrict__ bins, size_t stride, int F, const int *__restrict__ t_fid,
