@@ -310,6 +310,17 @@ def test_deep_trees(arb, oracle, depth, objective, trick, upload):
     assert_same_training(arb, oracle, X, y, cfg, rounds=2, check_hist=(depth <= 11))
 
 
+@pytest.mark.parametrize("depth", [11, 12])
+def test_deep_trees_on_28_features(arb, oracle, depth):
+    # logistic, inspection off, 7 quads: the last pass keeps the 128 KB histogram of the next root,
+    # the node table, the leaf weights and the exp table in LDS; at depth 11 they just fit (152 KB),
+    # at depth 12 they do not and the pass runs without the histogram
+    X, y = make_data(100000, 28, 1, seed=100 + depth, nan_frac=0.01)
+    cfg = {"objective": 1, "method": 1, "internals": {"hist_size": 255, "double_precision": True},
+           "tree": {"max_depth": depth, "eta": 0.3, "lambda": 1.0, "min_child_weight": 0.0, "min_leaf_size": 0}}
+    assert_same_training(arb, oracle, X, y, cfg, rounds=3, check_hist=False)
+
+
 def test_depth_limit_is_an_error(arb):
     X, y = make_data(1000, 3, 0, seed=1)
     cfg = {"objective": 0, "method": 1, "internals": {"hist_size": 16}, "tree": {"max_depth": 14}}
