@@ -184,8 +184,8 @@ constexpr size_t FinalHistLdsBytes(int nq, int depth) {
 // Last pass of a tree fused with the root histogram of the next one
 // (logistic objective, resident matrix, all quads in one LDS histogram): the
 // rows are read once.  The histogram updates set the duration (the LDS is
-// busy 85 % of it); the leaf walk, the prediction update and the new
-// gradients run in their shadow as far as the waves of a CU interleave.
+// busy three quarters of it); the leaf walk, the prediction update and the
+// new gradients run in their shadow as far as the waves of a CU interleave.
 // One workgroup per root work item; LDS: FinalHistLdsBytes.
 // leaf_of may be null: the leaf ids are then not recorded (k_leaf_ids
 // computes them on demand).  root_tot (may be null): the gradient totals of
