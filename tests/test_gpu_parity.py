@@ -492,6 +492,40 @@ def test_softmax_matches_oracle(arb, oracle):
     assert acc > 0.45     # far above chance (1/3): the trees learn
 
 
+@pytest.mark.parametrize("seed", range(8))
+def test_softmax_random_configurations(arb, oracle, seed):
+    # both soft-max objectives over drawn shapes: class counts, depths, bin counts, missing values,
+    # resident and streamed bins, with and without sibling subtraction and inspection
+    rng = np.random.default_rng(900 + seed)
+    n = int(rng.choice([257, 3000, 20000]))
+    F = int(rng.choice([2, 7, 28, 33]))
+    K = int(rng.choice([2, 3, 7]))
+    X = rng.normal(size=(n, F)).astype(np.float32)
+    X[rng.random(X.shape) < 0.02] = np.nan
+    W = rng.normal(size=(F, K))
+    labels = np.argmax(np.nan_to_num(X) @ W + rng.gumbel(size=(n, K)), axis=1).astype(np.uint8)
+    labels[:K] = np.arange(K, dtype=np.uint8)   # every class present
+    cfg = {"objective": int(rng.choice([3, 4])), "method": 1,
+           "internals": {"hist_size": int(rng.choice([16, 64, 255])), "double_precision": bool(rng.integers(0, 2)),
+                         "use_hist_subtraction_trick": bool(rng.integers(0, 2)),
+                         "upload_features": bool(rng.random() < 0.7), "stream_block_rows": 1000},
+           "tree": {"max_depth": int(rng.integers(1, 6)), "eta": 0.3, "lambda": float(rng.choice([0.5, 1.0])),
+                    "min_child_weight": float(rng.choice([0.0, 1.0])), "labels_count": K}}
+    ob = oracle.Booster(X, labels=labels, config=cfg)
+    data = arb.DMatrix(X, labels=labels)
+    g = arb.Garden(cfg, data)
+    g.set_inspect(bool(seed & 1))
+    for r in range(3):
+        ob.grow(1)
+        g.grow_tree()
+        for k in range(K):
+            to, tg = ob.tree(r * K + k), g.tree(r * K + k)
+            for key in ("fid", "quantized", "threshold", "gain", "weights"):
+                assert np.array_equal(to[key], tg[key], equal_nan=True), (key, r, k)
+        assert np.array_equal(ob.yhat(), g.train_yhat()), "y_hat round %d" % r
+    assert np.allclose(ob.predict(X), g.predict(data), rtol=0, atol=1e-6, equal_nan=True)
+
+
 # ------------------------------------------------------ reference goldens
 def _golden_cases(arb, fixture, X, y):
     for name, case in fixture["cases"].items():
