@@ -31,9 +31,17 @@
 //                       pinned: golden models and predictions of
 //                       tests/py/test_hist_regregression.py and
 //                       tests/py/test_hist_logregression.py
-//   softmax grad/hess   PARITY UNPINNED: the reference's kernel is empty
-//                       (src/core/objective.cu:91-100); only the commented
-//                       formula at objective.cu:60-89 exists.
+//   softmax grad/hess, softmax link
+//                       pinned by the mathematics: the reference's kernel is
+//                       empty (src/core/objective.cu:91-100) and holds the
+//                       formula only as the comment at objective.cu:60-89, the
+//                       link at objective.h:80-113.  Checked against a float64
+//                       scipy soft-max, the K = 2 reduction to the logistic
+//                       sigmoid, sum-to-zero / range invariants and the central
+//                       difference of the log-likelihood.
+//   column sampling     PARITY UNPINNED against the reference's std::shuffle
+//                       stream (garden.cu:126-165): no reference test holds a
+//                       sampled model; only the error strings are pinned.
 //   orc_expf            defined here (double polynomial, correctly rounded in
 //                       all but rare cases); checked against libm within 1 ulp.
 // ---------------------------------------------------------------------------
@@ -380,7 +388,7 @@ static float into_internal(int objective, float v) {
 
 // ------------------------------------------------------------ objectives
 // src/core/objective.cu:28-56 (squared, logistic); softmax after the
-// commented formula at objective.cu:60-89 (parity unpinned).
+// commented formula at objective.cu:60-89.
 static void update_grad(Booster &b) {
   const int64_t n = b.n;
   const int K = b.p.labels_count;

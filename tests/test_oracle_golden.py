@@ -260,3 +260,109 @@ def test_baseline_config_0_on_the_oracle(oracle):
     assert all(b < a for a, b in zip(errors, errors[1:]))
     assert errors[-1] < 0.25 * np.var(y)
     assert np.allclose(ob.predict(X), ob.yhat(), atol=1e-5)
+
+
+# ----------------------------------------------------------------- soft-max
+# The reference's soft-max gradient kernel is empty; what it holds is the formula in the
+# comment at src/core/objective.cu:60-89 (g = [k == label] - p_k, h = 2 p_k (1 - p_k)) and
+# the link at src/core/objective.h:80-113.  The checks below pin the checker's restatement
+# with routines that share no code with it: float64 numpy / scipy soft-max, the logistic
+# special case, and what the mathematics fixes.
+def _softmax_problem(K, n=4000, F=6, seed=11):
+    rng = np.random.default_rng(seed)
+    X = rng.normal(size=(n, F)).astype(np.float32)
+    W = rng.normal(size=(F, K))
+    labels = np.argmax(X @ W + rng.gumbel(size=(n, K)), axis=1).astype(np.uint8)
+    return X, labels
+
+
+def _softmax_cfg(K, objective=4, eta=0.5):
+    return {"objective": objective, "method": 1, "internals": {"hist_size": 63, "double_precision": True},
+            "tree": {"max_depth": 3, "eta": eta, "lambda": 1.0, "labels_count": K}}
+
+
+@pytest.mark.parametrize("objective", [3, 4])
+@pytest.mark.parametrize("K", [2, 3, 10])
+def test_softmax_gradients_against_an_independent_softmax(oracle, objective, K):
+    from scipy.special import softmax
+    X, labels = _softmax_problem(K)
+    b = oracle.Booster(X, labels=labels, config=_softmax_cfg(K, objective))
+    n = X.shape[0]
+    for rnd in range(3):
+        raw = b.yhat().astype(np.float64).reshape(K, n)     # class-major scores before the round
+        b.grow(1)
+        g, h = (a.astype(np.float64).reshape(K, n) for a in b.grad())
+        p = softmax(raw, axis=0)
+        onehot = (np.arange(K)[:, None] == labels[None, :]).astype(np.float64)
+        assert np.allclose(g, onehot - p, rtol=1e-6, atol=2e-7), "round %d" % rnd
+        assert np.allclose(h, 2.0 * p * (1.0 - p), rtol=1e-6, atol=2e-7), "round %d" % rnd
+        # what the mathematics fixes whatever the scores are
+        assert np.all(np.abs(g.sum(axis=0)) < 1e-6 * K)      # probabilities sum to one
+        assert h.min() >= 0.0 and h.max() <= 0.5             # 2 p (1 - p) on [0, 1]
+        lab_g = g[labels, np.arange(n)]
+        assert lab_g.min() >= 0.0                            # the label's own class is pushed up
+        assert (g.sum(axis=0) - lab_g).max() <= 0.0          # every other class down
+    # after the first round the scores differ between classes and rows
+    assert np.ptp(raw, axis=0).max() > 0.1
+
+
+def test_softmax_two_classes_is_the_logistic_sigmoid(oracle):
+    # K = 2: p_1 = sigmoid(s_1 - s_0); g_1 = y - p_1 and h = 2 p_1 (1 - p_1), i.e. twice the
+    # hessian of the (separately pinned) logistic objective on the score difference.
+    X, labels = _softmax_problem(2, seed=3)
+    b = oracle.Booster(X, labels=labels, config=_softmax_cfg(2))
+    n = X.shape[0]
+    b.grow(2)
+    raw = b.yhat().reshape(2, n)
+    b.grow(1)
+    g, h = (a.reshape(2, n) for a in b.grad())
+    d = (raw[1].astype(np.float64) - raw[0].astype(np.float64))
+    s = np.array([oracle.lib().orc_sigmoid(float(v)) for v in d.astype(np.float32)], np.float64)
+    assert np.allclose(g[1], labels - s, atol=3e-7)
+    assert np.allclose(g[0], -(labels - s), atol=3e-7)
+    assert np.allclose(h[1], 2 * s * (1 - s), atol=3e-7)
+    assert np.allclose(h[0], h[1], atol=3e-7)
+
+
+def test_softmax_link_against_scipy(oracle):
+    from scipy.special import softmax
+    K = 5
+    X, labels = _softmax_problem(K, seed=7)
+    b = oracle.Booster(X, labels=labels, config=_softmax_cfg(K))
+    n = X.shape[0]
+    b.grow(4)
+    # rows without a value exactly on a threshold: prediction walks the raw floats to the same
+    # leaves as training walked the bins, so the tracked scores are the raw scores of predict()
+    raw = b.yhat().astype(np.float64).reshape(K, n).T        # row-major (n, K)
+    out = b.predict(X)
+    assert out.shape == (n, K)                               # objective.h:93-95: row-major out
+    assert np.allclose(out.sum(axis=1), 1.0, atol=1e-6)
+    assert np.allclose(out, softmax(raw, axis=1), rtol=1e-6, atol=1e-7)
+    # n_rounds counts TREES (garden.cu:643-657): K trees = one round
+    b1 = oracle.Booster(X, labels=labels, config=_softmax_cfg(K))
+    b1.grow(1)
+    assert np.array_equal(b.predict(X, n_rounds=K), b1.predict(X))
+    # training moves probability mass towards the labels
+    p0 = np.full(n, 1.0 / K)
+    assert out[np.arange(n), labels].mean() > p0.mean() + 0.05
+
+
+def test_softmax_gradient_is_the_derivative_of_the_log_likelihood(oracle):
+    # g_k = d/ds_k log p_label by central differences on the checker's own link: ties the
+    # gradient formula to the link function instead of to a second soft-max routine.
+    from scipy.special import log_softmax
+    K = 4
+    X, labels = _softmax_problem(K, n=500, seed=5)
+    b = oracle.Booster(X, labels=labels, config=_softmax_cfg(K))
+    n = X.shape[0]
+    b.grow(2)
+    raw = b.yhat().astype(np.float64).reshape(K, n)
+    b.grow(1)
+    g = b.grad()[0].astype(np.float64).reshape(K, n)
+    eps = 1e-5
+    for k in range(K):
+        up, dn = raw.copy(), raw.copy()
+        up[k] += eps
+        dn[k] -= eps
+        num = (log_softmax(up, axis=0)[labels, np.arange(n)] - log_softmax(dn, axis=0)[labels, np.arange(n)]) / (2 * eps)
+        assert np.allclose(g[k], num, atol=1e-6)
