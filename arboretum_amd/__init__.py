@@ -1,6 +1,6 @@
 """MI355X-native histogram tree growing behind arboretum's C-ABI and Python API."""
 from .core import (ArboretumClassifier, ArboretumError, ArboretumRegression, DMatrix, Garden,
-                   copy_probe, device_count, load, train)
+                   copy_probe, device_count, hist_sum, load, train)
 
 __all__ = ["DMatrix", "Garden", "train", "load", "ArboretumRegression", "ArboretumClassifier",
-           "ArboretumError", "device_count"]
+           "ArboretumError", "device_count", "hist_sum"]

@@ -2,15 +2,18 @@
 import os
 import subprocess
 import sys
+from concurrent.futures import ThreadPoolExecutor
 
 HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(HERE, "csrc")
+OBJ = os.path.join(HERE, "build")
 LIB = os.path.join(HERE, "libarboretum.so")
-SOURCES = ["device_builder.hip", "quantiser.hip", "predictor.hip", "booster.cpp", "config.cpp", "wrapper.cpp"]
+SOURCES = ["device_builder.hip", "hist_sum.hip", "quantiser.hip", "predictor.hip", "booster.cpp", "config.cpp",
+           "wrapper.cpp"]
 # -ffp-contract=off: the gain arithmetic must round exactly like the host
 # restatement (no fused multiply-add).  packed-fp32-ops is switched off
 # because some packed forms have produced wrong results on this hardware.
-FLAGS = ["--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-shared", "-ffp-contract=off",
+FLAGS = ["--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-ffp-contract=off",
          "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops", "-Wall", "-Wno-unused-function",
          "-Wno-unknown-warning-option", "-pthread"]
 
@@ -22,8 +25,7 @@ def hipcc():
     raise RuntimeError("hipcc not found")
 
 
-def build(verbose=False):
-    cmd = [hipcc()] + FLAGS + os.environ.get("ARB_EXTRA_FLAGS", "").split() + ["-x", "hip"] + [os.path.join(CSRC, s) for s in SOURCES] + ["-o", LIB]
+def _run(cmd, verbose):
     if verbose:
         print(" ".join(cmd))
     res = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
@@ -32,8 +34,24 @@ def build(verbose=False):
         raise RuntimeError("hipcc failed building libarboretum.so")
     if verbose and res.stdout:
         print(res.stdout)
+
+
+def build(verbose=False, only=None):
+    """Compiles every source to an object file (in parallel) and links them.
+    only: names of the sources to recompile (the other objects must exist)."""
+    os.makedirs(OBJ, exist_ok=True)
+    extra = os.environ.get("ARB_EXTRA_FLAGS", "").split()
+    objs = [os.path.join(OBJ, os.path.splitext(s)[0] + ".o") for s in SOURCES]
+    jobs = []
+    for s, o in zip(SOURCES, objs):
+        if only is not None and s not in only and os.path.exists(o):
+            continue
+        jobs.append([hipcc()] + FLAGS + extra + ["-x", "hip", "-c", os.path.join(CSRC, s), "-o", o])
+    with ThreadPoolExecutor(max_workers=min(8, max(1, len(jobs)))) as ex:
+        list(ex.map(lambda c: _run(c, verbose), jobs))
+    _run([hipcc(), "--offload-arch=gfx950", "-shared", "-fPIC", "-pthread"] + objs + ["-o", LIB], verbose)
     return LIB
 
 
 if __name__ == "__main__":
-    build(verbose=True)
+    build(verbose=True, only=sys.argv[1:] or None)

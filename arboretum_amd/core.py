@@ -61,6 +61,8 @@ def _load_lib():
         "AGardenGetTimings": [c_void_p, c_void_p],
         "AGardenRowsScanned": [c_void_p, P(ctypes.c_ulonglong)],
         "AGardenSynchronize": [c_void_p],
+        "AHistSum": [c_void_p] * 10 + [ctypes.c_ulonglong, ctypes.c_longlong, c_int, c_int, c_int, c_int, c_int,
+                                       c_void_p],
     }
     for name, args in sigs.items():
         fn = getattr(lib, name)
@@ -86,6 +88,16 @@ def device_count():
 def copy_probe(nbytes):
     """One device-to-device copy kernel of known size (profile calibration)."""
     _check(_LIB.ADeviceCopyProbe(int(nbytes)))
+
+
+def hist_sum(sum_g, sum_h, bin_count, grad, hess, node_size, bins, stride, nrow, ncol, nodes, shift_g,
+             shift_h=0, use_trick=False, parent_g=None, parent_h=None, parent_c=None, stream=None):
+    """Histogram sums of node segments for data that lives on the GPU (AHistSum; the
+    reference's HistTreeGrower::HistSum over every feature at once).  Every array argument
+    is a DEVICE address (an int, e.g. `tensor.data_ptr()`), or None."""
+    _check(_LIB.AHistSum(sum_g, sum_h, bin_count, parent_g, parent_h, parent_c, grad, hess, node_size, bins,
+                         int(stride), int(nrow), int(ncol), int(nodes), int(bool(use_trick)), int(shift_g),
+                         int(shift_h), stream))
 
 
 def _fptr(a):

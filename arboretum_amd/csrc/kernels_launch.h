@@ -1,0 +1,50 @@
+// Host-side launch helpers shared by the translation units that run the
+// stand-alone histogram kernel.
+#ifndef ARBORETUM_AMD_KERNELS_LAUNCH_H_
+#define ARBORETUM_AMD_KERNELS_LAUNCH_H_
+#include <stdexcept>
+
+#include "device_common.h"
+#include "kernels_hist.h"
+
+namespace arb {
+namespace {
+
+// Raises the dynamic LDS limit of a kernel once (needed above 64 KB).
+template <typename K>
+void AllowLds(K kernel, size_t bytes) {
+  static size_t allowed = 0;  // one instance per kernel type/pointer value below
+  (void)allowed;
+  HIP_OK(hipFuncSetAttribute((const void *)kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)bytes));
+}
+
+template <bool PAIR, int NQ>
+void LaunchHistNQ(hipStream_t st, unsigned grid, const uint32_t *bins, size_t stride, int q0, int F,
+                  const float *g, const float *h, const int *shifts, const WorkItem *work,
+                  const unsigned *n_work, unsigned long long *slab, int slab_entries) {
+  const size_t lds = HistLdsBytes(NQ, PAIR);
+  static bool configured = false;
+  if (!configured) {
+    AllowLds(k_hist<PAIR, NQ>, lds);
+    configured = true;
+  }
+  hipLaunchKernelGGL((k_hist<PAIR, NQ>), dim3(grid), dim3(kHistThreads), lds, st, bins, stride, q0, F, g, h,
+                     shifts, work, n_work, slab, slab_entries);
+}
+
+template <bool PAIR>
+void LaunchHist(int nq, hipStream_t st, unsigned grid, const uint32_t *bins, size_t stride, int q0, int F,
+                const float *g, const float *h, const int *shifts, const WorkItem *work,
+                const unsigned *n_work, unsigned long long *slab, int slab_entries) {
+#define ARB_CASE(N) \
+  case N: LaunchHistNQ<PAIR, N>(st, grid, bins, stride, q0, F, g, h, shifts, work, n_work, slab, slab_entries); break;
+  switch (nq) {
+    ARB_CASE(1) ARB_CASE(2) ARB_CASE(3) ARB_CASE(4) ARB_CASE(5) ARB_CASE(6) ARB_CASE(7) ARB_CASE(8)
+    default: throw std::runtime_error("internal: bad quad count");
+  }
+#undef ARB_CASE
+}
+
+}  // namespace
+}  // namespace arb
+#endif  // ARBORETUM_AMD_KERNELS_LAUNCH_H_

@@ -618,19 +618,21 @@ k_hist_reduce(const unsigned long long *__restrict__ slab, int slab_entries, int
     }
     const size_t cell = plain ? (size_t)entry : (size_t)f * kSlots + bin;
     const size_t o = (size_t)nd * nbin_total + cell;
+    // without hessians (count as hessian) the caller may pass no hh / ph arrays
+    const bool with_h = PAIR || hh != nullptr;
     if (accumulate) {  // streamed matrices: one call per row block
       ag += hg[o];
-      ah += hh[o];
+      if (with_h) ah += hh[o];
       ac += hc[o];
     }
     hg[o] = ag;
-    hh[o] = ah;
+    if (with_h) hh[o] = ah;
     hc[o] = ac;
     if (trick) {
       const size_t po = (size_t)(nd >> 1) * nbin_total + cell;
       const size_t so = (size_t)(nd ^ 1) * nbin_total + cell;
       hg[so] = pg[po] - ag;
-      hh[so] = ph[po] - ah;
+      if (with_h) hh[so] = ph[po] - ah;
       hc[so] = pc[po] - ac;
     }
   }

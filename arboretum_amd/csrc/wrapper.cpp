@@ -11,6 +11,7 @@
 
 #include "../../include/arboretum_ext.h"
 #include "booster.h"
+#include "hist_sum.h"
 
 using namespace arb;
 
@@ -329,6 +330,18 @@ const char *AGardenRowsScanned(VoidPointer garden, unsigned long long *out) {
 }
 const char *AGardenSynchronize(VoidPointer garden) {
   return Guard([&] { BuilderOf(garden)->Synchronize(); });
+}
+
+const char *AHistSum(long long *sum_g, long long *sum_h, unsigned *bin_count, const long long *parent_g,
+                     const long long *parent_h, const unsigned *parent_c, const float *grad, const float *hess,
+                     const unsigned *node_size, const unsigned *bins, unsigned long long stride, long long nrow,
+                     int ncol, int nodes, int use_trick, int shift_g, int shift_h, void *stream) {
+  return Guard([&] {
+    if (DeviceCount() <= 0) throw std::runtime_error("no HIP device available");
+    HistSumArgs a{bins, stride, ncol, nrow, grad, hess, node_size, nodes, use_trick, parent_g, parent_h, parent_c,
+                  shift_g, shift_h, sum_g, sum_h, bin_count, stream};
+    HistSum(a);
+  });
 }
 
 }  // extern "C"

@@ -90,6 +90,35 @@ const char *AGardenRowsScanned(VoidPointer garden, unsigned long long *out);
 /* Waits for all device work of the booster. */
 const char *AGardenSynchronize(VoidPointer garden);
 
+/* Histogram sums of node segments on the device, for data that already lives
+ * there: the counterpart of HistTreeGrower::HistSum
+ * (src/core/hist_tree_grower.h:17-23, hist_tree_grower.cu:200-301; called
+ * directly by tests/cpp/test_hist_sum.cu), which takes one feature column per
+ * call; this one takes every feature of a quad-packed matrix.  EVERY POINTER
+ * IS A DEVICE POINTER.  Argument order follows the reference: outputs,
+ * parents, gradients, node offsets, bins, sizes, trick.
+ *   bins       [Q][stride] 32-bit words, Q = ceil(ncol / 4); byte k of word q
+ *              of a row is the 8-bit bin id of feature 4 q + k; rows in node
+ *              order (stride >= nrow, in words)
+ *   grad/hess  [nrow] floats; hess NULL: the row count is the hessian
+ *              (squared error) and sum_h / parent_h may be NULL
+ *   node_size  nodes + 1 non-decreasing row offsets (the reference's
+ *              node_size): node k owns rows [node_size[k], node_size[k + 1])
+ *   use_trick  nodes are sibling pairs (2 k, 2 k + 1): only the smaller one
+ *              (ties -> left, hist_grad_sum.cu:279-294) is accumulated, the
+ *              other is parent[k] - it
+ *   shift_g/h  sums are exact integers: every value is rounded once to
+ *              rint(v * 2^shift) (|v * 2^shift| <= 2^30 required) and the
+ *              integers are added, so the result does not depend on the order
+ *   sum_g, sum_h, bin_count
+ *              [nodes][4 Q][256]: cell (node, feature, bin)
+ * Allocates its work memory with hipMalloc, runs on `stream` (a hipStream_t,
+ * NULL = default stream) and waits for the result. */
+const char *AHistSum(long long *sum_g, long long *sum_h, unsigned *bin_count, const long long *parent_g,
+                     const long long *parent_h, const unsigned *parent_c, const float *grad, const float *hess,
+                     const unsigned *node_size, const unsigned *bins, unsigned long long stride, long long nrow,
+                     int ncol, int nodes, int use_trick, int shift_g, int shift_h, void *stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -125,15 +125,58 @@ def main():
                    "gain": 565504.0, "sums": [1861, 1625, 1405, 1201, 1013, 841, 685, 545]}]})
     json.dump(g, open(os.path.join(HERE, "gain.json"), "w"))
 
-    # ---- histogram goldens, tests/cpp/test_hist_sum.cu:425-599 (asymmetric, both orientations)
-    h = [{"name": "Asymmetric10", "cite": "tests/cpp/test_hist_sum.cu:425-536", "hist_size": 4,
-          "rows": 1280, "split_at": 10,
-          "count": [3, 3, 2, 2, 317, 317, 318, 318],
-          "sum": [12.0, 15.0, 8.0, 10.0, 204148.0, 204465.0, 204792.0, 205110.0]},
-         {"name": "Asymmetric1270", "cite": "tests/cpp/test_hist_sum.cu:538-599", "hist_size": 4,
-          "rows": 1280, "split_at": 1270,
-          "count": [318, 318, 317, 317, 2, 2, 3, 3],
-          "sum": [201612.0, 201930.0, 200978.0, 201295.0, 2548.0, 2550.0, 3822.0, 3825.0]}]
+    # ---- histogram goldens: all 17 cases of tests/cpp/test_hist_sum.cu.  Every case has
+    # grad[i] = float(i); "bins" names the rule of the test ("i", "0", "i%H"); "count" / "sum"
+    # map the flat cell index node * H + bin to the value the test asserts, "node_sum" holds
+    # the asserted totals over a node's cells.  The (BIN_T, SUM_T) variants of a test share
+    # one set of numbers and differ in "bin_type" / "sum_type".
+    h = []
+    blk = 128  # HIST_SUM_BLOCK_DIM, src/core/hist_grad_sum.cuh:6
+    variants = [("Float", "Bin16", 11, 71, 133), ("Float", "Bin8", 41, 102, 165),
+                ("Double", "Bin16", 197, 257, 319), ("Double", "Bin8", 227, 288, 351)]
+    for st, bt, l_naive, l_seg, l_full in variants:
+        base = {"sum_type": st.lower(), "bin_type": bt.lower(), "trick": False, "parent_count": None,
+                "parent_sum": None, "node_sum": None}
+        h.append(dict(base, name="SingleNodeHistSum%s%s.Naive" % (st, bt),
+                      cite="tests/cpp/test_hist_sum.cu:%d-%d" % (l_naive, l_naive + 28), rows=32, bins="i",
+                      hist_size=32, node_size=[0, 32], count={str(i): 1 for i in range(32)},
+                      sum={str(i): float(i) for i in range(32)}))
+        h.append(dict(base, name="SingleNodeHistSum%s%s.SingleSegment" % (st, bt),
+                      cite="tests/cpp/test_hist_sum.cu:%d-%d" % (l_seg, l_seg + 29), rows=32, bins="0",
+                      hist_size=32, node_size=[0, 32], count={"0": 32}, sum={"0": float(32 * 31 // 2)}))
+        n = blk * 10
+        h.append(dict(base, name="SingleNodeHistSum%s%s.SingleSegmentFullSize" % (st, bt),
+                      cite="tests/cpp/test_hist_sum.cu:%d-%d" % (l_full, l_full + 30), rows=n, bins="0",
+                      hist_size=256, node_size=[0, n], count={"0": n}, sum={"0": float(n * (n - 1) // 2)}))
+    n = blk * 10
+    multi = {"sum_type": "double", "bin_type": "bin16", "rows": n, "hist_size": 4}
+    h.append(dict(multi, name="MultiNodeHistSumDouble._2_NodesNoTrick", cite="tests/cpp/test_hist_sum.cu:383-424",
+                  bins="i%H", node_size=[0, n // 2, n], trick=False, parent_count=None, parent_sum=None,
+                  count={str(i): n // 8 for i in range(8)}, sum={},
+                  node_sum=[float((n // 2) * (n // 2 - 1) // 2), float((n // 2) * (n // 2 + n - 1) // 2)]))
+    asym_c = {str(i): v for i, v in enumerate([3, 3, 2, 2, 317, 317, 318, 318])}
+    asym_s = {str(i): v for i, v in enumerate([12.0, 15.0, 8.0, 10.0, 204148.0, 204465.0, 204792.0, 205110.0])}
+    par_c = [320, 320, 320, 320]
+    par_s = [204148.0 + 12.0, 204465.0 + 15.0, 204792.0 + 8.0, 205110.0 + 10.0]
+    h.append(dict(multi, name="MultiNodeHistSumDouble._2_NodesAsymmetricNoTrick",
+                  cite="tests/cpp/test_hist_sum.cu:426-477", bins="i%H", node_size=[0, 10, n], trick=False,
+                  parent_count=None, parent_sum=None, count=asym_c, sum=asym_s,
+                  node_sum=None, total_sum=float(n * (n - 1) // 2)))
+    h.append(dict(multi, name="MultiNodeHistSumDouble._2_NodesAsymmetricWithTrick",
+                  cite="tests/cpp/test_hist_sum.cu:479-538", bins="i%H", node_size=[0, 10, n], trick=True,
+                  parent_count=par_c, parent_sum=par_s, count=asym_c, sum=asym_s, node_sum=None))
+    h.append(dict(multi, name="MultiNodeHistSumDouble._2_NodesAsymmetricWithTrick2",
+                  cite="tests/cpp/test_hist_sum.cu:540-599", bins="i%H", node_size=[0, n - 10, n], trick=True,
+                  parent_count=par_c, parent_sum=par_s,
+                  count={str(i): v for i, v in enumerate([318, 318, 317, 317, 2, 2, 3, 3])},
+                  sum={str(i): v for i, v in enumerate([201612.0, 201930.0, 200978.0, 201295.0, 2548.0, 2550.0,
+                                                        3822.0, 3825.0])}, node_sum=None))
+    h.append(dict(multi, name="MultiNodeHistSumDouble.SingleSegmentWithTrick",
+                  cite="tests/cpp/test_hist_sum.cu:601-649", bins="0", node_size=[0, n // 2, n], trick=True,
+                  parent_count=[n, 0, 0, 0], parent_sum=[float(n * (n - 1) // 2), 0.0, 0.0, 0.0],
+                  count={"0": n // 2, "4": n // 2},
+                  sum={"0": float((n // 2) * (n // 2 - 1) // 2), "4": float((n // 2) * (n // 2 + n - 1) // 2)},
+                  node_sum=None))
     json.dump(h, open(os.path.join(HERE, "hist_sum.json"), "w"))
     print("fixtures written to", HERE)
 

@@ -6,7 +6,7 @@ import math
 import numpy as np
 import pytest
 
-from conftest import concrete_config, load_golden
+from conftest import check_hist_sum, concrete_config, hist_sum_inputs, load_golden
 
 
 # ---------------------------------------------------------------- quantiser
@@ -117,20 +117,28 @@ def test_gain_guards(oracle):
 # ---------------------------------------------------------------- histograms
 @pytest.mark.parametrize("case", load_golden("hist_sum.json"), ids=lambda c: c["name"])
 def test_hist_sum_golden(oracle, case):
-    n, B = case["rows"], case["hist_size"]
-    g = np.arange(n, dtype=np.float32)
-    bins = (np.arange(n) % B).astype(np.uint8).reshape(n, 1)
+    bins, g, offs = hist_sum_inputs(case)
+    n, H = case["rows"], case["hist_size"]
     shift = oracle.lib().orc_fix_shift(float(g.max()))
-    first = np.arange(n) < case["split_at"]
-    h0 = oracle.hist_fixed_u8(bins, g, None, shift, 0, sel=first)
-    h1 = oracle.hist_fixed_u8(bins, g, None, shift, 0, sel=~first)
-    par = oracle.hist_fixed_u8(bins, g, None, shift, 0)
-    # sibling subtraction is exact on the integers
-    assert np.array_equal(par - h0, h1)
-    got_c = np.concatenate([h0[0, :B, 2], h1[0, :B, 2]])
-    got_s = np.concatenate([h0[0, :B, 0], h1[0, :B, 0]]) * 2.0 ** -shift
-    assert got_c.tolist() == case["count"]
-    assert got_s.tolist() == case["sum"]
+    rows = np.arange(n)
+    nodes = len(offs) - 1
+    hists = [oracle.hist_fixed_u8(bins, g, None, shift, 0, sel=(rows >= offs[k]) & (rows < offs[k + 1]))[0]
+             for k in range(nodes)]
+    if case["trick"]:
+        # only the smaller sibling is accumulated (ties -> left, hist_grad_sum.cu:279-294); the
+        # other one is the parent the test passes in minus it
+        for k in range(0, nodes, 2):
+            par = np.zeros_like(hists[k])
+            par[:H, 0] = np.array(case["parent_sum"]) * 2.0 ** shift
+            par[:H, 2] = case["parent_count"]
+            left_built = offs[k + 1] - offs[k] <= offs[k + 2] - offs[k + 1]
+            derived = par - hists[k if left_built else k + 1]
+            # sibling subtraction is exact on the integers
+            assert np.array_equal(derived, hists[k + 1 if left_built else k])
+            hists[k + 1 if left_built else k] = derived
+    count = [h[:, 2] for h in hists]
+    total = [h[:, 0] * 2.0 ** -shift for h in hists]
+    check_hist_sum(case, count, total)
 
 
 def test_fixed_point_scale(oracle):
