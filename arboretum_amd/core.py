@@ -63,6 +63,8 @@ def _load_lib():
         "AGardenSynchronize": [c_void_p],
         "AHistSum": [c_void_p] * 10 + [ctypes.c_ulonglong, ctypes.c_longlong, c_int, c_int, c_int, c_int, c_int,
                                        c_void_p],
+        "AHistSumNoAlloc": [c_void_p] * 10 + [ctypes.c_ulonglong, ctypes.c_longlong, c_int, c_int, c_int, c_int,
+                                              c_int, c_void_p, c_void_p],
     }
     for name, args in sigs.items():
         fn = getattr(lib, name)
@@ -98,6 +100,16 @@ def hist_sum(sum_g, sum_h, bin_count, grad, hess, node_size, bins, stride, nrow,
     _check(_LIB.AHistSum(sum_g, sum_h, bin_count, parent_g, parent_h, parent_c, grad, hess, node_size, bins,
                          int(stride), int(nrow), int(ncol), int(nodes), int(bool(use_trick)), int(shift_g),
                          int(shift_h), stream))
+
+
+def hist_sum_no_alloc(sum_g, sum_h, bin_count, grad, hess, node_size, bins, stride, nrow, ncol, nodes, shift_g,
+                      shift_h=0, use_trick=False, parent_g=None, parent_h=None, parent_c=None, stream=None,
+                      status=None):
+    """hist_sum without any device allocation (AHistSumNoAlloc): static work memory, limited
+    sizes, enqueues on `stream` and returns without waiting; `status` is an optional device word."""
+    _check(_LIB.AHistSumNoAlloc(sum_g, sum_h, bin_count, parent_g, parent_h, parent_c, grad, hess, node_size,
+                                bins, int(stride), int(nrow), int(ncol), int(nodes), int(bool(use_trick)),
+                                int(shift_g), int(shift_h), stream, status))
 
 
 def _fptr(a):

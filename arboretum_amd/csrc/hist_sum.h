@@ -31,5 +31,11 @@ struct HistSumArgs {
 // Allocates its work memory (plan, per-work-item slabs), runs and waits.
 void HistSum(const HistSumArgs &args);
 
+// The same without any allocation: plan and slabs live in a static device
+// array of 32 MB + 192 KB per GPU; enqueues on args.stream and returns without
+// waiting.  status (device, may be null): 0, 1 = bad node offsets, 2 = internal.
+// Throws for sizes the array cannot hold.
+void HistSumNoAlloc(const HistSumArgs &args, unsigned *status);
+
 }  // namespace arb
 #endif  // ARBORETUM_AMD_HIST_SUM_H_

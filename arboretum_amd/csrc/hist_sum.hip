@@ -146,11 +146,12 @@ void Validate(const HistSumArgs &a) {
 }
 
 // Enqueues the kernels of one call on `st`.  `mem` holds HistSumHeadBytes(...)
-// + max_items * slab bytes.
+// + max_items * slab bytes, or the slabs start at slab_base.
 void Enqueue(const HistSumArgs &a, const Shape &sh, unsigned char *mem, unsigned max_items, unsigned per_item,
-             unsigned *status, hipStream_t st) {
+             unsigned *status, hipStream_t st, unsigned char *slab_base = nullptr) {
   const bool pair = a.hess != nullptr;
-  const HistSumScratch s = Carve(mem, a.nodes, max_items);
+  HistSumScratch s = Carve(mem, a.nodes, max_items);
+  if (slab_base) s.slab = reinterpret_cast<unsigned long long *>(slab_base);
   hipLaunchKernelGGL(k_hist_sum_setup, dim3(1), dim3(1024), 0, st, a.node_size, a.nodes, (unsigned)a.nrow, a.shift_g,
                      a.shift_h, s.tot, s.seg, s.n_work, s.overflow, s.shifts, status);
   hipLaunchKernelGGL(k_plan, dim3(1), dim3(1024), 0, st, s.tot, s.seg, a.nodes, a.use_trick ? 1 : 0, per_item, s.work,
@@ -181,7 +182,58 @@ void Enqueue(const HistSumArgs &a, const Shape &sh, unsigned char *mem, unsigned
   HIP_OK(hipGetLastError());
 }
 
+// ---- work memory of the entry point that allocates nothing -----------------
+// One array per GPU (each device that loads this library holds its own copy
+// until the process ends): the plan and counters of a call, then the slabs.
+// Its name is only a handle on the host; the address on the current device
+// comes from hipGetSymbolAddress, once per device.
+constexpr size_t kStaticSlabBytes = (size_t)32 << 20;
+constexpr unsigned kStaticMaxItems = 1024;
+constexpr size_t kStaticHeadBytes = (size_t)192 << 10;  // >= HistSumHeadBytes(kMaxPlanNodes, kStaticMaxItems)
+constexpr size_t kStaticBytes = kStaticHeadBytes + kStaticSlabBytes;
+static __device__ __align__(256) unsigned char scratch[kStaticBytes];
+
+constexpr int kMaxDevices = 64;
+std::mutex g_scratch_mutex;
+unsigned char *g_scratch_ptr[kMaxDevices] = {};
+
+unsigned char *ScratchOfCurrentDevice() {
+  int dev = 0;
+  HIP_OK(hipGetDevice(&dev));
+  if (dev < 0 || dev >= kMaxDevices) throw std::runtime_error("device index out of range");
+  std::lock_guard<std::mutex> lock(g_scratch_mutex);
+  if (!g_scratch_ptr[dev]) {
+    void *p = nullptr;
+    HIP_OK(hipGetSymbolAddress(&p, HIP_SYMBOL(scratch)));
+    if (!p) throw std::runtime_error("no device address for the static work memory");
+    g_scratch_ptr[dev] = static_cast<unsigned char *>(p);
+  }
+  return g_scratch_ptr[dev];
+}
+
 }  // namespace
+
+void HistSumNoAlloc(const HistSumArgs &a, unsigned *status) {
+  Validate(a);
+  const bool pair = a.hess != nullptr;
+  const Shape sh = ShapeOf(a.ncol, pair);
+  const size_t slab_bytes = sh.slab_words * 8;
+  static_assert(kStaticHeadBytes >= (size_t)kMaxPlanNodes * (sizeof(NodeSum) + 3 * sizeof(unsigned)) + 5 * 256 +
+                                        (size_t)kStaticMaxItems * sizeof(WorkItem) + 256,
+                "head of the static work memory too small");
+  const unsigned max_items = (unsigned)std::min<size_t>(kStaticMaxItems, kStaticSlabBytes / slab_bytes);
+  const unsigned per_item = RowsPerItem((size_t)a.nrow, a.nodes, max_items);
+  if (per_item == 0)
+    throw std::runtime_error(
+        "too large for the static work memory: it holds " + std::to_string(max_items) + " work items of " +
+        std::to_string(slab_bytes >> 10) + " KB for this width, each of at most " + std::to_string(kMaxHistRows) +
+        " rows, and every node takes two of them (use AHistSum)");
+  unsigned char *mem = ScratchOfCurrentDevice();
+  // the caller's status word, or one in the work memory that nobody reads
+  unsigned *st_word = status ? status : reinterpret_cast<unsigned *>(mem + kStaticHeadBytes - 256);
+  Enqueue(a, sh, mem, max_items, per_item, st_word, static_cast<hipStream_t>(a.stream),
+          mem + kStaticHeadBytes);
+}
 
 void HistSum(const HistSumArgs &a) {
   Validate(a);

@@ -344,4 +344,16 @@ const char *AHistSum(long long *sum_g, long long *sum_h, unsigned *bin_count, co
   });
 }
 
+const char *AHistSumNoAlloc(long long *sum_g, long long *sum_h, unsigned *bin_count, const long long *parent_g,
+                            const long long *parent_h, const unsigned *parent_c, const float *grad,
+                            const float *hess, const unsigned *node_size, const unsigned *bins,
+                            unsigned long long stride, long long nrow, int ncol, int nodes, int use_trick,
+                            int shift_g, int shift_h, void *stream, unsigned *status) {
+  return Guard([&] {
+    HistSumArgs a{bins, stride, ncol, nrow, grad, hess, node_size, nodes, use_trick, parent_g, parent_h, parent_c,
+                  shift_g, shift_h, sum_g, sum_h, bin_count, stream};
+    HistSumNoAlloc(a, status);
+  });
+}
+
 }  // extern "C"

@@ -119,6 +119,29 @@ const char *AHistSum(long long *sum_g, long long *sum_h, unsigned *bin_count, co
                      const unsigned *node_size, const unsigned *bins, unsigned long long stride, long long nrow,
                      int ncol, int nodes, int use_trick, int shift_g, int shift_h, void *stream);
 
+/* AHistSum for callers that cannot allocate device memory (code under HIP
+ * graph capture, tight serving loops, harnesses that forbid hipMalloc).  No
+ * counterpart in the reference.  Same arguments and results as AHistSum; the
+ * work plan and the per-work-item histograms live in a static device array of
+ * 32 MB + 192 KB that every GPU running this library holds until the process
+ * ends.  The call makes no hipMalloc / hipFree and no allocating library
+ * call; it enqueues its kernels on `stream` and returns WITHOUT waiting.
+ *   status   device word, may be NULL: written by the kernels, 0 = done,
+ *            1 = node_size is not non-decreasing within [0, nrow] (such nodes
+ *            are skipped), 2 = internal planning error
+ * Limits (an error string is returned beyond them, before anything runs): the
+ * array holds min(1024, 32 MB / slab) work items, slab = 64 KB per 16 features
+ * (128 KB with hessians); a work item covers at most 64512 rows and every node
+ * needs two spare items, so e.g. 28 features with hessians and 64 nodes allow
+ * 8.1 M rows.  All calls on one GPU share the array: calls that overlap in
+ * time on one GPU (two streams, two threads) race; calls on one stream, one
+ * after the other, are safe, and nothing has to be cleared between them. */
+const char *AHistSumNoAlloc(long long *sum_g, long long *sum_h, unsigned *bin_count, const long long *parent_g,
+                            const long long *parent_h, const unsigned *parent_c, const float *grad,
+                            const float *hess, const unsigned *node_size, const unsigned *bins,
+                            unsigned long long stride, long long nrow, int ncol, int nodes, int use_trick,
+                            int shift_g, int shift_h, void *stream, unsigned *status);
+
 #ifdef __cplusplus
 }
 #endif

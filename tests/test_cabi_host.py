@@ -168,3 +168,29 @@ def test_errors(arb):
     g = arb.Garden({"objective": 0, "method": 1})
     with pytest.raises(arb.ArboretumError):
         g.load('{"no_model": 1}')
+
+
+def test_no_alloc_histogram_size_limits_are_checked_before_the_gpu_is_touched():
+    # AHistSumNoAlloc keeps plan and slabs in a static device array (32 MB of slabs, at most
+    # 1024 work items of at most 64512 rows, two spare items per node): what cannot fit is
+    # refused on the host.  The addresses below are never dereferenced by host code.
+    import arboretum_amd as arb
+    p = 4096
+
+    def refused(stride, nrow, ncol, nodes):
+        try:
+            arb.hist_sum_no_alloc(p, p, p, p, p, p, p, stride, nrow, ncol, nodes, 30, 32)
+        except arb.ArboretumError as e:
+            return "too large for the static work memory" in str(e)
+        return False
+    assert refused(20000000, 20000000, 28, 1)            # 256 items x 64512 rows < 20 M rows
+    assert refused(64512 * 200, 64512 * 200, 28, 64)     # 128 of the 256 items go to the 64 nodes
+    assert refused(1024, 1000, 600, 6)                   # 2.4 MB per slab: 13 items < 2 * 6 + 2
+    assert refused(1 << 20, 1 << 20, 2100, 1)            # 8.4 MB per slab: 3 items
+    # sizes that fit pass the size check (and then fail here only for want of a GPU)
+    if arb.device_count() == 0:
+        with pytest.raises(arb.ArboretumError, match="HIP error"):
+            arb.hist_sum_no_alloc(p, p, p, p, p, p, p, 8000000, 8000000, 28, 64, 30, 32)
+    with pytest.raises(arb.ArboretumError, match="sibling pairs"):
+        arb.hist_sum_no_alloc(p, p, p, p, p, p, p, 1024, 1000, 28, 3, 30, 32, use_trick=True, parent_g=p,
+                              parent_h=p, parent_c=p)
