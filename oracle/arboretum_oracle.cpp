@@ -812,8 +812,10 @@ void *orc_create(const float *X, int64_t n, int F, const float *y, const uint8_t
   b->thr.resize(F);
   b->size.resize(F);
   b->bins.resize((size_t)n * F);
-  std::vector<float> col(n);
+  // the columns are independent (io.cu:349-435 handles them one after the other)
+#pragma omp parallel for schedule(dynamic, 1) num_threads(p->threads > 0 ? p->threads : omp_get_max_threads())
   for (int f = 0; f < F; ++f) {
+    std::vector<float> col(n);
     for (int64_t i = 0; i < n; ++i) col[i] = X[(size_t)i * F + f];
     QuantResult q = quantize_thresholds(col.data(), n, p->hist_size);
     b->thr[f] = q.thr;

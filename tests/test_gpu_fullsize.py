@@ -1,7 +1,7 @@
-"""Size-independent properties at the headline size (10.5 M rows x 28 features,
-256 bins, max_depth 8, logistic): the oracle is too slow here, so the HIP path
-is checked against itself along independent code paths and against invariants
-of the algorithm."""
+"""The headline size (10.5 M rows x 28 features, 256 bins, max_depth 8, logistic): the HIP path
+against the CPU checker bit for bit (three trees: splits, gains, leaf weights, every row's leaf,
+y_hat, the first tree's histograms at every level), against itself along independent code paths
+and against invariants of the algorithm."""
 import os
 import sys
 
@@ -115,3 +115,27 @@ def test_streamed_bins_same_trees(arb, workload, fused):
 
 def test_second_run_is_bit_identical(arb, workload, fused):
     _same_trees(fused, _grow(arb, workload, _config()))
+
+
+def test_headline_config_bit_exact_against_the_checker(arb, workload, fused, oracle):
+    # BASELINE configs[1] at its full size: same seeded input on both sides
+    X, y = workload
+    ob = oracle.Booster(X, y=y, config=_config(), threads=16)
+    ob.grow(1)
+    for level in range(8):      # the first tree's integer histograms, every node of every level
+        ho = ob.level_hist(level)
+        hg = fused["hists"][level]
+        assert np.array_equal(hg, ho[:, :, :hg.shape[2], :]), "histograms of level %d" % level
+        assert not ho[:, :, hg.shape[2]:, :].any()
+    ob.grow(ROUNDS - 1)
+    for r in range(ROUNDS):
+        to, tg = ob.tree(r), fused["trees"][r]
+        for key in ("fid", "quantized", "threshold", "gain"):
+            assert np.array_equal(to[key], tg[key]), "%s of tree %d" % (key, r)
+        assert np.array_equal(to["weights"], tg["weights"], equal_nan=True), "leaf weights of tree %d" % r
+        assert (tg["quantized"] >= 0).sum() > 200, "tree %d is not a full depth-8 tree" % r
+    assert np.array_equal(ob.leaf(), fused["leaves"]), "row -> leaf of the last tree"
+    assert np.array_equal(ob.yhat(), fused["yhat"]), "y_hat after %d trees" % ROUNDS
+    po = ob.predict(X)
+    pg = fused["garden"].predict(fused["data"])
+    assert np.abs(po - pg).max() < 1e-4
