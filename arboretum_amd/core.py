@@ -52,6 +52,7 @@ def _load_lib():
         "AGardenPredictOnDevice": [c_void_p, c_int],
         "AGardenNumTrees": [c_void_p, P(c_int)],
         "AGardenGetTree": [c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p],
+        "AGardenGetTreeDepth": [c_void_p, c_int, P(c_int)],
         "AGardenGetLeaves": [c_void_p, c_void_p],
         "AGardenGetTrainYHat": [c_void_p, c_void_p],
         "AGardenGetGrad": [c_void_p, c_void_p, c_void_p],
@@ -300,7 +301,10 @@ class Garden(object):
         return n.value
 
     def tree(self, t):
-        depth = self.config.get('tree', {}).get('max_depth', 7) + 1
+        # a loaded model's trees carry their own depth, which need not be the configuration's
+        d = ctypes.c_int(0)
+        _check(_LIB.AGardenGetTreeDepth(self.handle, t, ctypes.byref(d)))
+        depth = d.value
         ni, nl = (1 << (depth - 1)) - 1, 1 << (depth - 1)
         fid, q = np.empty(ni, np.int32), np.empty(ni, np.int32)
         thr, gain, w = np.empty(ni, np.float32), np.empty(ni, np.float32), np.empty(nl, np.float32)

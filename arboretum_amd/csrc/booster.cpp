@@ -152,6 +152,18 @@ void Garden::GrowTree(DataMatrix *data, const float *grad) {
     throw std::runtime_error("colsample_bytree is too small");
   if ((int)(cfg.tree.colsample_bytree * cfg.tree.colsample_bylevel * columns) == 0)
     throw std::runtime_error("colsample_bytree and colsample_bylevel are too small");
+  if (!builder_ && cfg.objective < kSoftMaxOneVsAll) {
+    // Gradients are accumulated in fixed point scaled by the largest one; a
+    // target that is NaN or infinite has no scale (the reference would carry
+    // the NaN into every sum it touches).
+    std::atomic<bool> bad{false};
+    ParallelFor(data->rows, [&](size_t b, size_t e) {
+      bool any = false;
+      for (size_t i = b; i < e; ++i) any = any || !std::isfinite(data->y[i]);
+      if (any) bad = true;
+    });
+    if (bad) throw std::runtime_error("y must be finite");
+  }
   if (DeviceCount() <= 0) throw std::runtime_error("no HIP device available: training needs an MI355X");
   if (!builder_) {
     // upload_features = false keeps the bins in pinned host memory and streams

@@ -496,7 +496,16 @@ class HipTreeBuilder : public TreeBuilder {
     d_active_ = DevAlloc<unsigned char>((size_t)(D_ - 1) * F_);
     rnd_.seed(cfg.internal.seed);  // garden.cu:87
     int shifts[2] = {30, 0};
-    if (cfg.objective == kLogisticRegression) shifts[1] = 32;  // 0 <= h <= 1/4
+    if (cfg.objective == kLogisticRegression) {
+      shifts[1] = 32;  // 0 <= h <= 1/4
+      // labels outside [0, 1] widen the gradient range
+      float ymin = 0.0f, ymax = 1.0f;
+      for (float v : data->y) {
+        ymin = std::min(ymin, v);
+        ymax = std::max(ymax, v);
+      }
+      shifts[0] = LogisticGradShift(ymin, ymax);
+    }
     if (cfg.objective >= kSoftMaxOneVsAll) shifts[1] = 31;     // 0 <= h <= 1/2
     HIP_OK(hipMemcpyAsync(d_shifts_, shifts, sizeof(shifts), hipMemcpyHostToDevice, stream_));
     HIP_OK(hipStreamSynchronize(stream_));

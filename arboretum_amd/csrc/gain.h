@@ -47,6 +47,15 @@ ARB_HD int FixShiftFromMax(float vmax) {
   return 30 - e;
 }
 
+// Logistic gradients g = y - s with 0 <= s <= 1 lie in [ymin - 1, ymax] (float
+// subtraction is monotonic, so the bounds hold for the rounded values too).
+// Labels in [0, 1] give |g| <= 1 and shift 30; any other finite labels get
+// the shift of their own bound.
+ARB_HD int LogisticGradShift(float ymin, float ymax) {
+  const float bound = fmaxf(fabsf(ymin - 1.0f), fabsf(ymax));
+  return bound <= 1.0f ? 30 : FixShiftFromMax(bound);
+}
+
 ARB_HD long long ToFixed(float v, int shift) {
   // Scaling by a power of two is exact in fp32, and so is rounding the result
   // to an integer (at or above 2^23 it is one already): the value is

@@ -283,6 +283,15 @@ const char *AGardenGetTree(VoidPointer garden, int t, int *fid, int *bin, float 
   });
 }
 
+const char *AGardenGetTreeDepth(VoidPointer garden, int t, int *depth) {
+  return Guard([&] {
+    Garden &g = AsGarden(garden)->garden;
+    if (t < 0 || (size_t)t >= g.num_trees()) throw std::runtime_error("tree index out of range");
+    if (!depth) throw std::runtime_error("bad arguments");
+    *depth = (int)g.tree(t).depth;
+  });
+}
+
 const char *AGardenGetLeaves(VoidPointer garden, unsigned *out) {
   return Guard([&] { BuilderOf(garden)->GetLeaves(out); });
 }

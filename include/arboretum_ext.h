@@ -56,7 +56,10 @@ const char *AGardenPredictOnDevice(VoidPointer garden, int on);
 const char *AGardenSetInspect(VoidPointer garden, int on);      /* keep per-level histograms */
 const char *AGardenNumTrees(VoidPointer garden, int *out);
 /* Tree t: fid/bin/threshold/gain of the 2^(depth-1)-1 internal nodes in heap
- * order (bin -1 = not split), 2^(depth-1) leaf weights.  Any pointer may be NULL. */
+ * order (bin -1 = not split), 2^(depth-1) leaf weights.  Any pointer may be
+ * NULL.  depth is the tree's own (AGardenGetTreeDepth: max_depth + 1 for a
+ * grown tree, the model's "depth" for a loaded one); size the arrays from it. */
+const char *AGardenGetTreeDepth(VoidPointer garden, int t, int *depth);
 const char *AGardenGetTree(VoidPointer garden, int t, int *fid, int *bin, float *threshold,
                            float *gain, float *weights);
 /* Leaf index of every training row in the last tree, original row order

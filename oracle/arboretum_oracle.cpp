@@ -323,6 +323,7 @@ static float weight_any(int kind, double g, double h, unsigned c, const GainPara
 // so |q| <= 2^30 and any sum over fewer than 2^32 rows fits in int64.
 //   logistic: |g| <= 1 -> shift 30; 0 <= h <= 1/4 -> shift 32
 //   softmax : |g| <= 1 -> shift 30; 0 <= h <= 1/2 -> shift 31
+//   logistic with labels outside [0, 1]: shift of max(|ymin - 1|, |ymax|)
 //   squared : e from frexp(max |g|) (max = m * 2^e, 1/2 <= m < 1); h is the count
 static inline int fix_shift_from_max(float vmax) {
   if (!(vmax > 0.0f) || std::isinf(vmax)) return 30;
@@ -496,7 +497,14 @@ static void grow_tree(Booster &b, int label) {
     b.shift_g = fix_shift_from_max(gmax);
     b.shift_h = 0;
   } else if (b.p.objective == 1) {
-    b.shift_g = 30;
+    // g = y - s, 0 <= s <= 1: |g| <= max(|ymin - 1|, |ymax|); 1 for labels in [0, 1]
+    float ymin = 0.0f, ymax = 1.0f;
+    for (int64_t i = 0; i < n; ++i) {
+      ymin = std::min(ymin, b.y[i]);
+      ymax = std::max(ymax, b.y[i]);
+    }
+    const float bound = std::max(std::fabs(ymin - 1.0f), std::fabs(ymax));
+    b.shift_g = bound <= 1.0f ? 30 : fix_shift_from_max(bound);
     b.shift_h = 32;
   } else {
     b.shift_g = 30;

@@ -159,6 +159,19 @@ def test_training_without_gpu_fails_loudly(arb):
         g.grow_tree()
 
 
+@pytest.mark.parametrize("bad", [np.nan, np.inf, -np.inf])
+@pytest.mark.parametrize("objective", [0, 1])
+def test_non_finite_targets_are_refused(arb, bad, objective):
+    # the fixed-point scale of the gradients has no meaning with a NaN or infinite target;
+    # refused on the host, before any device work
+    X = np.random.default_rng(0).normal(size=(50, 3)).astype(np.float32)
+    y = (X[:, 0] > 0).astype(np.float32)
+    y[17] = bad
+    g = arb.Garden({"objective": objective, "method": 1, "tree": {"max_depth": 2}}, arb.DMatrix(X, y=y))
+    with pytest.raises(arb.ArboretumError, match="y must be finite"):
+        g.grow_tree()
+
+
 def test_errors(arb):
     X = np.zeros((4, 2), np.float32)
     with pytest.raises(ValueError):
@@ -194,3 +207,20 @@ def test_no_alloc_histogram_size_limits_are_checked_before_the_gpu_is_touched():
     with pytest.raises(arb.ArboretumError, match="sibling pairs"):
         arb.hist_sum_no_alloc(p, p, p, p, p, p, p, 1024, 1000, 28, 3, 30, 32, use_trick=True, parent_g=p,
                               parent_h=p, parent_c=p)
+
+
+def test_tree_arrays_follow_the_depth_of_a_loaded_tree(arb):
+    # a model whose trees are deeper (and shallower) than the booster's configuration
+    def tree(depth):
+        ni = (1 << (depth - 1)) - 1
+        nodes = [{"id": i, "leaf": False, "left": 2 * i + 1, "right": 2 * i + 2, "threshold": float(i), "fid": i % 3}
+                 for i in range(ni)]
+        nodes += [{"id": ni + k, "leaf": True, "idx": k} for k in range(1 << (depth - 1))]
+        return {"nodes": nodes, "weights": [float(k) for k in range(1 << (depth - 1))], "depth": depth}
+    g = arb.Garden({"objective": 0, "method": 1, "tree": {"max_depth": 2}})
+    g.load(json.dumps({"model": [tree(5), tree(2)]}))
+    deep, shallow = g.tree(0), g.tree(1)
+    assert deep["fid"].shape == (15,) and deep["weights"].shape == (16,)
+    assert shallow["fid"].shape == (1,) and shallow["weights"].tolist() == [0.0, 1.0]
+    assert deep["weights"].tolist() == [float(k) for k in range(16)]
+    assert deep["threshold"].tolist() == [float(i) for i in range(15)]

@@ -159,6 +159,37 @@ def test_logistic_with_fractional_labels(arb, oracle, inspect, trick):
     assert_same_training(arb, oracle, X, y, cfg, rounds=4, check_hist=inspect)
 
 
+@pytest.mark.parametrize("labels,shift_g", [((-1.0, 1.0), 28), ((0.0, 2.5), 28), ((-6.0, 0.5), 27)])
+def test_logistic_with_labels_outside_0_1(arb, oracle, labels, shift_g):
+    # g = y - sigmoid leaves [-1, 1] when a label does: the fixed-point scale follows the label
+    # range (max(|ymin - 1|, |ymax|) = 2, 2.5, 7 here) instead of dropping such rows
+    X, y = make_data(20000, 9, 1, seed=17)
+    y = np.where(y > 0, labels[1], labels[0]).astype(np.float32)
+    cfg = {"objective": 1, "method": 1, "internals": {"hist_size": 64, "double_precision": True},
+           "tree": {"max_depth": 5, "eta": 0.3, "lambda": 1.0}}
+    ob, g = assert_same_training(arb, oracle, X, y, cfg, rounds=3)
+    assert g.shifts() == (shift_g, 32)
+    # no gradient was dropped: the root's integer total is the sum of the rows' fixed-point values
+    gg, _ = g.grad()
+    total = int(np.rint(gg.astype(np.float64) * 2.0 ** shift_g).sum())
+    assert int(g.level_hist(0)[0, 0, :, 0].sum()) == total and total != 0
+
+
+def test_heavy_tailed_regression_targets(arb, oracle):
+    # five targets 2^21 times larger than the rest set the fixed-point scale of every row (7
+    # fractional bits for the typical residual); the device must still equal the checker bit
+    # for bit, and the checker's splits equal those of fp64 accumulation (CPU test)
+    rng = np.random.default_rng(1)
+    n, F = 20000, 8
+    X = rng.normal(size=(n, F)).astype(np.float32)
+    y = (X[:, 0] * 2 + np.sin(X[:, 1] * 3) + 0.1 * rng.normal(size=n)).astype(np.float32)
+    y[rng.choice(n, 5, replace=False)] *= 2.0 ** 21
+    cfg = {"objective": 0, "method": 1, "internals": {"hist_size": 63, "double_precision": True},
+           "tree": {"max_depth": 5, "eta": 0.3, "lambda": 1.0, "min_leaf_size": 50}}
+    ob, g = assert_same_training(arb, oracle, X, y, cfg, rounds=4)
+    assert g.shifts()[0] <= 8
+
+
 @pytest.mark.parametrize("inspect", [True, False])
 @pytest.mark.parametrize("eta", [30.0, 70.0, 1e4])
 def test_logistic_with_saturated_predictions(arb, oracle, inspect, eta):

@@ -374,3 +374,50 @@ def test_softmax_gradient_is_the_derivative_of_the_log_likelihood(oracle):
         dn[k] -= eps
         num = (log_softmax(up, axis=0)[labels, np.arange(n)] - log_softmax(dn, axis=0)[labels, np.arange(n)]) / (2 * eps)
         assert np.allclose(g[k], num, atol=1e-6)
+
+
+def test_heavy_tailed_regression_fixed_point_keeps_the_split_choice(oracle):
+    # Squared error scales the fixed point by the round's largest residual: with five targets
+    # 2^21 times larger than the rest a typical residual keeps 7 fractional bits.  The splits
+    # must still be those of fp64 accumulation (the reference's double_precision=true sums).
+    rng = np.random.default_rng(1)
+    n, F = 20000, 8
+    X = rng.normal(size=(n, F)).astype(np.float32)
+    y = (X[:, 0] * 2 + np.sin(X[:, 1] * 3) + 0.1 * rng.normal(size=n)).astype(np.float32)
+    y[rng.choice(n, 5, replace=False)] *= 2.0 ** 21
+    cfg = {"objective": 0, "method": 1, "internals": {"hist_size": 63, "double_precision": True},
+           "tree": {"max_depth": 5, "eta": 0.3, "lambda": 1.0, "min_leaf_size": 50}}
+    fixed, native = oracle.Booster(X, y=y, config=cfg, accum=0), oracle.Booster(X, y=y, config=cfg, accum=1)
+    for r in range(4):
+        fixed.grow(1)
+        native.grow(1)
+        a, b = fixed.tree(r), native.tree(r)
+        assert fixed.shifts()[0] <= 8
+        assert np.array_equal(a["fid"], b["fid"]) and np.array_equal(a["quantized"], b["quantized"])
+        # nodes that hold no outlier see the coarse scale: their gains agree to 1e-3 relative only
+        # (the documented limit of one scale per round), nodes with outliers to 1e-5
+        assert np.allclose(a["gain"], b["gain"], rtol=2e-3)
+        big = b["gain"] > 1e6
+        assert big.any() and np.allclose(a["gain"][big], b["gain"][big], rtol=1e-5)
+        assert np.allclose(a["weights"], b["weights"], rtol=1e-5, atol=1e-3)
+    assert np.array_equal(fixed.leaf(), native.leaf())
+
+
+def test_logistic_labels_outside_0_1_keep_their_gradients(oracle):
+    # the fixed-point scale follows the label range: no row's gradient is dropped
+    rng = np.random.default_rng(2)
+    X = rng.normal(size=(3000, 4)).astype(np.float32)
+    y = np.where(X[:, 0] > 0, 1.0, -1.0).astype(np.float32)
+    cfg = {"objective": 1, "method": 1, "internals": {"hist_size": 31, "double_precision": True},
+           "tree": {"max_depth": 3, "eta": 0.3, "lambda": 1.0}}
+    b = oracle.Booster(X, y=y, config=cfg)
+    b.grow(1)
+    assert b.shifts() == (28, 32)
+    g, _ = b.grad()
+    assert g.min() < -1.0      # y = -1 rows: g = -1 - s
+    root = b.level_hist(0)[0, 0]
+    assert int(root[:, 0].sum()) == int(np.rint(g.astype(np.float64) * 2.0 ** 28).sum())
+    native = oracle.Booster(X, y=y, config=cfg, accum=1)
+    native.grow(1)
+    assert np.array_equal(b.tree(0)["fid"], native.tree(0)["fid"])
+    assert np.array_equal(b.tree(0)["quantized"], native.tree(0)["quantized"])
