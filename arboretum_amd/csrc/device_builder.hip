@@ -335,8 +335,8 @@ struct FusedArgs {
   const unsigned *seg_start;
   const WorkItem *work;
   const unsigned *n_work;
-  const unsigned *wave_left;
-  const unsigned *item_left;
+  unsigned *cursor;     // claims destinations (null: read item_base)
+  unsigned *item_base;  // claimed destination bases, two per work item
   unsigned long long *slab;
   int slab_entries;
   const uint32_t *split_bins;  // start of the whole matrix
@@ -354,7 +354,7 @@ void LaunchFusedNQ(hipStream_t st, unsigned grid, const FusedArgs &a) {
   hipLaunchKernelGGL((k_part_hist<PAIR, NQ, WRITE, GROUP, PACK>), dim3(grid), dim3(kHistThreads), lds, st,
                      a.bins + (size_t)a.q0 * a.stride, a.bins_out ? a.bins_out + (size_t)a.q0 * a.stride : nullptr,
                      a.stride, a.F, a.g, a.g_out, a.h, a.h_out, a.shifts, a.split, a.tot, a.seg_start, a.work,
-                     a.n_work, a.wave_left, a.item_left, a.slab, a.slab_entries, a.split_bins, a.q0);
+                     a.n_work, a.cursor, a.item_base, a.slab, a.slab_entries, a.split_bins, a.q0);
 }
 
 template <bool PAIR, bool WRITE, bool GROUP, bool PACK>
@@ -478,7 +478,8 @@ class HipTreeBuilder : public TreeBuilder {
     d_pwork_ = DevAlloc<WorkItem>(max_part_items_);
     d_nwork_ = DevAlloc<unsigned>(2);
     d_wave_left_ = DevAlloc<unsigned>((size_t)max_part_items_ * kItemWaves);
-    d_item_left_ = DevAlloc<unsigned>(max_part_items_);
+    d_item_left_ = DevAlloc<unsigned>((size_t)2 * max_part_items_);  // also the claimed bases of the fused pass
+    d_cursor2_ = DevAlloc<unsigned>((size_t)2 * last_nodes);
     d_slab_ = DevAlloc<unsigned long long>((size_t)std::max(max_hist_items_, max_part_items_) * slab_entries_ * (pair_ ? 2 : 1));
     d_shifts_ = DevAlloc<int>(2);
     d_records_ = DevAlloc<uint32_t>(kRecordRing * RecordWords());
@@ -515,7 +516,7 @@ class HipTreeBuilder : public TreeBuilder {
     (void)hipStreamSynchronize(stream_);
     void *ptrs[] = {d_y_, d_labels_, d_yhat_, d_g_, d_h_, d_leaf_, d_split_, d_cand_, d_node_first_,
                     d_node_items_, d_hwork_, d_pwork_, d_nwork_, d_wave_left_, d_item_left_, d_slab_,
-                    d_shifts_, d_gmax_, d_rows_scanned_, d_tfid_, d_tbin_, d_tgain_, d_weights_, d_active_, d_overflow_, d_records_};
+                    d_shifts_, d_gmax_, d_rows_scanned_, d_tfid_, d_tbin_, d_tgain_, d_weights_, d_active_, d_overflow_, d_records_, d_cursor2_};
     for (void *p : ptrs)
       if (p) (void)hipFree(p);
     for (int b = 0; b < 2; ++b) {
@@ -837,11 +838,6 @@ class HipTreeBuilder : public TreeBuilder {
         if (fused_) {
           // the work plan was written together with the splits of the parents
           const unsigned grid = FusedGrid(PL);
-          if (!last) {  // destination offsets; the last level moves no rows
-            Mark(kPartition);
-            hipLaunchKernelGGL(k_part_count, dim3(grid), dim3(kHistThreads), 0, stream_, src.bins, stride_, d_split_,
-                               d_pwork_, d_nwork_ + 1, d_wave_left_, d_item_left_, code_);
-          }
           Mark(last ? kFusedLast : kHistDeep);
           // matrices wider than one LDS histogram: one launch per group of
           // quads; the first one moves the gradients
@@ -849,7 +845,8 @@ class HipTreeBuilder : public TreeBuilder {
             const int nq = std::min(quads_per_group_, Q_ - q0);
             FusedArgs a{src.bins, last ? nullptr : dst.bins, stride_, F_, src.g, q0 == 0 ? dst.g : nullptr, src.h,
                         q0 == 0 ? dst.h : nullptr, d_shifts_, d_split_, d_tot_[ps], d_seg_[ps], d_pwork_,
-                        d_nwork_ + 1, d_wave_left_, d_item_left_, d_slab_, slab_entries_, src.bins, q0};
+                        d_nwork_ + 1, q0 == 0 ? d_cursor2_ : nullptr, d_item_left_, d_slab_, slab_entries_, src.bins,
+                        q0};
 #define ARB_FUSED(P, W)                                                       \
   do {                                                                        \
     if (P && pack_ && single_group_) LaunchFused<P, W, false, P>(nq, stream_, grid, a); \
@@ -963,7 +960,7 @@ class HipTreeBuilder : public TreeBuilder {
                      d_hh_[hb], d_hc_[hb], nbin_total_, F_, slots_, L, d_tot_[state], d_shifts_, gp, hs,          \
                      d_seg_[state], d_tot_[state ^ 1], d_seg_[state ^ 1], d_split_, d_tfid_, d_tbin_, d_tgain_,   \
                      L - 1, active, plan_next ? 1 : 0, per_item, d_pwork_, d_nwork_ + 1, d_node_first_,           \
-                     d_node_items_, d_rows_scanned_, FusedGrid(L), d_overflow_)
+                     d_node_items_, d_rows_scanned_, FusedGrid(L), d_overflow_, d_cursor2_)
       if (pair_ && f64_) ARB_SCAN_SELECT(true, true);
       else if (pair_) ARB_SCAN_SELECT(true, false);
       else if (f64_) ARB_SCAN_SELECT(false, true);
@@ -984,7 +981,7 @@ class HipTreeBuilder : public TreeBuilder {
       hipLaunchKernelGGL(k_select_plan, dim3(1), dim3(1024), 0, stream_, d_cand_, F_, L, d_tot_[state],
                          d_seg_[state], d_tot_[state ^ 1], d_seg_[state ^ 1], d_split_, d_tfid_, d_tbin_, d_tgain_,
                          L - 1, active, per_item, d_pwork_, d_nwork_ + 1, d_node_first_, d_node_items_,
-                         d_rows_scanned_, FusedGrid(L), d_overflow_);
+                         d_rows_scanned_, FusedGrid(L), d_overflow_, d_cursor2_);
     } else {
       hipLaunchKernelGGL(k_split_select, dim3((L + 15) / 16), dim3(1024), 0, stream_, d_cand_, F_, L,
                          d_tot_[state], d_seg_[state], d_tot_[state ^ 1], d_seg_[state ^ 1], d_split_,
@@ -1248,7 +1245,7 @@ class HipTreeBuilder : public TreeBuilder {
   std::default_random_engine rnd_;
   bool sampling_ = false;
   unsigned *d_leaf_ = nullptr, *d_node_first_ = nullptr, *d_node_items_ = nullptr, *d_nwork_ = nullptr,
-           *d_wave_left_ = nullptr, *d_item_left_ = nullptr, *d_gmax_ = nullptr;
+           *d_wave_left_ = nullptr, *d_item_left_ = nullptr, *d_gmax_ = nullptr, *d_cursor2_ = nullptr;
   RowBuffers buf_[2];
   // streamed matrices: two block buffers filled by the copy stream, a staging
   // buffer with the rows of the built nodes, a resident node id per row

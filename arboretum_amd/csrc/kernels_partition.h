@@ -112,6 +112,86 @@ __device__ __forceinline__ void WaveOffsets(const WorkItem &it, const SplitRec &
   *ro = start + (unsigned)s.left.c + rows_before - lefts_before;
 }
 
+// Rows of this wave going left, counted by the wave itself over its own chunks
+// (the fused pass does this instead of a separate counting launch).  The chunks
+// are read last one first: the lines the pass reads first are then the ones
+// most recently brought into the cache.  Wave-uniform result.
+__device__ __forceinline__ unsigned CountWaveLefts(const WorkItem &it, const SplitRec &s, const uint32_t *__restrict__ col,
+                                                  int wave, int lane) {
+  const unsigned cb = ChunkOrigin(it);
+  const unsigned wb = cb + (unsigned)wave * kChunkRows, we = it.end;
+  unsigned cnt = 0;
+  if (wb < we) {
+    const int nk = (int)((we - wb + kChunkStep - 1) / kChunkStep);  // chunks of this wave
+    if (s.fid < 0) {  // not split: every row stays left
+      for (int k = 0; k < nk; ++k) {
+        const unsigned base = wb + (unsigned)k * kChunkStep;
+        cnt += min(base + kChunkRows, we) - max(base, it.begin);
+      }
+      return cnt;
+    }
+    const int fs = 8 * (s.fid & 3);
+    constexpr int kBatch = 24;  // loads in flight per wave: all of a typical item at once
+    for (int k0 = nk - 1; k0 >= 0; k0 -= kBatch) {
+      uint32_t v0[kBatch], v1[kBatch];
+#pragma unroll
+      for (int j = 0; j < kBatch; ++j) {
+        const int k = max(k0 - j, 0);
+        const unsigned r0 = wb + (unsigned)k * kChunkStep + lane, r1 = r0 + 64;
+        v0[j] = col[min(r0, we - 1)];
+        v1[j] = col[min(r1, we - 1)];
+      }
+#pragma unroll
+      for (int j = 0; j < kBatch; ++j) {
+        const int k = k0 - j;
+        const unsigned r0 = wb + (unsigned)max(k, 0) * kChunkStep + lane, r1 = r0 + 64;
+        if (k >= 0 && r0 >= it.begin && r0 < we) cnt += ((int)((v0[j] >> fs) & 255u) > s.bin) ? 0u : 1u;
+        if (k >= 0 && r1 < we) cnt += ((int)((v1[j] >> fs) & 255u) > s.bin) ? 0u : 1u;
+      }
+    }
+  }
+  for (int off = 32; off > 0; off >>= 1) cnt += __shfl_xor(cnt, off);
+  return cnt;
+}
+
+// Destination offsets of a wave of the fused pass without a counting launch:
+// the waves count their rows going left (CountWaveLefts), the workgroup claims
+// its share of the two children's row ranges with one atomic add per child on
+// the node's pair of cursors (zero at launch), and the waves take their parts
+// in wave order.  The order of the work items inside a child's range depends
+// on the order of the claims; no result depends on it (all sums are integers).
+// The claims of work item w are kept in item_base[2 w], [2 w + 1]: a matrix
+// wider than one LDS histogram takes several launches per level, which must
+// all send a row to the same place; only the first one claims (cursor set),
+// the others read what it claimed (cursor null).
+// Called by the whole workgroup; s_tmp holds kItemWaves + 2 words.
+__device__ __forceinline__ void ClaimOffsets(const WorkItem &it, unsigned w, const SplitRec &s, unsigned start,
+                                             const uint32_t *__restrict__ col, unsigned *__restrict__ cursor,
+                                             unsigned *__restrict__ item_base, int wave, int lane,
+                                             unsigned *s_tmp, unsigned *lo, unsigned *ro) {
+  const unsigned mine = CountWaveLefts(it, s, col, wave, lane);
+  if (lane == 0) s_tmp[wave] = mine;
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    if (cursor != nullptr) {
+      unsigned lefts = 0;
+      for (int k = 0; k < kItemWaves; ++k) lefts += s_tmp[k];
+      const unsigned rows = it.end - it.begin;
+      item_base[2 * w] = s_tmp[kItemWaves] = atomicAdd(&cursor[2 * it.node], lefts);
+      item_base[2 * w + 1] = s_tmp[kItemWaves + 1] = atomicAdd(&cursor[2 * it.node + 1], rows - lefts);
+    } else {
+      s_tmp[kItemWaves] = item_base[2 * w];
+      s_tmp[kItemWaves + 1] = item_base[2 * w + 1];
+    }
+  }
+  __syncthreads();
+  unsigned lefts_before = 0;
+  for (int k = 0; k < wave; ++k) lefts_before += s_tmp[k];
+  const unsigned rows_before = RowsOfEarlierWaves(it, wave);
+  *lo = start + s_tmp[kItemWaves] + lefts_before;
+  *ro = start + (unsigned)s.left.c + s_tmp[kItemWaves + 1] + rows_before - lefts_before;
+}
+
 // Destination lane of this lane's row when the rows flagged in the
 // wave-uniform mask m are packed, in lane order, into lanes first, first + 1,
 // ... (mod 64) of a wave: the flagged rows first, the others behind them, so
@@ -295,11 +375,11 @@ k_part_hist(const uint32_t *__restrict__ bins, uint32_t *__restrict__ bins_out, 
             float *__restrict__ h_out, const int *__restrict__ shifts,
             const SplitRec *__restrict__ split, const NodeSum *__restrict__ tot,
             const unsigned *__restrict__ seg_start, const WorkItem *__restrict__ work,
-            const unsigned *__restrict__ n_work, const unsigned *__restrict__ wave_left,
-            const unsigned *__restrict__ item_left, unsigned long long *__restrict__ slab,
+            const unsigned *__restrict__ n_work, unsigned *__restrict__ cursor,
+            unsigned *__restrict__ item_base, unsigned long long *__restrict__ slab,
             int slab_entries, const uint32_t *__restrict__ split_bins, int q0) {
   extern __shared__ unsigned long long lds[];
-  __shared__ unsigned s_tmp[kItemWaves + 1];
+  __shared__ unsigned s_tmp[kItemWaves + 2];
   const unsigned w = blockIdx.x;
   if (w >= *n_work) return;
   const WorkItem it = work[w];
@@ -311,13 +391,12 @@ k_part_hist(const uint32_t *__restrict__ bins, uint32_t *__restrict__ bins_out, 
   const int sg = shifts[0], sh = shifts[1];
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const unsigned wb = ChunkOrigin(it) + wave * kChunkRows, we = it.end;
-  unsigned lo = 0, ro = 0;
-  if (WRITE) {
-    const unsigned before = LeftsBefore(it, w, wave, wave_left, item_left, s_tmp);
-    WaveOffsets(it, s, seg_start[it.node], before, wave, &lo, &ro);
-  }
-  __syncthreads();
   const int fq = s.fid >> 2, fs = 8 * (s.fid & 3);
+  unsigned lo = 0, ro = 0;
+  if (WRITE)
+    ClaimOffsets(it, w, s, seg_start[it.node], split_bins + (size_t)(s.fid < 0 ? 0 : fq) * stride, cursor, item_base,
+                 wave, lane, s_tmp, &lo, &ro);
+  __syncthreads();
   if constexpr (WRITE) {
     // QB: rows of the child whose histogram is built, QO: the other child
     RowQueue<NQ> QB, QO;

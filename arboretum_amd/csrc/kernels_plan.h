@@ -14,6 +14,8 @@ namespace {
 // rows_scanned (optional) is advanced by the rows that will be accumulated
 // into histograms: the selected rows, or, when `split` is given (fused
 // partition + histogram over parent nodes), the smaller side of every split.
+// cursor (optional): two words per node, cleared here; the fused pass claims
+// the destination ranges of its work items on them.
 // One workgroup.
 __device__ __forceinline__ void PlanBody(const NodeSum *__restrict__ tot, const unsigned *__restrict__ seg_start,
                                          int L, int select, unsigned rows_per_item,
@@ -21,7 +23,8 @@ __device__ __forceinline__ void PlanBody(const NodeSum *__restrict__ tot, const 
                                          unsigned *__restrict__ node_first, unsigned *__restrict__ node_items,
                                          unsigned long long *__restrict__ rows_scanned,
                                          const SplitRec *__restrict__ split, unsigned max_items,
-                                         unsigned *__restrict__ overflow) {
+                                         unsigned *__restrict__ overflow,
+                                         unsigned *__restrict__ cursor = nullptr) {
   __shared__ unsigned s_base[kMaxPlanNodes + 1];
   __shared__ unsigned s_wave[16];
   __shared__ unsigned s_carry;
@@ -55,6 +58,10 @@ __device__ __forceinline__ void PlanBody(const NodeSum *__restrict__ tot, const 
         atomicAdd(&s_rows, acc);
       }
       node_items[nd] = sel ? cnt : 0xffffffffu;  // 0xffffffff marks "not selected"
+      if (cursor) {  // destination cursors of the node's two children in the fused pass
+        cursor[2 * nd] = 0;
+        cursor[2 * nd + 1] = 0;
+      }
     }
     // block exclusive scan of cnt
     unsigned incl = cnt;

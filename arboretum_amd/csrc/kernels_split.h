@@ -231,13 +231,13 @@ k_select_plan(const Cand *__restrict__ cand, int F, int L, const NodeSum *__rest
               WorkItem *__restrict__ work, unsigned *__restrict__ n_work,
               unsigned *__restrict__ node_first, unsigned *__restrict__ node_items,
               unsigned long long *__restrict__ rows_scanned, unsigned max_items,
-              unsigned *__restrict__ overflow) {
+              unsigned *__restrict__ overflow, unsigned *__restrict__ cursor) {
   for (int nd = threadIdx.x >> 6; nd < L; nd += 16)
     SelectNode(nd, threadIdx.x & 63, cand, F, tot, seg_start, tot_next, seg_next, split, t_fid, t_bin, t_gain,
                heap_off, active);
   __syncthreads();  // the splits written above are read by the plan
   PlanBody(tot, seg_start, L, 0, rows_per_item, work, n_work, node_first, node_items, rows_scanned, split,
-           max_items, overflow);
+           max_items, overflow, cursor);
 }
 
 // Split scan and selection in one launch: workgroup `nd` < L scans the
@@ -257,10 +257,10 @@ k_scan_select(const long long *__restrict__ hg, const long long *__restrict__ hh
               const unsigned char *__restrict__ active, int plan, unsigned rows_per_item,
               WorkItem *__restrict__ work, unsigned *__restrict__ n_work, unsigned *__restrict__ node_first,
               unsigned *__restrict__ node_items, unsigned long long *__restrict__ rows_scanned,
-              unsigned max_items, unsigned *__restrict__ overflow) {
+              unsigned max_items, unsigned *__restrict__ overflow, unsigned *__restrict__ cursor) {
   if ((int)blockIdx.x >= L) {  // uniform per workgroup
     PlanBody(tot, seg_start, L, 0, rows_per_item, work, n_work, node_first, node_items, nullptr, nullptr, max_items,
-             overflow);
+             overflow, cursor);
     return;
   }
   __shared__ Cand s_cand[16];
