@@ -61,6 +61,7 @@ def _load_lib():
         "AGardenEnableTiming": [c_void_p, c_int],
         "AGardenGetTimings": [c_void_p, c_void_p],
         "AGardenRowsScanned": [c_void_p, P(ctypes.c_ulonglong)],
+        "AGardenRowsScannedByLevel": [c_void_p, c_void_p],
         "AGardenSynchronize": [c_void_p],
         "AHistSum": [c_void_p] * 10 + [ctypes.c_ulonglong, ctypes.c_longlong, c_int, c_int, c_int, c_int, c_int,
                                        c_void_p],
@@ -291,6 +292,12 @@ class Garden(object):
         v = ctypes.c_ulonglong()
         _check(_LIB.AGardenRowsScanned(self.handle, ctypes.byref(v)))
         return v.value
+
+    def rows_scanned_by_level(self):
+        """Rows accumulated into histograms so far, per tree level (root = 0)."""
+        out = np.zeros(32, dtype=np.uint64)
+        _check(_LIB.AGardenRowsScannedByLevel(self.handle, out.ctypes.data_as(ctypes.c_void_p)))
+        return out
 
     def synchronize(self):
         _check(_LIB.AGardenSynchronize(self.handle))

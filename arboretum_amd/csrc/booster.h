@@ -118,6 +118,7 @@ class TreeBuilder {
   virtual void EnableTiming(int level) = 0;
   virtual BuilderTimings GetTimings() = 0;
   virtual unsigned long long RowsScanned() = 0;            // rows accumulated into histograms
+  virtual void RowsScannedByLevel(unsigned long long *out) = 0;  // the same per tree level, 32 entries
   virtual void Synchronize() = 0;
 };
 

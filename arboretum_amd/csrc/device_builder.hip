@@ -484,10 +484,10 @@ class HipTreeBuilder : public TreeBuilder {
     d_shifts_ = DevAlloc<int>(2);
     d_records_ = DevAlloc<uint32_t>(kRecordRing * RecordWords());
     d_gmax_ = DevAlloc<unsigned>(1);
-    d_rows_scanned_ = DevAlloc<unsigned long long>(1);
+    d_rows_scanned_ = DevAlloc<unsigned long long>(kScanLevels);  // one counter per tree level
     d_overflow_ = DevAlloc<unsigned>(1);
     HIP_OK(hipMemsetAsync(d_overflow_, 0, sizeof(unsigned), stream_));
-    HIP_OK(hipMemsetAsync(d_rows_scanned_, 0, sizeof(unsigned long long), stream_));
+    HIP_OK(hipMemsetAsync(d_rows_scanned_, 0, kScanLevels * sizeof(unsigned long long), stream_));
     HIP_OK(hipMemsetAsync(d_gmax_, 0, sizeof(unsigned), stream_));
     const int internal = (1 << (D_ - 1)) - 1;
     d_tfid_ = DevAlloc<int>(internal);
@@ -660,10 +660,14 @@ class HipTreeBuilder : public TreeBuilder {
     return timings_;
   }
   unsigned long long RowsScanned() override {
-    unsigned long long v = 0;
+    unsigned long long v[kScanLevels], sum = 0;
+    RowsScannedByLevel(v);
+    for (int k = 0; k < kScanLevels; ++k) sum += v[k];
+    return sum;
+  }
+  void RowsScannedByLevel(unsigned long long *out) override {  // kScanLevels entries
     HIP_OK(hipStreamSynchronize(stream_));
-    HIP_OK(hipMemcpy(&v, d_rows_scanned_, sizeof(v), hipMemcpyDeviceToHost));
-    return v;
+    HIP_OK(hipMemcpy(out, d_rows_scanned_, kScanLevels * sizeof(unsigned long long), hipMemcpyDeviceToHost));
   }
   void Synchronize() override {
     HIP_OK(hipStreamSynchronize(stream_));
@@ -723,24 +727,27 @@ class HipTreeBuilder : public TreeBuilder {
     return (unsigned)std::min<size_t>(std::max<size_t>(t, kHistThreads), kMaxHistRows);
   }
 
+  // the counter of rows accumulated into histograms at `level` (levels past the last counter share it)
+  unsigned long long *ScanCounter(int level) { return d_rows_scanned_ + std::min(level, kScanLevels - 1); }
+  // count_level >= 0: the planned rows are histogram work of that tree level
   void Plan(int state, int L, int select, unsigned rows_per_item, WorkItem *work, unsigned *n_work,
-            bool count_rows, const SplitRec *split, unsigned max_items) {
-    PlanOn(d_tot_[state], d_seg_[state], L, select, rows_per_item, work, n_work, count_rows, split, max_items);
+            int count_level, const SplitRec *split, unsigned max_items) {
+    PlanOn(d_tot_[state], d_seg_[state], L, select, rows_per_item, work, n_work, count_level, split, max_items);
   }
   void PlanOn(const NodeSum *tot, const unsigned *seg, int L, int select, unsigned rows_per_item, WorkItem *work,
-              unsigned *n_work, bool count_rows, const SplitRec *split, unsigned max_items) {
+              unsigned *n_work, int count_level, const SplitRec *split, unsigned max_items) {
     hipLaunchKernelGGL(k_plan, dim3(1), dim3(1024), 0, stream_, tot, seg, L, select,
                        rows_per_item, work, n_work, d_node_first_, d_node_items_,
-                       count_rows ? d_rows_scanned_ : (unsigned long long *)nullptr, split, max_items, d_overflow_);
+                       count_level >= 0 ? ScanCounter(count_level) : (unsigned long long *)nullptr, split, max_items, d_overflow_);
   }
 
   // Histograms of contiguous node ranges in `cur` (level order), feature group by group.
-  void HistOfNodes(const RowBuffers &cur, int state, int L, bool select_smaller, size_t rows_max, bool root) {
+  void HistOfNodes(const RowBuffers &cur, int state, int L, bool select_smaller, size_t rows_max, bool root, int level) {
     // the root level is one node: one item per CU avoids a second, partial round
     const unsigned per_item = HistRowsPerItem(rows_max, root ? 256 : 512);
     const unsigned grid = (unsigned)std::min<size_t>(rows_max / per_item + 2 * L + 1, max_hist_items_);
     Mark(kPlan);
-    Plan(state, L, select_smaller ? 1 : 0, per_item, d_hwork_, d_nwork_, true, nullptr, grid);
+    Plan(state, L, select_smaller ? 1 : 0, per_item, d_hwork_, d_nwork_, level, nullptr, grid);
     Mark(root ? kHistRoot : kHistDeep);
     if (wide_) {
       for (int f0 = 0; f0 < F_; f0 += wide_group_) {
@@ -823,7 +830,7 @@ class HipTreeBuilder : public TreeBuilder {
       const bool last = level + 2 >= D_;
       if (level == 0) {
         // the slabs of the root may have been written by the last pass of the previous tree
-        if (!root_hist_ready_) HistOfNodes(orig, state, 1, false, n_, true);
+        if (!root_hist_ready_) HistOfNodes(orig, state, 1, false, n_, true, 0);
         root_hist_ready_ = false;
         Reduce(1, hb, false, state, false);
         // (the last pass of the previous tree has also summed the root's totals)
@@ -869,12 +876,12 @@ class HipTreeBuilder : public TreeBuilder {
         } else {
           const unsigned grid = (unsigned)std::min<size_t>(n_ / kPartRows + 2 * PL + 1, max_part_items_);
           Mark(kPlan);
-          Plan(ps, PL, 0, kPartRows, d_pwork_, d_nwork_ + 1, false, nullptr, grid);
+          Plan(ps, PL, 0, kPartRows, d_pwork_, d_nwork_ + 1, -1, nullptr, grid);
           Mark(kPartition);
           hipLaunchKernelGGL(k_part_count, dim3(grid), dim3(kHistThreads), 0, stream_, src.bins, stride_, d_split_,
                              d_pwork_, d_nwork_ + 1, d_wave_left_, d_item_left_, code_);
           LaunchPartRows(grid, src, dst, ps);
-          HistOfNodes(dst, state, L, trick_, trick_ ? n_ / 2 : n_, false);
+          HistOfNodes(dst, state, L, trick_, trick_ ? n_ / 2 : n_, false, level);
           Reduce(L, hb, false, ps, trick_);
         }
       }
@@ -960,7 +967,7 @@ class HipTreeBuilder : public TreeBuilder {
                      d_hh_[hb], d_hc_[hb], nbin_total_, F_, slots_, L, d_tot_[state], d_shifts_, gp, hs,          \
                      d_seg_[state], d_tot_[state ^ 1], d_seg_[state ^ 1], d_split_, d_tfid_, d_tbin_, d_tgain_,   \
                      L - 1, active, plan_next ? 1 : 0, per_item, d_pwork_, d_nwork_ + 1, d_node_first_,           \
-                     d_node_items_, d_rows_scanned_, FusedGrid(L), d_overflow_, d_cursor2_)
+                     d_node_items_, ScanCounter(level + 1), FusedGrid(L), d_overflow_, d_cursor2_)
       if (pair_ && f64_) ARB_SCAN_SELECT(true, true);
       else if (pair_) ARB_SCAN_SELECT(true, false);
       else if (f64_) ARB_SCAN_SELECT(false, true);
@@ -981,7 +988,7 @@ class HipTreeBuilder : public TreeBuilder {
       hipLaunchKernelGGL(k_select_plan, dim3(1), dim3(1024), 0, stream_, d_cand_, F_, L, d_tot_[state],
                          d_seg_[state], d_tot_[state ^ 1], d_seg_[state ^ 1], d_split_, d_tfid_, d_tbin_, d_tgain_,
                          L - 1, active, per_item, d_pwork_, d_nwork_ + 1, d_node_first_, d_node_items_,
-                         d_rows_scanned_, FusedGrid(L), d_overflow_, d_cursor2_);
+                         ScanCounter(level + 1), FusedGrid(L), d_overflow_, d_cursor2_);
     } else {
       hipLaunchKernelGGL(k_split_select, dim3((L + 15) / 16), dim3(1024), 0, stream_, d_cand_, F_, L,
                          d_tot_[state], d_seg_[state], d_tot_[state ^ 1], d_seg_[state ^ 1], d_split_,
@@ -1129,7 +1136,7 @@ class HipTreeBuilder : public TreeBuilder {
         const unsigned per_item = HistRowsPerItem(rows);
         const unsigned grid = (unsigned)std::min<size_t>(rows / per_item + 2 * L + 1, max_hist_items_);
         Mark(kPlan);
-        PlanOn(d_blk_tot_, d_blk_seg_, L, 0, per_item, d_hwork_, d_nwork_, true, nullptr, grid);
+        PlanOn(d_blk_tot_, d_blk_seg_, L, 0, per_item, d_hwork_, d_nwork_, level, nullptr, grid);
         Mark(level == 0 ? kHistRoot : kHistDeep);
         for (int q0 = 0; q0 < Q_; q0 += quads_per_group_) {
           const int nq = std::min(quads_per_group_, Q_ - q0);
@@ -1226,6 +1233,7 @@ class HipTreeBuilder : public TreeBuilder {
   int wide_group_ = 2;    // features per histogram launch with 16-bit bins
   BinCode code_ = BinCode{2, 8};
   bool root_hist_ready_ = false;  // the slabs hold the root histogram of the tree grown next
+  static constexpr int kScanLevels = 32;      // per-level counters of rows accumulated into histograms
   static constexpr size_t kRecordRing = 64;  // trees whose records may wait on the device
   uint32_t *d_records_ = nullptr;
   std::vector<size_t> pending_;              // indices into *owner_ of the trees not fetched yet

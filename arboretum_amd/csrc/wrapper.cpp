@@ -337,6 +337,9 @@ const char *AGardenGetTimings(VoidPointer garden, double *out) {
 const char *AGardenRowsScanned(VoidPointer garden, unsigned long long *out) {
   return Guard([&] { *out = BuilderOf(garden)->RowsScanned(); });
 }
+const char *AGardenRowsScannedByLevel(VoidPointer garden, unsigned long long *out) {
+  return Guard([&] { BuilderOf(garden)->RowsScannedByLevel(out); });
+}
 const char *AGardenSynchronize(VoidPointer garden) {
   return Guard([&] { BuilderOf(garden)->Synchronize(); });
 }

@@ -10,7 +10,14 @@ matrix.  Prints ONE JSON line.
   ms_per_step  milliseconds per tree
   roofline     the dominant kernel (fused partition + histogram pass):
                algorithmic bytes of its launches / their summed duration (HIP
-               events on the builder's stream), against 8 TB/s
+               events on the builder's stream), against 8 TB/s.  Algorithmic
+               bytes of a launch over the rows of a level's parents:
+                 rows scanned (smaller children) x (F bin bytes + 8 gradient bytes)
+                 + all rows x 9 (partition: 4 index + 1 node + 4 index)
+                 + built nodes x F x 256 x 20 (histogram cells written once)
+               `moved_*` keys give what this implementation moves instead (it
+               re-orders the rows themselves), `traffic` the HBM bytes per
+               launch from hardware counters of a committed profile
   cpu_baseline the CPU checker (oracle/, OpenMP) on a bounded row sample of the
                same workload, timed on this host
 """
@@ -25,8 +32,36 @@ import numpy as np
 ROOT = os.path.dirname(os.path.abspath(__file__))
 sys.path.insert(0, ROOT)
 
-MEASURED_FUSED_TRAFFIC_BYTES = 709.9e6  # 323.5 MiB fetched + 351.6 MiB written per launch
 HBM_PEAK = 8.0e12  # bytes/s, MI355X
+TRAFFIC_PROFILE = os.path.join(ROOT, "profiles", "hbm_traffic_config2_10.5Mx28_depth8.txt")
+KERNEL_SOURCES = ["kernels_partition.h", "kernels_hist.h", "device_common.h"]
+
+
+def kernel_source_digest():
+    """sha1 over the sources of the dominant kernel: a profile applies to exactly one version of them."""
+    import hashlib
+    h = hashlib.sha1()
+    for name in KERNEL_SOURCES:
+        with open(os.path.join(ROOT, "arboretum_amd", "csrc", name), "rb") as f:
+            h.update(f.read())
+    return h.hexdigest()
+
+
+def profiled_traffic():
+    """HBM bytes per launch of the fused pass from the committed counter profile (FETCH_SIZE +
+    WRITE_SIZE of two rocprofv3 --pmc runs), or None when the profile was taken on other kernel
+    sources than the ones in the tree."""
+    try:
+        text = open(TRAFFIC_PROFILE).read()
+    except OSError:
+        return None
+    digest, value = None, None
+    for line in text.splitlines():
+        if line.startswith("kernel_source_sha1:"):
+            digest = line.split(":", 1)[1].strip()
+        if line.startswith("fused_pass_hbm_bytes_per_launch:"):
+            value = float(line.split(":", 1)[1].strip())
+    return value if digest == kernel_source_digest() else None
 
 
 def make_workload(rows, features=28, seed=0):
@@ -194,13 +229,14 @@ def main():
     # every fourth tree; the phase breakdown comes from a few more trees grown afterwards with
     # every phase bracketed (about 35 event records per tree, which costs 5 % of the tree time).
     model.enable_timing(3)
-    scanned0 = model.rows_scanned()
+    levels0 = model.rows_scanned_by_level().astype(np.int64)
     t0 = time.perf_counter()
     for _ in range(args.steps):
         model.grow_tree()
     model.synchronize()
     dt = time.perf_counter() - t0
-    scanned = model.rows_scanned() - scanned0
+    by_level = model.rows_scanned_by_level().astype(np.int64) - levels0   # rows accumulated per tree level
+    scanned = int(by_level.sum())
     tm_dominant = model.timings()
     phase_trees = min(args.steps, 10)
     model.enable_timing(1)
@@ -213,60 +249,58 @@ def main():
     tm = {k: tm_after[k] - tm_dominant[k] for k in tm_after}
     fused_ms_timed, fused_launches_timed = tm_dominant["hist_deep_ms"], tm_dominant["hist_deep_launches"]
 
-    F = args.features
+    F, R, D = args.features, args.rows, args.max_depth
     updates = scanned * F
-    row_bytes = F + 8  # uint8 bins of all features + one (g, h) pair: the algorithmic figure
-    # what the kernels move: with 0/1 labels (this workload) the pair travels as one float
-    moved_row_bytes = F + 4
-    cell_bytes = 16    # one histogram cell as written by a workgroup (two 64-bit words)
+    PAIR_BYTES = 8        # one (g, h) float pair per row
+    PART_BYTES = 9        # partition of a level: 4 (index read) + 1 (row's node) + 4 (index written) per row
+    CELL_BYTES = 20       # one histogram entry written: two 8-byte sums and a 4-byte count
+    row_bytes = F + PAIR_BYTES
     # Dominant kernel: the fused partition + histogram pass of levels 1..max_depth-2
-    # (k_part_hist<true, 7, true, false, true>).  Algorithmic bytes of one launch: every row is
-    # read once and written once in the children order, and the smaller child of
-    # each parent gets one histogram written.
+    # (k_part_hist<true, 7, true, false, true>), one launch per level over all rows.
+    fused_levels = list(range(1, max(D - 1, 1)))
     fl = max(fused_launches_timed, 1)
-    # parents whose smaller child got a histogram in the measured launches (levels 1..max_depth-2
-    # of the sampled trees)
-    launches_per_tree = max(args.max_depth - 2, 1)
-    parents = sum(1 << (l - 1) for l in range(1, args.max_depth - 1)) * fl / launches_per_tree
-    fused_bytes = fl * args.rows * 2 * row_bytes + parents * F * 256 * cell_bytes
-    fused_s = fused_ms_timed * 1e-3
-    achieved = fused_bytes / fused_s if fused_s > 0 else 0.0
-    # root level (k_hist<true, 7>): reads every row, writes one histogram
-    root_bytes = tm["hist_root_rows"] * row_bytes + phase_trees * F * 256 * cell_bytes
-    root_s = tm["hist_root_ms"] * 1e-3
-    # last level (k_part_hist<true, 7, false, false, true>): moves no rows; reads the split feature's quad
-    # of every row and then the rows of the smaller children, which are spread over nearly every
-    # 32-byte sector: counted as one full read of the rows (the counters show 387 MiB fetched)
-    last_bytes = tm["fused_last_launches"] * args.rows * row_bytes
-    last_s = tm["fused_last_ms"] * 1e-3
-
-    # HBM bytes per launch of the dominant kernel from hardware counters: two rocprofv3 --pmc
-    # runs of this file (FETCH_SIZE, WRITE_SIZE), scaled by the same counters over a copy of
-    # known size (--copy-probe); summary and commands in profiles/hbm_traffic_config2_*.txt.
-    # Only known for the default workload.
-    default_workload = (args.rows, F, args.hist_size, args.max_depth) == (10500000, 28, 256, 8)
-    traffic = MEASURED_FUSED_TRAFFIC_BYTES if default_workload else None
+    # rows accumulated and nodes built per launch, averaged over the levels of the timed trees
+    scanned_per_launch = float(by_level[fused_levels].sum()) / (len(fused_levels) * args.steps) if fused_levels else 0.0
+    built_per_launch = sum(1 << (l - 1) for l in fused_levels) / max(len(fused_levels), 1)
+    algo_bytes = scanned_per_launch * row_bytes + R * PART_BYTES + built_per_launch * F * 256 * CELL_BYTES
+    fused_s = fused_ms_timed * 1e-3 / fl            # average duration of one launch
+    achieved = algo_bytes / fused_s if fused_s > 0 else 0.0
+    # what this implementation moves per launch: every row read and written (bins + the gradient
+    # pair, which travels as one float with 0/1 labels), the split quad read once more by the
+    # left-row count, one 16-byte-per-cell slab per work item (about 250)
+    moved_row_bytes = F + 4
+    moved_bytes = R * (2 * moved_row_bytes + 4) + 250 * 8192 * 16
+    traffic = profiled_traffic() if (R, F, args.hist_size, D) == (10500000, 28, 256, 8) else None
 
     def frac(b, t):
         return (b / t) / HBM_PEAK if t > 0 else 0.0
 
-    other = {"k_part_hist<true,7,false,false,true> (last level)": {
-        "frac_of_hbm": frac(last_bytes, last_s),
-        "avg_launch_us": tm["fused_last_ms"] * 1e3 / max(tm["fused_last_launches"], 1)}}
+    # the other row passes, by the same accounting
+    last_scanned = float(by_level[D - 1]) / args.steps if D >= 2 else 0.0
+    last_bytes = last_scanned * row_bytes + R * PART_BYTES + (1 << max(D - 2, 0)) * F * 256 * CELL_BYTES
+    last_s = tm["fused_last_ms"] * 1e-3 / max(tm["fused_last_launches"], 1)
+    other = {"k_part_hist<true,7,false,false,true> (last level, moves no rows)": {
+        "frac_of_hbm": frac(last_bytes, last_s), "avg_launch_us": last_s * 1e6,
+        "updates_per_s": last_scanned * F / last_s if last_s > 0 else 0.0}}
     if tm["hist_root_launches"] > 0:
+        root_s = tm["hist_root_ms"] * 1e-3 / tm["hist_root_launches"]
         other["k_hist<true,7> (root level)"] = {
-            "frac_of_hbm": frac(root_bytes, root_s),
-            "avg_launch_us": tm["hist_root_ms"] * 1e3 / tm["hist_root_launches"],
-            "updates_per_s": tm["hist_root_rows"] * F / root_s if root_s > 0 else 0.0}
+            "frac_of_hbm": frac(R * row_bytes + F * 256 * CELL_BYTES, root_s), "avg_launch_us": root_s * 1e6,
+            "updates_per_s": R * F / root_s if root_s > 0 else 0.0}
     else:
-        # the last pass of a tree (leaf of every row, prediction update, next gradients)
-        # also builds the root histogram of the next tree: rows read once (bins, y_hat, y),
-        # leaf id, y_hat, g, h written
-        final_bytes = phase_trees * (args.rows * (F + 8 + 16) + F * 256 * cell_bytes * 256)
-        other["k_final_hist<7> (last pass of a tree + root histogram of the next)"] = {
-            "frac_of_hbm": frac(final_bytes, tm["leaf_ms"] * 1e-3),
-            "avg_launch_us": tm["leaf_ms"] * 1e3 / phase_trees,
-            "updates_per_s": phase_trees * args.rows * F / (tm["leaf_ms"] * 1e-3) if tm["leaf_ms"] > 0 else 0.0}
+        # the last pass of a tree (leaf of every row, prediction update R x 10, next gradients
+        # R x 16) also builds the root histogram of the next tree (R x (F + 8))
+        final_s = tm["leaf_ms"] * 1e-3 / phase_trees
+        other["k_final_hist<7> (prediction update + gradients + root histogram of the next tree)"] = {
+            "frac_of_hbm": frac(R * (row_bytes + 10 + 16) + F * 256 * CELL_BYTES, final_s),
+            "avg_launch_us": final_s * 1e6,
+            "updates_per_s": R * F / final_s if final_s > 0 else 0.0}
+    # whole tree by the same accounting: histogram build of every level, partition of every
+    # split level, gradient pass, prediction update
+    sec_per_tree = dt / args.steps
+    nodes_built = 1 + sum(1 << (l - 1) for l in range(1, D))
+    tree_bytes = (scanned / args.steps) * row_bytes + nodes_built * F * 256 * CELL_BYTES + D * R * PART_BYTES \
+        + R * 16 + R * 10
 
     out = {
         "metric": "row*feature hist updates/s + sec/tree at 10M x 28 depth 8; % of HBM peak",
@@ -275,8 +309,8 @@ def main():
         "n_gpus": 1,
         "steps": args.steps,
         "warmup": args.warmup,
-        "ms_per_step": dt / args.steps * 1e3,
-        "sec_per_tree": dt / args.steps,
+        "ms_per_step": sec_per_tree * 1e3,
+        "sec_per_tree": sec_per_tree,
         "higher_is_better": True,
         "scaling": "weak",
         "vs_baseline": None,
@@ -284,21 +318,28 @@ def main():
         "data": "synthetic",
         "config": {"workload": "binary classification %d rows x %d dense fp32 features (BASELINE configs[1]), "
                                "%d bins, max_depth %d, logistic, eta 0.1, lambda 1, min_child_weight 1"
-                               % (args.rows, F, args.hist_size, args.max_depth),
-                   "rows": args.rows, "features": F, "bins": args.hist_size, "max_depth": args.max_depth},
+                               % (R, F, args.hist_size, D),
+                   "rows": R, "features": F, "bins": args.hist_size, "max_depth": D},
         "roofline": {"bound": "hbm", "achieved": achieved / 1e9, "peak": HBM_PEAK / 1e9, "unit": "GB/s",
                      "frac": achieved / HBM_PEAK, "traffic": traffic,
                      "kernel": "k_part_hist<true,7,true,false,true> (fused partition + histogram, levels 1..%d)"
-                               % (args.max_depth - 2),
+                               % (D - 2),
                      "launches": int(fused_launches_timed),
-                     "avg_launch_us": fused_ms_timed * 1e3 / fl,
-                     "bytes_per_launch": fused_bytes / fl,
-                     # (g, h) packed in 4 bytes: bytes the kernel needs to move per launch
-                     "bytes_moved_per_launch": (fused_bytes - fl * args.rows * 2 * (row_bytes - moved_row_bytes)) / fl},
+                     "avg_launch_us": fused_s * 1e6,
+                     "bytes_per_launch": algo_bytes,
+                     "rows_scanned_per_launch": scanned_per_launch,
+                     # bytes this implementation moves (rows re-ordered physically) and the rate / share of
+                     # the HBM peak that movement runs at
+                     "moved_bytes_per_launch": moved_bytes,
+                     "moved_frac": frac(moved_bytes, fused_s),
+                     "traffic_over_algorithmic": traffic / algo_bytes if traffic else None,
+                     "traffic_source": "profiles/" + os.path.basename(TRAFFIC_PROFILE) if traffic else None},
         "other_kernels": other,
-        "tree_algorithmic_floor_frac_of_hbm": (2.9e9 / (dt / args.steps)) / HBM_PEAK,
+        "tree_algorithmic_bytes": tree_bytes,
+        "tree_algorithmic_floor_frac_of_hbm": (tree_bytes / sec_per_tree) / HBM_PEAK,
+        "rows_scanned_per_tree_by_level": [float(v) / args.steps for v in by_level[:D]],
         "phase_ms_per_tree": dict({k: v / phase_trees for k, v in tm.items() if k.endswith("_ms")},
-                                  hist_deep_ms=fused_ms_timed / (fl / launches_per_tree)),
+                                  hist_deep_ms=fused_ms_timed / (fl / max(len(fused_levels), 1))),
         "phase_trees": phase_trees,
         "quantise_s": t_quant,
     }

@@ -90,6 +90,9 @@ const char *AGardenEnableTiming(VoidPointer garden, int on);
 const char *AGardenGetTimings(VoidPointer garden, double *out);
 /* Rows accumulated into histograms so far (x ncol = histogram updates). */
 const char *AGardenRowsScanned(VoidPointer garden, unsigned long long *out);
+/* The same per tree level: out[32], out[l] = rows accumulated at level l (the
+ * root is level 0; levels past 31 share the last entry). */
+const char *AGardenRowsScannedByLevel(VoidPointer garden, unsigned long long *out);
 /* Waits for all device work of the booster. */
 const char *AGardenSynchronize(VoidPointer garden);
 
