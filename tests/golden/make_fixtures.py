@@ -87,6 +87,24 @@ def main():
                "X": X, "target": t, "config": _config_of(log), "cases": _calls(log)},
               open(os.path.join(HERE, "hist_logistic_iris.json"), "w"))
 
+    # ---- sklearn-style classifier golden, tests/py/test_sklearn_classification.py:9-61: the default
+    # value of the test's `y_pred` argument and the keyword arguments of its ArboretumClassifier(...)
+    cls = os.path.join(REF, "tests/py/test_sklearn_classification.py")
+    tree = ast.parse(open(cls).read())
+    fn = next(f for f in tree.body if isinstance(f, ast.FunctionDef) and f.name == "test_single_tree")
+    y_pred = ast.literal_eval(fn.args.defaults[-1])[0]
+    call = next(n for n in ast.walk(fn) if isinstance(n, ast.Call) and getattr(n.func, "attr", "") == "ArboretumClassifier")
+    params = {}
+    for kw in call.keywords:
+        params[kw.arg] = "$" + kw.value.id if isinstance(kw.value, ast.Name) else ast.literal_eval(kw.value)
+    sweep = {}
+    for dec in fn.decorator_list:  # @pytest.mark.parametrize("name", [values])
+        sweep[ast.literal_eval(dec.args[0])] = ast.literal_eval(dec.args[1])
+    Xi, ti = iris()
+    json.dump({"source": "tests/py/test_sklearn_classification.py:9-61", "X": Xi, "target": ti,
+               "label_rule": "target != 2", "params": params, "sweep": sweep, "y_pred": y_pred},
+              open(os.path.join(HERE, "sklearn_classification_iris.json"), "w"))
+
     # ---- quantiser goldens, tests/cpp/test_datamatrix.cu
     q = []
     q.append({"name": "HistWideRange", "cite": "tests/cpp/test_datamatrix.cu:25-46", "hist_size": 8,
