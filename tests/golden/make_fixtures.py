@@ -133,7 +133,13 @@ def main():
                    "h": [1.0] * 32, "best_bin": 1, "gain": 2048.0}]})
     # :123-259 level 1: node 0 = positions 0..15 (bin p/2), node 1 = positions
     # 16..31 (bin 7-(p-16)/2), grad (p*p,1): best global idx 4 and 11
-    g.append({"name": "Level1Search", "cite": "tests/cpp/test_hist.cu:123-259", "hist_size": 8,
+    # the same sums, best bins and gains are asserted by every Level1Search variant of the file
+    # (NoTrickDynamic :123, _Upload :262, NoTrickStatic :594, WithTrickDynamic :702, WithTrickStatic
+    # :811): they differ in how the reference gets there (launch mode, streaming, subtraction)
+    g.append({"name": "Level1Search", "cite": "tests/cpp/test_hist.cu:123-259",
+              "same_numbers_in": ["tests/cpp/test_hist.cu:262-400", "tests/cpp/test_hist.cu:594-700",
+                                  "tests/cpp/test_hist.cu:702-809", "tests/cpp/test_hist.cu:811-921"],
+              "hist_size": 8,
               "params": [0, 0, 0, 0, 0, 0], "nodes": [
                   {"bins": [p // 2 for p in range(16)], "g": [float(p * p) for p in range(16)],
                    "h": [1.0] * 16, "best_bin": 4, "gain": 64026.672,
