@@ -139,7 +139,7 @@ void Garden::FromInternal(const float *in, size_t count, float *out) const {
 }
 
 void Garden::GrowTree(DataMatrix *data, const float *grad) {
-  if (cfg.method != kHist) throw std::runtime_error("only method 1 (hist) is implemented");
+  if (cfg.method != kHist && cfg.method != kExact) throw std::runtime_error("unknown method");
   if (grad != nullptr) throw std::runtime_error("user-supplied gradients are not supported");
   if (cfg.objective >= kSoftMaxOneVsAll) {
     if (data->labels.size() != data->rows) throw std::runtime_error("labels are not set");
@@ -169,7 +169,7 @@ void Garden::GrowTree(DataMatrix *data, const float *grad) {
     // upload_features = false keeps the bins in pinned host memory and streams
     // them (src/core/garden.cu:603-604, hist_tree_grower.cu:335-366)
     QuantiseOnDevice(data, cfg.internal.hist_size, cfg.verbose.data, !cfg.internal.upload_features,
-                     cfg.internal.stream_block_rows);
+                     cfg.internal.stream_block_rows, cfg.method == kExact);
     builder_.reset(CreateTreeBuilder(cfg, data));
     builder_->SetInspect(inspect_);
     builder_->EnableTiming(timing_);

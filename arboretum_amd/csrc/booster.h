@@ -48,7 +48,8 @@ class DataMatrix {
   // Quantiser output (io.h:24, 32): thresholds[f] has hist_size entries,
   // reduced_size[f] real bins.
   bool quantised = false;
-  int hist_size = 0;
+  bool quantised_exact = false;  // bin ids are ranks among the distinct values (exact method)
+  int hist_size = 0;             // exact method: the largest number of distinct values of a feature
   std::vector<std::vector<float>> thresholds;
   std::vector<int> reduced_size;
   DeviceMatrix *device = nullptr;
@@ -131,8 +132,10 @@ void DeviceThresholds(SortWorkspace *ws, const float *d_col, std::vector<float> 
 // device_builder.hip
 // streamed = false: bins resident in HBM; true: bins in pinned host blocks of
 // block_rows rows, copied to the GPU block by block at every tree level.
+// exact: no quantisation, every distinct value of a feature is a bin (the exact method;
+// at most 4096 distinct values per feature).
 void QuantiseOnDevice(DataMatrix *data, int hist_size, bool verbose, bool streamed = false,
-                      size_t block_rows = 0);
+                      size_t block_rows = 0, bool exact = false);
 void FreeDeviceMatrix(DeviceMatrix *m);
 void GetDeviceBins(const DataMatrix &data, uint8_t *out);  // row-major [rows][F], 8-bit bins
 void GetDeviceBins16(const DataMatrix &data, uint16_t *out);  // row-major [rows][F], 16-bit bins

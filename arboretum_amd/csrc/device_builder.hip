@@ -116,11 +116,59 @@ void FreeDeviceMatrix(DeviceMatrix *m) {
   delete m;
 }
 
-void QuantiseOnDevice(DataMatrix *data, int hist_size, bool verbose, bool streamed, size_t block_rows) {
+// Exact method (DataMatrix::InitExact, src/io/io.cu:437-482): every value becomes its rank
+// among the sorted distinct values of its column.  Returns the ranks row-major [rows][F] and
+// fills data->thresholds / reduced_size: the split "ranks <= q left" separates at the value
+// of rank q + 1 (the smallest value that goes right, src/core/garden.cu:463-467).
+static std::vector<uint16_t> ExactRanks(DataMatrix *data, size_t *most_distinct) {
+  const size_t n = data->rows;
+  const int F = (int)data->columns_dense;
+  std::vector<uint16_t> ranks(n * F);
+  std::vector<std::vector<float>> mapping(F);
+  std::atomic<bool> has_nan{false};
+  std::atomic<int> too_many{-1};
+  ParallelFor((size_t)F, [&](size_t fb, size_t fe) {
+    for (size_t f = fb; f < fe; ++f) {
+      std::vector<float> m(data->data[f]);
+      for (float v : m)
+        if (v != v) has_nan = true;
+      if (has_nan) return;
+      std::sort(m.begin(), m.end());
+      m.erase(std::unique(m.begin(), m.end()), m.end());
+      if (m.size() > (size_t)kMaxWideSlots) {
+        too_many = (int)f;
+        return;
+      }
+      const float *col = data->data[f].data();
+      for (size_t i = 0; i < n; ++i)
+        ranks[i * F + f] = (uint16_t)(std::lower_bound(m.begin(), m.end(), col[i]) - m.begin());
+      mapping[f].swap(m);
+    }
+  });
+  if (has_nan) throw std::runtime_error("the exact method does not take missing values (NaN); use method 1 (hist)");
+  if (too_many >= 0)
+    throw std::runtime_error("the exact method handles up to " + std::to_string(kMaxWideSlots) +
+                             " distinct values per feature; feature " + std::to_string((int)too_many) +
+                             " has more: use method 1 (hist)");
+  size_t most = 1;
+  for (int f = 0; f < F; ++f) most = std::max(most, mapping[f].size());
+  *most_distinct = most;
+  for (int f = 0; f < F; ++f) {
+    data->reduced_size[f] = (int)mapping[f].size();
+    data->thresholds[f].assign(most, std::numeric_limits<float>::infinity());
+    for (size_t k = 0; k + 1 < mapping[f].size(); ++k) data->thresholds[f][k] = mapping[f][k + 1];
+  }
+  return ranks;
+}
+
+void QuantiseOnDevice(DataMatrix *data, int hist_size, bool verbose, bool streamed, size_t block_rows, bool exact) {
   if (data->quantised) {
-    if (data->hist_size != hist_size) throw std::runtime_error("data matrix was quantised with another hist_size");
+    if (data->quantised_exact != exact) throw std::runtime_error("data matrix was prepared for the other method");
+    if (!exact && data->hist_size != hist_size) throw std::runtime_error("data matrix was quantised with another hist_size");
     return;
   }
+  if (exact && data->is_prebinned) throw std::runtime_error("the exact method needs float features, not bin ids");
+  if (exact) hist_size = 1;  // set below from the data
   if (hist_size < 1) throw std::runtime_error("hist_size must be positive");
   const size_t n = data->rows;
   const int F = (int)data->columns_dense;
@@ -160,8 +208,35 @@ void QuantiseOnDevice(DataMatrix *data, int hist_size, bool verbose, bool stream
   data->thresholds.assign(F, {});
   data->reduced_size.assign(F, 0);
 
-  if (data->is_prebinned) {
-    for (int f = 0; f < F; ++f) {
+  if (exact) {
+    size_t most = 1;
+    std::vector<uint16_t> ranks = ExactRanks(data, &most);
+    hist_size = (int)most;
+    if (most <= (size_t)kSlots) {
+      // 8-bit ids: through the pre-quantised path below
+      data->prebinned.resize(n * F);
+      for (size_t i = 0; i < n * F; ++i) data->prebinned[i] = (uint8_t)ranks[i];
+    } else {
+      if (streamed) throw std::runtime_error("a feature has more than 256 distinct values: 16-bit ids are not built for streamed matrices");
+      int slots = kSlots;
+      while ((size_t)slots < most) slots *= 2;
+      dm->bits = 16;
+      dm->slots = slots;
+      dm->Q = (F + 1) / 2;
+      HIP_OK(hipFree(dm->bins));
+      dm->bins = DevAlloc<uint32_t>((size_t)dm->Q * dm->stride);
+      uint16_t *d_in = DevAlloc<uint16_t>(n * F);
+      HIP_OK(hipMemcpy(d_in, ranks.data(), n * F * sizeof(uint16_t), hipMemcpyHostToDevice));
+      hipLaunchKernelGGL(k_pack_prebinned16, dim3(GridFor(n, 256)), dim3(256), 0, 0, d_in, F, dm->Q, dm->bins,
+                         dm->stride, n);
+      HIP_OK(hipDeviceSynchronize());
+      HIP_OK(hipFree(d_in));
+    }
+  }
+  if (exact && dm->bits == 16) {
+    // done above
+  } else if (data->is_prebinned || exact) {
+    for (int f = 0; f < F && !exact; ++f) {
       data->thresholds[f].resize(hist_size);
       for (int k = 0; k < hist_size; ++k) data->thresholds[f][k] = (float)k + 0.5f;
       data->reduced_size[f] = std::min(hist_size, kSlots);
@@ -270,9 +345,11 @@ void QuantiseOnDevice(DataMatrix *data, int hist_size, bool verbose, bool stream
     data->stream_blocks = dm->host_blocks;
     data->stream_block_rows = block_rows;
   }
+  if (exact) std::vector<uint8_t>().swap(data->prebinned);  // prediction walks the float columns
   data->device = dm.release();
   data->hist_size = hist_size;
   data->quantised = true;
+  data->quantised_exact = exact;
 }
 
 void GetBinLayout(const DataMatrix &data, int *bits, int *slots) {
@@ -954,7 +1031,7 @@ class HipTreeBuilder : public TreeBuilder {
   // plan_next: also plan the fused pass of the next level over these nodes
   void LaunchSplit(int level, int L, int hb, int state, const GainParams &gp, bool plan_next = false) {
     Mark(kSplit);
-    const int hs = std::min(cfg_.internal.hist_size, slots_);
+    const int hs = std::min(data_->hist_size, slots_);  // data_->hist_size: the configuration's, or the distinct values (exact method)
     const unsigned char *active = sampling_ ? d_active_ + (size_t)level * F_ : (const unsigned char *)nullptr;
     const unsigned per_item = FusedRowsPerItem(L);
     // From 32 nodes on, one launch: a workgroup per node scans its features and

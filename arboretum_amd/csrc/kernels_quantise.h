@@ -93,6 +93,19 @@ __global__ void k_pack_prebinned(const uint8_t *__restrict__ in, int F, int Q,
   }
 }
 
+// row-major uint16 [n][F] -> words of two 16-bit ids
+__global__ void k_pack_prebinned16(const uint16_t *__restrict__ in, int F, int Q,
+                                   uint32_t *__restrict__ out, size_t stride, size_t n) {
+  for (size_t r = (size_t)blockIdx.x * blockDim.x + threadIdx.x; r < n;
+       r += (size_t)gridDim.x * blockDim.x) {
+    for (int q = 0; q < Q; ++q) {
+      uint32_t packed = in[r * F + 2 * q];
+      if (2 * q + 1 < F) packed |= (uint32_t)in[r * F + 2 * q + 1] << 16;
+      out[(size_t)q * stride + r] = packed;
+    }
+  }
+}
+
 }  // namespace
 }  // namespace arb
 #endif  // ARBORETUM_AMD_KERNELS_QUANTISE_H_

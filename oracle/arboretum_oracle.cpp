@@ -81,6 +81,7 @@ struct OrcParams {
   float colsample_bytree;
   float colsample_bylevel;
   unsigned seed;
+  int method;             // 1 = hist, 0 = exact (param.h:16)
 };
 
 // ------------------------------------------------------------------- exp
@@ -820,6 +821,46 @@ void *orc_create(const float *X, int64_t n, int F, const float *y, const uint8_t
   b->thr.resize(F);
   b->size.resize(F);
   b->bins.resize((size_t)n * F);
+  if (p->method == 0) {
+    // Exact method.  DataMatrix::InitExact (src/io/io.cu:437-482): every value is replaced by its
+    // rank among the column's sorted distinct values (`data_reduced_mapping`).  The grower
+    // (src/core/continuous_tree_grower.cu:9-49) sorts each node's rows by rank, takes the
+    // exclusive prefix sum of the gradients and evaluates gain_func at every position i where the
+    // rank changes (left = the rows before i), keeping the best gain and, on equal gains, the
+    // highest position (updateAtomicMax packs (gain, i)); the split value is the rank r at that
+    // position, rows with rank >= r go right (builder.h:107-123) and the node's threshold is
+    // mapping[r] (garden.cu:463-467).  Left of position i are exactly the rows of rank < r, so
+    // the candidates are the prefixes of a histogram over ranks: slot q = r - 1 with "bins <= q
+    // left", ties to the highest slot.  That is the histogram scan below with one slot per
+    // distinct value and thresholds thr[q] = mapping[q + 1].
+    std::vector<std::vector<float>> mapping(F);
+    size_t most = 1;
+    for (int f = 0; f < F; ++f) {
+      std::vector<float> &m = mapping[f];
+      m.resize(n);
+      for (int64_t i = 0; i < n; ++i) m[i] = X[(size_t)i * F + f];
+      std::sort(m.begin(), m.end());
+      m.erase(std::unique(m.begin(), m.end()), m.end());
+      most = std::max(most, m.size());
+      for (int64_t i = 0; i < n; ++i)
+        b->bins[(size_t)i * F + f] =
+            (uint16_t)(std::lower_bound(m.begin(), m.end(), X[(size_t)i * F + f]) - m.begin());
+    }
+    if (most > 65535) {
+      delete b;
+      return nullptr;
+    }
+    b->p.hist_size = (int)most;
+    b->slots = (int)most + 1;
+    for (int f = 0; f < F; ++f) {
+      b->size[f] = (int)mapping[f].size();
+      b->thr[f].assign(most, std::numeric_limits<float>::infinity());
+      for (size_t k = 0; k + 1 < mapping[f].size(); ++k) b->thr[f][k] = mapping[f][k + 1];
+    }
+    b->yhat.assign((size_t)n * p->labels_count, into_internal(p->objective, p->initial_y));
+    b->rnd.seed(p->seed);
+    return b;
+  }
   // the columns are independent (io.cu:349-435 handles them one after the other)
 #pragma omp parallel for schedule(dynamic, 1) num_threads(p->threads > 0 ? p->threads : omp_get_max_threads())
   for (int f = 0; f < F; ++f) {
@@ -866,6 +907,7 @@ void orc_grow_round(void *hd) {
   for (int k = 0; k < b.p.labels_count; ++k) grow_tree(b, k);
 }
 
+int orc_hist_size(void *hd) { return static_cast<Booster *>(hd)->p.hist_size; }  // exact: distinct values
 int orc_num_trees(void *hd) { return (int)static_cast<Booster *>(hd)->trees.size(); }
 uint64_t orc_updates(void *hd) { return static_cast<Booster *>(hd)->updates; }
 

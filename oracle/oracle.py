@@ -32,6 +32,7 @@ class OrcParams(ctypes.Structure):
         ("colsample_bytree", ctypes.c_float),
         ("colsample_bylevel", ctypes.c_float),
         ("seed", ctypes.c_uint),
+        ("method", ctypes.c_int),
     ]
 
 
@@ -82,6 +83,7 @@ def lib():
         L.orc_create_binned.argtypes = L.orc_create.argtypes
         L.orc_free.argtypes = [ctypes.c_void_p]
         L.orc_grow_round.argtypes = [ctypes.c_void_p]
+        L.orc_hist_size.argtypes = [ctypes.c_void_p]
         L.orc_num_trees.argtypes = [ctypes.c_void_p]
         L.orc_updates.restype = ctypes.c_uint64
         L.orc_updates.argtypes = [ctypes.c_void_p]
@@ -131,6 +133,7 @@ def params_from_config(config, accum=0, threads=0):
         colsample_bytree=float(t.get("colsample_bytree", 1.0)),
         colsample_bylevel=float(t.get("colsample_bylevel", 1.0)),
         seed=int(it.get("seed", 0)),
+        method=int(config.get("method", 1)),
     )
 
 
@@ -168,7 +171,10 @@ class Booster:
             X = np.ascontiguousarray(X, dtype=np.float32)
             self.h = lib().orc_create(_p(X), self.n, self.F, _p(y), _p(labels),
                                       ctypes.byref(self.params))
+        if not self.h:
+            raise ValueError("the checker's exact mode holds at most 65535 distinct values per feature")
         self.K = self.params.labels_count
+        self.params.hist_size = lib().orc_hist_size(self.h)   # exact method: the largest number of distinct values
 
     def __del__(self):
         if getattr(self, "h", None):

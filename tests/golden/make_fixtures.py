@@ -87,6 +87,18 @@ def main():
                "X": X, "target": t, "config": _config_of(log), "cases": _calls(log)},
               open(os.path.join(HERE, "hist_logistic_iris.json"), "w"))
 
+    # ---- exact-method goldens (method 0), tests/py/test_regression.py and test_logresression.py
+    ereg = os.path.join(REF, "tests/py/test_regression.py")
+    elog = os.path.join(REF, "tests/py/test_logresression.py")
+    X, y = boston10()
+    json.dump({"source": "tests/py/test_regression.py:14-53 (config), :56-91 (cases)",
+               "X": X, "y": y, "config": _config_of(ereg), "cases": _calls(ereg)},
+              open(os.path.join(HERE, "exact_regression_boston10.json"), "w"))
+    X, t = iris()
+    json.dump({"source": "tests/py/test_logresression.py:9-43 (config), :46-135 (cases)",
+               "X": X, "target": t, "config": _config_of(elog), "cases": _calls(elog)},
+              open(os.path.join(HERE, "exact_logistic_iris.json"), "w"))
+
     # ---- sklearn-style classifier golden, tests/py/test_sklearn_classification.py:9-61: the default
     # value of the test's `y_pred` argument and the keyword arguments of its ArboretumClassifier(...)
     cls = os.path.join(REF, "tests/py/test_sklearn_classification.py")

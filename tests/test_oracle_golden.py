@@ -169,15 +169,79 @@ def _run_cases(oracle, fixture, X, y):
                                       upload_features=upload, depth=case["max_depth"])
                 b = oracle.Booster(X, y=y, config=cfg, accum=accum)
                 b.grow(case["trees"])
-                for i in range(case["trees"]):
-                    pred = b.predict(X, i + 1)
-                    assert np.allclose(pred, case["true_values"][i]), (name, dp, trick, accum, i)
+                if isinstance(case["true_values"][0], list):   # predictions after every tree
+                    for i in range(case["trees"]):
+                        pred = b.predict(X, i + 1)
+                        assert np.allclose(pred, case["true_values"][i]), (name, dp, trick, accum, i)
+                else:                                           # predictions of the whole model
+                    assert np.allclose(b.predict(X), case["true_values"]), (name, dp, trick, accum)
                 model = b.model_dict()
                 true = case["true_model"]["model"]
                 assert len(true) == len(model["model"])
                 for tt, ct in zip(true, model["model"]):
                     assert np.allclose(tt["weights"], ct["weights"], rtol=1e-4, atol=1e-6), name
                     assert tt["nodes"] == ct["nodes"], (name, dp, trick, accum)
+
+
+def test_golden_exact_regression_boston(oracle):
+    # method 0 (exact): tests/py/test_regression.py of the reference
+    fx = load_golden("exact_regression_boston10.json")
+    _run_cases(oracle, fx, np.array(fx["X"], np.float32), np.array(fx["y"], np.float32))
+
+
+def test_golden_exact_logistic_iris(oracle):
+    # method 0 (exact): tests/py/test_logresression.py of the reference
+    fx = load_golden("exact_logistic_iris.json")
+    _run_cases(oracle, fx, np.array(fx["X"], np.float32), (np.array(fx["target"]) != 2).astype(np.float32))
+
+
+def _brute_force_exact_root(oracle, X, g, h, kind, params):
+    """The reference's exact split search (continuous_tree_grower.cu:9-49) on one node, in plain
+    Python: per feature sort the rows by value, exclusive prefix sums, the gain at every position
+    where the value changes, best gain with ties to the highest position, then to the lowest
+    feature.  Returns (feature, threshold value, gain)."""
+    mls, mcw, ga, gr, lam, alpha = params
+    n, F = X.shape
+    GT, HT = float(np.sum(g.astype(np.float64))), float(np.sum(h.astype(np.float64)))
+    best = (-1, None, 0.0)
+    for f in range(F):
+        order = np.argsort(X[:, f], kind="stable")
+        xs, gs, hs = X[order, f], g[order].astype(np.float64), h[order].astype(np.float64)
+        cg, ci = 0.0, -1
+        for i in range(1, n):
+            if xs[i] != xs[i - 1]:
+                gain = oracle.lib().orc_gain(kind, float(gs[:i].sum()), float(hs[:i].sum()), i, GT, HT, n, mls,
+                                             mcw, ga, gr, lam, alpha, 0.0)
+                if gain > 0 and gain >= cg:
+                    cg, ci = gain, i
+        if ci >= 0 and (best[0] < 0 or cg > best[2]):
+            best = (f, float(xs[ci]), cg)
+    return best
+
+
+@pytest.mark.parametrize("objective", [0, 1])
+@pytest.mark.parametrize("seed", range(6))
+def test_exact_root_split_against_brute_force(oracle, objective, seed):
+    rng = np.random.default_rng(100 + seed)
+    n, F = 60, 4
+    X = np.round(rng.normal(size=(n, F)) * 3).astype(np.float32) / 2      # many repeated values
+    X[:, 1] = rng.normal(size=n).astype(np.float32)                       # and one all-distinct column
+    y = (X[:, 0] + X[:, 1] > 0).astype(np.float32) if objective else (X[:, 0] * 2 + rng.normal(size=n)).astype(np.float32)
+    cfg = {"objective": objective, "method": 0, "internals": {"double_precision": True},
+           "tree": {"max_depth": 1, "eta": 1.0, "lambda": 0.5, "min_child_weight": 0.0, "min_leaf_size": 1,
+                    "initial_y": 0.5}}
+    b = oracle.Booster(X, y=y, config=cfg, accum=1)
+    b.grow(1)
+    g, h = b.grad()
+    if objective == 0:
+        h = np.ones_like(g)
+    f, thr, gain = _brute_force_exact_root(oracle, X, g, h, 1 if objective == 0 else 3, (1, 0.0, 0.0, 0.0, 0.5, 0.0))
+    t = b.tree(0)
+    assert f >= 0 and t["fid"][0] == f
+    assert t["threshold"][0] == np.float32(thr)           # the smallest value that goes right
+    assert t["gain"][0] == pytest.approx(gain, rel=1e-6)
+    # the rows: value < threshold left, as prediction walks them
+    assert np.array_equal(b.leaf(), (X[:, f] >= thr).astype(np.uint32))
 
 
 def test_golden_regression_boston(oracle):
