@@ -43,6 +43,7 @@ def _load_lib():
         "ADeviceCount": [P(c_int)],
         "ADeviceCopyProbe": [ctypes.c_ulonglong],
         "ACreateFromQuantized": [c_void_p, ctypes.c_longlong, c_int, P(c_void_p)],
+        "ACreateFromQuantizedBlocks": [c_void_p, c_int, ctypes.c_longlong, ctypes.c_longlong, c_int, P(c_void_p)],
         "AQuantize": [c_void_p, c_int],
         "AGetBins": [c_void_p, c_void_p],
         "AGetBins16": [c_void_p, c_void_p],
@@ -170,6 +171,32 @@ class DMatrix(object):
             self.handle = None
 
     # ---- extensions
+    @classmethod
+    def from_blocks(cls, block_addresses, block_rows, rows, columns, y=None, labels=None):
+        """Matrix over bin ids that stay in caller-owned host blocks (ACreateFromQuantizedBlocks): for
+        matrices beyond HBM and beyond 2^31 rows.  block_addresses: host addresses (ints) of the
+        blocks, each 32-bit words [ceil(columns / 4)][block_rows]; the caller keeps them alive.
+        Train with internals.upload_features = False."""
+        self = cls.__new__(cls)
+        self.handle = None
+        self.labels_count = 1
+        self.rows, self.columns = int(rows), int(columns)
+        ptrs = (ctypes.c_void_p * len(block_addresses))(*[int(a) for a in block_addresses])
+        handle = ctypes.c_void_p()
+        _check(_LIB.ACreateFromQuantizedBlocks(ptrs, len(block_addresses), int(block_rows), self.rows, self.columns,
+                                               ctypes.byref(handle)))
+        self.handle = handle
+        if y is not None:
+            assert self.rows == len(y)
+            yy = np.ascontiguousarray(np.asarray(y).reshape(self.rows), dtype=np.float32)
+            _check(_LIB.ASetY(self.handle, _fptr(yy)))
+        elif labels is not None:
+            assert self.rows == len(labels)
+            self.labels_count = int(np.max(labels)) + 1
+            ll = np.ascontiguousarray(np.asarray(labels).reshape(self.rows), dtype=np.uint8)
+            _check(_LIB.ASetLabel(self.handle, ll.ctypes.data_as(ctypes.POINTER(ctypes.c_ubyte))))
+        return self
+
     def quantize(self, hist_size):
         _check(_LIB.AQuantize(self.handle, int(hist_size)))
 

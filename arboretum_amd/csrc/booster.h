@@ -57,6 +57,8 @@ class DataMatrix {
   // holds rows [b * stream_block_rows, ...) as quads [Q][stream_block_rows].
   std::vector<uint32_t *> stream_blocks;
   size_t stream_block_rows = 0;
+  // The blocks belong to the caller (ACreateFromQuantizedBlocks): never copied, never freed.
+  bool external_blocks = false;
 
   // Feature value as seen by host prediction.
   inline float value(size_t f, size_t i) const {

@@ -80,6 +80,7 @@ struct DeviceMatrix {
   bool streamed = false;
   size_t block_rows = 0;
   std::vector<uint32_t *> host_blocks;
+  bool owns_blocks = true;  // false: the caller's blocks (ACreateFromQuantizedBlocks)
 };
 
 // Plain device-to-device copy of `bytes` bytes: a kernel of exactly known HBM
@@ -111,8 +112,9 @@ int DeviceCount() {
 void FreeDeviceMatrix(DeviceMatrix *m) {
   if (!m) return;
   if (m->bins) (void)hipFree(m->bins);
-  for (uint32_t *b : m->host_blocks)
-    if (b) (void)hipHostFree(b);
+  if (m->owns_blocks)
+    for (uint32_t *b : m->host_blocks)
+      if (b) (void)hipHostFree(b);
   delete m;
 }
 
@@ -173,7 +175,34 @@ void QuantiseOnDevice(DataMatrix *data, int hist_size, bool verbose, bool stream
   const size_t n = data->rows;
   const int F = (int)data->columns_dense;
   if (n == 0 || F == 0) throw std::runtime_error("empty data matrix");
-  if (n >= (1ull << 31)) throw std::runtime_error("too many rows");
+  // Rows are indexed with 32 bits inside a block of a streamed matrix and with 64 bits across
+  // blocks; a resident matrix and the quantiser's sort index whole columns with 32 bits.
+  if (n >= (1ull << 31) && !(streamed && data->is_prebinned))
+    throw std::runtime_error("too many rows: 2^31 and more need bin ids (ACreateFromQuantized...) and "
+                             "internals.upload_features = false");
+  if (data->external_blocks) {
+    if (!streamed) throw std::runtime_error("a matrix over caller-owned blocks is streamed: set internals.upload_features to false");
+    std::unique_ptr<DeviceMatrix, void (*)(DeviceMatrix *)> ext(new DeviceMatrix(), FreeDeviceMatrix);
+    ext->rows = n;
+    ext->F = F;
+    ext->Q = (F + 3) / 4;
+    ext->stride = (n + 63) / 64 * 64;
+    ext->streamed = true;
+    ext->owns_blocks = false;
+    ext->block_rows = data->stream_block_rows;
+    ext->host_blocks = data->stream_blocks;
+    data->thresholds.assign(F, {});
+    data->reduced_size.assign(F, 0);
+    for (int f = 0; f < F; ++f) {
+      data->thresholds[f].resize(hist_size);
+      for (int k = 0; k < hist_size; ++k) data->thresholds[f][k] = (float)k + 0.5f;
+      data->reduced_size[f] = std::min(hist_size, kSlots);
+    }
+    data->device = ext.release();
+    data->hist_size = hist_size;
+    data->quantised = true;
+    return;
+  }
   std::unique_ptr<DeviceMatrix, void (*)(DeviceMatrix *)> dm(new DeviceMatrix(), FreeDeviceMatrix);
   dm->rows = n;
   dm->F = F;
@@ -548,9 +577,11 @@ class HipTreeBuilder : public TreeBuilder {
     d_cand_ = DevAlloc<Cand>((size_t)last_nodes * F_);
     d_node_first_ = DevAlloc<unsigned>(last_nodes);
     d_node_items_ = DevAlloc<unsigned>(last_nodes);
-    max_hist_items_ = (unsigned)(n_ / HistRowsPerItem(n_)) + 2 * last_nodes + 2;
+    // row passes of a streamed matrix cover one block at a time
+    const size_t plan_rows = dm_->streamed ? std::min(n_, dm_->block_rows) : n_;
+    max_hist_items_ = (unsigned)(plan_rows / HistRowsPerItem(plan_rows)) + 2 * last_nodes + 2;
     max_hist_items_ = std::max<unsigned>(max_hist_items_, 1024 + 2 * last_nodes + 2);
-    max_part_items_ = std::max<unsigned>((unsigned)(n_ / kPartRows + 1) + 2 * last_nodes, max_hist_items_);
+    max_part_items_ = std::max<unsigned>((unsigned)(plan_rows / kPartRows + 1) + 2 * last_nodes, max_hist_items_);
     d_hwork_ = DevAlloc<WorkItem>(max_hist_items_);
     d_pwork_ = DevAlloc<WorkItem>(max_part_items_);
     d_nwork_ = DevAlloc<unsigned>(2);

@@ -97,8 +97,10 @@ ARB_HD double ShrinkD(double g, float alpha) {
 }
 
 // Weight(): gain.cu:34-76.  PAIR: hessian is h; else the row count.
+// The count is 64 bits wide: a streamed matrix may hold more than 2^32 rows
+// (the reference's counts are 32-bit, like its `int` row count).
 template <bool PAIR, bool F64>
-ARB_HD float LeafWeight(double g, double h, unsigned c, const GainParams &p) {
+ARB_HD float LeafWeight(double g, double h, unsigned long long c, const GainParams &p) {
   float w = 0.0f;
   if (PAIR) {
     if (F64) {
@@ -167,9 +169,9 @@ ARB_HD float SplitGain(double gl, double hl, unsigned long long cl, double gt, d
         return 0.0f;
     }
   }
-  const float wl = LeafWeight<PAIR, F64>(gl, hl, (unsigned)cl, p);
-  const float wr = LeafWeight<PAIR, F64>(gr, hr, (unsigned)cr, p);
-  const float wp = LeafWeight<PAIR, F64>(gt, ht, (unsigned)ct, p);
+  const float wl = LeafWeight<PAIR, F64>(gl, hl, cl, p);
+  const float wr = LeafWeight<PAIR, F64>(gr, hr, cr, p);
+  const float wp = LeafWeight<PAIR, F64>(gt, ht, ct, p);
   const float l = SideGain<PAIR, F64>(gl, hl, cl, wl, p);
   const float r = SideGain<PAIR, F64>(gr, hr, cr, wr, p);
   const float q = SideGain<PAIR, F64>(gt, ht, ct, wp, p);
@@ -186,7 +188,7 @@ ARB_HD float SplitGainKind(int kind, double gl, double hl, unsigned long long cl
     default: return SplitGain<true, true>(gl, hl, cl, gt, ht, ct, p);
   }
 }
-ARB_HD float LeafWeightKind(int kind, double g, double h, unsigned c, const GainParams &p) {
+ARB_HD float LeafWeightKind(int kind, double g, double h, unsigned long long c, const GainParams &p) {
   switch (kind) {
     case kCntF32: return LeafWeight<false, false>(g, h, c, p);
     case kCntF64: return LeafWeight<false, true>(g, h, c, p);

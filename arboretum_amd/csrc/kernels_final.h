@@ -29,8 +29,8 @@ __global__ void k_leaf_weights(const SplitRec *__restrict__ split, const NodeSum
     GR = (double)((float)GP - (float)GL);
     HR = (double)((float)HP - (float)HL);
   }
-  weights[2 * nd] = LeafWeight<PAIR, F64>(GL, HL, (unsigned)s.left.c, gp) * eta;
-  weights[2 * nd + 1] = LeafWeight<PAIR, F64>(GR, HR, (unsigned)(t.c - s.left.c), gp) * eta;
+  weights[2 * nd] = LeafWeight<PAIR, F64>(GL, HL, s.left.c, gp) * eta;
+  weights[2 * nd + 1] = LeafWeight<PAIR, F64>(GR, HR, t.c - s.left.c, gp) * eta;
 }
 
 // Leaf weights of a finished tree and, in the same launch, what would
@@ -96,8 +96,8 @@ k_tree_end(const SplitRec *__restrict__ split, const NodeSum *__restrict__ tot, 
     root_tot[0].c = n;
     root_seg[0] = 0;
   }
-  const float wl = LeafWeight<PAIR, F64>(GL, HL, (unsigned)s.left.c, gp) * eta;
-  const float wr = LeafWeight<PAIR, F64>(GR, HR, (unsigned)(t.c - s.left.c), gp) * eta;
+  const float wl = LeafWeight<PAIR, F64>(GL, HL, s.left.c, gp) * eta;
+  const float wr = LeafWeight<PAIR, F64>(GR, HR, t.c - s.left.c, gp) * eta;
   weights[2 * nd] = wl;
   weights[2 * nd + 1] = wr;
   record[3 * internal + 2 * nd] = __float_as_uint(wl);

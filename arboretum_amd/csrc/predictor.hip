@@ -174,7 +174,9 @@ struct DevicePredictor {
   const float *Run(const DataMatrix &data, const std::vector<RegTree> &trees, size_t use, size_t labels, float init) {
     const size_t n = data.rows, F = data.columns_dense;
     if (n == 0 || F == 0) throw std::runtime_error("empty data matrix");
-    if (n >= (1ull << 31)) throw std::runtime_error("too many rows");
+    // only the block-wise walk of a streamed matrix indexes rows with 64 bits
+    if (n >= (1ull << 31) && !(data.is_prebinned && data.prebinned.empty() && !data.stream_blocks.empty()))
+      throw std::runtime_error("too many rows");
     if (!stream) {
       HIP_OK(hipStreamCreate(&stream));
       for (int k = 0; k < 2; ++k) HIP_OK(hipEventCreateWithFlags(&copied[k], hipEventDisableTiming));

@@ -222,6 +222,27 @@ const char *ACreateFromQuantized(const unsigned char *bins, long long nrow, int 
   });
 }
 
+const char *ACreateFromQuantizedBlocks(const unsigned *const *blocks, int nblocks, long long block_rows,
+                                       long long nrow, int ncol, VoidPointer *out) {
+  return Guard([&] {
+    if (!blocks || !out || nblocks <= 0 || block_rows <= 0 || nrow <= 0 || ncol <= 0)
+      throw std::runtime_error("bad arguments");
+    if (block_rows % 64 != 0) throw std::runtime_error("block_rows must be a multiple of 64");
+    if (block_rows >= (1ll << 31)) throw std::runtime_error("a block holds fewer than 2^31 rows");
+    if ((long long)(nblocks - 1) * block_rows >= nrow || (long long)nblocks * block_rows < nrow)
+      throw std::runtime_error("nrow does not match nblocks blocks of block_rows rows (the last one may be shorter)");
+    for (int b = 0; b < nblocks; ++b)
+      if (!blocks[b]) throw std::runtime_error("null block pointer");
+    DataMatrix *mat = new DataMatrix((size_t)nrow, (size_t)ncol, 0);
+    mat->is_prebinned = true;
+    mat->external_blocks = true;
+    mat->stream_block_rows = (size_t)block_rows;
+    mat->stream_blocks.resize(nblocks);
+    for (int b = 0; b < nblocks; ++b) mat->stream_blocks[b] = const_cast<uint32_t *>(blocks[b]);
+    *out = mat;
+  });
+}
+
 const char *AQuantize(VoidPointer data, int hist_size) {
   return Guard([&] {
     if (DeviceCount() <= 0) throw std::runtime_error("no HIP device available: the quantiser needs an MI355X");

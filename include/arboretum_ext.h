@@ -30,6 +30,22 @@ const char *ADeviceCopyProbe(unsigned long long bytes);
 const char *ACreateFromQuantized(const unsigned char *bins, long long nrow, int ncol,
                                  VoidPointer *out);
 
+/* Data matrix over bin ids that stay where the caller keeps them: for matrices
+ * beyond HBM and beyond the reference's `int nrow` (python-wrapper/
+ * arboretum_wrapper.h:6-10 takes one fp32 array and an int row count).  The
+ * rows live in `nblocks` caller-owned host blocks of `block_rows` rows (a
+ * multiple of 64, below 2^31; the last block may hold fewer: nrow in all, any
+ * 64-bit count); nothing is copied and nothing is freed with the matrix.
+ * Block layout (what the GPU streams as it is): 32-bit words
+ * [Q][block_rows], Q = ceil(ncol / 4), word q * block_rows + r = bin ids of
+ * features 4 q .. 4 q + 3 of the block's row r, one byte each, lowest byte
+ * first.  Allocate the blocks with hipHostMalloc for the full host-to-device
+ * rate.  Training needs `internals.upload_features: false` (the blocks are
+ * streamed once per tree level); several descriptors may name the same block.
+ * Thresholds are reported as bin + 0.5, as for ACreateFromQuantized. */
+const char *ACreateFromQuantizedBlocks(const unsigned *const *blocks, int nblocks, long long block_rows,
+                                       long long nrow, int ncol, VoidPointer *out);
+
 /* Runs the quantiser now (the reference defers it to the first AGrowTree,
  * src/core/garden.cu:586-589).  Needs a GPU. */
 const char *AQuantize(VoidPointer data, int hist_size);

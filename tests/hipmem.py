@@ -56,3 +56,25 @@ class DeviceArray:
         if getattr(self, "ptr", None):
             hip().hipFree(self.ptr)
             self.ptr = None
+
+
+class PinnedArray:
+    """Pinned host memory (hipHostMalloc) seen as a numpy array."""
+
+    def __init__(self, shape, dtype):
+        self.shape, self.dtype = tuple(shape), np.dtype(dtype)
+        self.nbytes = int(np.prod(self.shape)) * self.dtype.itemsize
+        lib = hip()
+        lib.hipHostMalloc.argtypes = [ctypes.POINTER(ctypes.c_void_p), ctypes.c_size_t, ctypes.c_uint]
+        lib.hipHostFree.argtypes = [ctypes.c_void_p]
+        p = ctypes.c_void_p()
+        _ok(lib.hipHostMalloc(ctypes.byref(p), max(self.nbytes, 256), 0), "hipHostMalloc")
+        self.ptr = p.value
+        buf = (ctypes.c_ubyte * self.nbytes).from_address(self.ptr)
+        self.array = np.frombuffer(buf, dtype=self.dtype).reshape(self.shape)
+
+    def __del__(self):
+        if getattr(self, "ptr", None):
+            self.array = None
+            hip().hipHostFree(self.ptr)
+            self.ptr = None
