@@ -51,6 +51,9 @@ struct InternalConfiguration {  // param.h:54-64
   // Extension (not a reference key): rows per pinned-host block when the bins
   // are streamed (upload_features = false); 0 = chosen from the matrix size.
   unsigned stream_block_rows = 0;
+  // Extension: matrices of more than 32 features keep their rows in place and
+  // re-order (row id, gradients) only; false selects the row-moving passes.
+  bool wide_rows_in_place = true;
 };
 
 struct Configuration {  // param.h:66-74

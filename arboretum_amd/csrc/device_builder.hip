@@ -60,6 +60,7 @@
 #include "gain.h"
 #include "kernels_final.h"
 #include "kernels_hist.h"
+#include "kernels_indexed.h"
 #include "kernels_launch.h"
 #include "kernels_objective.h"
 #include "kernels_partition.h"
@@ -76,6 +77,9 @@ struct DeviceMatrix {
   int bits = 8;              // bits per bin id: 8 (four features per word) or 16 (two)
   int slots = kSlots;        // histogram slots per feature
   uint32_t *bins = nullptr;  // resident: [Q][stride] in HBM
+  // wide resident matrices, built on first use: the same bins row-major, RS words per row
+  uint32_t *rec = nullptr;
+  int RS = 0;
   // streamed: pinned host blocks [Q][block_rows], block b = rows [b*block_rows, ...)
   bool streamed = false;
   size_t block_rows = 0;
@@ -112,6 +116,7 @@ int DeviceCount() {
 void FreeDeviceMatrix(DeviceMatrix *m) {
   if (!m) return;
   if (m->bins) (void)hipFree(m->bins);
+  if (m->rec) (void)hipFree(m->rec);
   if (m->owns_blocks)
     for (uint32_t *b : m->host_blocks)
       if (b) (void)hipHostFree(b);
@@ -424,7 +429,29 @@ namespace {
 struct RowBuffers {
   uint32_t *bins = nullptr;
   float *g = nullptr, *h = nullptr;
+  unsigned *ids = nullptr;  // indexed mode: the row at each position (null: position = row)
 };
+
+template <bool PAIR>
+void LaunchHistRec(int nq, hipStream_t st, unsigned grid, const uint32_t *rec, int RS, const unsigned *ids, int q0,
+                   int F, const float *g, const float *h, const int *shifts, const WorkItem *work,
+                   const unsigned *n_work, unsigned long long *slab, int slab_entries) {
+#define ARB_CASE(N)                                                                                              \
+  case N: {                                                                                                      \
+    static bool configured = false;                                                                              \
+    if (!configured) {                                                                                           \
+      AllowLds(k_hist_rec<PAIR, N>, HistLdsBytes(N, PAIR));                                                      \
+      configured = true;                                                                                         \
+    }                                                                                                            \
+    hipLaunchKernelGGL((k_hist_rec<PAIR, N>), dim3(grid), dim3(kHistThreads), HistLdsBytes(N, PAIR), st, rec, RS, \
+                       ids, q0, F, g, h, shifts, work, n_work, slab, slab_entries);                              \
+  } break;
+  switch (nq) {
+    ARB_CASE(1) ARB_CASE(2) ARB_CASE(3) ARB_CASE(4) ARB_CASE(5) ARB_CASE(6) ARB_CASE(7) ARB_CASE(8)
+    default: throw std::runtime_error("internal: bad quad count");
+  }
+#undef ARB_CASE
+}
 
 struct FusedArgs {
   const uint32_t *bins;
@@ -511,8 +538,11 @@ class HipTreeBuilder : public TreeBuilder {
     quads_per_group_ = std::min(quads_per_group_, Q_);
     // the fused partition + histogram pass holds one histogram of all
     // features and builds only the smaller child
-    fused_ = trick_ && !wide_;
     single_group_ = Q_ <= quads_per_group_;
+    // Matrices wider than one group of quads: rows stay in place as records, only (row id,
+    // gradients) are re-ordered (kernels_indexed.h).
+    indexed_ = !wide_ && !dm_->streamed && !single_group_ && D_ > 2 && cfg.internal.wide_rows_in_place;
+    fused_ = trick_ && !wide_ && !indexed_;
     if (wide_) {
       // features per histogram launch (an even number, two per word)
       const size_t per_feature = (size_t)slots_ * 8 * (pair_ ? 2 : 1);
@@ -526,7 +556,7 @@ class HipTreeBuilder : public TreeBuilder {
     streamed_ = dm_->streamed;
     // Logistic gradients of 0/1 labels travel as one float per row (PackGrad):
     // there is no h array then, and kernels given h == nullptr unpack g.
-    pack_ = cfg.objective == kLogisticRegression && !streamed_ && !wide_ && data->y.size() == n_ &&
+    pack_ = cfg.objective == kLogisticRegression && !streamed_ && !wide_ && Q_ <= kMaxGroupQuads && data->y.size() == n_ &&
             std::all_of(data->y.begin(), data->y.end(), [](float v) { return v == 0.0f || v == 1.0f; });
     d_g_ = DevAlloc<float>(n_ * K_);
     d_h_ = pack_ ? nullptr : DevAlloc<float>(n_ * K_);
@@ -559,9 +589,21 @@ class HipTreeBuilder : public TreeBuilder {
     // ping-pong row buffers in node order (not needed for a single split level)
     if (D_ > 2 && !streamed_) {
       for (int b = 0; b < 2; ++b) {
-        buf_[b].bins = DevAlloc<uint32_t>((size_t)Q_ * stride_);
+        if (indexed_) buf_[b].ids = DevAlloc<unsigned>(n_);
+        else buf_[b].bins = DevAlloc<uint32_t>((size_t)Q_ * stride_);
         buf_[b].g = DevAlloc<float>(n_);
         buf_[b].h = pack_ ? nullptr : DevAlloc<float>(n_);
+      }
+    }
+    if (indexed_) {
+      d_dec_ = DevAlloc<uint8_t>(n_);
+      if (!dm_->rec) {  // records: 32-byte aligned, built once per matrix
+        dm_->RS = (Q_ + 7) / 8 * 8;
+        dm_->rec = DevAlloc<uint32_t>(n_ * (size_t)dm_->RS);
+        hipLaunchKernelGGL(k_to_records, dim3((unsigned)((n_ + 63) / 64)), dim3(256),
+                           (size_t)64 * (dm_->RS + 1) * sizeof(uint32_t), stream_, dm_->bins, stride_, Q_, dm_->rec,
+                           dm_->RS, n_);
+        HIP_OK(hipGetLastError());
       }
     }
     // level state
@@ -624,11 +666,11 @@ class HipTreeBuilder : public TreeBuilder {
     (void)hipStreamSynchronize(stream_);
     void *ptrs[] = {d_y_, d_labels_, d_yhat_, d_g_, d_h_, d_leaf_, d_split_, d_cand_, d_node_first_,
                     d_node_items_, d_hwork_, d_pwork_, d_nwork_, d_wave_left_, d_item_left_, d_slab_,
-                    d_shifts_, d_gmax_, d_rows_scanned_, d_tfid_, d_tbin_, d_tgain_, d_weights_, d_active_, d_overflow_, d_records_, d_cursor2_};
+                    d_shifts_, d_gmax_, d_rows_scanned_, d_tfid_, d_tbin_, d_tgain_, d_weights_, d_active_, d_overflow_, d_records_, d_cursor2_, d_dec_};
     for (void *p : ptrs)
       if (p) (void)hipFree(p);
     for (int b = 0; b < 2; ++b) {
-      void *q[] = {buf_[b].bins, buf_[b].g, buf_[b].h, d_tot_[b], d_seg_[b], d_hg_[b], d_hh_[b], d_hc_[b]};
+      void *q[] = {buf_[b].bins, buf_[b].g, buf_[b].h, buf_[b].ids, d_tot_[b], d_seg_[b], d_hg_[b], d_hh_[b], d_hc_[b]};
       for (void *p : q)
         if (p) (void)hipFree(p);
     }
@@ -877,10 +919,16 @@ class HipTreeBuilder : public TreeBuilder {
     }
     for (int q0 = 0; q0 < Q_; q0 += quads_per_group_) {
       const int nq = std::min(quads_per_group_, Q_ - q0);
-      if (pair_)
+      if (indexed_) {
+        if (pair_)
+          LaunchHistRec<true>(nq, stream_, grid, dm_->rec, dm_->RS, cur.ids, q0, F_, cur.g, cur.h, d_shifts_, d_hwork_, d_nwork_, d_slab_, slab_entries_);
+        else
+          LaunchHistRec<false>(nq, stream_, grid, dm_->rec, dm_->RS, cur.ids, q0, F_, cur.g, cur.h, d_shifts_, d_hwork_, d_nwork_, d_slab_, slab_entries_);
+      } else if (pair_) {
         LaunchHist<true>(nq, stream_, grid, cur.bins, stride_, q0, F_, cur.g, cur.h, d_shifts_, d_hwork_, d_nwork_, d_slab_, slab_entries_);
-      else
+      } else {
         LaunchHist<false>(nq, stream_, grid, cur.bins, stride_, q0, F_, cur.g, cur.h, d_shifts_, d_hwork_, d_nwork_, d_slab_, slab_entries_);
+      }
       if (timing_) ++(root ? timings_.hist_root_launches : timings_.hist_deep_launches);
     }
     if (timing_ && root) timings_.hist_root_rows += n_;
@@ -986,9 +1034,22 @@ class HipTreeBuilder : public TreeBuilder {
           Mark(kPlan);
           Plan(ps, PL, 0, kPartRows, d_pwork_, d_nwork_ + 1, -1, nullptr, grid);
           Mark(kPartition);
-          hipLaunchKernelGGL(k_part_count, dim3(grid), dim3(kHistThreads), 0, stream_, src.bins, stride_, d_split_,
-                             d_pwork_, d_nwork_ + 1, d_wave_left_, d_item_left_, code_);
-          LaunchPartRows(grid, src, dst, ps);
+          if (indexed_) {
+            hipLaunchKernelGGL(k_ix_decide, dim3(grid), dim3(kHistThreads), 0, stream_, dm_->rec, dm_->RS, src.ids,
+                               d_split_, d_pwork_, d_nwork_ + 1, d_dec_, d_wave_left_, d_item_left_);
+            if (pair_)
+              hipLaunchKernelGGL(k_ix_part<true>, dim3(grid), dim3(kHistThreads), 0, stream_, src.ids, dst.ids, src.g,
+                                 dst.g, src.h, dst.h, d_dec_, d_split_, d_seg_[ps], d_pwork_, d_nwork_ + 1,
+                                 d_wave_left_, d_item_left_);
+            else
+              hipLaunchKernelGGL(k_ix_part<false>, dim3(grid), dim3(kHistThreads), 0, stream_, src.ids, dst.ids, src.g,
+                                 dst.g, src.h, dst.h, d_dec_, d_split_, d_seg_[ps], d_pwork_, d_nwork_ + 1,
+                                 d_wave_left_, d_item_left_);
+          } else {
+            hipLaunchKernelGGL(k_part_count, dim3(grid), dim3(kHistThreads), 0, stream_, src.bins, stride_, d_split_,
+                               d_pwork_, d_nwork_ + 1, d_wave_left_, d_item_left_, code_);
+            LaunchPartRows(grid, src, dst, ps);
+          }
           HistOfNodes(dst, state, L, trick_, trick_ ? n_ / 2 : n_, false, level);
           Reduce(L, hb, false, ps, trick_);
         }
@@ -1336,6 +1397,8 @@ class HipTreeBuilder : public TreeBuilder {
   int F_ = 0, Q_ = 0, K_ = 1, D_ = 2, nbin_total_ = 0;
   int slab_entries_ = 0;  // histogram entries of one work item's slab (whole 16-feature blocks)
   bool single_group_ = true;  // all quads fit one LDS histogram
+  bool indexed_ = false;      // wide matrix: rows stay in place, (row id, gradients) are re-ordered
+  uint8_t *d_dec_ = nullptr;  // indexed mode: split decision of the row at each position
   bool wide_ = false;     // 16-bit bins: two features per word, slots_ histogram slots per feature
   int slots_ = kSlots;
   int wide_group_ = 2;    // features per histogram launch with 16-bit bins

@@ -1,0 +1,212 @@
+// Kernels for matrices too wide for the fused pass (more than 32 features):
+// the rows stay where they are and only (row id, gradients) are re-ordered.
+//
+// Moving a row of F bin bytes at every level costs 2 F bytes per row and
+// level; from a few dozen features on that dominates everything else.  A row
+// kept as one contiguous record of at least 128 bytes can be gathered through
+// an index list at the rate of a stream (each record fills whole memory
+// lines), so for wide matrices the bins are stored a second time row-major
+// ("records"), the node order of a level is a list of row ids with the rows'
+// gradients beside it, a level's partition moves 12 bytes per row, and the
+// histogram kernel gathers the records of the smaller children.
+#ifndef ARBORETUM_AMD_KERNELS_INDEXED_H_
+#define ARBORETUM_AMD_KERNELS_INDEXED_H_
+#include "device_common.h"
+#include "kernels_hist.h"
+#include "kernels_partition.h"
+
+namespace arb {
+namespace {
+
+// Quad columns [Q][stride] -> records [rows][RS] (RS words per row, the words
+// past Q zero).  A workgroup transposes 64 rows through LDS: the reads are
+// coalesced along the rows, the writes along the record.
+__global__ void __launch_bounds__(256)
+k_to_records(const uint32_t *__restrict__ bins, size_t stride, int Q, uint32_t *__restrict__ rec, int RS,
+             size_t n) {
+  extern __shared__ uint32_t s_tile[];  // [64][RS + 1]
+  const size_t r0 = (size_t)blockIdx.x * 64;
+  const int lane = threadIdx.x & 63, part = threadIdx.x >> 6;  // 4 parts
+  for (int q = part; q < RS; q += 4) {
+    uint32_t v = 0;
+    if (q < Q && r0 + lane < n) v = bins[(size_t)q * stride + r0 + lane];
+    s_tile[lane * (RS + 1) + q] = v;
+  }
+  __syncthreads();
+  const size_t rows = min((size_t)64, n - r0);
+  for (size_t e = threadIdx.x; e < rows * RS; e += 256) {
+    const size_t r = e / RS, q = e % RS;
+    rec[(r0 + r) * RS + q] = s_tile[r * (RS + 1) + q];
+  }
+}
+
+// Split decision of every row of the parents of a level, in node order:
+// dec[p] = 1 when the row at position p goes right (builder.h:107-123), and the
+// rows going left per (work item, wave) as k_part_count gives them.  ids: the
+// row at each position (null: position = row, the first level).
+__global__ void __launch_bounds__(kHistThreads)
+k_ix_decide(const uint32_t *__restrict__ rec, int RS, const unsigned *__restrict__ ids,
+            const SplitRec *__restrict__ split, const WorkItem *__restrict__ work,
+            const unsigned *__restrict__ n_work, uint8_t *__restrict__ dec, unsigned *__restrict__ wave_left,
+            unsigned *__restrict__ item_left) {
+  const unsigned w = blockIdx.x;
+  if (w >= *n_work) return;
+  const WorkItem it = work[w];
+  const SplitRec s = split[it.node];
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int fq = s.fid < 0 ? 0 : s.fid >> 2, fs = 8 * (s.fid & 3);
+  unsigned cnt = 0;
+  const unsigned cb = ChunkOrigin(it);
+  constexpr int kBatch = 4;  // 8 ids, then 8 gathers in flight per lane
+  for (unsigned base = cb + wave * kChunkRows; base < it.end; base += kBatch * kChunkStep) {
+    unsigned id[2 * kBatch];
+    uint32_t word[2 * kBatch];
+#pragma unroll
+    for (int k = 0; k < 2 * kBatch; ++k) {
+      const unsigned r = base + (k >> 1) * kChunkStep + (k & 1) * 64 + lane;
+      const unsigned a = min(r, it.end - 1);
+      id[k] = ids ? ids[a] : a;
+    }
+#pragma unroll
+    for (int k = 0; k < 2 * kBatch; ++k) word[k] = s.fid < 0 ? 0u : rec[(size_t)id[k] * RS + fq];
+#pragma unroll
+    for (int k = 0; k < 2 * kBatch; ++k) {
+      const unsigned r = base + (k >> 1) * kChunkStep + (k & 1) * 64 + lane;
+      if (r >= it.begin && r < it.end) {
+        const bool right = s.fid >= 0 && (int)((word[k] >> fs) & 255u) > s.bin;
+        dec[r] = right ? 1 : 0;
+        cnt += right ? 0u : 1u;
+      }
+    }
+  }
+  for (int off = 32; off > 0; off >>= 1) cnt += __shfl_down(cnt, off);
+  if (lane == 0) wave_left[(size_t)w * kItemWaves + wave] = cnt;
+  __shared__ unsigned s_cnt[kItemWaves];
+  if (lane == 0) s_cnt[wave] = cnt;
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    unsigned t = 0;
+    for (int k = 0; k < kItemWaves; ++k) t += s_cnt[k];
+    item_left[w] = t;
+  }
+}
+
+// Stable partition of (row id, gradients) into the children order by the
+// decisions of k_ix_decide, through the register queues of the row passes.
+// ids null: position = row.
+template <bool PAIR>
+__global__ void __launch_bounds__(kHistThreads)
+k_ix_part(const unsigned *__restrict__ ids, unsigned *__restrict__ ids_out, const float *__restrict__ g,
+          float *__restrict__ g_out, const float *__restrict__ h, float *__restrict__ h_out,
+          const uint8_t *__restrict__ dec, const SplitRec *__restrict__ split,
+          const unsigned *__restrict__ seg_start, const WorkItem *__restrict__ work,
+          const unsigned *__restrict__ n_work, const unsigned *__restrict__ wave_left,
+          const unsigned *__restrict__ item_left) {
+  __shared__ unsigned s_tmp[kItemWaves + 1];
+  const unsigned w = blockIdx.x;
+  if (w >= *n_work) return;
+  const WorkItem it = work[w];
+  const SplitRec s = split[it.node];
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const unsigned wb = ChunkOrigin(it) + wave * kChunkRows, we = it.end;
+  unsigned lo, ro;
+  const unsigned before = LeftsBefore(it, w, wave, wave_left, item_left, s_tmp);
+  WaveOffsets(it, s, seg_start[it.node], before, wave, &lo, &ro);
+  if (wb >= we) return;
+  RowQueue<1> QL, QR;
+  QL.Init(lo);
+  QR.Init(ro);
+  struct Rows {
+    RowSet<1> r;
+    uint32_t d0, d1;
+  };
+  auto load = [&](Rows &R, unsigned base) {
+    const unsigned a0 = min(base + lane, we - 1), a1 = min(base + 64 + lane, we - 1);
+    R.r.b0[0] = ids ? ids[a0] : a0;
+    R.r.b1[0] = ids ? ids[a1] : a1;
+    R.d0 = dec[a0];
+    R.d1 = dec[a1];
+    R.r.g0 = g[a0];
+    R.r.g1 = g[a1];
+    R.r.h0 = PAIR ? h[a0] : 0.0f;
+    R.r.h1 = PAIR ? h[a1] : 0.0f;
+  };
+  auto process = [&](const Rows &R, unsigned base) {
+    const unsigned r0 = base + lane, r1 = r0 + 64;
+    const bool v0 = r0 >= it.begin && r0 < we, v1 = r1 < we;
+    const bool right0 = v0 && R.d0 != 0, right1 = v1 && R.d1 != 0;
+    const unsigned long long lm0 = __ballot(v0 && !right0), rm0 = __ballot(right0);
+    const unsigned long long lm1 = __ballot(v1 && !right1), rm1 = __ballot(right1);
+    uint32_t *out = ids_out;
+    MergeRows<PAIR, 1, false, true>(nullptr, QL, R.r.b0, R.r.g0, R.r.h0, lm0, false, out, 0, g_out, h_out, lane, 0, 0, 0);
+    MergeRows<PAIR, 1, false, true>(nullptr, QR, R.r.b0, R.r.g0, R.r.h0, rm0, false, out, 0, g_out, h_out, lane, 0, 0, 0);
+    MergeRows<PAIR, 1, false, true>(nullptr, QL, R.r.b1, R.r.g1, R.r.h1, lm1, false, out, 0, g_out, h_out, lane, 0, 0, 0);
+    MergeRows<PAIR, 1, false, true>(nullptr, QR, R.r.b1, R.r.g1, R.r.h1, rm1, false, out, 0, g_out, h_out, lane, 0, 0, 0);
+  };
+  Rows A, B;
+  load(A, wb);
+  for (unsigned base = wb;; base += 2 * kChunkStep) {
+    load(B, base + kChunkStep);
+    process(A, base);
+    if (base + kChunkStep >= we) break;  // wave-uniform
+    load(A, base + 2 * kChunkStep);
+    process(B, base + kChunkStep);
+    if (base + 2 * kChunkStep >= we) break;
+  }
+  FlushQueue<PAIR, 1, false, true>(nullptr, QL, false, ids_out, 0, g_out, h_out, lane, 0, 0, 0);
+  FlushQueue<PAIR, 1, false, true>(nullptr, QR, false, ids_out, 0, g_out, h_out, lane, 0, 0, 0);
+}
+
+// k_hist over records: the row at position p of a work item is ids[p] (null:
+// p itself), its quads [q0, q0 + NQ) are words q0.. of its record (q0 a
+// multiple of 8, records 32-byte aligned: two 16-byte loads per row when
+// NQ = 8), its gradients are g[p], h[p].
+template <bool PAIR, int NQ>
+__global__ void __launch_bounds__(kHistThreads)
+k_hist_rec(const uint32_t *__restrict__ rec, int RS, const unsigned *__restrict__ ids, int q0, int F,
+           const float *__restrict__ g, const float *__restrict__ h, const int *__restrict__ shifts,
+           const WorkItem *__restrict__ work, const unsigned *__restrict__ n_work,
+           unsigned long long *__restrict__ slab, int slab_entries) {
+  extern __shared__ unsigned long long lds[];
+  const unsigned w = blockIdx.x;
+  if (w >= *n_work) return;
+  const WorkItem it = work[w];
+  constexpr int words = (int)(HistLdsBytes(NQ, PAIR) / 8);
+  for (int i = threadIdx.x; i < words; i += kHistThreads) lds[i] = 0ull;
+  __syncthreads();
+  const int sg = shifts[0], sh = shifts[1];
+  // ids of the next pair of rows are requested while the current pair is accumulated
+  auto row_at = [&](unsigned r) {
+    const unsigned a = r < it.end ? r : it.begin;
+    return ids ? ids[a] : a;
+  };
+  unsigned n0 = row_at(it.begin + threadIdx.x), n1 = row_at(it.begin + threadIdx.x + kHistThreads);
+  for (unsigned base = it.begin; base < it.end; base += 2 * kHistThreads) {
+    const unsigned r0 = base + threadIdx.x, r1 = r0 + kHistThreads;
+    const bool v0 = r0 < it.end, v1 = r1 < it.end;
+    const unsigned a0 = v0 ? r0 : it.begin, a1 = v1 ? r1 : it.begin;
+    const unsigned id0 = n0, id1 = n1;
+    uint32_t b0[NQ], b1[NQ];
+    const uint32_t *p0 = rec + (size_t)id0 * RS + q0, *p1 = rec + (size_t)id1 * RS + q0;
+#pragma unroll
+    for (int q = 0; q < NQ; ++q) {
+      b0[q] = p0[q];
+      b1[q] = p1[q];
+    }
+    n0 = row_at(r0 + 2 * kHistThreads);
+    n1 = row_at(r1 + 2 * kHistThreads);
+    const float g0 = g[a0], g1 = g[a1];
+    float h0 = 0.0f, h1 = 0.0f;
+    if (PAIR) {
+      h0 = h[a0];
+      h1 = h[a1];
+    }
+    if (v0) AccumulateRow<PAIR, NQ>(lds, b0, g0, h0, sg, sh, q0, F);
+    if (v1) AccumulateRow<PAIR, NQ>(lds, b1, g1, h1, sg, sh, q0, F);
+  }
+  FlushSlab<PAIR, NQ>(lds, slab, w, slab_entries, q0);
+}
+
+}  // namespace
+}  // namespace arb
+#endif  // ARBORETUM_AMD_KERNELS_INDEXED_H_

@@ -152,6 +152,97 @@ def stream_mode(args, arb):
                               if args.stream_timing else None)}))
 
 
+def make_config2_bins(rows, features=200, seed=2):
+    """BASELINE configs[2] as the kernels see it: 64 bins per feature plus the missing-value bin (id
+    64, 30 % of the values, uniformly placed); half the columns uniform over the 64 bins, half
+    integer categories 0..49 under Zipf(1.1); regression target = 20 random piecewise-constant
+    functions of the bins plus noise.  Generated in row chunks (the fp32 matrix would be 40 GB)."""
+    rng = np.random.default_rng(seed)
+    base_rows = min(rows, 5_000_000)   # a base tile is generated and repeated (generation time)
+    if rows > base_rows:
+        tile, ty = make_config2_bins(base_rows, features, seed)
+        reps = (rows + base_rows - 1) // base_rows
+        bins = np.tile(tile, (reps, 1))[:rows]
+        y = np.tile(ty, reps)[:rows] + 0.05 * rng.standard_normal(rows, dtype=np.float32)
+        return bins, y.astype(np.float32)
+    bins = np.empty((rows, features), dtype=np.uint8)
+    y = np.zeros(rows, dtype=np.float32)
+    steps = [(int(rng.integers(0, features)), int(rng.integers(8, 56)), float(rng.normal()), float(rng.normal()))
+             for _ in range(20)]
+    # min(Zipf(1.1) - 1, 49) by table lookup on 16 random bits (numpy's zipf sampler is slow)
+    from scipy.special import zeta
+    pk = np.arange(1, 50, dtype=np.float64) ** -1.1 / zeta(1.1)
+    cdf = np.concatenate([np.cumsum(pk), [1.0]])
+    zipf_table = np.searchsorted(cdf, (np.arange(65536) + 0.5) / 65536.0).astype(np.uint8)
+    chunk = 1 << 20
+    for r0 in range(0, rows, chunk):
+        r1 = min(rows, r0 + chunk)
+        b = bins[r0:r1]
+        b[:, :features // 2] = rng.integers(0, 64, size=(r1 - r0, features // 2), dtype=np.uint8)
+        b[:, features // 2:] = zipf_table[rng.integers(0, 65536, size=(r1 - r0, features - features // 2), dtype=np.uint16)]
+        yy = y[r0:r1]
+        for f, t, lo, hi in steps:
+            yy += np.where(b[:, f] > t, hi, lo).astype(np.float32)
+        b[rng.integers(0, 256, size=b.shape, dtype=np.uint8) < 77] = 64     # 77 / 256 = 30.1 % missing
+    y += 0.1 * rng.standard_normal(rows, dtype=np.float32)
+    return bins, y
+
+
+def make_config3(rows, features=100, classes=10, seed=3):
+    """BASELINE configs[3]: N(0,1) features, labels = argmax(X W + Gumbel noise)."""
+    rng = np.random.default_rng(seed)
+    X = rng.standard_normal(size=(rows, features), dtype=np.float32)
+    W = rng.standard_normal(size=(features, classes)).astype(np.float32)
+    labels = np.empty(rows, dtype=np.uint8)
+    chunk = 1 << 20
+    for r0 in range(0, rows, chunk):
+        r1 = min(rows, r0 + chunk)
+        labels[r0:r1] = np.argmax(X[r0:r1] @ W + rng.gumbel(size=(r1 - r0, classes)).astype(np.float32), axis=1)
+    return X, labels
+
+
+def other_config(args, arb):
+    """BASELINE configs[2] / configs[3] at full size: seconds per tree (not the headline metric;
+    prints its own JSON line)."""
+    t0 = time.perf_counter()
+    if args.workload == "config2":
+        rows = args.rows if args.rows != 10_500_000 else 50_000_000
+        F = 200
+        bins, y = make_config2_bins(rows, F)
+        data = arb.DMatrix(bins, y=y, quantized=True)
+        del bins
+        cfg = {"objective": 0, "method": 1, "internals": {"hist_size": 64, "double_precision": True},
+               "tree": {"max_depth": 10, "eta": 0.3, "lambda": 1.0}}
+        trees_per_round, name = 1, "configs[2]: %d x 200, 64 bins + missing bin (30 %%), squared error, max_depth 10" % rows
+    else:
+        rows = args.rows if args.rows != 10_500_000 else 20_000_000
+        F, K = 100, 10
+        X, labels = make_config3(rows, F, K)
+        data = arb.DMatrix(X, labels=labels)
+        del X
+        cfg = {"objective": 4, "method": 1, "internals": {"hist_size": 256, "double_precision": True},
+               "tree": {"max_depth": 6, "eta": 0.2, "lambda": 1.0, "labels_count": K}}
+        trees_per_round, name = K, "configs[3]: %d x 100, 10 classes soft-max, 256 bins, max_depth 6" % rows
+    t_gen = time.perf_counter() - t0
+    model = arb.Garden(cfg, data)
+    t0 = time.perf_counter()
+    model.grow_tree()
+    model.synchronize()
+    t_first = time.perf_counter() - t0
+    s0 = model.rows_scanned()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        model.grow_tree()
+    model.synchronize()
+    dt = time.perf_counter() - t0
+    scanned = model.rows_scanned() - s0
+    trees = args.steps * trees_per_round
+    print(json.dumps({"metric": "seconds per tree", "workload": name, "rows": rows, "features": F,
+                      "rounds": args.steps, "trees": trees, "sec_per_tree": dt / trees, "sec_per_round": dt / args.steps,
+                      "hist_updates_per_s": scanned * F / dt, "first_round_with_quantisation_s": t_first,
+                      "generate_s": t_gen}))
+
+
 def cpu_baseline(X, y, cfg, sample_rows, trees):
     """The CPU checker on the first `sample_rows` rows (same columns, same
     configuration), all host cores."""
@@ -188,6 +279,8 @@ def main():
                     help="stress variant: this fraction of the feature values is replaced by NaN (all land in "
                          "one bin per feature; needs --hist-size <= 255)")
     ap.add_argument("--mode", choices=["resident", "stream"], default="resident")
+    ap.add_argument("--workload", choices=["headline", "config2", "config3"], default="headline",
+                    help="config2 / config3: BASELINE configs[2] / configs[3] at full size, seconds per tree only")
     ap.add_argument("--stream-rows", type=int, default=64_000_000)
     ap.add_argument("--stream-features", type=int, default=128)
     ap.add_argument("--stream-block-rows", type=int, default=1 << 22)
@@ -207,6 +300,9 @@ def main():
         arb.copy_probe(args.copy_probe << 20)
     if args.mode == "stream":
         stream_mode(args, arb)
+        return
+    if args.workload != "headline":
+        other_config(args, arb)
         return
 
     X, y = make_workload(args.rows, args.features)

@@ -299,13 +299,29 @@ def test_training_many_features_uses_feature_groups(arb, oracle):
     assert_same_training(arb, oracle, X, y, cfg, rounds=2)
 
 
+@pytest.mark.parametrize("in_place", [True, False])
 @pytest.mark.parametrize("objective,F", [(0, 36), (1, 33), (0, 70)])
-def test_quad_groups_of_the_fused_pass(arb, oracle, objective, F):
-    # 33 and 36 features: a group of eight quads and a group of one; 70: three groups
+def test_quad_groups_of_wide_matrices(arb, oracle, objective, F, in_place):
+    # 33 and 36 features: a group of eight quads and a group of one; 70: three groups.  in_place:
+    # rows stay where they are as records and (row id, gradients) are re-ordered (the default for
+    # more than 32 features); otherwise the fused pass moves the rows once per group of quads
     X, y = make_data(20000, F, objective, seed=F, nan_frac=0.05)
-    cfg = {"objective": objective, "method": 1, "internals": {"hist_size": 100, "double_precision": True},
+    cfg = {"objective": objective, "method": 1,
+           "internals": {"hist_size": 100, "double_precision": True, "wide_rows_in_place": in_place},
            "tree": {"max_depth": 6, "eta": 0.3, "lambda": 1.0}}
     assert_same_training(arb, oracle, X, y, cfg, rounds=2)
+
+
+@pytest.mark.parametrize("trick", [True, False])
+@pytest.mark.parametrize("n,F,depth,objective", [(1, 40, 3, 0), (63, 33, 4, 1), (4097, 130, 5, 1), (50000, 200, 7, 0)])
+def test_rows_in_place_shapes(arb, oracle, n, F, depth, objective, trick):
+    # the records path on ragged row counts, record widths that are not a multiple of eight words,
+    # with and without sibling subtraction, inspection on (histograms compared) and off
+    X, y = make_data(n, F, objective, seed=n + F, nan_frac=0.02)
+    cfg = {"objective": objective, "method": 1,
+           "internals": {"hist_size": 63, "double_precision": True, "use_hist_subtraction_trick": trick},
+           "tree": {"max_depth": depth, "eta": 0.3, "lambda": 1.0}}
+    assert_same_training(arb, oracle, X, y, cfg, rounds=2, check_hist=n < 10000)
 
 
 def test_many_trees_without_reading_the_model(arb, oracle):
