@@ -36,15 +36,19 @@ def _run(cmd, verbose):
         print(res.stdout)
 
 
-def build(verbose=False, only=None):
+def build(verbose=False, changed_only=False):
     """Compiles every source to an object file (in parallel) and links them.
-    only: names of the sources to recompile (the other objects must exist)."""
+    changed_only: keep the objects that are newer than their source and every header."""
     os.makedirs(OBJ, exist_ok=True)
     extra = os.environ.get("ARB_EXTRA_FLAGS", "").split()
     objs = [os.path.join(OBJ, os.path.splitext(s)[0] + ".o") for s in SOURCES]
+    headers = [os.path.join(CSRC, f) for f in os.listdir(CSRC) if f.endswith(".h")]
+    headers += [os.path.join(HERE, "..", "include", f) for f in os.listdir(os.path.join(HERE, "..", "include"))]
+    newest_header = max(os.path.getmtime(h) for h in headers)
     jobs = []
     for s, o in zip(SOURCES, objs):
-        if only is not None and s not in only and os.path.exists(o):
+        if changed_only and os.path.exists(o) and \
+                os.path.getmtime(o) > max(newest_header, os.path.getmtime(os.path.join(CSRC, s))):
             continue
         jobs.append([hipcc()] + FLAGS + extra + ["-x", "hip", "-c", os.path.join(CSRC, s), "-o", o])
     with ThreadPoolExecutor(max_workers=min(8, max(1, len(jobs)))) as ex:
@@ -54,4 +58,4 @@ def build(verbose=False, only=None):
 
 
 if __name__ == "__main__":
-    build(verbose=True, only=sys.argv[1:] or None)
+    build(verbose=True, changed_only="--changed" in sys.argv[1:])

@@ -52,6 +52,7 @@ class DataMatrix {
   int hist_size = 0;             // exact method: the largest number of distinct values of a feature
   std::vector<std::vector<float>> thresholds;
   std::vector<int> reduced_size;
+  int max_bin = 255;  // largest bin id in the quantised matrix (the missing-value bin included)
   DeviceMatrix *device = nullptr;
   // Streamed matrices (bins in pinned host blocks instead of HBM): block b
   // holds rows [b * stream_block_rows, ...) as quads [Q][stream_block_rows].

@@ -379,6 +379,28 @@ void QuantiseOnDevice(DataMatrix *data, int hist_size, bool verbose, bool stream
     data->stream_blocks = dm->host_blocks;
     data->stream_block_rows = block_rows;
   }
+  // the largest bin id of the matrix: bin ids from the quantiser stop at a feature's number of
+  // real bins (the missing-value bin), ranks at the largest number of distinct values less one,
+  // bin ids handed in are looked at
+  data->max_bin = 255;
+  if (dm->bits == 8) {
+    if (exact) {
+      data->max_bin = hist_size - 1;
+    } else if (!data->is_prebinned) {
+      data->max_bin = 0;
+      for (int f = 0; f < F; ++f) data->max_bin = std::max(data->max_bin, std::min(data->reduced_size[f], 255));
+    } else if (!data->prebinned.empty()) {
+      std::atomic<int> most{0};
+      ParallelFor(data->prebinned.size(), [&](size_t b, size_t e) {
+        int m = 0;
+        for (size_t i = b; i < e; ++i) m = std::max(m, (int)data->prebinned[i]);
+        int seen = most.load();
+        while (m > seen && !most.compare_exchange_weak(seen, m)) {
+        }
+      });
+      data->max_bin = most;
+    }
+  }
   if (exact) std::vector<uint8_t>().swap(data->prebinned);  // prediction walks the float columns
   data->device = dm.release();
   data->hist_size = hist_size;
@@ -431,27 +453,6 @@ struct RowBuffers {
   float *g = nullptr, *h = nullptr;
   unsigned *ids = nullptr;  // indexed mode: the row at each position (null: position = row)
 };
-
-template <bool PAIR>
-void LaunchHistRec(int nq, hipStream_t st, unsigned grid, const uint32_t *rec, int RS, const unsigned *ids, int q0,
-                   int F, const float *g, const float *h, const int *shifts, const WorkItem *work,
-                   const unsigned *n_work, unsigned long long *slab, int slab_entries) {
-#define ARB_CASE(N)                                                                                              \
-  case N: {                                                                                                      \
-    static bool configured = false;                                                                              \
-    if (!configured) {                                                                                           \
-      AllowLds(k_hist_rec<PAIR, N>, HistLdsBytes(N, PAIR));                                                      \
-      configured = true;                                                                                         \
-    }                                                                                                            \
-    hipLaunchKernelGGL((k_hist_rec<PAIR, N>), dim3(grid), dim3(kHistThreads), HistLdsBytes(N, PAIR), st, rec, RS, \
-                       ids, q0, F, g, h, shifts, work, n_work, slab, slab_entries);                              \
-  } break;
-  switch (nq) {
-    ARB_CASE(1) ARB_CASE(2) ARB_CASE(3) ARB_CASE(4) ARB_CASE(5) ARB_CASE(6) ARB_CASE(7) ARB_CASE(8)
-    default: throw std::runtime_error("internal: bad quad count");
-  }
-#undef ARB_CASE
-}
 
 struct FusedArgs {
   const uint32_t *bins;
@@ -541,7 +542,12 @@ class HipTreeBuilder : public TreeBuilder {
     single_group_ = Q_ <= quads_per_group_;
     // Matrices wider than one group of quads: rows stay in place as records, only (row id,
     // gradients) are re-ordered (kernels_indexed.h).
-    indexed_ = !wide_ && !dm_->streamed && !single_group_ && D_ > 2 && cfg.internal.wide_rows_in_place;
+    // Taken when every feature fits ONE LDS histogram of the bins in use (a record is then read
+    // once per level, whole): e.g. 200 features of 65 bins with one word per cell.
+    rec_slots_ = std::min(kSlots, data->max_bin + 1);
+    const size_t rec_lds = (size_t)HistBlocks(Q_) * kBlockFeatures * rec_slots_ * 8 * (pair_ ? 2 : 1);
+    indexed_ = !wide_ && !dm_->streamed && !single_group_ && D_ > 2 && cfg.internal.wide_rows_in_place &&
+               rec_lds <= kLdsBudget - 1024;
     fused_ = trick_ && !wide_ && !indexed_;
     if (wide_) {
       // features per histogram launch (an even number, two per word)
@@ -919,11 +925,19 @@ class HipTreeBuilder : public TreeBuilder {
     }
     for (int q0 = 0; q0 < Q_; q0 += quads_per_group_) {
       const int nq = std::min(quads_per_group_, Q_ - q0);
-      if (indexed_) {
-        if (pair_)
-          LaunchHistRec<true>(nq, stream_, grid, dm_->rec, dm_->RS, cur.ids, q0, F_, cur.g, cur.h, d_shifts_, d_hwork_, d_nwork_, d_slab_, slab_entries_);
-        else
-          LaunchHistRec<false>(nq, stream_, grid, dm_->rec, dm_->RS, cur.ids, q0, F_, cur.g, cur.h, d_shifts_, d_hwork_, d_nwork_, d_slab_, slab_entries_);
+      if (indexed_) {  // one launch for every feature
+        const size_t lds = (size_t)HistBlocks(Q_) * kBlockFeatures * rec_slots_ * 8 * (pair_ ? 2 : 1);
+        if (pair_) {
+          AllowLds(k_hist_rec<true>, kLdsBudget);
+          hipLaunchKernelGGL(k_hist_rec<true>, dim3(grid), dim3(kHistThreads), lds, stream_, dm_->rec, dm_->RS, cur.ids,
+                             Q_, rec_slots_, cur.g, cur.h, d_shifts_, d_hwork_, d_nwork_, d_slab_);
+        } else {
+          AllowLds(k_hist_rec<false>, kLdsBudget);
+          hipLaunchKernelGGL(k_hist_rec<false>, dim3(grid), dim3(kHistThreads), lds, stream_, dm_->rec, dm_->RS, cur.ids,
+                             Q_, rec_slots_, cur.g, cur.h, d_shifts_, d_hwork_, d_nwork_, d_slab_);
+        }
+        if (timing_) ++(root ? timings_.hist_root_launches : timings_.hist_deep_launches);
+        break;
       } else if (pair_) {
         LaunchHist<true>(nq, stream_, grid, cur.bins, stride_, q0, F_, cur.g, cur.h, d_shifts_, d_hwork_, d_nwork_, d_slab_, slab_entries_);
       } else {
@@ -944,7 +958,8 @@ class HipTreeBuilder : public TreeBuilder {
   hipLaunchKernelGGL((k_hist_reduce<P, LN>), grid, dim3(1024), 0, stream_, d_slab_, slab_entries_, nbin_total_,   \
                      d_node_first_, d_node_items_, by_parent ? 1 : 0, d_split_, d_tot_[parent_state], d_hg_[hb], \
                      d_hh_[hb], d_hc_[hb], d_hg_[hb ^ 1], d_hh_[hb ^ 1], d_hc_[hb ^ 1], trick ? 1 : 0,           \
-                     accumulate ? 1 : 0, wide_ ? 1 : 0, HistBlocks(quads_per_group_))
+                     accumulate ? 1 : 0, wide_ ? 1 : 0, indexed_ ? HistBlocks(Q_) : HistBlocks(quads_per_group_), \
+                     indexed_ ? rec_slots_ : kSlots)
     if (pair_) {
       if (wide_blocks) ARB_REDUCE(true, 4);
       else ARB_REDUCE(true, 16);
@@ -1035,7 +1050,7 @@ class HipTreeBuilder : public TreeBuilder {
           Plan(ps, PL, 0, kPartRows, d_pwork_, d_nwork_ + 1, -1, nullptr, grid);
           Mark(kPartition);
           if (indexed_) {
-            hipLaunchKernelGGL(k_ix_decide, dim3(grid), dim3(kHistThreads), 0, stream_, dm_->rec, dm_->RS, src.ids,
+            hipLaunchKernelGGL(k_ix_decide, dim3(grid), dim3(kHistThreads), 0, stream_, dm_->bins, stride_, src.ids,
                                d_split_, d_pwork_, d_nwork_ + 1, d_dec_, d_wave_left_, d_item_left_);
             if (pair_)
               hipLaunchKernelGGL(k_ix_part<true>, dim3(grid), dim3(kHistThreads), 0, stream_, src.ids, dst.ids, src.g,
@@ -1398,6 +1413,7 @@ class HipTreeBuilder : public TreeBuilder {
   int slab_entries_ = 0;  // histogram entries of one work item's slab (whole 16-feature blocks)
   bool single_group_ = true;  // all quads fit one LDS histogram
   bool indexed_ = false;      // wide matrix: rows stay in place, (row id, gradients) are re-ordered
+  int rec_slots_ = kSlots;    // bins per feature of the one LDS histogram of that mode
   uint8_t *d_dec_ = nullptr;  // indexed mode: split decision of the row at each position
   bool wide_ = false;     // 16-bit bins: two features per word, slots_ histogram slots per feature
   int slots_ = kSlots;

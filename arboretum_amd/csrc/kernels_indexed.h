@@ -43,9 +43,12 @@ k_to_records(const uint32_t *__restrict__ bins, size_t stride, int Q, uint32_t *
 // Split decision of every row of the parents of a level, in node order:
 // dec[p] = 1 when the row at position p goes right (builder.h:107-123), and the
 // rows going left per (work item, wave) as k_part_count gives them.  ids: the
-// row at each position (null: position = row, the first level).
+// row at each position (null: position = row, the first level).  The split
+// feature's word is read from the quad columns, not from the records: the ids of
+// a node ascend, so the reads of a node walk one column forwards, and a column
+// is small enough for the caches to help.
 __global__ void __launch_bounds__(kHistThreads)
-k_ix_decide(const uint32_t *__restrict__ rec, int RS, const unsigned *__restrict__ ids,
+k_ix_decide(const uint32_t *__restrict__ bins, size_t stride, const unsigned *__restrict__ ids,
             const SplitRec *__restrict__ split, const WorkItem *__restrict__ work,
             const unsigned *__restrict__ n_work, uint8_t *__restrict__ dec, unsigned *__restrict__ wave_left,
             unsigned *__restrict__ item_left) {
@@ -68,7 +71,7 @@ k_ix_decide(const uint32_t *__restrict__ rec, int RS, const unsigned *__restrict
       id[k] = ids ? ids[a] : a;
     }
 #pragma unroll
-    for (int k = 0; k < 2 * kBatch; ++k) word[k] = s.fid < 0 ? 0u : rec[(size_t)id[k] * RS + fq];
+    for (int k = 0; k < 2 * kBatch; ++k) word[k] = s.fid < 0 ? 0u : bins[(size_t)fq * stride + id[k]];
 #pragma unroll
     for (int k = 0; k < 2 * kBatch; ++k) {
       const unsigned r = base + (k >> 1) * kChunkStep + (k & 1) * 64 + lane;
@@ -157,54 +160,89 @@ k_ix_part(const unsigned *__restrict__ ids, unsigned *__restrict__ ids_out, cons
   FlushQueue<PAIR, 1, false, true>(nullptr, QR, false, ids_out, 0, g_out, h_out, lane, 0, 0, 0);
 }
 
-// k_hist over records: the row at position p of a work item is ids[p] (null:
-// p itself), its quads [q0, q0 + NQ) are words q0.. of its record (q0 a
-// multiple of 8, records 32-byte aligned: two 16-byte loads per row when
-// NQ = 8), its gradients are g[p], h[p].
-template <bool PAIR, int NQ>
+// Adds one row per lane to an LDS histogram of `blocks` 16-feature blocks and
+// `slots` bins per feature (bin-major: word0 of (feature f, bin) at
+// bin * bin_stride + (f / 16) * (PAIR ? 32 : 16) + f % 16, bin_stride =
+// blocks * (PAIR ? 32 : 16); word1 16 words further): the eight quads b of the
+// row starting at block block0, of which the first nq exist.  The lanes of a
+// 16-lane pass work on 16 different features as in AccumulateRow; a bin id is
+// clamped to the histogram, so that no input can write outside it.
+template <bool PAIR>
+__device__ __forceinline__ void AccumulateQuads8(unsigned long long *__restrict__ lds, const uint32_t (&b)[8],
+                                                 unsigned long long w0, unsigned long long w1,
+                                                 unsigned bin_stride, unsigned block0, int nq, unsigned last_bin) {
+  constexpr unsigned per = PAIR ? 2 : 1;
+  const unsigned j = (threadIdx.x >> 2) & 3u, i = threadIdx.x & 3u;
+#pragma unroll
+  for (int k = 0; k < 2; ++k) {
+    const uint32_t r0 = b[4 * k], r1 = b[4 * k + 1], r2 = b[4 * k + 2], r3 = b[4 * k + 3];
+#pragma unroll
+    for (int s_ = 0; s_ < 4; ++s_) {
+      const unsigned qi = ((unsigned)s_ + j) & 3u;
+      const uint32_t ra = s_ == 0 ? r0 : s_ == 1 ? r1 : s_ == 2 ? r2 : r3;
+      const uint32_t rb = s_ == 0 ? r1 : s_ == 1 ? r2 : s_ == 2 ? r3 : r0;
+      const uint32_t rc = s_ == 0 ? r2 : s_ == 1 ? r3 : s_ == 2 ? r0 : r1;
+      const uint32_t rd = s_ == 0 ? r3 : s_ == 1 ? r0 : s_ == 2 ? r1 : r2;
+      const uint32_t lo = (j & 1u) ? rb : ra, hi = (j & 1u) ? rd : rc;
+      const uint32_t sel = (j & 2u) ? hi : lo;   // quad (s_ + j) % 4 of the block
+      if (4 * k + (int)qi < nq) {
+#pragma unroll
+        for (int t = 0; t < 4; ++t) {
+          const unsigned bi = ((unsigned)t + i) & 3u;
+          const unsigned bin = min(__builtin_amdgcn_ubfe(sel, 8u * bi, 8u), last_bin);
+          unsigned long long *cell = &lds[bin * bin_stride + (block0 + (unsigned)k) * (per * kBlockFeatures) + 4u * qi + bi];
+          atomicAdd(cell, w0);
+          if (PAIR) atomicAdd(cell + kWord1, w1);
+        }
+      }
+    }
+  }
+}
+
+// Histogram over records, every feature in one LDS histogram of `slots` bins
+// per feature (possible when features x slots is small enough: 200 features of
+// 65 bins with one word per cell take 108 KB): the record of a row is read
+// once, whole, eight quads at a time.  The row at position p of a work item
+// is ids[p] (null: p itself), its gradients are g[p], h[p].  The slab of a work
+// item is the LDS image: blocks * 16 * slots entries of one or two words.
+template <bool PAIR>
 __global__ void __launch_bounds__(kHistThreads)
-k_hist_rec(const uint32_t *__restrict__ rec, int RS, const unsigned *__restrict__ ids, int q0, int F,
+k_hist_rec(const uint32_t *__restrict__ rec, int RS, const unsigned *__restrict__ ids, int Q, int slots,
            const float *__restrict__ g, const float *__restrict__ h, const int *__restrict__ shifts,
            const WorkItem *__restrict__ work, const unsigned *__restrict__ n_work,
-           unsigned long long *__restrict__ slab, int slab_entries) {
+           unsigned long long *__restrict__ slab) {
   extern __shared__ unsigned long long lds[];
   const unsigned w = blockIdx.x;
   if (w >= *n_work) return;
   const WorkItem it = work[w];
-  constexpr int words = (int)(HistLdsBytes(NQ, PAIR) / 8);
-  for (int i = threadIdx.x; i < words; i += kHistThreads) lds[i] = 0ull;
+  constexpr unsigned per = PAIR ? 2 : 1;
+  const unsigned blocks = (unsigned)HistBlocks(Q), bin_stride = blocks * per * kBlockFeatures;
+  const unsigned words = (unsigned)slots * bin_stride;
+  for (unsigned i = threadIdx.x; i < words; i += kHistThreads) lds[i] = 0ull;
   __syncthreads();
   const int sg = shifts[0], sh = shifts[1];
-  // ids of the next pair of rows are requested while the current pair is accumulated
-  auto row_at = [&](unsigned r) {
-    const unsigned a = r < it.end ? r : it.begin;
-    return ids ? ids[a] : a;
-  };
-  unsigned n0 = row_at(it.begin + threadIdx.x), n1 = row_at(it.begin + threadIdx.x + kHistThreads);
-  for (unsigned base = it.begin; base < it.end; base += 2 * kHistThreads) {
-    const unsigned r0 = base + threadIdx.x, r1 = r0 + kHistThreads;
-    const bool v0 = r0 < it.end, v1 = r1 < it.end;
-    const unsigned a0 = v0 ? r0 : it.begin, a1 = v1 ? r1 : it.begin;
-    const unsigned id0 = n0, id1 = n1;
-    uint32_t b0[NQ], b1[NQ];
-    const uint32_t *p0 = rec + (size_t)id0 * RS + q0, *p1 = rec + (size_t)id1 * RS + q0;
-#pragma unroll
-    for (int q = 0; q < NQ; ++q) {
-      b0[q] = p0[q];
-      b1[q] = p1[q];
+  const unsigned last_bin = (unsigned)slots - 1u;
+  for (unsigned base = it.begin; base < it.end; base += kHistThreads) {
+    const unsigned r = base + threadIdx.x;
+    const bool v = r < it.end;
+    const unsigned a = v ? r : it.begin;
+    const unsigned id = ids ? ids[a] : a;
+    const uint4 *p = reinterpret_cast<const uint4 *>(rec + (size_t)id * RS);  // records are 32-byte aligned
+    const unsigned long long w0 = (1ull << kCountShift) + (unsigned long long)ToFixed(g[a], sg);
+    const unsigned long long w1 = PAIR ? (unsigned long long)ToFixed(h[a], sh) : 0ull;
+    uint4 lo = p[0], hi = p[1];
+    for (int q0 = 0; q0 < Q; q0 += 8) {
+      const uint32_t b[8] = {lo.x, lo.y, lo.z, lo.w, hi.x, hi.y, hi.z, hi.w};
+      if (q0 + 8 < Q) {  // the next eight quads are on their way while these are accumulated
+        lo = p[(q0 >> 2) + 2];
+        hi = p[(q0 >> 2) + 3];
+      }
+      if (v) AccumulateQuads8<PAIR>(lds, b, w0, w1, bin_stride, (unsigned)(q0 >> 2), min(8, Q - q0), last_bin);
     }
-    n0 = row_at(r0 + 2 * kHistThreads);
-    n1 = row_at(r1 + 2 * kHistThreads);
-    const float g0 = g[a0], g1 = g[a1];
-    float h0 = 0.0f, h1 = 0.0f;
-    if (PAIR) {
-      h0 = h[a0];
-      h1 = h[a1];
-    }
-    if (v0) AccumulateRow<PAIR, NQ>(lds, b0, g0, h0, sg, sh, q0, F);
-    if (v1) AccumulateRow<PAIR, NQ>(lds, b1, g1, h1, sg, sh, q0, F);
   }
-  FlushSlab<PAIR, NQ>(lds, slab, w, slab_entries, q0);
+  __syncthreads();
+  unsigned long long *out = slab + (size_t)w * words;
+  for (unsigned e = threadIdx.x; e < words; e += kHistThreads) out[e] = lds[e];
 }
 
 }  // namespace

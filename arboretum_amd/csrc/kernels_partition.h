@@ -633,7 +633,8 @@ k_hist_reduce(const unsigned long long *__restrict__ slab, int slab_entries, int
               const NodeSum *__restrict__ parent_tot, long long *__restrict__ hg,
               long long *__restrict__ hh, unsigned *__restrict__ hc,
               const long long *__restrict__ pg, const long long *__restrict__ ph,
-              const unsigned *__restrict__ pc, int trick, int accumulate, int plain, int group_blocks) {
+              const unsigned *__restrict__ pc, int trick, int accumulate, int plain, int group_blocks,
+              int lds_slots = kSlots) {
   // LANES threads share the slabs of one entry; a block covers 1024 / LANES
   // consecutive entries (with 4 lanes: 16 bins x 16 features, so the
   // feature-major output is written in runs of 16 bins)
@@ -661,7 +662,11 @@ k_hist_reduce(const unsigned long long *__restrict__ slab, int slab_entries, int
   const int f = (entry / kBlockEntries) * kBlockFeatures + (entry & (kBlockFeatures - 1));
   const int bin = (entry / kBlockFeatures) & (kSlots - 1);
   // the last 16-feature block may have fewer than 16 features
-  const bool live = plain ? entry < nbin_total : f * kSlots < nbin_total;
+  // lds_slots < 256: the slabs hold that many bins per feature only (the rest are empty)
+  const bool live = (plain ? entry < nbin_total : f * kSlots < nbin_total);
+  const bool stored = plain || bin < lds_slots;
+  const size_t slab_words = plain ? (size_t)slab_entries * (PAIR ? 2 : 1)
+                                  : (size_t)slab_entries / kSlots * (size_t)lds_slots * (PAIR ? 2 : 1);
   long long ag = 0, ah = 0;
   unsigned ac = 0;
   if (live) {
@@ -676,8 +681,8 @@ k_hist_reduce(const unsigned long long *__restrict__ slab, int slab_entries, int
       i0 = (unsigned)(group * group_blocks * kBlockEntries) * (PAIR ? 2u : 1u) + HistWord<PAIR>(in_group, blocks_here);
       i1 = i0 + kWord1;
     }
-    for (unsigned s = lane; s < items; s += LANES) {
-      const unsigned long long *p = slab + (size_t)(first + s) * slab_entries * (PAIR ? 2 : 1);
+    for (unsigned s = lane; s < items && stored; s += LANES) {
+      const unsigned long long *p = slab + (size_t)(first + s) * slab_words;
       const unsigned long long w0 = p[i0];
       const long long gq = ((long long)(w0 << (64 - kCountShift))) >> (64 - kCountShift);
       ag += gq;
