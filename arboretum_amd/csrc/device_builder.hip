@@ -547,7 +547,7 @@ class HipTreeBuilder : public TreeBuilder {
     rec_slots_ = std::min(kSlots, data->max_bin + 1);
     const size_t rec_lds = (size_t)HistBlocks(Q_) * kBlockFeatures * rec_slots_ * 8 * (pair_ ? 2 : 1);
     indexed_ = !wide_ && !dm_->streamed && !single_group_ && D_ > 2 && cfg.internal.wide_rows_in_place &&
-               rec_lds <= kLdsBudget - 1024;
+               rec_lds <= kLdsBudget - 1024 && Q_ <= 256;  // a wave reads whole records: at most 64 pieces of 16 bytes
     fused_ = trick_ && !wide_ && !indexed_;
     if (wide_) {
       // features per histogram launch (an even number, two per word)

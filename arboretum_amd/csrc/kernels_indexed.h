@@ -160,51 +160,26 @@ k_ix_part(const unsigned *__restrict__ ids, unsigned *__restrict__ ids_out, cons
   FlushQueue<PAIR, 1, false, true>(nullptr, QR, false, ids_out, 0, g_out, h_out, lane, 0, 0, 0);
 }
 
-// Adds one row per lane to an LDS histogram of `blocks` 16-feature blocks and
-// `slots` bins per feature (bin-major: word0 of (feature f, bin) at
-// bin * bin_stride + (f / 16) * (PAIR ? 32 : 16) + f % 16, bin_stride =
-// blocks * (PAIR ? 32 : 16); word1 16 words further): the eight quads b of the
-// row starting at block block0, of which the first nq exist.  The lanes of a
-// 16-lane pass work on 16 different features as in AccumulateRow; a bin id is
-// clamped to the histogram, so that no input can write outside it.
-template <bool PAIR>
-__device__ __forceinline__ void AccumulateQuads8(unsigned long long *__restrict__ lds, const uint32_t (&b)[8],
-                                                 unsigned long long w0, unsigned long long w1,
-                                                 unsigned bin_stride, unsigned block0, int nq, unsigned last_bin) {
-  constexpr unsigned per = PAIR ? 2 : 1;
-  const unsigned j = (threadIdx.x >> 2) & 3u, i = threadIdx.x & 3u;
-#pragma unroll
-  for (int k = 0; k < 2; ++k) {
-    const uint32_t r0 = b[4 * k], r1 = b[4 * k + 1], r2 = b[4 * k + 2], r3 = b[4 * k + 3];
-#pragma unroll
-    for (int s_ = 0; s_ < 4; ++s_) {
-      const unsigned qi = ((unsigned)s_ + j) & 3u;
-      const uint32_t ra = s_ == 0 ? r0 : s_ == 1 ? r1 : s_ == 2 ? r2 : r3;
-      const uint32_t rb = s_ == 0 ? r1 : s_ == 1 ? r2 : s_ == 2 ? r3 : r0;
-      const uint32_t rc = s_ == 0 ? r2 : s_ == 1 ? r3 : s_ == 2 ? r0 : r1;
-      const uint32_t rd = s_ == 0 ? r3 : s_ == 1 ? r0 : s_ == 2 ? r1 : r2;
-      const uint32_t lo = (j & 1u) ? rb : ra, hi = (j & 1u) ? rd : rc;
-      const uint32_t sel = (j & 2u) ? hi : lo;   // quad (s_ + j) % 4 of the block
-      if (4 * k + (int)qi < nq) {
-#pragma unroll
-        for (int t = 0; t < 4; ++t) {
-          const unsigned bi = ((unsigned)t + i) & 3u;
-          const unsigned bin = min(__builtin_amdgcn_ubfe(sel, 8u * bi, 8u), last_bin);
-          unsigned long long *cell = &lds[bin * bin_stride + (block0 + (unsigned)k) * (per * kBlockFeatures) + 4u * qi + bi];
-          atomicAdd(cell, w0);
-          if (PAIR) atomicAdd(cell + kWord1, w1);
-        }
-      }
-    }
-  }
-}
-
 // Histogram over records, every feature in one LDS histogram of `slots` bins
 // per feature (possible when features x slots is small enough: 200 features of
 // 65 bins with one word per cell take 108 KB): the record of a row is read
-// once, whole, eight quads at a time.  The row at position p of a work item
-// is ids[p] (null: p itself), its gradients are g[p], h[p].  The slab of a work
-// item is the LDS image: blocks * 16 * slots entries of one or two words.
+// once, whole.  The row at position p of a work item is ids[p] (null: p itself),
+// its gradients are g[p], h[p].
+//
+// A lane owns one 16-byte piece of a record, i.e. one 16-feature block of one
+// row: consecutive lanes read consecutive pieces, so a wave reads 64 / P whole
+// records per load (P = pieces per record) as contiguous runs.  One row per lane
+// would touch 64 records 16 bytes at a time and come back to each of them P
+// times, with far more data in flight than the caches hold.  The 16 updates of
+// a lane go to features (t + lane) % 16 of its block in step t, so the 16 lanes
+// of a pass of the LDS atomic unit still hit 16 different bank pairs, whatever
+// rows and blocks they own.
+//
+// LDS layout (bin-major, as the other histograms): word0 of (feature f, bin) at
+// bin * bin_stride + (f / 16) * (PAIR ? 32 : 16) + f % 16, bin_stride = blocks *
+// (PAIR ? 32 : 16), word1 16 words further.  A bin id is clamped to the
+// histogram, so that no input can write outside it.  The slab of a work item is
+// the LDS image: blocks * 16 * slots entries of one or two words.
 template <bool PAIR>
 __global__ void __launch_bounds__(kHistThreads)
 k_hist_rec(const uint32_t *__restrict__ rec, int RS, const unsigned *__restrict__ ids, int Q, int slots,
@@ -222,22 +197,60 @@ k_hist_rec(const uint32_t *__restrict__ rec, int RS, const unsigned *__restrict_
   __syncthreads();
   const int sg = shifts[0], sh = shifts[1];
   const unsigned last_bin = (unsigned)slots - 1u;
-  for (unsigned base = it.begin; base < it.end; base += kHistThreads) {
-    const unsigned r = base + threadIdx.x;
-    const bool v = r < it.end;
-    const unsigned a = v ? r : it.begin;
-    const unsigned id = ids ? ids[a] : a;
-    const uint4 *p = reinterpret_cast<const uint4 *>(rec + (size_t)id * RS);  // records are 32-byte aligned
-    const unsigned long long w0 = (1ull << kCountShift) + (unsigned long long)ToFixed(g[a], sg);
-    const unsigned long long w1 = PAIR ? (unsigned long long)ToFixed(h[a], sh) : 0ull;
-    uint4 lo = p[0], hi = p[1];
-    for (int q0 = 0; q0 < Q; q0 += 8) {
-      const uint32_t b[8] = {lo.x, lo.y, lo.z, lo.w, hi.x, hi.y, hi.z, hi.w};
-      if (q0 + 8 < Q) {  // the next eight quads are on their way while these are accumulated
-        lo = p[(q0 >> 2) + 2];
-        hi = p[(q0 >> 2) + 3];
+  const unsigned lane = threadIdx.x & 63u, wave = threadIdx.x >> 6;
+  const unsigned P = (unsigned)RS / 4u;          // pieces per record; the host keeps P <= 64
+  const unsigned rpw = 64u / P;                   // rows a wave reads per load
+  const unsigned my_row = lane / P, piece = lane % P;
+  const bool lane_on = my_row < rpw && piece < blocks;
+  const unsigned j = (lane >> 2) & 3u, i4 = lane & 3u;
+  unsigned long long *cell0 = lds + piece * (per * kBlockFeatures);
+  constexpr int kSteps = 4;                       // row groups in flight per wave
+  const unsigned group = rpw * kItemWaves;        // rows of the workgroup per step
+  for (unsigned base = it.begin + wave * rpw; base < it.end; base += kSteps * group) {
+    unsigned id[kSteps];
+    bool v[kSteps];
+#pragma unroll
+    for (int k = 0; k < kSteps; ++k) {
+      const unsigned r = base + (unsigned)k * group + my_row;
+      v[k] = lane_on && r < it.end && base + (unsigned)k * group < it.end;
+      const unsigned a = v[k] ? r : it.begin;
+      id[k] = ids ? ids[a] : a;
+    }
+    uint4 q[kSteps];
+    float gv[kSteps], hv[kSteps];
+#pragma unroll
+    for (int k = 0; k < kSteps; ++k) {
+      const unsigned r = base + (unsigned)k * group + my_row;
+      const unsigned a = v[k] ? r : it.begin;
+      q[k] = *reinterpret_cast<const uint4 *>(rec + (size_t)id[k] * RS + 4u * (lane_on ? piece : 0u));
+      gv[k] = g[a];
+      hv[k] = PAIR ? h[a] : 0.0f;
+    }
+#pragma unroll
+    for (int k = 0; k < kSteps; ++k) {
+      if (!v[k]) continue;
+      const unsigned long long w0 = (1ull << kCountShift) + (unsigned long long)ToFixed(gv[k], sg);
+      const unsigned long long w1 = PAIR ? (unsigned long long)ToFixed(hv[k], sh) : 0ull;
+#pragma unroll
+      for (int s_ = 0; s_ < 4; ++s_) {
+        const unsigned qi = ((unsigned)s_ + j) & 3u;   // quad of the block this lane works on
+        const uint32_t ra = s_ == 0 ? q[k].x : s_ == 1 ? q[k].y : s_ == 2 ? q[k].z : q[k].w;
+        const uint32_t rb = s_ == 0 ? q[k].y : s_ == 1 ? q[k].z : s_ == 2 ? q[k].w : q[k].x;
+        const uint32_t rc = s_ == 0 ? q[k].z : s_ == 1 ? q[k].w : s_ == 2 ? q[k].x : q[k].y;
+        const uint32_t rd = s_ == 0 ? q[k].w : s_ == 1 ? q[k].x : s_ == 2 ? q[k].y : q[k].z;
+        const uint32_t lo = (j & 1u) ? rb : ra, hi = (j & 1u) ? rd : rc;
+        const uint32_t sel = (j & 2u) ? hi : lo;
+        if (4u * piece + qi < (unsigned)Q) {           // quads past the matrix do not exist
+#pragma unroll
+          for (int t = 0; t < 4; ++t) {
+            const unsigned bi = ((unsigned)t + i4) & 3u;
+            const unsigned bin = min(__builtin_amdgcn_ubfe(sel, 8u * bi, 8u), last_bin);
+            unsigned long long *cell = cell0 + bin * bin_stride + 4u * qi + bi;
+            atomicAdd(cell, w0);
+            if (PAIR) atomicAdd(cell + kWord1, w1);
+          }
+        }
       }
-      if (v) AccumulateQuads8<PAIR>(lds, b, w0, w1, bin_stride, (unsigned)(q0 >> 2), min(8, Q - q0), last_bin);
     }
   }
   __syncthreads();

@@ -201,12 +201,11 @@ def make_config3(rows, features=100, classes=10, seed=3):
     return X, labels
 
 
-def other_config(args, arb):
-    """BASELINE configs[2] / configs[3] at full size: seconds per tree (not the headline metric;
-    prints its own JSON line)."""
+def other_config(arb, workload, rows_arg, steps):
+    """BASELINE configs[2] / configs[3] at full size: seconds per tree (not the headline metric)."""
     t0 = time.perf_counter()
-    if args.workload == "config2":
-        rows = args.rows if args.rows != 10_500_000 else 50_000_000
+    if workload == "config2":
+        rows = rows_arg if rows_arg != 10_500_000 else 50_000_000
         F = 200
         bins, y = make_config2_bins(rows, F)
         data = arb.DMatrix(bins, y=y, quantized=True)
@@ -215,7 +214,7 @@ def other_config(args, arb):
                "tree": {"max_depth": 10, "eta": 0.3, "lambda": 1.0}}
         trees_per_round, name = 1, "configs[2]: %d x 200, 64 bins + missing bin (30 %%), squared error, max_depth 10" % rows
     else:
-        rows = args.rows if args.rows != 10_500_000 else 20_000_000
+        rows = rows_arg if rows_arg != 10_500_000 else 20_000_000
         F, K = 100, 10
         X, labels = make_config3(rows, F, K)
         data = arb.DMatrix(X, labels=labels)
@@ -231,16 +230,16 @@ def other_config(args, arb):
     t_first = time.perf_counter() - t0
     s0 = model.rows_scanned()
     t0 = time.perf_counter()
-    for _ in range(args.steps):
+    for _ in range(steps):
         model.grow_tree()
     model.synchronize()
     dt = time.perf_counter() - t0
     scanned = model.rows_scanned() - s0
-    trees = args.steps * trees_per_round
-    print(json.dumps({"metric": "seconds per tree", "workload": name, "rows": rows, "features": F,
-                      "rounds": args.steps, "trees": trees, "sec_per_tree": dt / trees, "sec_per_round": dt / args.steps,
-                      "hist_updates_per_s": scanned * F / dt, "first_round_with_quantisation_s": t_first,
-                      "generate_s": t_gen}))
+    trees = steps * trees_per_round
+    return {"metric": "seconds per tree", "workload": name, "rows": rows, "features": F,
+            "rounds": steps, "trees": trees, "sec_per_tree": dt / trees, "sec_per_round": dt / steps,
+            "hist_updates_per_s": scanned * F / dt, "first_round_with_quantisation_s": t_first,
+            "generate_s": t_gen}
 
 
 def cpu_baseline(X, y, cfg, sample_rows, trees):
@@ -275,6 +274,8 @@ def main():
     ap.add_argument("--cpu-rows", type=int, default=10_500_000)
     ap.add_argument("--cpu-trees", type=int, default=16)
     ap.add_argument("--no-cpu", action="store_true")
+    ap.add_argument("--no-other-configs", action="store_true",
+                    help="skip the full-size runs of BASELINE configs[2] and configs[3] reported under other_configs")
     ap.add_argument("--nan-frac", type=float, default=0.0,
                     help="stress variant: this fraction of the feature values is replaced by NaN (all land in "
                          "one bin per feature; needs --hist-size <= 255)")
@@ -302,7 +303,7 @@ def main():
         stream_mode(args, arb)
         return
     if args.workload != "headline":
-        other_config(args, arb)
+        print(json.dumps(other_config(arb, args.workload, args.rows, args.steps)))
         return
 
     X, y = make_workload(args.rows, args.features)
@@ -441,6 +442,11 @@ def main():
     }
     if not args.no_cpu and args.cpu_trees > 0:
         out["cpu_baseline"] = cpu_baseline(X, y, cfg, min(args.cpu_rows, args.rows), args.cpu_trees)
+    if not args.no_other_configs and (R, F, args.hist_size, D) == (10500000, 28, 256, 8):
+        # the wide configurations at their full sizes, a few trees each (seconds per tree only)
+        del model, data, X, y
+        out["other_configs"] = {"configs[2]": other_config(arb, "config2", 10_500_000, 3),
+                                "configs[3]": other_config(arb, "config3", 10_500_000, 2)}
     print(json.dumps(out))
 
 
