@@ -562,7 +562,9 @@ class HipTreeBuilder : public TreeBuilder {
     streamed_ = dm_->streamed;
     // Logistic gradients of 0/1 labels travel as one float per row (PackGrad):
     // there is no h array then, and kernels given h == nullptr unpack g.
-    pack_ = cfg.objective == kLogisticRegression && !streamed_ && !wide_ && Q_ <= kMaxGroupQuads && data->y.size() == n_ &&
+    // (never together with rows kept in place: those kernels take g and h as two arrays)
+    pack_ = cfg.objective == kLogisticRegression && !streamed_ && !wide_ && !indexed_ && Q_ <= kMaxGroupQuads &&
+            data->y.size() == n_ &&
             std::all_of(data->y.begin(), data->y.end(), [](float v) { return v == 0.0f || v == 1.0f; });
     d_g_ = DevAlloc<float>(n_ * K_);
     d_h_ = pack_ ? nullptr : DevAlloc<float>(n_ * K_);

@@ -33,7 +33,7 @@ ROOT = os.path.dirname(os.path.abspath(__file__))
 sys.path.insert(0, ROOT)
 
 HBM_PEAK = 8.0e12  # bytes/s, MI355X
-TRAFFIC_PROFILE = os.path.join(ROOT, "profiles", "hbm_traffic_config2_10.5Mx28_depth8.txt")
+TRAFFIC_PROFILE = os.path.join(ROOT, "profiles", "hbm_traffic_headline_10.5Mx28_depth8.txt")
 KERNEL_SOURCES = ["kernels_partition.h", "kernels_hist.h", "device_common.h"]
 
 
