@@ -608,6 +608,7 @@ class HipTreeBuilder : public TreeBuilder {
       if (!dm_->rec) {  // records: 32-byte aligned, built once per matrix
         dm_->RS = (Q_ + 7) / 8 * 8;
         dm_->rec = DevAlloc<uint32_t>(n_ * (size_t)dm_->RS);
+        AllowLds(k_to_records, (size_t)64 * (dm_->RS + 1) * sizeof(uint32_t));
         hipLaunchKernelGGL(k_to_records, dim3((unsigned)((n_ + 63) / 64)), dim3(256),
                            (size_t)64 * (dm_->RS + 1) * sizeof(uint32_t), stream_, dm_->bins, stride_, Q_, dm_->rec,
                            dm_->RS, n_);

@@ -204,40 +204,55 @@ k_hist_rec(const uint32_t *__restrict__ rec, int RS, const unsigned *__restrict_
   const bool lane_on = my_row < rpw && piece < blocks;
   const unsigned j = (lane >> 2) & 3u, i4 = lane & 3u;
   unsigned long long *cell0 = lds + piece * (per * kBlockFeatures);
-  constexpr int kSteps = 4;                       // row groups in flight per wave
-  const unsigned group = rpw * kItemWaves;        // rows of the workgroup per step
-  for (unsigned base = it.begin + wave * rpw; base < it.end; base += kSteps * group) {
-    unsigned id[kSteps];
-    bool v[kSteps];
-#pragma unroll
-    for (int k = 0; k < kSteps; ++k) {
-      const unsigned r = base + (unsigned)k * group + my_row;
-      v[k] = lane_on && r < it.end && base + (unsigned)k * group < it.end;
-      const unsigned a = v[k] ? r : it.begin;
-      id[k] = ids ? ids[a] : a;
-    }
+  constexpr int kSteps = 4;                       // row groups per wave and step
+  const unsigned group = rpw * kItemWaves;        // rows of the workgroup per group
+  const unsigned step = kSteps * group;
+  // One step of a wave: the row ids of its kSteps groups, then their record pieces and
+  // gradients, then the updates.  The three stages of consecutive steps overlap: while the
+  // updates of a step run, the records of the next one and the row ids of the one after are in
+  // flight.  Loads are issued for steps that begin inside the work item only, and every address
+  // is clamped to a row of the item.
+  struct RowIds { unsigned id[kSteps]; };
+  struct Pieces {
     uint4 q[kSteps];
     float gv[kSteps], hv[kSteps];
+    bool v[kSteps];
+  };
+  auto position = [&](unsigned base, int k, bool *valid) {
+    const unsigned r = base + (unsigned)k * group + my_row;
+    *valid = lane_on && r < it.end && base + (unsigned)k * group < it.end;
+    return *valid ? r : it.begin;
+  };
+  auto load_ids = [&](unsigned base, RowIds &I) {
 #pragma unroll
     for (int k = 0; k < kSteps; ++k) {
-      const unsigned r = base + (unsigned)k * group + my_row;
-      const unsigned a = v[k] ? r : it.begin;
-      q[k] = *reinterpret_cast<const uint4 *>(rec + (size_t)id[k] * RS + 4u * (lane_on ? piece : 0u));
-      gv[k] = g[a];
-      hv[k] = PAIR ? h[a] : 0.0f;
+      bool valid;
+      const unsigned a = position(base, k, &valid);
+      I.id[k] = ids ? ids[a] : a;
     }
+  };
+  auto load_pieces = [&](unsigned base, const RowIds &I, Pieces &R) {
 #pragma unroll
     for (int k = 0; k < kSteps; ++k) {
-      if (!v[k]) continue;
-      const unsigned long long w0 = (1ull << kCountShift) + (unsigned long long)ToFixed(gv[k], sg);
-      const unsigned long long w1 = PAIR ? (unsigned long long)ToFixed(hv[k], sh) : 0ull;
+      const unsigned a = position(base, k, &R.v[k]);
+      R.q[k] = *reinterpret_cast<const uint4 *>(rec + (size_t)I.id[k] * RS + 4u * (lane_on ? piece : 0u));
+      R.gv[k] = g[a];
+      R.hv[k] = PAIR ? h[a] : 0.0f;
+    }
+  };
+  auto accumulate = [&](const Pieces &R) {
+#pragma unroll
+    for (int k = 0; k < kSteps; ++k) {
+      if (!R.v[k]) continue;
+      const unsigned long long w0 = (1ull << kCountShift) + (unsigned long long)ToFixed(R.gv[k], sg);
+      const unsigned long long w1 = PAIR ? (unsigned long long)ToFixed(R.hv[k], sh) : 0ull;
 #pragma unroll
       for (int s_ = 0; s_ < 4; ++s_) {
         const unsigned qi = ((unsigned)s_ + j) & 3u;   // quad of the block this lane works on
-        const uint32_t ra = s_ == 0 ? q[k].x : s_ == 1 ? q[k].y : s_ == 2 ? q[k].z : q[k].w;
-        const uint32_t rb = s_ == 0 ? q[k].y : s_ == 1 ? q[k].z : s_ == 2 ? q[k].w : q[k].x;
-        const uint32_t rc = s_ == 0 ? q[k].z : s_ == 1 ? q[k].w : s_ == 2 ? q[k].x : q[k].y;
-        const uint32_t rd = s_ == 0 ? q[k].w : s_ == 1 ? q[k].x : s_ == 2 ? q[k].y : q[k].z;
+        const uint32_t ra = s_ == 0 ? R.q[k].x : s_ == 1 ? R.q[k].y : s_ == 2 ? R.q[k].z : R.q[k].w;
+        const uint32_t rb = s_ == 0 ? R.q[k].y : s_ == 1 ? R.q[k].z : s_ == 2 ? R.q[k].w : R.q[k].x;
+        const uint32_t rc = s_ == 0 ? R.q[k].z : s_ == 1 ? R.q[k].w : s_ == 2 ? R.q[k].x : R.q[k].y;
+        const uint32_t rd = s_ == 0 ? R.q[k].w : s_ == 1 ? R.q[k].x : s_ == 2 ? R.q[k].y : R.q[k].z;
         const uint32_t lo = (j & 1u) ? rb : ra, hi = (j & 1u) ? rd : rc;
         const uint32_t sel = (j & 2u) ? hi : lo;
         if (4u * piece + qi < (unsigned)Q) {           // quads past the matrix do not exist
@@ -251,6 +266,27 @@ k_hist_rec(const uint32_t *__restrict__ rec, int RS, const unsigned *__restrict_
           }
         }
       }
+    }
+  };
+  unsigned base = it.begin + wave * rpw;
+  if (base < it.end) {                            // wave-uniform, as every branch below
+    RowIds I;
+    Pieces R;
+    load_ids(base, I);
+    load_pieces(base, I, R);
+    unsigned next = base + step;
+    if (next < it.end) load_ids(next, I);
+    for (;;) {
+      const bool more = next < it.end;
+      Pieces N;
+      if (more) {
+        load_pieces(next, I, N);
+        if (next + step < it.end) load_ids(next + step, I);
+      }
+      accumulate(R);
+      if (!more) break;
+      R = N;
+      next += step;
     }
   }
   __syncthreads();

@@ -313,7 +313,7 @@ def test_quad_groups_of_wide_matrices(arb, oracle, objective, F, in_place):
 
 
 @pytest.mark.parametrize("trick", [True, False])
-@pytest.mark.parametrize("n,F,depth,objective", [(1, 40, 3, 0), (63, 33, 4, 1), (4097, 130, 5, 1), (50000, 200, 7, 0)])
+@pytest.mark.parametrize("n,F,depth,objective", [(1, 40, 3, 0), (63, 33, 4, 1), (4097, 130, 5, 1), (50000, 200, 7, 0), (3000, 300, 4, 0)])
 def test_rows_in_place_shapes(arb, oracle, n, F, depth, objective, trick):
     # the records path on ragged row counts, record widths that are not a multiple of eight words,
     # with and without sibling subtraction, inspection on (histograms compared) and off
@@ -322,6 +322,14 @@ def test_rows_in_place_shapes(arb, oracle, n, F, depth, objective, trick):
            "internals": {"hist_size": 63, "double_precision": True, "use_hist_subtraction_trick": trick},
            "tree": {"max_depth": depth, "eta": 0.3, "lambda": 1.0}}
     assert_same_training(arb, oracle, X, y, cfg, rounds=2, check_hist=n < 10000)
+
+
+def test_rows_in_place_thousand_features(arb, oracle):
+    # 1000 features of at most 8 bins: records of 256 words, a wave reads one record at a time
+    X, y = make_data(2000, 1000, 0, seed=1000, nan_frac=0.02)
+    cfg = {"objective": 0, "method": 1, "internals": {"hist_size": 7, "double_precision": True},
+           "tree": {"max_depth": 3, "eta": 0.3, "lambda": 1.0}}
+    assert_same_training(arb, oracle, X, y, cfg, rounds=2)
 
 
 def test_many_trees_without_reading_the_model(arb, oracle):
