@@ -244,6 +244,91 @@ def test_exact_root_split_against_brute_force(oracle, objective, seed):
     assert np.array_equal(b.leaf(), (X[:, f] >= thr).astype(np.uint32))
 
 
+@pytest.mark.parametrize("objective", [0, 1])
+@pytest.mark.parametrize("seed", range(6))
+def test_hist_root_split_against_brute_force(oracle, objective, seed):
+    # The histogram method chooses among the bins what the exact search chooses among the values
+    # when the bin ids are taken as the values: left of a candidate are the rows of the bins up to
+    # it, equal gains go to the highest bin (empty bins included, so the winner is the bin just
+    # below the first bin that goes right), then to the lowest feature; NaN sits in the last bin
+    # and always goes right.
+    rng = np.random.default_rng(300 + seed)
+    n, F = 80, 5
+    X = np.round(rng.normal(size=(n, F)) * 2).astype(np.float32)          # few distinct values: empty bins
+    X[:, 2] = rng.normal(size=n).astype(np.float32)
+    X[rng.random((n, F)) < 0.1] = np.nan
+    s = np.nan_to_num(X[:, 0]) + np.nan_to_num(X[:, 2])
+    y = (s > 0).astype(np.float32) if objective else (2 * s + rng.normal(size=n)).astype(np.float32)
+    cfg = {"objective": objective, "method": 1, "internals": {"hist_size": 16, "double_precision": True},
+           "tree": {"max_depth": 1, "eta": 1.0, "lambda": 0.5, "min_child_weight": 0.0, "min_leaf_size": 1,
+                    "initial_y": 0.5}}
+    b = oracle.Booster(X, y=y, config=cfg, accum=1)
+    b.grow(1)
+    g, h = b.grad()
+    if objective == 0:
+        h = np.ones_like(g)
+    bins = b.bins().astype(np.float32)
+    f, first_right, gain = _brute_force_exact_root(oracle, bins, g, h, 1 if objective == 0 else 3,
+                                                   (1, 0.0, 0.0, 0.0, 0.5, 0.0))
+    t = b.tree(0)
+    assert f >= 0 and t["fid"][0] == f
+    assert t["quantized"][0] == int(first_right) - 1
+    assert t["gain"][0] == pytest.approx(gain, rel=1e-6)
+    assert np.array_equal(b.leaf(), (bins[:, f] >= first_right).astype(np.uint32))
+    # the threshold reported is the one prediction needs: raw values below it are the left rows
+    thr = t["threshold"][0]
+    assert np.array_equal(X[:, f] < thr, bins[:, f] < first_right)
+
+
+@pytest.mark.parametrize("objective", [0, 1])
+@pytest.mark.parametrize("seed", range(4))
+def test_hist_tree_against_node_by_node_brute_force(oracle, objective, seed):
+    # A whole tree of depth 3, node by node in heap order: every node's split from the brute-force
+    # search over its own rows, rows below the first right bin to child 2i+1 (left) and the others
+    # to 2i+2, an unsplit or empty node sends everything left and is recorded as fid 0 / bin -1,
+    # leaf weight = eta * G / (H + lambda) of the leaf's rows (H = row count for squared error).
+    rng = np.random.default_rng(400 + seed)
+    n, F, depth, lam, eta = 120, 4, 3, 0.5, 0.7
+    X = np.round(rng.normal(size=(n, F)) * 2).astype(np.float32)
+    X[:, 1] = rng.normal(size=n).astype(np.float32)
+    s = X[:, 0] - X[:, 1] * X[:, 2]
+    y = (s > 0).astype(np.float32) if objective else (s + 0.3 * rng.normal(size=n)).astype(np.float32)
+    cfg = {"objective": objective, "method": 1, "internals": {"hist_size": 12, "double_precision": True},
+           "tree": {"max_depth": depth, "eta": eta, "lambda": lam, "min_child_weight": 0.0, "min_leaf_size": 1,
+                    "initial_y": 0.5}}
+    b = oracle.Booster(X, y=y, config=cfg, accum=1)
+    b.grow(1)
+    g, h = b.grad()
+    if objective == 0:
+        h = np.ones_like(g)
+    bins = b.bins().astype(np.float32)
+    t = b.tree(0)
+    rows = {0: np.arange(n)}
+    for i in range((1 << depth) - 1):
+        r = rows[i]
+        f, first_right = -1, None
+        if len(r) > 1:
+            f, first_right, gain = _brute_force_exact_root(oracle, bins[r], g[r], h[r], 1 if objective == 0 else 3,
+                                                           (1, 0.0, 0.0, 0.0, lam, 0.0))
+        if f >= 0:
+            assert (t["fid"][i], t["quantized"][i]) == (f, int(first_right) - 1), "node %d" % i
+            assert t["gain"][i] == pytest.approx(gain, rel=1e-5)
+            right = bins[r, f] >= first_right
+        else:
+            assert t["quantized"][i] == -1 and t["fid"][i] == 0 and np.isinf(t["threshold"][i]), "node %d" % i
+            right = np.zeros(len(r), bool)
+        rows[2 * i + 1], rows[2 * i + 2] = r[~right], r[right]
+    first_leaf = (1 << depth) - 1
+    leaf = np.empty(n, np.uint32)
+    for k in range(1 << depth):
+        r = rows[first_leaf + k]
+        leaf[r] = k
+        if len(r):
+            G, H = g[r].astype(np.float64).sum(), h[r].astype(np.float64).sum()
+            assert t["weights"][k] == pytest.approx(eta * G / (H + lam), rel=1e-5, abs=1e-7), "leaf %d" % k
+    assert np.array_equal(b.leaf(), leaf)
+
+
 def test_golden_regression_boston(oracle):
     fx = load_golden("hist_regression_boston10.json")
     _run_cases(oracle, fx, np.array(fx["X"], np.float32), np.array(fx["y"], np.float32))
