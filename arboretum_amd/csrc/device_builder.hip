@@ -632,6 +632,16 @@ class HipTreeBuilder : public TreeBuilder {
     const size_t plan_rows = dm_->streamed ? std::min(n_, dm_->block_rows) : n_;
     max_hist_items_ = (unsigned)(plan_rows / HistRowsPerItem(plan_rows)) + 2 * last_nodes + 2;
     max_hist_items_ = std::max<unsigned>(max_hist_items_, 1024 + 2 * last_nodes + 2);
+    {
+      hipDeviceProp_t prop;
+      int dev = 0;
+      HIP_OK(hipGetDevice(&dev));
+      HIP_OK(hipGetDeviceProperties(&prop, dev));
+      cus_ = (unsigned)std::max(prop.multiProcessorCount, 1);
+      // the balanced plans of un-fused histogram launches: whole rounds of cus_ items
+      for (int level = 0; level + 1 < D_; ++level)
+        max_hist_items_ = std::max(max_hist_items_, BalancedPlanItems(plan_rows, 1u << level, kMaxHistRows, cus_));
+    }
     max_part_items_ = std::max<unsigned>((unsigned)(plan_rows / kPartRows + 1) + 2 * last_nodes, max_hist_items_);
     d_hwork_ = DevAlloc<WorkItem>(max_hist_items_);
     d_pwork_ = DevAlloc<WorkItem>(max_part_items_);
@@ -890,23 +900,27 @@ class HipTreeBuilder : public TreeBuilder {
   unsigned long long *ScanCounter(int level) { return d_rows_scanned_ + std::min(level, kScanLevels - 1); }
   // count_level >= 0: the planned rows are histogram work of that tree level
   void Plan(int state, int L, int select, unsigned rows_per_item, WorkItem *work, unsigned *n_work,
-            int count_level, const SplitRec *split, unsigned max_items) {
-    PlanOn(d_tot_[state], d_seg_[state], L, select, rows_per_item, work, n_work, count_level, split, max_items);
+            int count_level, const SplitRec *split, unsigned max_items, unsigned balance_cus = 0) {
+    PlanOn(d_tot_[state], d_seg_[state], L, select, rows_per_item, work, n_work, count_level, split, max_items,
+           balance_cus);
   }
   void PlanOn(const NodeSum *tot, const unsigned *seg, int L, int select, unsigned rows_per_item, WorkItem *work,
-              unsigned *n_work, int count_level, const SplitRec *split, unsigned max_items) {
+              unsigned *n_work, int count_level, const SplitRec *split, unsigned max_items,
+              unsigned balance_cus = 0) {
     hipLaunchKernelGGL(k_plan, dim3(1), dim3(1024), 0, stream_, tot, seg, L, select,
                        rows_per_item, work, n_work, d_node_first_, d_node_items_,
-                       count_level >= 0 ? ScanCounter(count_level) : (unsigned long long *)nullptr, split, max_items, d_overflow_);
+                       count_level >= 0 ? ScanCounter(count_level) : (unsigned long long *)nullptr, split, max_items,
+                       d_overflow_, balance_cus);
   }
 
   // Histograms of contiguous node ranges in `cur` (level order), feature group by group.
   void HistOfNodes(const RowBuffers &cur, int state, int L, bool select_smaller, size_t rows_max, bool root, int level) {
-    // the root level is one node: one item per CU avoids a second, partial round
-    const unsigned per_item = HistRowsPerItem(rows_max, root ? 256 : 512);
-    const unsigned grid = (unsigned)std::min<size_t>(rows_max / per_item + 2 * L + 1, max_hist_items_);
+    // A CU holds one work item at a time, so the launch runs in rounds of cus_ items: the planner
+    // sizes the items from the rows and nodes it finds selected so that the rounds are full
+    // (one item per CU at the root); the grid holds the rounds of the largest case.
+    const unsigned grid = std::min(BalancedPlanItems(rows_max, (unsigned)L, kMaxHistRows, cus_), max_hist_items_);
     Mark(kPlan);
-    Plan(state, L, select_smaller ? 1 : 0, per_item, d_hwork_, d_nwork_, level, nullptr, grid);
+    Plan(state, L, select_smaller ? 1 : 0, kMaxHistRows, d_hwork_, d_nwork_, level, nullptr, grid, cus_);
     Mark(root ? kHistRoot : kHistDeep);
     if (wide_) {
       for (int f0 = 0; f0 < F_; f0 += wide_group_) {
@@ -1414,6 +1428,7 @@ class HipTreeBuilder : public TreeBuilder {
   size_t n_ = 0, stride_ = 0;
   int F_ = 0, Q_ = 0, K_ = 1, D_ = 2, nbin_total_ = 0;
   int slab_entries_ = 0;  // histogram entries of one work item's slab (whole 16-feature blocks)
+  unsigned cus_ = 256;        // compute units of the device
   bool single_group_ = true;  // all quads fit one LDS histogram
   bool indexed_ = false;      // wide matrix: rows stay in place, (row id, gradients) are re-ordered
   int rec_slots_ = kSlots;    // bins per feature of the one LDS histogram of that mode

@@ -156,7 +156,7 @@ void Enqueue(const HistSumArgs &a, const Shape &sh, unsigned char *mem, unsigned
                      a.shift_h, s.tot, s.seg, s.n_work, s.overflow, s.shifts, status);
   hipLaunchKernelGGL(k_plan, dim3(1), dim3(1024), 0, st, s.tot, s.seg, a.nodes, a.use_trick ? 1 : 0, per_item, s.work,
                      s.n_work, s.node_first, s.node_items, (unsigned long long *)nullptr, (const SplitRec *)nullptr,
-                     max_items, s.overflow);
+                     max_items, s.overflow, 0u);
   const unsigned grid = (unsigned)std::min<size_t>((size_t)a.nrow / per_item + 2 * (size_t)a.nodes + 1, max_items);
   for (int q0 = 0; q0 < sh.Q; q0 += sh.quads_per_group) {
     const int nq = std::min(sh.quads_per_group, sh.Q - q0);

@@ -167,13 +167,14 @@ k_ix_part(const unsigned *__restrict__ ids, unsigned *__restrict__ ids_out, cons
 // its gradients are g[p], h[p].
 //
 // A lane owns one 16-byte piece of a record, i.e. one 16-feature block of one
-// row: consecutive lanes read consecutive pieces, so a wave reads 64 / P whole
-// records per load (P = pieces per record) as contiguous runs.  One row per lane
-// would touch 64 records 16 bytes at a time and come back to each of them P
-// times, with far more data in flight than the caches hold.  The 16 updates of
-// a lane go to features (t + lane) % 16 of its block in step t, so the 16 lanes
-// of a pass of the LDS atomic unit still hit 16 different bank pairs, whatever
-// rows and blocks they own.
+// row: the (row, piece) pairs of a work item are dealt to the lanes in row-major
+// order, so consecutive lanes read consecutive pieces and a wave's load covers
+// whole records as contiguous runs, with every lane busy whatever the number of
+// pieces per record.  One row per lane would touch 64 records 16 bytes at a time
+// and come back to each of them once per piece, with far more data in flight
+// than the caches hold.  The 16 updates of a lane go to features (t + lane) % 16
+// of its block in step t, so the 16 lanes of a pass of the LDS atomic unit still
+// hit 16 different bank pairs, whatever rows and blocks they own.
 //
 // LDS layout (bin-major, as the other histograms): word0 of (feature f, bin) at
 // bin * bin_stride + (f / 16) * (PAIR ? 32 : 16) + f % 16, bin_stride = blocks *
@@ -198,52 +199,65 @@ k_hist_rec(const uint32_t *__restrict__ rec, int RS, const unsigned *__restrict_
   const int sg = shifts[0], sh = shifts[1];
   const unsigned last_bin = (unsigned)slots - 1u;
   const unsigned lane = threadIdx.x & 63u, wave = threadIdx.x >> 6;
-  const unsigned P = (unsigned)RS / 4u;          // pieces per record; the host keeps P <= 64
-  const unsigned rpw = 64u / P;                   // rows a wave reads per load
-  const unsigned my_row = lane / P, piece = lane % P;
-  const bool lane_on = my_row < rpw && piece < blocks;
   const unsigned j = (lane >> 2) & 3u, i4 = lane & 3u;
-  unsigned long long *cell0 = lds + piece * (per * kBlockFeatures);
-  constexpr int kSteps = 4;                       // row groups per wave and step
-  const unsigned group = rpw * kItemWaves;        // rows of the workgroup per group
-  const unsigned step = kSteps * group;
+  // The (row, piece) pairs of the work item, row-major, are dealt out 64 at a time: wave v takes
+  // pairs [1024 G + 64 v, + 64) of group G, its lane l the pair 1024 G + 64 v + l.  Every lane has
+  // work until the item runs out, however many pieces a record has.
+  const unsigned n_rows = it.end - it.begin;
+  const unsigned n_pairs = n_rows * blocks;                  // at most 64512 x 64 < 2^22
+  const unsigned inv_blocks = (unsigned)(((1ull << 32) + blocks - 1u) / blocks);  // exact quotients below 2^22
+  constexpr int kSteps = 4;                       // groups per wave and step
+  constexpr unsigned kGroupPairs = kItemWaves * 64u;
+  constexpr unsigned kStepPairs = kSteps * kGroupPairs;
   // One step of a wave: the row ids of its kSteps groups, then their record pieces and
   // gradients, then the updates.  The three stages of consecutive steps overlap: while the
   // updates of a step run, the records of the next one and the row ids of the one after are in
   // flight.  Loads are issued for steps that begin inside the work item only, and every address
-  // is clamped to a row of the item.
+  // is clamped to a row of the item and a piece of a record.
   struct RowIds { unsigned id[kSteps]; };
   struct Pieces {
     uint4 q[kSteps];
     float gv[kSteps], hv[kSteps];
+    unsigned piece[kSteps];
     bool v[kSteps];
   };
-  auto position = [&](unsigned base, int k, bool *valid) {
-    const unsigned r = base + (unsigned)k * group + my_row;
-    *valid = lane_on && r < it.end && base + (unsigned)k * group < it.end;
-    return *valid ? r : it.begin;
+  // position in the item's row range and piece of this lane's pair in group k of the step at `first`
+  auto locate = [&](unsigned first, int k, unsigned *piece, bool *valid) {
+    const unsigned pair = first + (unsigned)k * kGroupPairs + wave * 64u + lane;
+    *valid = pair < n_pairs;
+    const unsigned pr = *valid ? pair : 0u;
+    const unsigned rel = min(blocks == 1u ? pr : __umulhi(pr, inv_blocks), n_rows - 1u);   // pair / blocks
+    *piece = min(pr - rel * blocks, blocks - 1u);
+    return it.begin + rel;
   };
-  auto load_ids = [&](unsigned base, RowIds &I) {
+  auto load_ids = [&](unsigned first, RowIds &I) {
 #pragma unroll
     for (int k = 0; k < kSteps; ++k) {
+      unsigned piece;
       bool valid;
-      const unsigned a = position(base, k, &valid);
+      const unsigned a = locate(first, k, &piece, &valid);
       I.id[k] = ids ? ids[a] : a;
     }
   };
-  auto load_pieces = [&](unsigned base, const RowIds &I, Pieces &R) {
+  auto load_pieces = [&](unsigned first, const RowIds &I, Pieces &R) {
 #pragma unroll
     for (int k = 0; k < kSteps; ++k) {
-      const unsigned a = position(base, k, &R.v[k]);
-      R.q[k] = *reinterpret_cast<const uint4 *>(rec + (size_t)I.id[k] * RS + 4u * (lane_on ? piece : 0u));
+      const unsigned a = locate(first, k, &R.piece[k], &R.v[k]);
+      R.q[k] = *reinterpret_cast<const uint4 *>(rec + (size_t)I.id[k] * RS + 4u * R.piece[k]);
       R.gv[k] = g[a];
       R.hv[k] = PAIR ? h[a] : 0.0f;
     }
   };
+  unsigned char *lds_b = reinterpret_cast<unsigned char *>(lds);
+  const unsigned bin_stride_b = bin_stride * 8u;    // at most 64 x 2 x 16 x 8 = 16 KB
   auto accumulate = [&](const Pieces &R) {
 #pragma unroll
     for (int k = 0; k < kSteps; ++k) {
       if (!R.v[k]) continue;
+      // byte offsets into the histogram; the products fit 24 bits (v_mad_u32_u24 is a
+      // full-rate instruction, a 32-bit multiply takes four times as long)
+      const unsigned piece_b = R.piece[k] * (per * kBlockFeatures * 8u);
+      const unsigned piece = R.piece[k];
       const unsigned long long w0 = (1ull << kCountShift) + (unsigned long long)ToFixed(R.gv[k], sg);
       const unsigned long long w1 = PAIR ? (unsigned long long)ToFixed(R.hv[k], sh) : 0ull;
 #pragma unroll
@@ -260,7 +274,8 @@ k_hist_rec(const uint32_t *__restrict__ rec, int RS, const unsigned *__restrict_
           for (int t = 0; t < 4; ++t) {
             const unsigned bi = ((unsigned)t + i4) & 3u;
             const unsigned bin = min(__builtin_amdgcn_ubfe(sel, 8u * bi, 8u), last_bin);
-            unsigned long long *cell = cell0 + bin * bin_stride + 4u * qi + bi;
+            const unsigned off = __umul24(bin, bin_stride_b) + (piece_b + (4u * qi + bi) * 8u);
+            unsigned long long *cell = reinterpret_cast<unsigned long long *>(lds_b + off);
             atomicAdd(cell, w0);
             if (PAIR) atomicAdd(cell + kWord1, w1);
           }
@@ -268,25 +283,24 @@ k_hist_rec(const uint32_t *__restrict__ rec, int RS, const unsigned *__restrict_
       }
     }
   };
-  unsigned base = it.begin + wave * rpw;
-  if (base < it.end) {                            // wave-uniform, as every branch below
+  if (n_pairs != 0) {                             // uniform over the workgroup, as every branch below
     RowIds I;
     Pieces R;
-    load_ids(base, I);
-    load_pieces(base, I, R);
-    unsigned next = base + step;
-    if (next < it.end) load_ids(next, I);
+    load_ids(0u, I);
+    load_pieces(0u, I, R);
+    unsigned next = kStepPairs;
+    if (next < n_pairs) load_ids(next, I);
     for (;;) {
-      const bool more = next < it.end;
+      const bool more = next < n_pairs;
       Pieces N;
       if (more) {
         load_pieces(next, I, N);
-        if (next + step < it.end) load_ids(next + step, I);
+        if (next + kStepPairs < n_pairs) load_ids(next + kStepPairs, I);
       }
       accumulate(R);
       if (!more) break;
       R = N;
-      next += step;
+      next += kStepPairs;
     }
   }
   __syncthreads();
