@@ -547,7 +547,8 @@ class HipTreeBuilder : public TreeBuilder {
     rec_slots_ = std::min(kSlots, data->max_bin + 1);
     const size_t rec_lds = (size_t)HistBlocks(Q_) * kBlockFeatures * rec_slots_ * 8 * (pair_ ? 2 : 1);
     indexed_ = !wide_ && !dm_->streamed && !single_group_ && D_ > 2 && cfg.internal.wide_rows_in_place &&
-               rec_lds <= kLdsBudget - 1024 && Q_ <= 256;  // a wave reads whole records: at most 64 pieces of 16 bytes
+               Q_ <= 256;  // at most 64 pieces of 16 bytes per record
+    rec_one_launch_ = rec_lds <= kLdsBudget - 1024;  // else groups of quads_per_group_ quads at 256 bins
     fused_ = trick_ && !wide_ && !indexed_;
     if (wide_) {
       // features per histogram launch (an even number, two per word)
@@ -639,8 +640,12 @@ class HipTreeBuilder : public TreeBuilder {
       HIP_OK(hipGetDeviceProperties(&prop, dev));
       cus_ = (unsigned)std::max(prop.multiProcessorCount, 1);
       // the balanced plans of un-fused histogram launches: whole rounds of cus_ items
+      // records read once per group of quads: the groups of a work item run side by side, on
+      // that many compute units
+      rec_groups_ = rec_one_launch_ ? 1 : (HistBlocks(Q_) + HistBlocks(quads_per_group_) - 1) / HistBlocks(quads_per_group_);
+      hist_cus_ = indexed_ ? std::max(1u, cus_ / (unsigned)rec_groups_) : cus_;
       for (int level = 0; level + 1 < D_; ++level)
-        max_hist_items_ = std::max(max_hist_items_, BalancedPlanItems(plan_rows, 1u << level, kMaxHistRows, cus_));
+        max_hist_items_ = std::max(max_hist_items_, BalancedPlanItems(plan_rows, 1u << level, kMaxHistRows, hist_cus_));
     }
     max_part_items_ = std::max<unsigned>((unsigned)(plan_rows / kPartRows + 1) + 2 * last_nodes, max_hist_items_);
     d_hwork_ = DevAlloc<WorkItem>(max_hist_items_);
@@ -918,9 +923,9 @@ class HipTreeBuilder : public TreeBuilder {
     // A CU holds one work item at a time, so the launch runs in rounds of cus_ items: the planner
     // sizes the items from the rows and nodes it finds selected so that the rounds are full
     // (one item per CU at the root); the grid holds the rounds of the largest case.
-    const unsigned grid = std::min(BalancedPlanItems(rows_max, (unsigned)L, kMaxHistRows, cus_), max_hist_items_);
+    const unsigned grid = std::min(BalancedPlanItems(rows_max, (unsigned)L, kMaxHistRows, hist_cus_), max_hist_items_);
     Mark(kPlan);
-    Plan(state, L, select_smaller ? 1 : 0, kMaxHistRows, d_hwork_, d_nwork_, level, nullptr, grid, cus_);
+    Plan(state, L, select_smaller ? 1 : 0, kMaxHistRows, d_hwork_, d_nwork_, level, nullptr, grid, hist_cus_);
     Mark(root ? kHistRoot : kHistDeep);
     if (wide_) {
       for (int f0 = 0; f0 < F_; f0 += wide_group_) {
@@ -942,16 +947,28 @@ class HipTreeBuilder : public TreeBuilder {
     }
     for (int q0 = 0; q0 < Q_; q0 += quads_per_group_) {
       const int nq = std::min(quads_per_group_, Q_ - q0);
-      if (indexed_) {  // one launch for every feature
-        const size_t lds = (size_t)HistBlocks(Q_) * kBlockFeatures * rec_slots_ * 8 * (pair_ ? 2 : 1);
+      if (indexed_) {
+        // one launch: every feature in one LDS histogram at rec_slots_ bins, or the groups of
+        // quads at 256 bins side by side (a workgroup per work item and group)
+        const int total = HistBlocks(Q_);
+        const int pieces = rec_one_launch_ ? total : HistBlocks(quads_per_group_);
+        const int ngroups = (total + pieces - 1) / pieces;
+        const int slots = rec_one_launch_ ? rec_slots_ : kSlots;
+        const size_t lds = (size_t)pieces * kBlockFeatures * slots * 8 * (pair_ ? 2 : 1);
+        const size_t item_words = rec_one_launch_ ? lds / 8 : (size_t)slab_entries_ * (pair_ ? 2 : 1);
+        if (lds > kLdsBudget || (size_t)total * 4 > (size_t)dm_->RS || ngroups != rec_groups_)
+          throw std::runtime_error("internal: record histogram launch does not fit");
+        const unsigned blocks = (grid + 7u) / 8u * 8u * (unsigned)ngroups;
         if (pair_) {
           AllowLds(k_hist_rec<true>, kLdsBudget);
-          hipLaunchKernelGGL(k_hist_rec<true>, dim3(grid), dim3(kHistThreads), lds, stream_, dm_->rec, dm_->RS, cur.ids,
-                             Q_, rec_slots_, cur.g, cur.h, d_shifts_, d_hwork_, d_nwork_, d_slab_);
+          hipLaunchKernelGGL(k_hist_rec<true>, dim3(blocks), dim3(kHistThreads), lds, stream_, dm_->rec, dm_->RS,
+                             cur.ids, Q_, slots, cur.g, cur.h, d_shifts_, d_hwork_, d_nwork_, d_slab_, pieces, total,
+                             ngroups, item_words);
         } else {
           AllowLds(k_hist_rec<false>, kLdsBudget);
-          hipLaunchKernelGGL(k_hist_rec<false>, dim3(grid), dim3(kHistThreads), lds, stream_, dm_->rec, dm_->RS, cur.ids,
-                             Q_, rec_slots_, cur.g, cur.h, d_shifts_, d_hwork_, d_nwork_, d_slab_);
+          hipLaunchKernelGGL(k_hist_rec<false>, dim3(blocks), dim3(kHistThreads), lds, stream_, dm_->rec, dm_->RS,
+                             cur.ids, Q_, slots, cur.g, cur.h, d_shifts_, d_hwork_, d_nwork_, d_slab_, pieces, total,
+                             ngroups, item_words);
         }
         if (timing_) ++(root ? timings_.hist_root_launches : timings_.hist_deep_launches);
         break;
@@ -975,8 +992,9 @@ class HipTreeBuilder : public TreeBuilder {
   hipLaunchKernelGGL((k_hist_reduce<P, LN>), grid, dim3(1024), 0, stream_, d_slab_, slab_entries_, nbin_total_,   \
                      d_node_first_, d_node_items_, by_parent ? 1 : 0, d_split_, d_tot_[parent_state], d_hg_[hb], \
                      d_hh_[hb], d_hc_[hb], d_hg_[hb ^ 1], d_hh_[hb ^ 1], d_hc_[hb ^ 1], trick ? 1 : 0,           \
-                     accumulate ? 1 : 0, wide_ ? 1 : 0, indexed_ ? HistBlocks(Q_) : HistBlocks(quads_per_group_), \
-                     indexed_ ? rec_slots_ : kSlots)
+                     accumulate ? 1 : 0, wide_ ? 1 : 0,                                                           \
+                     indexed_ && rec_one_launch_ ? HistBlocks(Q_) : HistBlocks(quads_per_group_),                \
+                     indexed_ && rec_one_launch_ ? rec_slots_ : kSlots)
     if (pair_) {
       if (wide_blocks) ARB_REDUCE(true, 4);
       else ARB_REDUCE(true, 16);
@@ -1429,9 +1447,12 @@ class HipTreeBuilder : public TreeBuilder {
   int F_ = 0, Q_ = 0, K_ = 1, D_ = 2, nbin_total_ = 0;
   int slab_entries_ = 0;  // histogram entries of one work item's slab (whole 16-feature blocks)
   unsigned cus_ = 256;        // compute units of the device
+  unsigned hist_cus_ = 256;   // work items of an un-fused histogram launch that run at a time
+  int rec_groups_ = 1;        // groups of quads a record is read in (rows in place)
   bool single_group_ = true;  // all quads fit one LDS histogram
   bool indexed_ = false;      // wide matrix: rows stay in place, (row id, gradients) are re-ordered
   int rec_slots_ = kSlots;    // bins per feature of the one LDS histogram of that mode
+  bool rec_one_launch_ = true;  // every feature fits one LDS histogram at rec_slots_ bins
   uint8_t *d_dec_ = nullptr;  // indexed mode: split decision of the row at each position
   bool wide_ = false;     // 16-bit bins: two features per word, slots_ histogram slots per feature
   int slots_ = kSlots;

@@ -176,6 +176,14 @@ k_ix_part(const unsigned *__restrict__ ids, unsigned *__restrict__ ids_out, cons
 // of its block in step t, so the 16 lanes of a pass of the LDS atomic unit still
 // hit 16 different bank pairs, whatever rows and blocks they own.
 //
+// A workgroup covers the pieces [piece0, piece0 + npieces) of the records of its work item: all
+// of them when the whole histogram fits the LDS at `slots` bins per feature (one group; the slab
+// of a work item is the LDS image, item_words its size), else one of `ngroups` groups of
+// group_pieces 16-feature blocks at 256 bins per feature; the slab of a work item then holds
+// the images of the groups one after the other, as the histogram kernels of row-moving
+// matrices write them (item_words = words of all groups).  The grid is ngroups times the number
+// of work items rounded up to a multiple of eight.
+//
 // LDS layout (bin-major, as the other histograms): word0 of (feature f, bin) at
 // bin * bin_stride + (f / 16) * (PAIR ? 32 : 16) + f % 16, bin_stride = blocks *
 // (PAIR ? 32 : 16), word1 16 words further.  A bin id is clamped to the
@@ -186,13 +194,21 @@ __global__ void __launch_bounds__(kHistThreads)
 k_hist_rec(const uint32_t *__restrict__ rec, int RS, const unsigned *__restrict__ ids, int Q, int slots,
            const float *__restrict__ g, const float *__restrict__ h, const int *__restrict__ shifts,
            const WorkItem *__restrict__ work, const unsigned *__restrict__ n_work,
-           unsigned long long *__restrict__ slab) {
+           unsigned long long *__restrict__ slab, int group_pieces, int total_pieces, int ngroups,
+           size_t item_words) {
   extern __shared__ unsigned long long lds[];
-  const unsigned w = blockIdx.x;
+  // Workgroup -> (work item, group of pieces): workgroups are dealt to the eight XCDs in turn
+  // (workgroup b runs on XCD b % 8), and the groups of one work item read the same records, so
+  // they are given ids that differ by 8: they start together on the same XCD, and what the first
+  // of them fetches the others find in that XCD's L2.
+  const unsigned xcd = blockIdx.x & 7u, turn = blockIdx.x >> 3;
+  const unsigned w = (turn / (unsigned)ngroups) * 8u + xcd;
   if (w >= *n_work) return;
+  const int piece0 = (int)(turn % (unsigned)ngroups) * group_pieces;
+  const int npieces = min(group_pieces, total_pieces - piece0);
   const WorkItem it = work[w];
   constexpr unsigned per = PAIR ? 2 : 1;
-  const unsigned blocks = (unsigned)HistBlocks(Q), bin_stride = blocks * per * kBlockFeatures;
+  const unsigned blocks = (unsigned)npieces, bin_stride = blocks * per * kBlockFeatures;
   const unsigned words = (unsigned)slots * bin_stride;
   for (unsigned i = threadIdx.x; i < words; i += kHistThreads) lds[i] = 0ull;
   __syncthreads();
@@ -243,7 +259,7 @@ k_hist_rec(const uint32_t *__restrict__ rec, int RS, const unsigned *__restrict_
 #pragma unroll
     for (int k = 0; k < kSteps; ++k) {
       const unsigned a = locate(first, k, &R.piece[k], &R.v[k]);
-      R.q[k] = *reinterpret_cast<const uint4 *>(rec + (size_t)I.id[k] * RS + 4u * R.piece[k]);
+      R.q[k] = *reinterpret_cast<const uint4 *>(rec + (size_t)I.id[k] * RS + 4u * ((unsigned)piece0 + R.piece[k]));
       R.gv[k] = g[a];
       R.hv[k] = PAIR ? h[a] : 0.0f;
     }
@@ -269,7 +285,7 @@ k_hist_rec(const uint32_t *__restrict__ rec, int RS, const unsigned *__restrict_
         const uint32_t rd = s_ == 0 ? R.q[k].w : s_ == 1 ? R.q[k].x : s_ == 2 ? R.q[k].y : R.q[k].z;
         const uint32_t lo = (j & 1u) ? rb : ra, hi = (j & 1u) ? rd : rc;
         const uint32_t sel = (j & 2u) ? hi : lo;
-        if (4u * piece + qi < (unsigned)Q) {           // quads past the matrix do not exist
+        if (4u * ((unsigned)piece0 + piece) + qi < (unsigned)Q) {   // quads past the matrix do not exist
 #pragma unroll
           for (int t = 0; t < 4; ++t) {
             const unsigned bi = ((unsigned)t + i4) & 3u;
@@ -304,7 +320,7 @@ k_hist_rec(const uint32_t *__restrict__ rec, int RS, const unsigned *__restrict_
     }
   }
   __syncthreads();
-  unsigned long long *out = slab + (size_t)w * words;
+  unsigned long long *out = slab + (size_t)w * item_words + (size_t)piece0 * (kBlockEntries * per);
   for (unsigned e = threadIdx.x; e < words; e += kHistThreads) out[e] = lds[e];
 }
 

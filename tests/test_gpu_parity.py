@@ -324,6 +324,19 @@ def test_rows_in_place_shapes(arb, oracle, n, F, depth, objective, trick):
     assert_same_training(arb, oracle, X, y, cfg, rounds=2, check_hist=n < 10000)
 
 
+@pytest.mark.parametrize("trick", [True, False])
+@pytest.mark.parametrize("n,F,depth,objective,hist", [(4097, 100, 5, 1, 255), (20000, 33, 6, 0, 256),
+                                                      (63, 130, 4, 1, 200), (30000, 70, 6, 1, 256)])
+def test_rows_in_place_in_groups(arb, oracle, n, F, depth, objective, hist, trick):
+    # histograms too large for one LDS: the records are read once per group of 32 features (one
+    # or two 16-byte pieces per launch), 256 bins per feature; the last group holds fewer blocks
+    X, y = make_data(n, F, objective, seed=n + F + 1, nan_frac=0.02)
+    cfg = {"objective": objective, "method": 1,
+           "internals": {"hist_size": hist, "double_precision": True, "use_hist_subtraction_trick": trick},
+           "tree": {"max_depth": depth, "eta": 0.3, "lambda": 1.0}}
+    assert_same_training(arb, oracle, X, y, cfg, rounds=2, check_hist=n < 10000)
+
+
 def test_rows_in_place_thousand_features(arb, oracle):
     # 1000 features of at most 8 bins: records of 256 words, a wave reads one record at a time
     X, y = make_data(2000, 1000, 0, seed=1000, nan_frac=0.02)
