@@ -959,17 +959,21 @@ class HipTreeBuilder : public TreeBuilder {
         if (lds > kLdsBudget || (size_t)total * 4 > (size_t)dm_->RS || ngroups != rec_groups_)
           throw std::runtime_error("internal: record histogram launch does not fit");
         const unsigned blocks = (grid + 7u) / 8u * 8u * (unsigned)ngroups;
-        if (pair_) {
-          AllowLds(k_hist_rec<true>, kLdsBudget);
-          hipLaunchKernelGGL(k_hist_rec<true>, dim3(blocks), dim3(kHistThreads), lds, stream_, dm_->rec, dm_->RS,
-                             cur.ids, Q_, slots, cur.g, cur.h, d_shifts_, d_hwork_, d_nwork_, d_slab_, pieces, total,
-                             ngroups, item_words);
-        } else {
-          AllowLds(k_hist_rec<false>, kLdsBudget);
-          hipLaunchKernelGGL(k_hist_rec<false>, dim3(blocks), dim3(kHistThreads), lds, stream_, dm_->rec, dm_->RS,
-                             cur.ids, Q_, slots, cur.g, cur.h, d_shifts_, d_hwork_, d_nwork_, d_slab_, pieces, total,
-                             ngroups, item_words);
-        }
+        // 256 bins and every group (the last may hold fewer blocks) a power of two of blocks
+        const int last_pieces = total - (ngroups - 1) * pieces;
+        const bool full = slots == kSlots && (pieces & (pieces - 1)) == 0 && (last_pieces & (last_pieces - 1)) == 0;
+#define ARB_REC(P, FULL)                                                                                          \
+  do {                                                                                                            \
+    AllowLds((k_hist_rec<P, FULL>), kLdsBudget);                                                                  \
+    hipLaunchKernelGGL((k_hist_rec<P, FULL>), dim3(blocks), dim3(kHistThreads), lds, stream_, dm_->rec, dm_->RS,  \
+                       cur.ids, Q_, slots, cur.g, cur.h, d_shifts_, d_hwork_, d_nwork_, d_slab_, pieces, total,   \
+                       ngroups, item_words);                                                                      \
+  } while (0)
+        if (pair_ && full) ARB_REC(true, true);
+        else if (pair_) ARB_REC(true, false);
+        else if (full) ARB_REC(false, true);
+        else ARB_REC(false, false);
+#undef ARB_REC
         if (timing_) ++(root ? timings_.hist_root_launches : timings_.hist_deep_launches);
         break;
       } else if (pair_) {

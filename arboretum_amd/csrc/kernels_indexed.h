@@ -189,7 +189,9 @@ k_ix_part(const unsigned *__restrict__ ids, unsigned *__restrict__ ids_out, cons
 // (PAIR ? 32 : 16), word1 16 words further.  A bin id is clamped to the
 // histogram, so that no input can write outside it.  The slab of a work item is
 // the LDS image: blocks * 16 * slots entries of one or two words.
-template <bool PAIR>
+// FULL: 256 bins per feature and a power of two of bytes between bins (stride_shift): the
+// offset of a cell is a shift and an add, and no bin id can leave the histogram.
+template <bool PAIR, bool FULL = false>
 __global__ void __launch_bounds__(kHistThreads)
 k_hist_rec(const uint32_t *__restrict__ rec, int RS, const unsigned *__restrict__ ids, int Q, int slots,
            const float *__restrict__ g, const float *__restrict__ h, const int *__restrict__ shifts,
@@ -266,6 +268,7 @@ k_hist_rec(const uint32_t *__restrict__ rec, int RS, const unsigned *__restrict_
   };
   unsigned char *lds_b = reinterpret_cast<unsigned char *>(lds);
   const unsigned bin_stride_b = bin_stride * 8u;    // at most 64 x 2 x 16 x 8 = 16 KB
+  const unsigned stride_shift = 31u - (unsigned)__clz((int)bin_stride_b);   // FULL: bin_stride_b = 1 << stride_shift
   auto accumulate = [&](const Pieces &R) {
 #pragma unroll
     for (int k = 0; k < kSteps; ++k) {
@@ -289,8 +292,13 @@ k_hist_rec(const uint32_t *__restrict__ rec, int RS, const unsigned *__restrict_
 #pragma unroll
           for (int t = 0; t < 4; ++t) {
             const unsigned bi = ((unsigned)t + i4) & 3u;
-            const unsigned bin = min(__builtin_amdgcn_ubfe(sel, 8u * bi, 8u), last_bin);
-            const unsigned off = __umul24(bin, bin_stride_b) + (piece_b + (4u * qi + bi) * 8u);
+            unsigned off;
+            if (FULL) {
+              off = (__builtin_amdgcn_ubfe(sel, 8u * bi, 8u) << stride_shift) + (piece_b + (4u * qi + bi) * 8u);
+            } else {
+              const unsigned bin = min(__builtin_amdgcn_ubfe(sel, 8u * bi, 8u), last_bin);
+              off = __umul24(bin, bin_stride_b) + (piece_b + (4u * qi + bi) * 8u);
+            }
             unsigned long long *cell = reinterpret_cast<unsigned long long *>(lds_b + off);
             atomicAdd(cell, w0);
             if (PAIR) atomicAdd(cell + kWord1, w1);
