@@ -646,6 +646,7 @@ class HipTreeBuilder : public TreeBuilder {
       hist_cus_ = indexed_ ? std::max(1u, cus_ / (unsigned)rec_groups_) : cus_;
       for (int level = 0; level + 1 < D_; ++level)
         max_hist_items_ = std::max(max_hist_items_, BalancedPlanItems(plan_rows, 1u << level, kMaxHistRows, hist_cus_));
+      max_hist_items_ = std::max(max_hist_items_, BalancedPlanItems(plan_rows, 1u, kMaxHistRows, cus_));
     }
     max_part_items_ = std::max<unsigned>((unsigned)(plan_rows / kPartRows + 1) + 2 * last_nodes, max_hist_items_);
     d_hwork_ = DevAlloc<WorkItem>(max_hist_items_);
@@ -923,9 +924,14 @@ class HipTreeBuilder : public TreeBuilder {
     // A CU holds one work item at a time, so the launch runs in rounds of cus_ items: the planner
     // sizes the items from the rows and nodes it finds selected so that the rounds are full
     // (one item per CU at the root); the grid holds the rounds of the largest case.
-    const unsigned grid = std::min(BalancedPlanItems(rows_max, (unsigned)L, kMaxHistRows, hist_cus_), max_hist_items_);
+    // Rows in place in groups of quads: the root, whose rows are the matrix in its own order,
+    // is read from the quad columns like a narrow matrix (one launch per group streams its
+    // columns once; the groups of the record kernel share only half of their reads there).
+    const bool records = indexed_ && (rec_one_launch_ || !root);
+    const unsigned cus = records ? hist_cus_ : cus_;
+    const unsigned grid = std::min(BalancedPlanItems(rows_max, (unsigned)L, kMaxHistRows, cus), max_hist_items_);
     Mark(kPlan);
-    Plan(state, L, select_smaller ? 1 : 0, kMaxHistRows, d_hwork_, d_nwork_, level, nullptr, grid, hist_cus_);
+    Plan(state, L, select_smaller ? 1 : 0, kMaxHistRows, d_hwork_, d_nwork_, level, nullptr, grid, cus);
     Mark(root ? kHistRoot : kHistDeep);
     if (wide_) {
       for (int f0 = 0; f0 < F_; f0 += wide_group_) {
@@ -947,7 +953,7 @@ class HipTreeBuilder : public TreeBuilder {
     }
     for (int q0 = 0; q0 < Q_; q0 += quads_per_group_) {
       const int nq = std::min(quads_per_group_, Q_ - q0);
-      if (indexed_) {
+      if (records) {
         // one launch: every feature in one LDS histogram at rec_slots_ bins, or the groups of
         // quads at 256 bins side by side (a workgroup per work item and group)
         const int total = HistBlocks(Q_);
