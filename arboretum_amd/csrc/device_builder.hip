@@ -624,6 +624,11 @@ class HipTreeBuilder : public TreeBuilder {
       d_hg_[b] = DevAlloc<long long>((size_t)last_nodes * nbin_total_);
       d_hh_[b] = DevAlloc<long long>((size_t)last_nodes * nbin_total_);
       d_hc_[b] = DevAlloc<unsigned>((size_t)last_nodes * nbin_total_);
+      // cells of bins that no row can have are never written (rows in place with fewer than 256
+      // bins in use) and must read as zero
+      HIP_OK(hipMemsetAsync(d_hg_[b], 0, (size_t)last_nodes * nbin_total_ * sizeof(long long), stream_));
+      HIP_OK(hipMemsetAsync(d_hh_[b], 0, (size_t)last_nodes * nbin_total_ * sizeof(long long), stream_));
+      HIP_OK(hipMemsetAsync(d_hc_[b], 0, (size_t)last_nodes * nbin_total_ * sizeof(unsigned), stream_));
     }
     d_split_ = DevAlloc<SplitRec>(last_nodes);
     d_cand_ = DevAlloc<Cand>((size_t)last_nodes * F_);

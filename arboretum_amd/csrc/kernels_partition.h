@@ -694,7 +694,8 @@ k_hist_reduce(const unsigned long long *__restrict__ slab, int slab_entries, int
   s_h[lane][e] = ah;
   s_c[lane][e] = ac;
   __syncthreads();
-  if (lane == 0 && live) {
+  // cells of bins the slabs do not hold are zero in every node histogram, once and for all
+  if (lane == 0 && live && stored) {
     for (int k = 1; k < LANES; ++k) {
       ag += s_g[k][e];
       ah += s_h[k][e];

@@ -41,9 +41,12 @@ __device__ __forceinline__ Cand ScanFeature(const long long *__restrict__ hg, co
       unsigned long long c4[4];
 #pragma unroll
       for (int j = 0; j < 4; ++j) {
-        g4[j] = hg[base + j];
-        h4[j] = PAIR ? hh[base + j] : 0;
-        c4[j] = hc[base + j];
+        // the slots from hist_size on (missing values, unused slots) are no candidates and in no
+        // candidate's prefix
+        const bool read = chunk + lane * 4 + j < hist_size;
+        g4[j] = read ? hg[base + j] : 0;
+        h4[j] = PAIR && read ? hh[base + j] : 0;
+        c4[j] = read ? hc[base + j] : 0;
       }
 #pragma unroll
       for (int j = 1; j < 4; ++j) {
