@@ -1002,14 +1002,18 @@ class HipTreeBuilder : public TreeBuilder {
     // many nodes: few slabs per node and the output dominates -> longer output runs per block
     const bool wide_blocks = L >= 32;
     const int entries = wide_blocks ? 256 : 64;
-    dim3 grid((slab_entries_ + entries - 1) / entries, L);
+    const int lds_slots = indexed_ && rec_one_launch_ ? rec_slots_ : kSlots;
+    // 16-bit bins: feature-major slabs; else the entries of the bins in use of every 16-feature block
+    dim3 grid(wide_ ? (slab_entries_ + entries - 1) / entries
+                    : slab_entries_ / kBlockEntries * ((lds_slots * kBlockFeatures + entries - 1) / entries),
+              L);
 #define ARB_REDUCE(P, LN)                                                                                          \
   hipLaunchKernelGGL((k_hist_reduce<P, LN>), grid, dim3(1024), 0, stream_, d_slab_, slab_entries_, nbin_total_,   \
                      d_node_first_, d_node_items_, by_parent ? 1 : 0, d_split_, d_tot_[parent_state], d_hg_[hb], \
                      d_hh_[hb], d_hc_[hb], d_hg_[hb ^ 1], d_hh_[hb ^ 1], d_hc_[hb ^ 1], trick ? 1 : 0,           \
                      accumulate ? 1 : 0, wide_ ? 1 : 0,                                                           \
                      indexed_ && rec_one_launch_ ? HistBlocks(Q_) : HistBlocks(quads_per_group_),                \
-                     indexed_ && rec_one_launch_ ? rec_slots_ : kSlots)
+                     lds_slots)
     if (pair_) {
       if (wide_blocks) ARB_REDUCE(true, 4);
       else ARB_REDUCE(true, 16);

@@ -657,7 +657,11 @@ k_hist_reduce(const unsigned long long *__restrict__ slab, int slab_entries, int
     if (items == 0xffffffffu) return;  // derived from its sibling
   }
   const int e = threadIdx.x % kEntries, lane = threadIdx.x / kEntries;
-  const int entry = blockIdx.x * kEntries + e;  // slab order
+  // slab order; with fewer than 256 bins per feature in the slabs only the first lds_slots * 16
+  // entries of every 16-feature block hold anything, and the grid covers only those
+  const int per_block = plain ? 1 : (lds_slots * kBlockFeatures + kEntries - 1) / kEntries;
+  const int entry = plain ? (int)blockIdx.x * kEntries + e
+                          : ((int)blockIdx.x / per_block) * kBlockEntries + ((int)blockIdx.x % per_block) * kEntries + e;
   // plain: the slabs are feature-major already (16-bit bins)
   const int f = (entry / kBlockEntries) * kBlockFeatures + (entry & (kBlockFeatures - 1));
   const int bin = (entry / kBlockFeatures) & (kSlots - 1);
