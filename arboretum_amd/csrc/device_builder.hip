@@ -80,6 +80,9 @@ struct DeviceMatrix {
   // wide resident matrices, built on first use: the same bins row-major, RS words per row
   uint32_t *rec = nullptr;
   int RS = 0;
+  // and column-major with one byte per bin id: [4 Q][stride8]
+  uint8_t *bytes = nullptr;
+  size_t stride8 = 0;
   // streamed: pinned host blocks [Q][block_rows], block b = rows [b*block_rows, ...)
   bool streamed = false;
   size_t block_rows = 0;
@@ -117,6 +120,7 @@ void FreeDeviceMatrix(DeviceMatrix *m) {
   if (!m) return;
   if (m->bins) (void)hipFree(m->bins);
   if (m->rec) (void)hipFree(m->rec);
+  if (m->bytes) (void)hipFree(m->bytes);
   if (m->owns_blocks)
     for (uint32_t *b : m->host_blocks)
       if (b) (void)hipHostFree(b);
@@ -615,6 +619,13 @@ class HipTreeBuilder : public TreeBuilder {
                            dm_->RS, n_);
         HIP_OK(hipGetLastError());
       }
+      if (!dm_->bytes) {
+        dm_->stride8 = (n_ + 255) / 256 * 256;
+        dm_->bytes = DevAlloc<uint8_t>((size_t)Q_ * 4 * dm_->stride8);
+        hipLaunchKernelGGL(k_to_byte_columns, dim3((unsigned)((n_ + 255) / 256)), dim3(256), 0, stream_, dm_->bins,
+                           stride_, Q_, dm_->bytes, dm_->stride8, n_);
+        HIP_OK(hipGetLastError());
+      }
     }
     // level state
     const int max_nodes = 1 << (D_ - 1);
@@ -1104,7 +1115,7 @@ class HipTreeBuilder : public TreeBuilder {
           Plan(ps, PL, 0, kPartRows, d_pwork_, d_nwork_ + 1, -1, nullptr, grid);
           Mark(kPartition);
           if (indexed_) {
-            hipLaunchKernelGGL(k_ix_decide, dim3(grid), dim3(kHistThreads), 0, stream_, dm_->bins, stride_, src.ids,
+            hipLaunchKernelGGL(k_ix_decide, dim3(grid), dim3(kHistThreads), 0, stream_, dm_->bytes, dm_->stride8, src.ids,
                                d_split_, d_pwork_, d_nwork_ + 1, d_dec_, d_wave_left_, d_item_left_);
             if (pair_)
               hipLaunchKernelGGL(k_ix_part<true>, dim3(grid), dim3(kHistThreads), 0, stream_, src.ids, dst.ids, src.g,

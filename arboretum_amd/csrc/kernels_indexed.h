@@ -40,15 +40,30 @@ k_to_records(const uint32_t *__restrict__ bins, size_t stride, int Q, uint32_t *
   }
 }
 
+// Quad columns [Q][stride] -> byte columns [4 Q][stride8]: one byte per row and feature, so that
+// a 64-byte fetch of a feature's column holds 64 rows instead of 16.
+__global__ void __launch_bounds__(256)
+k_to_byte_columns(const uint32_t *__restrict__ bins, size_t stride, int Q, uint8_t *__restrict__ bytes,
+                  size_t stride8, size_t n) {
+  const size_t r = (size_t)blockIdx.x * 256 + threadIdx.x;
+  if (r >= n) return;
+  for (int q = 0; q < Q; ++q) {
+    const uint32_t v = bins[(size_t)q * stride + r];
+#pragma unroll
+    for (int b = 0; b < 4; ++b) bytes[(size_t)(4 * q + b) * stride8 + r] = (uint8_t)(v >> (8 * b));
+  }
+}
+
 // Split decision of every row of the parents of a level, in node order:
 // dec[p] = 1 when the row at position p goes right (builder.h:107-123), and the
 // rows going left per (work item, wave) as k_part_count gives them.  ids: the
 // row at each position (null: position = row, the first level).  The split
-// feature's word is read from the quad columns, not from the records: the ids of
-// a node ascend, so the reads of a node walk one column forwards, and a column
-// is small enough for the caches to help.
+// feature's bin is read from the byte columns, not from the records: the ids of
+// a node ascend, so the reads of a node walk one column forwards, and the deeper
+// the level, the fewer rows of a node share a 64-byte fetch: with a byte per
+// row that happens two levels later than with a word per row.
 __global__ void __launch_bounds__(kHistThreads)
-k_ix_decide(const uint32_t *__restrict__ bins, size_t stride, const unsigned *__restrict__ ids,
+k_ix_decide(const uint8_t *__restrict__ bytes, size_t stride8, const unsigned *__restrict__ ids,
             const SplitRec *__restrict__ split, const WorkItem *__restrict__ work,
             const unsigned *__restrict__ n_work, uint8_t *__restrict__ dec, unsigned *__restrict__ wave_left,
             unsigned *__restrict__ item_left) {
@@ -57,13 +72,13 @@ k_ix_decide(const uint32_t *__restrict__ bins, size_t stride, const unsigned *__
   const WorkItem it = work[w];
   const SplitRec s = split[it.node];
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-  const int fq = s.fid < 0 ? 0 : s.fid >> 2, fs = 8 * (s.fid & 3);
+  const uint8_t *col = bytes + (size_t)(s.fid < 0 ? 0 : s.fid) * stride8;
   unsigned cnt = 0;
   const unsigned cb = ChunkOrigin(it);
   constexpr int kBatch = 4;  // 8 ids, then 8 gathers in flight per lane
   for (unsigned base = cb + wave * kChunkRows; base < it.end; base += kBatch * kChunkStep) {
     unsigned id[2 * kBatch];
-    uint32_t word[2 * kBatch];
+    unsigned bin[2 * kBatch];
 #pragma unroll
     for (int k = 0; k < 2 * kBatch; ++k) {
       const unsigned r = base + (k >> 1) * kChunkStep + (k & 1) * 64 + lane;
@@ -71,12 +86,12 @@ k_ix_decide(const uint32_t *__restrict__ bins, size_t stride, const unsigned *__
       id[k] = ids ? ids[a] : a;
     }
 #pragma unroll
-    for (int k = 0; k < 2 * kBatch; ++k) word[k] = s.fid < 0 ? 0u : bins[(size_t)fq * stride + id[k]];
+    for (int k = 0; k < 2 * kBatch; ++k) bin[k] = col[id[k]];
 #pragma unroll
     for (int k = 0; k < 2 * kBatch; ++k) {
       const unsigned r = base + (k >> 1) * kChunkStep + (k & 1) * 64 + lane;
       if (r >= it.begin && r < it.end) {
-        const bool right = s.fid >= 0 && (int)((word[k] >> fs) & 255u) > s.bin;
+        const bool right = s.fid >= 0 && (int)bin[k] > s.bin;
         dec[r] = right ? 1 : 0;
         cnt += right ? 0u : 1u;
       }
