@@ -1306,12 +1306,15 @@ class HipTreeBuilder : public TreeBuilder {
     const size_t lds = (size_t)internal * 2 * sizeof(int);
     float *yh = d_yhat_ + (size_t)label * n_ + row0;
     const int grid = GridFor(rows, 256, 8192);
+    // the byte columns of a matrix whose rows stay in place (whole matrix only)
+    const uint8_t *walk_bytes = indexed_ && bins == dm_->bins && row0 == 0 ? dm_->bytes : nullptr;
     int mode = 0;
     if (next_grad && cfg_.objective == kLinearRegression) mode = 1;
     if (next_grad && cfg_.objective == kLogisticRegression) mode = 2;
 #define ARB_FINAL(M, N) \
   hipLaunchKernelGGL((k_final<M, N>), dim3(grid), dim3(256), lds, stream_, bins, stride, d_tfid_, d_tbin_, D_, \
-                     d_weights_, yh, d_y_ + row0, d_leaf_ + row0, d_g_ + row0, d_h_ ? d_h_ + row0 : nullptr, d_gmax_, rows, code_)
+                     d_weights_, yh, d_y_ + row0, d_leaf_ + row0, d_g_ + row0, d_h_ ? d_h_ + row0 : nullptr, d_gmax_, rows, code_, \
+                     walk_bytes, dm_->stride8)
 #define ARB_FINAL_Q(N) \
   do { if (mode == 1) ARB_FINAL(1, N); else if (mode == 2) ARB_FINAL(2, N); else ARB_FINAL(0, N); } while (0)
     switch (Q_ <= 8 && !wide_ ? Q_ : 0) {

@@ -110,15 +110,15 @@ k_tree_end(const SplitRec *__restrict__ split, const NodeSum *__restrict__ tot, 
 // 0, write the gradients of the next round (objective.cu:28-56):
 // 1 = squared (also max |g|), 2 = logistic (h == nullptr: packed into g, PackGrad).
 // NQ > 0: the matrix has NQ quads, all loaded up front (coalesced, independent
-// loads) and selected in registers; NQ == 0: any width, one dependent 4-byte
-// load per level.
+// loads) and selected in registers; NQ == 0: any width, one dependent load per
+// level, from the byte columns when the matrix has them (bytes != null).
 template <int NEXT_GRAD, int NQ>
 __global__ void __launch_bounds__(256)
 k_final(const uint32_t *__restrict__ bins, size_t stride, const int *__restrict__ t_fid,
         const int *__restrict__ t_bin, int depth, const float *__restrict__ weights,
         float *__restrict__ yhat, const float *__restrict__ y, unsigned *__restrict__ leaf_of,
         float *__restrict__ g, float *__restrict__ h, unsigned *__restrict__ gmax_bits, size_t n,
-        BinCode code) {
+        BinCode code, const uint8_t *__restrict__ bytes, size_t stride8) {
   extern __shared__ int s_nodes[];  // fid[internal], bin[internal]
   const int internal = (1 << (depth - 1)) - 1;
   for (int i = threadIdx.x; i < internal; i += blockDim.x) {
@@ -146,6 +146,8 @@ k_final(const uint32_t *__restrict__ bins, size_t stride, const int *__restrict_
 #pragma unroll
           for (int q = 0; q < NQ; ++q) b4 = q == fq ? b[q] : b4;
           right = (int)((b4 >> (8 * (fid & 3))) & 255u) > bin ? 1u : 0u;
+        } else if (bytes != nullptr) {  // byte columns [F][stride8] of a wide matrix: a quarter of the bytes fetched
+          right = (int)bytes[(size_t)fid * stride8 + i] > bin ? 1u : 0u;
         } else {
           right = (int)code.Bin(bins[(size_t)code.Word(fid) * stride + i], fid) > bin ? 1u : 0u;
         }
