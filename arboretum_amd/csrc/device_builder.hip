@@ -553,6 +553,16 @@ class HipTreeBuilder : public TreeBuilder {
     indexed_ = !wide_ && !dm_->streamed && !single_group_ && D_ > 2 && cfg.internal.wide_rows_in_place &&
                Q_ <= 256;  // at most 64 pieces of 16 bytes per record
     rec_one_launch_ = rec_lds <= kLdsBudget - 1024;  // else groups of quads_per_group_ quads at 256 bins
+    // one launch: a power of two of blocks between the bins of the LDS image when that still fits
+    rec_lay_blocks_ = 0;
+    if (rec_one_launch_) {
+      int p2 = 1;
+      while (p2 < HistBlocks(Q_)) p2 *= 2;
+      // ... in the LDS and in the slab of a work item, which holds 256 bins of the blocks the matrix has
+      if ((size_t)p2 * kBlockFeatures * rec_slots_ * 8 * (pair_ ? 2 : 1) <= kLdsBudget - 1024 &&
+          (size_t)p2 * rec_slots_ <= (size_t)HistBlocks(Q_) * kSlots)
+        rec_lay_blocks_ = p2;
+    }
     fused_ = trick_ && !wide_ && !indexed_;
     if (wide_) {
       // features per histogram launch (an even number, two per word)
@@ -610,8 +620,8 @@ class HipTreeBuilder : public TreeBuilder {
     }
     if (indexed_) {
       d_dec_ = DevAlloc<uint8_t>(n_);
-      if (!dm_->rec) {  // records: 32-byte aligned, built once per matrix
-        dm_->RS = (Q_ + 7) / 8 * 8;
+      if (!dm_->rec) {  // records: whole 64-byte units (what memory answers a gather with), built once per matrix
+        dm_->RS = (Q_ + 15) / 16 * 16;
         dm_->rec = DevAlloc<uint32_t>(n_ * (size_t)dm_->RS);
         AllowLds(k_to_records, (size_t)64 * (dm_->RS + 1) * sizeof(uint32_t));
         hipLaunchKernelGGL(k_to_records, dim3((unsigned)((n_ + 63) / 64)), dim3(256),
@@ -976,25 +986,34 @@ class HipTreeBuilder : public TreeBuilder {
         const int pieces = rec_one_launch_ ? total : HistBlocks(quads_per_group_);
         const int ngroups = (total + pieces - 1) / pieces;
         const int slots = rec_one_launch_ ? rec_slots_ : kSlots;
-        const size_t lds = (size_t)pieces * kBlockFeatures * slots * 8 * (pair_ ? 2 : 1);
+        const int lay = rec_one_launch_ ? rec_lay_blocks_ : 0;   // blocks the LDS image is laid out for
+        const size_t lds = (size_t)(lay > 0 ? lay : pieces) * kBlockFeatures * slots * 8 * (pair_ ? 2 : 1);
         const size_t item_words = rec_one_launch_ ? lds / 8 : (size_t)slab_entries_ * (pair_ ? 2 : 1);
-        if (lds > kLdsBudget || (size_t)total * 4 > (size_t)dm_->RS || ngroups != rec_groups_)
+        if (lds > kLdsBudget || (size_t)total * 4 > (size_t)dm_->RS || ngroups != rec_groups_ ||
+            item_words > (size_t)slab_entries_ * (pair_ ? 2 : 1))
           throw std::runtime_error("internal: record histogram launch does not fit");
         const unsigned blocks = (grid + 7u) / 8u * 8u * (unsigned)ngroups;
-        // 256 bins and every group (the last may hold fewer blocks) a power of two of blocks
+        // a power of two of blocks in every group (the last may hold fewer), or in the padded layout
         const int last_pieces = total - (ngroups - 1) * pieces;
-        const bool full = slots == kSlots && (pieces & (pieces - 1)) == 0 && (last_pieces & (last_pieces - 1)) == 0;
-#define ARB_REC(P, FULL)                                                                                          \
+        const bool pow2 = lay > 0 ? (lay & (lay - 1)) == 0
+                                  : (pieces & (pieces - 1)) == 0 && (last_pieces & (last_pieces - 1)) == 0;
+        const bool clamp = slots < kSlots;
+#define ARB_REC(P, POW2, CLAMP)                                                                                   \
   do {                                                                                                            \
-    AllowLds((k_hist_rec<P, FULL>), kLdsBudget);                                                                  \
-    hipLaunchKernelGGL((k_hist_rec<P, FULL>), dim3(blocks), dim3(kHistThreads), lds, stream_, dm_->rec, dm_->RS,  \
-                       cur.ids, Q_, slots, cur.g, cur.h, d_shifts_, d_hwork_, d_nwork_, d_slab_, pieces, total,   \
-                       ngroups, item_words);                                                                      \
+    AllowLds((k_hist_rec<P, POW2, CLAMP>), kLdsBudget);                                                           \
+    hipLaunchKernelGGL((k_hist_rec<P, POW2, CLAMP>), dim3(blocks), dim3(kHistThreads), lds, stream_, dm_->rec,    \
+                       dm_->RS, cur.ids, Q_, slots, cur.g, cur.h, d_shifts_, d_hwork_, d_nwork_, d_slab_, pieces, \
+                       total, ngroups, item_words, lay);                                                          \
   } while (0)
-        if (pair_ && full) ARB_REC(true, true);
-        else if (pair_) ARB_REC(true, false);
-        else if (full) ARB_REC(false, true);
-        else ARB_REC(false, false);
+#define ARB_REC_P(P)                                      \
+  do {                                                    \
+    if (pow2 && clamp) ARB_REC(P, true, true);            \
+    else if (pow2) ARB_REC(P, true, false);               \
+    else ARB_REC(P, false, true);                         \
+  } while (0)
+        if (pair_) ARB_REC_P(true);
+        else ARB_REC_P(false);
+#undef ARB_REC_P
 #undef ARB_REC
         if (timing_) ++(root ? timings_.hist_root_launches : timings_.hist_deep_launches);
         break;
@@ -1014,6 +1033,7 @@ class HipTreeBuilder : public TreeBuilder {
     const bool wide_blocks = L >= 32;
     const int entries = wide_blocks ? 256 : 64;
     const int lds_slots = indexed_ && rec_one_launch_ ? rec_slots_ : kSlots;
+    const int lay_blocks = indexed_ && rec_one_launch_ ? rec_lay_blocks_ : 0;
     // 16-bit bins: feature-major slabs; else the entries of the bins in use of every 16-feature block
     dim3 grid(wide_ ? (slab_entries_ + entries - 1) / entries
                     : slab_entries_ / kBlockEntries * ((lds_slots * kBlockFeatures + entries - 1) / entries),
@@ -1024,7 +1044,7 @@ class HipTreeBuilder : public TreeBuilder {
                      d_hh_[hb], d_hc_[hb], d_hg_[hb ^ 1], d_hh_[hb ^ 1], d_hc_[hb ^ 1], trick ? 1 : 0,           \
                      accumulate ? 1 : 0, wide_ ? 1 : 0,                                                           \
                      indexed_ && rec_one_launch_ ? HistBlocks(Q_) : HistBlocks(quads_per_group_),                \
-                     lds_slots)
+                     lds_slots, lay_blocks)
     if (pair_) {
       if (wide_blocks) ARB_REDUCE(true, 4);
       else ARB_REDUCE(true, 16);
@@ -1486,6 +1506,7 @@ class HipTreeBuilder : public TreeBuilder {
   bool indexed_ = false;      // wide matrix: rows stay in place, (row id, gradients) are re-ordered
   int rec_slots_ = kSlots;    // bins per feature of the one LDS histogram of that mode
   bool rec_one_launch_ = true;  // every feature fits one LDS histogram at rec_slots_ bins
+  int rec_lay_blocks_ = 0;      // blocks that histogram is laid out for (a power of two), 0: as many as the matrix has
   uint8_t *d_dec_ = nullptr;  // indexed mode: split decision of the row at each position
   bool wide_ = false;     // 16-bit bins: two features per word, slots_ histogram slots per feature
   int slots_ = kSlots;

@@ -204,15 +204,18 @@ k_ix_part(const unsigned *__restrict__ ids, unsigned *__restrict__ ids_out, cons
 // (PAIR ? 32 : 16), word1 16 words further.  A bin id is clamped to the
 // histogram, so that no input can write outside it.  The slab of a work item is
 // the LDS image: blocks * 16 * slots entries of one or two words.
-// FULL: 256 bins per feature and a power of two of bytes between bins (stride_shift): the
-// offset of a cell is a shift and an add, and no bin id can leave the histogram.
-template <bool PAIR, bool FULL = false>
+// POW2: a power of two of bytes between the bins of the LDS image (stride_shift): the offset of
+// a cell is a shift and an add instead of a multiply and an add.  CLAMP: fewer than 256 bins per
+// feature, bin ids are clamped to the histogram (with 256 no bin id can leave it).
+// lay_blocks: 16-feature blocks the image is laid out for (0: the pieces of the workgroup's
+// group); more than the matrix has makes the stride a power of two.
+template <bool PAIR, bool POW2 = false, bool CLAMP = true>
 __global__ void __launch_bounds__(kHistThreads)
 k_hist_rec(const uint32_t *__restrict__ rec, int RS, const unsigned *__restrict__ ids, int Q, int slots,
            const float *__restrict__ g, const float *__restrict__ h, const int *__restrict__ shifts,
            const WorkItem *__restrict__ work, const unsigned *__restrict__ n_work,
            unsigned long long *__restrict__ slab, int group_pieces, int total_pieces, int ngroups,
-           size_t item_words) {
+           size_t item_words, int lay_blocks) {
   extern __shared__ unsigned long long lds[];
   // Workgroup -> (work item, group of pieces): workgroups are dealt to the eight XCDs in turn
   // (workgroup b runs on XCD b % 8), and the groups of one work item read the same records, so
@@ -225,7 +228,8 @@ k_hist_rec(const uint32_t *__restrict__ rec, int RS, const unsigned *__restrict_
   const int npieces = min(group_pieces, total_pieces - piece0);
   const WorkItem it = work[w];
   constexpr unsigned per = PAIR ? 2 : 1;
-  const unsigned blocks = (unsigned)npieces, bin_stride = blocks * per * kBlockFeatures;
+  const unsigned blocks = (unsigned)npieces;
+  const unsigned bin_stride = (lay_blocks > 0 ? (unsigned)lay_blocks : blocks) * per * kBlockFeatures;
   const unsigned words = (unsigned)slots * bin_stride;
   for (unsigned i = threadIdx.x; i < words; i += kHistThreads) lds[i] = 0ull;
   __syncthreads();
@@ -283,7 +287,7 @@ k_hist_rec(const uint32_t *__restrict__ rec, int RS, const unsigned *__restrict_
   };
   unsigned char *lds_b = reinterpret_cast<unsigned char *>(lds);
   const unsigned bin_stride_b = bin_stride * 8u;    // at most 64 x 2 x 16 x 8 = 16 KB
-  const unsigned stride_shift = 31u - (unsigned)__clz((int)bin_stride_b);   // FULL: bin_stride_b = 1 << stride_shift
+  const unsigned stride_shift = 31u - (unsigned)__clz((int)bin_stride_b);   // POW2: bin_stride_b = 1 << stride_shift
   auto accumulate = [&](const Pieces &R) {
 #pragma unroll
     for (int k = 0; k < kSteps; ++k) {
@@ -308,12 +312,10 @@ k_hist_rec(const uint32_t *__restrict__ rec, int RS, const unsigned *__restrict_
           for (int t = 0; t < 4; ++t) {
             const unsigned bi = ((unsigned)t + i4) & 3u;
             unsigned off;
-            if (FULL) {
-              off = (__builtin_amdgcn_ubfe(sel, 8u * bi, 8u) << stride_shift) + (piece_b + (4u * qi + bi) * 8u);
-            } else {
-              const unsigned bin = min(__builtin_amdgcn_ubfe(sel, 8u * bi, 8u), last_bin);
-              off = __umul24(bin, bin_stride_b) + (piece_b + (4u * qi + bi) * 8u);
-            }
+            unsigned bin = __builtin_amdgcn_ubfe(sel, 8u * bi, 8u);
+            if (CLAMP) bin = min(bin, last_bin);
+            if (POW2) off = (bin << stride_shift) + (piece_b + (4u * qi + bi) * 8u);
+            else off = __umul24(bin, bin_stride_b) + (piece_b + (4u * qi + bi) * 8u);
             unsigned long long *cell = reinterpret_cast<unsigned long long *>(lds_b + off);
             atomicAdd(cell, w0);
             if (PAIR) atomicAdd(cell + kWord1, w1);

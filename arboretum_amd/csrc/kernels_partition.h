@@ -634,7 +634,7 @@ k_hist_reduce(const unsigned long long *__restrict__ slab, int slab_entries, int
               long long *__restrict__ hh, unsigned *__restrict__ hc,
               const long long *__restrict__ pg, const long long *__restrict__ ph,
               const unsigned *__restrict__ pc, int trick, int accumulate, int plain, int group_blocks,
-              int lds_slots = kSlots) {
+              int lds_slots = kSlots, int lay_blocks = 0) {
   // LANES threads share the slabs of one entry; a block covers 1024 / LANES
   // consecutive entries (with 4 lanes: 16 bins x 16 features, so the
   // feature-major output is written in runs of 16 bins)
@@ -669,8 +669,11 @@ k_hist_reduce(const unsigned long long *__restrict__ slab, int slab_entries, int
   // lds_slots < 256: the slabs hold that many bins per feature only (the rest are empty)
   const bool live = (plain ? entry < nbin_total : f * kSlots < nbin_total);
   const bool stored = plain || bin < lds_slots;
+  // lay_blocks > 0: the slabs are laid out for that many 16-feature blocks (a power of two of
+  // bytes between bins), of which the matrix has slab_entries / 4096
   const size_t slab_words = plain ? (size_t)slab_entries * (PAIR ? 2 : 1)
-                                  : (size_t)slab_entries / kSlots * (size_t)lds_slots * (PAIR ? 2 : 1);
+                            : lay_blocks > 0 ? (size_t)lay_blocks * kBlockFeatures * (size_t)lds_slots * (PAIR ? 2 : 1)
+                                             : (size_t)slab_entries / kSlots * (size_t)lds_slots * (PAIR ? 2 : 1);
   long long ag = 0, ah = 0;
   unsigned ac = 0;
   if (live) {
@@ -682,7 +685,8 @@ k_hist_reduce(const unsigned long long *__restrict__ slab, int slab_entries, int
       const int block = entry / kBlockEntries, group = block / group_blocks;
       const int blocks_here = min(group_blocks, slab_entries / kBlockEntries - group * group_blocks);
       const unsigned in_group = (unsigned)(entry - group * group_blocks * kBlockEntries);
-      i0 = (unsigned)(group * group_blocks * kBlockEntries) * (PAIR ? 2u : 1u) + HistWord<PAIR>(in_group, blocks_here);
+      i0 = (unsigned)(group * group_blocks * kBlockEntries) * (PAIR ? 2u : 1u) +
+           HistWord<PAIR>(in_group, lay_blocks > 0 ? lay_blocks : blocks_here);
       i1 = i0 + kWord1;
     }
     for (unsigned s = lane; s < items && stored; s += LANES) {
