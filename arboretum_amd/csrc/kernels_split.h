@@ -40,13 +40,16 @@ __device__ __forceinline__ Cand ScanFeature(const long long *__restrict__ hg, co
       long long g4[4], h4[4];
       unsigned long long c4[4];
 #pragma unroll
-      for (int j = 0; j < 4; ++j) {
-        // the slots from hist_size on (missing values, unused slots) are no candidates and in no
-        // candidate's prefix
-        const bool read = chunk + lane * 4 + j < hist_size;
-        g4[j] = read ? hg[base + j] : 0;
-        h4[j] = PAIR && read ? hh[base + j] : 0;
-        c4[j] = read ? hc[base + j] : 0;
+      for (int j = 0; j < 4; ++j) g4[j] = h4[j] = 0, c4[j] = 0;
+      // lanes whose four slots all lie at or past hist_size (missing values, unused slots) hold no
+      // candidate and are in no candidate's prefix: they read nothing
+      if (chunk + lane * 4 < hist_size) {
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+          g4[j] = hg[base + j];
+          h4[j] = PAIR ? hh[base + j] : 0;
+          c4[j] = hc[base + j];
+        }
       }
 #pragma unroll
       for (int j = 1; j < 4; ++j) {
