@@ -39,9 +39,13 @@
 //                       scipy soft-max, the K = 2 reduction to the logistic
 //                       sigmoid, sum-to-zero / range invariants and the central
 //                       difference of the log-likelihood.
-//   column sampling     PARITY UNPINNED against the reference's std::shuffle
-//                       stream (garden.cu:126-165): no reference test holds a
-//                       sampled model; only the error strings are pinned.
+//   column sampling     pinned (garden.cu:126-165, 249-253): the active ids of
+//                       every (tree, level) against literal vectors written by
+//                       tests/golden/make_shuffle_vectors.cpp, a program that
+//                       holds nothing but the reference's calls on the random
+//                       engine; set sizes and split-feature membership; the
+//                       two error strings.  (The draw itself is the standard
+//                       library's std::shuffle on std::default_random_engine.)
 //   orc_expf            defined here (double polynomial, correctly rounded in
 //                       all but rare cases); checked against libm within 1 ulp.
 // ---------------------------------------------------------------------------
@@ -373,6 +377,9 @@ struct Booster {
   std::vector<std::vector<Acc>> lvl_tot;   // [level][node]
   int shift_g = 30, shift_h = 32;
   std::default_random_engine rnd;  // garden.cu:87, seeded with internals.seed
+  // inspection: the features a split may use, per grown tree and level, in the
+  // order they stand at the front of the shuffled id list
+  std::vector<std::vector<std::vector<unsigned>>> active_log;
   uint64_t updates = 0;  // rows*features actually accumulated (work counter)
   int kind() const { return (p.objective == 0 ? 0 : 2) + (p.double_precision ? 1 : 0); }
 };
@@ -531,8 +538,8 @@ static void grow_tree(Booster &b, int label) {
   // per tree, InitTreeLevel (:162-165) reshuffles the first
   // int(colsample_bytree * columns) per level, and FindBestSplits (:252-253,
   // 309-310) takes the first unsigned(bylevel * bytree * columns) as active.
-  // Parity with the reference's random stream is unpinned (it depends on the
-  // standard library's shuffle); with both ratios 1.0 every feature is active.
+  // With both ratios 1.0 every feature is active.
+  b.active_log.emplace_back();
   std::vector<unsigned> active_fids(F);
   for (int f = 0; f < F; ++f) active_fids[f] = f;
   std::shuffle(active_fids.begin(), active_fids.end(), b.rnd);
@@ -560,6 +567,8 @@ static void grow_tree(Booster &b, int label) {
     std::shuffle(active_fids.begin(), active_fids.begin() + take_tree, b.rnd);
     std::vector<uint8_t> is_active(F, 0);
     for (unsigned j = 0; j < take_level && j < (unsigned)F; ++j) is_active[active_fids[j]] = 1;
+    b.active_log.back().emplace_back(active_fids.begin(),
+                                     active_fids.begin() + std::min<unsigned>(take_level, (unsigned)F));
     std::vector<Acc> &hist = b.lvl_hist[level];
     hist.assign((size_t)L * F * SL, Acc());
     b.lvl_tot[level] = tot;
@@ -900,11 +909,28 @@ void *orc_create_binned(const uint8_t *bins, int64_t n, int F, const float *y,
 
 void orc_free(void *h) { delete static_cast<Booster *>(h); }
 
-// One boosting round = labels_count trees (garden.cu:585-625)
-void orc_grow_round(void *hd) {
+// One boosting round = labels_count trees (garden.cu:585-625).  Returns NULL,
+// or the message InitGrowingTree throws before anything is drawn
+// (garden.cu:127-140): the round then grows nothing.
+const char *orc_grow_round(void *hd) {
   Booster &b = *static_cast<Booster *>(hd);
+  if ((int)(b.p.colsample_bytree * (size_t)b.F) == 0) return "colsample_bytree is too small";
+  if ((int)(b.p.colsample_bytree * b.p.colsample_bylevel * (size_t)b.F) == 0)
+    return "colsample_bytree and colsample_bylevel are too small";
   update_grad(b);
   for (int k = 0; k < b.p.labels_count; ++k) grow_tree(b, k);
+  return nullptr;
+}
+
+// Ids of the features that tree `t` may split on at `level`, in the order they
+// stand in the shuffled list.  Returns their number, -1 for a bad index.
+int orc_get_active(void *hd, int t, int level, unsigned *out) {
+  Booster &b = *static_cast<Booster *>(hd);
+  if (t < 0 || t >= (int)b.active_log.size() || level < 0 || level >= (int)b.active_log[t].size())
+    return -1;
+  const std::vector<unsigned> &a = b.active_log[t][level];
+  if (out) std::memcpy(out, a.data(), a.size() * sizeof(unsigned));
+  return (int)a.size();
 }
 
 int orc_hist_size(void *hd) { return static_cast<Booster *>(hd)->p.hist_size; }  // exact: distinct values

@@ -82,7 +82,9 @@ def lib():
         L.orc_create_binned.restype = ctypes.c_void_p
         L.orc_create_binned.argtypes = L.orc_create.argtypes
         L.orc_free.argtypes = [ctypes.c_void_p]
+        L.orc_grow_round.restype = ctypes.c_char_p
         L.orc_grow_round.argtypes = [ctypes.c_void_p]
+        L.orc_get_active.argtypes = [ctypes.c_void_p, ctypes.c_int, ctypes.c_int, ctypes.c_void_p]
         L.orc_hist_size.argtypes = [ctypes.c_void_p]
         L.orc_num_trees.argtypes = [ctypes.c_void_p]
         L.orc_updates.restype = ctypes.c_uint64
@@ -183,7 +185,18 @@ class Booster:
 
     def grow(self, rounds=1):
         for _ in range(rounds):
-            lib().orc_grow_round(self.h)
+            err = lib().orc_grow_round(self.h)
+            if err is not None:      # the literal the reference throws (garden.cu:127-140)
+                raise ValueError(err.decode())
+
+    def active_features(self, t, level):
+        """Feature ids tree `t` may split on at `level` (garden.cu:162-165, 252-253)."""
+        n = lib().orc_get_active(self.h, t, level, None)
+        if n < 0:
+            raise IndexError((t, level))
+        out = np.empty(n, np.uint32)
+        lib().orc_get_active(self.h, t, level, _p(out))
+        return out
 
     @property
     def num_trees(self):

@@ -570,3 +570,128 @@ def test_logistic_labels_outside_0_1_keep_their_gradients(oracle):
     native.grow(1)
     assert np.array_equal(b.tree(0)["fid"], native.tree(0)["fid"])
     assert np.array_equal(b.tree(0)["quantized"], native.tree(0)["quantized"])
+
+
+# ------------------------------------------------------- column sampling
+# Reference: InitGrowingTree / InitTreeLevel / FindBestSplits, src/core/garden.cu:126-165, 249-253.
+# The literal id vectors of column_sampling.json come from tests/golden/make_shuffle_vectors.cpp,
+# which holds the reference's calls on its random engine and nothing else.
+def _sampling_booster(oracle, case, trees, max_depth, objective=1, rows=600):
+    rng = np.random.default_rng(17)
+    F = case["columns"]
+    X = rng.normal(size=(rows, F)).astype(np.float32)
+    s = X @ rng.normal(size=F)
+    y = (s > 0).astype(np.float32) if objective else (s + 0.1 * rng.normal(size=rows)).astype(np.float32)
+    cfg = {"objective": objective, "method": 1,
+           "internals": {"hist_size": 16, "double_precision": True, "seed": case["seed"]},
+           "tree": {"max_depth": max_depth, "eta": 0.3, "lambda": 1.0, "min_child_weight": 0.0,
+                    "colsample_bytree": case["colsample_bytree"], "colsample_bylevel": case["colsample_bylevel"]}}
+    b = oracle.Booster(X, y=y, config=cfg, accum=1)
+    b.grow(trees)
+    return b, X, y, cfg
+
+
+@pytest.mark.parametrize("case", load_golden("column_sampling.json"),
+                         ids=lambda c: "seed%d-F%d-%g-%g" % (c["seed"], c["columns"], c["colsample_bytree"],
+                                                             c["colsample_bylevel"]))
+def test_column_sampling_active_ids_equal_the_reference_call_sequence(oracle, case):
+    # A re-shuffle of the wrong range (all ids instead of the first int(bytree*F)), a wrong prefix
+    # (bytree*F instead of bylevel*bytree*F ids), ids not reset per tree, or one engine per tree
+    # instead of one per booster all change these vectors.
+    trees, levels = len(case["active"]), len(case["active"][0])
+    b, _, _, _ = _sampling_booster(oracle, case, trees, levels)
+    F, bt, bl = case["columns"], np.float32(case["colsample_bytree"]), np.float32(case["colsample_bylevel"])
+    per_tree, per_level = int(bt * np.float32(F)), int(np.float32(bl * bt) * np.float32(F))
+    for t in range(trees):
+        seen = set()
+        for level in range(levels):
+            ids = b.active_features(t, level).tolist()
+            assert ids == case["active"][t][level], (t, level)
+            assert len(ids) == per_level and len(set(ids)) == per_level
+            seen |= set(ids)
+            # every split of the level uses one of its active features
+            tr = b.tree(t)
+            for nd in range((1 << level) - 1, (2 << level) - 1):
+                if tr["quantized"][nd] >= 0:
+                    assert tr["fid"][nd] in ids, (t, level, nd)
+        assert len(seen) <= per_tree       # the levels draw from the tree's int(bytree*F) ids only
+    with pytest.raises(IndexError):
+        b.active_features(trees, 0)
+
+
+def test_column_sampling_fixture_tells_the_shuffle_ranges_apart():
+    # the fixture must be able to fail: with bytree < 1 some level of some tree shows an id set
+    # that differs from the previous level's (the per-level re-shuffle is visible), and the
+    # trees differ from each other (one engine per booster, ids reset per tree)
+    for case in load_golden("column_sampling.json"):
+        if case["colsample_bytree"] * case["colsample_bylevel"] == 1.0:
+            assert all(sorted(lv) == list(range(case["columns"])) for tr in case["active"] for lv in tr)
+            continue
+        assert any(tr[i] != tr[i + 1] for tr in case["active"] for i in range(len(tr) - 1))
+        assert case["active"][0] != case["active"][1]
+
+
+@pytest.mark.parametrize("objective", [0, 1])
+def test_column_sampling_searches_exactly_the_active_features(oracle, objective):
+    # node by node: the split of a node is the brute-force best over the ACTIVE features of its
+    # level (lowest feature id on equal gains, whatever the shuffled order), found on its own rows
+    case = {"seed": 9, "columns": 6, "colsample_bytree": 0.7, "colsample_bylevel": 0.8}
+    depth, lam = 3, 1.0
+    b, X, y, cfg = _sampling_booster(oracle, case, 2, depth, objective=objective, rows=150)
+    bins = b.bins().astype(np.float32)
+    g, h = b.grad()                      # gradients of the LAST round = those tree 1 was grown on
+    if objective == 0:
+        h = np.ones_like(g)
+    t = b.tree(1)
+    rows = {0: np.arange(len(y))}
+    some_feature_left_out = False
+    for i in range((1 << depth) - 1):
+        level = int(np.log2(i + 1))
+        act = np.sort(b.active_features(1, level))
+        assert len(act) == int(np.float32(np.float32(0.7) * np.float32(0.8)) * np.float32(6)) == 3
+        r = rows[i]
+        f = -1
+        if len(r) > 1:
+            f, first_right, gain = _brute_force_exact_root(oracle, bins[np.ix_(r, act)], g[r], h[r],
+                                                           1 if objective == 0 else 3, (1, 0.0, 0.0, 0.0, lam, 0.0))
+            all_f, _, all_gain = _brute_force_exact_root(oracle, bins[r], g[r], h[r],
+                                                         1 if objective == 0 else 3, (1, 0.0, 0.0, 0.0, lam, 0.0))
+            some_feature_left_out |= all_f >= 0 and all_f not in act and (f < 0 or all_gain > gain)
+        if f >= 0:
+            assert (t["fid"][i], t["quantized"][i]) == (act[f], int(first_right) - 1), "node %d" % i
+            assert t["gain"][i] == pytest.approx(gain, rel=1e-5)
+            right = bins[r, act[f]] >= first_right
+        else:
+            assert t["quantized"][i] == -1 and t["fid"][i] == 0, "node %d" % i
+            right = np.zeros(len(r), bool)
+        rows[2 * i + 1], rows[2 * i + 2] = r[~right], r[right]
+    assert some_feature_left_out         # sampling changed at least one decision on this input
+
+
+def test_column_sampling_same_seed_same_trees_and_ratio_one_is_no_sampling(oracle):
+    case = {"seed": 4, "columns": 9, "colsample_bytree": 0.6, "colsample_bylevel": 0.9}
+    a, X, y, cfg = _sampling_booster(oracle, case, 3, 3)
+    b, _, _, _ = _sampling_booster(oracle, case, 3, 3)
+    c, _, _, _ = _sampling_booster(oracle, dict(case, seed=5), 3, 3)
+    same = lambda p, q: all(np.array_equal(p.tree(t)[k], q.tree(t)[k]) for t in range(3)
+                            for k in ("fid", "quantized", "weights"))
+    assert same(a, b) and not same(a, c)
+    full = dict(case, colsample_bytree=1.0, colsample_bylevel=1.0)
+    d, _, _, _ = _sampling_booster(oracle, full, 3, 3)
+    e, _, _, _ = _sampling_booster(oracle, dict(full, seed=77), 3, 3)       # the order drawn does not matter
+    assert same(d, e) and not same(a, d)
+    assert sorted(d.active_features(2, 1).tolist()) == list(range(9))
+
+
+def test_column_sampling_too_small_raises_the_reference_messages(oracle):
+    # garden.cu:127-140: the two literals, the first one wins; nothing is grown
+    X = np.random.default_rng(0).normal(size=(50, 3)).astype(np.float32)
+    y = (X[:, 0] > 0).astype(np.float32)
+    for tree, msg in (({"colsample_bytree": 0.1}, "colsample_bytree is too small"),
+                      ({"colsample_bytree": 0.1, "colsample_bylevel": 0.1}, "colsample_bytree is too small"),
+                      ({"colsample_bytree": 0.5, "colsample_bylevel": 0.5},
+                       "colsample_bytree and colsample_bylevel are too small")):
+        b = oracle.Booster(X, y=y, config={"objective": 1, "method": 1, "tree": dict(tree, max_depth=2)})
+        with pytest.raises(ValueError) as e:
+            b.grow(1)
+        assert str(e.value) == msg and b.num_trees == 0
