@@ -207,7 +207,8 @@ class DMatrix(object):
         return bits.value, slots.value
 
     def bins(self):
-        if self.bin_layout()[0] == 16:
+        bits, slots = self.bin_layout()
+        if bits == 16 or slots > 256:      # ids above 255: 16-bit ids, or bytes with a ninth bit
             out = np.empty((self.rows, self.columns), dtype=np.uint16)
             _check(_LIB.AGetBins16(self.handle, out.ctypes.data_as(ctypes.c_void_p)))
             return out

@@ -76,14 +76,19 @@ struct DeviceMatrix {
   int F = 0, Q = 0;          // Q words of 32 bits per row
   int bits = 8;              // bits per bin id: 8 (four features per word) or 16 (two)
   int slots = kSlots;        // histogram slots per feature
-  uint32_t *bins = nullptr;  // resident: [Q][stride] in HBM
+  // 8-bit ids with a ninth-bit word per row in column Q (ids up to 256, at most 32 features):
+  // a feature that fills 256 value bins and has missing values besides (SplitTest)
+  bool hi = false;
+  int W() const { return Q + (hi ? 1 : 0); }  // words of a row that kernels read and move
+  int cols = 0;              // columns allocated per row (Q, or Q + 1 when ninth bits might be needed)
+  uint32_t *bins = nullptr;  // resident: [cols][stride] in HBM
   // wide resident matrices, built on first use: the same bins row-major, RS words per row
   uint32_t *rec = nullptr;
   int RS = 0;
   // and column-major with one byte per bin id: [4 Q][stride8]
   uint8_t *bytes = nullptr;
   size_t stride8 = 0;
-  // streamed: pinned host blocks [Q][block_rows], block b = rows [b*block_rows, ...)
+  // streamed: pinned host blocks [cols][block_rows], block b = rows [b*block_rows, ...)
   bool streamed = false;
   size_t block_rows = 0;
   std::vector<uint32_t *> host_blocks;
@@ -195,6 +200,7 @@ void QuantiseOnDevice(DataMatrix *data, int hist_size, bool verbose, bool stream
     ext->rows = n;
     ext->F = F;
     ext->Q = (F + 3) / 4;
+    ext->cols = ext->Q;
     ext->stride = (n + 63) / 64 * 64;
     ext->streamed = true;
     ext->owns_blocks = false;
@@ -218,7 +224,12 @@ void QuantiseOnDevice(DataMatrix *data, int hist_size, bool verbose, bool stream
   dm->Q = (F + 3) / 4;
   dm->stride = (n + 63) / 64 * 64;
   dm->streamed = streamed;
+  // Only a quantiser run at hist_size 256 and more can hand out the id 256; a matrix of at most 32
+  // features then gets room for a ninth-bit word per row (used if some feature turns out to need it).
+  const bool may_need_hi = !exact && !data->is_prebinned && hist_size >= kSlots && F <= 32;
+  dm->cols = dm->Q + (may_need_hi ? 1 : 0);
   uint32_t *d_col = nullptr;  // streamed: one quad column at a time on the device
+  uint32_t *d_hi = nullptr;   // the column of ninth-bit words while the features are quantised
   size_t nblocks = 0;
   if (streamed) {
     // default: 16M-row blocks (2 GB of bins at 128 features), large enough that
@@ -230,16 +241,19 @@ void QuantiseOnDevice(DataMatrix *data, int hist_size, bool verbose, bool stream
     nblocks = (n + block_rows - 1) / block_rows;
     dm->host_blocks.assign(nblocks, nullptr);
     for (size_t b = 0; b < nblocks; ++b)
-      HIP_OK(hipHostMalloc((void **)&dm->host_blocks[b], (size_t)dm->Q * block_rows * sizeof(uint32_t), hipHostMallocDefault));
+      HIP_OK(hipHostMalloc((void **)&dm->host_blocks[b], (size_t)dm->cols * block_rows * sizeof(uint32_t), hipHostMallocDefault));
     d_col = DevAlloc<uint32_t>(dm->stride);
+    if (may_need_hi) d_hi = DevAlloc<uint32_t>(dm->stride);
   } else {
-    dm->bins = DevAlloc<uint32_t>((size_t)dm->Q * dm->stride);
+    dm->bins = DevAlloc<uint32_t>((size_t)dm->cols * dm->stride);
+    if (may_need_hi) d_hi = dm->bins + (size_t)dm->Q * dm->stride;
   }
+  if (d_hi) HIP_OK(hipMemset(d_hi, 0, dm->stride * sizeof(uint32_t)));
   // streamed: quad q of all rows (in d_col) -> its slice of every host block
-  auto store_quad = [&](int q) {
+  auto store_quad = [&](int q, const uint32_t *col) {
     for (size_t b = 0; b < nblocks; ++b) {
       const size_t r0 = b * block_rows, rows = std::min(block_rows, n - r0);
-      HIP_OK(hipMemcpy(dm->host_blocks[b] + (size_t)q * block_rows, d_col + r0, rows * sizeof(uint32_t),
+      HIP_OK(hipMemcpy(dm->host_blocks[b] + (size_t)q * block_rows, col + r0, rows * sizeof(uint32_t),
                        hipMemcpyDeviceToHost));
     }
   };
@@ -260,7 +274,7 @@ void QuantiseOnDevice(DataMatrix *data, int hist_size, bool verbose, bool stream
       while ((size_t)slots < most) slots *= 2;
       dm->bits = 16;
       dm->slots = slots;
-      dm->Q = (F + 1) / 2;
+      dm->Q = dm->cols = (F + 1) / 2;
       HIP_OK(hipFree(dm->bins));
       dm->bins = DevAlloc<uint32_t>((size_t)dm->Q * dm->stride);
       uint16_t *d_in = DevAlloc<uint16_t>(n * F);
@@ -336,7 +350,11 @@ void QuantiseOnDevice(DataMatrix *data, int hist_size, bool verbose, bool stream
           HIP_OK(hipMemcpy(d_x + (size_t)c * n, stage[f & 1], n * sizeof(float), hipMemcpyHostToDevice));
           bool has_nan = false;
           DeviceThresholds(ws.get(), d_x + (size_t)c * n, &data->thresholds[f], &data->reduced_size[f], &has_nan);
-          if (bits == 8 && data->reduced_size[f] + (has_nan ? 1 : 0) > kSlots) return false;
+          if (bits == 8 && data->reduced_size[f] + (has_nan ? 1 : 0) > kSlots) {
+            // id 256: the ninth-bit word takes it, where the matrix has one
+            if (d_hi == nullptr || data->reduced_size[f] + 1 > kSlots + 1) return false;
+            dm->hi = true;
+          }
           if (verbose)
             printf("feature %d has been reduced to %d bits \n", f,
                    32 - __builtin_clz((unsigned)data->reduced_size[f]));
@@ -348,14 +366,15 @@ void QuantiseOnDevice(DataMatrix *data, int hist_size, bool verbose, bool stream
         uint32_t *out = streamed ? d_col : dm->bins + (size_t)q * dm->stride;
         if (bits == 8)
           hipLaunchKernelGGL(k_bin_assign, dim3(GridFor(n, 256)), dim3(256), 0, 0, d_x, nc, d_thr, hist_size, d_size,
-                             out, n);
+                             out, n, d_hi, q * W);
         else
           hipLaunchKernelGGL(k_bin_assign_wide, dim3(GridFor(n, 256)), dim3(256),
                              2 * (size_t)hist_size * sizeof(float), 0, d_x, nc, d_thr, hist_size, d_size, out, n);
         HIP_OK(hipGetLastError());
         HIP_OK(hipDeviceSynchronize());
-        if (streamed) store_quad(q);
+        if (streamed) store_quad(q, d_col);
       }
+      if (streamed && dm->hi) store_quad(dm->Q, d_hi);
       return true;
     };
     if (!quantise_columns(8)) {
@@ -369,7 +388,9 @@ void QuantiseOnDevice(DataMatrix *data, int hist_size, bool verbose, bool stream
       dm->bins = nullptr;
       dm->bits = 16;
       dm->slots = slots;
-      dm->Q = (F + 1) / 2;
+      dm->hi = false;
+      d_hi = nullptr;  // (was a part of dm->bins: a resident matrix)
+      dm->Q = dm->cols = (F + 1) / 2;
       dm->bins = DevAlloc<uint32_t>((size_t)dm->Q * dm->stride);
       if (!quantise_columns(16)) throw std::runtime_error("internal: 16-bit quantisation failed");
     }
@@ -379,6 +400,8 @@ void QuantiseOnDevice(DataMatrix *data, int hist_size, bool verbose, bool stream
     for (int k = 0; k < 2; ++k) HIP_OK(hipHostFree(stage[k]));
   }
   if (d_col) HIP_OK(hipFree(d_col));
+  if (streamed && d_hi) HIP_OK(hipFree(d_hi));
+  if (dm->hi) dm->slots = kSlots + 1;
   if (streamed) {
     data->stream_blocks = dm->host_blocks;
     data->stream_block_rows = block_rows;
@@ -422,6 +445,22 @@ void GetBinLayout(const DataMatrix &data, int *bits, int *slots) {
 void GetDeviceBins16(const DataMatrix &data, uint16_t *out) {
   const DeviceMatrix *dm = data.device;
   if (!dm) throw std::runtime_error("data matrix is not quantised");
+  if (dm->bits == 8 && dm->hi) {
+    // byte + ninth bit; resident or in pinned blocks
+    std::vector<uint32_t> q;
+    if (!dm->streamed) {
+      q.resize((size_t)dm->W() * dm->stride);
+      HIP_OK(hipMemcpy(q.data(), dm->bins, q.size() * sizeof(uint32_t), hipMemcpyDeviceToHost));
+    }
+    for (size_t r = 0; r < dm->rows; ++r) {
+      const uint32_t *base = dm->streamed ? dm->host_blocks[r / dm->block_rows] : q.data();
+      const size_t st = dm->streamed ? dm->block_rows : dm->stride, at = dm->streamed ? r % dm->block_rows : r;
+      const uint32_t hi = base[(size_t)dm->Q * st + at];
+      for (int f = 0; f < dm->F; ++f)
+        out[r * dm->F + f] = (uint16_t)(((base[(size_t)(f >> 2) * st + at] >> (8 * (f & 3))) & 255u) + ((hi >> f) & 1u));
+    }
+    return;
+  }
   if (dm->bits != 16) throw std::runtime_error("the matrix has 8-bit bins");
   std::vector<uint32_t> q((size_t)dm->Q * dm->stride);
   HIP_OK(hipMemcpy(q.data(), dm->bins, q.size() * sizeof(uint32_t), hipMemcpyDeviceToHost));
@@ -434,6 +473,7 @@ void GetDeviceBins(const DataMatrix &data, uint8_t *out) {
   const DeviceMatrix *dm = data.device;
   if (!dm) throw std::runtime_error("data matrix is not quantised");
   if (dm->bits != 8) throw std::runtime_error("the matrix has 16-bit bins");
+  if (dm->hi) throw std::runtime_error("the matrix has bin ids up to 256: ask for 16-bit ids");
   if (dm->streamed) {
     for (size_t r = 0; r < dm->rows; ++r) {
       const uint32_t *blk = dm->host_blocks[r / dm->block_rows];
@@ -481,24 +521,24 @@ struct FusedArgs {
   int q0;                      // first quad of this launch
 };
 
-template <bool PAIR, int NQ, bool WRITE, bool GROUP, bool PACK>
+template <bool PAIR, int NQ, bool WRITE, bool GROUP, bool PACK, int HI>
 void LaunchFusedNQ(hipStream_t st, unsigned grid, const FusedArgs &a) {
-  const size_t lds = HistLdsBytes(NQ, PAIR);
+  const size_t lds = HistLdsBytes(NQ, PAIR, HI != 0);
   static bool configured = false;
   if (!configured) {
-    AllowLds(k_part_hist<PAIR, NQ, WRITE, GROUP, PACK>, lds);
+    AllowLds(k_part_hist<PAIR, NQ, WRITE, GROUP, PACK, HI>, lds);
     configured = true;
   }
-  hipLaunchKernelGGL((k_part_hist<PAIR, NQ, WRITE, GROUP, PACK>), dim3(grid), dim3(kHistThreads), lds, st,
+  hipLaunchKernelGGL((k_part_hist<PAIR, NQ, WRITE, GROUP, PACK, HI>), dim3(grid), dim3(kHistThreads), lds, st,
                      a.bins + (size_t)a.q0 * a.stride, a.bins_out ? a.bins_out + (size_t)a.q0 * a.stride : nullptr,
                      a.stride, a.F, a.g, a.g_out, a.h, a.h_out, a.shifts, a.split, a.tot, a.seg_start, a.work,
                      a.n_work, a.cursor, a.item_base, a.slab, a.slab_entries, a.split_bins, a.q0);
 }
 
-template <bool PAIR, bool WRITE, bool GROUP, bool PACK>
+template <bool PAIR, bool WRITE, bool GROUP, bool PACK, int HI = 0>
 void LaunchFused(int nq, hipStream_t st, unsigned grid, const FusedArgs &a) {
 #define ARB_CASE(N) \
-  case N: LaunchFusedNQ<PAIR, N, WRITE, GROUP, PACK>(st, grid, a); break;
+  case N: LaunchFusedNQ<PAIR, N, WRITE, GROUP, PACK, HI>(st, grid, a); break;
   switch (nq) {
     ARB_CASE(1) ARB_CASE(2) ARB_CASE(3) ARB_CASE(4) ARB_CASE(5) ARB_CASE(6) ARB_CASE(7) ARB_CASE(8)
     default: throw std::runtime_error("internal: bad quad count");
@@ -520,16 +560,23 @@ class HipTreeBuilder : public TreeBuilder {
     f64_ = cfg.internal.double_precision;
     trick_ = cfg.internal.use_hist_subtraction_trick;
     wide_ = dm_->bits == 16;
-    slots_ = dm_->slots;
+    hi_ = dm_->hi;
+    W_ = dm_->W();
+    hi_word_ = hi_ ? Q_ : -1;
+    report_slots_ = dm_->slots;
+    slots_ = hi_ ? kSlots : dm_->slots;  // bin 256 lives in a cell of its own behind the 256-bin histograms
     code_ = BinCode::Of(dm_->bits);
     if (wide_) {
       if (dm_->streamed) throw std::runtime_error("16-bit bins are not built for streamed matrices");
       nbin_total_ = F_ * slots_;
       slab_entries_ = nbin_total_;  // slabs are feature-major
     } else {
-      nbin_total_ = Q_ * 4 * kSlots;
+      hi_base_ = hi_ ? Q_ * 4 * kSlots : 0;
+      nbin_total_ = Q_ * 4 * kSlots + (hi_ ? Q_ * 4 : 0);
       slab_entries_ = HistBlocks(Q_) * kBlockEntries;
     }
+    // entries between the slabs of two work items: with ninth bits one more row, bin 256
+    slab_stride_ = wide_ ? slab_entries_ : HistBlocks(Q_) * (kBlockEntries + (hi_ ? kBlockFeatures : 0));
     if (cfg.objective >= kSoftMaxOneVsAll && K_ < 2) throw std::runtime_error("soft-max needs labels_count >= 2");
     if (cfg.objective < kSoftMaxOneVsAll && K_ != 1) throw std::runtime_error("labels_count must be 1 for this objective");
     const int last_nodes = 1 << (D_ - 2);
@@ -544,6 +591,8 @@ class HipTreeBuilder : public TreeBuilder {
     // the fused partition + histogram pass holds one histogram of all
     // features and builds only the smaller child
     single_group_ = Q_ <= quads_per_group_;
+    if (hi_ && (!single_group_ || HistLdsBytes(Q_, pair_, true) > kLdsBudget - 1024))
+      throw std::runtime_error("internal: ninth-bit ids need a matrix of one group of quads");
     // Matrices wider than one group of quads: rows stay in place as records, only (row id,
     // gradients) are re-ordered (kernels_indexed.h).
     // Taken when every feature fits ONE LDS histogram of the bins in use (a record is then read
@@ -595,11 +644,11 @@ class HipTreeBuilder : public TreeBuilder {
       const size_t br = dm_->block_rows;
       HIP_OK(hipStreamCreateWithFlags(&copy_stream_, hipStreamNonBlocking));
       for (int b = 0; b < 2; ++b) {
-        blk_[b] = DevAlloc<uint32_t>((size_t)Q_ * br);
+        blk_[b] = DevAlloc<uint32_t>((size_t)W_ * br);
         HIP_OK(hipEventCreateWithFlags(&ev_ready_[b], hipEventDisableTiming));
         HIP_OK(hipEventCreateWithFlags(&ev_free_[b], hipEventDisableTiming));
       }
-      stage_.bins = DevAlloc<uint32_t>((size_t)Q_ * br);
+      stage_.bins = DevAlloc<uint32_t>((size_t)W_ * br);
       stage_.g = DevAlloc<float>(br);
       stage_.h = DevAlloc<float>(br);
       d_node_of_ = DevAlloc<unsigned>(n_);
@@ -613,7 +662,7 @@ class HipTreeBuilder : public TreeBuilder {
     if (D_ > 2 && !streamed_) {
       for (int b = 0; b < 2; ++b) {
         if (indexed_) buf_[b].ids = DevAlloc<unsigned>(n_);
-        else buf_[b].bins = DevAlloc<uint32_t>((size_t)Q_ * stride_);
+        else buf_[b].bins = DevAlloc<uint32_t>((size_t)W_ * stride_);
         buf_[b].g = DevAlloc<float>(n_);
         buf_[b].h = pack_ ? nullptr : DevAlloc<float>(n_);
       }
@@ -644,12 +693,12 @@ class HipTreeBuilder : public TreeBuilder {
       d_seg_[b] = DevAlloc<unsigned>(max_nodes);
       d_hg_[b] = DevAlloc<long long>((size_t)last_nodes * nbin_total_);
       d_hh_[b] = DevAlloc<long long>((size_t)last_nodes * nbin_total_);
-      d_hc_[b] = DevAlloc<unsigned>((size_t)last_nodes * nbin_total_);
+      d_hc_[b] = DevAlloc<unsigned long long>((size_t)last_nodes * nbin_total_);
       // cells of bins that no row can have are never written (rows in place with fewer than 256
       // bins in use) and must read as zero
       HIP_OK(hipMemsetAsync(d_hg_[b], 0, (size_t)last_nodes * nbin_total_ * sizeof(long long), stream_));
       HIP_OK(hipMemsetAsync(d_hh_[b], 0, (size_t)last_nodes * nbin_total_ * sizeof(long long), stream_));
-      HIP_OK(hipMemsetAsync(d_hc_[b], 0, (size_t)last_nodes * nbin_total_ * sizeof(unsigned), stream_));
+      HIP_OK(hipMemsetAsync(d_hc_[b], 0, (size_t)last_nodes * nbin_total_ * sizeof(unsigned long long), stream_));
     }
     d_split_ = DevAlloc<SplitRec>(last_nodes);
     d_cand_ = DevAlloc<Cand>((size_t)last_nodes * F_);
@@ -681,7 +730,7 @@ class HipTreeBuilder : public TreeBuilder {
     d_wave_left_ = DevAlloc<unsigned>((size_t)max_part_items_ * kItemWaves);
     d_item_left_ = DevAlloc<unsigned>((size_t)2 * max_part_items_);  // also the claimed bases of the fused pass
     d_cursor2_ = DevAlloc<unsigned>((size_t)2 * last_nodes);
-    d_slab_ = DevAlloc<unsigned long long>((size_t)std::max(max_hist_items_, max_part_items_) * slab_entries_ * (pair_ ? 2 : 1));
+    d_slab_ = DevAlloc<unsigned long long>((size_t)std::max(max_hist_items_, max_part_items_) * slab_stride_ * (pair_ ? 2 : 1));
     d_shifts_ = DevAlloc<int>(2);
     d_records_ = DevAlloc<uint32_t>(kRecordRing * RecordWords());
     d_gmax_ = DevAlloc<unsigned>(1);
@@ -805,7 +854,7 @@ class HipTreeBuilder : public TreeBuilder {
   void GetLeaves(uint32_t *out) override {
     if (!leaf_valid_) {  // the last pass did not record them: walk the last tree now
       hipLaunchKernelGGL(k_leaf_ids, dim3(GridFor(n_, 256, 8192)), dim3(256), 0, stream_, dm_->bins, stride_, d_tfid_,
-                         d_tbin_, D_, d_leaf_, n_, code_);
+                         d_tbin_, D_, d_leaf_, n_, code_, hi_word_);
       HIP_OK(hipGetLastError());
       leaf_valid_ = true;
     }
@@ -1017,14 +1066,24 @@ class HipTreeBuilder : public TreeBuilder {
 #undef ARB_REC
         if (timing_) ++(root ? timings_.hist_root_launches : timings_.hist_deep_launches);
         break;
-      } else if (pair_) {
-        LaunchHist<true>(nq, stream_, grid, cur.bins, stride_, q0, F_, cur.g, cur.h, d_shifts_, d_hwork_, d_nwork_, d_slab_, slab_entries_);
       } else {
-        LaunchHist<false>(nq, stream_, grid, cur.bins, stride_, q0, F_, cur.g, cur.h, d_shifts_, d_hwork_, d_nwork_, d_slab_, slab_entries_);
+        HistLaunch(nq, grid, cur.bins, stride_, q0, cur.g, cur.h);
       }
       if (timing_) ++(root ? timings_.hist_root_launches : timings_.hist_deep_launches);
     }
     if (timing_ && root) timings_.hist_root_rows += n_;
+  }
+
+  // k_hist over quads [q0, q0 + nq) of rows laid out with `stride` words between columns
+  void HistLaunch(int nq, unsigned grid, const uint32_t *bins, size_t stride, int q0, const float *g, const float *h) {
+    if (hi_ && pair_)
+      LaunchHist<true, 1>(nq, stream_, grid, bins, stride, q0, F_, g, h, d_shifts_, d_hwork_, d_nwork_, d_slab_, slab_stride_);
+    else if (hi_)
+      LaunchHist<false, 1>(nq, stream_, grid, bins, stride, q0, F_, g, h, d_shifts_, d_hwork_, d_nwork_, d_slab_, slab_stride_);
+    else if (pair_)
+      LaunchHist<true>(nq, stream_, grid, bins, stride, q0, F_, g, h, d_shifts_, d_hwork_, d_nwork_, d_slab_, slab_stride_);
+    else
+      LaunchHist<false>(nq, stream_, grid, bins, stride, q0, F_, g, h, d_shifts_, d_hwork_, d_nwork_, d_slab_, slab_stride_);
   }
 
   void Reduce(int L, int hb, bool by_parent, int parent_state, bool trick, bool accumulate = false) {
@@ -1036,15 +1095,15 @@ class HipTreeBuilder : public TreeBuilder {
     const int lay_blocks = indexed_ && rec_one_launch_ ? rec_lay_blocks_ : 0;
     // 16-bit bins: feature-major slabs; else the entries of the bins in use of every 16-feature block
     dim3 grid(wide_ ? (slab_entries_ + entries - 1) / entries
-                    : slab_entries_ / kBlockEntries * ((lds_slots * kBlockFeatures + entries - 1) / entries),
+                    : slab_entries_ / kBlockEntries * ((lds_slots * kBlockFeatures + entries - 1) / entries) + (hi_ ? 1 : 0),
               L);
 #define ARB_REDUCE(P, LN)                                                                                          \
-  hipLaunchKernelGGL((k_hist_reduce<P, LN>), grid, dim3(1024), 0, stream_, d_slab_, slab_entries_, nbin_total_,   \
+  hipLaunchKernelGGL((k_hist_reduce<P, LN, unsigned long long>), grid, dim3(1024), 0, stream_, d_slab_, slab_entries_, nbin_total_,   \
                      d_node_first_, d_node_items_, by_parent ? 1 : 0, d_split_, d_tot_[parent_state], d_hg_[hb], \
                      d_hh_[hb], d_hc_[hb], d_hg_[hb ^ 1], d_hh_[hb ^ 1], d_hc_[hb ^ 1], trick ? 1 : 0,           \
                      accumulate ? 1 : 0, wide_ ? 1 : 0,                                                           \
                      indexed_ && rec_one_launch_ ? HistBlocks(Q_) : HistBlocks(quads_per_group_),                \
-                     lds_slots, lay_blocks)
+                     lds_slots, lay_blocks, hi_base_)
     if (pair_) {
       if (wide_blocks) ARB_REDUCE(true, 4);
       else ARB_REDUCE(true, 16);
@@ -1076,7 +1135,7 @@ class HipTreeBuilder : public TreeBuilder {
     // one: logistic objective, gradients of the next round wanted, all quads in
     // one LDS histogram next to the node arrays.
     const bool next_grad = !inspect_ && K_ == 1;
-    const size_t final_lds = FinalHistLdsBytes(Q_, D_);
+    const size_t final_lds = FinalHistLdsBytes(Q_, D_, hi_);
     const bool final_hist = next_grad && cfg_.objective == kLogisticRegression && single_group_ && !wide_ &&
                             final_lds <= kLdsBudget;
     int state = 0;  // d_tot_/d_seg_[state] describe the nodes of the current level
@@ -1091,7 +1150,7 @@ class HipTreeBuilder : public TreeBuilder {
         Reduce(1, hb, false, state, false);
         // (the last pass of the previous tree has also summed the root's totals)
         if (!root_totals_ready_)
-          hipLaunchKernelGGL(k_root_from_hist, dim3(1), dim3(64), 0, stream_, d_hg_[hb], d_hh_[hb], d_tot_[state], slots_);
+          hipLaunchKernelGGL(k_root_from_hist, dim3(1), dim3(64), 0, stream_, d_hg_[hb], d_hh_[hb], d_tot_[state], slots_, hi_base_);
         root_totals_ready_ = false;
       } else {
         // rows are in the order of level-1; the parents' state is state ^ 1
@@ -1108,11 +1167,13 @@ class HipTreeBuilder : public TreeBuilder {
             const int nq = std::min(quads_per_group_, Q_ - q0);
             FusedArgs a{src.bins, last ? nullptr : dst.bins, stride_, F_, src.g, q0 == 0 ? dst.g : nullptr, src.h,
                         q0 == 0 ? dst.h : nullptr, d_shifts_, d_split_, d_tot_[ps], d_seg_[ps], d_pwork_,
-                        d_nwork_ + 1, q0 == 0 ? d_cursor2_ : nullptr, d_item_left_, d_slab_, slab_entries_, src.bins,
+                        d_nwork_ + 1, q0 == 0 ? d_cursor2_ : nullptr, d_item_left_, d_slab_, slab_stride_, src.bins,
                         q0};
 #define ARB_FUSED(P, W)                                                       \
   do {                                                                        \
-    if (P && pack_ && single_group_) LaunchFused<P, W, false, P>(nq, stream_, grid, a); \
+    if (hi_ && P && pack_) LaunchFused<P, W, false, P, 1>(nq, stream_, grid, a); \
+    else if (hi_) LaunchFused<P, W, false, false, 1>(nq, stream_, grid, a);   \
+    else if (P && pack_ && single_group_) LaunchFused<P, W, false, P>(nq, stream_, grid, a); \
     else if (P && pack_) LaunchFused<P, W, true, P>(nq, stream_, grid, a);    \
     else if (single_group_) LaunchFused<P, W, false, false>(nq, stream_, grid, a); \
     else LaunchFused<P, W, true, false>(nq, stream_, grid, a);                \
@@ -1147,7 +1208,7 @@ class HipTreeBuilder : public TreeBuilder {
                                  d_wave_left_, d_item_left_);
           } else {
             hipLaunchKernelGGL(k_part_count, dim3(grid), dim3(kHistThreads), 0, stream_, src.bins, stride_, d_split_,
-                               d_pwork_, d_nwork_ + 1, d_wave_left_, d_item_left_, code_);
+                               d_pwork_, d_nwork_ + 1, d_wave_left_, d_item_left_, code_, hi_word_);
             LaunchPartRows(grid, src, dst, ps);
           }
           HistOfNodes(dst, state, L, trick_, trick_ ? n_ / 2 : n_, false, level);
@@ -1213,7 +1274,7 @@ class HipTreeBuilder : public TreeBuilder {
   int CopyBlockIn(size_t b) {
     const int buf = (int)(next_copy_++ & 1);
     if (buf_used_[buf]) HIP_OK(hipStreamWaitEvent(copy_stream_, ev_free_[buf], 0));
-    HIP_OK(hipMemcpyAsync(blk_[buf], dm_->host_blocks[b], (size_t)Q_ * dm_->block_rows * sizeof(uint32_t),
+    HIP_OK(hipMemcpyAsync(blk_[buf], dm_->host_blocks[b], (size_t)W_ * dm_->block_rows * sizeof(uint32_t),
                           hipMemcpyHostToDevice, copy_stream_));
     HIP_OK(hipEventRecord(ev_ready_[buf], copy_stream_));
     buf_used_[buf] = true;
@@ -1268,12 +1329,12 @@ class HipTreeBuilder : public TreeBuilder {
   // Stand-alone partition: groups of up to eight words per launch; the first
   // launch also moves the gradients.
   void LaunchPartRows(unsigned grid, const RowBuffers &src, const RowBuffers &dst, int ps) {
-    for (int q0 = 0; q0 < Q_; q0 += 8) {
-      const int nq = std::min(8, Q_ - q0);
+    for (int q0 = 0; q0 < W_; q0 += 8) {  // (the ninth-bit word moves like a quad)
+      const int nq = std::min(8, W_ - q0);
 #define ARB_PART(P, N, G)                                                                                        \
   hipLaunchKernelGGL((k_part_rows<P, N, G>), dim3(grid), dim3(kHistThreads), 0, stream_, src.bins, dst.bins,    \
                      stride_, q0, src.g, dst.g, src.h, dst.h, d_split_, d_seg_[ps], d_pwork_, d_nwork_ + 1,      \
-                     d_wave_left_, d_item_left_, code_)
+                     d_wave_left_, d_item_left_, code_, hi_word_)
 #define ARB_PART_N(N)                                          \
   case N:                                                      \
     if (q0 == 0) {                                             \
@@ -1334,7 +1395,7 @@ class HipTreeBuilder : public TreeBuilder {
 #define ARB_FINAL(M, N) \
   hipLaunchKernelGGL((k_final<M, N>), dim3(grid), dim3(256), lds, stream_, bins, stride, d_tfid_, d_tbin_, D_, \
                      d_weights_, yh, d_y_ + row0, d_leaf_ + row0, d_g_ + row0, d_h_ ? d_h_ + row0 : nullptr, d_gmax_, rows, code_, \
-                     walk_bytes, dm_->stride8)
+                     walk_bytes, dm_->stride8, hi_word_)
 #define ARB_FINAL_Q(N) \
   do { if (mode == 1) ARB_FINAL(1, N); else if (mode == 2) ARB_FINAL(2, N); else ARB_FINAL(0, N); } while (0)
     switch (Q_ <= 8 && !wide_ ? Q_ : 0) {
@@ -1354,22 +1415,28 @@ class HipTreeBuilder : public TreeBuilder {
 
   void LaunchFinalHist(unsigned grid, int label, size_t lds) {
     float *yh = d_yhat_ + (size_t)label * n_;
-#define ARB_CASE(N)                                                                                              \
-  case N: {                                                                                                      \
+#define ARB_FH(N, H)                                                                                             \
+  do {                                                                                                           \
     static bool configured = false;                                                                              \
     if (!configured) {                                                                                           \
-      AllowLds(k_final_hist<N>, kLdsBudget);                                                                     \
+      AllowLds(k_final_hist<N, H>, kLdsBudget);                                                                  \
       configured = true;                                                                                         \
     }                                                                                                            \
-    hipLaunchKernelGGL((k_final_hist<N>), dim3(grid), dim3(kHistThreads), lds, stream_, dm_->bins, stride_, F_, \
-                       d_tfid_, d_tbin_, D_, d_weights_, yh, d_y_, (unsigned *)nullptr, d_g_, d_h_, d_shifts_,   \
-                       d_hwork_, d_nwork_, d_slab_, slab_entries_, d_tot_[0]);                                   \
-  } break;
+    hipLaunchKernelGGL((k_final_hist<N, H>), dim3(grid), dim3(kHistThreads), lds, stream_, dm_->bins, stride_,  \
+                       F_, d_tfid_, d_tbin_, D_, d_weights_, yh, d_y_, (unsigned *)nullptr, d_g_, d_h_,          \
+                       d_shifts_, d_hwork_, d_nwork_, d_slab_, slab_stride_, d_tot_[0]);                         \
+  } while (0)
+#define ARB_CASE(N)           \
+  case N:                     \
+    if (hi_) ARB_FH(N, 1);    \
+    else ARB_FH(N, 0);        \
+    break;
     switch (Q_) {
       ARB_CASE(1) ARB_CASE(2) ARB_CASE(3) ARB_CASE(4) ARB_CASE(5) ARB_CASE(6) ARB_CASE(7) ARB_CASE(8)
       default: throw std::runtime_error("internal: bad quad count");
     }
 #undef ARB_CASE
+#undef ARB_FH
   }
 
   // One tree over a streamed matrix: every level copies every block in once
@@ -1392,16 +1459,16 @@ class HipTreeBuilder : public TreeBuilder {
         HIP_OK(hipStreamWaitEvent(stream_, ev_ready_[buf], 0));
         Mark(kPartition);
         hipLaunchKernelGGL(k_stream_route, dim3(GridFor(rows, 256, 1024)), dim3(256), 0, stream_, blk_[buf], br, rows,
-                           level, trick ? 1 : 0, d_split_, d_tot_[state], d_node_of_ + row0, d_blk_cnt_);
+                           level, trick ? 1 : 0, d_split_, d_tot_[state], d_node_of_ + row0, d_blk_cnt_, hi_word_);
         hipLaunchKernelGGL(k_stream_segments, dim3(1), dim3(1024), 0, stream_, d_blk_cnt_, L, d_blk_tot_, d_blk_seg_,
                            d_cursor_);
         if (pair_)
           hipLaunchKernelGGL(k_stream_gather<true>, dim3(GridFor(rows, 256, 2048)), dim3(256), 0, stream_, blk_[buf],
-                             br, Q_, rows, orig.g + row0, orig.h + row0, d_node_of_ + row0, level, trick ? 1 : 0,
+                             br, W_, rows, orig.g + row0, orig.h + row0, d_node_of_ + row0, level, trick ? 1 : 0,
                              d_tot_[state], d_cursor_, stage_.bins, br, stage_.g, stage_.h);
         else
           hipLaunchKernelGGL(k_stream_gather<false>, dim3(GridFor(rows, 256, 2048)), dim3(256), 0, stream_, blk_[buf],
-                             br, Q_, rows, orig.g + row0, orig.h + row0, d_node_of_ + row0, level, trick ? 1 : 0,
+                             br, W_, rows, orig.g + row0, orig.h + row0, d_node_of_ + row0, level, trick ? 1 : 0,
                              d_tot_[state], d_cursor_, stage_.bins, br, stage_.g, stage_.h);
         HIP_OK(hipEventRecord(ev_free_[buf], stream_));
         // histograms of the gathered rows, added to the level's histograms
@@ -1412,17 +1479,12 @@ class HipTreeBuilder : public TreeBuilder {
         Mark(level == 0 ? kHistRoot : kHistDeep);
         for (int q0 = 0; q0 < Q_; q0 += quads_per_group_) {
           const int nq = std::min(quads_per_group_, Q_ - q0);
-          if (pair_)
-            LaunchHist<true>(nq, stream_, grid, stage_.bins, br, q0, F_, stage_.g, stage_.h, d_shifts_, d_hwork_,
-                             d_nwork_, d_slab_, slab_entries_);
-          else
-            LaunchHist<false>(nq, stream_, grid, stage_.bins, br, q0, F_, stage_.g, stage_.h, d_shifts_, d_hwork_,
-                              d_nwork_, d_slab_, slab_entries_);
+          HistLaunch(nq, grid, stage_.bins, br, q0, stage_.g, stage_.h);
         }
         Reduce(L, hb, false, state, false, b > 0);
       }
       if (level == 0)
-        hipLaunchKernelGGL(k_root_from_hist, dim3(1), dim3(64), 0, stream_, d_hg_[hb], d_hh_[hb], d_tot_[state], slots_);
+        hipLaunchKernelGGL(k_root_from_hist, dim3(1), dim3(64), 0, stream_, d_hg_[hb], d_hh_[hb], d_tot_[state], slots_, hi_base_);
       if (trick)
         hipLaunchKernelGGL(k_sibling, dim3((nbin_total_ + 255) / 256, L), dim3(256), 0, stream_, d_hg_[hb], d_hh_[hb],
                            d_hc_[hb], d_hg_[hb ^ 1], d_hh_[hb ^ 1], d_hc_[hb ^ 1], d_tot_[state], level, nbin_total_);
@@ -1474,19 +1536,20 @@ class HipTreeBuilder : public TreeBuilder {
   void KeepHist(int level, int L, int hb) {
     const size_t cells = (size_t)L * nbin_total_;
     std::vector<long long> g(cells), h(cells);
-    std::vector<unsigned> c(cells);
+    std::vector<unsigned long long> c(cells);
     HIP_OK(hipStreamSynchronize(stream_));
     HIP_OK(hipMemcpy(g.data(), d_hg_[hb], cells * sizeof(long long), hipMemcpyDeviceToHost));
     HIP_OK(hipMemcpy(h.data(), d_hh_[hb], cells * sizeof(long long), hipMemcpyDeviceToHost));
-    HIP_OK(hipMemcpy(c.data(), d_hc_[hb], cells * sizeof(unsigned), hipMemcpyDeviceToHost));
+    HIP_OK(hipMemcpy(c.data(), d_hc_[hb], cells * sizeof(unsigned long long), hipMemcpyDeviceToHost));
     // keep [node][F][slots][3] (padding features of the last quad dropped)
     std::vector<int64_t> &out = kept_hist_[level];
-    out.resize((size_t)L * F_ * slots_ * 3);
+    out.resize((size_t)L * F_ * report_slots_ * 3);
     for (int nd = 0; nd < L; ++nd)
       for (int f = 0; f < F_; ++f)
-        for (int b = 0; b < slots_; ++b) {
-          const size_t s = (size_t)nd * nbin_total_ + (size_t)f * slots_ + b;
-          const size_t d = (((size_t)nd * F_ + f) * slots_ + b) * 3;
+        for (int b = 0; b < report_slots_; ++b) {
+          // (ninth bits: bin 256 of feature f is cell hi_base_ + f of the node)
+          const size_t s = (size_t)nd * nbin_total_ + (b < slots_ ? (size_t)f * slots_ + b : (size_t)hi_base_ + f);
+          const size_t d = (((size_t)nd * F_ + f) * report_slots_ + b) * 3;
           out[d] = g[s];
           out[d + 1] = pair_ ? h[s] : 0;
           out[d + 2] = c[s];
@@ -1509,6 +1572,12 @@ class HipTreeBuilder : public TreeBuilder {
   int rec_lay_blocks_ = 0;      // blocks that histogram is laid out for (a power of two), 0: as many as the matrix has
   uint8_t *d_dec_ = nullptr;  // indexed mode: split decision of the row at each position
   bool wide_ = false;     // 16-bit bins: two features per word, slots_ histogram slots per feature
+  bool hi_ = false;       // 8-bit bins plus a ninth-bit word per row (ids up to 256)
+  int W_ = 0;             // words of a row: Q_, one more with ninth bits
+  int hi_word_ = -1;      // column of the ninth-bit word, -1: none
+  int hi_base_ = 0;       // first cell of the bin-256 cells of a node's histogram, 0: none
+  int slab_stride_ = 0;   // histogram entries from one work item's slab to the next
+  int report_slots_ = kSlots;  // slots per feature as GetLevelHist reports them
   int slots_ = kSlots;
   int wide_group_ = 2;    // features per histogram launch with 16-bit bins
   BinCode code_ = BinCode{2, 8};
@@ -1552,7 +1621,7 @@ class HipTreeBuilder : public TreeBuilder {
   NodeSum *d_tot_[2] = {nullptr, nullptr};
   unsigned *d_seg_[2] = {nullptr, nullptr};
   long long *d_hg_[2] = {nullptr, nullptr}, *d_hh_[2] = {nullptr, nullptr};
-  unsigned *d_hc_[2] = {nullptr, nullptr};
+  unsigned long long *d_hc_[2] = {nullptr, nullptr};  // 64-bit: a cell of a streamed matrix may hold 2^32 rows and more
   SplitRec *d_split_ = nullptr;
   Cand *d_cand_ = nullptr;
   WorkItem *d_hwork_ = nullptr, *d_pwork_ = nullptr;

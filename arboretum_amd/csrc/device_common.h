@@ -45,9 +45,10 @@ constexpr int kBlockFeatures = 16;
 constexpr int kBlockQuads = 4;
 constexpr int kBlockEntries = kBlockFeatures * kSlots;  // 4096
 constexpr int HistBlocks(int nq) { return (nq + kBlockQuads - 1) / kBlockQuads; }
-// LDS bytes of a histogram of nq quads
-constexpr size_t HistLdsBytes(int nq, bool pair) {
-  return (size_t)HistBlocks(nq) * kBlockEntries * 8 * (pair ? 2 : 1);
+// LDS bytes of a histogram of nq quads; hi: one more row of entries, bin 256
+// of every feature (the ninth-bit word, see SplitTest)
+constexpr size_t HistLdsBytes(int nq, bool pair, bool hi = false) {
+  return (size_t)HistBlocks(nq) * (kBlockEntries + (hi ? kBlockFeatures : 0)) * 8 * (pair ? 2 : 1);
 }
 
 // Logistic gradients of 0/1 labels can travel as ONE float per row:
@@ -103,6 +104,32 @@ struct BinCode {
     return (word >> (bits * (fid & ((1 << wshift) - 1)))) & ((1u << bits) - 1u);
   }
 };
+
+// Bin id 256.  With hist_size 256 a feature that fills all 256 value bins and
+// also has missing values needs 257 ids (NaN -> bin `size`,
+// src/core/cuda_helpers.h:207-222).  Such an id is stored as byte 255 plus one
+// bit in an extra word of the row, the "ninth-bit word": bit f set means the id
+// of feature f is 256.  The word follows the quads of the row (column Q of a
+// matrix of Q quads, at most 32 features) and moves with them.
+//
+// The test "id > split bin" on one 32-bit word of a row:
+//   split bin < 255 (or no ninth bits): the feature's byte against the bin (an
+//     id of 256 has byte 255, which is larger than any such bin);
+//   split bin 255: only an id of 256 goes right: the feature's ninth bit;
+//   node not split: nobody goes right.
+struct SplitTest {
+  int word;  // column of the row the test reads
+  unsigned shift, mask;
+  int thr;
+  __device__ __forceinline__ bool Right(uint32_t v) const { return (int)((v >> shift) & mask) > thr; }
+};
+// hi_word: column of the ninth-bit word, negative when the matrix has none
+__device__ __forceinline__ SplitTest MakeSplitTest(const SplitRec &s, BinCode code, int hi_word) {
+  if (s.fid < 0) return SplitTest{0, 0u, 0u, 0};
+  if (hi_word >= 0 && s.bin >= 255) return SplitTest{hi_word, (unsigned)s.fid, 1u, 0};
+  return SplitTest{code.Word(s.fid), (unsigned)(code.bits * (s.fid & ((1 << code.wshift) - 1))),
+                   (1u << code.bits) - 1u, s.bin};
+}
 
 __device__ __forceinline__ float WaveMaxF(float v) {
   for (int off = 32; off > 0; off >>= 1) v = fmaxf(v, __shfl_down(v, off));

@@ -112,13 +112,15 @@ k_tree_end(const SplitRec *__restrict__ split, const NodeSum *__restrict__ tot, 
 // NQ > 0: the matrix has NQ quads, all loaded up front (coalesced, independent
 // loads) and selected in registers; NQ == 0: any width, one dependent load per
 // level, from the byte columns when the matrix has them (bytes != null).
+// hi_word >= 0: column of the rows' ninth-bit word; a split at bin 255 sends
+// right only the rows whose id is 256 (SplitTest).
 template <int NEXT_GRAD, int NQ>
 __global__ void __launch_bounds__(256)
 k_final(const uint32_t *__restrict__ bins, size_t stride, const int *__restrict__ t_fid,
         const int *__restrict__ t_bin, int depth, const float *__restrict__ weights,
         float *__restrict__ yhat, const float *__restrict__ y, unsigned *__restrict__ leaf_of,
         float *__restrict__ g, float *__restrict__ h, unsigned *__restrict__ gmax_bits, size_t n,
-        BinCode code, const uint8_t *__restrict__ bytes, size_t stride8) {
+        BinCode code, const uint8_t *__restrict__ bytes, size_t stride8, int hi_word) {
   extern __shared__ int s_nodes[];  // fid[internal], bin[internal]
   const int internal = (1 << (depth - 1)) - 1;
   for (int i = threadIdx.x; i < internal; i += blockDim.x) {
@@ -139,7 +141,9 @@ k_final(const uint32_t *__restrict__ bins, size_t stride, const int *__restrict_
       const int id = (1 << level) - 1 + (int)node;
       const int fid = s_nodes[id], bin = s_nodes[internal + id];
       unsigned right = 0;
-      if (bin >= 0) {
+      if (bin >= 255 && hi_word >= 0) {
+        right = (bins[(size_t)hi_word * stride + i] >> fid) & 1u;
+      } else if (bin >= 0) {
         if (NQ > 0) {  // 8-bit bins, all quads in registers
           uint32_t b4 = 0;
           const int fq = fid >> 2;
@@ -179,8 +183,8 @@ k_final(const uint32_t *__restrict__ bins, size_t stride, const int *__restrict_
 }
 
 // LDS bytes of k_final_hist: histogram, node table, exp table, leaf weights
-constexpr size_t FinalHistLdsBytes(int nq, int depth) {
-  return HistLdsBytes(nq, true) + (size_t)((1 << (depth - 1)) - 1) * 8 + 32 * 8 + ((size_t)1 << (depth - 1)) * 4;
+constexpr size_t FinalHistLdsBytes(int nq, int depth, bool hi = false) {
+  return HistLdsBytes(nq, true, hi) + (size_t)((1 << (depth - 1)) - 1) * 8 + 32 * 8 + ((size_t)1 << (depth - 1)) * 4;
 }
 
 // Last pass of a tree fused with the root histogram of the next one
@@ -192,7 +196,8 @@ constexpr size_t FinalHistLdsBytes(int nq, int depth) {
 // leaf_of may be null: the leaf ids are then not recorded (k_leaf_ids
 // computes them on demand).  root_tot (may be null): the gradient totals of
 // the next root are added to root_tot[0].g / .h, which the caller has zeroed.
-template <int NQ>
+// HI: column NQ of the rows is their ninth-bit word (SplitTest).
+template <int NQ, int HI = 0>
 __global__ void __launch_bounds__(kHistThreads)
 k_final_hist(const uint32_t *__restrict__ bins, size_t stride, int F, const int *__restrict__ t_fid,
              const int *__restrict__ t_bin, int depth, const float *__restrict__ weights,
@@ -204,12 +209,15 @@ k_final_hist(const uint32_t *__restrict__ bins, size_t stride, int F, const int 
   const unsigned w = blockIdx.x;
   if (w >= *n_work) return;
   const WorkItem it = work[w];
-  constexpr int words = (int)(HistLdsBytes(NQ, true) / 8);
+  constexpr int NW = NQ + HI;
+  constexpr int words = (int)(HistLdsBytes(NQ, true, HI != 0) / 8);
   // Node table for the walk, two words per internal node: a byte selector for
   // v_perm_b32 that picks byte fid % 8 out of a pair of quads (the other three
   // result bytes are zero), and the split bin in bits 0-7 with the pair fid / 8
-  // in bits 8-9.  A node that was not split compares against 255: no bin id is
-  // larger, so every row stays left.
+  // in bits 8-9.  A node that was not split compares against 255: no byte is
+  // larger, so every row stays left.  HI: a node split at bin 255 has bit 31
+  // set and the feature in bits 16-20: the row goes right when that bit of its
+  // ninth-bit word is set (its id is 256).
   uint2 *s_tree = reinterpret_cast<uint2 *>(lds + words);
   const int internal = (1 << (depth - 1)) - 1, leaves = internal + 1;
   // the exp table and the leaf weights are read from LDS as well
@@ -223,14 +231,15 @@ k_final_hist(const uint32_t *__restrict__ bins, size_t stride, int F, const int 
     uint2 nd;
     nd.x = 0x0c0c0c00u | (unsigned)(fid & 7);
     nd.y = (bin < 0 ? 255u : (unsigned)bin) | ((unsigned)(fid >> 3) << 8);
+    if (HI && bin >= 255) nd.y |= 0x80000000u | ((unsigned)fid << 16);
     s_tree[i] = nd;
   }
   __syncthreads();
   const int sg = shifts[0], sh = shifts[1];
   // quad q of a row, zero past the last one
-  auto quad = [](const uint32_t (&b)[NQ], int q) { return q < NQ ? b[q < NQ ? q : 0] : 0u; };
+  auto quad = [](const uint32_t (&b)[NW], int q) { return q < NQ ? b[q < NQ ? q : 0] : 0u; };
   // one step of the walk of a row from `node`, whose table entry is nd
-  auto step_at = [&](const uint32_t (&b)[NQ], unsigned node, uint2 nd) {
+  auto step_at = [&](const uint32_t (&b)[NW], unsigned node, uint2 nd) {
     // the row's bin of the split feature: byte fid % 8 of each pair of quads, then the pair
     const uint32_t t0 = __builtin_amdgcn_perm(quad(b, 1), quad(b, 0), nd.x);
     const uint32_t t1 = __builtin_amdgcn_perm(quad(b, 3), quad(b, 2), nd.x);
@@ -239,9 +248,11 @@ k_final_hist(const uint32_t *__restrict__ bins, size_t stride, int F, const int 
     const unsigned pair = nd.y >> 8;
     const uint32_t lo = pair == 1u ? t1 : t0, hi = pair == 3u ? t3 : t2;
     const uint32_t v = pair >= 2u ? hi : lo;
-    return node * 2 + (v > (nd.y & 255u) ? 1u : 0u);  // bin >= q + 1 goes right (builder.h:107-123)
+    unsigned right = v > (nd.y & 255u) ? 1u : 0u;  // bin >= q + 1 goes right (builder.h:107-123)
+    if (HI) right = (int)nd.y < 0 ? (b[NW - 1] >> ((nd.y >> 16) & 31u)) & 1u : right;
+    return node * 2 + right;
   };
-  auto step = [&](const uint32_t (&b)[NQ], unsigned node, int level) {
+  auto step = [&](const uint32_t (&b)[NW], unsigned node, int level) {
     return step_at(b, node, s_tree[(1 << level) - 1 + (int)node]);
   };
   // The entries of the two top levels stay in registers: every row passes
@@ -264,9 +275,9 @@ k_final_hist(const uint32_t *__restrict__ bins, size_t stride, int F, const int 
     const unsigned r0 = base + threadIdx.x, r1 = r0 + kHistThreads;
     const bool v0 = r0 < it.end, v1 = r1 < it.end;
     const unsigned a0 = v0 ? r0 : it.begin, a1 = v1 ? r1 : it.begin;
-    uint32_t b0[NQ], b1[NQ];
+    uint32_t b0[NW], b1[NW];
 #pragma unroll
-    for (int q = 0; q < NQ; ++q) {
+    for (int q = 0; q < NW; ++q) {
       b0[q] = __builtin_nontemporal_load(&bins[(size_t)q * stride + a0]);
       b1[q] = __builtin_nontemporal_load(&bins[(size_t)q * stride + a1]);
     }
@@ -299,18 +310,18 @@ k_final_hist(const uint32_t *__restrict__ bins, size_t stride, int F, const int 
     const float h0 = s0 * (1.0f - s0), h1 = s1 * (1.0f - s1);
     if (v0) record(n0, yh0, s0, y0, g0, h0, r0);
     if (v1) record(n1, yh1, s1, y1, g1, h1, r1);
-    if (v0) AccumulateRow<true, NQ>(lds, b0, g0, h0, sg, sh, 0, F);
-    if (v1) AccumulateRow<true, NQ>(lds, b1, g1, h1, sg, sh, 0, F);
+    if (v0) AccumulateRow<true, NQ, HI>(lds, b0, g0, h0, sg, sh, 0, F);
+    if (v1) AccumulateRow<true, NQ, HI>(lds, b1, g1, h1, sg, sh, 0, F);
   }
-  FlushSlab<true, NQ>(lds, slab, w, slab_entries, 0);
+  FlushSlab<true, NQ, HI>(lds, slab, w, slab_entries, 0);
   // Totals of the next root (garden.cu:432-435 reduces the gradient array):
   // every row sits in exactly one slot of feature 0, so this item's share is
   // the sum of that feature's slots; integers, so the order of the adds over
   // the work items does not matter.  root_tot starts at zero.
   if (root_tot != nullptr && threadIdx.x < 64) {
     long long a = 0, b = 0;
-    for (int bin = threadIdx.x; bin < kSlots; bin += 64) {
-      const unsigned word = HistWord<true>(bin * kBlockFeatures, HistLds<NQ>::blocks);
+    for (int bin = threadIdx.x; bin < kSlots + HI; bin += 64) {  // (bin 256: the row behind the 256 bins)
+      const unsigned word = (unsigned)bin * (2u * kBlockFeatures * HistLds<NQ>::blocks);  // feature 0
       const unsigned long long w0 = lds[word];
       a += ((long long)(w0 << (64 - kCountShift))) >> (64 - kCountShift);
       b += (long long)lds[word + kWord1];
@@ -328,7 +339,8 @@ k_final_hist(const uint32_t *__restrict__ bins, size_t stride, int F, const int 
 // caller that asks after a last pass that did not record the leaves.
 __global__ void __launch_bounds__(256)
 k_leaf_ids(const uint32_t *__restrict__ bins, size_t stride, const int *__restrict__ t_fid,
-           const int *__restrict__ t_bin, int depth, unsigned *__restrict__ leaf_of, size_t n, BinCode code) {
+           const int *__restrict__ t_bin, int depth, unsigned *__restrict__ leaf_of, size_t n, BinCode code,
+           int hi_word) {
   for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < n;
        i += (size_t)gridDim.x * blockDim.x) {
     unsigned node = 0;
@@ -336,7 +348,8 @@ k_leaf_ids(const uint32_t *__restrict__ bins, size_t stride, const int *__restri
       const int id = (1 << level) - 1 + (int)node;
       const int fid = t_fid[id], bin = t_bin[id];
       unsigned right = 0;
-      if (bin >= 0) right = (int)code.Bin(bins[(size_t)code.Word(fid) * stride + i], fid) > bin ? 1u : 0u;
+      if (bin >= 255 && hi_word >= 0) right = (bins[(size_t)hi_word * stride + i] >> fid) & 1u;
+      else if (bin >= 0) right = (int)code.Bin(bins[(size_t)code.Word(fid) * stride + i], fid) > bin ? 1u : 0u;
       node = node * 2 + right;
     }
     leaf_of[i] = node;

@@ -38,9 +38,12 @@ __host__ __device__ __forceinline__ unsigned HistWord(unsigned entry, int blocks
 // byte (t + l) % 4 of that quad, so the 16 lanes of a pass of the LDS atomic
 // touch 16 different features = 16 different bank pairs.  q_first: first quad
 // of this launch (a multiple of 4).
-template <bool PAIR, int NQ>
+// HI: b[NQ] is the row's ninth-bit word (bit f set: the id of feature f is
+// 256, its byte 255); such an id falls into the row of entries that follows bin
+// 255 in this bin-major layout, so the address arithmetic is the same.
+template <bool PAIR, int NQ, int HI = 0>
 __device__ __forceinline__ void AccumulateRow(unsigned long long *__restrict__ lds,
-                                              const uint32_t (&b)[NQ], float gv, float hv, int sg,
+                                              const uint32_t (&b)[NQ + HI], float gv, float hv, int sg,
                                               int sh, int q_first, int F) {
   using L = HistLds<NQ>;
   const unsigned long long w0 = (1ull << kCountShift) + (unsigned long long)ToFixed(gv, sg);
@@ -62,8 +65,9 @@ __device__ __forceinline__ void AccumulateRow(unsigned long long *__restrict__ l
 #pragma unroll
       for (int t = 0; t < 4; ++t) {
         const unsigned bi = ((unsigned)t + i) & 3u;  // byte of the quad
-        const unsigned bin = __builtin_amdgcn_ubfe(sel, 8u * bi, 8u);  // one v_bfe_u32
+        unsigned bin = __builtin_amdgcn_ubfe(sel, 8u * bi, 8u);  // one v_bfe_u32
         const unsigned f16 = 4u * qi + bi;
+        if (HI) bin += __builtin_amdgcn_ubfe(b[NQ], 16u * (unsigned)k + f16, 1u);
         // Quads past NQ do not exist.  Padding features of the last quad of
         // the matrix (bin 0 in every row) are accumulated like real ones into
         // slots nobody reads: cheaper than a per-update test.
@@ -85,22 +89,25 @@ __device__ __forceinline__ void AccumulateRow(unsigned long long *__restrict__ l
 // slab_entries entries (one or two words each): the histograms of the
 // launches (groups of quads) of a level one after the other, each in the
 // layout of HistLds for its own number of blocks; q_first is a multiple of 4.
-template <bool PAIR, int NQ>
+// HI: the image is one row of entries longer (bin 256), and so is the slab:
+// slab_entries counts that row too.
+template <bool PAIR, int NQ, int HI = 0>
 __device__ __forceinline__ void FlushSlab(const unsigned long long *__restrict__ lds,
                                           unsigned long long *__restrict__ slab, unsigned w,
                                           int slab_entries, int q_first) {
-  using L = HistLds<NQ>;
+  constexpr int words = (int)(HistLdsBytes(NQ, PAIR, HI != 0) / 8);
   constexpr int per = PAIR ? 2 : 1;
   __syncthreads();
   unsigned long long *out =
       slab + ((size_t)w * slab_entries + (size_t)(q_first / kBlockQuads) * kBlockEntries) * per;
-  for (int e = threadIdx.x; e < L::entries * per; e += kHistThreads) out[e] = lds[e];
+  for (int e = threadIdx.x; e < words; e += kHistThreads) out[e] = lds[e];
 }
 
 // Histogram of contiguous row ranges: one workgroup per work item, quads
 // [q0, q0+NQ).  LDS: NQ*1024 word0 entries, then (PAIR) as many word1 entries.
 // PAIR with h == nullptr: g holds packed logistic gradients (PackGrad).
-template <bool PAIR, int NQ>
+// HI: the rows carry a ninth-bit word in column q0 + NQ.
+template <bool PAIR, int NQ, int HI = 0>
 __global__ void __launch_bounds__(kHistThreads)
 k_hist(const uint32_t *__restrict__ bins, size_t stride, int q0, int F,
        const float *__restrict__ g, const float *__restrict__ h, const int *__restrict__ shifts,
@@ -110,7 +117,7 @@ k_hist(const uint32_t *__restrict__ bins, size_t stride, int q0, int F,
   const unsigned w = blockIdx.x;
   if (w >= *n_work) return;
   const WorkItem it = work[w];
-  constexpr int words = (int)(HistLdsBytes(NQ, PAIR) / 8);
+  constexpr int words = (int)(HistLdsBytes(NQ, PAIR, HI != 0) / 8);
   for (int i = threadIdx.x; i < words; i += kHistThreads) lds[i] = 0ull;
   __syncthreads();
   const int sg = shifts[0], sh = shifts[1];
@@ -119,9 +126,9 @@ k_hist(const uint32_t *__restrict__ bins, size_t stride, int q0, int F,
     const unsigned r0 = base + threadIdx.x, r1 = r0 + kHistThreads;
     const bool v0 = r0 < it.end, v1 = r1 < it.end;
     const unsigned a0 = v0 ? r0 : it.begin, a1 = v1 ? r1 : it.begin;
-    uint32_t b0[NQ], b1[NQ];
+    uint32_t b0[NQ + HI], b1[NQ + HI];
 #pragma unroll
-    for (int q = 0; q < NQ; ++q) {
+    for (int q = 0; q < NQ + HI; ++q) {
       b0[q] = __builtin_nontemporal_load(&bq[(size_t)q * stride + a0]);
       b1[q] = __builtin_nontemporal_load(&bq[(size_t)q * stride + a1]);
     }
@@ -136,10 +143,10 @@ k_hist(const uint32_t *__restrict__ bins, size_t stride, int q0, int F,
         UnpackGrad(g1, &g1, &h1);
       }
     }
-    if (v0) AccumulateRow<PAIR, NQ>(lds, b0, g0, h0, sg, sh, q0, F);
-    if (v1) AccumulateRow<PAIR, NQ>(lds, b1, g1, h1, sg, sh, q0, F);
+    if (v0) AccumulateRow<PAIR, NQ, HI>(lds, b0, g0, h0, sg, sh, q0, F);
+    if (v1) AccumulateRow<PAIR, NQ, HI>(lds, b1, g1, h1, sg, sh, q0, F);
   }
-  FlushSlab<PAIR, NQ>(lds, slab, w, slab_entries, q0);
+  FlushSlab<PAIR, NQ, HI>(lds, slab, w, slab_entries, q0);
 }
 
 // Histogram of contiguous row ranges with 16-bit bins: features [f0, f0 + nf)

@@ -10,11 +10,12 @@ namespace {
 
 // ---------------------------------------------------------------- partition
 __device__ __forceinline__ bool GoesRight(const uint32_t *__restrict__ bins, size_t stride,
-                                          const SplitRec &s, unsigned r, BinCode code = BinCode{2, 8}) {
+                                          const SplitRec &s, unsigned r, BinCode code = BinCode{2, 8},
+                                          int hi_word = -1) {
   // builder.h:107-123: bin >= q + 1 goes right
   if (s.fid < 0) return false;
-  const uint32_t word = bins[(size_t)code.Word(s.fid) * stride + r];
-  return (int)code.Bin(word, s.fid) > s.bin;
+  const SplitTest t = MakeSplitTest(s, code, hi_word);
+  return t.Right(bins[(size_t)t.word * stride + r]);
 }
 
 // The 128-row chunks of a work item are cut from its begin rounded down to a
@@ -29,11 +30,12 @@ __device__ __forceinline__ unsigned ChunkOrigin(const WorkItem &it) { return it.
 __global__ void __launch_bounds__(kHistThreads)
 k_part_count(const uint32_t *__restrict__ bins, size_t stride, const SplitRec *__restrict__ split,
              const WorkItem *__restrict__ work, const unsigned *__restrict__ n_work,
-             unsigned *__restrict__ wave_left, unsigned *__restrict__ item_left, BinCode code) {
+             unsigned *__restrict__ wave_left, unsigned *__restrict__ item_left, BinCode code, int hi_word) {
   const unsigned w = blockIdx.x;
   if (w >= *n_work) return;
   const WorkItem it = work[w];
   const SplitRec s = split[it.node];
+  const SplitTest test = MakeSplitTest(s, code, hi_word);
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   unsigned cnt = 0;
   // chunks are cut from the item's begin rounded down to 64 rows (ChunkOrigin)
@@ -42,7 +44,7 @@ k_part_count(const uint32_t *__restrict__ bins, size_t stride, const SplitRec *_
     for (unsigned base = cb + wave * kChunkRows; base < it.end; base += kChunkStep)
       cnt += lane == 0 ? min(base + kChunkRows, it.end) - max(base, it.begin) : 0u;
   } else {
-    const uint32_t *col = bins + (size_t)code.Word(s.fid) * stride;
+    const uint32_t *col = bins + (size_t)test.word * stride;
     // eight chunks (16 loads) in flight per wave: the pass is latency-bound
     constexpr int kBatch = 8;
     for (unsigned base = cb + wave * kChunkRows; base < it.end; base += kBatch * kChunkStep) {
@@ -56,8 +58,8 @@ k_part_count(const uint32_t *__restrict__ bins, size_t stride, const SplitRec *_
 #pragma unroll
       for (int k = 0; k < kBatch; ++k) {
         const unsigned r0 = base + k * kChunkStep + lane, r1 = r0 + 64;
-        if (r0 >= it.begin && r0 < it.end) cnt += ((int)code.Bin(v0[k], s.fid) > s.bin) ? 0u : 1u;
-        if (r1 < it.end) cnt += ((int)code.Bin(v1[k], s.fid) > s.bin) ? 0u : 1u;
+        if (r0 >= it.begin && r0 < it.end) cnt += test.Right(v0[k]) ? 0u : 1u;
+        if (r1 < it.end) cnt += test.Right(v1[k]) ? 0u : 1u;
       }
     }
   }
@@ -116,8 +118,10 @@ __device__ __forceinline__ void WaveOffsets(const WorkItem &it, const SplitRec &
 // (the fused pass does this instead of a separate counting launch).  The chunks
 // are read last one first: the lines the pass reads first are then the ones
 // most recently brought into the cache.  Wave-uniform result.
-__device__ __forceinline__ unsigned CountWaveLefts(const WorkItem &it, const SplitRec &s, const uint32_t *__restrict__ col,
-                                                  int wave, int lane) {
+// `col` is the column the decision reads: the split feature's quad, or (HI) test.word.
+template <int HI>
+__device__ __forceinline__ unsigned CountWaveLefts(const WorkItem &it, const SplitRec &s, const SplitTest &test,
+                                                  const uint32_t *__restrict__ col, int wave, int lane) {
   const unsigned cb = ChunkOrigin(it);
   const unsigned wb = cb + (unsigned)wave * kChunkRows, we = it.end;
   unsigned cnt = 0;
@@ -131,6 +135,11 @@ __device__ __forceinline__ unsigned CountWaveLefts(const WorkItem &it, const Spl
       return cnt;
     }
     const int fs = 8 * (s.fid & 3);
+    // (without ninth bits the byte test is spelled out: the fused pass has no register to spare)
+    auto right = [&](uint32_t v) {
+      if constexpr (HI != 0) return test.Right(v);
+      else return (int)((v >> fs) & 255u) > s.bin;
+    };
     constexpr int kBatch = 24;  // loads in flight per wave: all of a typical item at once
     for (int k0 = nk - 1; k0 >= 0; k0 -= kBatch) {
       uint32_t v0[kBatch], v1[kBatch];
@@ -145,8 +154,8 @@ __device__ __forceinline__ unsigned CountWaveLefts(const WorkItem &it, const Spl
       for (int j = 0; j < kBatch; ++j) {
         const int k = k0 - j;
         const unsigned r0 = wb + (unsigned)max(k, 0) * kChunkStep + lane, r1 = r0 + 64;
-        if (k >= 0 && r0 >= it.begin && r0 < we) cnt += ((int)((v0[j] >> fs) & 255u) > s.bin) ? 0u : 1u;
-        if (k >= 0 && r1 < we) cnt += ((int)((v1[j] >> fs) & 255u) > s.bin) ? 0u : 1u;
+        if (k >= 0 && r0 >= it.begin && r0 < we) cnt += right(v0[j]) ? 0u : 1u;
+        if (k >= 0 && r1 < we) cnt += right(v1[j]) ? 0u : 1u;
       }
     }
   }
@@ -165,11 +174,13 @@ __device__ __forceinline__ unsigned CountWaveLefts(const WorkItem &it, const Spl
 // all send a row to the same place; only the first one claims (cursor set),
 // the others read what it claimed (cursor null).
 // Called by the whole workgroup; s_tmp holds kItemWaves + 2 words.
-__device__ __forceinline__ void ClaimOffsets(const WorkItem &it, unsigned w, const SplitRec &s, unsigned start,
+template <int HI>
+__device__ __forceinline__ void ClaimOffsets(const WorkItem &it, unsigned w, const SplitRec &s, const SplitTest &test,
+                                             unsigned start,
                                              const uint32_t *__restrict__ col, unsigned *__restrict__ cursor,
                                              unsigned *__restrict__ item_base, int wave, int lane,
                                              unsigned *s_tmp, unsigned *lo, unsigned *ro) {
-  const unsigned mine = CountWaveLefts(it, s, col, wave, lane);
+  const unsigned mine = CountWaveLefts<HI>(it, s, test, col, wave, lane);
   if (lane == 0) s_tmp[wave] = mine;
   __syncthreads();
   if (threadIdx.x == 0) {
@@ -246,15 +257,17 @@ struct RowQueue {
     hbase = 0u;
   }
 };
-template <bool PAIR, bool PACK>
-constexpr bool HeadKept() { return !PAIR || PACK; }
+// (nor with a ninth-bit word: nine more registers per queue do not fit)
+template <bool PAIR, bool PACK, int HI = 0>
+constexpr bool HeadKept() { return (!PAIR || PACK) && HI == 0; }
 
 // Writes lanes [from, to) of Q to their destination and, for the child whose
 // histogram is built, adds them to the LDS histogram.
 // HIST: the kernel builds a histogram; GH: the gradients move with the rows;
 // PACK: Q.g holds packed logistic gradients (PackGrad), there is no h array.
-template <bool PAIR, int NQ, bool HIST = true, bool GH = true, bool PACK = false>
-__device__ __forceinline__ void EmitRows(unsigned long long *__restrict__ lds, const RowQueue<NQ> &Q,
+// NQ quads and, with HI, the ninth-bit word behind them (moved like a quad).
+template <bool PAIR, int NQ, bool HIST = true, bool GH = true, bool PACK = false, int HI = 0>
+__device__ __forceinline__ void EmitRows(unsigned long long *__restrict__ lds, const RowQueue<NQ + HI> &Q,
                                          unsigned from, unsigned to, bool built,
                                          uint32_t *__restrict__ bins_out, size_t stride,
                                          float *__restrict__ g_out, float *__restrict__ h_out, int lane,
@@ -263,7 +276,7 @@ __device__ __forceinline__ void EmitRows(unsigned long long *__restrict__ lds, c
     // streaming stores and loads: the pass touches every byte once
     const unsigned d = Q.base + (unsigned)lane;
 #pragma unroll
-    for (int q = 0; q < NQ; ++q) __builtin_nontemporal_store(Q.b[q], &bins_out[(size_t)q * stride + d]);
+    for (int q = 0; q < NQ + HI; ++q) __builtin_nontemporal_store(Q.b[q], &bins_out[(size_t)q * stride + d]);
     if (GH && g_out != nullptr) {  // a group pass after the first leaves the gradients alone
       __builtin_nontemporal_store(Q.g, &g_out[d]);
       if (PAIR && !PACK) __builtin_nontemporal_store(Q.h, &h_out[d]);
@@ -271,33 +284,33 @@ __device__ __forceinline__ void EmitRows(unsigned long long *__restrict__ lds, c
     if (HIST && built) {
       float gv = Q.g, hv = Q.h;
       if (PACK) UnpackGrad(Q.g, &gv, &hv);
-      AccumulateRow<PAIR, NQ>(lds, Q.b, gv, hv, sg, sh, 0, F);
+      AccumulateRow<PAIR, NQ, HI>(lds, Q.b, gv, hv, sg, sh, 0, F);
     }
   }
 }
 
 // The kept first batch of a wave (plain stores: it is about to be completed by
 // a neighbour), then what is left in the queue.
-template <bool PAIR, int NQ, bool HIST = true, bool GH = true, bool PACK = false>
-__device__ __forceinline__ void FlushQueue(unsigned long long *__restrict__ lds, const RowQueue<NQ> &Q, bool built,
+template <bool PAIR, int NQ, bool HIST = true, bool GH = true, bool PACK = false, int HI = 0>
+__device__ __forceinline__ void FlushQueue(unsigned long long *__restrict__ lds, const RowQueue<NQ + HI> &Q, bool built,
                                            uint32_t *__restrict__ bins_out, size_t stride,
                                            float *__restrict__ g_out, float *__restrict__ h_out, int lane,
                                            int sg, int sh, int F) {
-  if (HeadKept<PAIR, PACK>() && (unsigned)lane >= Q.hskip) {
+  if (HeadKept<PAIR, PACK, HI>() && (unsigned)lane >= Q.hskip) {
     const unsigned d = Q.hbase + (unsigned)lane;
 #pragma unroll
-    for (int q = 0; q < NQ; ++q) bins_out[(size_t)q * stride + d] = Q.hb[q];
+    for (int q = 0; q < NQ + HI; ++q) bins_out[(size_t)q * stride + d] = Q.hb[q];
     if (GH && g_out != nullptr) g_out[d] = Q.hg;
   }
-  EmitRows<PAIR, NQ, HIST, GH, PACK>(lds, Q, Q.skip, Q.n, built, bins_out, stride, g_out, h_out, lane, sg, sh, F);
+  EmitRows<PAIR, NQ, HIST, GH, PACK, HI>(lds, Q, Q.skip, Q.n, built, bins_out, stride, g_out, h_out, lane, sg, sh, F);
 }
 
 // Appends the rows of X flagged in xm (wave-uniform mask, one row per lane) to
 // Q in row order with one lane permute (ds_permute_b32) per register; a full queue is emitted
 // and the rest of X starts the next batch.
-template <bool PAIR, int NQ, bool HIST = true, bool GH = true, bool PACK = false>
-__device__ __forceinline__ void MergeRows(unsigned long long *__restrict__ lds, RowQueue<NQ> &Q,
-                                          const uint32_t (&xb)[NQ], float xg, float xh,
+template <bool PAIR, int NQ, bool HIST = true, bool GH = true, bool PACK = false, int HI = 0>
+__device__ __forceinline__ void MergeRows(unsigned long long *__restrict__ lds, RowQueue<NQ + HI> &Q,
+                                          const uint32_t (&xb)[NQ + HI], float xg, float xh,
                                           unsigned long long xm, bool built,
                                           uint32_t *__restrict__ bins_out, size_t stride,
                                           float *__restrict__ g_out, float *__restrict__ h_out, int lane,
@@ -308,42 +321,43 @@ __device__ __forceinline__ void MergeRows(unsigned long long *__restrict__ lds, 
   // the current batch, lanes < n hold what overflows into the next one
   const unsigned k = ((unsigned)lane - Q.n) & 63u;
   const int dst = PackedLane(xm, Q.n, lane);
-  uint32_t vb[NQ];
+  constexpr int NW = NQ + HI;
+  uint32_t vb[NW];
 #pragma unroll
-  for (int q = 0; q < NQ; ++q) vb[q] = SendTo(dst, xb[q]);
+  for (int q = 0; q < NW; ++q) vb[q] = SendTo(dst, xb[q]);
   const float vg = GH ? __uint_as_float(SendTo(dst, __float_as_uint(xg))) : 0.0f;
   const float vh = GH && PAIR && !PACK ? __uint_as_float(SendTo(dst, __float_as_uint(xh))) : 0.0f;
   if (Q.n + nx >= 64u) {  // wave-uniform: the batch is complete
     const bool fill = (unsigned)lane >= Q.n;
 #pragma unroll
-    for (int q = 0; q < NQ; ++q) Q.b[q] = fill ? vb[q] : Q.b[q];
+    for (int q = 0; q < NW; ++q) Q.b[q] = fill ? vb[q] : Q.b[q];
     Q.g = fill ? vg : Q.g;
     Q.h = fill ? vh : Q.h;
-    if (HeadKept<PAIR, PACK>() && Q.skip != 0u) {  // wave-uniform: the wave's first, partial batch
+    if (HeadKept<PAIR, PACK, HI>() && Q.skip != 0u) {  // wave-uniform: the wave's first, partial batch
 #pragma unroll
-      for (int q = 0; q < NQ; ++q) Q.hb[q] = Q.b[q];
+      for (int q = 0; q < NW; ++q) Q.hb[q] = Q.b[q];
       Q.hg = Q.g;
       Q.hskip = Q.skip;
       Q.hbase = Q.base;
       if (HIST && built && (unsigned)lane >= Q.skip) {
         float gv = Q.g, hv = 0.0f;
         if (PACK) UnpackGrad(Q.g, &gv, &hv);
-        AccumulateRow<PAIR, NQ>(lds, Q.b, gv, hv, sg, sh, 0, F);
+        AccumulateRow<PAIR, NQ, HI>(lds, Q.b, gv, hv, sg, sh, 0, F);
       }
     } else {
-      EmitRows<PAIR, NQ, HIST, GH, PACK>(lds, Q, Q.skip, 64u, built, bins_out, stride, g_out, h_out, lane, sg, sh, F);
+      EmitRows<PAIR, NQ, HIST, GH, PACK, HI>(lds, Q, Q.skip, 64u, built, bins_out, stride, g_out, h_out, lane, sg, sh, F);
     }
     Q.base += 64u;
     Q.skip = 0u;
 #pragma unroll
-    for (int q = 0; q < NQ; ++q) Q.b[q] = vb[q];
+    for (int q = 0; q < NW; ++q) Q.b[q] = vb[q];
     Q.g = vg;
     Q.h = vh;
     Q.n = Q.n + nx - 64u;
   } else {
     const bool fill = (unsigned)lane >= Q.n && k < nx;
 #pragma unroll
-    for (int q = 0; q < NQ; ++q) Q.b[q] = fill ? vb[q] : Q.b[q];
+    for (int q = 0; q < NW; ++q) Q.b[q] = fill ? vb[q] : Q.b[q];
     Q.g = fill ? vg : Q.g;
     Q.h = fill ? vh : Q.h;
     Q.n += nx;
@@ -368,7 +382,10 @@ __device__ __forceinline__ void MergeRows(unsigned long long *__restrict__ lds, 
 // earlier group of the same level).
 // PACK (with PAIR): g holds packed logistic gradients (PackGrad); h and h_out
 // are not touched.
-template <bool PAIR, int NQ, bool WRITE, bool GROUP = false, bool PACK = false>
+// HI (not with GROUP): column NQ of the rows is their ninth-bit word (SplitTest);
+// it moves with the quads, and ids of 256 are accumulated in a 257th row of
+// entries of the LDS histogram and of the slab.
+template <bool PAIR, int NQ, bool WRITE, bool GROUP = false, bool PACK = false, int HI = 0>
 __global__ void __launch_bounds__(kHistThreads)
 k_part_hist(const uint32_t *__restrict__ bins, uint32_t *__restrict__ bins_out, size_t stride, int F,
             const float *__restrict__ g, float *__restrict__ g_out, const float *__restrict__ h,
@@ -386,31 +403,40 @@ k_part_hist(const uint32_t *__restrict__ bins, uint32_t *__restrict__ bins_out, 
   const SplitRec s = split[it.node];
   const unsigned long long cl = s.left.c, cr = tot[it.node].c - cl;
   const bool build_right = cl > cr;  // ties -> left (hist_grad_sum.cu:288-290)
-  constexpr int words = (int)(HistLdsBytes(NQ, PAIR) / 8);
+  static_assert(!(HI && GROUP), "ninth bits: one group of quads only");
+  constexpr int NW = NQ + HI;  // words of a row
+  constexpr int words = (int)(HistLdsBytes(NQ, PAIR, HI != 0) / 8);
   for (int i = threadIdx.x; i < words; i += kHistThreads) lds[i] = 0ull;
   const int sg = shifts[0], sh = shifts[1];
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const unsigned wb = ChunkOrigin(it) + wave * kChunkRows, we = it.end;
-  const int fq = s.fid >> 2, fs = 8 * (s.fid & 3);
+  // which word of a row decides, and how (HI: the ninth-bit word for a split at bin 255; without
+  // ninth bits the byte test is spelled out, the pass has no register to spare)
+  const SplitTest test = MakeSplitTest(s, BinCode{2, 8}, HI ? NQ : -1);
+  const int fq = HI ? test.word : (s.fid < 0 ? 0 : s.fid >> 2), fs = 8 * (s.fid & 3);
+  auto goes_right = [&](uint32_t v) {
+    if constexpr (HI != 0) return test.Right(v);
+    else return s.fid >= 0 && (int)((v >> fs) & 255u) > s.bin;
+  };
   unsigned lo = 0, ro = 0;
   if (WRITE)
-    ClaimOffsets(it, w, s, seg_start[it.node], split_bins + (size_t)(s.fid < 0 ? 0 : fq) * stride, cursor, item_base,
-                 wave, lane, s_tmp, &lo, &ro);
+    ClaimOffsets<HI>(it, w, s, test, seg_start[it.node], split_bins + (size_t)fq * stride, cursor, item_base,
+                     wave, lane, s_tmp, &lo, &ro);
   __syncthreads();
   if constexpr (WRITE) {
     // QB: rows of the child whose histogram is built, QO: the other child
-    RowQueue<NQ> QB, QO;
+    RowQueue<NW> QB, QO;
     QB.Init(build_right ? ro : lo);
     QO.Init(build_right ? lo : ro);
     // Two register sets of 128 rows each: while one is processed the other is
     // in flight.  The loads are unconditional (addresses clamped to the last
     // row of the item) and the sets are never copied, so every wait in the loop
     // is for exactly the set that is needed next.
-    const uint32_t *split_col = split_bins + (size_t)(s.fid < 0 ? 0 : fq) * stride;
-    auto load = [&](RowSet<NQ> &R, unsigned base) {
+    const uint32_t *split_col = split_bins + (size_t)fq * stride;
+    auto load = [&](RowSet<NW> &R, unsigned base) {
       const unsigned a0 = min(base + lane, we - 1), a1 = min(base + 64 + lane, we - 1);
 #pragma unroll
-      for (int q = 0; q < NQ; ++q) {
+      for (int q = 0; q < NW; ++q) {
         R.b0[q] = __builtin_nontemporal_load(&bins[(size_t)q * stride + a0]);
         R.b1[q] = __builtin_nontemporal_load(&bins[(size_t)q * stride + a1]);
       }
@@ -423,7 +449,7 @@ k_part_hist(const uint32_t *__restrict__ bins, uint32_t *__restrict__ bins_out, 
       R.h0 = PAIR && !PACK ? __builtin_nontemporal_load(&h[a0]) : 0.0f;
       R.h1 = PAIR && !PACK ? __builtin_nontemporal_load(&h[a1]) : 0.0f;
     };
-    auto process = [&](const RowSet<NQ> &R, unsigned base) {
+    auto process = [&](const RowSet<NW> &R, unsigned base) {
       const unsigned r0 = base + lane, r1 = r0 + 64;
       const bool v0 = r0 >= it.begin && r0 < we, v1 = r1 < we;
       uint32_t s0 = 0, s1 = 0;
@@ -432,22 +458,22 @@ k_part_hist(const uint32_t *__restrict__ bins, uint32_t *__restrict__ bins_out, 
         s1 = R.s1;
       } else {
 #pragma unroll
-        for (int q = 0; q < NQ; ++q) {
+        for (int q = 0; q < NW; ++q) {
           s0 = q == fq ? R.b0[q] : s0;
           s1 = q == fq ? R.b1[q] : s1;
         }
       }
-      const bool right0 = v0 && s.fid >= 0 && (int)((s0 >> fs) & 255u) > s.bin;
-      const bool right1 = v1 && s.fid >= 0 && (int)((s1 >> fs) & 255u) > s.bin;
+      const bool right0 = v0 && goes_right(s0);
+      const bool right1 = v1 && goes_right(s1);
       const unsigned long long b0 = __ballot(v0 && right0 == build_right), o0 = __ballot(v0 && right0 != build_right);
       const unsigned long long b1 = __ballot(v1 && right1 == build_right), o1 = __ballot(v1 && right1 != build_right);
-      MergeRows<PAIR, NQ, true, true, PACK>(lds, QO, R.b0, R.g0, R.h0, o0, false, bins_out, stride, g_out, h_out, lane, sg, sh, F);
-      MergeRows<PAIR, NQ, true, true, PACK>(lds, QB, R.b0, R.g0, R.h0, b0, true, bins_out, stride, g_out, h_out, lane, sg, sh, F);
-      MergeRows<PAIR, NQ, true, true, PACK>(lds, QO, R.b1, R.g1, R.h1, o1, false, bins_out, stride, g_out, h_out, lane, sg, sh, F);
-      MergeRows<PAIR, NQ, true, true, PACK>(lds, QB, R.b1, R.g1, R.h1, b1, true, bins_out, stride, g_out, h_out, lane, sg, sh, F);
+      MergeRows<PAIR, NQ, true, true, PACK, HI>(lds, QO, R.b0, R.g0, R.h0, o0, false, bins_out, stride, g_out, h_out, lane, sg, sh, F);
+      MergeRows<PAIR, NQ, true, true, PACK, HI>(lds, QB, R.b0, R.g0, R.h0, b0, true, bins_out, stride, g_out, h_out, lane, sg, sh, F);
+      MergeRows<PAIR, NQ, true, true, PACK, HI>(lds, QO, R.b1, R.g1, R.h1, o1, false, bins_out, stride, g_out, h_out, lane, sg, sh, F);
+      MergeRows<PAIR, NQ, true, true, PACK, HI>(lds, QB, R.b1, R.g1, R.h1, b1, true, bins_out, stride, g_out, h_out, lane, sg, sh, F);
     };
     if (wb < we) {
-      RowSet<NQ> A, B;
+      RowSet<NW> A, B;
       load(A, wb);
       for (unsigned base = wb;; base += 2 * kChunkStep) {
         load(B, base + kChunkStep);
@@ -458,8 +484,8 @@ k_part_hist(const uint32_t *__restrict__ bins, uint32_t *__restrict__ bins_out, 
         if (base + 2 * kChunkStep >= we) break;
       }
     }
-    FlushQueue<PAIR, NQ, true, true, PACK>(lds, QO, false, bins_out, stride, g_out, h_out, lane, sg, sh, F);
-    FlushQueue<PAIR, NQ, true, true, PACK>(lds, QB, true, bins_out, stride, g_out, h_out, lane, sg, sh, F);
+    FlushQueue<PAIR, NQ, true, true, PACK, HI>(lds, QO, false, bins_out, stride, g_out, h_out, lane, sg, sh, F);
+    FlushQueue<PAIR, NQ, true, true, PACK, HI>(lds, QB, true, bins_out, stride, g_out, h_out, lane, sg, sh, F);
   } else {
     // Rows selected for the histogram are queued by row id (slot 64 * j + lane
     // of the queue is lane `lane` of q[j]; slots [0, np) are occupied) and read
@@ -469,12 +495,12 @@ k_part_hist(const uint32_t *__restrict__ bins, uint32_t *__restrict__ bins_out, 
     // and the wave never waits for its LDS atomics.
     unsigned q0 = it.begin, q1 = it.begin, q2 = it.begin;
     unsigned np = 0;
-    uint32_t gb[NQ];
+    uint32_t gb[NW];
     float gg = 0.0f, gh = 0.0f;
     auto gather = [&](bool valid) {  // requests the rows of queue slots [0, 64)
       const unsigned a = valid ? q0 : it.begin;
 #pragma unroll
-      for (int q = 0; q < NQ; ++q) gb[q] = bins[(size_t)q * stride + a];
+      for (int q = 0; q < NW; ++q) gb[q] = bins[(size_t)q * stride + a];
       gg = g[a];
       gh = PAIR && !PACK ? h[a] : 0.0f;
       q0 = q1;
@@ -501,14 +527,14 @@ k_part_hist(const uint32_t *__restrict__ bins, uint32_t *__restrict__ bins_out, 
         const bool valid = (unsigned)lane < take;
         gather(valid);
         if (PACK) UnpackGrad(gg, &gg, &gh);
-        if (valid) AccumulateRow<PAIR, NQ>(lds, gb, gg, gh, sg, sh, 0, F);
+        if (valid) AccumulateRow<PAIR, NQ, HI>(lds, gb, gg, gh, sg, sh, 0, F);
         np -= take;
       }
     };
     if (wb < we) {
       // last level: only the quad of the split feature decides; the selected
       // rows are read when they are accumulated
-      const uint32_t *col = split_bins + (size_t)(s.fid < 0 ? 0 : fq) * stride;
+      const uint32_t *col = split_bins + (size_t)fq * stride;
       auto step = [&](uint32_t s0, uint32_t s1, uint32_t &n0, uint32_t &n1, unsigned base) {
         const bool full = np >= 64u;  // wave-uniform
         if (full) {
@@ -519,13 +545,13 @@ k_part_hist(const uint32_t *__restrict__ bins, uint32_t *__restrict__ bins_out, 
         n1 = col[min(base + kChunkStep + 64 + lane, we - 1)];
         const unsigned r0 = base + lane, r1 = r0 + 64;
         const bool v0 = r0 >= it.begin && r0 < we, v1 = r1 < we;
-        const bool right0 = v0 && s.fid >= 0 && (int)((s0 >> fs) & 255u) > s.bin;
-        const bool right1 = v1 && s.fid >= 0 && (int)((s1 >> fs) & 255u) > s.bin;
+        const bool right0 = v0 && goes_right(s0);
+        const bool right1 = v1 && goes_right(s1);
         enqueue(base, __ballot(v0 && right0 == build_right));
         enqueue(base + 64, __ballot(v1 && right1 == build_right));
         if (full) {
           if (PACK) UnpackGrad(gg, &gg, &gh);
-          AccumulateRow<PAIR, NQ>(lds, gb, gg, gh, sg, sh, 0, F);
+          AccumulateRow<PAIR, NQ, HI>(lds, gb, gg, gh, sg, sh, 0, F);
         }
         drain(127u);
       };
@@ -539,7 +565,7 @@ k_part_hist(const uint32_t *__restrict__ bins, uint32_t *__restrict__ bins_out, 
     }
     drain(0u);
   }
-  FlushSlab<PAIR, NQ>(lds, slab, w, slab_entries, q0);
+  FlushSlab<PAIR, NQ, HI>(lds, slab, w, slab_entries, q0);
 }
 
 // Stable partition alone (matrices too wide for the fused pass, 16-bit bins):
@@ -553,7 +579,7 @@ k_part_rows(const uint32_t *__restrict__ bins, uint32_t *__restrict__ bins_out, 
             float *__restrict__ h_out, const SplitRec *__restrict__ split,
             const unsigned *__restrict__ seg_start, const WorkItem *__restrict__ work,
             const unsigned *__restrict__ n_work, const unsigned *__restrict__ wave_left,
-            const unsigned *__restrict__ item_left, BinCode code) {
+            const unsigned *__restrict__ item_left, BinCode code, int hi_word) {
   __shared__ unsigned s_tmp[kItemWaves + 1];
   const unsigned w = blockIdx.x;
   if (w >= *n_work) return;
@@ -567,7 +593,8 @@ k_part_rows(const uint32_t *__restrict__ bins, uint32_t *__restrict__ bins_out, 
   if (wb >= we) return;
   const uint32_t *group = bins + (size_t)q0 * stride;
   uint32_t *group_out = bins_out + (size_t)q0 * stride;
-  const uint32_t *split_col = bins + (size_t)(s.fid < 0 ? 0 : code.Word(s.fid)) * stride;
+  const SplitTest test = MakeSplitTest(s, code, hi_word);
+  const uint32_t *split_col = bins + (size_t)test.word * stride;
   RowQueue<NQ> QL, QR;
   QL.Init(lo);
   QR.Init(ro);
@@ -592,8 +619,8 @@ k_part_rows(const uint32_t *__restrict__ bins, uint32_t *__restrict__ bins_out, 
   auto process = [&](const Rows &R, unsigned base) {
     const unsigned r0 = base + lane, r1 = r0 + 64;
     const bool v0 = r0 >= it.begin && r0 < we, v1 = r1 < we;
-    const bool right0 = v0 && s.fid >= 0 && (int)code.Bin(R.s0, s.fid) > s.bin;
-    const bool right1 = v1 && s.fid >= 0 && (int)code.Bin(R.s1, s.fid) > s.bin;
+    const bool right0 = v0 && test.Right(R.s0);
+    const bool right1 = v1 && test.Right(R.s1);
     const unsigned long long lm0 = __ballot(v0 && !right0), rm0 = __ballot(right0);
     const unsigned long long lm1 = __ballot(v1 && !right1), rm1 = __ballot(right1);
     MergeRows<PAIR, NQ, false, GH>(nullptr, QL, R.r.b0, R.r.g0, R.r.h0, lm0, false, group_out, stride, g_out, h_out, lane, 0, 0, 0);
@@ -625,23 +652,30 @@ k_part_rows(const uint32_t *__restrict__ bins, uint32_t *__restrict__ bins_out, 
 //               (node_items == 0xffffffff marks a derived node);
 //   by_parent = 1: slabs belong to work items of the parent (fused pass); the
 //               built child is the smaller one, ties -> left.
-template <bool PAIR, int LANES>
+// hi_base > 0: the slabs hold one more row of entries, bin 256 of every feature
+// (matrices with a ninth-bit word); one more block of the grid (the last one)
+// reduces it into cell hi_base + f of the node's histogram, behind the 256-bin
+// histograms of the features.
+// CNT: type of the row counts of the node histograms.  The tree builder keeps
+// 64-bit counts: a streamed matrix may hold 2^32 rows and more, all of which can
+// sit in one cell (a constant feature, the bin of the missing values).
+template <bool PAIR, int LANES, typename CNT = unsigned>
 __global__ void __launch_bounds__(1024)
 k_hist_reduce(const unsigned long long *__restrict__ slab, int slab_entries, int nbin_total,
               const unsigned *__restrict__ node_first, const unsigned *__restrict__ node_items,
               int by_parent, const SplitRec *__restrict__ parent_split,
               const NodeSum *__restrict__ parent_tot, long long *__restrict__ hg,
-              long long *__restrict__ hh, unsigned *__restrict__ hc,
+              long long *__restrict__ hh, CNT *__restrict__ hc,
               const long long *__restrict__ pg, const long long *__restrict__ ph,
-              const unsigned *__restrict__ pc, int trick, int accumulate, int plain, int group_blocks,
-              int lds_slots = kSlots, int lay_blocks = 0) {
+              const CNT *__restrict__ pc, int trick, int accumulate, int plain, int group_blocks,
+              int lds_slots = kSlots, int lay_blocks = 0, int hi_base = 0) {
   // LANES threads share the slabs of one entry; a block covers 1024 / LANES
   // consecutive entries (with 4 lanes: 16 bins x 16 features, so the
   // feature-major output is written in runs of 16 bins)
   constexpr int kEntries = 1024 / LANES;
   __shared__ long long s_g[LANES][kEntries];
   __shared__ long long s_h[LANES][kEntries];
-  __shared__ unsigned s_c[LANES][kEntries];
+  __shared__ unsigned s_c[LANES][kEntries];  // (the slabs of one call hold fewer than 2^32 rows)
   const int nd = blockIdx.y;
   unsigned items, first;
   if (by_parent) {
@@ -660,20 +694,24 @@ k_hist_reduce(const unsigned long long *__restrict__ slab, int slab_entries, int
   // slab order; with fewer than 256 bins per feature in the slabs only the first lds_slots * 16
   // entries of every 16-feature block hold anything, and the grid covers only those
   const int per_block = plain ? 1 : (lds_slots * kBlockFeatures + kEntries - 1) / kEntries;
-  const int entry = plain ? (int)blockIdx.x * kEntries + e
-                          : ((int)blockIdx.x / per_block) * kBlockEntries + ((int)blockIdx.x % per_block) * kEntries + e;
+  // the block behind those of the 256 bins takes the row of bin 256: entry e is feature e
+  const bool hi_row = hi_base > 0 && (int)blockIdx.x == slab_entries / kBlockEntries * per_block;
+  const int entry = hi_row ? e
+                    : plain ? (int)blockIdx.x * kEntries + e
+                            : ((int)blockIdx.x / per_block) * kBlockEntries + ((int)blockIdx.x % per_block) * kEntries + e;
   // plain: the slabs are feature-major already (16-bit bins)
-  const int f = (entry / kBlockEntries) * kBlockFeatures + (entry & (kBlockFeatures - 1));
+  const int f = hi_row ? e : (entry / kBlockEntries) * kBlockFeatures + (entry & (kBlockFeatures - 1));
   const int bin = (entry / kBlockFeatures) & (kSlots - 1);
   // the last 16-feature block may have fewer than 16 features
   // lds_slots < 256: the slabs hold that many bins per feature only (the rest are empty)
-  const bool live = (plain ? entry < nbin_total : f * kSlots < nbin_total);
-  const bool stored = plain || bin < lds_slots;
+  const int hist_cells = hi_base > 0 ? hi_base : nbin_total;  // cells of the 256-bin histograms
+  const bool live = hi_row ? f < hist_cells / kSlots : (plain ? entry < nbin_total : f * kSlots < hist_cells);
+  const bool stored = plain || hi_row || bin < lds_slots;
   // lay_blocks > 0: the slabs are laid out for that many 16-feature blocks (a power of two of
   // bytes between bins), of which the matrix has slab_entries / 4096
   const size_t slab_words = plain ? (size_t)slab_entries * (PAIR ? 2 : 1)
                             : lay_blocks > 0 ? (size_t)lay_blocks * kBlockFeatures * (size_t)lds_slots * (PAIR ? 2 : 1)
-                                             : (size_t)slab_entries / kSlots * (size_t)lds_slots * (PAIR ? 2 : 1);
+                                             : (size_t)slab_entries / kSlots * (size_t)(lds_slots + (hi_base > 0 ? 1 : 0)) * (PAIR ? 2 : 1);
   long long ag = 0, ah = 0;
   unsigned ac = 0;
   if (live) {
@@ -681,7 +719,12 @@ k_hist_reduce(const unsigned long long *__restrict__ slab, int slab_entries, int
     // launches of the level (groups of group_blocks blocks, the last one maybe
     // shorter) one after the other, each in its LDS layout
     unsigned i0 = (unsigned)entry, i1 = (unsigned)(slab_entries + entry);
-    if (!plain) {
+    if (hi_row) {
+      // behind the image of the 256 bins, laid out like one more bin
+      i0 = (unsigned)slab_entries * (PAIR ? 2u : 1u) + (unsigned)(f / kBlockFeatures) * (PAIR ? 2u : 1u) * kBlockFeatures +
+           (unsigned)(f % kBlockFeatures);
+      i1 = i0 + kWord1;
+    } else if (!plain) {
       const int block = entry / kBlockEntries, group = block / group_blocks;
       const int blocks_here = min(group_blocks, slab_entries / kBlockEntries - group * group_blocks);
       const unsigned in_group = (unsigned)(entry - group * group_blocks * kBlockEntries);
@@ -709,24 +752,25 @@ k_hist_reduce(const unsigned long long *__restrict__ slab, int slab_entries, int
       ah += s_h[k][e];
       ac += s_c[k][e];
     }
-    const size_t cell = plain ? (size_t)entry : (size_t)f * kSlots + bin;
+    const size_t cell = hi_row ? (size_t)hi_base + f : plain ? (size_t)entry : (size_t)f * kSlots + bin;
     const size_t o = (size_t)nd * nbin_total + cell;
     // without hessians (count as hessian) the caller may pass no hh / ph arrays
     const bool with_h = PAIR || hh != nullptr;
+    CNT cnt = ac;
     if (accumulate) {  // streamed matrices: one call per row block
       ag += hg[o];
       if (with_h) ah += hh[o];
-      ac += hc[o];
+      cnt += hc[o];
     }
     hg[o] = ag;
     if (with_h) hh[o] = ah;
-    hc[o] = ac;
+    hc[o] = cnt;
     if (trick) {
       const size_t po = (size_t)(nd >> 1) * nbin_total + cell;
       const size_t so = (size_t)(nd ^ 1) * nbin_total + cell;
       hg[so] = pg[po] - ag;
       if (with_h) hh[so] = ph[po] - ah;
-      hc[so] = pc[po] - ac;
+      hc[so] = pc[po] - cnt;
     }
   }
 }
@@ -734,13 +778,18 @@ k_hist_reduce(const unsigned long long *__restrict__ slab, int slab_entries, int
 // Root totals = sum over the slots of feature 0 of the root histogram (every
 // row, NaN included, sits in exactly one slot).  Replaces the reduction over
 // the gradient array of garden.cu:432-435.  One wave.
+// hi_cell > 0: the cell of feature 0's bin 256 (matrices with a ninth-bit word).
 __global__ void __launch_bounds__(64)
 k_root_from_hist(const long long *__restrict__ hg, const long long *__restrict__ hh,
-                 NodeSum *__restrict__ tot, int slots) {
+                 NodeSum *__restrict__ tot, int slots, int hi_cell = 0) {
   long long a = 0, b = 0;
   for (int i = threadIdx.x; i < slots; i += 64) {
     a += hg[i];
     b += hh[i];
+  }
+  if (hi_cell > 0 && threadIdx.x == 0) {
+    a += hg[hi_cell];
+    b += hh[hi_cell];
   }
   a = WaveSumLL(a);
   b = WaveSumLL(b);

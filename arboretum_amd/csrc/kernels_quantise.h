@@ -10,9 +10,12 @@ namespace {
 // bin(x) = first l in [0,size] with x <= v[l], v[t] = thr[t] for t < size-1,
 // +INF above (src/core/cuda_helpers.h:207-222, src/io/io.cu:297-302); NaN
 // compares false everywhere and lands in bin `size`.
+// An id of 256 (a feature of 256 value bins with missing values) is stored as
+// byte 255 plus bit f0 + c of hi[r], the row's ninth-bit word (f0: the matrix
+// feature of column 0 of this launch); without `hi` no id may exceed 255.
 __global__ void k_bin_assign(const float *__restrict__ x, int ncols, const float *__restrict__ thr,
                              int thr_stride, const int *__restrict__ sizes,
-                             uint32_t *__restrict__ out, size_t n) {
+                             uint32_t *__restrict__ out, size_t n, uint32_t *__restrict__ hi, int f0) {
   __shared__ float s_thr[4][kSlots];
   __shared__ int s_size[4];
   for (int i = threadIdx.x; i < 4 * kSlots; i += blockDim.x) {
@@ -25,7 +28,7 @@ __global__ void k_bin_assign(const float *__restrict__ x, int ncols, const float
   __syncthreads();
   for (size_t r = (size_t)blockIdx.x * blockDim.x + threadIdx.x; r < n;
        r += (size_t)gridDim.x * blockDim.x) {
-    uint32_t packed = 0;
+    uint32_t packed = 0, over = 0;
 #pragma unroll
     for (int c = 0; c < 4; ++c) {
       if (c < ncols) {
@@ -38,10 +41,12 @@ __global__ void k_bin_assign(const float *__restrict__ x, int ncols, const float
           else
             l = mid + 1;
         }
-        packed |= l << (8 * c);
+        over |= (l > 255u ? 1u : 0u) << c;
+        packed |= min(l, 255u) << (8 * c);
       }
     }
     out[r] = packed;
+    if (hi != nullptr && over != 0u) hi[r] |= over << f0;  // launches of one matrix run one after the other
   }
 }
 

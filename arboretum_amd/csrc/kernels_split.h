@@ -20,7 +20,7 @@ struct Cand {
 // feature's slot 0 in the histogram arrays.  The result is valid in lane 0.
 template <bool PAIR, bool F64>
 __device__ __forceinline__ Cand ScanFeature(const long long *__restrict__ hg, const long long *__restrict__ hh,
-                                            const unsigned *__restrict__ hc, size_t first, int slots,
+                                            const unsigned long long *__restrict__ hc, size_t first, int slots,
                                             const NodeSum &t, const int *__restrict__ shifts,
                                             const GainParams &gp, int hist_size, int lane) {
   Cand best;
@@ -115,7 +115,7 @@ __device__ __forceinline__ Cand ScanFeature(const long long *__restrict__ hg, co
 template <bool PAIR, bool F64>
 __global__ void __launch_bounds__(64)
 k_split_scan(const long long *__restrict__ hg, const long long *__restrict__ hh,
-             const unsigned *__restrict__ hc, int nbin_total, int F, int slots,
+             const unsigned long long *__restrict__ hc, int nbin_total, int F, int slots,
              const NodeSum *__restrict__ tot, const int *__restrict__ shifts, GainParams gp,
              int hist_size, Cand *__restrict__ cand) {
   const int f = blockIdx.x, nd = blockIdx.y, lane = threadIdx.x;
@@ -255,7 +255,7 @@ k_select_plan(const Cand *__restrict__ cand, int F, int L, const NodeSum *__rest
 template <bool PAIR, bool F64>
 __global__ void __launch_bounds__(1024)
 k_scan_select(const long long *__restrict__ hg, const long long *__restrict__ hh,
-              const unsigned *__restrict__ hc, int nbin_total, int F, int slots, int L,
+              const unsigned long long *__restrict__ hc, int nbin_total, int F, int slots, int L,
               const NodeSum *__restrict__ tot, const int *__restrict__ shifts, GainParams gp, int hist_size,
               const unsigned *__restrict__ seg_start, NodeSum *__restrict__ tot_next,
               unsigned *__restrict__ seg_next, SplitRec *__restrict__ split, int *__restrict__ t_fid,

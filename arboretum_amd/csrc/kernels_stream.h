@@ -28,7 +28,7 @@ __device__ __forceinline__ bool NodeIsBuilt(const NodeSum *__restrict__ tot, uns
 __global__ void __launch_bounds__(256)
 k_stream_route(const uint32_t *__restrict__ bins, size_t bstride, unsigned rows, int level, int trick,
                const SplitRec *__restrict__ split, const NodeSum *__restrict__ tot,
-               unsigned *__restrict__ node_of, unsigned *__restrict__ blk_cnt) {
+               unsigned *__restrict__ node_of, unsigned *__restrict__ blk_cnt, int hi_word) {
   __shared__ unsigned s_cnt[kMaxPlanNodes];
   const int L = 1 << level;
   for (int i = threadIdx.x; i < L; i += blockDim.x) s_cnt[i] = 0;
@@ -42,7 +42,7 @@ k_stream_route(const uint32_t *__restrict__ bins, size_t bstride, unsigned rows,
     if (r < rows) {
       if (level > 0) {
         const unsigned parent = node_of[r];
-        nd = parent * 2u + (GoesRight(bins, bstride, split[parent], r) ? 1u : 0u);
+        nd = parent * 2u + (GoesRight(bins, bstride, split[parent], r, BinCode{2, 8}, hi_word) ? 1u : 0u);
       }
       node_of[r] = nd;
       built = NodeIsBuilt(tot, nd, level, trick);
@@ -141,9 +141,9 @@ k_stream_gather(const uint32_t *__restrict__ bins, size_t bstride, int Q, unsign
 }
 
 // sibling = parent - built child for every node that was not built directly
-__global__ void k_sibling(long long *__restrict__ hg, long long *__restrict__ hh, unsigned *__restrict__ hc,
+__global__ void k_sibling(long long *__restrict__ hg, long long *__restrict__ hh, unsigned long long *__restrict__ hc,
                           const long long *__restrict__ pg, const long long *__restrict__ ph,
-                          const unsigned *__restrict__ pc, const NodeSum *__restrict__ tot, int level,
+                          const unsigned long long *__restrict__ pc, const NodeSum *__restrict__ tot, int level,
                           int nbin_total) {
   const unsigned nd = blockIdx.y;
   if (NodeIsBuilt(tot, nd, level, 1)) return;

@@ -229,6 +229,8 @@ const char *ACreateFromQuantizedBlocks(const unsigned *const *blocks, int nblock
       throw std::runtime_error("bad arguments");
     if (block_rows % 64 != 0) throw std::runtime_error("block_rows must be a multiple of 64");
     if (block_rows >= (1ll << 31)) throw std::runtime_error("a block holds fewer than 2^31 rows");
+    // gradients are added as integers of up to 2^30 in magnitude: 2^33 of them can leave 64 bits
+    if (nrow >= (1ll << 33)) throw std::runtime_error("too many rows: a matrix holds fewer than 2^33 rows");
     if ((long long)(nblocks - 1) * block_rows >= nrow || (long long)nblocks * block_rows < nrow)
       throw std::runtime_error("nrow does not match nblocks blocks of block_rows rows (the last one may be shorter)");
     for (int b = 0; b < nblocks; ++b)

@@ -34,8 +34,10 @@ const char *ACreateFromQuantized(const unsigned char *bins, long long nrow, int 
  * beyond HBM and beyond the reference's `int nrow` (python-wrapper/
  * arboretum_wrapper.h:6-10 takes one fp32 array and an int row count).  The
  * rows live in `nblocks` caller-owned host blocks of `block_rows` rows (a
- * multiple of 64, below 2^31; the last block may hold fewer: nrow in all, any
- * 64-bit count); nothing is copied and nothing is freed with the matrix.
+ * multiple of 64, below 2^31; the last block may hold fewer: nrow in all, a
+ * 64-bit count below 2^33, the limit of the 64-bit integer gradient sums; row
+ * counts per histogram cell are 64-bit as well); nothing is copied and nothing
+ * is freed with the matrix.
  * Block layout (what the GPU streams as it is): 32-bit words
  * [Q][block_rows], Q = ceil(ncol / 4), word q * block_rows + r = bin ids of
  * features 4 q .. 4 q + 3 of the block's row r, one byte each, lowest byte
@@ -57,9 +59,14 @@ const char *AGetBins(VoidPointer data, unsigned char *out);
 const char *AGetThresholds(VoidPointer data, int fid, float *thr, int *size);
 /* Bin ids take 8 bits unless a feature has more than 256 of them (hist_size
  * above 255 on a column with that many distinct values): then 16 bits, as the
- * reference switches BIN_T by hist_size (src/core/garden.cu:506-569).
+ * reference switches BIN_T by hist_size (src/core/garden.cu:506-569).  The one
+ * id past a byte that hist_size 256 produces (256 value bins plus the bin of
+ * the missing values, src/core/cuda_helpers.h:207-222) is kept beside 8-bit ids
+ * as a ninth bit per feature when the matrix has at most 32 features: the
+ * layout then reports 8 bits and 257 slots.
  * AGetBinLayout: bits per bin id (8 or 16) and histogram slots per feature;
- * AGetBins16: the bins as row-major uint16 [nrow][ncol] (AGetBins is for 8). */
+ * AGetBins16: the bins as row-major uint16 [nrow][ncol] (AGetBins is for 8 bits
+ * and 256 slots). */
 const char *AGetBinLayout(VoidPointer data, int *bits, int *slots);
 const char *AGetBins16(VoidPointer data, unsigned short *out);
 

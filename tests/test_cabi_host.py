@@ -209,6 +209,19 @@ def test_no_alloc_histogram_size_limits_are_checked_before_the_gpu_is_touched():
                               parent_h=p, parent_c=p)
 
 
+def test_block_matrix_arguments_are_checked_on_the_host(arb):
+    # ACreateFromQuantizedBlocks: nothing is dereferenced when the matrix is created
+    p, br = 4096, 1 << 30
+    for blocks, block_rows, rows, msg in (([p], 100, 100, "multiple of 64"),
+                                          ([p], 1 << 31, 1 << 31, "fewer than 2\\^31"),
+                                          ([p, p], 128, 128, "does not match"),
+                                          ([p, 0], 128, 200, "null block"),
+                                          # integer gradient sums of 2^30 per row leave 64 bits from 2^33 rows on
+                                          ([p] * 8, br, 1 << 33, "fewer than 2\\^33 rows")):
+        with pytest.raises(arb.ArboretumError, match=msg):
+            arb.DMatrix.from_blocks(blocks, block_rows, rows, 4)
+
+
 def test_tree_arrays_follow_the_depth_of_a_loaded_tree(arb):
     # a model whose trees are deeper (and shallower) than the booster's configuration
     def tree(depth):

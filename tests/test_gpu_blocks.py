@@ -133,3 +133,56 @@ def test_four_billion_rows(arb, objective):
     leaves = big.leaves()
     assert np.array_equal(leaves[:block_rows], base.leaves())
     assert np.array_equal(leaves[-block_rows:], base.leaves())
+
+
+@pytest.mark.timeout(900)
+def test_one_histogram_cell_holds_more_than_2_32_rows(arb):
+    # 1032 descriptors of one 4 M-row block = 2^32 + 2^25 rows; feature 3 is 0 in all but 1000 rows
+    # of the block, so its cell (feature 3, bin 0) counts more than 2^32 rows, and with squared error
+    # the count is the hessian: a 32-bit count would change the gain of 'feature 3 = 0 against the
+    # rest', which the target makes the best split of the root.  Every integer sum is 1032 times the
+    # block's, so the splits must be those of the block alone and the leaf weights equal up to the
+    # rounding of G / H in another scale.
+    block_rows, reps, F = 1 << 22, 1032, 4
+    rows = block_rows * reps
+    assert (1 << 32) < rows < (1 << 33)
+    rng = np.random.default_rng(9)
+    bins = rng.integers(0, 255, size=(block_rows, F), dtype=np.uint8)
+    bins[:, 3] = 0
+    flagged = rng.choice(block_rows, size=1000, replace=False)
+    bins[flagged, 3] = 1
+    yb = (bins[:, 0].astype(np.float32) / 128 + 0.1 * rng.normal(size=block_rows)).astype(np.float32)
+    yb[flagged] += 400.0
+    blk = to_block(bins, block_rows)
+    # (one split level: below the root the gains of neighbouring bins lie within the rounding of
+    # another scale, and 1032 is not a power of two)
+    cfg = config(0, 1, min_child_weight=0.0, min_leaf_size=1)
+    cfg["tree"]["lambda"] = 0.0
+    base = arb.Garden(cfg, arb.DMatrix.from_blocks([blk.ptr], block_rows, block_rows, F, y=yb))
+    base.grow_tree()
+    tb = base.tree(0)
+    assert (tb["fid"][0], tb["quantized"][0]) == (3, 0)
+    print("block grown; building the targets of %d rows" % rows, flush=True)
+    y = np.tile(yb, reps)
+    data = arb.DMatrix.from_blocks([blk.ptr] * reps, block_rows, rows, F, y=y)
+    del y
+    big = arb.Garden(cfg, data)
+    big.set_inspect(True)
+    print("growing on %d rows" % rows, flush=True)
+    big.grow_tree()
+    big.synchronize()
+    print("tree grown", flush=True)
+    tg = big.tree(0)
+    for key in ("fid", "quantized", "threshold"):
+        assert np.array_equal(tb[key], tg[key]), key
+    assert np.allclose(tb["weights"], tg["weights"], rtol=1e-5, atol=0)
+    assert np.allclose(tb["gain"] * np.float32(reps), tg["gain"], rtol=1e-5, atol=0)
+    h = big.level_hist(0)
+    assert int(h[0, 3, 0, 2]) == reps * (block_rows - 1000) > (1 << 32)     # the cell's count, all 64 bits
+    assert int(h[0, 3, 1, 2]) == reps * 1000
+    assert int(h[0, 0, :, 2].sum()) == rows
+    # the rows of the two leaves, from the prediction update: all of the block's copies alike
+    yhat = big.train_yhat()
+    base_yhat = base.train_yhat()
+    for rep in (0, 517, reps - 1):
+        assert np.allclose(yhat[rep * block_rows:(rep + 1) * block_rows], base_yhat, rtol=1e-5, atol=1e-6), rep
