@@ -63,6 +63,7 @@ def _load_lib():
         "AGardenGetTimings": [c_void_p, c_void_p],
         "AGardenRowsScanned": [c_void_p, P(ctypes.c_ulonglong)],
         "AGardenRowsScannedByLevel": [c_void_p, c_void_p],
+        "AGardenStreamResidency": [c_void_p, P(ctypes.c_ulonglong), P(ctypes.c_ulonglong)],
         "AGardenSynchronize": [c_void_p],
         "AHistSum": [c_void_p] * 10 + [ctypes.c_ulonglong, ctypes.c_longlong, c_int, c_int, c_int, c_int, c_int,
                                        c_void_p],
@@ -320,6 +321,12 @@ class Garden(object):
         v = ctypes.c_ulonglong()
         _check(_LIB.AGardenRowsScanned(self.handle, ctypes.byref(v)))
         return v.value
+
+    def stream_residency(self):
+        """(row blocks kept in device memory, row blocks) of a streamed matrix; (0, 0) otherwise."""
+        a, b = ctypes.c_ulonglong(), ctypes.c_ulonglong()
+        _check(_LIB.AGardenStreamResidency(self.handle, ctypes.byref(a), ctypes.byref(b)))
+        return a.value, b.value
 
     def rows_scanned_by_level(self):
         """Rows accumulated into histograms so far, per tree level (root = 0)."""

@@ -123,6 +123,8 @@ class TreeBuilder {
   virtual BuilderTimings GetTimings() = 0;
   virtual unsigned long long RowsScanned() = 0;            // rows accumulated into histograms
   virtual void RowsScannedByLevel(unsigned long long *out) = 0;  // the same per tree level, 32 entries
+  // streamed matrix: row blocks kept in device memory and row blocks in all (0, 0: not streamed)
+  virtual void StreamResidency(unsigned long long *resident, unsigned long long *blocks) = 0;
   virtual void Synchronize() = 0;
 };
 

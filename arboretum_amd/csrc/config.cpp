@@ -52,6 +52,7 @@ Configuration Configuration::Parse(const char *text) {
     GetBool(*v, "upload_features", &cfg.internal.upload_features);
     GetNum(*v, "hist_size", &cfg.internal.hist_size);
     GetNum(*v, "stream_block_rows", &cfg.internal.stream_block_rows);
+    GetNum(*v, "stream_resident_bytes", &cfg.internal.stream_resident_bytes);
     GetBool(*v, "wide_rows_in_place", &cfg.internal.wide_rows_in_place);
   }
   return cfg;

@@ -51,6 +51,11 @@ struct InternalConfiguration {  // param.h:54-64
   // Extension (not a reference key): rows per pinned-host block when the bins
   // are streamed (upload_features = false); 0 = chosen from the matrix size.
   unsigned stream_block_rows = 0;
+  // Extension: bytes of a streamed matrix that stay in device memory (whole row blocks, spread
+  // evenly over the matrix; only the others are copied at every level).  Negative: as many as
+  // fit into 0.9 of the free device memory, the reference's rule for the columns it keeps
+  // (src/io/io.cu:496-507); 0: every block is streamed.
+  long long stream_resident_bytes = -1;
   // Extension: matrices of more than 32 features keep their rows in place and
   // re-order (row id, gradients) only; false selects the row-moving passes.
   bool wide_rows_in_place = true;

@@ -760,6 +760,7 @@ class HipTreeBuilder : public TreeBuilder {
     if (cfg.objective >= kSoftMaxOneVsAll) shifts[1] = 31;     // 0 <= h <= 1/2
     HIP_OK(hipMemcpyAsync(d_shifts_, shifts, sizeof(shifts), hipMemcpyHostToDevice, stream_));
     HIP_OK(hipStreamSynchronize(stream_));
+    if (streamed_) KeepBlocksResident(cfg.internal.stream_resident_bytes);
   }
 
   ~HipTreeBuilder() override {
@@ -775,6 +776,8 @@ class HipTreeBuilder : public TreeBuilder {
         if (p) (void)hipFree(p);
     }
     for (hipEvent_t e : event_pool_) (void)hipEventDestroy(e);
+    for (uint32_t *p : resident_)
+      if (p) (void)hipFree(p);
     if (streamed_) {
       (void)hipStreamSynchronize(copy_stream_);
       void *sp[] = {blk_[0], blk_[1], stage_.bins, stage_.g, stage_.h, d_node_of_, d_blk_cnt_, d_blk_seg_,
@@ -918,6 +921,10 @@ class HipTreeBuilder : public TreeBuilder {
   void RowsScannedByLevel(unsigned long long *out) override {  // kScanLevels entries
     HIP_OK(hipStreamSynchronize(stream_));
     HIP_OK(hipMemcpy(out, d_rows_scanned_, kScanLevels * sizeof(unsigned long long), hipMemcpyDeviceToHost));
+  }
+  void StreamResidency(unsigned long long *resident, unsigned long long *blocks) override {
+    *resident = resident_blocks_;
+    *blocks = resident_.size();
   }
   void Synchronize() override {
     HIP_OK(hipStreamSynchronize(stream_));
@@ -1271,6 +1278,45 @@ class HipTreeBuilder : public TreeBuilder {
   // Block `b` of the matrix into one of the two device buffers, on the copy
   // stream; returns the buffer index.  The compute stream waits for ev_ready_
   // before reading and records ev_free_ when it is done with the buffer.
+  // Blocks that stay in device memory (the reference keeps as many columns as fit into 0.9 of the
+  // free memory and streams the others, src/io/io.cu:496-507, src/core/garden.cu:296-347; here the
+  // unit is the row block).  budget < 0: that rule; else at most `budget` bytes.  The resident
+  // blocks are spread evenly over the matrix, so that the copies of the others run while the
+  // kernels work on resident ones.
+  void KeepBlocksResident(long long budget) {
+    const size_t nblocks = dm_->host_blocks.size();
+    const size_t block_bytes = (size_t)W_ * dm_->block_rows * sizeof(uint32_t);
+    size_t free_b = 0, total_b = 0;
+    HIP_OK(hipMemGetInfo(&free_b, &total_b));
+    size_t allowed = (size_t)(0.9 * (double)free_b);
+    if (budget >= 0) allowed = std::min(allowed, (size_t)budget);
+    const size_t keep = std::min(nblocks, allowed / block_bytes);
+    resident_.assign(nblocks, nullptr);
+    for (size_t b = 0; b < nblocks; ++b) {
+      if ((b + 1) * keep / nblocks == b * keep / nblocks) continue;  // keep of nblocks, evenly spread
+      resident_[b] = DevAlloc<uint32_t>((size_t)W_ * dm_->block_rows);
+      HIP_OK(hipMemcpy(resident_[b], dm_->host_blocks[b], block_bytes, hipMemcpyHostToDevice));
+      ++resident_blocks_;
+    }
+  }
+
+  // Block b in device memory for the kernels enqueued next: its resident copy, or one of the two
+  // copy buffers, filled on the copy stream (the compute stream then waits for the copy).
+  // Returns the buffer index, -1 for a resident block; DoneWithBlock after the last kernel that
+  // reads it.
+  const uint32_t *BlockOnDevice(size_t b, int *buf) {
+    if (resident_[b]) {
+      *buf = -1;
+      return resident_[b];
+    }
+    *buf = CopyBlockIn(b);
+    HIP_OK(hipStreamWaitEvent(stream_, ev_ready_[*buf], 0));
+    return blk_[*buf];
+  }
+  void DoneWithBlock(int buf) {
+    if (buf >= 0) HIP_OK(hipEventRecord(ev_free_[buf], stream_));
+  }
+
   int CopyBlockIn(size_t b) {
     const int buf = (int)(next_copy_++ & 1);
     if (buf_used_[buf]) HIP_OK(hipStreamWaitEvent(copy_stream_, ev_free_[buf], 0));
@@ -1455,22 +1501,37 @@ class HipTreeBuilder : public TreeBuilder {
       for (size_t b = 0; b < nblocks; ++b) {
         const size_t row0 = b * br;
         const unsigned rows = (unsigned)std::min(br, n_ - row0);
-        const int buf = CopyBlockIn(b);
-        HIP_OK(hipStreamWaitEvent(stream_, ev_ready_[buf], 0));
+        int buf = -1;
+        const uint32_t *blk = BlockOnDevice(b, &buf);
         Mark(kPartition);
-        hipLaunchKernelGGL(k_stream_route, dim3(GridFor(rows, 256, 1024)), dim3(256), 0, stream_, blk_[buf], br, rows,
+        hipLaunchKernelGGL(k_stream_route, dim3(GridFor(rows, 256, 1024)), dim3(256), 0, stream_, blk, br, rows,
                            level, trick ? 1 : 0, d_split_, d_tot_[state], d_node_of_ + row0, d_blk_cnt_, hi_word_);
         hipLaunchKernelGGL(k_stream_segments, dim3(1), dim3(1024), 0, stream_, d_blk_cnt_, L, d_blk_tot_, d_blk_seg_,
                            d_cursor_);
-        if (pair_)
-          hipLaunchKernelGGL(k_stream_gather<true>, dim3(GridFor(rows, 256, 2048)), dim3(256), 0, stream_, blk_[buf],
-                             br, W_, rows, orig.g + row0, orig.h + row0, d_node_of_ + row0, level, trick ? 1 : 0,
-                             d_tot_[state], d_cursor_, stage_.bins, br, stage_.g, stage_.h);
-        else
-          hipLaunchKernelGGL(k_stream_gather<false>, dim3(GridFor(rows, 256, 2048)), dim3(256), 0, stream_, blk_[buf],
-                             br, W_, rows, orig.g + row0, orig.h + row0, d_node_of_ + row0, level, trick ? 1 : 0,
-                             d_tot_[state], d_cursor_, stage_.bins, br, stage_.g, stage_.h);
-        HIP_OK(hipEventRecord(ev_free_[buf], stream_));
+        // the root's rows are the block as it is; deeper, the rows of the built nodes are gathered
+        // node by node into the staging buffer
+        const bool in_place = level == 0;
+        const uint32_t *hist_bins = in_place ? blk : stage_.bins;
+        const float *hist_g = in_place ? orig.g + row0 : stage_.g, *hist_h = in_place ? orig.h + row0 : stage_.h;
+        if (!in_place) {
+          const unsigned tiles = (rows + kGatherTile - 1) / kGatherTile;
+          const size_t lds = GatherLdsBytes(L);
+          static bool configured = false;
+          if (!configured) {
+            AllowLds(k_stream_gather<true>, kLdsBudget);
+            AllowLds(k_stream_gather<false>, kLdsBudget);
+            configured = true;
+          }
+          if (pair_)
+            hipLaunchKernelGGL(k_stream_gather<true>, dim3(tiles), dim3(1024), lds, stream_, blk, br, W_, rows,
+                               orig.g + row0, orig.h + row0, d_node_of_ + row0, level, trick ? 1 : 0, d_tot_[state],
+                               d_cursor_, stage_.bins, br, stage_.g, stage_.h);
+          else
+            hipLaunchKernelGGL(k_stream_gather<false>, dim3(tiles), dim3(1024), lds, stream_, blk, br, W_, rows,
+                               orig.g + row0, orig.h + row0, d_node_of_ + row0, level, trick ? 1 : 0, d_tot_[state],
+                               d_cursor_, stage_.bins, br, stage_.g, stage_.h);
+          DoneWithBlock(buf);
+        }
         // histograms of the gathered rows, added to the level's histograms
         const unsigned per_item = HistRowsPerItem(rows);
         const unsigned grid = (unsigned)std::min<size_t>(rows / per_item + 2 * L + 1, max_hist_items_);
@@ -1479,8 +1540,9 @@ class HipTreeBuilder : public TreeBuilder {
         Mark(level == 0 ? kHistRoot : kHistDeep);
         for (int q0 = 0; q0 < Q_; q0 += quads_per_group_) {
           const int nq = std::min(quads_per_group_, Q_ - q0);
-          HistLaunch(nq, grid, stage_.bins, br, q0, stage_.g, stage_.h);
+          HistLaunch(nq, grid, hist_bins, br, q0, hist_g, hist_h);
         }
+        if (in_place) DoneWithBlock(buf);
         Reduce(L, hb, false, state, false, b > 0);
       }
       if (level == 0)
@@ -1500,10 +1562,10 @@ class HipTreeBuilder : public TreeBuilder {
     for (size_t b = 0; b < nblocks; ++b) {
       const size_t row0 = b * br;
       const size_t rows = std::min(br, n_ - row0);
-      const int buf = CopyBlockIn(b);
-      HIP_OK(hipStreamWaitEvent(stream_, ev_ready_[buf], 0));
-      LaunchFinal(blk_[buf], br, row0, rows, label, next_grad);
-      HIP_OK(hipEventRecord(ev_free_[buf], stream_));
+      int buf = -1;
+      const uint32_t *blk = BlockOnDevice(b, &buf);
+      LaunchFinal(blk, br, row0, rows, label, next_grad);
+      DoneWithBlock(buf);
     }
     grad_ready_ = next_grad;
     EnqueueRecord();
@@ -1612,6 +1674,8 @@ class HipTreeBuilder : public TreeBuilder {
   bool pack_ = false;  // logistic gradients packed into one float per row, no h arrays
   hipStream_t copy_stream_ = nullptr;
   uint32_t *blk_[2] = {nullptr, nullptr};
+  std::vector<uint32_t *> resident_;  // per block: its copy in device memory, or null (copied in when needed)
+  size_t resident_blocks_ = 0;
   hipEvent_t ev_ready_[2] = {nullptr, nullptr}, ev_free_[2] = {nullptr, nullptr};
   bool buf_used_[2] = {false, false};
   size_t next_copy_ = 0;  // running block-copy counter (selects the buffer)

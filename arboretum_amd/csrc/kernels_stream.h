@@ -101,42 +101,111 @@ k_stream_segments(unsigned *__restrict__ blk_cnt, int L, NodeSum *__restrict__ b
 
 // Copies the rows of the built nodes into the staging buffer, node by node.
 // The order inside a node is whatever the atomics give; sums are integers.
+// A workgroup takes a tile of kGatherTile consecutive rows and sorts it by node
+// in LDS first (rank of every row among the tile's rows of its node, one LDS
+// atomic per distinct node of a wave; start of every node inside the tile by a
+// scan; one global cursor atomic per node present in the tile), so that the
+// tile's rows of one node go to consecutive places of the staging buffer and a
+// wave writes runs of them instead of 64 single words: with every lane of a
+// wave writing its own row to wherever its node's cursor stood, a store touched
+// 64 lines for 256 bytes (measured 1.8 ms per block of 4 M rows x 128
+// features, 0.3 TB/s).
+// grid ceil(rows / kGatherTile), 1024 threads; LDS: GatherLdsBytes(L).
+constexpr unsigned kGatherTile = 8192;
+constexpr int kGatherPerThread = kGatherTile / 1024;
+inline size_t GatherLdsBytes(int L) { return (size_t)2 * kGatherTile * 4 + (size_t)3 * L * 4 + 64; }
+
 template <bool PAIR>
-__global__ void __launch_bounds__(256)
+__global__ void __launch_bounds__(1024)
 k_stream_gather(const uint32_t *__restrict__ bins, size_t bstride, int Q, unsigned rows,
                 const float *__restrict__ g, const float *__restrict__ h,
                 const unsigned *__restrict__ node_of, int level, int trick,
                 const NodeSum *__restrict__ tot, unsigned *__restrict__ cursor,
                 uint32_t *__restrict__ st_bins, size_t sstride, float *__restrict__ st_g,
                 float *__restrict__ st_h) {
-  const int lane = threadIdx.x & 63;
-  const unsigned step = gridDim.x * blockDim.x;
-  for (unsigned r0 = blockIdx.x * blockDim.x; r0 < rows; r0 += step) {  // whole waves stay together
-    const unsigned r = r0 + threadIdx.x;
-    unsigned nd = 0;
+  extern __shared__ unsigned s_gather[];
+  const int L = 1 << level;
+  unsigned *s_src = s_gather;                 // row of the block at every sorted place of the tile
+  unsigned *s_dst = s_src + kGatherTile;      // its place in the staging buffer
+  unsigned *s_cnt = s_dst + kGatherTile;      // rows of the tile per node
+  unsigned *s_start = s_cnt + L;              // first sorted place of every node
+  unsigned *s_base = s_start + L;             // first staging place claimed for the tile's rows of every node
+  unsigned *s_misc = s_base + L;              // [0..15] wave sums, [16] carry
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const unsigned tile0 = blockIdx.x * kGatherTile;
+  for (int i = tid; i < L; i += 1024) s_cnt[i] = 0;
+  if (tid == 0) s_misc[16] = 0;
+  __syncthreads();
+  unsigned nd[kGatherPerThread], rk[kGatherPerThread];
+  unsigned built_mask = 0;
+#pragma unroll
+  for (int k = 0; k < kGatherPerThread; ++k) {
+    const unsigned r = tile0 + (unsigned)k * 1024u + (unsigned)tid;  // whole waves stay together
+    nd[k] = 0;
+    rk[k] = 0;
     bool built = false;
     if (r < rows) {
-      nd = node_of[r];
-      built = NodeIsBuilt(tot, nd, level, trick);
+      nd[k] = node_of[r];
+      built = NodeIsBuilt(tot, nd[k], level, trick);
     }
-    // one cursor atomic per distinct node of the wave
-    unsigned d = 0;
     unsigned long long todo = __ballot(built);
     while (todo) {
       const int leader = __ffsll((long long)todo) - 1;
-      const unsigned lead_nd = (unsigned)__shfl((int)nd, leader);
-      const unsigned long long same = __ballot(built && nd == lead_nd);
+      const unsigned lead_nd = (unsigned)__shfl((int)nd[k], leader);
+      const unsigned long long same = __ballot(built && nd[k] == lead_nd);
       unsigned base = 0;
-      if (lane == leader) base = atomicAdd(&cursor[lead_nd], (unsigned)__popcll(same));
+      if (lane == leader) base = atomicAdd(&s_cnt[lead_nd], (unsigned)__popcll(same));
       base = (unsigned)__shfl((int)base, leader);
-      if (built && nd == lead_nd) d = base + RankBelow(same);
+      if (built && nd[k] == lead_nd) rk[k] = base + RankBelow(same);
       todo &= ~same;
     }
-    if (built) {
-      for (int q = 0; q < Q; ++q) st_bins[(size_t)q * sstride + d] = bins[(size_t)q * bstride + r];
-      st_g[d] = g[r];
-      if (PAIR) st_h[d] = h[r];
+    built_mask |= built ? 1u << k : 0u;
+  }
+  __syncthreads();
+  // exclusive scan of the counts; claims in the staging buffer
+  for (int base = 0; base < L; base += 1024) {
+    const int i = base + tid;
+    const unsigned c = i < L ? s_cnt[i] : 0u;
+    unsigned incl = c;
+    for (int off = 1; off < 64; off <<= 1) {
+      const unsigned o = __shfl_up(incl, off);
+      if (lane >= off) incl += o;
     }
+    if (lane == 63) s_misc[wave] = incl;
+    __syncthreads();
+    unsigned off = s_misc[16];
+    for (int w = 0; w < wave; ++w) off += s_misc[w];
+    if (i < L) {
+      s_start[i] = off + incl - c;
+      s_base[i] = c ? atomicAdd(&cursor[i], c) : 0u;
+    }
+    __syncthreads();
+    if (tid == 1023) s_misc[16] = off + incl;
+    __syncthreads();
+  }
+  const unsigned total = s_misc[16];
+#pragma unroll
+  for (int k = 0; k < kGatherPerThread; ++k) {
+    if (built_mask >> k & 1u) {
+      const unsigned p = s_start[nd[k]] + rk[k];
+      s_src[p] = tile0 + (unsigned)k * 1024u + (unsigned)tid;
+      s_dst[p] = s_base[nd[k]] + rk[k];
+    }
+  }
+  __syncthreads();
+  for (unsigned p = tid; p < total; p += 1024) {
+    const unsigned r = s_src[p], d = s_dst[p];
+    int q = 0;
+    for (; q + 8 <= Q; q += 8) {  // eight loads in flight
+      uint32_t v[8];
+#pragma unroll
+      for (int j = 0; j < 8; ++j) v[j] = bins[(size_t)(q + j) * bstride + r];
+#pragma unroll
+      for (int j = 0; j < 8; ++j) __builtin_nontemporal_store(v[j], &st_bins[(size_t)(q + j) * sstride + d]);
+    }
+    for (; q < Q; ++q) __builtin_nontemporal_store(bins[(size_t)q * bstride + r], &st_bins[(size_t)q * sstride + d]);
+    st_g[d] = g[r];
+    if (PAIR) st_h[d] = h[r];
   }
 }
 

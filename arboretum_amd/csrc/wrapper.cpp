@@ -363,6 +363,9 @@ const char *AGardenRowsScanned(VoidPointer garden, unsigned long long *out) {
 const char *AGardenRowsScannedByLevel(VoidPointer garden, unsigned long long *out) {
   return Guard([&] { BuilderOf(garden)->RowsScannedByLevel(out); });
 }
+const char *AGardenStreamResidency(VoidPointer garden, unsigned long long *resident, unsigned long long *blocks) {
+  return Guard([&] { BuilderOf(garden)->StreamResidency(resident, blocks); });
+}
 const char *AGardenSynchronize(VoidPointer garden) {
   return Guard([&] { BuilderOf(garden)->Synchronize(); });
 }

@@ -34,7 +34,25 @@ sys.path.insert(0, ROOT)
 
 HBM_PEAK = 8.0e12  # bytes/s, MI355X
 TRAFFIC_PROFILE = os.path.join(ROOT, "profiles", "hbm_traffic_headline_10.5Mx28_depth8.txt")
-KERNEL_SOURCES = ["kernels_partition.h", "kernels_hist.h", "device_common.h"]
+# every source that shapes the dominant launch: the kernel, the LDS update order, the work plan
+# (item sizes, claims) and the host code that sizes and launches it
+KERNEL_SOURCES = ["kernels_partition.h", "kernels_hist.h", "device_common.h", "kernels_plan.h", "kernels_launch.h",
+                  "kernels_split.h", "device_builder.hip"]
+# The LDS co-limit of the kernels that accumulate histograms: an update of one wave (64 rows, one
+# feature each) is two ds_add_u64 wave instructions (sum of g with the count, sum of h); the LDS
+# atomic unit of a compute unit sustains one such instruction per 7.3 cycles at 2.4 GHz when no
+# two lanes of a 16-lane pass share a bank pair (measured: profiles/lds_counters_headline_*), and
+# a row costs 16 update slots per block of 16 features, idle slots included.
+CUS = 256
+LDS_CYCLES_PER_ATOMIC = 7.3
+CLOCK_HZ = 2.4e9
+
+
+def lds_floor_us(rows_accumulated, features, words=2):
+    """Time the LDS atomics alone need for `rows_accumulated` rows spread over all compute units."""
+    slots = 16 * ((features + 15) // 16)
+    instr_per_cu = rows_accumulated / 64.0 * slots * words / CUS
+    return instr_per_cu * LDS_CYCLES_PER_ATOMIC / CLOCK_HZ * 1e6
 
 
 def kernel_source_digest():
@@ -125,6 +143,11 @@ def stream_mode(args, arb):
     cfg = config(args.max_depth, 256)
     cfg["internals"]["upload_features"] = False
     cfg["internals"]["stream_block_rows"] = args.stream_block_rows
+    host_bytes = args.stream_rows * ((args.stream_features + 3) // 4 * 4)
+    # share of the matrix kept in device memory (whole blocks); negative: as many blocks as fit
+    # into 0.9 of the free device memory, the library's default and the reference's rule
+    if 0 <= args.stream_resident_frac < 1:
+        cfg["internals"]["stream_resident_bytes"] = int(args.stream_resident_frac * host_bytes) + 4096
     data = arb.DMatrix(bins, y=y, quantized=True)
     del bins
     model = arb.Garden(cfg, data)
@@ -139,14 +162,16 @@ def stream_mode(args, arb):
     model.synchronize()
     dt = time.perf_counter() - t0
     scanned = model.rows_scanned() - s0
-    passes = args.max_depth + 1    # one copy of every block per level + the leaf pass
-    host_bytes = args.stream_rows * ((args.stream_features + 3) // 4 * 4)
+    passes = args.max_depth + 1    # one pass over every block per level + the leaf pass
+    resident, blocks = model.stream_residency()
+    streamed_bytes = host_bytes * (blocks - resident) / max(blocks, 1)   # copied per pass
     print(json.dumps({
         "metric": "streamed (out-of-core) tree growing, bins in pinned host memory",
         "sec_per_tree": dt / args.steps, "steps": args.steps,
         "rows": args.stream_rows, "features": args.stream_features, "block_rows": args.stream_block_rows,
         "host_bin_bytes": host_bytes, "passes_per_tree": passes,
-        "h2d_GBps": host_bytes * passes * args.steps / dt / 1e9,
+        "blocks": blocks, "blocks_resident": resident, "bytes_copied_per_pass": streamed_bytes,
+        "h2d_GBps": streamed_bytes * passes * args.steps / dt / 1e9,
         "hist_updates_per_s": scanned * args.stream_features / dt,
         "phase_ms_per_tree": ({k: v / args.steps for k, v in model.timings().items() if k.endswith("_ms")}
                               if args.stream_timing else None)}))
@@ -278,7 +303,8 @@ def main():
                     help="skip the full-size runs of BASELINE configs[2] and configs[3] reported under other_configs")
     ap.add_argument("--nan-frac", type=float, default=0.0,
                     help="stress variant: this fraction of the feature values is replaced by NaN (all land in "
-                         "one bin per feature; needs --hist-size <= 255)")
+                         "one bin per feature; below 1/256 with --hist-size 256 every feature then has 257 bin "
+                         "ids, the last one kept as a ninth bit)")
     ap.add_argument("--mode", choices=["resident", "stream"], default="resident")
     ap.add_argument("--workload", choices=["headline", "config2", "config3"], default="headline",
                     help="config2 / config3: BASELINE configs[2] / configs[3] at full size, seconds per tree only")
@@ -286,6 +312,9 @@ def main():
     ap.add_argument("--stream-features", type=int, default=128)
     ap.add_argument("--stream-block-rows", type=int, default=1 << 22)
     ap.add_argument("--stream-timing", action="store_true")
+    ap.add_argument("--stream-resident-frac", type=float, default=0.0,
+                    help="--mode stream: share of the matrix kept in device memory, 0 .. 1 (0: every block is "
+                         "copied at every level, the out-of-core case); negative or 1: as much as fits")
     ap.add_argument("--copy-probe", type=int, default=0, metavar="MiB",
                     help="also run one device-to-device copy of this many MiB (a kernel of known traffic, "
                          "used to scale the FETCH_SIZE / WRITE_SIZE counters of a rocprofv3 --pmc run)")
@@ -376,22 +405,30 @@ def main():
     last_scanned = float(by_level[D - 1]) / args.steps if D >= 2 else 0.0
     last_bytes = last_scanned * row_bytes + R * PART_BYTES + (1 << max(D - 2, 0)) * F * 256 * CELL_BYTES
     last_s = tm["fused_last_ms"] * 1e-3 / max(tm["fused_last_launches"], 1)
-    other = {"k_part_hist<true,7,false,false,true> (last level, moves no rows)": {
+    def with_lds(entry, rows_accumulated):
+        # the co-limit these kernels are bound by: share of their duration that the LDS atomics
+        # of their rows take at the measured rate (1.0 = at the LDS floor)
+        floor = lds_floor_us(rows_accumulated, F)
+        entry["lds_floor_us"] = floor
+        entry["frac_of_lds_floor"] = floor / entry["avg_launch_us"] if entry["avg_launch_us"] > 0 else 0.0
+        return entry
+
+    other = {"k_part_hist<true,7,false,false,true> (last level, moves no rows)": with_lds({
         "frac_of_hbm": frac(last_bytes, last_s), "avg_launch_us": last_s * 1e6,
-        "updates_per_s": last_scanned * F / last_s if last_s > 0 else 0.0}}
+        "updates_per_s": last_scanned * F / last_s if last_s > 0 else 0.0}, last_scanned)}
     if tm["hist_root_launches"] > 0:
         root_s = tm["hist_root_ms"] * 1e-3 / tm["hist_root_launches"]
-        other["k_hist<true,7> (root level)"] = {
+        other["k_hist<true,7> (root level)"] = with_lds({
             "frac_of_hbm": frac(R * row_bytes + F * 256 * CELL_BYTES, root_s), "avg_launch_us": root_s * 1e6,
-            "updates_per_s": R * F / root_s if root_s > 0 else 0.0}
+            "updates_per_s": R * F / root_s if root_s > 0 else 0.0}, R)
     else:
         # the last pass of a tree (leaf of every row, prediction update R x 10, next gradients
         # R x 16) also builds the root histogram of the next tree (R x (F + 8))
         final_s = tm["leaf_ms"] * 1e-3 / phase_trees
-        other["k_final_hist<7> (prediction update + gradients + root histogram of the next tree)"] = {
+        other["k_final_hist<7> (prediction update + gradients + root histogram of the next tree)"] = with_lds({
             "frac_of_hbm": frac(R * (row_bytes + 10 + 16) + F * 256 * CELL_BYTES, final_s),
             "avg_launch_us": final_s * 1e6,
-            "updates_per_s": R * F / final_s if final_s > 0 else 0.0}
+            "updates_per_s": R * F / final_s if final_s > 0 else 0.0}, R)
     # whole tree by the same accounting: histogram build of every level, partition of every
     # split level, gradient pass, prediction update
     sec_per_tree = dt / args.steps
@@ -429,9 +466,19 @@ def main():
                      # the HBM peak that movement runs at
                      "moved_bytes_per_launch": moved_bytes,
                      "moved_frac": frac(moved_bytes, fused_s),
+                     # LDS co-limit of the same launch (the rows it accumulates: the smaller children)
+                     "lds_floor_us": lds_floor_us(scanned_per_launch, F),
+                     "frac_of_lds_floor": lds_floor_us(scanned_per_launch, F) / (fused_s * 1e6) if fused_s > 0 else 0.0,
                      "traffic_over_algorithmic": traffic / algo_bytes if traffic else None,
                      "traffic_source": "profiles/" + os.path.basename(TRAFFIC_PROFILE) if traffic else None},
         "other_kernels": other,
+        # north_star asks for the histogram build at >= 0.60 of the HBM peak: not met.  The kernels
+        # that only build histograms are bound by the LDS atomic unit (frac_of_lds_floor above),
+        # whose floor for one pass over all rows is lds_floor_us_all_rows; 0.60 of the HBM peak
+        # would be 79 us for the same pass.
+        "histogram_build": {"target_frac_of_hbm": 0.60, "met": False,
+                            "lds_floor_us_all_rows": lds_floor_us(R, F),
+                            "hbm_target_us_all_rows": R * row_bytes / (0.60 * HBM_PEAK) * 1e6},
         "tree_algorithmic_bytes": tree_bytes,
         "tree_algorithmic_floor_frac_of_hbm": (tree_bytes / sec_per_tree) / HBM_PEAK,
         "rows_scanned_per_tree_by_level": [float(v) / args.steps for v in by_level[:D]],

@@ -116,6 +116,14 @@ const char *AGardenRowsScanned(VoidPointer garden, unsigned long long *out);
 /* The same per tree level: out[32], out[l] = rows accumulated at level l (the
  * root is level 0; levels past 31 share the last entry). */
 const char *AGardenRowsScannedByLevel(VoidPointer garden, unsigned long long *out);
+/* Streamed matrix (internals.upload_features false): row blocks that stay in
+ * device memory and row blocks in all.  As many blocks as fit into 0.9 of the
+ * free device memory are kept, spread evenly over the matrix, and only the
+ * others are copied at every level: the reference's rule for the columns it
+ * keeps (src/io/io.cu:496-507; pipeline src/core/garden.cu:296-347), with row
+ * blocks as the unit.  internals.stream_resident_bytes (an extension key) caps
+ * the bytes kept; 0 streams every block.  0 of 0 for a resident matrix. */
+const char *AGardenStreamResidency(VoidPointer garden, unsigned long long *resident, unsigned long long *blocks);
 /* Waits for all device work of the booster. */
 const char *AGardenSynchronize(VoidPointer garden);
 

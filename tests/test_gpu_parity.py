@@ -249,14 +249,43 @@ def test_inspection_switched_on_between_rounds(arb, oracle):
 def test_streamed_bins_match_oracle(arb, oracle, objective, trick, block_rows):
     # upload_features = false: bins stay in pinned host blocks and are copied in
     # block by block at every level (reference: garden.cu:603-604,
-    # hist_tree_grower.cu:335-366); results must not depend on it
+    # hist_tree_grower.cu:335-366); results must not depend on it.
+    # stream_resident_bytes 0: no block is kept in device memory, every one is copied at every level
     X, y = make_data(9000, 11, objective, seed=13, nan_frac=0.02)
     cfg = {"objective": objective, "method": 1,
            "internals": {"hist_size": 63, "double_precision": True, "use_hist_subtraction_trick": trick,
-                         "upload_features": False, "stream_block_rows": block_rows},
+                         "upload_features": False, "stream_block_rows": block_rows, "stream_resident_bytes": 0},
            "tree": {"max_depth": 5, "eta": 0.3, "lambda": 1.0}}
-    assert_same_training(arb, oracle, X, y, cfg, rounds=3)
+    ob, g = assert_same_training(arb, oracle, X, y, cfg, rounds=3)
+    assert g.stream_residency() == (0, (9000 + max(block_rows, 64) - 1) // max(block_rows, 64))
     assert_same_training(arb, oracle, X, y, cfg, rounds=3, check_hist=False)
+
+
+@pytest.mark.parametrize("objective", [0, 1])
+@pytest.mark.parametrize("resident_blocks", [0, 1, 5, 9, -1])
+def test_partly_resident_equals_resident_equals_streamed(arb, oracle, objective, resident_blocks):
+    # The reference keeps as many columns on the device as fit into 0.9 of the free memory and
+    # streams the others (src/io/io.cu:496-507, src/core/garden.cu:296-347); here whole row blocks
+    # are kept.  Whatever share is resident, the trees are the checker's (and so those of the
+    # resident matrix and of the fully streamed one).
+    n, F, block_rows = 40000, 20, 4096           # 10 blocks of 5 quads x 4096 rows x 4 bytes
+    X, y = make_data(n, F, objective, seed=23, nan_frac=0.03)
+    block_bytes = 5 * block_rows * 4
+    cfg = {"objective": objective, "method": 1,
+           "internals": {"hist_size": 100, "double_precision": True, "upload_features": False,
+                         "stream_block_rows": block_rows,
+                         "stream_resident_bytes": -1 if resident_blocks < 0 else resident_blocks * block_bytes + 100},
+           "tree": {"max_depth": 6, "eta": 0.3, "lambda": 1.0}}
+    ob, g = assert_same_training(arb, oracle, X, y, cfg, rounds=3)
+    assert g.stream_residency() == (10 if resident_blocks < 0 else resident_blocks, 10)
+    ob, g = assert_same_training(arb, oracle, X, y, cfg, rounds=4, check_hist=False)
+    resident = dict(cfg, internals=dict(cfg["internals"], upload_features=True))
+    r = arb.Garden(resident, arb.DMatrix(X, y=y))
+    for t in range(4):
+        r.grow_tree()
+        for key in ("fid", "quantized", "threshold", "gain", "weights"):
+            assert np.array_equal(r.tree(t)[key], g.tree(t)[key], equal_nan=True), (t, key)
+    assert r.stream_residency() == (0, 0)
 
 
 def test_streamed_wide_matrix_and_prequantised(arb, oracle):
