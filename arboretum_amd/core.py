@@ -67,6 +67,7 @@ def _load_lib():
         "AGardenSynchronize": [c_void_p],
         "AHistSum": [c_void_p] * 10 + [ctypes.c_ulonglong, ctypes.c_longlong, c_int, c_int, c_int, c_int, c_int,
                                        c_void_p],
+        "AHistSumPlan": [ctypes.c_longlong, c_int, P(ctypes.c_uint), P(ctypes.c_uint)],
         "AHistSumNoAlloc": [c_void_p] * 10 + [ctypes.c_ulonglong, ctypes.c_longlong, c_int, c_int, c_int, c_int,
                                               c_int, c_void_p, c_void_p],
     }
@@ -104,6 +105,13 @@ def hist_sum(sum_g, sum_h, bin_count, grad, hess, node_size, bins, stride, nrow,
     _check(_LIB.AHistSum(sum_g, sum_h, bin_count, parent_g, parent_h, parent_c, grad, hess, node_size, bins,
                          int(stride), int(nrow), int(ncol), int(nodes), int(bool(use_trick)), int(shift_g),
                          int(shift_h), stream))
+
+
+def hist_sum_plan(nrow, nodes):
+    """(rows per work item, work items) of the plan hist_sum makes (AHistSumPlan; no GPU needed)."""
+    a, b = ctypes.c_uint(), ctypes.c_uint()
+    _check(_LIB.AHistSumPlan(int(nrow), int(nodes), ctypes.byref(a), ctypes.byref(b)))
+    return a.value, b.value
 
 
 def hist_sum_no_alloc(sum_g, sum_h, bin_count, grad, hess, node_size, bins, stride, nrow, ncol, nodes, shift_g,

@@ -524,11 +524,8 @@ struct FusedArgs {
 template <bool PAIR, int NQ, bool WRITE, bool GROUP, bool PACK, int HI>
 void LaunchFusedNQ(hipStream_t st, unsigned grid, const FusedArgs &a) {
   const size_t lds = HistLdsBytes(NQ, PAIR, HI != 0);
-  static bool configured = false;
-  if (!configured) {
-    AllowLds(k_part_hist<PAIR, NQ, WRITE, GROUP, PACK, HI>, lds);
-    configured = true;
-  }
+  static std::once_flag configured;
+  AllowLdsOnce(configured, k_part_hist<PAIR, NQ, WRITE, GROUP, PACK, HI>, lds);
   hipLaunchKernelGGL((k_part_hist<PAIR, NQ, WRITE, GROUP, PACK, HI>), dim3(grid), dim3(kHistThreads), lds, st,
                      a.bins + (size_t)a.q0 * a.stride, a.bins_out ? a.bins_out + (size_t)a.q0 * a.stride : nullptr,
                      a.stride, a.F, a.g, a.g_out, a.h, a.h_out, a.shifts, a.split, a.tot, a.seg_start, a.work,
@@ -668,7 +665,6 @@ class HipTreeBuilder : public TreeBuilder {
       }
     }
     if (indexed_) {
-      d_dec_ = DevAlloc<uint8_t>(n_);
       if (!dm_->rec) {  // records: whole 64-byte units (what memory answers a gather with), built once per matrix
         dm_->RS = (Q_ + 15) / 16 * 16;
         dm_->rec = DevAlloc<uint32_t>(n_ * (size_t)dm_->RS);
@@ -767,7 +763,7 @@ class HipTreeBuilder : public TreeBuilder {
     (void)hipStreamSynchronize(stream_);
     void *ptrs[] = {d_y_, d_labels_, d_yhat_, d_g_, d_h_, d_leaf_, d_split_, d_cand_, d_node_first_,
                     d_node_items_, d_hwork_, d_pwork_, d_nwork_, d_wave_left_, d_item_left_, d_slab_,
-                    d_shifts_, d_gmax_, d_rows_scanned_, d_tfid_, d_tbin_, d_tgain_, d_weights_, d_active_, d_overflow_, d_records_, d_cursor2_, d_dec_};
+                    d_shifts_, d_gmax_, d_rows_scanned_, d_tfid_, d_tbin_, d_tgain_, d_weights_, d_active_, d_overflow_, d_records_, d_cursor2_};
     for (void *p : ptrs)
       if (p) (void)hipFree(p);
     for (int b = 0; b < 2; ++b) {
@@ -987,18 +983,20 @@ class HipTreeBuilder : public TreeBuilder {
   // the counter of rows accumulated into histograms at `level` (levels past the last counter share it)
   unsigned long long *ScanCounter(int level) { return d_rows_scanned_ + std::min(level, kScanLevels - 1); }
   // count_level >= 0: the planned rows are histogram work of that tree level
+  // cursor: two claim cursors per node, cleared by the plan (passes that claim their output ranges)
   void Plan(int state, int L, int select, unsigned rows_per_item, WorkItem *work, unsigned *n_work,
-            int count_level, const SplitRec *split, unsigned max_items, unsigned balance_cus = 0) {
+            int count_level, const SplitRec *split, unsigned max_items, unsigned balance_cus = 0,
+            unsigned *cursor = nullptr) {
     PlanOn(d_tot_[state], d_seg_[state], L, select, rows_per_item, work, n_work, count_level, split, max_items,
-           balance_cus);
+           balance_cus, cursor);
   }
   void PlanOn(const NodeSum *tot, const unsigned *seg, int L, int select, unsigned rows_per_item, WorkItem *work,
               unsigned *n_work, int count_level, const SplitRec *split, unsigned max_items,
-              unsigned balance_cus = 0) {
+              unsigned balance_cus = 0, unsigned *cursor = nullptr) {
     hipLaunchKernelGGL(k_plan, dim3(1), dim3(1024), 0, stream_, tot, seg, L, select,
                        rows_per_item, work, n_work, d_node_first_, d_node_items_,
                        count_level >= 0 ? ScanCounter(count_level) : (unsigned long long *)nullptr, split, max_items,
-                       d_overflow_, balance_cus);
+                       d_overflow_, balance_cus, cursor);
   }
 
   // Histograms of contiguous node ranges in `cur` (level order), feature group by group.
@@ -1020,11 +1018,13 @@ class HipTreeBuilder : public TreeBuilder {
         const int nf = std::min(wide_group_, F_ - f0);
         const size_t lds = (size_t)nf * slots_ * 8 * (pair_ ? 2 : 1);
         if (pair_) {
-          AllowLds(k_hist_wide<true>, kLdsBudget);
+          static std::once_flag configured;
+          AllowLdsOnce(configured, k_hist_wide<true>, kLdsBudget);
           hipLaunchKernelGGL(k_hist_wide<true>, dim3(grid), dim3(kHistThreads), lds, stream_, cur.bins, stride_, f0, nf,
                              slots_, cur.g, cur.h, d_shifts_, d_hwork_, d_nwork_, d_slab_, slab_entries_);
         } else {
-          AllowLds(k_hist_wide<false>, kLdsBudget);
+          static std::once_flag configured;
+          AllowLdsOnce(configured, k_hist_wide<false>, kLdsBudget);
           hipLaunchKernelGGL(k_hist_wide<false>, dim3(grid), dim3(kHistThreads), lds, stream_, cur.bins, stride_, f0, nf,
                              slots_, cur.g, cur.h, d_shifts_, d_hwork_, d_nwork_, d_slab_, slab_entries_);
         }
@@ -1056,7 +1056,8 @@ class HipTreeBuilder : public TreeBuilder {
         const bool clamp = slots < kSlots;
 #define ARB_REC(P, POW2, CLAMP)                                                                                   \
   do {                                                                                                            \
-    AllowLds((k_hist_rec<P, POW2, CLAMP>), kLdsBudget);                                                           \
+    static std::once_flag configured;                                                                             \
+    AllowLdsOnce(configured, (k_hist_rec<P, POW2, CLAMP>), kLdsBudget);                                           \
     hipLaunchKernelGGL((k_hist_rec<P, POW2, CLAMP>), dim3(blocks), dim3(kHistThreads), lds, stream_, dm_->rec,    \
                        dm_->RS, cur.ids, Q_, slots, cur.g, cur.h, d_shifts_, d_hwork_, d_nwork_, d_slab_, pieces, \
                        total, ngroups, item_words, lay);                                                          \
@@ -1200,19 +1201,18 @@ class HipTreeBuilder : public TreeBuilder {
         } else {
           const unsigned grid = (unsigned)std::min<size_t>(n_ / kPartRows + 2 * PL + 1, max_part_items_);
           Mark(kPlan);
-          Plan(ps, PL, 0, kPartRows, d_pwork_, d_nwork_ + 1, -1, nullptr, grid);
+          Plan(ps, PL, 0, kPartRows, d_pwork_, d_nwork_ + 1, -1, nullptr, grid, 0, indexed_ ? d_cursor2_ : nullptr);
           Mark(kPartition);
           if (indexed_) {
-            hipLaunchKernelGGL(k_ix_decide, dim3(grid), dim3(kHistThreads), 0, stream_, dm_->bytes, dm_->stride8, src.ids,
-                               d_split_, d_pwork_, d_nwork_ + 1, d_dec_, d_wave_left_, d_item_left_);
+            // decisions, claims of the children's ranges and the move of (row id, g, h) in one launch
             if (pair_)
-              hipLaunchKernelGGL(k_ix_part<true>, dim3(grid), dim3(kHistThreads), 0, stream_, src.ids, dst.ids, src.g,
-                                 dst.g, src.h, dst.h, d_dec_, d_split_, d_seg_[ps], d_pwork_, d_nwork_ + 1,
-                                 d_wave_left_, d_item_left_);
+              hipLaunchKernelGGL(k_ix_part<true>, dim3(grid), dim3(kHistThreads), 0, stream_, dm_->bytes, dm_->stride8,
+                                 src.ids, dst.ids, src.g, dst.g, src.h, dst.h, d_split_, d_seg_[ps], d_pwork_,
+                                 d_nwork_ + 1, d_cursor2_, d_item_left_);
             else
-              hipLaunchKernelGGL(k_ix_part<false>, dim3(grid), dim3(kHistThreads), 0, stream_, src.ids, dst.ids, src.g,
-                                 dst.g, src.h, dst.h, d_dec_, d_split_, d_seg_[ps], d_pwork_, d_nwork_ + 1,
-                                 d_wave_left_, d_item_left_);
+              hipLaunchKernelGGL(k_ix_part<false>, dim3(grid), dim3(kHistThreads), 0, stream_, dm_->bytes, dm_->stride8,
+                                 src.ids, dst.ids, src.g, dst.g, src.h, dst.h, d_split_, d_seg_[ps], d_pwork_,
+                                 d_nwork_ + 1, d_cursor2_, d_item_left_);
           } else {
             hipLaunchKernelGGL(k_part_count, dim3(grid), dim3(kHistThreads), 0, stream_, src.bins, stride_, d_split_,
                                d_pwork_, d_nwork_ + 1, d_wave_left_, d_item_left_, code_, hi_word_);
@@ -1463,11 +1463,8 @@ class HipTreeBuilder : public TreeBuilder {
     float *yh = d_yhat_ + (size_t)label * n_;
 #define ARB_FH(N, H)                                                                                             \
   do {                                                                                                           \
-    static bool configured = false;                                                                              \
-    if (!configured) {                                                                                           \
-      AllowLds(k_final_hist<N, H>, kLdsBudget);                                                                  \
-      configured = true;                                                                                         \
-    }                                                                                                            \
+    static std::once_flag configured;                                                                            \
+    AllowLdsOnce(configured, k_final_hist<N, H>, kLdsBudget);                                                    \
     hipLaunchKernelGGL((k_final_hist<N, H>), dim3(grid), dim3(kHistThreads), lds, stream_, dm_->bins, stride_,  \
                        F_, d_tfid_, d_tbin_, D_, d_weights_, yh, d_y_, (unsigned *)nullptr, d_g_, d_h_,          \
                        d_shifts_, d_hwork_, d_nwork_, d_slab_, slab_stride_, d_tot_[0]);                         \
@@ -1516,12 +1513,11 @@ class HipTreeBuilder : public TreeBuilder {
         if (!in_place) {
           const unsigned tiles = (rows + kGatherTile - 1) / kGatherTile;
           const size_t lds = GatherLdsBytes(L);
-          static bool configured = false;
-          if (!configured) {
+          static std::once_flag configured;
+          std::call_once(configured, [] {
             AllowLds(k_stream_gather<true>, kLdsBudget);
             AllowLds(k_stream_gather<false>, kLdsBudget);
-            configured = true;
-          }
+          });
           if (pair_)
             hipLaunchKernelGGL(k_stream_gather<true>, dim3(tiles), dim3(1024), lds, stream_, blk, br, W_, rows,
                                orig.g + row0, orig.h + row0, d_node_of_ + row0, level, trick ? 1 : 0, d_tot_[state],
@@ -1632,7 +1628,6 @@ class HipTreeBuilder : public TreeBuilder {
   int rec_slots_ = kSlots;    // bins per feature of the one LDS histogram of that mode
   bool rec_one_launch_ = true;  // every feature fits one LDS histogram at rec_slots_ bins
   int rec_lay_blocks_ = 0;      // blocks that histogram is laid out for (a power of two), 0: as many as the matrix has
-  uint8_t *d_dec_ = nullptr;  // indexed mode: split decision of the row at each position
   bool wide_ = false;     // 16-bit bins: two features per word, slots_ histogram slots per feature
   bool hi_ = false;       // 8-bit bins plus a ninth-bit word per row (ids up to 256)
   int W_ = 0;             // words of a row: Q_, one more with ninth bits

@@ -1,6 +1,7 @@
 // Stand-alone histogram sums of node segments on the device (hist_sum.hip).
 #ifndef ARBORETUM_AMD_HIST_SUM_H_
 #define ARBORETUM_AMD_HIST_SUM_H_
+#include <cstddef>
 #include <cstdint>
 
 namespace arb {
@@ -30,6 +31,8 @@ struct HistSumArgs {
 
 // Allocates its work memory (plan, per-work-item slabs), runs and waits.
 void HistSum(const HistSumArgs &args);
+// Rows per work item HistSum plans for nrow rows in `nodes` segments (host arithmetic only).
+unsigned HistSumRowsPerItem(size_t nrow, int nodes);
 
 // The same without any allocation: plan and slabs live in a static device
 // array of 32 MB + 192 KB per GPU; enqueues on args.stream and returns without

@@ -235,13 +235,21 @@ void HistSumNoAlloc(const HistSumArgs &a, unsigned *status) {
           mem + kStaticHeadBytes);
 }
 
+// Rows per work item of AHistSum: about 512 items where items of at most kMaxHistRows rows
+// allow it, else items of that many rows (more than 512 x 64512 rows: more items, never
+// smaller ones).
+unsigned HistSumRowsPerItem(size_t nrow, int nodes) {
+  const unsigned want = 512u + 2u * (unsigned)nodes + 2u;
+  const unsigned fit = RowsPerItem(nrow, nodes, want);
+  return fit != 0 ? std::max(fit, (unsigned)kHistThreads) : kMaxHistRows;
+}
+
 void HistSum(const HistSumArgs &a) {
   Validate(a);
   const bool pair = a.hess != nullptr;
   const Shape sh = ShapeOf(a.ncol, pair);
   // one work item per CU and round where the rows allow it, as the tree builder plans a level
-  const unsigned want = 512u + 2u * (unsigned)a.nodes + 2u;
-  const unsigned per_item = std::max(RowsPerItem((size_t)a.nrow, a.nodes, want), (unsigned)kHistThreads);
+  const unsigned per_item = HistSumRowsPerItem((size_t)a.nrow, a.nodes);
   const unsigned max_items = (unsigned)((size_t)a.nrow / per_item + 2 * (size_t)a.nodes + 2);
   const size_t bytes = HistSumHeadBytes(a.nodes, max_items) + (size_t)max_items * sh.slab_words * 8 + 256;
   unsigned char *mem = nullptr;

@@ -54,121 +54,105 @@ k_to_byte_columns(const uint32_t *__restrict__ bins, size_t stride, int Q, uint8
   }
 }
 
-// Split decision of every row of the parents of a level, in node order:
-// dec[p] = 1 when the row at position p goes right (builder.h:107-123), and the
-// rows going left per (work item, wave) as k_part_count gives them.  ids: the
-// row at each position (null: position = row, the first level).  The split
-// feature's bin is read from the byte columns, not from the records: the ids of
-// a node ascend, so the reads of a node walk one column forwards, and the deeper
-// the level, the fewer rows of a node share a 64-byte fetch: with a byte per
-// row that happens two levels later than with a word per row.
-__global__ void __launch_bounds__(kHistThreads)
-k_ix_decide(const uint8_t *__restrict__ bytes, size_t stride8, const unsigned *__restrict__ ids,
-            const SplitRec *__restrict__ split, const WorkItem *__restrict__ work,
-            const unsigned *__restrict__ n_work, uint8_t *__restrict__ dec, unsigned *__restrict__ wave_left,
-            unsigned *__restrict__ item_left) {
-  const unsigned w = blockIdx.x;
-  if (w >= *n_work) return;
-  const WorkItem it = work[w];
-  const SplitRec s = split[it.node];
-  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-  const uint8_t *col = bytes + (size_t)(s.fid < 0 ? 0 : s.fid) * stride8;
-  unsigned cnt = 0;
-  const unsigned cb = ChunkOrigin(it);
-  constexpr int kBatch = 4;  // 8 ids, then 8 gathers in flight per lane
-  for (unsigned base = cb + wave * kChunkRows; base < it.end; base += kBatch * kChunkStep) {
-    unsigned id[2 * kBatch];
-    unsigned bin[2 * kBatch];
-#pragma unroll
-    for (int k = 0; k < 2 * kBatch; ++k) {
-      const unsigned r = base + (k >> 1) * kChunkStep + (k & 1) * 64 + lane;
-      const unsigned a = min(r, it.end - 1);
-      id[k] = ids ? ids[a] : a;
-    }
-#pragma unroll
-    for (int k = 0; k < 2 * kBatch; ++k) bin[k] = col[id[k]];
-#pragma unroll
-    for (int k = 0; k < 2 * kBatch; ++k) {
-      const unsigned r = base + (k >> 1) * kChunkStep + (k & 1) * 64 + lane;
-      if (r >= it.begin && r < it.end) {
-        const bool right = s.fid >= 0 && (int)bin[k] > s.bin;
-        dec[r] = right ? 1 : 0;
-        cnt += right ? 0u : 1u;
-      }
-    }
-  }
-  for (int off = 32; off > 0; off >>= 1) cnt += __shfl_down(cnt, off);
-  if (lane == 0) wave_left[(size_t)w * kItemWaves + wave] = cnt;
-  __shared__ unsigned s_cnt[kItemWaves];
-  if (lane == 0) s_cnt[wave] = cnt;
-  __syncthreads();
-  if (threadIdx.x == 0) {
-    unsigned t = 0;
-    for (int k = 0; k < kItemWaves; ++k) t += s_cnt[k];
-    item_left[w] = t;
-  }
-}
-
-// Stable partition of (row id, gradients) into the children order by the
-// decisions of k_ix_decide, through the register queues of the row passes.
-// ids null: position = row.
+// Partition of (row id, gradients) of the parents of a level into the children order, one launch
+// per level, rows in place.  ids: the row at each position (null: position = row, the first
+// level).  Each wave first decides its own rows: the split feature's bin of a row is read from
+// the byte columns, not from the records (the ids of a node ascend, so the reads of a node walk
+// one column forwards, and the deeper the level, the fewer rows of a node share a 64-byte fetch:
+// with a byte per row that happens two levels later than with a word per row).  A work item
+// holds at most kPartRows rows, eight 128-row chunks per wave, so the sixteen decisions of a
+// lane stay in the bits of one register; the workgroup then claims its share of the two
+// children's ranges on the node's cursors (ClaimWithCount: zero at launch, the planner clears
+// them) and the waves move their rows through the register queues of the row passes: the bin
+// is gathered once, and no decision array or counting launch exists.  Within a child the work
+// items lie in the order of their claims; no result depends on it (integer sums).
+constexpr int kIxChunks = (int)(kPartRows / kChunkStep);  // chunks of a wave in one work item
+static_assert(kIxChunks * 2 <= 32, "a lane's decisions of one work item must fit one register");
 template <bool PAIR>
 __global__ void __launch_bounds__(kHistThreads)
-k_ix_part(const unsigned *__restrict__ ids, unsigned *__restrict__ ids_out, const float *__restrict__ g,
-          float *__restrict__ g_out, const float *__restrict__ h, float *__restrict__ h_out,
-          const uint8_t *__restrict__ dec, const SplitRec *__restrict__ split,
+k_ix_part(const uint8_t *__restrict__ bytes, size_t stride8, const unsigned *__restrict__ ids,
+          unsigned *__restrict__ ids_out, const float *__restrict__ g, float *__restrict__ g_out,
+          const float *__restrict__ h, float *__restrict__ h_out, const SplitRec *__restrict__ split,
           const unsigned *__restrict__ seg_start, const WorkItem *__restrict__ work,
-          const unsigned *__restrict__ n_work, const unsigned *__restrict__ wave_left,
-          const unsigned *__restrict__ item_left) {
-  __shared__ unsigned s_tmp[kItemWaves + 1];
+          const unsigned *__restrict__ n_work, unsigned *__restrict__ cursor, unsigned *__restrict__ item_base) {
+  __shared__ unsigned s_tmp[kItemWaves + 2];
   const unsigned w = blockIdx.x;
   if (w >= *n_work) return;
   const WorkItem it = work[w];
   const SplitRec s = split[it.node];
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const unsigned wb = ChunkOrigin(it) + wave * kChunkRows, we = it.end;
+  const uint8_t *col = bytes + (size_t)(s.fid < 0 ? 0 : s.fid) * stride8;
+  // decisions of this lane's rows: bit 2 k + half = row (chunk k, half) goes right
+  unsigned right_bits = 0, lefts = 0;
+  if (s.fid >= 0) {
+    constexpr int kBatch = 4;  // 8 ids, then 8 gathers in flight per lane
+#pragma unroll
+    for (int k0 = 0; k0 < kIxChunks; k0 += kBatch) {
+      if (wb + (unsigned)k0 * kChunkStep < we) {  // wave-uniform
+        unsigned id[2 * kBatch], bin[2 * kBatch];
+#pragma unroll
+        for (int k = 0; k < 2 * kBatch; ++k) {
+          const unsigned r = wb + (unsigned)(k0 + (k >> 1)) * kChunkStep + (k & 1) * 64 + lane;
+          const unsigned a = min(r, we - 1);
+          id[k] = ids ? ids[a] : a;
+        }
+#pragma unroll
+        for (int k = 0; k < 2 * kBatch; ++k) bin[k] = col[id[k]];
+#pragma unroll
+        for (int k = 0; k < 2 * kBatch; ++k) {
+          const unsigned r = wb + (unsigned)(k0 + (k >> 1)) * kChunkStep + (k & 1) * 64 + lane;
+          const bool valid = r >= it.begin && r < we;
+          const bool right = (int)bin[k] > s.bin;  // builder.h:107-123
+          right_bits |= (valid && right ? 1u : 0u) << (2 * k0 + k);
+          lefts += valid && !right ? 1u : 0u;
+        }
+      }
+    }
+  } else {  // not split: every row stays left
+#pragma unroll
+    for (int k = 0; k < 2 * kIxChunks; ++k) {
+      const unsigned r = wb + (unsigned)(k >> 1) * kChunkStep + (k & 1) * 64 + lane;
+      lefts += r >= it.begin && r < we ? 1u : 0u;
+    }
+  }
+  for (int off = 32; off > 0; off >>= 1) lefts += __shfl_xor(lefts, off);
   unsigned lo, ro;
-  const unsigned before = LeftsBefore(it, w, wave, wave_left, item_left, s_tmp);
-  WaveOffsets(it, s, seg_start[it.node], before, wave, &lo, &ro);
+  ClaimWithCount(it, w, s, seg_start[it.node], lefts, cursor, item_base, wave, lane, s_tmp, &lo, &ro);
   if (wb >= we) return;
   RowQueue<1> QL, QR;
   QL.Init(lo);
   QR.Init(ro);
-  struct Rows {
-    RowSet<1> r;
-    uint32_t d0, d1;
-  };
-  auto load = [&](Rows &R, unsigned base) {
+  auto load = [&](RowSet<1> &R, unsigned base) {
     const unsigned a0 = min(base + lane, we - 1), a1 = min(base + 64 + lane, we - 1);
-    R.r.b0[0] = ids ? ids[a0] : a0;
-    R.r.b1[0] = ids ? ids[a1] : a1;
-    R.d0 = dec[a0];
-    R.d1 = dec[a1];
-    R.r.g0 = g[a0];
-    R.r.g1 = g[a1];
-    R.r.h0 = PAIR ? h[a0] : 0.0f;
-    R.r.h1 = PAIR ? h[a1] : 0.0f;
+    R.b0[0] = ids ? ids[a0] : a0;
+    R.b1[0] = ids ? ids[a1] : a1;
+    R.g0 = g[a0];
+    R.g1 = g[a1];
+    R.h0 = PAIR ? h[a0] : 0.0f;
+    R.h1 = PAIR ? h[a1] : 0.0f;
   };
-  auto process = [&](const Rows &R, unsigned base) {
+  auto process = [&](const RowSet<1> &R, unsigned base, unsigned chunk) {
     const unsigned r0 = base + lane, r1 = r0 + 64;
     const bool v0 = r0 >= it.begin && r0 < we, v1 = r1 < we;
-    const bool right0 = v0 && R.d0 != 0, right1 = v1 && R.d1 != 0;
-    const unsigned long long lm0 = __ballot(v0 && !right0), rm0 = __ballot(right0);
-    const unsigned long long lm1 = __ballot(v1 && !right1), rm1 = __ballot(right1);
+    const bool right0 = (right_bits >> (2u * chunk)) & 1u, right1 = (right_bits >> (2u * chunk + 1u)) & 1u;
+    const unsigned long long lm0 = __ballot(v0 && !right0), rm0 = __ballot(v0 && right0);
+    const unsigned long long lm1 = __ballot(v1 && !right1), rm1 = __ballot(v1 && right1);
     uint32_t *out = ids_out;
-    MergeRows<PAIR, 1, false, true>(nullptr, QL, R.r.b0, R.r.g0, R.r.h0, lm0, false, out, 0, g_out, h_out, lane, 0, 0, 0);
-    MergeRows<PAIR, 1, false, true>(nullptr, QR, R.r.b0, R.r.g0, R.r.h0, rm0, false, out, 0, g_out, h_out, lane, 0, 0, 0);
-    MergeRows<PAIR, 1, false, true>(nullptr, QL, R.r.b1, R.r.g1, R.r.h1, lm1, false, out, 0, g_out, h_out, lane, 0, 0, 0);
-    MergeRows<PAIR, 1, false, true>(nullptr, QR, R.r.b1, R.r.g1, R.r.h1, rm1, false, out, 0, g_out, h_out, lane, 0, 0, 0);
+    MergeRows<PAIR, 1, false, true>(nullptr, QL, R.b0, R.g0, R.h0, lm0, false, out, 0, g_out, h_out, lane, 0, 0, 0);
+    MergeRows<PAIR, 1, false, true>(nullptr, QR, R.b0, R.g0, R.h0, rm0, false, out, 0, g_out, h_out, lane, 0, 0, 0);
+    MergeRows<PAIR, 1, false, true>(nullptr, QL, R.b1, R.g1, R.h1, lm1, false, out, 0, g_out, h_out, lane, 0, 0, 0);
+    MergeRows<PAIR, 1, false, true>(nullptr, QR, R.b1, R.g1, R.h1, rm1, false, out, 0, g_out, h_out, lane, 0, 0, 0);
   };
-  Rows A, B;
+  RowSet<1> A, B;
   load(A, wb);
-  for (unsigned base = wb;; base += 2 * kChunkStep) {
+  unsigned chunk = 0;
+  for (unsigned base = wb;; base += 2 * kChunkStep, chunk += 2) {
     load(B, base + kChunkStep);
-    process(A, base);
+    process(A, base, chunk);
     if (base + kChunkStep >= we) break;  // wave-uniform
     load(A, base + 2 * kChunkStep);
-    process(B, base + kChunkStep);
+    process(B, base + kChunkStep, chunk + 1);
     if (base + 2 * kChunkStep >= we) break;
   }
   FlushQueue<PAIR, 1, false, true>(nullptr, QL, false, ids_out, 0, g_out, h_out, lane, 0, 0, 0);

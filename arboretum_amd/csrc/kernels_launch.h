@@ -2,6 +2,7 @@
 // stand-alone histogram kernel.
 #ifndef ARBORETUM_AMD_KERNELS_LAUNCH_H_
 #define ARBORETUM_AMD_KERNELS_LAUNCH_H_
+#include <mutex>
 #include <stdexcept>
 
 #include "device_common.h"
@@ -10,12 +11,16 @@
 namespace arb {
 namespace {
 
-// Raises the dynamic LDS limit of a kernel once (needed above 64 KB).
+// Raises the dynamic LDS limit of a kernel (needed above 64 KB).
 template <typename K>
 void AllowLds(K kernel, size_t bytes) {
-  static size_t allowed = 0;  // one instance per kernel type/pointer value below
-  (void)allowed;
   HIP_OK(hipFuncSetAttribute((const void *)kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)bytes));
+}
+// The same once per process and call site: `flag` is a static of the caller, one per kernel
+// instance.  Safe from several host threads; a later launch pays nothing.
+template <typename K>
+void AllowLdsOnce(std::once_flag &flag, K kernel, size_t bytes) {
+  std::call_once(flag, [&] { AllowLds(kernel, bytes); });
 }
 
 template <bool PAIR, int NQ, int HI = 0>
@@ -23,11 +28,8 @@ void LaunchHistNQ(hipStream_t st, unsigned grid, const uint32_t *bins, size_t st
                   const float *g, const float *h, const int *shifts, const WorkItem *work,
                   const unsigned *n_work, unsigned long long *slab, int slab_entries) {
   const size_t lds = HistLdsBytes(NQ, PAIR, HI != 0);
-  static bool configured = false;
-  if (!configured) {
-    AllowLds(k_hist<PAIR, NQ, HI>, lds);
-    configured = true;
-  }
+  static std::once_flag configured;
+  AllowLdsOnce(configured, k_hist<PAIR, NQ, HI>, lds);
   hipLaunchKernelGGL((k_hist<PAIR, NQ, HI>), dim3(grid), dim3(kHistThreads), lds, st, bins, stride, q0, F, g, h,
                      shifts, work, n_work, slab, slab_entries);
 }

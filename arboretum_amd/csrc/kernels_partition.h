@@ -174,13 +174,11 @@ __device__ __forceinline__ unsigned CountWaveLefts(const WorkItem &it, const Spl
 // all send a row to the same place; only the first one claims (cursor set),
 // the others read what it claimed (cursor null).
 // Called by the whole workgroup; s_tmp holds kItemWaves + 2 words.
-template <int HI>
-__device__ __forceinline__ void ClaimOffsets(const WorkItem &it, unsigned w, const SplitRec &s, const SplitTest &test,
-                                             unsigned start,
-                                             const uint32_t *__restrict__ col, unsigned *__restrict__ cursor,
-                                             unsigned *__restrict__ item_base, int wave, int lane,
-                                             unsigned *s_tmp, unsigned *lo, unsigned *ro) {
-  const unsigned mine = CountWaveLefts<HI>(it, s, test, col, wave, lane);
+// ClaimWithCount: the same from `mine`, the wave's own count of its rows going left.
+__device__ __forceinline__ void ClaimWithCount(const WorkItem &it, unsigned w, const SplitRec &s, unsigned start,
+                                               unsigned mine, unsigned *__restrict__ cursor,
+                                               unsigned *__restrict__ item_base, int wave, int lane,
+                                               unsigned *s_tmp, unsigned *lo, unsigned *ro) {
   if (lane == 0) s_tmp[wave] = mine;
   __syncthreads();
   if (threadIdx.x == 0) {
@@ -201,6 +199,15 @@ __device__ __forceinline__ void ClaimOffsets(const WorkItem &it, unsigned w, con
   const unsigned rows_before = RowsOfEarlierWaves(it, wave);
   *lo = start + s_tmp[kItemWaves] + lefts_before;
   *ro = start + (unsigned)s.left.c + s_tmp[kItemWaves + 1] + rows_before - lefts_before;
+}
+template <int HI>
+__device__ __forceinline__ void ClaimOffsets(const WorkItem &it, unsigned w, const SplitRec &s, const SplitTest &test,
+                                             unsigned start,
+                                             const uint32_t *__restrict__ col, unsigned *__restrict__ cursor,
+                                             unsigned *__restrict__ item_base, int wave, int lane,
+                                             unsigned *s_tmp, unsigned *lo, unsigned *ro) {
+  ClaimWithCount(it, w, s, start, CountWaveLefts<HI>(it, s, test, col, wave, lane), cursor, item_base, wave, lane,
+                 s_tmp, lo, ro);
 }
 
 // Destination lane of this lane's row when the rows flagged in the

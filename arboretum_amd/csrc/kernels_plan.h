@@ -188,9 +188,10 @@ k_plan(const NodeSum *__restrict__ tot, const unsigned *__restrict__ seg_start, 
        unsigned rows_per_item, WorkItem *__restrict__ work, unsigned *__restrict__ n_work,
        unsigned *__restrict__ node_first, unsigned *__restrict__ node_items,
        unsigned long long *__restrict__ rows_scanned, const SplitRec *__restrict__ split,
-       unsigned max_items, unsigned *__restrict__ overflow, unsigned balance_cus) {
+       unsigned max_items, unsigned *__restrict__ overflow, unsigned balance_cus,
+       unsigned *__restrict__ cursor = nullptr) {
   PlanBody(tot, seg_start, L, select, rows_per_item, work, n_work, node_first, node_items, rows_scanned, split,
-           max_items, overflow, nullptr, balance_cus);
+           max_items, overflow, cursor, balance_cus);
 }
 
 

@@ -382,6 +382,14 @@ const char *AHistSum(long long *sum_g, long long *sum_h, unsigned *bin_count, co
   });
 }
 
+const char *AHistSumPlan(long long nrow, int nodes, unsigned *rows_per_item, unsigned *work_items) {
+  return Guard([&] {
+    if (nrow < 1 || nodes < 1 || !rows_per_item || !work_items) throw std::runtime_error("bad arguments");
+    *rows_per_item = HistSumRowsPerItem((size_t)nrow, nodes);
+    *work_items = (unsigned)((size_t)nrow / *rows_per_item + 2 * (size_t)nodes + 2);
+  });
+}
+
 const char *AHistSumNoAlloc(long long *sum_g, long long *sum_h, unsigned *bin_count, const long long *parent_g,
                             const long long *parent_h, const unsigned *parent_c, const float *grad,
                             const float *hess, const unsigned *node_size, const unsigned *bins,

@@ -156,6 +156,13 @@ const char *AHistSum(long long *sum_g, long long *sum_h, unsigned *bin_count, co
                      const unsigned *node_size, const unsigned *bins, unsigned long long stride, long long nrow,
                      int ncol, int nodes, int use_trick, int shift_g, int shift_h, void *stream);
 
+/* The work plan AHistSum makes for nrow rows in `nodes` segments, host arithmetic
+ * only: rows per work item (about 512 items where items of at most 64512 rows
+ * allow it, else items of that many rows) and the work items it sizes its
+ * work memory for (one slab of 64 KB per 16 features, 128 KB with hessians,
+ * each). */
+const char *AHistSumPlan(long long nrow, int nodes, unsigned *rows_per_item, unsigned *work_items);
+
 /* AHistSum for callers that cannot allocate device memory (code under HIP
  * graph capture, tight serving loops, harnesses that forbid hipMalloc).  No
  * counterpart in the reference.  Same arguments and results as AHistSum; the
@@ -172,7 +179,13 @@ const char *AHistSum(long long *sum_g, long long *sum_h, unsigned *bin_count, co
  * needs two spare items, so e.g. 28 features with hessians and 64 nodes allow
  * 8.1 M rows.  All calls on one GPU share the array: calls that overlap in
  * time on one GPU (two streams, two threads) race; calls on one stream, one
- * after the other, are safe, and nothing has to be cleared between them. */
+ * after the other, are safe, and nothing has to be cleared between them.
+ * The FIRST call on a device, and the first call for a feature count (in steps
+ * of 4 up to 32) and hessian choice, also resolves the array's device address
+ * (hipGetSymbolAddress) and raises the LDS limit of the kernels it uses
+ * (hipFuncSetAttribute): calls outside any stream, made once per process.  A
+ * caller under graph capture makes one call of the shape it will capture
+ * beforehand. */
 const char *AHistSumNoAlloc(long long *sum_g, long long *sum_h, unsigned *bin_count, const long long *parent_g,
                             const long long *parent_h, const unsigned *parent_c, const float *grad,
                             const float *hess, const unsigned *node_size, const unsigned *bins,

@@ -25,6 +25,13 @@ def _ok(rc, what):
         raise RuntimeError("%s failed with HIP error %d" % (what, rc))
 
 
+def free_device_bytes():
+    """Free device memory as hipMemGetInfo reports it."""
+    free, total = ctypes.c_size_t(), ctypes.c_size_t()
+    _ok(hip().hipMemGetInfo(ctypes.byref(free), ctypes.byref(total)), "hipMemGetInfo")
+    return free.value
+
+
 def synchronize():
     _ok(hip().hipDeviceSynchronize(), "hipDeviceSynchronize")
 

@@ -209,6 +209,20 @@ def test_no_alloc_histogram_size_limits_are_checked_before_the_gpu_is_touched():
                               parent_h=p, parent_c=p)
 
 
+def test_hist_sum_plans_items_of_the_largest_size_for_many_rows(arb):
+    # about 512 work items while items of at most 64512 rows allow it; beyond 512 x 64512 = 33 M rows
+    # the items keep that size and their number grows (it must not fall back to 1024-row items:
+    # 50 M rows would then take 49 000 slabs of 128 KB)
+    per, items = arb.hist_sum_plan(10_500_000, 1)
+    assert per % 1024 == 0 and 500 <= items <= 520 and per * (items - 4) <= 10_500_000 <= per * items
+    for rows, nodes in ((33_100_000, 1), (50_000_000, 8), (2_000_000_000, 64)):
+        per, items = arb.hist_sum_plan(rows, nodes)
+        assert per == 64512, (rows, per)
+        assert items == rows // 64512 + 2 * nodes + 2
+    per, items = arb.hist_sum_plan(1000, 2)
+    assert per == 1024 and items == 6
+
+
 def test_block_matrix_arguments_are_checked_on_the_host(arb):
     # ACreateFromQuantizedBlocks: nothing is dereferenced when the matrix is created
     p, br = 4096, 1 << 30

@@ -374,6 +374,35 @@ def test_rows_in_place_thousand_features(arb, oracle):
     assert_same_training(arb, oracle, X, y, cfg, rounds=2)
 
 
+@pytest.mark.parametrize("objective", [0, 1])
+def test_one_launch_records_leave_the_cells_of_unused_bins_zero(arb, oracle, objective):
+    # 40 features whose bin ids stop at 64 under hist_size 256: every feature fits ONE LDS histogram of
+    # the 65 bins in use, the slab reduction writes only those, and the split scan and the root totals
+    # still read 256 cells per feature: the cells above the bins in use must be zero in every node
+    # histogram of every level of every tree (they are cleared once, when the booster is created)
+    rng = np.random.default_rng(40)
+    n, F = 30000, 40
+    bins = rng.integers(0, 65, size=(n, F), dtype=np.uint8)
+    s = bins[:, 3].astype(np.float32) / 16 - (bins[:, 17] > 30) + (bins[:, 39] == 64) + 0.3 * rng.normal(size=n)
+    y = s.astype(np.float32) if objective == 0 else (s > 1).astype(np.float32)
+    cfg = {"objective": objective, "method": 1, "internals": {"hist_size": 256, "double_precision": True},
+           "tree": {"max_depth": 5, "eta": 0.3, "lambda": 1.0}}
+    ob = oracle.Booster(bins, y=y, config=cfg, binned=True)
+    g = arb.Garden(cfg, arb.DMatrix(bins, y=y, quantized=True))
+    g.set_inspect(True)
+    for r in range(4):
+        ob.grow(1)
+        g.grow_tree()
+        for level in range(5):
+            hg, ho = g.level_hist(level), ob.level_hist(level)
+            assert hg.shape[2] == 256
+            assert np.array_equal(hg, ho[:, :, :256, :]), (r, level)
+            assert not hg[:, :, 65:, :].any()
+        for key in ("fid", "quantized", "gain", "weights"):
+            assert np.array_equal(ob.tree(r)[key], g.tree(r)[key]), (r, key)
+    assert np.array_equal(ob.yhat(), g.train_yhat())
+
+
 def test_many_trees_without_reading_the_model(arb, oracle):
     # tree records wait on the device (a ring of 64) until the model is read
     X, y = make_data(3000, 6, 1, seed=64)

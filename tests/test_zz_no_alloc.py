@@ -4,7 +4,7 @@ call left in the shared work memory would show."""
 import numpy as np
 import pytest
 
-from hipmem import DeviceArray, synchronize
+from hipmem import DeviceArray, free_device_bytes, synchronize
 from test_gpu_hist_sum import arb, oracle_nodes, run_hist_sum  # noqa: F401
 
 pytestmark = pytest.mark.gpu
@@ -49,6 +49,33 @@ def test_no_alloc_equals_allocating_entry_point_twice(arb, oracle, pair):
         if trick:  # and both equal the checker
             assert np.array_equal(got[0][:, :F], want[..., 0])
             assert np.array_equal(got[2][:, :F].astype(np.int64), want[..., 2])
+
+
+def test_no_alloc_leaves_the_free_device_memory_alone(arb):
+    # after a first call of the same shape (one-time set-up: symbol address, LDS limits), further
+    # calls neither take nor return device memory
+    bins, g, h, offs = _case(5, 200000, 28, 4, True)
+    Q, n = 7, len(g)
+    d_bins = DeviceArray(np.ascontiguousarray(
+        np.pad(bins, ((0, 0), (0, 0))).view(np.uint32).reshape(n, Q).T))
+    d_g, d_h, d_off = DeviceArray(g), DeviceArray(h), DeviceArray(offs)
+    out_g = DeviceArray(shape=(4, 28, 256), dtype=np.int64)
+    out_h = DeviceArray(shape=(4, 28, 256), dtype=np.int64)
+    out_c = DeviceArray(shape=(4, 28, 256), dtype=np.uint32)
+    status = DeviceArray(np.array([0], np.uint32))
+
+    def call():
+        arb.hist_sum_no_alloc(out_g.ptr, out_h.ptr, out_c.ptr, d_g.ptr, d_h.ptr, d_off.ptr, d_bins.ptr, n, n, 28, 4,
+                              30, 32, status=status.ptr)
+        synchronize()
+    call()
+    first = out_c.get().copy()
+    before = free_device_bytes()
+    for _ in range(3):
+        call()
+        assert free_device_bytes() == before
+    assert int(status.get()[0]) == 0
+    assert np.array_equal(out_c.get(), first) and int(first[:, 0].sum()) == n
 
 
 def test_no_alloc_reports_bad_offsets_in_the_status_word(arb):
