@@ -53,7 +53,8 @@ Configuration Configuration::Parse(const char *text) {
     GetNum(*v, "hist_size", &cfg.internal.hist_size);
     GetNum(*v, "stream_block_rows", &cfg.internal.stream_block_rows);
     GetNum(*v, "stream_resident_bytes", &cfg.internal.stream_resident_bytes);
-    GetBool(*v, "wide_rows_in_place", &cfg.internal.wide_rows_in_place);
+    if (const json::Value *w = v->find("wide_rows_in_place"))
+      cfg.internal.wide_rows_in_place = w->is_number() ? (int)w->number() : (w->boolean() ? 1 : 0);
   }
   return cfg;
 }

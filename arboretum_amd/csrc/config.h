@@ -57,8 +57,11 @@ struct InternalConfiguration {  // param.h:54-64
   // (src/io/io.cu:496-507); 0: every block is streamed.
   long long stream_resident_bytes = -1;
   // Extension: matrices of more than 32 features keep their rows in place and
-  // re-order (row id, gradients) only; false selects the row-moving passes.
-  bool wide_rows_in_place = true;
+  // re-order (row id, gradients) only, where that is the faster way (true, the
+  // default: from 48 features on, and for any width whose bins in use fit one
+  // LDS histogram); false selects the row-moving passes, the number 2 rows in
+  // place for every width above 32 features.
+  int wide_rows_in_place = 1;
 };
 
 struct Configuration {  // param.h:66-74

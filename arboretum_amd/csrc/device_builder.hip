@@ -596,9 +596,15 @@ class HipTreeBuilder : public TreeBuilder {
     // once per level, whole): e.g. 200 features of 65 bins with one word per cell.
     rec_slots_ = std::min(kSlots, data->max_bin + 1);
     const size_t rec_lds = (size_t)HistBlocks(Q_) * kBlockFeatures * rec_slots_ * 8 * (pair_ ? 2 : 1);
-    indexed_ = !wide_ && !dm_->streamed && !single_group_ && D_ > 2 && cfg.internal.wide_rows_in_place &&
-               Q_ <= 256;  // at most 64 pieces of 16 bytes per record
     rec_one_launch_ = rec_lds <= kLdsBudget - 1024;  // else groups of quads_per_group_ quads at 256 bins
+    // Measured per tree at 10.5 M rows, 256 bins, max_depth 8 (rows in place / rows moved once per
+    // group of eight quads): 33 features 2.47 / 2.39 ms, 40: 2.52 / 2.44, 44: 2.69 / 2.54, 48: 2.56 /
+    // 2.68, 64: 2.59 / 3.27, 128: 3.88 / 6.21; with the bins in use in one LDS histogram (64 bins)
+    // 33: 2.10 / 2.40, 44: 2.24 / 2.53.  So rows stay in place from 48 features (twelve quads) on,
+    // and at any width when one launch builds the whole histogram.
+    const bool in_place_pays = rec_one_launch_ || Q_ >= 12;
+    indexed_ = !wide_ && !dm_->streamed && !single_group_ && D_ > 2 && Q_ <= 256 &&  // at most 64 pieces of 16 bytes per record
+               (cfg.internal.wide_rows_in_place >= 2 || (cfg.internal.wide_rows_in_place == 1 && in_place_pays));
     // one launch: a power of two of blocks between the bins of the LDS image when that still fits
     rec_lay_blocks_ = 0;
     if (rec_one_launch_) {

@@ -328,15 +328,20 @@ def test_training_many_features_uses_feature_groups(arb, oracle):
     assert_same_training(arb, oracle, X, y, cfg, rounds=2)
 
 
-@pytest.mark.parametrize("in_place", [True, False])
-@pytest.mark.parametrize("objective,F", [(0, 36), (1, 33), (0, 70)])
-def test_quad_groups_of_wide_matrices(arb, oracle, objective, F, in_place):
-    # 33 and 36 features: a group of eight quads and a group of one; 70: three groups.  in_place:
-    # rows stay where they are as records and (row id, gradients) are re-ordered (the default for
-    # more than 32 features); otherwise the fused pass moves the rows once per group of quads
+@pytest.mark.parametrize("in_place", [2, 1, False])
+@pytest.mark.parametrize("objective,F,hist", [(0, 36, 100), (1, 33, 100), (0, 70, 100), (1, 44, 256), (0, 48, 256),
+                                              (1, 47, 255)])
+def test_quad_groups_of_wide_matrices(arb, oracle, objective, F, hist, in_place):
+    # 33 and 36 features: a group of eight quads and a group of one; 70: three groups.  in_place 2:
+    # rows stay where they are as records and (row id, gradients) are re-ordered; False: the fused
+    # pass moves the rows once per group of quads; 1 (the default): whichever was measured faster
+    # for the shape (in place from 48 features on, or when the bins in use fit one LDS histogram:
+    # 44 and 47 features at 256 bins move their rows, 48 do not)
     X, y = make_data(20000, F, objective, seed=F, nan_frac=0.05)
+    if hist >= 255:     # continuous columns, so that the features use all the bins
+        X[:, F // 2:] = np.random.default_rng(F).normal(size=(20000, F - F // 2)).astype(np.float32)
     cfg = {"objective": objective, "method": 1,
-           "internals": {"hist_size": 100, "double_precision": True, "wide_rows_in_place": in_place},
+           "internals": {"hist_size": hist, "double_precision": True, "wide_rows_in_place": in_place},
            "tree": {"max_depth": 6, "eta": 0.3, "lambda": 1.0}}
     assert_same_training(arb, oracle, X, y, cfg, rounds=2)
 
