@@ -67,7 +67,7 @@ __device__ __forceinline__ void AccumulateRow(unsigned long long *__restrict__ l
         const unsigned bi = ((unsigned)t + i) & 3u;  // byte of the quad
         unsigned bin = __builtin_amdgcn_ubfe(sel, 8u * bi, 8u);  // one v_bfe_u32
         const unsigned f16 = 4u * qi + bi;
-        if (HI) bin += __builtin_amdgcn_ubfe(b[NQ], 16u * (unsigned)k + f16, 1u);
+        if constexpr (HI != 0) bin += __builtin_amdgcn_ubfe(b[NQ], 16u * (unsigned)k + f16, 1u);
         // Quads past NQ do not exist.  Padding features of the last quad of
         // the matrix (bin 0 in every row) are accumulated like real ones into
         // slots nobody reads: cheaper than a per-update test.

@@ -261,10 +261,40 @@ def other_config(arb, workload, rows_arg, steps):
     dt = time.perf_counter() - t0
     scanned = model.rows_scanned() - s0
     trees = steps * trees_per_round
+    # The histogram kernels of these matrices (rows in place: k_hist_rec over the records of the
+    # smaller children, the root of configs[3] from the quad columns by k_hist) against the HBM
+    # roofline, by the same accounting as the headline: rows accumulated x (F bin bytes + 4 row id
+    # + the gradient pair) + cells written once; and against the LDS atomic floor of those rows.
+    # Phase times come from one more round with every phase bracketed by events.
+    model.enable_timing(1)
+    s1 = model.rows_scanned()
+    model.grow_tree()
+    model.synchronize()
+    tm = model.timings()
+    model.enable_timing(0)
+    acc_rows = (model.rows_scanned() - s1) / trees_per_round
+    pair = cfg["objective"] != 0
+    depth = cfg["tree"]["max_depth"]
+    slots_used = cfg["internals"]["hist_size"] + 1 if workload == "config2" else 256
+    cell_bytes = 20 if pair else 12
+    hist_bytes = acc_rows * (F + 4 + (8 if pair else 4)) + (1 << (depth - 1)) * F * slots_used * cell_bytes
+    hist_s = (tm["hist_root_ms"] + tm["hist_deep_ms"]) * 1e-3 / trees_per_round
+    part_s = tm["partition_ms"] * 1e-3 / trees_per_round
+    floor_s = lds_floor_us(acc_rows, F, 2 if pair else 1) * 1e-6
+    roofline = {"bound": "hbm", "kernel": "k_hist_rec (rows in place as records" +
+                (")" if workload == "config2" else "; the root level by k_hist from the quad columns)"),
+                "achieved": hist_bytes / hist_s / 1e9 if hist_s > 0 else 0.0, "peak": HBM_PEAK / 1e9, "unit": "GB/s",
+                "frac": hist_bytes / hist_s / HBM_PEAK if hist_s > 0 else 0.0, "traffic": None,
+                "bytes_per_tree": hist_bytes, "rows_accumulated_per_tree": acc_rows,
+                "hist_ms_per_tree": hist_s * 1e3, "lds_floor_ms_per_tree": floor_s * 1e3,
+                "frac_of_lds_floor": floor_s / hist_s if hist_s > 0 else 0.0,
+                # partition of (row id, g, h): rows x 9 bytes by the same accounting, per split level
+                "partition_ms_per_tree": part_s * 1e3,
+                "partition_frac_of_hbm": (rows * 9 * (depth - 1) / part_s) / HBM_PEAK if part_s > 0 else 0.0}
     return {"metric": "seconds per tree", "workload": name, "rows": rows, "features": F,
             "rounds": steps, "trees": trees, "sec_per_tree": dt / trees, "sec_per_round": dt / steps,
             "hist_updates_per_s": scanned * F / dt, "first_round_with_quantisation_s": t_first,
-            "generate_s": t_gen}
+            "generate_s": t_gen, "roofline": roofline}
 
 
 def cpu_baseline(X, y, cfg, sample_rows, trees):
