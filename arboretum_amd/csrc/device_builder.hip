@@ -519,6 +519,7 @@ struct FusedArgs {
   int slab_entries;
   const uint32_t *split_bins;  // start of the whole matrix
   int q0;                      // first quad of this launch
+  LevelScan scan;              // hg set: the pass finds the splits of its parents itself
 };
 
 template <bool PAIR, int NQ, bool WRITE, bool GROUP, bool PACK, int HI>
@@ -529,7 +530,7 @@ void LaunchFusedNQ(hipStream_t st, unsigned grid, const FusedArgs &a) {
   hipLaunchKernelGGL((k_part_hist<PAIR, NQ, WRITE, GROUP, PACK, HI>), dim3(grid), dim3(kHistThreads), lds, st,
                      a.bins + (size_t)a.q0 * a.stride, a.bins_out ? a.bins_out + (size_t)a.q0 * a.stride : nullptr,
                      a.stride, a.F, a.g, a.g_out, a.h, a.h_out, a.shifts, a.split, a.tot, a.seg_start, a.work,
-                     a.n_work, a.cursor, a.item_base, a.slab, a.slab_entries, a.split_bins, a.q0);
+                     a.n_work, a.cursor, a.item_base, a.slab, a.slab_entries, a.split_bins, a.q0, a.scan);
 }
 
 template <bool PAIR, bool WRITE, bool GROUP, bool PACK, int HI = 0>
@@ -704,8 +705,13 @@ class HipTreeBuilder : public TreeBuilder {
     }
     d_split_ = DevAlloc<SplitRec>(last_nodes);
     d_cand_ = DevAlloc<Cand>((size_t)last_nodes * F_);
-    d_node_first_ = DevAlloc<unsigned>(last_nodes);
-    d_node_items_ = DevAlloc<unsigned>(last_nodes);
+    // two sets of (first item, items) per node: a slab reduction reads the plan of the pass before it
+    // while it writes the plan of the pass after it
+    d_node_first2_ = DevAlloc<unsigned>((size_t)2 * last_nodes);
+    d_node_items2_ = DevAlloc<unsigned>((size_t)2 * last_nodes);
+    d_node_first_ = d_node_first2_;
+    d_node_items_ = d_node_items2_;
+    own_scan_ = fused_ && single_group_ && std::getenv("ARB_SEPARATE_SCAN") == nullptr;
     // row passes of a streamed matrix cover one block at a time
     const size_t plan_rows = dm_->streamed ? std::min(n_, dm_->block_rows) : n_;
     max_hist_items_ = (unsigned)(plan_rows / HistRowsPerItem(plan_rows)) + 2 * last_nodes + 2;
@@ -767,8 +773,8 @@ class HipTreeBuilder : public TreeBuilder {
 
   ~HipTreeBuilder() override {
     (void)hipStreamSynchronize(stream_);
-    void *ptrs[] = {d_y_, d_labels_, d_yhat_, d_g_, d_h_, d_leaf_, d_split_, d_cand_, d_node_first_,
-                    d_node_items_, d_hwork_, d_pwork_, d_nwork_, d_wave_left_, d_item_left_, d_slab_,
+    void *ptrs[] = {d_y_, d_labels_, d_yhat_, d_g_, d_h_, d_leaf_, d_split_, d_cand_, d_node_first2_,
+                    d_node_items2_, d_hwork_, d_pwork_, d_nwork_, d_wave_left_, d_item_left_, d_slab_,
                     d_shifts_, d_gmax_, d_rows_scanned_, d_tfid_, d_tbin_, d_tgain_, d_weights_, d_active_, d_overflow_, d_records_, d_cursor2_};
     for (void *p : ptrs)
       if (p) (void)hipFree(p);
@@ -1100,8 +1106,28 @@ class HipTreeBuilder : public TreeBuilder {
       LaunchHist<false>(nq, stream_, grid, bins, stride, q0, F_, g, h, d_shifts_, d_hwork_, d_nwork_, d_slab_, slab_stride_);
   }
 
-  void Reduce(int L, int hb, bool by_parent, int parent_state, bool trick, bool accumulate = false) {
+  // plan_state >= 0: one more block plans the fused pass over this level's nodes (d_tot_ / d_seg_
+  // [plan_state]) into the other set of (first item, items) per node, which is in use afterwards
+  void Reduce(int L, int hb, bool by_parent, int parent_state, bool trick, bool accumulate = false,
+              int plan_state = -1) {
     Mark(kReduce);
+    const size_t last_nodes = (size_t)1 << (D_ - 2);
+    unsigned *next_first = d_node_first_ == d_node_first2_ ? d_node_first2_ + last_nodes : d_node_first2_;
+    unsigned *next_items = d_node_items_ == d_node_items2_ ? d_node_items2_ + last_nodes : d_node_items2_;
+    NextPlan plan;
+    if (plan_state >= 0) {
+      plan.tot = d_tot_[plan_state];
+      plan.seg_start = d_seg_[plan_state];
+      plan.L = L;
+      plan.rows_per_item = FusedRowsPerItem(L);
+      plan.work = d_pwork_;
+      plan.n_work = d_nwork_ + 1;
+      plan.node_first = next_first;
+      plan.node_items = next_items;
+      plan.max_items = FusedGrid(L);
+      plan.overflow = d_overflow_;
+      plan.cursor = d_cursor2_;
+    }
     // many nodes: few slabs per node and the output dominates -> longer output runs per block
     const bool wide_blocks = L >= 32;
     const int entries = wide_blocks ? 256 : 64;
@@ -1111,13 +1137,14 @@ class HipTreeBuilder : public TreeBuilder {
     dim3 grid(wide_ ? (slab_entries_ + entries - 1) / entries
                     : slab_entries_ / kBlockEntries * ((lds_slots * kBlockFeatures + entries - 1) / entries) + (hi_ ? 1 : 0),
               L);
+    if (plan_state >= 0) grid.x += 1;
 #define ARB_REDUCE(P, LN)                                                                                          \
   hipLaunchKernelGGL((k_hist_reduce<P, LN, unsigned long long>), grid, dim3(1024), 0, stream_, d_slab_, slab_entries_, nbin_total_,   \
                      d_node_first_, d_node_items_, by_parent ? 1 : 0, d_split_, d_tot_[parent_state], d_hg_[hb], \
                      d_hh_[hb], d_hc_[hb], d_hg_[hb ^ 1], d_hh_[hb ^ 1], d_hc_[hb ^ 1], trick ? 1 : 0,           \
                      accumulate ? 1 : 0, wide_ ? 1 : 0,                                                           \
                      indexed_ && rec_one_launch_ ? HistBlocks(Q_) : HistBlocks(quads_per_group_),                \
-                     lds_slots, lay_blocks, hi_base_)
+                     lds_slots, lay_blocks, hi_base_, plan)
     if (pair_) {
       if (wide_blocks) ARB_REDUCE(true, 4);
       else ARB_REDUCE(true, 16);
@@ -1126,6 +1153,10 @@ class HipTreeBuilder : public TreeBuilder {
       else ARB_REDUCE(false, 16);
     }
 #undef ARB_REDUCE
+    if (plan_state >= 0) {
+      d_node_first_ = next_first;
+      d_node_items_ = next_items;
+    }
   }
 
   void GrowOne(int label) {
@@ -1161,7 +1192,7 @@ class HipTreeBuilder : public TreeBuilder {
         // the slabs of the root may have been written by the last pass of the previous tree
         if (!root_hist_ready_) HistOfNodes(orig, state, 1, false, n_, true, 0);
         root_hist_ready_ = false;
-        Reduce(1, hb, false, state, false);
+        Reduce(1, hb, false, state, false, false, own_scan_ && !last ? state : -1);
         // (the last pass of the previous tree has also summed the root's totals)
         if (!root_totals_ready_)
           hipLaunchKernelGGL(k_root_from_hist, dim3(1), dim3(64), 0, stream_, d_hg_[hb], d_hh_[hb], d_tot_[state], slots_, hi_base_);
@@ -1179,10 +1210,26 @@ class HipTreeBuilder : public TreeBuilder {
           // quads; the first one moves the gradients
           for (int q0 = 0; q0 < Q_; q0 += quads_per_group_) {
             const int nq = std::min(quads_per_group_, Q_ - q0);
+            LevelScan scan{};
+            if (own_scan_) {  // the parents' splits are selected by the pass itself, from the scan's candidates
+              scan.cand = d_cand_;
+              scan.F = F_;
+              scan.L = PL;
+              scan.tot_next = d_tot_[state];
+              scan.seg_next = d_seg_[state];
+              scan.split = d_split_;
+              scan.t_fid = d_tfid_;
+              scan.t_bin = d_tbin_;
+              scan.t_gain = d_tgain_;
+              scan.heap_off = PL - 1;
+              scan.active = sampling_ ? d_active_ + (size_t)(level - 1) * F_ : (const unsigned char *)nullptr;
+              scan.node_first = d_node_first_;
+              scan.rows_scanned = ScanCounter(level);
+            }
             FusedArgs a{src.bins, last ? nullptr : dst.bins, stride_, F_, src.g, q0 == 0 ? dst.g : nullptr, src.h,
                         q0 == 0 ? dst.h : nullptr, d_shifts_, d_split_, d_tot_[ps], d_seg_[ps], d_pwork_,
                         d_nwork_ + 1, q0 == 0 ? d_cursor2_ : nullptr, d_item_left_, d_slab_, slab_stride_, src.bins,
-                        q0};
+                        q0, scan};
 #define ARB_FUSED(P, W)                                                       \
   do {                                                                        \
     if (hi_ && P && pack_) LaunchFused<P, W, false, P, 1>(nq, stream_, grid, a); \
@@ -1203,7 +1250,7 @@ class HipTreeBuilder : public TreeBuilder {
             if (timing_ && (last || !dominant_only_ || trees_grown_ % sample_every_ == 0))
             ++(last ? timings_.fused_last_launches : timings_.hist_deep_launches);
           }
-          Reduce(L, hb, true, ps, true);
+          Reduce(L, hb, true, ps, true, false, own_scan_ && !last ? state : -1);
         } else {
           const unsigned grid = (unsigned)std::min<size_t>(n_ / kPartRows + 2 * PL + 1, max_part_items_);
           Mark(kPlan);
@@ -1229,7 +1276,8 @@ class HipTreeBuilder : public TreeBuilder {
         }
       }
       if (inspect_) KeepHist(level, L, hb);
-      LaunchSplit(level, L, hb, state, gp, fused_ && !last);
+      // (own_scan_: only the scan; the pass of the next level selects the splits of this level's nodes)
+      LaunchSplit(level, L, hb, state, gp, fused_ && !last, own_scan_ && !last);
       if (last && !final_hist) LaunchLeafWeights(L, state, gp);
       state ^= 1;
     }
@@ -1334,7 +1382,9 @@ class HipTreeBuilder : public TreeBuilder {
   }
 
   // plan_next: also plan the fused pass of the next level over these nodes
-  void LaunchSplit(int level, int L, int hb, int state, const GainParams &gp, bool plan_next = false) {
+  // scan_only: candidates per (node, feature) only (k_split_scan); the next fused pass selects
+  void LaunchSplit(int level, int L, int hb, int state, const GainParams &gp, bool plan_next = false,
+                   bool scan_only = false) {
     Mark(kSplit);
     const int hs = std::min(data_->hist_size, slots_);  // data_->hist_size: the configuration's, or the distinct values (exact method)
     const unsigned char *active = sampling_ ? d_active_ + (size_t)level * F_ : (const unsigned char *)nullptr;
@@ -1343,7 +1393,7 @@ class HipTreeBuilder : public TreeBuilder {
     // selects.  With fewer nodes that would leave the gain arithmetic (28
     // features x 256 bins in double precision per node) on a few CUs, and the
     // scan over (feature, node) waves followed by the selection is faster.
-    if (L >= 32) {
+    if (L >= 32 && !scan_only) {
 #define ARB_SCAN_SELECT(P, D)                                                                                     \
   hipLaunchKernelGGL((k_scan_select<P, D>), dim3(L + (plan_next ? 1 : 0)), dim3(1024), 0, stream_, d_hg_[hb],     \
                      d_hh_[hb], d_hc_[hb], nbin_total_, F_, slots_, L, d_tot_[state], d_shifts_, gp, hs,          \
@@ -1366,6 +1416,7 @@ class HipTreeBuilder : public TreeBuilder {
     else if (f64_) ARB_SCAN(false, true);
     else ARB_SCAN(false, false);
 #undef ARB_SCAN
+    if (scan_only) return;
     if (plan_next) {
       hipLaunchKernelGGL(k_select_plan, dim3(1), dim3(1024), 0, stream_, d_cand_, F_, L, d_tot_[state],
                          d_seg_[state], d_tot_[state ^ 1], d_seg_[state ^ 1], d_split_, d_tfid_, d_tbin_, d_tgain_,
@@ -1664,6 +1715,8 @@ class HipTreeBuilder : public TreeBuilder {
   std::vector<unsigned char> active_host_;
   std::default_random_engine rnd_;
   bool sampling_ = false;
+  unsigned *d_node_first2_ = nullptr, *d_node_items2_ = nullptr;  // both sets; d_node_first_ / d_node_items_: the one in use
+  bool own_scan_ = false;  // the fused passes find the splits of their parents themselves (LevelScan)
   unsigned *d_leaf_ = nullptr, *d_node_first_ = nullptr, *d_node_items_ = nullptr, *d_nwork_ = nullptr,
            *d_wave_left_ = nullptr, *d_item_left_ = nullptr, *d_gmax_ = nullptr, *d_cursor2_ = nullptr;
   RowBuffers buf_[2];

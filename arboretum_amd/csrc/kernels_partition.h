@@ -4,6 +4,7 @@
 #include "device_common.h"
 #include "kernels_hist.h"
 #include "kernels_plan.h"
+#include "kernels_split.h"
 
 namespace arb {
 namespace {
@@ -392,6 +393,9 @@ __device__ __forceinline__ void MergeRows(unsigned long long *__restrict__ lds, 
 // HI (not with GROUP): column NQ of the rows is their ninth-bit word (SplitTest);
 // it moves with the quads, and ids of 256 are accumulated in a 257th row of
 // entries of the LDS histogram and of the slab.
+// scan.cand set (not with GROUP): the splits of the parents are not read from
+// `split` but selected here, from the candidates of the split scan (LevelScan):
+// no selection kernel runs between the split scan of a level and this pass.
 template <bool PAIR, int NQ, bool WRITE, bool GROUP = false, bool PACK = false, int HI = 0>
 __global__ void __launch_bounds__(kHistThreads)
 k_part_hist(const uint32_t *__restrict__ bins, uint32_t *__restrict__ bins_out, size_t stride, int F,
@@ -401,13 +405,18 @@ k_part_hist(const uint32_t *__restrict__ bins, uint32_t *__restrict__ bins_out, 
             const unsigned *__restrict__ seg_start, const WorkItem *__restrict__ work,
             const unsigned *__restrict__ n_work, unsigned *__restrict__ cursor,
             unsigned *__restrict__ item_base, unsigned long long *__restrict__ slab,
-            int slab_entries, const uint32_t *__restrict__ split_bins, int q0) {
+            int slab_entries, const uint32_t *__restrict__ split_bins, int q0, const LevelScan scan) {
   extern __shared__ unsigned long long lds[];
   __shared__ unsigned s_tmp[kItemWaves + 2];
+  __shared__ SplitRec s_rec;
   const unsigned w = blockIdx.x;
+  const bool own_scan = !GROUP && scan.cand != nullptr;  // uniform over the launch
+  if (own_scan && w == 0) WriteEmptyNodes(scan, tot, seg_start);
   if (w >= *n_work) return;
   const WorkItem it = work[w];
-  const SplitRec s = split[it.node];
+  const SplitRec s = own_scan ? SelectInPass(scan, (int)it.node, tot[it.node], seg_start,
+                                             w == scan.node_first[it.node], &s_rec)
+                              : split[it.node];
   const unsigned long long cl = s.left.c, cr = tot[it.node].c - cl;
   const bool build_right = cl > cr;  // ties -> left (hist_grad_sum.cu:288-290)
   static_assert(!(HI && GROUP), "ninth bits: one group of quads only");
@@ -663,6 +672,20 @@ k_part_rows(const uint32_t *__restrict__ bins, uint32_t *__restrict__ bins_out, 
 // (matrices with a ninth-bit word); one more block of the grid (the last one)
 // reduces it into cell hi_base + f of the node's histogram, behind the 256-bin
 // histograms of the features.
+// Work plan of the next fused pass, made by one more block of the slab reduction (the ranges of
+// the nodes are known since their parents were split): work == null, none.  node_first /
+// node_items must be other arrays than the ones this reduction reads.
+struct NextPlan {
+  const NodeSum *tot = nullptr;
+  const unsigned *seg_start = nullptr;
+  int L = 0;
+  unsigned rows_per_item = 0;
+  WorkItem *work = nullptr;
+  unsigned *n_work = nullptr, *node_first = nullptr, *node_items = nullptr;
+  unsigned max_items = 0;
+  unsigned *overflow = nullptr, *cursor = nullptr;
+};
+
 // CNT: type of the row counts of the node histograms.  The tree builder keeps
 // 64-bit counts: a streamed matrix may hold 2^32 rows and more, all of which can
 // sit in one cell (a constant feature, the bin of the missing values).
@@ -675,7 +698,15 @@ k_hist_reduce(const unsigned long long *__restrict__ slab, int slab_entries, int
               long long *__restrict__ hh, CNT *__restrict__ hc,
               const long long *__restrict__ pg, const long long *__restrict__ ph,
               const CNT *__restrict__ pc, int trick, int accumulate, int plain, int group_blocks,
-              int lds_slots = kSlots, int lay_blocks = 0, int hi_base = 0) {
+              int lds_slots = kSlots, int lay_blocks = 0, int hi_base = 0, const NextPlan plan = NextPlan{}) {
+  // one more block in the grid's x direction (for node 0 only) cuts the row ranges of this
+  // level's nodes into the work items of the fused pass that follows
+  if (plan.work != nullptr && blockIdx.x + 1 == gridDim.x) {
+    if (blockIdx.y == 0)
+      PlanBody(plan.tot, plan.seg_start, plan.L, 0, plan.rows_per_item, plan.work, plan.n_work, plan.node_first,
+               plan.node_items, nullptr, nullptr, plan.max_items, plan.overflow, plan.cursor);
+    return;
+  }
   // LANES threads share the slabs of one entry; a block covers 1024 / LANES
   // consecutive entries (with 4 lanes: 16 bins x 16 features, so the
   // feature-major output is written in runs of 16 bins)

@@ -127,7 +127,7 @@ k_split_scan(const long long *__restrict__ hg, const long long *__restrict__ hh,
 
 // Record of one node from its best candidate (fid < 0: none, every row stays
 // left): split, totals and row ranges of the two children, tree arrays.
-__device__ __forceinline__ void WriteNode(int nd, const NodeSum &t, float gain, int fid, int bin, long long lg,
+__device__ __forceinline__ SplitRec WriteNode(int nd, const NodeSum &t, float gain, int fid, int bin, long long lg,
                                           long long lh, unsigned long long lc,
                                           const unsigned *__restrict__ seg_start, NodeSum *__restrict__ tot_next,
                                           unsigned *__restrict__ seg_next, SplitRec *__restrict__ split,
@@ -157,6 +157,127 @@ __device__ __forceinline__ void WriteNode(int nd, const NodeSum &t, float gain, 
   t_fid[heap_off + nd] = rec.fid < 0 ? 0 : rec.fid;  // garden.cu:471-481
   t_bin[heap_off + nd] = rec.fid < 0 ? -1 : rec.bin;
   t_gain[heap_off + nd] = rec.gain;
+  return rec;
+}
+
+// What a fused pass over the rows of a level's nodes needs to select the splits of those nodes
+// itself, in its prologue, from the per-feature candidates of the split scan (k_split_scan)
+// instead of reading them from a selection kernel launched before it: one launch less per level
+// on the critical path.  Every workgroup of the pass selects for ITS node; the node's first work
+// item also writes the node's record.  cand == null: the splits are read from `split` as before.
+struct LevelScan {
+  const Cand *cand;
+  int F, L;
+  NodeSum *tot_next;
+  unsigned *seg_next;
+  SplitRec *split;
+  int *t_fid, *t_bin;
+  float *t_gain;
+  int heap_off;
+  const unsigned char *active;
+  const unsigned *node_first;         // first work item of every node: that item writes the node's record
+  unsigned long long *rows_scanned;   // advanced by the rows of the smaller side of every split
+};
+
+// Split of node nd (totals t) from its candidates: wave 0 of the workgroup keeps the candidate
+// with the highest gain, ties to the lowest feature id (hist_tree_grower.cu:59-60), over the
+// features active at this level; every thread returns the node's record.  `write`: this
+// workgroup also stores the record, the children's totals and row ranges and the tree arrays
+// (WriteNode).  Called by all threads of the workgroup; s_rec holds one record.
+__device__ __forceinline__ SplitRec SelectInPass(const LevelScan &a, int nd, const NodeSum &t,
+                                                 const unsigned *__restrict__ seg_start, bool write,
+                                                 SplitRec *s_rec) {
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  if (wave == 0) {
+    float gain = 0.0f;
+    int fid = -1, bin = -1;
+    long long lg = 0, lh = 0;
+    unsigned long long lc = 0;
+    if (t.c != 0) {
+      for (int f = lane; f < a.F; f += 64) {
+        if (a.active && !a.active[f]) continue;  // feature not sampled at this level
+        const Cand c = a.cand[(size_t)nd * a.F + f];
+        if (c.bin >= 0 && (fid < 0 || gain < c.gain)) {
+          gain = c.gain;
+          fid = f;
+          bin = c.bin;
+          lg = c.left.g;
+          lh = c.left.h;
+          lc = c.left.c;
+        }
+      }
+    }
+    for (int off = 32; off > 0; off >>= 1) {
+      const float og = __shfl_down(gain, off);
+      const int of = __shfl_down(fid, off);
+      const int ob = __shfl_down(bin, off);
+      const long long olg = __shfl_down(lg, off);
+      const long long olh = __shfl_down(lh, off);
+      const unsigned long long olc = __shfl_down(lc, off);
+      if (of >= 0 && (fid < 0 || og > gain || (og == gain && of < fid))) {
+        gain = og;
+        fid = of;
+        bin = ob;
+        lg = olg;
+        lh = olh;
+        lc = olc;
+      }
+    }
+    if (lane == 0) {
+      SplitRec rec;
+      if (write) {
+        rec = WriteNode(nd, t, gain, fid, bin, lg, lh, lc, seg_start, a.tot_next, a.seg_next, a.split, a.t_fid,
+                        a.t_bin, a.t_gain, a.heap_off);
+        if (a.rows_scanned && t.c != 0) {
+          const unsigned long long cl = fid < 0 ? t.c : lc;
+          atomicAdd(a.rows_scanned, min(cl, t.c - cl));
+        }
+      } else {
+        rec.gain = fid < 0 ? 0.0f : gain;
+        rec.fid = fid;
+        rec.bin = fid < 0 ? -1 : bin;
+        rec.pad = 0;
+        rec.left = t;
+        if (fid >= 0) {
+          rec.left.g = lg;
+          rec.left.h = lh;
+          rec.left.c = lc;
+        }
+      }
+      *s_rec = rec;
+    }
+  }
+  __syncthreads();
+  // the record as wave-uniform values (it steers the whole pass)
+  SplitRec r;
+  r.gain = __uint_as_float(__builtin_amdgcn_readfirstlane(__float_as_uint(s_rec->gain)));
+  r.fid = __builtin_amdgcn_readfirstlane(s_rec->fid);
+  r.bin = __builtin_amdgcn_readfirstlane(s_rec->bin);
+  r.pad = 0;
+  const unsigned long long *p = reinterpret_cast<const unsigned long long *>(&s_rec->left);
+  unsigned long long v[3];
+#pragma unroll
+  for (int k = 0; k < 3; ++k) {
+    const unsigned lo = __builtin_amdgcn_readfirstlane((unsigned)p[k]);
+    const unsigned hi = __builtin_amdgcn_readfirstlane((unsigned)(p[k] >> 32));
+    v[k] = ((unsigned long long)hi << 32) | lo;
+  }
+  r.left.g = (long long)v[0];
+  r.left.h = (long long)v[1];
+  r.left.c = v[2];
+  return r;
+}
+
+// Records of the nodes of a level that hold no row (no work item of the pass stands for them):
+// not split, both children empty.  Called by one workgroup.
+__device__ __forceinline__ void WriteEmptyNodes(const LevelScan &a, const NodeSum *__restrict__ tot,
+                                                const unsigned *__restrict__ seg_start) {
+  for (int nd = threadIdx.x; nd < a.L; nd += blockDim.x) {
+    const NodeSum t = tot[nd];
+    if (t.c == 0)
+      WriteNode(nd, t, 0.0f, -1, -1, 0, 0, 0, seg_start, a.tot_next, a.seg_next, a.split, a.t_fid, a.t_bin, a.t_gain,
+                a.heap_off);
+  }
 }
 
 
