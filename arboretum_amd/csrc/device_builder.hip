@@ -711,7 +711,7 @@ class HipTreeBuilder : public TreeBuilder {
     d_node_items2_ = DevAlloc<unsigned>((size_t)2 * last_nodes);
     d_node_first_ = d_node_first2_;
     d_node_items_ = d_node_items2_;
-    own_scan_ = fused_ && single_group_ && std::getenv("ARB_SEPARATE_SCAN") == nullptr;
+    own_scan_ = fused_ && single_group_;
     // row passes of a streamed matrix cover one block at a time
     const size_t plan_rows = dm_->streamed ? std::min(n_, dm_->block_rows) : n_;
     max_hist_items_ = (unsigned)(plan_rows / HistRowsPerItem(plan_rows)) + 2 * last_nodes + 2;

@@ -393,9 +393,12 @@ __device__ __forceinline__ void MergeRows(unsigned long long *__restrict__ lds, 
 // HI (not with GROUP): column NQ of the rows is their ninth-bit word (SplitTest);
 // it moves with the quads, and ids of 256 are accumulated in a 257th row of
 // entries of the LDS histogram and of the slab.
-// scan.cand set (not with GROUP): the splits of the parents are not read from
-// `split` but selected here, from the candidates of the split scan (LevelScan):
-// no selection kernel runs between the split scan of a level and this pass.
+// Without GROUP the splits of the parents are not read from `split` but selected
+// here, from the candidates of the split scan (`scan`, LevelScan): no selection
+// kernel runs between the split scan of a level and this pass.  (With HI the
+// choice is also made at run time, on scan.cand: the register allocation of
+// that instance happens to come out with fewer spills that way, 8 bytes per
+// lane against 52.)
 template <bool PAIR, int NQ, bool WRITE, bool GROUP = false, bool PACK = false, int HI = 0>
 __global__ void __launch_bounds__(kHistThreads)
 k_part_hist(const uint32_t *__restrict__ bins, uint32_t *__restrict__ bins_out, size_t stride, int F,
@@ -410,7 +413,7 @@ k_part_hist(const uint32_t *__restrict__ bins, uint32_t *__restrict__ bins_out, 
   __shared__ unsigned s_tmp[kItemWaves + 2];
   __shared__ SplitRec s_rec;
   const unsigned w = blockIdx.x;
-  const bool own_scan = !GROUP && scan.cand != nullptr;  // uniform over the launch
+  const bool own_scan = !GROUP && (HI == 0 || scan.cand != nullptr);  // uniform over the launch
   if (own_scan && w == 0) WriteEmptyNodes(scan, tot, seg_start);
   if (w >= *n_work) return;
   const WorkItem it = work[w];
