@@ -55,31 +55,38 @@ def lds_floor_us(rows_accumulated, features, words=2):
     return instr_per_cu * LDS_CYCLES_PER_ATOMIC / CLOCK_HZ * 1e6
 
 
-def kernel_source_digest():
+# the same for the matrices whose rows stay in place (configs[2], configs[3])
+WIDE_KERNEL_SOURCES = ["kernels_indexed.h", "kernels_hist.h", "device_common.h", "kernels_plan.h", "kernels_launch.h",
+                       "device_builder.hip"]
+WIDE_TRAFFIC_PROFILES = {"config2": "hbm_traffic_configs2_50Mx200_missing_depth10.txt",
+                         "config3": "hbm_traffic_configs3_20Mx100_softmax10_depth6.txt"}
+
+
+def kernel_source_digest(sources=None):
     """sha1 over the sources of the dominant kernel: a profile applies to exactly one version of them."""
     import hashlib
     h = hashlib.sha1()
-    for name in KERNEL_SOURCES:
+    for name in (sources or KERNEL_SOURCES):
         with open(os.path.join(ROOT, "arboretum_amd", "csrc", name), "rb") as f:
             h.update(f.read())
     return h.hexdigest()
 
 
-def profiled_traffic():
-    """HBM bytes per launch of the fused pass from the committed counter profile (FETCH_SIZE +
-    WRITE_SIZE of two rocprofv3 --pmc runs), or None when the profile was taken on other kernel
-    sources than the ones in the tree."""
+def profiled_traffic(profile=TRAFFIC_PROFILE, key="fused_pass_hbm_bytes_per_launch", sources=None):
+    """HBM bytes per launch of the fused pass (or per tree of the histogram kernels of a wide
+    workload) from the committed counter profile (FETCH_SIZE + WRITE_SIZE of two rocprofv3 --pmc
+    runs), or None when the profile was taken on other kernel sources than the ones in the tree."""
     try:
-        text = open(TRAFFIC_PROFILE).read()
+        text = open(profile).read()
     except OSError:
         return None
     digest, value = None, None
     for line in text.splitlines():
         if line.startswith("kernel_source_sha1:"):
             digest = line.split(":", 1)[1].strip()
-        if line.startswith("fused_pass_hbm_bytes_per_launch:"):
+        if line.startswith(key + ":"):
             value = float(line.split(":", 1)[1].strip())
-    return value if digest == kernel_source_digest() else None
+    return value if digest == kernel_source_digest(sources) else None
 
 
 def make_workload(rows, features=28, seed=0):
@@ -284,7 +291,11 @@ def other_config(arb, workload, rows_arg, steps):
     roofline = {"bound": "hbm", "kernel": "k_hist_rec (rows in place as records" +
                 (")" if workload == "config2" else "; the root level by k_hist from the quad columns)"),
                 "achieved": hist_bytes / hist_s / 1e9 if hist_s > 0 else 0.0, "peak": HBM_PEAK / 1e9, "unit": "GB/s",
-                "frac": hist_bytes / hist_s / HBM_PEAK if hist_s > 0 else 0.0, "traffic": None,
+                "frac": hist_bytes / hist_s / HBM_PEAK if hist_s > 0 else 0.0,
+                # HBM bytes per tree of the same kernels from hardware counters (committed profile)
+                "traffic": profiled_traffic(os.path.join(ROOT, "profiles", WIDE_TRAFFIC_PROFILES[workload]),
+                                            "hist_hbm_bytes_per_tree", WIDE_KERNEL_SOURCES)
+                if rows == (50_000_000 if workload == "config2" else 20_000_000) else None,
                 "bytes_per_tree": hist_bytes, "rows_accumulated_per_tree": acc_rows,
                 "hist_ms_per_tree": hist_s * 1e3, "lds_floor_ms_per_tree": floor_s * 1e3,
                 "frac_of_lds_floor": floor_s / hist_s if hist_s > 0 else 0.0,
