@@ -76,11 +76,15 @@ struct DeviceMatrix {
   int F = 0, Q = 0;          // Q words of 32 bits per row
   int bits = 8;              // bits per bin id: 8 (four features per word) or 16 (two)
   int slots = kSlots;        // histogram slots per feature
-  // 8-bit ids with a ninth-bit word per row in column Q (ids up to 256, at most 32 features):
-  // a feature that fills 256 value bins and has missing values besides (SplitTest)
+  // 8-bit ids with ninth-bit words per row in columns Q .. Q + H - 1 (ids up to 256; a word per 32
+  // features): a feature that fills 256 value bins and has missing values besides (SplitTest)
   bool hi = false;
-  int W() const { return Q + (hi ? 1 : 0); }  // words of a row that kernels read and move
-  int cols = 0;              // columns allocated per row (Q, or Q + 1 when ninth bits might be needed)
+  int H = 0;                 // ninth-bit words per row in use (0 without ninth bits)
+  int W() const { return Q + H; }  // words of a row that kernels read and move
+  int cols = 0;              // columns allocated per row (Q, or more when ninth bits might be needed)
+  // matrices of several ninth-bit words whose rows stay in place: the bits as bit columns [F][strideb]
+  uint8_t *hibits = nullptr;
+  size_t strideb = 0;
   uint32_t *bins = nullptr;  // resident: [cols][stride] in HBM
   // wide resident matrices, built on first use: the same bins row-major, RS words per row
   uint32_t *rec = nullptr;
@@ -126,6 +130,7 @@ void FreeDeviceMatrix(DeviceMatrix *m) {
   if (m->bins) (void)hipFree(m->bins);
   if (m->rec) (void)hipFree(m->rec);
   if (m->bytes) (void)hipFree(m->bytes);
+  if (m->hibits) (void)hipFree(m->hibits);
   if (m->owns_blocks)
     for (uint32_t *b : m->host_blocks)
       if (b) (void)hipHostFree(b);
@@ -224,10 +229,11 @@ void QuantiseOnDevice(DataMatrix *data, int hist_size, bool verbose, bool stream
   dm->Q = (F + 3) / 4;
   dm->stride = (n + 63) / 64 * 64;
   dm->streamed = streamed;
-  // Only a quantiser run at hist_size 256 and more can hand out the id 256; a matrix of at most 32
-  // features then gets room for a ninth-bit word per row (used if some feature turns out to need it).
-  const bool may_need_hi = !exact && !data->is_prebinned && hist_size >= kSlots && F <= 32;
-  dm->cols = dm->Q + (may_need_hi ? 1 : 0);
+  // Only a quantiser run at hist_size 256 and more can hand out the id 256; the matrix then gets
+  // room for ninth-bit words, one per 32 features (used if some feature turns out to need them).
+  const bool may_need_hi = !exact && !data->is_prebinned && hist_size >= kSlots;
+  const int hi_words = (F + 31) / 32;
+  dm->cols = dm->Q + (may_need_hi ? hi_words : 0);
   uint32_t *d_col = nullptr;  // streamed: one quad column at a time on the device
   uint32_t *d_hi = nullptr;   // the column of ninth-bit words while the features are quantised
   size_t nblocks = 0;
@@ -243,12 +249,12 @@ void QuantiseOnDevice(DataMatrix *data, int hist_size, bool verbose, bool stream
     for (size_t b = 0; b < nblocks; ++b)
       HIP_OK(hipHostMalloc((void **)&dm->host_blocks[b], (size_t)dm->cols * block_rows * sizeof(uint32_t), hipHostMallocDefault));
     d_col = DevAlloc<uint32_t>(dm->stride);
-    if (may_need_hi) d_hi = DevAlloc<uint32_t>(dm->stride);
+    if (may_need_hi) d_hi = DevAlloc<uint32_t>((size_t)hi_words * dm->stride);
   } else {
     dm->bins = DevAlloc<uint32_t>((size_t)dm->cols * dm->stride);
     if (may_need_hi) d_hi = dm->bins + (size_t)dm->Q * dm->stride;
   }
-  if (d_hi) HIP_OK(hipMemset(d_hi, 0, dm->stride * sizeof(uint32_t)));
+  if (d_hi) HIP_OK(hipMemset(d_hi, 0, (size_t)hi_words * dm->stride * sizeof(uint32_t)));
   // streamed: quad q of all rows (in d_col) -> its slice of every host block
   auto store_quad = [&](int q, const uint32_t *col) {
     for (size_t b = 0; b < nblocks; ++b) {
@@ -351,9 +357,10 @@ void QuantiseOnDevice(DataMatrix *data, int hist_size, bool verbose, bool stream
           bool has_nan = false;
           DeviceThresholds(ws.get(), d_x + (size_t)c * n, &data->thresholds[f], &data->reduced_size[f], &has_nan);
           if (bits == 8 && data->reduced_size[f] + (has_nan ? 1 : 0) > kSlots) {
-            // id 256: the ninth-bit word takes it, where the matrix has one
+            // id 256: the ninth-bit words take it, where the matrix has them
             if (d_hi == nullptr || data->reduced_size[f] + 1 > kSlots + 1) return false;
             dm->hi = true;
+            dm->H = hi_words;
           }
           if (verbose)
             printf("feature %d has been reduced to %d bits \n", f,
@@ -366,7 +373,7 @@ void QuantiseOnDevice(DataMatrix *data, int hist_size, bool verbose, bool stream
         uint32_t *out = streamed ? d_col : dm->bins + (size_t)q * dm->stride;
         if (bits == 8)
           hipLaunchKernelGGL(k_bin_assign, dim3(GridFor(n, 256)), dim3(256), 0, 0, d_x, nc, d_thr, hist_size, d_size,
-                             out, n, d_hi, q * W);
+                             out, n, d_hi ? d_hi + (size_t)((q * W) >> 5) * dm->stride : nullptr, (q * W) & 31);
         else
           hipLaunchKernelGGL(k_bin_assign_wide, dim3(GridFor(n, 256)), dim3(256),
                              2 * (size_t)hist_size * sizeof(float), 0, d_x, nc, d_thr, hist_size, d_size, out, n);
@@ -374,7 +381,7 @@ void QuantiseOnDevice(DataMatrix *data, int hist_size, bool verbose, bool stream
         HIP_OK(hipDeviceSynchronize());
         if (streamed) store_quad(q, d_col);
       }
-      if (streamed && dm->hi) store_quad(dm->Q, d_hi);
+      for (int w = 0; streamed && w < dm->H; ++w) store_quad(dm->Q + w, d_hi + (size_t)w * dm->stride);
       return true;
     };
     if (!quantise_columns(8)) {
@@ -389,6 +396,7 @@ void QuantiseOnDevice(DataMatrix *data, int hist_size, bool verbose, bool stream
       dm->bits = 16;
       dm->slots = slots;
       dm->hi = false;
+      dm->H = 0;
       d_hi = nullptr;  // (was a part of dm->bins: a resident matrix)
       dm->Q = dm->cols = (F + 1) / 2;
       dm->bins = DevAlloc<uint32_t>((size_t)dm->Q * dm->stride);
@@ -455,9 +463,10 @@ void GetDeviceBins16(const DataMatrix &data, uint16_t *out) {
     for (size_t r = 0; r < dm->rows; ++r) {
       const uint32_t *base = dm->streamed ? dm->host_blocks[r / dm->block_rows] : q.data();
       const size_t st = dm->streamed ? dm->block_rows : dm->stride, at = dm->streamed ? r % dm->block_rows : r;
-      const uint32_t hi = base[(size_t)dm->Q * st + at];
-      for (int f = 0; f < dm->F; ++f)
-        out[r * dm->F + f] = (uint16_t)(((base[(size_t)(f >> 2) * st + at] >> (8 * (f & 3))) & 255u) + ((hi >> f) & 1u));
+      for (int f = 0; f < dm->F; ++f) {
+        const uint32_t hi = base[(size_t)(dm->Q + (f >> 5)) * st + at];
+        out[r * dm->F + f] = (uint16_t)(((base[(size_t)(f >> 2) * st + at] >> (8 * (f & 3))) & 255u) + ((hi >> (f & 31)) & 1u));
+      }
     }
     return;
   }
@@ -559,6 +568,10 @@ class HipTreeBuilder : public TreeBuilder {
     trick_ = cfg.internal.use_hist_subtraction_trick;
     wide_ = dm_->bits == 16;
     hi_ = dm_->hi;
+    // one ninth-bit word (at most 32 features, one LDS histogram): ids of 256 are accumulated in a
+    // 257th row of entries; several words: they are left out of the histograms (AccumulateRow)
+    hi_rows_ = hi_ && dm_->H == 1;
+    hi_skip_ = hi_ && !hi_rows_;
     W_ = dm_->W();
     hi_word_ = hi_ ? Q_ : -1;
     report_slots_ = dm_->slots;
@@ -569,12 +582,12 @@ class HipTreeBuilder : public TreeBuilder {
       nbin_total_ = F_ * slots_;
       slab_entries_ = nbin_total_;  // slabs are feature-major
     } else {
-      hi_base_ = hi_ ? Q_ * 4 * kSlots : 0;
-      nbin_total_ = Q_ * 4 * kSlots + (hi_ ? Q_ * 4 : 0);
+      hi_base_ = hi_rows_ ? Q_ * 4 * kSlots : 0;
+      nbin_total_ = Q_ * 4 * kSlots + (hi_rows_ ? Q_ * 4 : 0);
       slab_entries_ = HistBlocks(Q_) * kBlockEntries;
     }
     // entries between the slabs of two work items: with ninth bits one more row, bin 256
-    slab_stride_ = wide_ ? slab_entries_ : HistBlocks(Q_) * (kBlockEntries + (hi_ ? kBlockFeatures : 0));
+    slab_stride_ = wide_ ? slab_entries_ : HistBlocks(Q_) * (kBlockEntries + (hi_rows_ ? kBlockFeatures : 0));
     if (cfg.objective >= kSoftMaxOneVsAll && K_ < 2) throw std::runtime_error("soft-max needs labels_count >= 2");
     if (cfg.objective < kSoftMaxOneVsAll && K_ != 1) throw std::runtime_error("labels_count must be 1 for this objective");
     const int last_nodes = 1 << (D_ - 2);
@@ -589,8 +602,10 @@ class HipTreeBuilder : public TreeBuilder {
     // the fused partition + histogram pass holds one histogram of all
     // features and builds only the smaller child
     single_group_ = Q_ <= quads_per_group_;
-    if (hi_ && (!single_group_ || HistLdsBytes(Q_, pair_, true) > kLdsBudget - 1024))
-      throw std::runtime_error("internal: ninth-bit ids need a matrix of one group of quads");
+    if (hi_rows_ && (!single_group_ || HistLdsBytes(Q_, pair_, true) > kLdsBudget - 1024))
+      throw std::runtime_error("internal: ninth-bit ids in a 257th row need a matrix of one group of quads");
+    if (hi_skip_ && !dm_->streamed && D_ > 2 && Q_ > 256)
+      throw std::runtime_error("more than 1024 features with 257 bin ids per feature: use hist_size 255");
     // Matrices wider than one group of quads: rows stay in place as records, only (row id,
     // gradients) are re-ordered (kernels_indexed.h).
     // Taken when every feature fits ONE LDS histogram of the bins in use (a record is then read
@@ -604,8 +619,10 @@ class HipTreeBuilder : public TreeBuilder {
     // 33: 2.10 / 2.40, 44: 2.24 / 2.53.  So rows stay in place from 48 features (twelve quads) on,
     // and at any width when one launch builds the whole histogram.
     const bool in_place_pays = rec_one_launch_ || Q_ >= 12;
+    // (with ninth bits in several words the rows always stay in place: the row-moving group passes do not carry them)
     indexed_ = !wide_ && !dm_->streamed && !single_group_ && D_ > 2 && Q_ <= 256 &&  // at most 64 pieces of 16 bytes per record
-               (cfg.internal.wide_rows_in_place >= 2 || (cfg.internal.wide_rows_in_place == 1 && in_place_pays));
+               (hi_skip_ || cfg.internal.wide_rows_in_place >= 2 ||
+                (cfg.internal.wide_rows_in_place == 1 && in_place_pays));
     // one launch: a power of two of blocks between the bins of the LDS image when that still fits
     rec_lay_blocks_ = 0;
     if (rec_one_launch_) {
@@ -673,12 +690,20 @@ class HipTreeBuilder : public TreeBuilder {
     }
     if (indexed_) {
       if (!dm_->rec) {  // records: whole 64-byte units (what memory answers a gather with), built once per matrix
-        dm_->RS = (Q_ + 15) / 16 * 16;
+        dm_->RS = (W_ + 15) / 16 * 16;  // (the ninth-bit words of a row follow its quads, in the columns and in the record)
         dm_->rec = DevAlloc<uint32_t>(n_ * (size_t)dm_->RS);
         AllowLds(k_to_records, (size_t)64 * (dm_->RS + 1) * sizeof(uint32_t));
         hipLaunchKernelGGL(k_to_records, dim3((unsigned)((n_ + 63) / 64)), dim3(256),
-                           (size_t)64 * (dm_->RS + 1) * sizeof(uint32_t), stream_, dm_->bins, stride_, Q_, dm_->rec,
+                           (size_t)64 * (dm_->RS + 1) * sizeof(uint32_t), stream_, dm_->bins, stride_, W_, dm_->rec,
                            dm_->RS, n_);
+        HIP_OK(hipGetLastError());
+      }
+      if (hi_skip_ && !dm_->hibits) {
+        dm_->strideb = (n_ + 7) / 8;
+        dm_->strideb = (dm_->strideb + 63) / 64 * 64;
+        dm_->hibits = DevAlloc<uint8_t>((size_t)F_ * dm_->strideb);
+        hipLaunchKernelGGL(k_to_hi_bits, dim3((unsigned)((n_ / 8 + 256) / 256)), dim3(256), 0, stream_,
+                           dm_->bins + (size_t)Q_ * stride_, stride_, F_, dm_->hibits, dm_->strideb, n_);
         HIP_OK(hipGetLastError());
       }
       if (!dm_->bytes) {
@@ -1066,19 +1091,22 @@ class HipTreeBuilder : public TreeBuilder {
         const bool pow2 = lay > 0 ? (lay & (lay - 1)) == 0
                                   : (pieces & (pieces - 1)) == 0 && (last_pieces & (last_pieces - 1)) == 0;
         const bool clamp = slots < kSlots;
-#define ARB_REC(P, POW2, CLAMP)                                                                                   \
+#define ARB_REC(P, POW2, CLAMP, H)                                                                                \
   do {                                                                                                            \
     static std::once_flag configured;                                                                             \
-    AllowLdsOnce(configured, (k_hist_rec<P, POW2, CLAMP>), kLdsBudget);                                           \
-    hipLaunchKernelGGL((k_hist_rec<P, POW2, CLAMP>), dim3(blocks), dim3(kHistThreads), lds, stream_, dm_->rec,    \
+    AllowLdsOnce(configured, (k_hist_rec<P, POW2, CLAMP, H>), kLdsBudget);                                        \
+    hipLaunchKernelGGL((k_hist_rec<P, POW2, CLAMP, H>), dim3(blocks), dim3(kHistThreads), lds, stream_, dm_->rec, \
                        dm_->RS, cur.ids, Q_, slots, cur.g, cur.h, d_shifts_, d_hwork_, d_nwork_, d_slab_, pieces, \
                        total, ngroups, item_words, lay);                                                          \
   } while (0)
-#define ARB_REC_P(P)                                      \
-  do {                                                    \
-    if (pow2 && clamp) ARB_REC(P, true, true);            \
-    else if (pow2) ARB_REC(P, true, false);               \
-    else ARB_REC(P, false, true);                         \
+#define ARB_REC_P(P)                                             \
+  do {                                                           \
+    if (hi_skip_ && pow2 && clamp) ARB_REC(P, true, true, true); \
+    else if (hi_skip_ && pow2) ARB_REC(P, true, false, true);    \
+    else if (hi_skip_) ARB_REC(P, false, true, true);            \
+    else if (pow2 && clamp) ARB_REC(P, true, true, false);       \
+    else if (pow2) ARB_REC(P, true, false, false);               \
+    else ARB_REC(P, false, true, false);                         \
   } while (0)
         if (pair_) ARB_REC_P(true);
         else ARB_REC_P(false);
@@ -1094,12 +1122,30 @@ class HipTreeBuilder : public TreeBuilder {
     if (timing_ && root) timings_.hist_root_rows += n_;
   }
 
+  // Gradient totals of the root: the sum over the slots of feature 0 of the root histogram, or, when
+  // ids of 256 are left out of the histograms, over the gradients themselves (tot[0].g / .h are
+  // zero: k_init_root).
+  void RootTotals(int hb, int state, const RowBuffers &orig) {
+    if (hi_skip_)
+      hipLaunchKernelGGL(k_sum_grad, dim3(GridFor(n_, 256, 2048)), dim3(256), 0, stream_, orig.g, pair_ ? orig.h : nullptr,
+                         n_, d_shifts_, d_tot_[state]);
+    else
+      hipLaunchKernelGGL(k_root_from_hist, dim3(1), dim3(64), 0, stream_, d_hg_[hb], d_hh_[hb], d_tot_[state], slots_,
+                         hi_base_);
+  }
+
   // k_hist over quads [q0, q0 + nq) of rows laid out with `stride` words between columns
   void HistLaunch(int nq, unsigned grid, const uint32_t *bins, size_t stride, int q0, const float *g, const float *h) {
-    if (hi_ && pair_)
-      LaunchHist<true, 1>(nq, stream_, grid, bins, stride, q0, F_, g, h, d_shifts_, d_hwork_, d_nwork_, d_slab_, slab_stride_);
-    else if (hi_)
-      LaunchHist<false, 1>(nq, stream_, grid, bins, stride, q0, F_, g, h, d_shifts_, d_hwork_, d_nwork_, d_slab_, slab_stride_);
+    // the ninth-bit words of the 32 features of a group of eight quads: column Q_ + q0 / 8
+    const uint32_t *hi_col = hi_ ? bins + (size_t)(Q_ + q0 / 8) * stride : nullptr;
+    if (hi_skip_ && pair_)
+      LaunchHist<true, 2>(nq, stream_, grid, bins, stride, q0, F_, g, h, d_shifts_, d_hwork_, d_nwork_, d_slab_, slab_stride_, hi_col);
+    else if (hi_skip_)
+      LaunchHist<false, 2>(nq, stream_, grid, bins, stride, q0, F_, g, h, d_shifts_, d_hwork_, d_nwork_, d_slab_, slab_stride_, hi_col);
+    else if (hi_rows_ && pair_)
+      LaunchHist<true, 1>(nq, stream_, grid, bins, stride, q0, F_, g, h, d_shifts_, d_hwork_, d_nwork_, d_slab_, slab_stride_, hi_col);
+    else if (hi_rows_)
+      LaunchHist<false, 1>(nq, stream_, grid, bins, stride, q0, F_, g, h, d_shifts_, d_hwork_, d_nwork_, d_slab_, slab_stride_, hi_col);
     else if (pair_)
       LaunchHist<true>(nq, stream_, grid, bins, stride, q0, F_, g, h, d_shifts_, d_hwork_, d_nwork_, d_slab_, slab_stride_);
     else
@@ -1135,7 +1181,7 @@ class HipTreeBuilder : public TreeBuilder {
     const int lay_blocks = indexed_ && rec_one_launch_ ? rec_lay_blocks_ : 0;
     // 16-bit bins: feature-major slabs; else the entries of the bins in use of every 16-feature block
     dim3 grid(wide_ ? (slab_entries_ + entries - 1) / entries
-                    : slab_entries_ / kBlockEntries * ((lds_slots * kBlockFeatures + entries - 1) / entries) + (hi_ ? 1 : 0),
+                    : slab_entries_ / kBlockEntries * ((lds_slots * kBlockFeatures + entries - 1) / entries) + (hi_rows_ ? 1 : 0),
               L);
     if (plan_state >= 0) grid.x += 1;
 #define ARB_REDUCE(P, LN)                                                                                          \
@@ -1180,7 +1226,7 @@ class HipTreeBuilder : public TreeBuilder {
     // one: logistic objective, gradients of the next round wanted, all quads in
     // one LDS histogram next to the node arrays.
     const bool next_grad = !inspect_ && K_ == 1;
-    const size_t final_lds = FinalHistLdsBytes(Q_, D_, hi_);
+    const size_t final_lds = FinalHistLdsBytes(Q_, D_, hi_rows_);
     const bool final_hist = next_grad && cfg_.objective == kLogisticRegression && single_group_ && !wide_ &&
                             final_lds <= kLdsBudget;
     int state = 0;  // d_tot_/d_seg_[state] describe the nodes of the current level
@@ -1194,8 +1240,7 @@ class HipTreeBuilder : public TreeBuilder {
         root_hist_ready_ = false;
         Reduce(1, hb, false, state, false, false, own_scan_ && !last ? state : -1);
         // (the last pass of the previous tree has also summed the root's totals)
-        if (!root_totals_ready_)
-          hipLaunchKernelGGL(k_root_from_hist, dim3(1), dim3(64), 0, stream_, d_hg_[hb], d_hh_[hb], d_tot_[state], slots_, hi_base_);
+        if (!root_totals_ready_) RootTotals(hb, state, orig);
         root_totals_ready_ = false;
       } else {
         // rows are in the order of level-1; the parents' state is state ^ 1
@@ -1232,8 +1277,8 @@ class HipTreeBuilder : public TreeBuilder {
                         q0, scan};
 #define ARB_FUSED(P, W)                                                       \
   do {                                                                        \
-    if (hi_ && P && pack_) LaunchFused<P, W, false, P, 1>(nq, stream_, grid, a); \
-    else if (hi_) LaunchFused<P, W, false, false, 1>(nq, stream_, grid, a);   \
+    if (hi_rows_ && P && pack_) LaunchFused<P, W, false, P, 1>(nq, stream_, grid, a); \
+    else if (hi_rows_) LaunchFused<P, W, false, false, 1>(nq, stream_, grid, a);   \
     else if (P && pack_ && single_group_) LaunchFused<P, W, false, P>(nq, stream_, grid, a); \
     else if (P && pack_) LaunchFused<P, W, true, P>(nq, stream_, grid, a);    \
     else if (single_group_) LaunchFused<P, W, false, false>(nq, stream_, grid, a); \
@@ -1261,11 +1306,11 @@ class HipTreeBuilder : public TreeBuilder {
             if (pair_)
               hipLaunchKernelGGL(k_ix_part<true>, dim3(grid), dim3(kHistThreads), 0, stream_, dm_->bytes, dm_->stride8,
                                  src.ids, dst.ids, src.g, dst.g, src.h, dst.h, d_split_, d_seg_[ps], d_pwork_,
-                                 d_nwork_ + 1, d_cursor2_, d_item_left_);
+                                 d_nwork_ + 1, d_cursor2_, d_item_left_, dm_->hibits, dm_->strideb);
             else
               hipLaunchKernelGGL(k_ix_part<false>, dim3(grid), dim3(kHistThreads), 0, stream_, dm_->bytes, dm_->stride8,
                                  src.ids, dst.ids, src.g, dst.g, src.h, dst.h, d_split_, d_seg_[ps], d_pwork_,
-                                 d_nwork_ + 1, d_cursor2_, d_item_left_);
+                                 d_nwork_ + 1, d_cursor2_, d_item_left_, dm_->hibits, dm_->strideb);
           } else {
             hipLaunchKernelGGL(k_part_count, dim3(grid), dim3(kHistThreads), 0, stream_, src.bins, stride_, d_split_,
                                d_pwork_, d_nwork_ + 1, d_wave_left_, d_item_left_, code_, hi_word_);
@@ -1275,7 +1320,7 @@ class HipTreeBuilder : public TreeBuilder {
           Reduce(L, hb, false, ps, trick_);
         }
       }
-      if (inspect_) KeepHist(level, L, hb);
+      if (inspect_) KeepHist(level, L, hb, state);
       // (own_scan_: only the scan; the pass of the next level selects the splits of this level's nodes)
       LaunchSplit(level, L, hb, state, gp, fused_ && !last, own_scan_ && !last);
       if (last && !final_hist) LaunchLeafWeights(L, state, gp);
@@ -1528,7 +1573,7 @@ class HipTreeBuilder : public TreeBuilder {
   } while (0)
 #define ARB_CASE(N)           \
   case N:                     \
-    if (hi_) ARB_FH(N, 1);    \
+    if (hi_rows_) ARB_FH(N, 1);    \
     else ARB_FH(N, 0);        \
     break;
     switch (Q_) {
@@ -1598,12 +1643,11 @@ class HipTreeBuilder : public TreeBuilder {
         if (in_place) DoneWithBlock(buf);
         Reduce(L, hb, false, state, false, b > 0);
       }
-      if (level == 0)
-        hipLaunchKernelGGL(k_root_from_hist, dim3(1), dim3(64), 0, stream_, d_hg_[hb], d_hh_[hb], d_tot_[state], slots_, hi_base_);
+      if (level == 0) RootTotals(hb, state, orig);
       if (trick)
         hipLaunchKernelGGL(k_sibling, dim3((nbin_total_ + 255) / 256, L), dim3(256), 0, stream_, d_hg_[hb], d_hh_[hb],
                            d_hc_[hb], d_hg_[hb ^ 1], d_hh_[hb ^ 1], d_hc_[hb ^ 1], d_tot_[state], level, nbin_total_);
-      if (inspect_) KeepHist(level, L, hb);
+      if (inspect_) KeepHist(level, L, hb, state);
       LaunchSplit(level, L, hb, state, gp);
       if (level + 2 >= D_) LaunchLeafWeights(L, state, gp);
       state ^= 1;
@@ -1648,7 +1692,7 @@ class HipTreeBuilder : public TreeBuilder {
     HIP_OK(hipMemcpy(d_active_, active_host_.data(), active_host_.size(), hipMemcpyHostToDevice));
   }
 
-  void KeepHist(int level, int L, int hb) {
+  void KeepHist(int level, int L, int hb, int state) {
     const size_t cells = (size_t)L * nbin_total_;
     std::vector<long long> g(cells), h(cells);
     std::vector<unsigned long long> c(cells);
@@ -1657,6 +1701,11 @@ class HipTreeBuilder : public TreeBuilder {
     HIP_OK(hipMemcpy(h.data(), d_hh_[hb], cells * sizeof(long long), hipMemcpyDeviceToHost));
     HIP_OK(hipMemcpy(c.data(), d_hc_[hb], cells * sizeof(unsigned long long), hipMemcpyDeviceToHost));
     // keep [node][F][slots][3] (padding features of the last quad dropped)
+    std::vector<NodeSum> tot;
+    if (hi_skip_) {  // ids of 256 were left out: a feature's bin 256 holds what its other bins lack of the node
+      tot.resize(L);
+      HIP_OK(hipMemcpy(tot.data(), d_tot_[state], (size_t)L * sizeof(NodeSum), hipMemcpyDeviceToHost));
+    }
     std::vector<int64_t> &out = kept_hist_[level];
     out.resize((size_t)L * F_ * report_slots_ * 3);
     for (int nd = 0; nd < L; ++nd)
@@ -1665,6 +1714,20 @@ class HipTreeBuilder : public TreeBuilder {
           // (ninth bits: bin 256 of feature f is cell hi_base_ + f of the node)
           const size_t s = (size_t)nd * nbin_total_ + (b < slots_ ? (size_t)f * slots_ + b : (size_t)hi_base_ + f);
           const size_t d = (((size_t)nd * F_ + f) * report_slots_ + b) * 3;
+          if (hi_skip_ && b >= slots_) {
+            long long sg = 0, sh = 0;
+            unsigned long long sc = 0;
+            for (int k = 0; k < slots_; ++k) {
+              const size_t e = (size_t)nd * nbin_total_ + (size_t)f * slots_ + k;
+              sg += g[e];
+              sh += pair_ ? h[e] : 0;
+              sc += c[e];
+            }
+            out[d] = tot[nd].g - sg;
+            out[d + 1] = pair_ ? tot[nd].h - sh : 0;
+            out[d + 2] = (int64_t)(tot[nd].c - sc);
+            continue;
+          }
           out[d] = g[s];
           out[d + 1] = pair_ ? h[s] : 0;
           out[d + 2] = c[s];
@@ -1686,7 +1749,9 @@ class HipTreeBuilder : public TreeBuilder {
   bool rec_one_launch_ = true;  // every feature fits one LDS histogram at rec_slots_ bins
   int rec_lay_blocks_ = 0;      // blocks that histogram is laid out for (a power of two), 0: as many as the matrix has
   bool wide_ = false;     // 16-bit bins: two features per word, slots_ histogram slots per feature
-  bool hi_ = false;       // 8-bit bins plus a ninth-bit word per row (ids up to 256)
+  bool hi_ = false;       // 8-bit bins plus ninth-bit words per row (ids up to 256)
+  bool hi_rows_ = false;  // ... one word: ids of 256 have a 257th row of entries in LDS histograms and slabs
+  bool hi_skip_ = false;  // ... several words: ids of 256 are left out of the histograms
   int W_ = 0;             // words of a row: Q_, one more with ninth bits
   int hi_word_ = -1;      // column of the ninth-bit word, -1: none
   int hi_base_ = 0;       // first cell of the bin-256 cells of a node's histogram, 0: none

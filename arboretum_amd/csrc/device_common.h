@@ -108,9 +108,10 @@ struct BinCode {
 // Bin id 256.  With hist_size 256 a feature that fills all 256 value bins and
 // also has missing values needs 257 ids (NaN -> bin `size`,
 // src/core/cuda_helpers.h:207-222).  Such an id is stored as byte 255 plus one
-// bit in an extra word of the row, the "ninth-bit word": bit f set means the id
-// of feature f is 256.  The word follows the quads of the row (column Q of a
-// matrix of Q quads, at most 32 features) and moves with them.
+// bit in an extra word of the row, a "ninth-bit word": bit f % 32 of word f / 32
+// set means the id of feature f is 256.  The words follow the quads of the row
+// (columns Q, Q + 1, ... of a matrix of Q quads; one word up to 32 features) and
+// move with them.
 //
 // The test "id > split bin" on one 32-bit word of a row:
 //   split bin < 255 (or no ninth bits): the feature's byte against the bin (an
@@ -123,10 +124,10 @@ struct SplitTest {
   int thr;
   __device__ __forceinline__ bool Right(uint32_t v) const { return (int)((v >> shift) & mask) > thr; }
 };
-// hi_word: column of the ninth-bit word, negative when the matrix has none
+// hi_word: column of the first ninth-bit word, negative when the matrix has none
 __device__ __forceinline__ SplitTest MakeSplitTest(const SplitRec &s, BinCode code, int hi_word) {
   if (s.fid < 0) return SplitTest{0, 0u, 0u, 0};
-  if (hi_word >= 0 && s.bin >= 255) return SplitTest{hi_word, (unsigned)s.fid, 1u, 0};
+  if (hi_word >= 0 && s.bin >= 255) return SplitTest{hi_word + (s.fid >> 5), (unsigned)(s.fid & 31), 1u, 0};
   return SplitTest{code.Word(s.fid), (unsigned)(code.bits * (s.fid & ((1 << code.wshift) - 1))),
                    (1u << code.bits) - 1u, s.bin};
 }

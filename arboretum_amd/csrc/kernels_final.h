@@ -112,8 +112,8 @@ k_tree_end(const SplitRec *__restrict__ split, const NodeSum *__restrict__ tot, 
 // NQ > 0: the matrix has NQ quads, all loaded up front (coalesced, independent
 // loads) and selected in registers; NQ == 0: any width, one dependent load per
 // level, from the byte columns when the matrix has them (bytes != null).
-// hi_word >= 0: column of the rows' ninth-bit word; a split at bin 255 sends
-// right only the rows whose id is 256 (SplitTest).
+// hi_word >= 0: column of the rows' first ninth-bit word; a split at bin 255
+// sends right only the rows whose id is 256 (SplitTest).
 template <int NEXT_GRAD, int NQ>
 __global__ void __launch_bounds__(256)
 k_final(const uint32_t *__restrict__ bins, size_t stride, const int *__restrict__ t_fid,
@@ -142,7 +142,7 @@ k_final(const uint32_t *__restrict__ bins, size_t stride, const int *__restrict_
       const int fid = s_nodes[id], bin = s_nodes[internal + id];
       unsigned right = 0;
       if (bin >= 255 && hi_word >= 0) {
-        right = (bins[(size_t)hi_word * stride + i] >> fid) & 1u;
+        right = (bins[(size_t)(hi_word + (fid >> 5)) * stride + i] >> (fid & 31)) & 1u;
       } else if (bin >= 0) {
         if (NQ > 0) {  // 8-bit bins, all quads in registers
           uint32_t b4 = 0;
@@ -348,7 +348,7 @@ k_leaf_ids(const uint32_t *__restrict__ bins, size_t stride, const int *__restri
       const int id = (1 << level) - 1 + (int)node;
       const int fid = t_fid[id], bin = t_bin[id];
       unsigned right = 0;
-      if (bin >= 255 && hi_word >= 0) right = (bins[(size_t)hi_word * stride + i] >> fid) & 1u;
+      if (bin >= 255 && hi_word >= 0) right = (bins[(size_t)(hi_word + (fid >> 5)) * stride + i] >> (fid & 31)) & 1u;
       else if (bin >= 0) right = (int)code.Bin(bins[(size_t)code.Word(fid) * stride + i], fid) > bin ? 1u : 0u;
       node = node * 2 + right;
     }

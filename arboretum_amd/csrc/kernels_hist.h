@@ -38,12 +38,15 @@ __host__ __device__ __forceinline__ unsigned HistWord(unsigned entry, int blocks
 // byte (t + l) % 4 of that quad, so the 16 lanes of a pass of the LDS atomic
 // touch 16 different features = 16 different bank pairs.  q_first: first quad
 // of this launch (a multiple of 4).
-// HI: b[NQ] is the row's ninth-bit word (bit f set: the id of feature f is
-// 256, its byte 255); such an id falls into the row of entries that follows bin
-// 255 in this bin-major layout, so the address arithmetic is the same.
+// HI: b[NQ] is the ninth-bit word of the row's features 4 q_first .. 4 q_first
+// + 31 (bit f set: the id of that feature is 256, its byte 255).  HI = 1: such
+// an id falls into the row of entries that follows bin 255 in this bin-major
+// layout, so the address arithmetic is the same.  HI = 2 (matrices of several
+// groups of quads): such an id is not accumulated at all; no split candidate's
+// left side holds it (candidates end at bin 255), so the scan never misses it.
 template <bool PAIR, int NQ, int HI = 0>
 __device__ __forceinline__ void AccumulateRow(unsigned long long *__restrict__ lds,
-                                              const uint32_t (&b)[NQ + HI], float gv, float hv, int sg,
+                                              const uint32_t (&b)[NQ + (HI != 0 ? 1 : 0)], float gv, float hv, int sg,
                                               int sh, int q_first, int F) {
   using L = HistLds<NQ>;
   const unsigned long long w0 = (1ull << kCountShift) + (unsigned long long)ToFixed(gv, sg);
@@ -67,12 +70,15 @@ __device__ __forceinline__ void AccumulateRow(unsigned long long *__restrict__ l
         const unsigned bi = ((unsigned)t + i) & 3u;  // byte of the quad
         unsigned bin = __builtin_amdgcn_ubfe(sel, 8u * bi, 8u);  // one v_bfe_u32
         const unsigned f16 = 4u * qi + bi;
-        if constexpr (HI != 0) bin += __builtin_amdgcn_ubfe(b[NQ], 16u * (unsigned)k + f16, 1u);
+        unsigned ninth = 0;
+        if constexpr (HI != 0) ninth = __builtin_amdgcn_ubfe(b[NQ], 16u * (unsigned)k + f16, 1u);
+        if constexpr (HI == 1) bin += ninth;
         // Quads past NQ do not exist.  Padding features of the last quad of
         // the matrix (bin 0 in every row) are accumulated like real ones into
         // slots nobody reads: cheaper than a per-update test.
         bool on = true;
         if (4 * k + 3 >= NQ) on = 4u * k + qi < (unsigned)NQ;
+        if constexpr (HI == 2) on = on && ninth == 0u;
         if (on) {
           constexpr unsigned per = PAIR ? 2 : 1;
           unsigned long long *cell = &lds[bin * (per * kBlockFeatures * L::blocks) + f16];
@@ -95,7 +101,7 @@ template <bool PAIR, int NQ, int HI = 0>
 __device__ __forceinline__ void FlushSlab(const unsigned long long *__restrict__ lds,
                                           unsigned long long *__restrict__ slab, unsigned w,
                                           int slab_entries, int q_first) {
-  constexpr int words = (int)(HistLdsBytes(NQ, PAIR, HI != 0) / 8);
+  constexpr int words = (int)(HistLdsBytes(NQ, PAIR, HI == 1) / 8);
   constexpr int per = PAIR ? 2 : 1;
   __syncthreads();
   unsigned long long *out =
@@ -106,18 +112,20 @@ __device__ __forceinline__ void FlushSlab(const unsigned long long *__restrict__
 // Histogram of contiguous row ranges: one workgroup per work item, quads
 // [q0, q0+NQ).  LDS: NQ*1024 word0 entries, then (PAIR) as many word1 entries.
 // PAIR with h == nullptr: g holds packed logistic gradients (PackGrad).
-// HI: the rows carry a ninth-bit word in column q0 + NQ.
+// HI: hi_col is the column of the ninth-bit words of features 4 q0 .. 4 q0 + 31
+// (AccumulateRow: 1 = accumulated in a 257th row of entries, 2 = skipped).
 template <bool PAIR, int NQ, int HI = 0>
 __global__ void __launch_bounds__(kHistThreads)
 k_hist(const uint32_t *__restrict__ bins, size_t stride, int q0, int F,
        const float *__restrict__ g, const float *__restrict__ h, const int *__restrict__ shifts,
        const WorkItem *__restrict__ work, const unsigned *__restrict__ n_work,
-       unsigned long long *__restrict__ slab, int slab_entries) {
+       unsigned long long *__restrict__ slab, int slab_entries, const uint32_t *__restrict__ hi_col = nullptr) {
   extern __shared__ unsigned long long lds[];
   const unsigned w = blockIdx.x;
   if (w >= *n_work) return;
   const WorkItem it = work[w];
-  constexpr int words = (int)(HistLdsBytes(NQ, PAIR, HI != 0) / 8);
+  constexpr int words = (int)(HistLdsBytes(NQ, PAIR, HI == 1) / 8);
+  constexpr int NH = HI != 0 ? 1 : 0;
   for (int i = threadIdx.x; i < words; i += kHistThreads) lds[i] = 0ull;
   __syncthreads();
   const int sg = shifts[0], sh = shifts[1];
@@ -126,11 +134,15 @@ k_hist(const uint32_t *__restrict__ bins, size_t stride, int q0, int F,
     const unsigned r0 = base + threadIdx.x, r1 = r0 + kHistThreads;
     const bool v0 = r0 < it.end, v1 = r1 < it.end;
     const unsigned a0 = v0 ? r0 : it.begin, a1 = v1 ? r1 : it.begin;
-    uint32_t b0[NQ + HI], b1[NQ + HI];
+    uint32_t b0[NQ + NH], b1[NQ + NH];
 #pragma unroll
-    for (int q = 0; q < NQ + HI; ++q) {
+    for (int q = 0; q < NQ; ++q) {
       b0[q] = __builtin_nontemporal_load(&bq[(size_t)q * stride + a0]);
       b1[q] = __builtin_nontemporal_load(&bq[(size_t)q * stride + a1]);
+    }
+    if constexpr (HI != 0) {
+      b0[NQ] = __builtin_nontemporal_load(&hi_col[a0]);
+      b1[NQ] = __builtin_nontemporal_load(&hi_col[a1]);
     }
     float g0 = g[a0], g1 = g[a1];
     float h0 = 0.0f, h1 = 0.0f;

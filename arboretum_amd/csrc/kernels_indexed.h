@@ -54,6 +54,47 @@ k_to_byte_columns(const uint32_t *__restrict__ bins, size_t stride, int Q, uint8
   }
 }
 
+// Ninth-bit words [H][stride] (bit f % 32 of word f / 32: the id of feature f is 256) -> bit
+// columns [F][strideb]: bit r % 8 of byte r / 8 of feature f's column, so that the partition can
+// gather the bit of one feature of a row with one byte fetch.
+__global__ void __launch_bounds__(256)
+k_to_hi_bits(const uint32_t *__restrict__ hi, size_t stride, int F, uint8_t *__restrict__ bits, size_t strideb,
+             size_t n) {
+  const size_t j = (size_t)blockIdx.x * 256 + threadIdx.x;  // byte of every column: rows 8 j .. 8 j + 7
+  if (j * 8 >= n) return;
+  for (int w = 0; w * 32 < F; ++w) {
+    uint32_t v[8];
+#pragma unroll
+    for (int k = 0; k < 8; ++k) v[k] = j * 8 + k < n ? hi[(size_t)w * stride + j * 8 + k] : 0u;
+    for (int b = 0; b < 32 && w * 32 + b < F; ++b) {
+      unsigned byte = 0;
+#pragma unroll
+      for (int k = 0; k < 8; ++k) byte |= ((v[k] >> b) & 1u) << k;
+      bits[(size_t)(w * 32 + b) * strideb + j] = (uint8_t)byte;
+    }
+  }
+}
+
+// Sum of the fixed-point gradients of all rows: the totals of the root when no feature's
+// histogram holds every row (ids of 256 are left out of the histograms of matrices with several
+// ninth-bit words).  tot[0].g / .h must be zero at launch; integer sums, any order.
+__global__ void __launch_bounds__(256)
+k_sum_grad(const float *__restrict__ g, const float *__restrict__ h, size_t n, const int *__restrict__ shifts,
+           NodeSum *__restrict__ tot) {
+  const int sg = shifts[0], sh = shifts[1];
+  long long a = 0, b = 0;
+  for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (size_t)gridDim.x * blockDim.x) {
+    a += ToFixed(g[i], sg);
+    if (h != nullptr) b += ToFixed(h[i], sh);
+  }
+  a = WaveSumLL(a);
+  b = WaveSumLL(b);
+  if ((threadIdx.x & 63) == 0) {
+    atomicAdd(reinterpret_cast<unsigned long long *>(&tot[0].g), (unsigned long long)a);
+    if (h != nullptr) atomicAdd(reinterpret_cast<unsigned long long *>(&tot[0].h), (unsigned long long)b);
+  }
+}
+
 // Partition of (row id, gradients) of the parents of a level into the children order, one launch
 // per level, rows in place.  ids: the row at each position (null: position = row, the first
 // level).  Each wave first decides its own rows: the split feature's bin of a row is read from
@@ -66,6 +107,8 @@ k_to_byte_columns(const uint32_t *__restrict__ bins, size_t stride, int Q, uint8
 // them) and the waves move their rows through the register queues of the row passes: the bin
 // is gathered once, and no decision array or counting launch exists.  Within a child the work
 // items lie in the order of their claims; no result depends on it (integer sums).
+// hibits (may be null): bit columns of the ninth bits (k_to_hi_bits); a split at bin 255 sends
+// right exactly the rows whose id is 256.
 constexpr int kIxChunks = (int)(kPartRows / kChunkStep);  // chunks of a wave in one work item
 static_assert(kIxChunks * 2 <= 32, "a lane's decisions of one work item must fit one register");
 template <bool PAIR>
@@ -74,7 +117,8 @@ k_ix_part(const uint8_t *__restrict__ bytes, size_t stride8, const unsigned *__r
           unsigned *__restrict__ ids_out, const float *__restrict__ g, float *__restrict__ g_out,
           const float *__restrict__ h, float *__restrict__ h_out, const SplitRec *__restrict__ split,
           const unsigned *__restrict__ seg_start, const WorkItem *__restrict__ work,
-          const unsigned *__restrict__ n_work, unsigned *__restrict__ cursor, unsigned *__restrict__ item_base) {
+          const unsigned *__restrict__ n_work, unsigned *__restrict__ cursor, unsigned *__restrict__ item_base,
+          const uint8_t *__restrict__ hibits, size_t strideb) {
   __shared__ unsigned s_tmp[kItemWaves + 2];
   const unsigned w = blockIdx.x;
   if (w >= *n_work) return;
@@ -82,7 +126,8 @@ k_ix_part(const uint8_t *__restrict__ bytes, size_t stride8, const unsigned *__r
   const SplitRec s = split[it.node];
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const unsigned wb = ChunkOrigin(it) + wave * kChunkRows, we = it.end;
-  const uint8_t *col = bytes + (size_t)(s.fid < 0 ? 0 : s.fid) * stride8;
+  const bool by_bit = hibits != nullptr && s.bin >= 255;  // uniform: only an id of 256 goes right
+  const uint8_t *col = by_bit ? hibits + (size_t)s.fid * strideb : bytes + (size_t)(s.fid < 0 ? 0 : s.fid) * stride8;
   // decisions of this lane's rows: bit 2 k + half = row (chunk k, half) goes right
   unsigned right_bits = 0, lefts = 0;
   if (s.fid >= 0) {
@@ -98,12 +143,12 @@ k_ix_part(const uint8_t *__restrict__ bytes, size_t stride8, const unsigned *__r
           id[k] = ids ? ids[a] : a;
         }
 #pragma unroll
-        for (int k = 0; k < 2 * kBatch; ++k) bin[k] = col[id[k]];
+        for (int k = 0; k < 2 * kBatch; ++k) bin[k] = by_bit ? (col[id[k] >> 3] >> (id[k] & 7u)) & 1u : col[id[k]];
 #pragma unroll
         for (int k = 0; k < 2 * kBatch; ++k) {
           const unsigned r = wb + (unsigned)(k0 + (k >> 1)) * kChunkStep + (k & 1) * 64 + lane;
           const bool valid = r >= it.begin && r < we;
-          const bool right = (int)bin[k] > s.bin;  // builder.h:107-123
+          const bool right = by_bit ? bin[k] != 0u : (int)bin[k] > s.bin;  // builder.h:107-123
           right_bits |= (valid && right ? 1u : 0u) << (2 * k0 + k);
           lefts += valid && !right ? 1u : 0u;
         }
@@ -193,7 +238,9 @@ k_ix_part(const uint8_t *__restrict__ bytes, size_t stride8, const unsigned *__r
 // feature, bin ids are clamped to the histogram (with 256 no bin id can leave it).
 // lay_blocks: 16-feature blocks the image is laid out for (0: the pieces of the workgroup's
 // group); more than the matrix has makes the stride a power of two.
-template <bool PAIR, bool POW2 = false, bool CLAMP = true>
+// HI: words Q, Q + 1, ... of a record are the row's ninth-bit words; a feature whose bit is set
+// (id 256) is not accumulated (AccumulateRow, HI = 2).
+template <bool PAIR, bool POW2 = false, bool CLAMP = true, bool HI = false>
 __global__ void __launch_bounds__(kHistThreads)
 k_hist_rec(const uint32_t *__restrict__ rec, int RS, const unsigned *__restrict__ ids, int Q, int slots,
            const float *__restrict__ g, const float *__restrict__ h, const int *__restrict__ shifts,
@@ -240,6 +287,7 @@ k_hist_rec(const uint32_t *__restrict__ rec, int RS, const unsigned *__restrict_
     uint4 q[kSteps];
     float gv[kSteps], hv[kSteps];
     unsigned piece[kSteps];
+    unsigned ninth[kSteps];  // HI: the ninth bits of the piece's 16 features
     bool v[kSteps];
   };
   // position in the item's row range and piece of this lane's pair in group k of the step at `first`
@@ -265,6 +313,12 @@ k_hist_rec(const uint32_t *__restrict__ rec, int RS, const unsigned *__restrict_
     for (int k = 0; k < kSteps; ++k) {
       const unsigned a = locate(first, k, &R.piece[k], &R.v[k]);
       R.q[k] = *reinterpret_cast<const uint4 *>(rec + (size_t)I.id[k] * RS + 4u * ((unsigned)piece0 + R.piece[k]));
+      if (HI) {
+        const unsigned p = (unsigned)piece0 + R.piece[k];
+        R.ninth[k] = (rec[(size_t)I.id[k] * RS + (unsigned)Q + (p >> 1)] >> (16u * (p & 1u))) & 0xffffu;
+      } else {
+        R.ninth[k] = 0u;
+      }
       R.gv[k] = g[a];
       R.hv[k] = PAIR ? h[a] : 0.0f;
     }
@@ -301,6 +355,7 @@ k_hist_rec(const uint32_t *__restrict__ rec, int RS, const unsigned *__restrict_
             if (POW2) off = (bin << stride_shift) + (piece_b + (4u * qi + bi) * 8u);
             else off = __umul24(bin, bin_stride_b) + (piece_b + (4u * qi + bi) * 8u);
             unsigned long long *cell = reinterpret_cast<unsigned long long *>(lds_b + off);
+            if (HI && ((R.ninth[k] >> (4u * qi + bi)) & 1u)) continue;  // id 256: in no candidate's left side
             atomicAdd(cell, w0);
             if (PAIR) atomicAdd(cell + kWord1, w1);
           }

@@ -26,21 +26,22 @@ void AllowLdsOnce(std::once_flag &flag, K kernel, size_t bytes) {
 template <bool PAIR, int NQ, int HI = 0>
 void LaunchHistNQ(hipStream_t st, unsigned grid, const uint32_t *bins, size_t stride, int q0, int F,
                   const float *g, const float *h, const int *shifts, const WorkItem *work,
-                  const unsigned *n_work, unsigned long long *slab, int slab_entries) {
-  const size_t lds = HistLdsBytes(NQ, PAIR, HI != 0);
+                  const unsigned *n_work, unsigned long long *slab, int slab_entries, const uint32_t *hi_col) {
+  const size_t lds = HistLdsBytes(NQ, PAIR, HI == 1);
   static std::once_flag configured;
   AllowLdsOnce(configured, k_hist<PAIR, NQ, HI>, lds);
   hipLaunchKernelGGL((k_hist<PAIR, NQ, HI>), dim3(grid), dim3(kHistThreads), lds, st, bins, stride, q0, F, g, h,
-                     shifts, work, n_work, slab, slab_entries);
+                     shifts, work, n_work, slab, slab_entries, hi_col);
 }
 
-// HI: the rows carry a ninth-bit word behind their nq quads (one launch for the whole matrix)
+// HI: hi_col holds the ninth-bit words of the features of this launch (k_hist)
 template <bool PAIR, int HI = 0>
 void LaunchHist(int nq, hipStream_t st, unsigned grid, const uint32_t *bins, size_t stride, int q0, int F,
                 const float *g, const float *h, const int *shifts, const WorkItem *work,
-                const unsigned *n_work, unsigned long long *slab, int slab_entries) {
+                const unsigned *n_work, unsigned long long *slab, int slab_entries,
+                const uint32_t *hi_col = nullptr) {
 #define ARB_CASE(N) \
-  case N: LaunchHistNQ<PAIR, N, HI>(st, grid, bins, stride, q0, F, g, h, shifts, work, n_work, slab, slab_entries); break;
+  case N: LaunchHistNQ<PAIR, N, HI>(st, grid, bins, stride, q0, F, g, h, shifts, work, n_work, slab, slab_entries, hi_col); break;
   switch (nq) {
     ARB_CASE(1) ARB_CASE(2) ARB_CASE(3) ARB_CASE(4) ARB_CASE(5) ARB_CASE(6) ARB_CASE(7) ARB_CASE(8)
     default: throw std::runtime_error("internal: bad quad count");

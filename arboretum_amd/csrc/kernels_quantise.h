@@ -11,8 +11,9 @@ namespace {
 // +INF above (src/core/cuda_helpers.h:207-222, src/io/io.cu:297-302); NaN
 // compares false everywhere and lands in bin `size`.
 // An id of 256 (a feature of 256 value bins with missing values) is stored as
-// byte 255 plus bit f0 + c of hi[r], the row's ninth-bit word (f0: the matrix
-// feature of column 0 of this launch); without `hi` no id may exceed 255.
+// byte 255 plus bit f0 + c of hi[r], the ninth-bit word of the row that holds
+// the features of this launch (f0: the place in that word of column 0 of this
+// launch); without `hi` no id may exceed 255.
 __global__ void k_bin_assign(const float *__restrict__ x, int ncols, const float *__restrict__ thr,
                              int thr_stride, const int *__restrict__ sizes,
                              uint32_t *__restrict__ out, size_t n, uint32_t *__restrict__ hi, int f0) {

@@ -1,8 +1,7 @@
 """hist_size 256 on a feature that fills all 256 value bins AND has missing values: 257 bin ids
 (NaN -> bin `size`, src/core/cuda_helpers.h:207-222; the reference switches to 16-bit ids at this
 hist_size, src/core/garden.cu:514-523).  The HIP path keeps 8-bit ids plus a ninth bit per feature
-for matrices of at most 32 features and must equal the CPU checker bit for bit on every path that
-reads a row: fused levels, the last level, the last pass with and without the next root histogram,
+and must equal the CPU checker bit for bit on every path that reads a row: fused levels, the last level, the last pass with and without the next root histogram,
 un-fused levels (no sibling subtraction), streamed blocks.  Needs an MI355X: run with `-m gpu`."""
 import numpy as np
 import pytest
@@ -107,7 +106,7 @@ def test_ninth_bit_ids_softmax(arb, oracle):
 
 def test_one_missing_value_keeps_the_headline_kernels(arb, oracle):
     # a single NaN in one of 28 continuous features: still 8-bit ids (with the ninth bit), same trees
-    # as the checker; a matrix wider than 32 features falls back to 16-bit ids
+    # as the checker; the same for a matrix wider than 32 features
     X, y = _data(50000, 28, 1, seed=21, nan_rows=0, informative_nan=False)
     X[123, 4] = np.nan
     ob, g = assert_same_training(arb, oracle, X, y, _cfg(1, 6), rounds=2, check_hist=False)
@@ -116,7 +115,52 @@ def test_one_missing_value_keeps_the_headline_kernels(arb, oracle):
     Xw[5, 7] = np.nan
     yw = (Xw[:, 0] > 0).astype(np.float32)
     ob, g = assert_same_training(arb, oracle, Xw, yw, _cfg(1, 3), rounds=1, check_hist=False)
-    assert g.data.bin_layout()[0] == 16
+    assert g.data.bin_layout() == (8, 257)
+
+
+@pytest.mark.parametrize("objective", [0, 1])
+@pytest.mark.parametrize("F,depth", [(33, 5), (40, 1), (64, 4), (100, 5), (130, 3)])
+def test_ninth_bit_ids_wide_matrices(arb, oracle, objective, F, depth):
+    # more than 32 features: a ninth-bit word per 32 features, rows in place as records (the words
+    # ride in the record), ids of 256 left out of the histograms (no candidate's left side holds
+    # them) and reported from the node totals; max_depth 1 takes the column kernels alone
+    X, y = _data(30000, F, objective, seed=100 + F)
+    ob, g = assert_same_training(arb, oracle, X, y, _cfg(objective, depth), rounds=2)
+    assert g.data.bin_layout() == (8, 257)
+    assert ob.bins().max() == 256
+    assert g.tree(0)["quantized"][0] == 255
+    assert_same_training(arb, oracle, X, y, _cfg(objective, depth, trick=False), rounds=2, check_hist=False)
+
+
+@pytest.mark.parametrize("resident", [0, -1])
+def test_ninth_bit_ids_wide_matrices_streamed(arb, oracle, resident):
+    X, y = _data(30000, 70, 1, seed=170)
+    cfg = _cfg(1, 4, upload=False, stream_block_rows=8192, stream_resident_bytes=resident)
+    ob, g = assert_same_training(arb, oracle, X, y, cfg, rounds=2)
+    assert g.data.bin_layout() == (8, 257)
+    assert g.tree(0)["quantized"][0] == 255
+
+
+def test_ninth_bit_ids_wide_softmax(arb, oracle):
+    rng = np.random.default_rng(12)
+    n, F, K = 20000, 48, 3
+    X = rng.normal(size=(n, F)).astype(np.float32)
+    labels = np.argmax(X[:, :K] + rng.gumbel(size=(n, K)), axis=1).astype(np.uint8)
+    X[rng.choice(n, size=25, replace=False), 40] = np.nan
+    cfg = _cfg(4, 4)
+    cfg["tree"]["labels_count"] = K
+    ob = oracle.Booster(X, labels=labels, config=cfg)
+    data = arb.DMatrix(X, labels=labels)
+    g = arb.Garden(cfg, data)
+    for r in range(2):
+        ob.grow(1)
+        g.grow_tree()
+    assert data.bin_layout() == (8, 257)
+    for t in range(2 * K):
+        a, b = ob.tree(t), g.tree(t)
+        for k in ("fid", "quantized", "threshold", "gain", "weights"):
+            assert np.array_equal(a[k], b[k]), (t, k)
+    assert np.array_equal(ob.yhat(), g.train_yhat())
 
 
 def test_no_missing_values_no_ninth_bit(arb, oracle):
