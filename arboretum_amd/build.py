@@ -8,7 +8,7 @@ HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(HERE, "csrc")
 OBJ = os.path.join(HERE, "build")
 LIB = os.path.join(HERE, "libarboretum.so")
-SOURCES = ["device_builder.hip", "hist_sum.hip", "quantiser.hip", "predictor.hip", "booster.cpp", "config.cpp",
+SOURCES = ["device_builder.hip", "exact_builder.hip", "hist_sum.hip", "quantiser.hip", "predictor.hip", "booster.cpp", "config.cpp",
            "wrapper.cpp"]
 # -ffp-contract=off: the gain arithmetic must round exactly like the host
 # restatement (no fused multiply-add).  packed-fp32-ops is switched off

@@ -36,6 +36,7 @@ DataMatrix::DataMatrix(size_t rows, size_t columns, size_t columns_category)
 
 DataMatrix::~DataMatrix() {
   if (device) FreeDeviceMatrix(device);
+  if (exact_sort) FreeExactSortData(exact_sort);
 }
 
 RegTree::RegTree(unsigned depth, unsigned label) : depth(depth), label(label) {
@@ -169,7 +170,7 @@ void Garden::GrowTree(DataMatrix *data, const float *grad) {
     // upload_features = false keeps the bins in pinned host memory and streams
     // them (src/core/garden.cu:603-604, hist_tree_grower.cu:335-366)
     QuantiseOnDevice(data, cfg.internal.hist_size, cfg.verbose.data, !cfg.internal.upload_features,
-                     cfg.internal.stream_block_rows, cfg.method == kExact);
+                     cfg.internal.stream_block_rows, cfg.method == kExact, cfg.internal.exact_sort);
     builder_.reset(CreateTreeBuilder(cfg, data));
     builder_->SetInspect(inspect_);
     builder_->EnableTiming(timing_);

@@ -19,6 +19,7 @@ namespace arb {
 void ParallelFor(size_t n, const std::function<void(size_t, size_t)> &fn);
 
 struct DeviceMatrix;  // quantised bins resident in HBM (device_builder.hip)
+struct ExactSortData;  // ranks and sorted row lists of every feature (exact_builder.hip)
 
 class DataMatrix {
  public:
@@ -54,6 +55,9 @@ class DataMatrix {
   std::vector<int> reduced_size;
   int max_bin = 255;  // largest bin id in the quantised matrix (the missing-value bin included)
   DeviceMatrix *device = nullptr;
+  // Exact method over sorted row lists (features with more distinct values than a histogram
+  // holds): set instead of `device`.
+  ExactSortData *exact_sort = nullptr;
   // Streamed matrices (bins in pinned host blocks instead of HBM): block b
   // holds rows [b * stream_block_rows, ...) as quads [Q][stream_block_rows].
   std::vector<uint32_t *> stream_blocks;
@@ -137,10 +141,15 @@ void DeviceThresholds(SortWorkspace *ws, const float *d_col, std::vector<float> 
 // device_builder.hip
 // streamed = false: bins resident in HBM; true: bins in pinned host blocks of
 // block_rows rows, copied to the GPU block by block at every tree level.
-// exact: no quantisation, every distinct value of a feature is a bin (the exact method;
-// at most 4096 distinct values per feature).
+// exact: no quantisation, every distinct value of a feature is a bin (the exact method).  Up to
+// 4096 distinct values per feature the ranks are bin ids of the histogram kernels; beyond that,
+// or always with exact_sort > 0, the matrix is kept as sorted row lists per feature
+// (exact_builder.hip); exact_sort == 0 makes more than 4096 distinct values an error.
 void QuantiseOnDevice(DataMatrix *data, int hist_size, bool verbose, bool streamed = false,
-                      size_t block_rows = 0, bool exact = false);
+                      size_t block_rows = 0, bool exact = false, int exact_sort = -1);
+void PrepareExactSort(DataMatrix *data);
+void FreeExactSortData(ExactSortData *d);
+TreeBuilder *CreateExactSortBuilder(const Configuration &cfg, DataMatrix *data);
 void FreeDeviceMatrix(DeviceMatrix *m);
 void GetDeviceBins(const DataMatrix &data, uint8_t *out);  // row-major [rows][F], 8-bit bins
 void GetDeviceBins16(const DataMatrix &data, uint16_t *out);  // row-major [rows][F], 16-bit bins

@@ -55,6 +55,8 @@ Configuration Configuration::Parse(const char *text) {
     GetNum(*v, "stream_resident_bytes", &cfg.internal.stream_resident_bytes);
     if (const json::Value *w = v->find("wide_rows_in_place"))
       cfg.internal.wide_rows_in_place = w->is_number() ? (int)w->number() : (w->boolean() ? 1 : 0);
+    if (const json::Value *w = v->find("exact_sort"))
+      cfg.internal.exact_sort = w->is_number() ? (int)w->number() : (w->boolean() ? 1 : 0);
   }
   return cfg;
 }

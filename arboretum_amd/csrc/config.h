@@ -62,6 +62,10 @@ struct InternalConfiguration {  // param.h:54-64
   // LDS histogram); false selects the row-moving passes, the number 2 rows in
   // place for every width above 32 features.
   int wide_rows_in_place = 1;
+  // Extension, exact method: features with more than 4096 distinct values are grown over sorted
+  // row lists instead of rank histograms (-1, the default); 1: every matrix is; 0: never (such
+  // features are an error).
+  int exact_sort = -1;
 };
 
 struct Configuration {  // param.h:66-74

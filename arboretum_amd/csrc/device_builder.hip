@@ -141,7 +141,9 @@ void FreeDeviceMatrix(DeviceMatrix *m) {
 // among the sorted distinct values of its column.  Returns the ranks row-major [rows][F] and
 // fills data->thresholds / reduced_size: the split "ranks <= q left" separates at the value
 // of rank q + 1 (the smallest value that goes right, src/core/garden.cu:463-467).
-static std::vector<uint16_t> ExactRanks(DataMatrix *data, size_t *most_distinct) {
+// A feature with more distinct values than the histograms hold: an error, or with allow_more an
+// empty result (the caller then keeps sorted row lists instead of bin ids).
+static std::vector<uint16_t> ExactRanks(DataMatrix *data, size_t *most_distinct, bool allow_more) {
   const size_t n = data->rows;
   const int F = (int)data->columns_dense;
   std::vector<uint16_t> ranks(n * F);
@@ -167,10 +169,15 @@ static std::vector<uint16_t> ExactRanks(DataMatrix *data, size_t *most_distinct)
     }
   });
   if (has_nan) throw std::runtime_error("the exact method does not take missing values (NaN); use method 1 (hist)");
-  if (too_many >= 0)
+  if (too_many >= 0) {
+    if (allow_more) {
+      *most_distinct = (size_t)kMaxWideSlots + 1;
+      return {};
+    }
     throw std::runtime_error("the exact method handles up to " + std::to_string(kMaxWideSlots) +
-                             " distinct values per feature; feature " + std::to_string((int)too_many) +
-                             " has more: use method 1 (hist)");
+                             " distinct values per feature without internals.exact_sort; feature " +
+                             std::to_string((int)too_many) + " has more: use method 1 (hist)");
+  }
   size_t most = 1;
   for (int f = 0; f < F; ++f) most = std::max(most, mapping[f].size());
   *most_distinct = most;
@@ -182,7 +189,8 @@ static std::vector<uint16_t> ExactRanks(DataMatrix *data, size_t *most_distinct)
   return ranks;
 }
 
-void QuantiseOnDevice(DataMatrix *data, int hist_size, bool verbose, bool streamed, size_t block_rows, bool exact) {
+void QuantiseOnDevice(DataMatrix *data, int hist_size, bool verbose, bool streamed, size_t block_rows, bool exact,
+                      int exact_sort) {
   if (data->quantised) {
     if (data->quantised_exact != exact) throw std::runtime_error("data matrix was prepared for the other method");
     if (!exact && data->hist_size != hist_size) throw std::runtime_error("data matrix was quantised with another hist_size");
@@ -268,7 +276,15 @@ void QuantiseOnDevice(DataMatrix *data, int hist_size, bool verbose, bool stream
 
   if (exact) {
     size_t most = 1;
-    std::vector<uint16_t> ranks = ExactRanks(data, &most);
+    std::vector<uint16_t> ranks;
+    if (exact_sort <= 0) ranks = ExactRanks(data, &most, exact_sort < 0);
+    if (ranks.empty()) {
+      // sorted row lists per feature instead of bin ids (exact_builder.hip)
+      if (streamed) throw std::runtime_error("the exact method over sorted row lists is not built for streamed matrices");
+      dm.reset();
+      PrepareExactSort(data);
+      return;
+    }
     hist_size = (int)most;
     if (most <= (size_t)kSlots) {
       // 8-bit ids: through the pre-quantised path below
@@ -444,6 +460,7 @@ void QuantiseOnDevice(DataMatrix *data, int hist_size, bool verbose, bool stream
 }
 
 void GetBinLayout(const DataMatrix &data, int *bits, int *slots) {
+  if (data.exact_sort) throw std::runtime_error("the matrix is kept as sorted row lists (exact method): it has no bin ids");
   const DeviceMatrix *dm = data.device;
   if (!dm) throw std::runtime_error("data matrix is not quantised");
   *bits = dm->bits;
@@ -1821,6 +1838,7 @@ class HipTreeBuilder : public TreeBuilder {
 }  // namespace
 
 TreeBuilder *CreateTreeBuilder(const Configuration &cfg, DataMatrix *data) {
+  if (data->exact_sort) return CreateExactSortBuilder(cfg, data);
   if (!data->device) throw std::runtime_error("data matrix is not quantised");
   return new HipTreeBuilder(cfg, data);
 }

@@ -1,0 +1,340 @@
+// Exact method over sorted row lists: features with more distinct values than a histogram holds.
+//
+// Every feature keeps the rows of every node of the current level as one list of row ids in
+// ascending order of the feature's value (the reference sorts every column once and keeps the
+// node segments sorted, src/core/continuous_tree_grower.cu).  Per level and feature: the running
+// sums of the gradients along the list give, at every place where the value changes, the
+// candidate "values up to here go left"; the best one per (node, feature) goes to the same
+// selection as the histogram method's candidates, and a stable partition by the selected splits
+// turns the lists of the parents into the lists of the children.
+//
+// The candidates are those of a histogram with one slot per distinct value (rank): a slot that
+// is empty in a node has the gain of the slot before it, and ties go to the highest slot
+// (builder.h:39-49), so the candidate between two neighbouring values of a node is the slot just
+// below the upper one, and its threshold is that upper value: the smallest value that goes right.
+#ifndef ARBORETUM_AMD_KERNELS_EXACT_H_
+#define ARBORETUM_AMD_KERNELS_EXACT_H_
+#include "device_common.h"
+#include "gain.h"
+#include "kernels_split.h"
+
+namespace arb {
+namespace {
+
+constexpr int kExThreads = 256;
+constexpr int kExPer = 8;                          // list places per thread
+constexpr unsigned kExItem = kExThreads * kExPer;  // list places per work item
+
+struct ExSum {
+  long long g, h;
+};
+__device__ __forceinline__ ExSum operator+(const ExSum &a, const ExSum &b) { return ExSum{a.g + b.g, a.h + b.h}; }
+__device__ __forceinline__ ExSum ExShflUp(const ExSum &v, int off) {
+  return ExSum{__shfl_up(v.g, off), __shfl_up(v.h, off)};
+}
+__device__ __forceinline__ unsigned ExShflUp(unsigned v, int off) { return __shfl_up(v, off); }
+__device__ __forceinline__ ExSum ExZero(const ExSum *) { return ExSum{0, 0}; }
+__device__ __forceinline__ unsigned ExZero(const unsigned *) { return 0u; }
+
+// Inclusive scan over the workgroup's threads (kExThreads of them) of one value per thread;
+// *total: the sum over all threads.  s_wave: kExThreads / 64 entries.
+template <typename T>
+__device__ __forceinline__ T ExBlockScan(T v, T *s_wave, T *total) {
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  for (int off = 1; off < 64; off <<= 1) {
+    const T o = ExShflUp(v, off);
+    if (lane >= off) v = v + o;
+  }
+  __syncthreads();  // s_wave may still be read from a scan before
+  if (lane == 63) s_wave[wave] = v;
+  __syncthreads();
+  T before = ExZero((const T *)nullptr), all = ExZero((const T *)nullptr);
+  for (int w = 0; w < kExThreads / 64; ++w) {
+    if (w < wave) before = before + s_wave[w];
+    all = all + s_wave[w];
+  }
+  *total = all;
+  return before + v;
+}
+
+// The fixed-point gradients of the rows at the places [p0, p0 + kExPer) of a list, zero past `end`.
+template <bool PAIR>
+__device__ __forceinline__ void ExLoadSums(const unsigned *__restrict__ list, const float *__restrict__ g,
+                                           const float *__restrict__ h, unsigned p0, unsigned end, int sg, int sh,
+                                           ExSum *v) {
+#pragma unroll
+  for (int j = 0; j < kExPer; ++j) {
+    v[j] = ExSum{0, 0};
+    if (p0 + j < end) {
+      const unsigned id = list[p0 + j];
+      v[j].g = ToFixed(g[id], sg);
+      if (PAIR) v[j].h = ToFixed(h[id], sh);
+    }
+  }
+}
+
+// grid (items, F): the sum of the gradients over every work item's piece of every feature's list.
+template <bool PAIR>
+__global__ void __launch_bounds__(kExThreads)
+k_ex_partial(const unsigned *__restrict__ lists, size_t stride, const float *__restrict__ g,
+             const float *__restrict__ h, const int *__restrict__ shifts, const WorkItem *__restrict__ work,
+             const unsigned *__restrict__ n_work, ExSum *__restrict__ part, unsigned max_items) {
+  __shared__ ExSum s_wave[kExThreads / 64];
+  const unsigned w = blockIdx.x, f = blockIdx.y;
+  if (w >= *n_work) return;
+  const WorkItem it = work[w];
+  ExSum v[kExPer];
+  ExLoadSums<PAIR>(lists + (size_t)f * stride, g, h, it.begin + threadIdx.x * kExPer, it.end, shifts[0], shifts[1], v);
+  ExSum mine = v[0];
+#pragma unroll
+  for (int j = 1; j < kExPer; ++j) mine = mine + v[j];
+  ExSum total;
+  ExBlockScan(mine, s_wave, &total);
+  if (threadIdx.x == 0) part[(size_t)f * max_items + w] = total;
+}
+
+// grid (L, F), one wave: exclusive scan of `part` over the work items of every node, per feature.
+template <typename T>
+__global__ void __launch_bounds__(64)
+k_ex_offsets(const T *__restrict__ part, T *__restrict__ off, const unsigned *__restrict__ node_first,
+             const unsigned *__restrict__ node_items, unsigned max_items) {
+  const unsigned nd = blockIdx.x, f = blockIdx.y, lane = threadIdx.x;
+  const unsigned first = node_first[nd];
+  unsigned cnt = node_items[nd];
+  if (cnt == 0xffffffffu) cnt = 0;
+  T carry = ExZero((const T *)nullptr);
+  for (unsigned base = 0; base < cnt; base += 64) {
+    const unsigned k = base + lane;
+    const T own = k < cnt ? part[(size_t)f * max_items + first + k] : ExZero((const T *)nullptr);
+    T v = own;
+    for (int o = 1; o < 64; o <<= 1) {
+      const T up = ExShflUp(v, o);
+      if ((int)lane >= o) v = v + up;
+    }
+    // exclusive: the sum of the items before this one
+    T excl = carry;
+    {
+      const T prev = ExShflUp(v, 1);
+      if (lane > 0) excl = excl + prev;
+    }
+    if (k < cnt) off[(size_t)f * max_items + first + k] = excl;
+    T last;
+    if constexpr (sizeof(T) == sizeof(unsigned)) {
+      last = __shfl(v, 63);
+    } else {
+      last = ExSum{__shfl(v.g, 63), __shfl(v.h, 63)};
+    }
+    carry = carry + last;
+  }
+}
+
+__device__ __forceinline__ bool ExBetter(float og, int ob, float gain, int bin) {
+  return ob >= 0 && (bin < 0 || og > gain || (og == gain && ob > bin));
+}
+
+// grid (items, F): running sums along every work item's piece of every list (on top of `off`, the
+// sums of the node's items before it), the gain wherever the rank changes to the next place of the
+// node, and the best candidate of the piece, ties to the highest rank.
+// ranks: [F][stride] by row.  best: [F][max_items].
+template <bool PAIR, bool F64>
+__global__ void __launch_bounds__(kExThreads)
+k_ex_scan(const unsigned *__restrict__ lists, const unsigned *__restrict__ ranks, size_t stride,
+          const float *__restrict__ g, const float *__restrict__ h, const int *__restrict__ shifts,
+          const WorkItem *__restrict__ work, const unsigned *__restrict__ n_work, const ExSum *__restrict__ off,
+          const NodeSum *__restrict__ tot, const unsigned *__restrict__ seg_start, GainParams gp,
+          Cand *__restrict__ best, unsigned max_items) {
+  __shared__ ExSum s_wave[kExThreads / 64];
+  __shared__ Cand s_best[kExThreads / 64];
+  const unsigned w = blockIdx.x, f = blockIdx.y;
+  if (w >= *n_work) return;
+  const WorkItem it = work[w];
+  const NodeSum t = tot[it.node];
+  const unsigned node_start = seg_start[it.node], node_end = node_start + (unsigned)t.c;
+  const unsigned *list = lists + (size_t)f * stride;
+  const unsigned *rank = ranks + (size_t)f * stride;
+  const int sg = shifts[0], sh = shifts[1];
+  const unsigned p0 = it.begin + threadIdx.x * kExPer;
+  ExSum v[kExPer];
+  ExLoadSums<PAIR>(list, g, h, p0, it.end, sg, sh, v);
+  // ranks at this thread's places and at the one after them (which may lie in the next item)
+  unsigned rk[kExPer + 1];
+#pragma unroll
+  for (int j = 0; j <= kExPer; ++j) rk[j] = p0 + j < node_end ? rank[list[p0 + j]] : 0u;
+#pragma unroll
+  for (int j = 1; j < kExPer; ++j) v[j] = v[j] + v[j - 1];
+  ExSum total;
+  const ExSum incl = ExBlockScan(v[kExPer - 1], s_wave, &total);
+  const ExSum base = off[(size_t)f * max_items + w];
+  const long long eg = base.g + incl.g - v[kExPer - 1].g, eh = base.h + incl.h - v[kExPer - 1].h;
+
+  Cand mine;
+  mine.gain = 0.0f;
+  mine.bin = -1;
+  mine.left.g = mine.left.h = 0;
+  mine.left.c = 0;
+  const double GT = FromFixed<F64>(t.g, sg);
+  const double HT = PAIR ? FromFixed<F64>(t.h, sh) : 0.0;
+#pragma unroll
+  for (int j = 0; j < kExPer; ++j) {
+    const unsigned p = p0 + j;
+    if (p < it.end && p + 1 < node_end && rk[j] != rk[j + 1]) {
+      const long long lg = eg + v[j].g, lh = eh + v[j].h;
+      const unsigned long long lc = p - node_start + 1;
+      const double GL = FromFixed<F64>(lg, sg);
+      const double HL = PAIR ? FromFixed<F64>(lh, sh) : 0.0;
+      const float gn = SplitGain<PAIR, F64>(GL, HL, lc, GT, HT, t.c, gp);
+      if (gn > 0.0f && gn >= mine.gain) {
+        mine.gain = gn;
+        mine.bin = (int)(rk[j + 1] - 1u);
+        mine.left.g = lg;
+        mine.left.h = lh;
+        mine.left.c = lc;
+      }
+    }
+  }
+  for (int o = 32; o > 0; o >>= 1) {
+    const float og = __shfl_down(mine.gain, o);
+    const int ob = __shfl_down(mine.bin, o);
+    const long long olg = __shfl_down(mine.left.g, o);
+    const long long olh = __shfl_down(mine.left.h, o);
+    const unsigned long long olc = __shfl_down(mine.left.c, o);
+    if (ExBetter(og, ob, mine.gain, mine.bin)) {
+      mine.gain = og;
+      mine.bin = ob;
+      mine.left.g = olg;
+      mine.left.h = olh;
+      mine.left.c = olc;
+    }
+  }
+  if ((threadIdx.x & 63) == 0) s_best[threadIdx.x >> 6] = mine;
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    for (int k = 1; k < kExThreads / 64; ++k)
+      if (ExBetter(s_best[k].gain, s_best[k].bin, mine.gain, mine.bin)) mine = s_best[k];
+    best[(size_t)f * max_items + w] = mine;
+  }
+}
+
+// grid (L, F), one wave: the best candidate of a node's work items -> cand[node * F + feature].
+__global__ void __launch_bounds__(64)
+k_ex_merge(const Cand *__restrict__ best, const unsigned *__restrict__ node_first,
+           const unsigned *__restrict__ node_items, unsigned max_items, int F, Cand *__restrict__ cand) {
+  const unsigned nd = blockIdx.x, f = blockIdx.y, lane = threadIdx.x;
+  const unsigned first = node_first[nd];
+  unsigned cnt = node_items[nd];
+  if (cnt == 0xffffffffu) cnt = 0;
+  Cand mine;
+  mine.gain = 0.0f;
+  mine.bin = -1;
+  mine.left.g = mine.left.h = 0;
+  mine.left.c = 0;
+  for (unsigned k = lane; k < cnt; k += 64) {
+    const Cand c = best[(size_t)f * max_items + first + k];
+    if (ExBetter(c.gain, c.bin, mine.gain, mine.bin)) mine = c;
+  }
+  for (int o = 32; o > 0; o >>= 1) {
+    const float og = __shfl_down(mine.gain, o);
+    const int ob = __shfl_down(mine.bin, o);
+    const long long olg = __shfl_down(mine.left.g, o);
+    const long long olh = __shfl_down(mine.left.h, o);
+    const unsigned long long olc = __shfl_down(mine.left.c, o);
+    if (ExBetter(og, ob, mine.gain, mine.bin)) {
+      mine.gain = og;
+      mine.bin = ob;
+      mine.left.g = olg;
+      mine.left.h = olh;
+      mine.left.c = olc;
+    }
+  }
+  if (lane == 0) cand[(size_t)nd * F + f] = mine;
+}
+
+// Every row to its child: node_of[row] = 2 * node + (rank of the split feature > split rank).
+__global__ void k_ex_decide(const unsigned *__restrict__ ranks, size_t stride, const SplitRec *__restrict__ split,
+                            unsigned *__restrict__ node_of, size_t n) {
+  for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (size_t)gridDim.x * blockDim.x) {
+    const unsigned nd = node_of[i];
+    const SplitRec s = split[nd];
+    const bool right = s.fid >= 0 && ranks[(size_t)s.fid * stride + i] > (unsigned)s.bin;
+    node_of[i] = 2 * nd + (right ? 1u : 0u);
+  }
+}
+
+// grid (items, F): rows of every piece that go left.
+__global__ void __launch_bounds__(kExThreads)
+k_ex_count(const unsigned *__restrict__ lists, size_t stride, const unsigned *__restrict__ node_of,
+           const WorkItem *__restrict__ work, const unsigned *__restrict__ n_work, unsigned *__restrict__ lefts,
+           unsigned max_items) {
+  __shared__ unsigned s_wave[kExThreads / 64];
+  const unsigned w = blockIdx.x, f = blockIdx.y;
+  if (w >= *n_work) return;
+  const WorkItem it = work[w];
+  const unsigned *list = lists + (size_t)f * stride;
+  const unsigned p0 = it.begin + threadIdx.x * kExPer;
+  unsigned mine = 0;
+#pragma unroll
+  for (int j = 0; j < kExPer; ++j)
+    if (p0 + j < it.end) mine += (node_of[list[p0 + j]] & 1u) ^ 1u;
+  unsigned total;
+  ExBlockScan(mine, s_wave, &total);
+  if (threadIdx.x == 0) lefts[(size_t)f * max_items + w] = total;
+}
+
+// grid (items, F): the stable partition of every piece into the lists of the two children.
+// left_off: rows of the node's earlier pieces that go left; seg_start / seg_next: first place of
+// the parents / of the children.
+__global__ void __launch_bounds__(kExThreads)
+k_ex_scatter(const unsigned *__restrict__ lists, unsigned *__restrict__ lists_out, size_t stride,
+             const unsigned *__restrict__ node_of, const WorkItem *__restrict__ work,
+             const unsigned *__restrict__ n_work, const unsigned *__restrict__ left_off,
+             const unsigned *__restrict__ seg_start, const unsigned *__restrict__ seg_next, unsigned max_items) {
+  __shared__ unsigned s_wave[kExThreads / 64];
+  const unsigned w = blockIdx.x, f = blockIdx.y;
+  if (w >= *n_work) return;
+  const WorkItem it = work[w];
+  const unsigned *list = lists + (size_t)f * stride;
+  unsigned *out = lists_out + (size_t)f * stride;
+  const unsigned p0 = it.begin + threadIdx.x * kExPer;
+  unsigned id[kExPer];
+  unsigned left_bits = 0, mine = 0;
+#pragma unroll
+  for (int j = 0; j < kExPer; ++j) {
+    id[j] = 0;
+    if (p0 + j < it.end) {
+      id[j] = list[p0 + j];
+      const unsigned l = (node_of[id[j]] & 1u) ^ 1u;
+      left_bits |= l << j;
+      mine += l;
+    }
+  }
+  unsigned total;
+  const unsigned incl = ExBlockScan(mine, s_wave, &total);
+  const unsigned before = left_off[(size_t)f * max_items + w];
+  // rows before this thread's first place: to the left / to the right
+  unsigned l_at = before + incl - mine;
+  unsigned r_at = (it.begin - seg_start[it.node]) + threadIdx.x * kExPer - l_at;
+  const unsigned l_base = seg_next[2 * it.node], r_base = seg_next[2 * it.node + 1];
+#pragma unroll
+  for (int j = 0; j < kExPer; ++j) {
+    if (p0 + j < it.end) {
+      if ((left_bits >> j) & 1u)
+        out[l_base + l_at++] = id[j];
+      else
+        out[r_base + r_at++] = id[j];
+    }
+  }
+}
+
+// The leaf of every row and its prediction (update_by_last_tree, src/core/garden.cu:45-76).
+__global__ void k_ex_final(const unsigned *__restrict__ node_of, const float *__restrict__ weights,
+                           float *__restrict__ yhat, unsigned *__restrict__ leaf_of, size_t n) {
+  for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (size_t)gridDim.x * blockDim.x) {
+    const unsigned leaf = node_of[i];
+    leaf_of[i] = leaf;
+    yhat[i] += weights[leaf];
+  }
+}
+
+}  // namespace
+}  // namespace arb
+#endif  // ARBORETUM_AMD_KERNELS_EXACT_H_
