@@ -16,9 +16,11 @@
 #include <cmath>
 #include <cstring>
 #include <limits>
+#include <memory>
 #include <random>
 #include <stdexcept>
 #include <string>
+#include <thread>
 #include <vector>
 
 #include "booster.h"
@@ -36,14 +38,16 @@ namespace arb {
 struct ExactSortData {
   size_t rows = 0, stride = 0;
   int F = 0;
-  uint32_t *ranks = nullptr;  // [F][stride] by row: rank of the row's value among the feature's distinct values
-  uint32_t *lists = nullptr;  // [F][stride]: the rows in ascending order of the feature's value
+  uint32_t *ranks = nullptr;       // [F][stride] by row: rank of the row's value among the feature's distinct values
+  uint32_t *lists = nullptr;       // [F][stride]: the rows in ascending order of the feature's value
+  uint32_t *list_ranks = nullptr;  // [F][stride]: the ranks in that order
 };
 
 void FreeExactSortData(ExactSortData *d) {
   if (!d) return;
   if (d->ranks) (void)hipFree(d->ranks);
   if (d->lists) (void)hipFree(d->lists);
+  if (d->list_ranks) (void)hipFree(d->list_ranks);
   delete d;
 }
 
@@ -54,31 +58,46 @@ void PrepareExactSort(DataMatrix *data) {
   const size_t n = data->rows;
   const int F = (int)data->columns_dense;
   const size_t stride = (n + 63) / 64 * 64;
-  std::vector<uint32_t> ranks((size_t)F * stride, 0u), lists((size_t)F * stride, 0u);
+  std::vector<uint32_t> ranks((size_t)F * stride, 0u), lists((size_t)F * stride, 0u), list_ranks((size_t)F * stride, 0u);
   std::vector<std::vector<float>> mapping(F);
   std::atomic<bool> has_nan{false};
-  ParallelFor((size_t)F, [&](size_t fb, size_t fe) {
-    std::vector<uint32_t> order(n);
-    for (size_t f = fb; f < fe; ++f) {
+  // one column per thread at a time (the columns are few and long)
+  std::atomic<size_t> next_feature{0};
+  auto sort_columns = [&]() {
+    // (value, row) packed into one integer that sorts like the pair: the float's bits with the
+    // sign folded so that unsigned order is numeric order, above the row id
+    std::vector<uint64_t> keyed(n);
+    for (size_t f = next_feature++; f < (size_t)F; f = next_feature++) {
       const float *col = data->data[f].data();
       for (size_t i = 0; i < n; ++i) {
-        order[i] = (uint32_t)i;
         if (col[i] != col[i]) has_nan = true;
+        uint32_t u;
+        std::memcpy(&u, &col[i], sizeof(u));
+        if (u == 0x80000000u) u = 0;  // -0 and +0 are one value
+        u = (u & 0x80000000u) ? ~u : (u | 0x80000000u);
+        keyed[i] = ((uint64_t)u << 32) | (uint64_t)i;
       }
       if (has_nan) return;
-      std::sort(order.begin(), order.end(), [col](uint32_t a, uint32_t b) {
-        return col[a] < col[b] || (col[a] == col[b] && a < b);
-      });
-      uint32_t *rk = ranks.data() + f * stride;
+      std::sort(keyed.begin(), keyed.end());
+      uint32_t *rk = ranks.data() + f * stride, *ls = lists.data() + f * stride, *lr = list_ranks.data() + f * stride;
       std::vector<float> &m = mapping[f];
       for (size_t k = 0; k < n; ++k) {
-        const float v = col[order[k]];
+        const uint32_t row = (uint32_t)keyed[k];
+        const float v = col[row];
         if (k == 0 || v != m.back()) m.push_back(v);
-        rk[order[k]] = (uint32_t)(m.size() - 1);
+        ls[k] = row;
+        lr[k] = rk[row] = (uint32_t)(m.size() - 1);
       }
-      std::memcpy(lists.data() + f * stride, order.data(), n * sizeof(uint32_t));
     }
-  });
+  };
+  {
+    const unsigned hw = std::thread::hardware_concurrency();
+    const size_t threads = std::max<size_t>(1, std::min<size_t>({(size_t)(hw ? hw : 1), (size_t)16, (size_t)F}));
+    std::vector<std::thread> pool;
+    for (size_t t = 1; t < threads; ++t) pool.emplace_back(sort_columns);
+    sort_columns();
+    for (std::thread &t : pool) t.join();
+  }
   if (has_nan) throw std::runtime_error("the exact method does not take missing values (NaN); use method 1 (hist)");
   size_t most = 1;
   data->thresholds.assign(F, {});
@@ -96,8 +115,10 @@ void PrepareExactSort(DataMatrix *data) {
   d->F = F;
   d->ranks = DevAlloc<uint32_t>(ranks.size());
   d->lists = DevAlloc<uint32_t>(lists.size());
+  d->list_ranks = DevAlloc<uint32_t>(list_ranks.size());
   HIP_OK(hipMemcpy(d->ranks, ranks.data(), ranks.size() * sizeof(uint32_t), hipMemcpyHostToDevice));
   HIP_OK(hipMemcpy(d->lists, lists.data(), lists.size() * sizeof(uint32_t), hipMemcpyHostToDevice));
+  HIP_OK(hipMemcpy(d->list_ranks, list_ranks.data(), list_ranks.size() * sizeof(uint32_t), hipMemcpyHostToDevice));
   data->exact_sort = d.release();
   data->hist_size = (int)most;
   data->max_bin = (int)std::min<size_t>(most - 1, (size_t)std::numeric_limits<int>::max());
@@ -141,8 +162,21 @@ class ExactSortBuilder : public TreeBuilder {
     hipLaunchKernelGGL(k_fill_f32, dim3(GridFor(n_ * K_, 256)), dim3(256), 0, stream_, d_yhat_, init, n_ * K_);
     data->y_hat.assign(n_ * K_, init);  // garden.cu:104
 
-    if (D_ > 2)
-      for (int b = 0; b < 2; ++b) d_lists_[b] = DevAlloc<uint32_t>((size_t)F_ * stride_);
+    d_went_right_ = DevAlloc<unsigned long long>(stride_ / 64);
+    d_gh_ = pair_ ? DevAlloc<float2>(n_) : nullptr;
+    // two sets of lists (ids, ranks, gradients in list order), written and read in turn by the
+    // levels; the gradients of the second set also serve the root's lists
+    const size_t words = (size_t)F_ * stride_;
+    for (int b = 0; b < 2; ++b) {
+      if (D_ > 2) {
+        d_ids_[b] = DevAlloc<uint32_t>(words);
+        d_ranks_[b] = DevAlloc<uint32_t>(words);
+      }
+      if (D_ > 2 || b == 1) {
+        d_lg_[b] = DevAlloc<float>(words);
+        d_lh_[b] = pair_ ? DevAlloc<float>(words) : nullptr;
+      }
+    }
     const int max_nodes = 1 << (D_ - 1);
     for (int s = 0; s < 2; ++s) {
       d_tot_[s] = DevAlloc<NodeSum>(max_nodes);
@@ -159,6 +193,7 @@ class ExactSortBuilder : public TreeBuilder {
     d_best_ = DevAlloc<Cand>((size_t)F_ * max_items_);
     d_lefts_ = DevAlloc<unsigned>((size_t)F_ * max_items_);
     d_left_off_ = DevAlloc<unsigned>((size_t)F_ * max_items_);
+    d_left_bits_ = DevAlloc<uint8_t>((size_t)F_ * max_items_ * kExThreads);
     d_shifts_ = DevAlloc<int>(2);
     d_records_ = DevAlloc<uint32_t>(kRecordRing * RecordWords());
     d_gmax_ = DevAlloc<unsigned>(1);
@@ -188,9 +223,10 @@ class ExactSortBuilder : public TreeBuilder {
 
   ~ExactSortBuilder() override {
     (void)hipStreamSynchronize(stream_);
-    void *all[] = {d_y_, d_labels_, d_yhat_, d_g_, d_h_, d_leaf_, d_node_of_, d_lists_[0], d_lists_[1], d_tot_[0],
+    void *all[] = {d_y_, d_labels_, d_yhat_, d_g_, d_h_, d_leaf_, d_node_of_, d_went_right_, d_gh_, d_ids_[0], d_ids_[1], d_ranks_[0],
+                   d_ranks_[1], d_lg_[0], d_lg_[1], d_lh_[0], d_lh_[1], d_tot_[0],
                    d_tot_[1], d_seg_[0], d_seg_[1], d_split_, d_cand_, d_work_, d_n_work_, d_node_first_,
-                   d_node_items_, d_part_, d_off_, d_best_, d_lefts_, d_left_off_, d_shifts_, d_records_, d_gmax_,
+                   d_node_items_, d_part_, d_off_, d_best_, d_lefts_, d_left_off_, d_left_bits_, d_shifts_, d_records_, d_gmax_,
                    d_overflow_, d_tfid_, d_tbin_, d_tgain_, d_weights_, d_active_};
     for (void *p : all)
       if (p) (void)hipFree(p);
@@ -321,7 +357,17 @@ class ExactSortBuilder : public TreeBuilder {
     hipLaunchKernelGGL(k_sum_grad, dim3(GridFor(n_, 256, 1024)), dim3(256), 0, stream_, g, h, n_, d_shifts_, d_tot_[0]);
     HIP_OK(hipMemsetAsync(d_node_of_, 0, n_ * sizeof(unsigned), stream_));
     int state = 0;
-    const uint32_t *lists = sd_->lists;  // the root's lists: every row, sorted once
+    // the root's lists: every row, sorted once; this tree's gradients in that order
+    const dim3 whole((unsigned)((n_ + kExItem - 1) / kExItem), (unsigned)F_);
+    if (pair_) {
+      hipLaunchKernelGGL(k_ex_pair, dim3(GridFor(n_, 256)), dim3(256), 0, stream_, g, h, d_gh_, n_);
+      hipLaunchKernelGGL((k_ex_gather<true>), whole, dim3(kExThreads), 0, stream_, sd_->lists, stride_, g, d_gh_,
+                         d_lg_[1], d_lh_[1], n_);
+    } else {
+      hipLaunchKernelGGL((k_ex_gather<false>), whole, dim3(kExThreads), 0, stream_, sd_->lists, stride_, g,
+                         (const float2 *)nullptr, d_lg_[1], d_lh_[1], n_);
+    }
+    ExLists lists{sd_->lists, sd_->list_ranks, d_lg_[1], d_lh_[1]};
     for (int level = 0; level + 1 < D_; ++level) {
       const int L = 1 << level;
       const bool last = level + 2 >= D_;
@@ -332,12 +378,12 @@ class ExactSortBuilder : public TreeBuilder {
                          (const SplitRec *)nullptr, grid_items, d_overflow_, 0u, (unsigned *)nullptr);
 #define ARB_EX(P, D)                                                                                                  \
   do {                                                                                                                \
-    hipLaunchKernelGGL((k_ex_partial<P>), per_item, dim3(kExThreads), 0, stream_, lists, stride_, g, h, d_shifts_,   \
-                       d_work_, d_n_work_, d_part_, max_items_);                                                      \
+    hipLaunchKernelGGL((k_ex_partial<P>), per_item, dim3(kExThreads), 0, stream_, lists, stride_, d_shifts_, d_work_, \
+                       d_n_work_, d_part_, max_items_);                                                               \
     hipLaunchKernelGGL((k_ex_offsets<ExSum>), per_node, dim3(64), 0, stream_, d_part_, d_off_, d_node_first_,        \
                        d_node_items_, max_items_);                                                                    \
-    hipLaunchKernelGGL((k_ex_scan<P, D>), per_item, dim3(kExThreads), 0, stream_, lists, sd_->ranks, stride_, g, h,  \
-                       d_shifts_, d_work_, d_n_work_, d_off_, d_tot_[state], d_seg_[state], gp, d_best_, max_items_); \
+    hipLaunchKernelGGL((k_ex_scan<P, D>), per_item, dim3(kExThreads), 0, stream_, lists, stride_, d_shifts_, d_work_, \
+                       d_n_work_, d_off_, d_tot_[state], d_seg_[state], gp, d_best_, max_items_);                     \
   } while (0)
       if (pair_ && f64_) ARB_EX(true, true);
       else if (pair_) ARB_EX(true, false);
@@ -350,7 +396,7 @@ class ExactSortBuilder : public TreeBuilder {
                          d_seg_[state], d_tot_[state ^ 1], d_seg_[state ^ 1], d_split_, d_tfid_, d_tbin_, d_tgain_,
                          L - 1, sampling_ ? d_active_ + (size_t)level * F_ : (const unsigned char *)nullptr);
       hipLaunchKernelGGL(k_ex_decide, dim3(GridFor(n_, 256)), dim3(256), 0, stream_, sd_->ranks, stride_, d_split_,
-                         d_node_of_, n_);
+                         d_node_of_, d_went_right_, n_);
       if (last) {
         const int blocks = (L + 127) / 128;
 #define ARB_LEAF(P, D)                                                                                          \
@@ -364,14 +410,20 @@ class ExactSortBuilder : public TreeBuilder {
         hipLaunchKernelGGL(k_ex_final, dim3(GridFor(n_, 256)), dim3(256), 0, stream_, d_node_of_, d_weights_,
                            d_yhat_ + (size_t)label * n_, d_leaf_, n_);
       } else {
-        uint32_t *out = d_lists_[level & 1];
-        hipLaunchKernelGGL(k_ex_count, per_item, dim3(kExThreads), 0, stream_, lists, stride_, d_node_of_, d_work_,
-                           d_n_work_, d_lefts_, max_items_);
+        const int b = level & 1;
+        hipLaunchKernelGGL(k_ex_count, per_item, dim3(kExThreads), 0, stream_, lists.ids, stride_, d_went_right_,
+                           d_work_, d_n_work_, d_lefts_, d_left_bits_, max_items_);
         hipLaunchKernelGGL((k_ex_offsets<unsigned>), per_node, dim3(64), 0, stream_, d_lefts_, d_left_off_,
                            d_node_first_, d_node_items_, max_items_);
-        hipLaunchKernelGGL(k_ex_scatter, per_item, dim3(kExThreads), 0, stream_, lists, out, stride_, d_node_of_,
-                           d_work_, d_n_work_, d_left_off_, d_seg_[state], d_seg_[state ^ 1], max_items_);
-        lists = out;
+        if (pair_)
+          hipLaunchKernelGGL((k_ex_scatter<true>), per_item, dim3(kExThreads), 0, stream_, lists, d_ids_[b], d_ranks_[b],
+                             d_lg_[b], d_lh_[b], stride_, d_left_bits_, d_work_, d_n_work_, d_left_off_,
+                             d_seg_[state], d_seg_[state ^ 1], max_items_);
+        else
+          hipLaunchKernelGGL((k_ex_scatter<false>), per_item, dim3(kExThreads), 0, stream_, lists, d_ids_[b], d_ranks_[b],
+                             d_lg_[b], d_lh_[b], stride_, d_left_bits_, d_work_, d_n_work_, d_left_off_,
+                             d_seg_[state], d_seg_[state ^ 1], max_items_);
+        lists = ExLists{d_ids_[b], d_ranks_[b], d_lg_[b], d_lh_[b]};
         state ^= 1;
       }
       HIP_OK(hipGetLastError());
@@ -399,7 +451,11 @@ class ExactSortBuilder : public TreeBuilder {
   unsigned *d_leaf_ = nullptr, *d_node_of_ = nullptr, *d_seg_[2] = {nullptr, nullptr}, *d_n_work_ = nullptr,
            *d_node_first_ = nullptr, *d_node_items_ = nullptr, *d_lefts_ = nullptr, *d_left_off_ = nullptr,
            *d_gmax_ = nullptr, *d_overflow_ = nullptr;
-  uint32_t *d_lists_[2] = {nullptr, nullptr}, *d_records_ = nullptr;
+  uint32_t *d_ids_[2] = {nullptr, nullptr}, *d_ranks_[2] = {nullptr, nullptr}, *d_records_ = nullptr;
+  float *d_lg_[2] = {nullptr, nullptr}, *d_lh_[2] = {nullptr, nullptr};
+  unsigned long long *d_went_right_ = nullptr;
+  uint8_t *d_left_bits_ = nullptr;
+  float2 *d_gh_ = nullptr;  // (g, h) of the tree's label side by side: one gather per row
   NodeSum *d_tot_[2] = {nullptr, nullptr};
   SplitRec *d_split_ = nullptr;
   Cand *d_cand_ = nullptr, *d_best_ = nullptr;

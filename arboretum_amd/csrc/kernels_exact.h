@@ -57,34 +57,58 @@ __device__ __forceinline__ T ExBlockScan(T v, T *s_wave, T *total) {
   return before + v;
 }
 
-// The fixed-point gradients of the rows at the places [p0, p0 + kExPer) of a list, zero past `end`.
+// The lists of a level: for every feature the rows of every node in ascending order of the
+// feature's value, and next to each row id what the passes need of that row, so that they read
+// it in list order instead of gathering it by row: the row's rank in this feature and its
+// gradients (the root's ids and ranks are the same for every tree; its gradients are gathered
+// once per tree, k_ex_gather).
+struct ExLists {
+  const unsigned *ids;    // [F][stride]
+  const unsigned *ranks;  // [F][stride]
+  const float *g, *h;     // [F][stride]; h null without hessians
+};
+
+// Eight consecutive words of a list from place p0, `fill` past `end`.
+template <typename T>
+__device__ __forceinline__ void ExLoad8(const T *__restrict__ base, unsigned p0, unsigned end, T fill, T *out) {
+  static_assert(sizeof(T) == 4, "lists hold 32-bit words");
+  if ((p0 & 3u) == 0 && p0 + kExPer <= end) {
+    const uint4 a = *reinterpret_cast<const uint4 *>(base + p0);
+    const uint4 b = *reinterpret_cast<const uint4 *>(base + p0 + 4);
+    const unsigned w[kExPer] = {a.x, a.y, a.z, a.w, b.x, b.y, b.z, b.w};
+#pragma unroll
+    for (int j = 0; j < kExPer; ++j) __builtin_memcpy(&out[j], &w[j], 4);
+  } else {
+#pragma unroll
+    for (int j = 0; j < kExPer; ++j) out[j] = p0 + j < end ? base[p0 + j] : fill;
+  }
+}
+
+// The fixed-point gradients of the rows at the places [p0, p0 + kExPer) of feature f's list, zero past `end`.
 template <bool PAIR>
-__device__ __forceinline__ void ExLoadSums(const unsigned *__restrict__ list, const float *__restrict__ g,
-                                           const float *__restrict__ h, unsigned p0, unsigned end, int sg, int sh,
+__device__ __forceinline__ void ExLoadSums(const ExLists &ls, size_t fbase, unsigned p0, unsigned end, int sg, int sh,
                                            ExSum *v) {
+  float gv[kExPer], hv[kExPer];
+  ExLoad8(ls.g + fbase, p0, end, 0.0f, gv);
+  if (PAIR) ExLoad8(ls.h + fbase, p0, end, 0.0f, hv);
 #pragma unroll
   for (int j = 0; j < kExPer; ++j) {
-    v[j] = ExSum{0, 0};
-    if (p0 + j < end) {
-      const unsigned id = list[p0 + j];
-      v[j].g = ToFixed(g[id], sg);
-      if (PAIR) v[j].h = ToFixed(h[id], sh);
-    }
+    v[j].g = p0 + j < end ? ToFixed(gv[j], sg) : 0;
+    v[j].h = PAIR && p0 + j < end ? ToFixed(hv[j], sh) : 0;
   }
 }
 
 // grid (items, F): the sum of the gradients over every work item's piece of every feature's list.
 template <bool PAIR>
 __global__ void __launch_bounds__(kExThreads)
-k_ex_partial(const unsigned *__restrict__ lists, size_t stride, const float *__restrict__ g,
-             const float *__restrict__ h, const int *__restrict__ shifts, const WorkItem *__restrict__ work,
+k_ex_partial(const ExLists ls, size_t stride, const int *__restrict__ shifts, const WorkItem *__restrict__ work,
              const unsigned *__restrict__ n_work, ExSum *__restrict__ part, unsigned max_items) {
   __shared__ ExSum s_wave[kExThreads / 64];
   const unsigned w = blockIdx.x, f = blockIdx.y;
   if (w >= *n_work) return;
   const WorkItem it = work[w];
   ExSum v[kExPer];
-  ExLoadSums<PAIR>(lists + (size_t)f * stride, g, h, it.begin + threadIdx.x * kExPer, it.end, shifts[0], shifts[1], v);
+  ExLoadSums<PAIR>(ls, (size_t)f * stride, it.begin + threadIdx.x * kExPer, it.end, shifts[0], shifts[1], v);
   ExSum mine = v[0];
 #pragma unroll
   for (int j = 1; j < kExPer; ++j) mine = mine + v[j];
@@ -135,11 +159,10 @@ __device__ __forceinline__ bool ExBetter(float og, int ob, float gain, int bin) 
 // grid (items, F): running sums along every work item's piece of every list (on top of `off`, the
 // sums of the node's items before it), the gain wherever the rank changes to the next place of the
 // node, and the best candidate of the piece, ties to the highest rank.
-// ranks: [F][stride] by row.  best: [F][max_items].
+// best: [F][max_items].
 template <bool PAIR, bool F64>
 __global__ void __launch_bounds__(kExThreads)
-k_ex_scan(const unsigned *__restrict__ lists, const unsigned *__restrict__ ranks, size_t stride,
-          const float *__restrict__ g, const float *__restrict__ h, const int *__restrict__ shifts,
+k_ex_scan(const ExLists ls, size_t stride, const int *__restrict__ shifts,
           const WorkItem *__restrict__ work, const unsigned *__restrict__ n_work, const ExSum *__restrict__ off,
           const NodeSum *__restrict__ tot, const unsigned *__restrict__ seg_start, GainParams gp,
           Cand *__restrict__ best, unsigned max_items) {
@@ -150,16 +173,15 @@ k_ex_scan(const unsigned *__restrict__ lists, const unsigned *__restrict__ ranks
   const WorkItem it = work[w];
   const NodeSum t = tot[it.node];
   const unsigned node_start = seg_start[it.node], node_end = node_start + (unsigned)t.c;
-  const unsigned *list = lists + (size_t)f * stride;
-  const unsigned *rank = ranks + (size_t)f * stride;
+  const size_t fbase = (size_t)f * stride;
   const int sg = shifts[0], sh = shifts[1];
   const unsigned p0 = it.begin + threadIdx.x * kExPer;
   ExSum v[kExPer];
-  ExLoadSums<PAIR>(list, g, h, p0, it.end, sg, sh, v);
+  ExLoadSums<PAIR>(ls, fbase, p0, it.end, sg, sh, v);
   // ranks at this thread's places and at the one after them (which may lie in the next item)
   unsigned rk[kExPer + 1];
-#pragma unroll
-  for (int j = 0; j <= kExPer; ++j) rk[j] = p0 + j < node_end ? rank[list[p0 + j]] : 0u;
+  ExLoad8(ls.ranks + fbase, p0, node_end, 0u, rk);
+  rk[kExPer] = p0 + kExPer < node_end ? ls.ranks[fbase + p0 + kExPer] : 0u;
 #pragma unroll
   for (int j = 1; j < kExPer; ++j) v[j] = v[j] + v[j - 1];
   ExSum total;
@@ -250,77 +272,136 @@ k_ex_merge(const Cand *__restrict__ best, const unsigned *__restrict__ node_firs
 }
 
 // Every row to its child: node_of[row] = 2 * node + (rank of the split feature > split rank).
-__global__ void k_ex_decide(const unsigned *__restrict__ ranks, size_t stride, const SplitRec *__restrict__ split,
-                            unsigned *__restrict__ node_of, size_t n) {
-  for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (size_t)gridDim.x * blockDim.x) {
-    const unsigned nd = node_of[i];
-    const SplitRec s = split[nd];
-    const bool right = s.fid >= 0 && ranks[(size_t)s.fid * stride + i] > (unsigned)s.bin;
-    node_of[i] = 2 * nd + (right ? 1u : 0u);
+// went_right: one bit per row (64 rows per word), small enough to stay in L2 while the lists are
+// partitioned.  ranks: [F][stride] by row.  Launched with whole waves over 64-aligned rows.
+__global__ void __launch_bounds__(256)
+k_ex_decide(const unsigned *__restrict__ ranks, size_t stride, const SplitRec *__restrict__ split,
+            unsigned *__restrict__ node_of, unsigned long long *__restrict__ went_right, size_t n) {
+  const size_t padded = (n + 63) / 64 * 64;
+  for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < padded; i += (size_t)gridDim.x * blockDim.x) {
+    bool right = false;
+    if (i < n) {
+      const unsigned nd = node_of[i];
+      const SplitRec s = split[nd];
+      right = s.fid >= 0 && ranks[(size_t)s.fid * stride + i] > (unsigned)s.bin;
+      node_of[i] = 2 * nd + (right ? 1u : 0u);
+    }
+    const unsigned long long m = __ballot(right);
+    if ((threadIdx.x & 63) == 0) went_right[i >> 6] = m;
   }
 }
 
-// grid (items, F): rows of every piece that go left.
+__device__ __forceinline__ unsigned ExGoesLeft(const unsigned long long *__restrict__ went_right, unsigned id) {
+  return (unsigned)(~(went_right[id >> 6] >> (id & 63u)) & 1ull);
+}
+
+// grid (items, F): rows of every piece that go left; left_bits: for every thread of every piece
+// the decisions of its kExPer places (bit j: place j goes left), which the partition reads back
+// instead of looking the rows up again.
 __global__ void __launch_bounds__(kExThreads)
-k_ex_count(const unsigned *__restrict__ lists, size_t stride, const unsigned *__restrict__ node_of,
+k_ex_count(const unsigned *__restrict__ ids, size_t stride, const unsigned long long *__restrict__ went_right,
            const WorkItem *__restrict__ work, const unsigned *__restrict__ n_work, unsigned *__restrict__ lefts,
-           unsigned max_items) {
+           uint8_t *__restrict__ left_bits, unsigned max_items) {
+  static_assert(kExPer == 8, "one byte of decisions per thread");
   __shared__ unsigned s_wave[kExThreads / 64];
   const unsigned w = blockIdx.x, f = blockIdx.y;
   if (w >= *n_work) return;
   const WorkItem it = work[w];
-  const unsigned *list = lists + (size_t)f * stride;
   const unsigned p0 = it.begin + threadIdx.x * kExPer;
-  unsigned mine = 0;
+  unsigned id[kExPer];
+  ExLoad8(ids + (size_t)f * stride, p0, it.end, 0u, id);
+  unsigned bits = 0;
 #pragma unroll
   for (int j = 0; j < kExPer; ++j)
-    if (p0 + j < it.end) mine += (node_of[list[p0 + j]] & 1u) ^ 1u;
+    if (p0 + j < it.end) bits |= ExGoesLeft(went_right, id[j]) << j;
+  left_bits[((size_t)f * max_items + w) * kExThreads + threadIdx.x] = (uint8_t)bits;
   unsigned total;
-  ExBlockScan(mine, s_wave, &total);
+  ExBlockScan((unsigned)__builtin_popcount(bits), s_wave, &total);
   if (threadIdx.x == 0) lefts[(size_t)f * max_items + w] = total;
 }
 
-// grid (items, F): the stable partition of every piece into the lists of the two children.
+// grid (items, F): the stable partition of every piece into the lists of the two children, with
+// the rank and the gradients of every row next to its id.  The piece is put in order in LDS
+// (the rows that go left, then the others) and written out from there, so that the stores of a
+// wave are consecutive.
 // left_off: rows of the node's earlier pieces that go left; seg_start / seg_next: first place of
 // the parents / of the children.
+template <bool PAIR>
 __global__ void __launch_bounds__(kExThreads)
-k_ex_scatter(const unsigned *__restrict__ lists, unsigned *__restrict__ lists_out, size_t stride,
-             const unsigned *__restrict__ node_of, const WorkItem *__restrict__ work,
+k_ex_scatter(const ExLists ls, unsigned *__restrict__ ids_out, unsigned *__restrict__ ranks_out,
+             float *__restrict__ g_out, float *__restrict__ h_out, size_t stride,
+             const uint8_t *__restrict__ left_bits, const WorkItem *__restrict__ work,
              const unsigned *__restrict__ n_work, const unsigned *__restrict__ left_off,
              const unsigned *__restrict__ seg_start, const unsigned *__restrict__ seg_next, unsigned max_items) {
   __shared__ unsigned s_wave[kExThreads / 64];
+  __shared__ unsigned s_id[kExItem], s_rk[kExItem];
+  __shared__ float s_g[kExItem], s_h[PAIR ? kExItem : 1];
   const unsigned w = blockIdx.x, f = blockIdx.y;
   if (w >= *n_work) return;
   const WorkItem it = work[w];
-  const unsigned *list = lists + (size_t)f * stride;
-  unsigned *out = lists_out + (size_t)f * stride;
+  const size_t fbase = (size_t)f * stride;
   const unsigned p0 = it.begin + threadIdx.x * kExPer;
-  unsigned id[kExPer];
-  unsigned left_bits = 0, mine = 0;
-#pragma unroll
-  for (int j = 0; j < kExPer; ++j) {
-    id[j] = 0;
-    if (p0 + j < it.end) {
-      id[j] = list[p0 + j];
-      const unsigned l = (node_of[id[j]] & 1u) ^ 1u;
-      left_bits |= l << j;
-      mine += l;
-    }
-  }
+  unsigned id[kExPer], rk[kExPer];
+  float gv[kExPer], hv[kExPer];
+  ExLoad8(ls.ids + fbase, p0, it.end, 0u, id);
+  ExLoad8(ls.ranks + fbase, p0, it.end, 0u, rk);
+  ExLoad8(ls.g + fbase, p0, it.end, 0.0f, gv);
+  if (PAIR) ExLoad8(ls.h + fbase, p0, it.end, 0.0f, hv);
+  const unsigned bits = left_bits[((size_t)f * max_items + w) * kExThreads + threadIdx.x];
+  const unsigned mine = (unsigned)__builtin_popcount(bits);
   unsigned total;
   const unsigned incl = ExBlockScan(mine, s_wave, &total);
-  const unsigned before = left_off[(size_t)f * max_items + w];
-  // rows before this thread's first place: to the left / to the right
-  unsigned l_at = before + incl - mine;
-  unsigned r_at = (it.begin - seg_start[it.node]) + threadIdx.x * kExPer - l_at;
-  const unsigned l_base = seg_next[2 * it.node], r_base = seg_next[2 * it.node + 1];
+  // places of this thread's rows in the ordered piece
+  unsigned l_at = incl - mine;
+  unsigned r_at = total + threadIdx.x * kExPer - l_at;
 #pragma unroll
   for (int j = 0; j < kExPer; ++j) {
     if (p0 + j < it.end) {
-      if ((left_bits >> j) & 1u)
-        out[l_base + l_at++] = id[j];
-      else
-        out[r_base + r_at++] = id[j];
+      const unsigned at = ((bits >> j) & 1u) ? l_at++ : r_at++;
+      s_id[at] = id[j];
+      s_rk[at] = rk[j];
+      s_g[at] = gv[j];
+      if (PAIR) s_h[at] = hv[j];
+    }
+  }
+  __syncthreads();
+  const unsigned before = left_off[(size_t)f * max_items + w];
+  const unsigned count = it.end - it.begin;
+  const size_t l_to = fbase + seg_next[2 * it.node] + before;
+  const size_t r_to = fbase + seg_next[2 * it.node + 1] + ((it.begin - seg_start[it.node]) - before);
+  for (unsigned k = threadIdx.x; k < count; k += kExThreads) {
+    const size_t at = k < total ? l_to + k : r_to + (k - total);
+    ids_out[at] = s_id[k];
+    ranks_out[at] = s_rk[k];
+    g_out[at] = s_g[k];
+    if (PAIR) h_out[at] = s_h[k];
+  }
+}
+
+// (g, h) of every row side by side, so that one access fetches both.
+__global__ void k_ex_pair(const float *__restrict__ g, const float *__restrict__ h, float2 *__restrict__ gh, size_t n) {
+  for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (size_t)gridDim.x * blockDim.x)
+    gh[i] = make_float2(g[i], h[i]);
+}
+
+// grid (ceil(n / kExItem), F): the gradients of this tree in the order of the root's lists.
+template <bool PAIR>
+__global__ void __launch_bounds__(kExThreads)
+k_ex_gather(const unsigned *__restrict__ ids, size_t stride, const float *__restrict__ g,
+            const float2 *__restrict__ gh, float *__restrict__ g_out, float *__restrict__ h_out, size_t n) {
+  const size_t fbase = (size_t)blockIdx.y * stride;
+#pragma unroll
+  for (int j = 0; j < kExPer; ++j) {
+    const size_t p = (size_t)blockIdx.x * kExItem + (size_t)j * kExThreads + threadIdx.x;
+    if (p < n) {
+      const unsigned id = ids[fbase + p];
+      if (PAIR) {
+        const float2 v = gh[id];
+        g_out[fbase + p] = v.x;
+        h_out[fbase + p] = v.y;
+      } else {
+        g_out[fbase + p] = g[id];
+      }
     }
   }
 }
