@@ -27,6 +27,19 @@ void ParallelFor(size_t n, const std::function<void(size_t, size_t)> &fn) {
   for (auto &t : th) t.join();
 }
 
+void ParallelTasks(size_t n, const std::function<void(size_t)> &fn) {
+  const unsigned hw = std::thread::hardware_concurrency();
+  const size_t nt = std::max<size_t>(1, std::min<size_t>({(size_t)(hw ? hw : 1), (size_t)16, n}));
+  std::atomic<size_t> next{0};
+  auto run = [&]() {
+    for (size_t i = next++; i < n; i = next++) fn(i);
+  };
+  std::vector<std::thread> th;
+  for (size_t t = 1; t < nt; ++t) th.emplace_back(run);
+  run();
+  for (auto &t : th) t.join();
+}
+
 namespace {
 std::atomic<uint64_t> g_next_matrix_uid{1};
 }

@@ -17,6 +17,8 @@ namespace arb {
 
 // Runs fn(begin, end) over [0, n) on a few host threads.
 void ParallelFor(size_t n, const std::function<void(size_t, size_t)> &fn);
+// fn(i) for every i in [0, n), a few long tasks (columns) handed out one at a time to up to 16 threads.
+void ParallelTasks(size_t n, const std::function<void(size_t)> &fn);
 
 struct DeviceMatrix;  // quantised bins resident in HBM (device_builder.hip)
 struct ExactSortData;  // ranks and sorted row lists of every feature (exact_builder.hip)

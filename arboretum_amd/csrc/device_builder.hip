@@ -150,23 +150,22 @@ static std::vector<uint16_t> ExactRanks(DataMatrix *data, size_t *most_distinct,
   std::vector<std::vector<float>> mapping(F);
   std::atomic<bool> has_nan{false};
   std::atomic<int> too_many{-1};
-  ParallelFor((size_t)F, [&](size_t fb, size_t fe) {
-    for (size_t f = fb; f < fe; ++f) {
-      std::vector<float> m(data->data[f]);
-      for (float v : m)
-        if (v != v) has_nan = true;
-      if (has_nan) return;
-      std::sort(m.begin(), m.end());
-      m.erase(std::unique(m.begin(), m.end()), m.end());
-      if (m.size() > (size_t)kMaxWideSlots) {
-        too_many = (int)f;
-        return;
-      }
-      const float *col = data->data[f].data();
-      for (size_t i = 0; i < n; ++i)
-        ranks[i * F + f] = (uint16_t)(std::lower_bound(m.begin(), m.end(), col[i]) - m.begin());
-      mapping[f].swap(m);
+  ParallelTasks((size_t)F, [&](size_t f) {
+    if (has_nan || too_many >= 0) return;
+    std::vector<float> m(data->data[f]);
+    for (float v : m)
+      if (v != v) has_nan = true;
+    if (has_nan) return;
+    std::sort(m.begin(), m.end());
+    m.erase(std::unique(m.begin(), m.end()), m.end());
+    if (m.size() > (size_t)kMaxWideSlots) {
+      too_many = (int)f;
+      return;
     }
+    const float *col = data->data[f].data();
+    for (size_t i = 0; i < n; ++i)
+      ranks[i * F + f] = (uint16_t)(std::lower_bound(m.begin(), m.end(), col[i]) - m.begin());
+    mapping[f].swap(m);
   });
   if (has_nan) throw std::runtime_error("the exact method does not take missing values (NaN); use method 1 (hist)");
   if (too_many >= 0) {

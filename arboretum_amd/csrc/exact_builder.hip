@@ -20,7 +20,6 @@
 #include <random>
 #include <stdexcept>
 #include <string>
-#include <thread>
 #include <vector>
 
 #include "booster.h"
@@ -62,42 +61,32 @@ void PrepareExactSort(DataMatrix *data) {
   std::vector<std::vector<float>> mapping(F);
   std::atomic<bool> has_nan{false};
   // one column per thread at a time (the columns are few and long)
-  std::atomic<size_t> next_feature{0};
-  auto sort_columns = [&]() {
+  ParallelTasks((size_t)F, [&](size_t f) {
+    if (has_nan) return;
     // (value, row) packed into one integer that sorts like the pair: the float's bits with the
     // sign folded so that unsigned order is numeric order, above the row id
     std::vector<uint64_t> keyed(n);
-    for (size_t f = next_feature++; f < (size_t)F; f = next_feature++) {
-      const float *col = data->data[f].data();
-      for (size_t i = 0; i < n; ++i) {
-        if (col[i] != col[i]) has_nan = true;
-        uint32_t u;
-        std::memcpy(&u, &col[i], sizeof(u));
-        if (u == 0x80000000u) u = 0;  // -0 and +0 are one value
-        u = (u & 0x80000000u) ? ~u : (u | 0x80000000u);
-        keyed[i] = ((uint64_t)u << 32) | (uint64_t)i;
-      }
-      if (has_nan) return;
-      std::sort(keyed.begin(), keyed.end());
-      uint32_t *rk = ranks.data() + f * stride, *ls = lists.data() + f * stride, *lr = list_ranks.data() + f * stride;
-      std::vector<float> &m = mapping[f];
-      for (size_t k = 0; k < n; ++k) {
-        const uint32_t row = (uint32_t)keyed[k];
-        const float v = col[row];
-        if (k == 0 || v != m.back()) m.push_back(v);
-        ls[k] = row;
-        lr[k] = rk[row] = (uint32_t)(m.size() - 1);
-      }
+    const float *col = data->data[f].data();
+    for (size_t i = 0; i < n; ++i) {
+      if (col[i] != col[i]) has_nan = true;
+      uint32_t u;
+      std::memcpy(&u, &col[i], sizeof(u));
+      if (u == 0x80000000u) u = 0;  // -0 and +0 are one value
+      u = (u & 0x80000000u) ? ~u : (u | 0x80000000u);
+      keyed[i] = ((uint64_t)u << 32) | (uint64_t)i;
     }
-  };
-  {
-    const unsigned hw = std::thread::hardware_concurrency();
-    const size_t threads = std::max<size_t>(1, std::min<size_t>({(size_t)(hw ? hw : 1), (size_t)16, (size_t)F}));
-    std::vector<std::thread> pool;
-    for (size_t t = 1; t < threads; ++t) pool.emplace_back(sort_columns);
-    sort_columns();
-    for (std::thread &t : pool) t.join();
-  }
+    if (has_nan) return;
+    std::sort(keyed.begin(), keyed.end());
+    uint32_t *rk = ranks.data() + f * stride, *ls = lists.data() + f * stride, *lr = list_ranks.data() + f * stride;
+    std::vector<float> &m = mapping[f];
+    for (size_t k = 0; k < n; ++k) {
+      const uint32_t row = (uint32_t)keyed[k];
+      const float v = col[row];
+      if (k == 0 || v != m.back()) m.push_back(v);
+      ls[k] = row;
+      lr[k] = rk[row] = (uint32_t)(m.size() - 1);
+    }
+  });
   if (has_nan) throw std::runtime_error("the exact method does not take missing values (NaN); use method 1 (hist)");
   size_t most = 1;
   data->thresholds.assign(F, {});

@@ -308,6 +308,30 @@ def other_config(arb, workload, rows_arg, steps):
             "generate_s": t_gen, "roofline": roofline}
 
 
+def exact_workload(arb, rows, features, steps):
+    """The exact method (method 0) on the headline matrix: its columns are continuous, so every
+    feature has far more distinct values than a rank histogram holds and the trees are grown over
+    sorted row lists.  Seconds per tree (not the headline metric)."""
+    X, y = make_workload(rows, features)
+    cfg = config()
+    cfg["method"] = 0
+    data = arb.DMatrix(X, y=y)
+    model = arb.Garden(cfg, data)
+    t0 = time.perf_counter()
+    model.grow_tree()
+    model.synchronize()
+    t_first = time.perf_counter() - t0
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        model.grow_tree()
+    model.synchronize()
+    dt = time.perf_counter() - t0
+    return {"metric": "seconds per tree", "rows": rows, "features": features, "trees": steps,
+            "workload": "exact method on the headline matrix (%d x %d continuous fp32 features, max_depth 8, "
+                        "logistic): sorted row lists per feature" % (rows, features),
+            "sec_per_tree": dt / steps, "first_tree_with_column_sorts_s": t_first}
+
+
 def cpu_baseline(X, y, cfg, sample_rows, trees):
     """The CPU checker on the first `sample_rows` rows (same columns, same
     configuration), all host cores."""
@@ -347,8 +371,9 @@ def main():
                          "one bin per feature; below 1/256 with --hist-size 256 every feature then has 257 bin "
                          "ids, the last one kept as a ninth bit)")
     ap.add_argument("--mode", choices=["resident", "stream"], default="resident")
-    ap.add_argument("--workload", choices=["headline", "config2", "config3"], default="headline",
-                    help="config2 / config3: BASELINE configs[2] / configs[3] at full size, seconds per tree only")
+    ap.add_argument("--workload", choices=["headline", "config2", "config3", "exact"], default="headline",
+                    help="config2 / config3: BASELINE configs[2] / configs[3] at full size, seconds per tree only; "
+                         "exact: the exact method (method 0) on the headline matrix, seconds per tree only")
     ap.add_argument("--stream-rows", type=int, default=64_000_000)
     ap.add_argument("--stream-features", type=int, default=128)
     ap.add_argument("--stream-block-rows", type=int, default=1 << 22)
@@ -371,6 +396,9 @@ def main():
         arb.copy_probe(args.copy_probe << 20)
     if args.mode == "stream":
         stream_mode(args, arb)
+        return
+    if args.workload == "exact":
+        print(json.dumps(exact_workload(arb, args.rows, args.features, args.steps)))
         return
     if args.workload != "headline":
         print(json.dumps(other_config(arb, args.workload, args.rows, args.steps)))

@@ -166,6 +166,33 @@ def test_sorted_lists_with_column_sampling_and_soft_max(arb, oracle):
         assert np.array_equal(ob.yhat(), g.train_yhat())
 
 
+@pytest.mark.parametrize("seed", range(16))
+def test_sorted_lists_on_random_configurations(arb, oracle, seed):
+    # columns of every kind (continuous, rounded so that values repeat, a handful of values, one
+    # constant), every tree parameter drawn at random: ties, empty and tiny nodes, rejected splits
+    rng = np.random.default_rng(1000 + seed)
+    n, F = int(rng.integers(40, 30000)), int(rng.integers(1, 9))
+    X = np.empty((n, F), np.float32)
+    for f in range(F):
+        kind = rng.integers(0, 4) if f else 0
+        col = rng.normal(size=n) * 10 ** rng.uniform(-3, 3)
+        X[:, f] = col if kind == 0 else np.round(col, 0) if kind == 1 else rng.integers(0, 4, size=n) if kind == 2 else 1.5
+    objective = int(rng.integers(0, 2))
+    s = X[:, 0] / np.abs(X[:, 0]).max() * 3 + (X[:, F - 1] > np.median(X[:, F - 1]))
+    y = (s + 0.3 * rng.normal(size=n)).astype(np.float32) if objective == 0 else \
+        (rng.random(n) < 1 / (1 + np.exp(-s))).astype(np.float32)
+    cfg = {"objective": objective, "method": 0,
+           "internals": {"double_precision": bool(rng.integers(0, 2)), "exact_sort": 1, "seed": int(rng.integers(0, 99))},
+           "tree": {"max_depth": int(rng.integers(1, 8)), "eta": float(rng.uniform(0.05, 1.0)),
+                    "lambda": float(rng.choice([0.0, 0.5, 2.0])), "alpha": float(rng.choice([0.0, 0.0, 0.3])),
+                    "min_child_weight": float(rng.choice([0.0, 1.0, 5.0])), "min_leaf_size": int(rng.choice([0, 1, 2, 20])),
+                    "gamma_absolute": float(rng.choice([0.0, 0.0, 0.5])), "gamma_relative": float(rng.choice([0.0, 0.0, 0.01])),
+                    "max_leaf_weight": float(rng.choice([0.0, 0.0, 0.7])),
+                    "colsample_bytree": float(rng.choice([1.0, 1.0, 0.8])) if F > 2 else 1.0,
+                    "colsample_bylevel": float(rng.choice([1.0, 1.0, 0.8])) if F > 2 else 1.0}}
+    _same_trees(oracle.Booster(X, y=y, config=cfg), arb.Garden(cfg, arb.DMatrix(X, y=y)), 3)
+
+
 def test_sorted_lists_beyond_the_checker(arb):
     # 300 000 distinct values per feature, more than the checker's exact mode holds: what does not
     # depend on the size.  A strictly increasing map of a feature changes no rank, so the trees
