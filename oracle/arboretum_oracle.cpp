@@ -46,6 +46,11 @@
 //                       engine; set sizes and split-feature membership; the
 //                       two error strings.  (The draw itself is the standard
 //                       library's std::shuffle on std::default_random_engine.)
+//   exact method        pinned: golden models of tests/py/test_regression.py and
+//                       tests/py/test_logresression.py, a plain-Python search over
+//                       every distinct value on seeded inputs; the 32-bit ranks of
+//                       features with more than 65535 distinct values against the
+//                       16-bit ones on the same input (orc_force_wide_ranks)
 //   orc_expf            defined here (double polynomial, correctly rounded in
 //                       all but rare cases); checked against libm within 1 ulp.
 // ---------------------------------------------------------------------------
@@ -368,6 +373,11 @@ struct Booster {
   std::vector<std::vector<float>> thr;
   std::vector<int> size;
   std::vector<uint16_t> bins;  // row-major [n][F]
+  // exact method with more than 65535 distinct values in a feature: the ranks, instead of `bins`
+  std::vector<uint32_t> wide_bins;
+  uint32_t bin_at(size_t i, int f) const {
+    return wide_bins.empty() ? bins[i * (size_t)F + f] : wide_bins[i * (size_t)F + f];
+  }
   std::vector<float> y, yhat, g, h;
   std::vector<uint8_t> labels;
   std::vector<TreeOut> trees;
@@ -597,9 +607,14 @@ static void grow_tree(Booster &b, int label) {
         uint32_t nd = node[i];
         if (!direct[nd]) continue;
         ++scanned;
-        const uint16_t *br = &b.bins[(size_t)i * F];
         Acc *hn = &hist[(size_t)nd * F * SL];
-        for (int f = 0; f < F; ++f) acc_add(hn[(size_t)f * SL + br[f]], b, g[i], pair ? h[i] : 0.0f, gq[i], hq[i]);
+        if (b.wide_bins.empty()) {
+          const uint16_t *br = &b.bins[(size_t)i * F];
+          for (int f = 0; f < F; ++f) acc_add(hn[(size_t)f * SL + br[f]], b, g[i], pair ? h[i] : 0.0f, gq[i], hq[i]);
+        } else {
+          const uint32_t *br = &b.wide_bins[(size_t)i * F];
+          for (int f = 0; f < F; ++f) acc_add(hn[(size_t)f * SL + br[f]], b, g[i], pair ? h[i] : 0.0f, gq[i], hq[i]);
+        }
       }
     } else {
 #ifdef _OPENMP
@@ -615,10 +630,9 @@ static void grow_tree(Booster &b, int label) {
           uint32_t nd = node[i];
           if (!direct[nd]) continue;
           ++scanned;
-          const uint16_t *br = &b.bins[(size_t)i * F];
           int64_t *hn = &pv[(size_t)nd * F * SL * 3];
           for (int f = 0; f < F; ++f) {
-            int64_t *c = hn + ((size_t)f * SL + br[f]) * 3;
+            int64_t *c = hn + ((size_t)f * SL + b.bin_at((size_t)i, f)) * 3;
             c[0] += gq[i];
             c[1] += hq[i];
             c[2] += 1;
@@ -716,7 +730,7 @@ static void grow_tree(Booster &b, int label) {
       uint32_t nd = node[i];
       const Best &bs = best[nd];
       uint32_t right = 0;
-      if (bs.fid >= 0) right = b.bins[(size_t)i * F + bs.fid] >= (unsigned)(bs.bin + 1);
+      if (bs.fid >= 0) right = b.bin_at((size_t)i, bs.fid) >= (unsigned)(bs.bin + 1);
       node[i] = nd * 2 + right;
     }
     tot.swap(next);
@@ -768,6 +782,8 @@ static void tree_predict(const TreeOut &t, const float *X, int64_t n, int F, flo
 }  // namespace
 
 // ============================================================== C interface
+static bool g_force_wide_ranks = false;
+
 extern "C" {
 
 float orc_expf(float x) { return orc_expf_impl(x); }
@@ -851,13 +867,20 @@ void *orc_create(const float *X, int64_t n, int F, const float *y, const uint8_t
       std::sort(m.begin(), m.end());
       m.erase(std::unique(m.begin(), m.end()), m.end());
       most = std::max(most, m.size());
-      for (int64_t i = 0; i < n; ++i)
-        b->bins[(size_t)i * F + f] =
-            (uint16_t)(std::lower_bound(m.begin(), m.end(), X[(size_t)i * F + f]) - m.begin());
     }
-    if (most > 65535) {
-      delete b;
-      return nullptr;
+    if (most > 65535 || g_force_wide_ranks) {  // ranks beyond 16 bits
+      b->bins.clear();
+      b->wide_bins.resize((size_t)n * F);
+    }
+    for (int f = 0; f < F; ++f) {
+      const std::vector<float> &m = mapping[f];
+      for (int64_t i = 0; i < n; ++i) {
+        const size_t r = std::lower_bound(m.begin(), m.end(), X[(size_t)i * F + f]) - m.begin();
+        if (b->wide_bins.empty())
+          b->bins[(size_t)i * F + f] = (uint16_t)r;
+        else
+          b->wide_bins[(size_t)i * F + f] = (uint32_t)r;
+      }
     }
     b->p.hist_size = (int)most;
     b->slots = (int)most + 1;
@@ -933,6 +956,9 @@ int orc_get_active(void *hd, int t, int level, unsigned *out) {
   return (int)a.size();
 }
 
+// Test switch: exact-mode boosters created from now on keep their ranks in 32 bits whatever the
+// number of distinct values (the branch that more than 65535 distinct values take).
+void orc_force_wide_ranks(int on) { g_force_wide_ranks = on != 0; }
 int orc_hist_size(void *hd) { return static_cast<Booster *>(hd)->p.hist_size; }  // exact: distinct values
 int orc_num_trees(void *hd) { return (int)static_cast<Booster *>(hd)->trees.size(); }
 uint64_t orc_updates(void *hd) { return static_cast<Booster *>(hd)->updates; }
@@ -961,7 +987,7 @@ void orc_get_grad(void *hd, float *g, float *h) {
   std::memcpy(g, b.g.data(), b.g.size() * sizeof(float));
   if (h) std::memcpy(h, b.h.data(), b.h.size() * sizeof(float));
 }
-void orc_get_bins(void *hd, uint16_t *out) {
+void orc_get_bins(void *hd, uint16_t *out) {  // (ranks beyond 16 bits are not handed out: nothing is written)
   Booster &b = *static_cast<Booster *>(hd);
   std::memcpy(out, b.bins.data(), b.bins.size() * sizeof(uint16_t));
 }

@@ -93,6 +93,7 @@ def lib():
         L.orc_get_leaf.argtypes = [ctypes.c_void_p, ctypes.c_void_p]
         L.orc_get_yhat.argtypes = [ctypes.c_void_p, ctypes.c_void_p]
         L.orc_get_grad.argtypes = [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p]
+        L.orc_force_wide_ranks.argtypes = [ctypes.c_int]
         L.orc_get_bins.argtypes = [ctypes.c_void_p, ctypes.c_void_p]
         L.orc_get_thresholds.argtypes = [ctypes.c_void_p, ctypes.c_int, ctypes.c_void_p,
                                          ctypes.POINTER(ctypes.c_int)]
@@ -139,6 +140,12 @@ def params_from_config(config, accum=0, threads=0):
     )
 
 
+def force_wide_ranks(on):
+    """Test switch: exact-mode boosters created from now on keep 32-bit ranks (the branch of more
+    than 65535 distinct values per feature)."""
+    lib().orc_force_wide_ranks(1 if on else 0)
+
+
 def quantize_column(x, hist_size):
     x = np.ascontiguousarray(x, dtype=np.float32)
     thr = np.empty(hist_size, dtype=np.float32)
@@ -174,7 +181,7 @@ class Booster:
             self.h = lib().orc_create(_p(X), self.n, self.F, _p(y), _p(labels),
                                       ctypes.byref(self.params))
         if not self.h:
-            raise ValueError("the checker's exact mode holds at most 65535 distinct values per feature")
+            raise ValueError("the checker could not take the matrix")
         self.K = self.params.labels_count
         self.params.hist_size = lib().orc_hist_size(self.h)   # exact method: the largest number of distinct values
 
@@ -234,6 +241,8 @@ class Booster:
         return g, h
 
     def bins(self):
+        if self.params.hist_size > 65535:
+            raise ValueError("ranks beyond 16 bits (exact mode, more than 65535 distinct values) are not handed out")
         out = np.empty((self.n, self.F), np.uint16)
         lib().orc_get_bins(self.h, _p(out))
         return out

@@ -110,7 +110,7 @@ def _same_trees(ob, g, rounds, data=None):
 @pytest.mark.parametrize("n,F,depth", [(30000, 4, 5), (60000, 3, 7), (5000, 5, 2)])
 def test_sorted_lists_match_the_checker(arb, oracle, objective, double_precision, n, F, depth):
     # more than 4096 distinct values per feature (5000 rows: forced): every feature keeps its rows
-    # sorted by value instead of a histogram over ranks; the checker's exact mode holds up to 65535
+    # sorted by value instead of a histogram over ranks
     X, y = _continuous(n, F, objective, seed=n + depth)
     assert len(np.unique(X[:, 0])) > min(n, 4096) * 0.99
     cfg = {"objective": objective, "method": 0,
@@ -193,9 +193,25 @@ def test_sorted_lists_on_random_configurations(arb, oracle, seed):
     _same_trees(oracle.Booster(X, y=y, config=cfg), arb.Garden(cfg, arb.DMatrix(X, y=y)), 3)
 
 
+@pytest.mark.parametrize("objective", [0, 1])
+def test_sorted_lists_match_the_checker_beyond_16_bit_ranks(arb, oracle, objective):
+    # 100 000 distinct values per feature: the checker's exact mode with 32-bit ranks
+    n = 100000
+    rng = np.random.default_rng(5 + objective)
+    X = (rng.permutation(2 * n).reshape(n, 2) / 8.0).astype(np.float32)        # all distinct, exact in float32
+    s = np.sin(X[:, 0] / 3000.0) + (X[:, 1] > 9000.0)
+    y = (s + 0.2 * rng.normal(size=n)).astype(np.float32) if objective == 0 else \
+        (rng.random(n) < 1 / (1 + np.exp(-2 * s + 1))).astype(np.float32)
+    cfg = {"objective": objective, "method": 0, "internals": {"double_precision": True},
+           "tree": {"max_depth": 5, "eta": 0.5, "lambda": 1.0, "min_child_weight": 1.0}}
+    ob = oracle.Booster(X, y=y, config=cfg)
+    assert ob.params.hist_size == n
+    _same_trees(ob, arb.Garden(cfg, arb.DMatrix(X, y=y)), 2)
+
+
 def test_sorted_lists_beyond_the_checker(arb):
-    # 300 000 distinct values per feature, more than the checker's exact mode holds: what does not
-    # depend on the size.  A strictly increasing map of a feature changes no rank, so the trees
+    # 300 000 distinct values per feature and six levels, more than the checker's rank histograms
+    # hold in reasonable memory: what does not depend on the size.  A strictly increasing map of a feature changes no rank, so the trees
     # keep their features, ranks, gains, weights and leaves, and every threshold maps with it; the
     # root split is the best of all places by a float64 restatement of the squared-error gain;
     # prediction from the thresholds reproduces the tracked y_hat (rank <= q <=> value < threshold).

@@ -245,6 +245,36 @@ def test_exact_root_split_against_brute_force(oracle, objective, seed):
 
 
 @pytest.mark.parametrize("objective", [0, 1])
+@pytest.mark.parametrize("accum", [0, 1])
+def test_exact_mode_with_ranks_beyond_16_bits(oracle, objective, accum):
+    # More than 65535 distinct values in a feature: the checker keeps 32-bit ranks.  Nothing else
+    # of the exact mode differs, so with the switch that forces that branch the trees, leaves and
+    # predictions are those of the 16-bit ranks (which the goldens and the brute force above pin).
+    rng = np.random.default_rng(77 + objective)
+    n, F = 3000, 4
+    X = rng.normal(size=(n, F)).astype(np.float32)
+    X[:, 2] = np.round(X[:, 2], 1)
+    y = (X[:, 0] + X[:, 2] > 0).astype(np.float32) if objective else (X[:, 0] * 2 + rng.normal(size=n)).astype(np.float32)
+    cfg = {"objective": objective, "method": 0, "internals": {"double_precision": True},
+           "tree": {"max_depth": 5, "eta": 0.5, "lambda": 1.0, "min_child_weight": 1.0}}
+    grown = []
+    try:
+        for wide in (False, True):
+            oracle.force_wide_ranks(wide)
+            b = oracle.Booster(X, y=y, config=cfg, accum=accum)
+            b.grow(3)
+            grown.append(([b.tree(t) for t in range(3)], b.leaf(), b.yhat(), b.predict(X)))
+    finally:
+        oracle.force_wide_ranks(False)
+    for ta, tb in zip(grown[0][0], grown[1][0]):
+        for key in ta:
+            assert np.array_equal(ta[key], tb[key], equal_nan=True), key
+    assert (grown[0][0][2]["quantized"] >= 0).sum() > 20
+    for k in (1, 2, 3):
+        assert np.array_equal(grown[0][k], grown[1][k])
+
+
+@pytest.mark.parametrize("objective", [0, 1])
 @pytest.mark.parametrize("seed", range(6))
 def test_hist_root_split_against_brute_force(oracle, objective, seed):
     # The histogram method chooses among the bins what the exact search chooses among the values
