@@ -29,9 +29,9 @@ def _draw(seed):
     cfg = {"objective": objective, "method": 1,
            "internals": {"hist_size": hist_size, "double_precision": bool(rng.integers(0, 2)),
                          "use_hist_subtraction_trick": bool(rng.integers(0, 2)),
-                         # 16-bit bins (more than 256 ids per feature: 256 thresholds and a bin for
-                         # missing values already need them) are resident only
-                         "upload_features": bool(rng.random() < 0.75) or hist_size > 255,
+                         # 16-bit bins (more than 257 ids per feature) are resident only; 256 thresholds
+                         # and a bin for missing values stay on the 8-bit kernels, streamed too
+                         "upload_features": bool(rng.random() < 0.75) or hist_size > 256,
                          "stream_block_rows": int(rng.choice([64, 1000, 5000, 1 << 20])),
                          "seed": int(rng.integers(0, 100))},
            "tree": {"max_depth": depth, "eta": float(rng.choice([0.1, 0.3, 1.0])),
