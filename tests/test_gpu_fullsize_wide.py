@@ -1,10 +1,10 @@
 """BASELINE configs[2] (50 M x 200, 30 % missing, 65 bin ids, squared error, max_depth 10) and
-configs[3] (20 M x 100, 10 soft-max classes, max_depth 6) at their full sizes.  The CPU checker
-does not finish these in a test's time, so the trees are checked through what holds at any size:
+configs[3] (20 M x 100, 10 soft-max classes, max_depth 6) at their full sizes, and the out-of-core
+shape (64 M x 128 streamed).  The trees are checked through what holds at any size:
 every row's leaf against a host walk of the tree over the bin ids, every leaf weight against its
 definition on the rows the leaf holds, the prediction update against leaf weight + old value, and
 the root split against histograms built with numpy (gain from the checker's pinned gain function,
-ties as the reference breaks them)."""
+ties as the reference breaks them); and, in tests of their own, against the CPU checker bit for bit."""
 import os
 import sys
 
@@ -165,3 +165,62 @@ def test_configs4_streamed_tree_properties(arb, oracle):
     assert np.array_equal(after, before + tree["weights"][leaf]), "prediction update"
     others = [int(f) for f in np.random.default_rng(8).choice(F, 5, replace=False)]
     _check_root_split(oracle, tree, bins, g, h, 3, sorted(set([int(tree["fid"][0])] + others)), 256, lam)
+
+
+def _same_as_checker(ob, model, trees, leaves=True):
+    for t in trees:
+        to, tg = ob.tree(t), model.tree(t)
+        for key in ("fid", "quantized", "gain"):
+            assert np.array_equal(to[key], tg[key]), (key, t)
+        assert np.array_equal(to["weights"], tg["weights"], equal_nan=True), t
+    if leaves:
+        assert np.array_equal(ob.leaf(), model.leaves())
+    assert np.array_equal(ob.yhat(), model.train_yhat())
+
+
+# The checker on the host cores of the GPU machine finishes a tree of these sizes in 10 to 25
+# seconds, so the full-size configurations are also held to it bit for bit: every split, gain and
+# leaf weight, the leaf of every row, the prediction update.
+
+@pytest.mark.timeout(900)
+def test_configs2_full_size_against_the_checker(arb, oracle):
+    import bench
+    bins, y = bench.make_config2_bins(50_000_000, 200)
+    cfg = {"objective": 0, "method": 1, "internals": {"hist_size": 64, "double_precision": True},
+           "tree": {"max_depth": 10, "eta": 0.3, "lambda": 1.0}}
+    model = arb.Garden(cfg, arb.DMatrix(bins, y=y, quantized=True))
+    ob = oracle.Booster(bins, y=y, config=cfg, binned=True)
+    for r in range(2):
+        ob.grow(1)
+        model.grow_tree()
+        _same_as_checker(ob, model, [r])
+
+
+@pytest.mark.timeout(900)
+def test_configs3_full_size_against_the_checker(arb, oracle):
+    import bench
+    K = 10
+    X, labels = bench.make_config3(20_000_000, 100, K)
+    cfg = {"objective": 4, "method": 1, "internals": {"hist_size": 256, "double_precision": True},
+           "tree": {"max_depth": 6, "eta": 0.2, "lambda": 1.0, "labels_count": K}}
+    model = arb.Garden(cfg, arb.DMatrix(X, labels=labels))
+    ob = oracle.Booster(X, labels=labels, config=cfg)
+    ob.grow(1)
+    model.grow_tree()
+    _same_as_checker(ob, model, range(K), leaves=False)
+
+
+@pytest.mark.timeout(900)
+def test_configs4_streamed_against_the_checker(arb, oracle):
+    # 64 M x 128 bin ids in pinned host blocks of 4 M rows, half of them kept in device memory
+    import bench
+    bins, y = bench.make_stream_workload(64_000_000, 128)
+    cfg = bench.config(8, 256)
+    cfg["internals"].update({"upload_features": False, "stream_block_rows": 1 << 22,
+                             "stream_resident_bytes": 8 * (1 << 22) * 128 + 4096})
+    model = arb.Garden(cfg, arb.DMatrix(bins, y=y, quantized=True))
+    ob = oracle.Booster(bins, y=y, config=cfg, binned=True)
+    ob.grow(1)
+    model.grow_tree()
+    _same_as_checker(ob, model, [0])
+    assert model.stream_residency() == (8, 16)
