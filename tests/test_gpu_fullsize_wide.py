@@ -4,7 +4,7 @@ shape (64 M x 128 streamed).  The trees are checked through what holds at any si
 every row's leaf against a host walk of the tree over the bin ids, every leaf weight against its
 definition on the rows the leaf holds, the prediction update against leaf weight + old value, and
 the root split against histograms built with numpy (gain from the checker's pinned gain function,
-ties as the reference breaks them); and, in tests of their own, against the CPU checker bit for bit."""
+ties as the reference breaks them); and the first trees of each against the CPU checker bit for bit."""
 import os
 import sys
 
@@ -80,8 +80,22 @@ def _check_root_split(oracle, tree, bins, g, h, kind, features, slots, lam):
                 "feature %d beats the chosen feature %d" % (f, f0)
 
 
+def _same_as_checker(ob, model, trees, leaves=True):
+    """Every split, gain and leaf weight of the given trees, the leaf of every row and the
+    predictions against the CPU checker, bit for bit (the checker on the host cores of the GPU
+    machine finishes a tree of these sizes in 10 to 25 seconds)."""
+    for t in trees:
+        to, tg = ob.tree(t), model.tree(t)
+        for key in ("fid", "quantized", "gain"):
+            assert np.array_equal(to[key], tg[key]), (key, t)
+        assert np.array_equal(to["weights"], tg["weights"], equal_nan=True), t
+    if leaves:
+        assert np.array_equal(ob.leaf(), model.leaves())
+    assert np.array_equal(ob.yhat(), model.train_yhat())
+
+
 @pytest.mark.timeout(900)
-def test_configs2_full_size_tree_properties(arb, oracle):
+def test_configs2_full_size(arb, oracle):
     import bench
     rows, F, depth, eta, lam = 50_000_000, 200, 10, 0.3, 1.0
     bins, y = bench.make_config2_bins(rows, F)
@@ -89,9 +103,15 @@ def test_configs2_full_size_tree_properties(arb, oracle):
     cfg = {"objective": 0, "method": 1, "internals": {"hist_size": 64, "double_precision": True},
            "tree": {"max_depth": depth, "eta": eta, "lambda": lam, "min_child_weight": 1.0, "min_leaf_size": 1}}
     model = arb.Garden(cfg, data)
+    ob = oracle.Booster(bins, y=y, config=cfg, binned=True)
     model.grow_tree()
+    ob.grow(1)
+    _same_as_checker(ob, model, [0])
     before = model.train_yhat()
     model.grow_tree()
+    ob.grow(1)
+    _same_as_checker(ob, model, [1])
+    del ob
     tree, leaf, after = model.tree(1), model.leaves(), model.train_yhat()
     assert (tree["quantized"] >= 0).sum() > 900, "not a full depth-10 tree"
     assert np.array_equal(leaf, _walk(tree, bins, depth)), "row -> leaf"
@@ -104,17 +124,21 @@ def test_configs2_full_size_tree_properties(arb, oracle):
 
 
 @pytest.mark.timeout(900)
-def test_configs3_full_size_tree_properties(arb, oracle):
+def test_configs3_full_size(arb, oracle):
     import bench
     rows, F, K, depth, eta, lam = 20_000_000, 100, 10, 6, 0.2, 1.0
     X, labels = bench.make_config3(rows, F, K)
     data = arb.DMatrix(X, labels=labels)
-    del X
     cfg = {"objective": 4, "method": 1, "internals": {"hist_size": 256, "double_precision": True},
            "tree": {"max_depth": depth, "eta": eta, "lambda": lam, "min_child_weight": 1.0, "min_leaf_size": 1,
                     "labels_count": K}}
     model = arb.Garden(cfg, data)
     model.grow_tree()
+    ob = oracle.Booster(X, labels=labels, config=cfg)      # the first round against the checker
+    del X
+    ob.grow(1)
+    _same_as_checker(ob, model, range(K), leaves=False)
+    del ob
     k = K - 1                                                 # the last tree of a round belongs to the last class
     start = model.train_yhat().reshape(K, rows).copy()        # the scores the second round starts from
     model.set_inspect(True)                                   # keeps the round's gradients for grad()
@@ -142,18 +166,24 @@ def test_configs3_full_size_tree_properties(arb, oracle):
 
 
 @pytest.mark.timeout(900)
-def test_configs4_streamed_tree_properties(arb, oracle):
+def test_configs4_streamed(arb, oracle):
     # the out-of-core shape as the benchmark runs it: 64 M x 128 bin ids (8.2 GB) in pinned host
-    # memory, streamed in blocks of 4 M rows at every level; logistic objective, max_depth 8
+    # memory in blocks of 4 M rows, half of them kept in device memory, the others streamed at every
+    # level; logistic objective, max_depth 8
     import bench
     rows, F, depth, eta, lam = 64_000_000, 128, 8, 0.1, 1.0
     bins, y = bench.make_stream_workload(rows, F)
     cfg = bench.config(depth, 256)
-    cfg["internals"]["upload_features"] = False
-    cfg["internals"]["stream_block_rows"] = 1 << 22
+    cfg["internals"].update({"upload_features": False, "stream_block_rows": 1 << 22,
+                             "stream_resident_bytes": 8 * (1 << 22) * F + 4096})
     data = arb.DMatrix(bins, y=y, quantized=True)
     model = arb.Garden(cfg, data)
+    ob = oracle.Booster(bins, y=y, config=cfg, binned=True)
     model.grow_tree()
+    ob.grow(1)
+    _same_as_checker(ob, model, [0])
+    del ob
+    assert model.stream_residency() == (8, 16)
     before = model.train_yhat()
     model.grow_tree()
     tree, leaf, after = model.tree(1), model.leaves(), model.train_yhat()
@@ -165,62 +195,3 @@ def test_configs4_streamed_tree_properties(arb, oracle):
     assert np.array_equal(after, before + tree["weights"][leaf]), "prediction update"
     others = [int(f) for f in np.random.default_rng(8).choice(F, 5, replace=False)]
     _check_root_split(oracle, tree, bins, g, h, 3, sorted(set([int(tree["fid"][0])] + others)), 256, lam)
-
-
-def _same_as_checker(ob, model, trees, leaves=True):
-    for t in trees:
-        to, tg = ob.tree(t), model.tree(t)
-        for key in ("fid", "quantized", "gain"):
-            assert np.array_equal(to[key], tg[key]), (key, t)
-        assert np.array_equal(to["weights"], tg["weights"], equal_nan=True), t
-    if leaves:
-        assert np.array_equal(ob.leaf(), model.leaves())
-    assert np.array_equal(ob.yhat(), model.train_yhat())
-
-
-# The checker on the host cores of the GPU machine finishes a tree of these sizes in 10 to 25
-# seconds, so the full-size configurations are also held to it bit for bit: every split, gain and
-# leaf weight, the leaf of every row, the prediction update.
-
-@pytest.mark.timeout(900)
-def test_configs2_full_size_against_the_checker(arb, oracle):
-    import bench
-    bins, y = bench.make_config2_bins(50_000_000, 200)
-    cfg = {"objective": 0, "method": 1, "internals": {"hist_size": 64, "double_precision": True},
-           "tree": {"max_depth": 10, "eta": 0.3, "lambda": 1.0}}
-    model = arb.Garden(cfg, arb.DMatrix(bins, y=y, quantized=True))
-    ob = oracle.Booster(bins, y=y, config=cfg, binned=True)
-    for r in range(2):
-        ob.grow(1)
-        model.grow_tree()
-        _same_as_checker(ob, model, [r])
-
-
-@pytest.mark.timeout(900)
-def test_configs3_full_size_against_the_checker(arb, oracle):
-    import bench
-    K = 10
-    X, labels = bench.make_config3(20_000_000, 100, K)
-    cfg = {"objective": 4, "method": 1, "internals": {"hist_size": 256, "double_precision": True},
-           "tree": {"max_depth": 6, "eta": 0.2, "lambda": 1.0, "labels_count": K}}
-    model = arb.Garden(cfg, arb.DMatrix(X, labels=labels))
-    ob = oracle.Booster(X, labels=labels, config=cfg)
-    ob.grow(1)
-    model.grow_tree()
-    _same_as_checker(ob, model, range(K), leaves=False)
-
-
-@pytest.mark.timeout(900)
-def test_configs4_streamed_against_the_checker(arb, oracle):
-    # 64 M x 128 bin ids in pinned host blocks of 4 M rows, half of them kept in device memory
-    import bench
-    bins, y = bench.make_stream_workload(64_000_000, 128)
-    cfg = bench.config(8, 256)
-    cfg["internals"].update({"upload_features": False, "stream_block_rows": 1 << 22,
-                             "stream_resident_bytes": 8 * (1 << 22) * 128 + 4096})
-    model = arb.Garden(cfg, arb.DMatrix(bins, y=y, quantized=True))
-    ob = oracle.Booster(bins, y=y, config=cfg, binned=True)
-    ob.grow(1)
-    model.grow_tree()
-    _same_as_checker(ob, model, [0])
-    assert model.stream_residency() == (8, 16)
