@@ -152,6 +152,39 @@ k_ex_offsets(const T *__restrict__ part, T *__restrict__ off, const unsigned *__
   }
 }
 
+// SplitGain (gain.h) with the parent's term, which is the same at every place of a node, taken
+// from the caller: `parent` = SideGain of the node's totals at their leaf weight.  The same
+// operations in the same order, so the same bits.
+template <bool PAIR, bool F64>
+__device__ __forceinline__ float ExParentGain(double gt, double ht, unsigned long long ct, const GainParams &p) {
+  return SideGain<PAIR, F64>(gt, ht, ct, LeafWeight<PAIR, F64>(gt, ht, ct, p), p);
+}
+template <bool PAIR, bool F64>
+__device__ __forceinline__ float ExSplitGain(double gl, double hl, unsigned long long cl, double gt, double ht,
+                                             unsigned long long ct, const GainParams &p, float parent) {
+  const unsigned long long cr = ct - cl;
+  double gr, hr;
+  if (F64) {
+    gr = gt - gl;
+    hr = ht - hl;
+  } else {
+    gr = (double)((float)gt - (float)gl);
+    hr = (double)((float)ht - (float)hl);
+  }
+  if (cl < p.min_leaf_size || cr < p.min_leaf_size) return 0.0f;
+  if (PAIR) {
+    if (F64) {
+      if (!(fabs(hl) >= (double)p.min_child_weight && fabs(hr) >= (double)p.min_child_weight)) return 0.0f;
+    } else {
+      if (!(fabsf((float)hl) >= p.min_child_weight && fabsf((float)hr) >= p.min_child_weight)) return 0.0f;
+    }
+  }
+  const float l = SideGain<PAIR, F64>(gl, hl, cl, LeafWeight<PAIR, F64>(gl, hl, cl, p), p);
+  const float r = SideGain<PAIR, F64>(gr, hr, cr, LeafWeight<PAIR, F64>(gr, hr, cr, p), p);
+  const float diff = l + r - parent;
+  return (float)(diff > p.gamma_absolute && diff > p.gamma_relative * parent) * diff;
+}
+
 __device__ __forceinline__ bool ExBetter(float og, int ob, float gain, int bin) {
   return ob >= 0 && (bin < 0 || og > gain || (og == gain && ob > bin));
 }
@@ -196,6 +229,7 @@ k_ex_scan(const ExLists ls, size_t stride, const int *__restrict__ shifts,
   mine.left.c = 0;
   const double GT = FromFixed<F64>(t.g, sg);
   const double HT = PAIR ? FromFixed<F64>(t.h, sh) : 0.0;
+  const float parent = ExParentGain<PAIR, F64>(GT, HT, t.c, gp);
 #pragma unroll
   for (int j = 0; j < kExPer; ++j) {
     const unsigned p = p0 + j;
@@ -204,7 +238,7 @@ k_ex_scan(const ExLists ls, size_t stride, const int *__restrict__ shifts,
       const unsigned long long lc = p - node_start + 1;
       const double GL = FromFixed<F64>(lg, sg);
       const double HL = PAIR ? FromFixed<F64>(lh, sh) : 0.0;
-      const float gn = SplitGain<PAIR, F64>(GL, HL, lc, GT, HT, t.c, gp);
+      const float gn = ExSplitGain<PAIR, F64>(GL, HL, lc, GT, HT, t.c, gp, parent);
       if (gn > 0.0f && gn >= mine.gain) {
         mine.gain = gn;
         mine.bin = (int)(rk[j + 1] - 1u);
