@@ -572,6 +572,18 @@ void LaunchFused(int nq, hipStream_t st, unsigned grid, const FusedArgs &a) {
 class HipTreeBuilder : public TreeBuilder {
  public:
   HipTreeBuilder(const Configuration &cfg, DataMatrix *data) : cfg_(cfg), data_(data) {
+    try {
+      Construct(cfg, data);
+    } catch (...) {  // e.g. out of device memory: give back what was allocated so far
+      Release();
+      throw;
+    }
+  }
+
+  ~HipTreeBuilder() override { Release(); }
+
+ private:
+  void Construct(const Configuration &cfg, DataMatrix *data) {
     dm_ = data->device;
     n_ = dm_->rows;
     F_ = dm_->F;
@@ -812,8 +824,8 @@ class HipTreeBuilder : public TreeBuilder {
     if (streamed_) KeepBlocksResident(cfg.internal.stream_resident_bytes);
   }
 
-  ~HipTreeBuilder() override {
-    (void)hipStreamSynchronize(stream_);
+  void Release() noexcept {
+    if (stream_) (void)hipStreamSynchronize(stream_);
     void *ptrs[] = {d_y_, d_labels_, d_yhat_, d_g_, d_h_, d_leaf_, d_split_, d_cand_, d_node_first2_,
                     d_node_items2_, d_hwork_, d_pwork_, d_nwork_, d_wave_left_, d_item_left_, d_slab_,
                     d_shifts_, d_gmax_, d_rows_scanned_, d_tfid_, d_tbin_, d_tgain_, d_weights_, d_active_, d_overflow_, d_records_, d_cursor2_};
@@ -828,20 +840,21 @@ class HipTreeBuilder : public TreeBuilder {
     for (uint32_t *p : resident_)
       if (p) (void)hipFree(p);
     if (streamed_) {
-      (void)hipStreamSynchronize(copy_stream_);
+      if (copy_stream_) (void)hipStreamSynchronize(copy_stream_);
       void *sp[] = {blk_[0], blk_[1], stage_.bins, stage_.g, stage_.h, d_node_of_, d_blk_cnt_, d_blk_seg_,
                     d_cursor_, d_blk_tot_};
       for (void *p : sp)
         if (p) (void)hipFree(p);
       for (int b = 0; b < 2; ++b) {
-        (void)hipEventDestroy(ev_ready_[b]);
-        (void)hipEventDestroy(ev_free_[b]);
+        if (ev_ready_[b]) (void)hipEventDestroy(ev_ready_[b]);
+        if (ev_free_[b]) (void)hipEventDestroy(ev_free_[b]);
       }
-      (void)hipStreamDestroy(copy_stream_);
+      if (copy_stream_) (void)hipStreamDestroy(copy_stream_);
     }
-    (void)hipStreamDestroy(stream_);
+    if (stream_) (void)hipStreamDestroy(stream_);
   }
 
+ public:
   void GrowRound(std::vector<RegTree> *trees) override {
     // Gradients of this round, unless the last pass of the previous tree has
     // already written them (single-output objectives, inspection off).

@@ -120,6 +120,17 @@ namespace {
 class ExactSortBuilder : public TreeBuilder {
  public:
   ExactSortBuilder(const Configuration &cfg, DataMatrix *data) : cfg_(cfg), data_(data) {
+    try {
+      Construct(cfg, data);
+    } catch (...) {  // e.g. out of device memory: give back what was allocated so far
+      Release();
+      throw;
+    }
+  }
+  ~ExactSortBuilder() override { Release(); }
+
+ private:
+  void Construct(const Configuration &cfg, DataMatrix *data) {
     sd_ = data->exact_sort;
     n_ = sd_->rows;
     F_ = sd_->F;
@@ -210,8 +221,8 @@ class ExactSortBuilder : public TreeBuilder {
     HIP_OK(hipStreamSynchronize(stream_));
   }
 
-  ~ExactSortBuilder() override {
-    (void)hipStreamSynchronize(stream_);
+  void Release() noexcept {
+    if (stream_) (void)hipStreamSynchronize(stream_);
     void *all[] = {d_y_, d_labels_, d_yhat_, d_g_, d_h_, d_leaf_, d_node_of_, d_went_right_, d_gh_, d_ids_[0], d_ids_[1], d_ranks_[0],
                    d_ranks_[1], d_lg_[0], d_lg_[1], d_lh_[0], d_lh_[1], d_tot_[0],
                    d_tot_[1], d_seg_[0], d_seg_[1], d_split_, d_cand_, d_work_, d_n_work_, d_node_first_,
@@ -219,9 +230,10 @@ class ExactSortBuilder : public TreeBuilder {
                    d_overflow_, d_tfid_, d_tbin_, d_tgain_, d_weights_, d_active_};
     for (void *p : all)
       if (p) (void)hipFree(p);
-    (void)hipStreamDestroy(stream_);
+    if (stream_) (void)hipStreamDestroy(stream_);
   }
 
+ public:
   void GrowRound(std::vector<RegTree> *trees) override {
     if (cfg_.objective == kLinearRegression) {
       HIP_OK(hipMemsetAsync(d_gmax_, 0, sizeof(unsigned), stream_));
