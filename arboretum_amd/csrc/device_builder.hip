@@ -88,6 +88,7 @@ struct DeviceMatrix {
   uint32_t *bins = nullptr;  // resident: [cols][stride] in HBM
   // wide resident matrices, built on first use: the same bins row-major, RS words per row
   uint32_t *rec = nullptr;
+  unsigned rec_largest_id = 0;  // the largest bin id (byte) seen while the records were built
   int RS = 0;
   // and column-major with one byte per bin id: [4 Q][stride8]
   uint8_t *bytes = nullptr;
@@ -721,11 +722,20 @@ class HipTreeBuilder : public TreeBuilder {
         dm_->RS = (W_ + 15) / 16 * 16;  // (the ninth-bit words of a row follow its quads, in the columns and in the record)
         dm_->rec = DevAlloc<uint32_t>(n_ * (size_t)dm_->RS);
         AllowLds(k_to_records, (size_t)64 * (dm_->RS + 1) * sizeof(uint32_t));
+        unsigned *d_largest = DevAlloc<unsigned>(1);
+        HIP_OK(hipMemsetAsync(d_largest, 0, sizeof(unsigned), stream_));
         hipLaunchKernelGGL(k_to_records, dim3((unsigned)((n_ + 63) / 64)), dim3(256),
                            (size_t)64 * (dm_->RS + 1) * sizeof(uint32_t), stream_, dm_->bins, stride_, W_, dm_->rec,
-                           dm_->RS, n_);
+                           dm_->RS, n_, Q_, d_largest);
         HIP_OK(hipGetLastError());
+        HIP_OK(hipMemcpyAsync(&dm_->rec_largest_id, d_largest, sizeof(unsigned), hipMemcpyDeviceToHost, stream_));
+        HIP_OK(hipStreamSynchronize(stream_));
+        HIP_OK(hipFree(d_largest));
       }
+      // the histogram over the records is sized by max_bin and does not look at the ids again
+      if ((int)dm_->rec_largest_id > data->max_bin)
+        throw std::runtime_error("internal: the matrix holds bin id " + std::to_string(dm_->rec_largest_id) +
+                                 ", more than the " + std::to_string(data->max_bin) + " it was prepared for");
       if (hi_skip_ && !dm_->hibits) {
         dm_->strideb = (n_ + 7) / 8;
         dm_->strideb = (dm_->strideb + 63) / 64 * 64;
@@ -1119,23 +1129,20 @@ class HipTreeBuilder : public TreeBuilder {
         const int last_pieces = total - (ngroups - 1) * pieces;
         const bool pow2 = lay > 0 ? (lay & (lay - 1)) == 0
                                   : (pieces & (pieces - 1)) == 0 && (last_pieces & (last_pieces - 1)) == 0;
-        const bool clamp = slots < kSlots;
-#define ARB_REC(P, POW2, CLAMP, H)                                                                                \
+#define ARB_REC(P, POW2, H)                                                                                      \
   do {                                                                                                            \
     static std::once_flag configured;                                                                             \
-    AllowLdsOnce(configured, (k_hist_rec<P, POW2, CLAMP, H>), kLdsBudget);                                        \
-    hipLaunchKernelGGL((k_hist_rec<P, POW2, CLAMP, H>), dim3(blocks), dim3(kHistThreads), lds, stream_, dm_->rec, \
+    AllowLdsOnce(configured, (k_hist_rec<P, POW2, H>), kLdsBudget);                                               \
+    hipLaunchKernelGGL((k_hist_rec<P, POW2, H>), dim3(blocks), dim3(kHistThreads), lds, stream_, dm_->rec,        \
                        dm_->RS, cur.ids, Q_, slots, cur.g, cur.h, d_shifts_, d_hwork_, d_nwork_, d_slab_, pieces, \
                        total, ngroups, item_words, lay);                                                          \
   } while (0)
-#define ARB_REC_P(P)                                             \
-  do {                                                           \
-    if (hi_skip_ && pow2 && clamp) ARB_REC(P, true, true, true); \
-    else if (hi_skip_ && pow2) ARB_REC(P, true, false, true);    \
-    else if (hi_skip_) ARB_REC(P, false, true, true);            \
-    else if (pow2 && clamp) ARB_REC(P, true, true, false);       \
-    else if (pow2) ARB_REC(P, true, false, false);               \
-    else ARB_REC(P, false, true, false);                         \
+#define ARB_REC_P(P)                                   \
+  do {                                                 \
+    if (hi_skip_ && pow2) ARB_REC(P, true, true);      \
+    else if (hi_skip_) ARB_REC(P, false, true);        \
+    else if (pow2) ARB_REC(P, true, false);            \
+    else ARB_REC(P, false, false);                     \
   } while (0)
         if (pair_) ARB_REC_P(true);
         else ARB_REC_P(false);

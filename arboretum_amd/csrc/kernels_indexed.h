@@ -19,19 +19,26 @@ namespace arb {
 namespace {
 
 // Quad columns [Q][stride] -> records [rows][RS] (RS words per row, the words
-// past Q zero).  A workgroup transposes 64 rows through LDS: the reads are
+// past Q zero); the first id_quads of them hold bin ids, four bytes each, whose
+// largest is reported (atomic max on *largest_id).  A workgroup transposes 64 rows through LDS: the reads are
 // coalesced along the rows, the writes along the record.
 __global__ void __launch_bounds__(256)
 k_to_records(const uint32_t *__restrict__ bins, size_t stride, int Q, uint32_t *__restrict__ rec, int RS,
-             size_t n) {
+             size_t n, int id_quads, unsigned *__restrict__ largest_id) {
   extern __shared__ uint32_t s_tile[];  // [64][RS + 1]
   const size_t r0 = (size_t)blockIdx.x * 64;
   const int lane = threadIdx.x & 63, part = threadIdx.x >> 6;  // 4 parts
+  unsigned top = 0;  // the largest bin id (byte) among the words this thread moves
   for (int q = part; q < RS; q += 4) {
     uint32_t v = 0;
     if (q < Q && r0 + lane < n) v = bins[(size_t)q * stride + r0 + lane];
+    if (q < id_quads) top = max(max(top, v & 255u), max(max((v >> 8) & 255u, (v >> 16) & 255u), v >> 24));
     s_tile[lane * (RS + 1) + q] = v;
   }
+  // (the histogram kernel over the records trusts the ids to be below its number of slots: the
+  // caller compares what was seen here with the bound it sizes the histogram by)
+  for (int off = 32; off > 0; off >>= 1) top = max(top, (unsigned)__shfl_down((int)top, off));
+  if (lane == 0 && top != 0) atomicMax(largest_id, top);
   __syncthreads();
   const size_t rows = min((size_t)64, n - r0);
   for (size_t e = threadIdx.x; e < rows * RS; e += 256) {
@@ -230,17 +237,16 @@ k_ix_part(const uint8_t *__restrict__ bytes, size_t stride8, const unsigned *__r
 //
 // LDS layout (bin-major, as the other histograms): word0 of (feature f, bin) at
 // bin * bin_stride + (f / 16) * (PAIR ? 32 : 16) + f % 16, bin_stride = blocks *
-// (PAIR ? 32 : 16), word1 16 words further.  A bin id is clamped to the
-// histogram, so that no input can write outside it.  The slab of a work item is
+// (PAIR ? 32 : 16), word1 16 words further.  The slab of a work item is
 // the LDS image: blocks * 16 * slots entries of one or two words.
 // POW2: a power of two of bytes between the bins of the LDS image (stride_shift): the offset of
-// a cell is a shift and an add instead of a multiply and an add.  CLAMP: fewer than 256 bins per
-// feature, bin ids are clamped to the histogram (with 256 no bin id can leave it).
+// a cell is a shift and an add instead of a multiply and an add.  Every bin id is below `slots`:
+// the caller sizes the histogram by the largest id the records hold (k_to_records reports it).
 // lay_blocks: 16-feature blocks the image is laid out for (0: the pieces of the workgroup's
 // group); more than the matrix has makes the stride a power of two.
 // HI: words Q, Q + 1, ... of a record are the row's ninth-bit words; a feature whose bit is set
 // (id 256) is not accumulated (AccumulateRow, HI = 2).
-template <bool PAIR, bool POW2 = false, bool CLAMP = true, bool HI = false>
+template <bool PAIR, bool POW2 = false, bool HI = false>
 __global__ void __launch_bounds__(kHistThreads)
 k_hist_rec(const uint32_t *__restrict__ rec, int RS, const unsigned *__restrict__ ids, int Q, int slots,
            const float *__restrict__ g, const float *__restrict__ h, const int *__restrict__ shifts,
@@ -265,7 +271,6 @@ k_hist_rec(const uint32_t *__restrict__ rec, int RS, const unsigned *__restrict_
   for (unsigned i = threadIdx.x; i < words; i += kHistThreads) lds[i] = 0ull;
   __syncthreads();
   const int sg = shifts[0], sh = shifts[1];
-  const unsigned last_bin = (unsigned)slots - 1u;
   const unsigned lane = threadIdx.x & 63u, wave = threadIdx.x >> 6;
   const unsigned j = (lane >> 2) & 3u, i4 = lane & 3u;
   // The (row, piece) pairs of the work item, row-major, are dealt out 64 at a time: wave v takes
@@ -344,14 +349,15 @@ k_hist_rec(const uint32_t *__restrict__ rec, int RS, const unsigned *__restrict_
         const uint32_t rc = s_ == 0 ? R.q[k].z : s_ == 1 ? R.q[k].w : s_ == 2 ? R.q[k].x : R.q[k].y;
         const uint32_t rd = s_ == 0 ? R.q[k].w : s_ == 1 ? R.q[k].x : s_ == 2 ? R.q[k].y : R.q[k].z;
         const uint32_t lo = (j & 1u) ? rb : ra, hi = (j & 1u) ? rd : rc;
-        const uint32_t sel = (j & 2u) ? hi : lo;
+        // the quad, turned so that the byte of step t sits at byte t whatever the lane: the byte
+        // is then picked by a constant (an operand modifier of the shift below, not an instruction)
+        const uint32_t sel = __builtin_amdgcn_alignbit((j & 2u) ? hi : lo, (j & 2u) ? hi : lo, 8u * i4);
         if (4u * ((unsigned)piece0 + piece) + qi < (unsigned)Q) {   // quads past the matrix do not exist
 #pragma unroll
           for (int t = 0; t < 4; ++t) {
             const unsigned bi = ((unsigned)t + i4) & 3u;
             unsigned off;
-            unsigned bin = __builtin_amdgcn_ubfe(sel, 8u * bi, 8u);
-            if (CLAMP) bin = min(bin, last_bin);
+            const unsigned bin = (sel >> (8 * t)) & 255u;
             if (POW2) off = (bin << stride_shift) + (piece_b + (4u * qi + bi) * 8u);
             else off = __umul24(bin, bin_stride_b) + (piece_b + (4u * qi + bi) * 8u);
             unsigned long long *cell = reinterpret_cast<unsigned long long *>(lds_b + off);
