@@ -151,8 +151,13 @@ class ExactSortBuilder : public TreeBuilder {
     d_y_ = DevAlloc<float>(n_);
     d_labels_ = DevAlloc<uint8_t>(n_);
     d_yhat_ = DevAlloc<float>(n_ * K_);
+    // Logistic gradients of 0/1 labels travel as one float per row (PackGrad): no h array, and
+    // 12 instead of 16 bytes per place of the lists.
+    pack_ = cfg.objective == kLogisticRegression && data->y.size() == n_ &&
+            std::all_of(data->y.begin(), data->y.end(), [](float v) { return v == 0.0f || v == 1.0f; });
+    harr_ = pair_ && !pack_;
     d_g_ = DevAlloc<float>(n_ * K_);
-    d_h_ = pair_ ? DevAlloc<float>(n_ * K_) : nullptr;
+    d_h_ = harr_ ? DevAlloc<float>(n_ * K_) : nullptr;
     d_leaf_ = DevAlloc<unsigned>(n_);
     d_node_of_ = DevAlloc<unsigned>(n_);
     if (!data->y.empty()) HIP_OK(hipMemcpy(d_y_, data->y.data(), n_ * sizeof(float), hipMemcpyHostToDevice));
@@ -163,7 +168,7 @@ class ExactSortBuilder : public TreeBuilder {
     data->y_hat.assign(n_ * K_, init);  // garden.cu:104
 
     d_went_right_ = DevAlloc<unsigned long long>(stride_ / 64);
-    d_gh_ = pair_ ? DevAlloc<float2>(n_) : nullptr;
+    d_gh_ = harr_ ? DevAlloc<float2>(n_) : nullptr;
     // two sets of lists (ids, ranks, gradients in list order), written and read in turn by the
     // levels; the gradients of the second set also serve the root's lists
     const size_t words = (size_t)F_ * stride_;
@@ -174,7 +179,7 @@ class ExactSortBuilder : public TreeBuilder {
       }
       if (D_ > 2 || b == 1) {
         d_lg_[b] = DevAlloc<float>(words);
-        d_lh_[b] = pair_ ? DevAlloc<float>(words) : nullptr;
+        d_lh_[b] = harr_ ? DevAlloc<float>(words) : nullptr;
       }
     }
     const int max_nodes = 1 << (D_ - 1);
@@ -240,7 +245,7 @@ class ExactSortBuilder : public TreeBuilder {
       hipLaunchKernelGGL(k_grad_squared, dim3(GridFor(n_, 256)), dim3(256), 0, stream_, d_y_, d_yhat_, d_g_, n_, d_gmax_);
       hipLaunchKernelGGL(k_set_shift, dim3(1), dim3(64), 0, stream_, d_gmax_, d_shifts_);
     } else if (cfg_.objective == kLogisticRegression) {
-      hipLaunchKernelGGL(k_grad_logistic, dim3(GridFor(n_, 256)), dim3(256), 0, stream_, d_y_, d_yhat_, d_g_, d_h_, n_);
+      hipLaunchKernelGGL(k_grad_logistic, dim3(GridFor(n_, 256)), dim3(256), 0, stream_, d_y_, d_yhat_, d_g_, d_h_, n_);  // (no d_h_: packed)
     } else {
       hipLaunchKernelGGL(k_grad_softmax, dim3(GridFor(n_, 256)), dim3(256), 0, stream_, d_labels_, d_yhat_, d_g_, d_h_, n_, K_);
     }
@@ -294,7 +299,14 @@ class ExactSortBuilder : public TreeBuilder {
     if (!inspect_) throw std::runtime_error("gradients of the last round are only kept with inspection on");
     HIP_OK(hipStreamSynchronize(stream_));
     HIP_OK(hipMemcpy(g, d_g_, n_ * K_ * sizeof(float), hipMemcpyDeviceToHost));
-    if (h) {
+    if (pack_) {
+      for (size_t i = 0; i < n_; ++i) {
+        float gv, hv;
+        UnpackGrad(g[i], &gv, &hv);
+        g[i] = gv;
+        if (h) h[i] = hv;
+      }
+    } else if (h) {
       if (pair_)
         HIP_OK(hipMemcpy(h, d_h_, n_ * K_ * sizeof(float), hipMemcpyDeviceToHost));
       else
@@ -355,12 +367,15 @@ class ExactSortBuilder : public TreeBuilder {
     SampleColumns();
     hipLaunchKernelGGL(k_init_root, dim3(1), dim3(64), 0, stream_, d_tot_[0], d_seg_[0], (unsigned long long)n_,
                        (unsigned *)nullptr);
-    hipLaunchKernelGGL(k_sum_grad, dim3(GridFor(n_, 256, 1024)), dim3(256), 0, stream_, g, h, n_, d_shifts_, d_tot_[0]);
+    if (pack_)
+      hipLaunchKernelGGL(k_ex_sum_packed, dim3(GridFor(n_, 256, 1024)), dim3(256), 0, stream_, g, n_, d_shifts_, d_tot_[0]);
+    else
+      hipLaunchKernelGGL(k_sum_grad, dim3(GridFor(n_, 256, 1024)), dim3(256), 0, stream_, g, h, n_, d_shifts_, d_tot_[0]);
     HIP_OK(hipMemsetAsync(d_node_of_, 0, n_ * sizeof(unsigned), stream_));
     int state = 0;
     // the root's lists: every row, sorted once; this tree's gradients in that order
     const dim3 whole((unsigned)((n_ + kExItem - 1) / kExItem), (unsigned)F_);
-    if (pair_) {
+    if (harr_) {
       hipLaunchKernelGGL(k_ex_pair, dim3(GridFor(n_, 256)), dim3(256), 0, stream_, g, h, d_gh_, n_);
       hipLaunchKernelGGL((k_ex_gather<true>), whole, dim3(kExThreads), 0, stream_, sd_->lists, stride_, g, d_gh_,
                          d_lg_[1], d_lh_[1], n_);
@@ -377,19 +392,21 @@ class ExactSortBuilder : public TreeBuilder {
       hipLaunchKernelGGL(k_plan, dim3(1), dim3(1024), 0, stream_, d_tot_[state], d_seg_[state], L, 0, kExItem, d_work_,
                          d_n_work_, d_node_first_, d_node_items_, (unsigned long long *)nullptr,
                          (const SplitRec *)nullptr, grid_items, d_overflow_, 0u, (unsigned *)nullptr);
-#define ARB_EX(P, D)                                                                                                  \
+#define ARB_EX(P, D, K)                                                                                               \
   do {                                                                                                                \
-    hipLaunchKernelGGL((k_ex_partial<P>), per_item, dim3(kExThreads), 0, stream_, lists, stride_, d_shifts_, d_work_, \
-                       d_n_work_, d_part_, max_items_);                                                               \
+    hipLaunchKernelGGL((k_ex_partial<P, K>), per_item, dim3(kExThreads), 0, stream_, lists, stride_, d_shifts_,      \
+                       d_work_, d_n_work_, d_part_, max_items_);                                                      \
     hipLaunchKernelGGL((k_ex_offsets<ExSum>), per_node, dim3(64), 0, stream_, d_part_, d_off_, d_node_first_,        \
                        d_node_items_, max_items_);                                                                    \
-    hipLaunchKernelGGL((k_ex_scan<P, D>), per_item, dim3(kExThreads), 0, stream_, lists, stride_, d_shifts_, d_work_, \
-                       d_n_work_, d_off_, d_tot_[state], d_seg_[state], gp, d_best_, max_items_);                     \
+    hipLaunchKernelGGL((k_ex_scan<P, D, K>), per_item, dim3(kExThreads), 0, stream_, lists, stride_, d_shifts_,      \
+                       d_work_, d_n_work_, d_off_, d_tot_[state], d_seg_[state], gp, d_best_, max_items_);            \
   } while (0)
-      if (pair_ && f64_) ARB_EX(true, true);
-      else if (pair_) ARB_EX(true, false);
-      else if (f64_) ARB_EX(false, true);
-      else ARB_EX(false, false);
+      if (pack_ && f64_) ARB_EX(true, true, true);
+      else if (pack_) ARB_EX(true, false, true);
+      else if (pair_ && f64_) ARB_EX(true, true, false);
+      else if (pair_) ARB_EX(true, false, false);
+      else if (f64_) ARB_EX(false, true, false);
+      else ARB_EX(false, false, false);
 #undef ARB_EX
       hipLaunchKernelGGL(k_ex_merge, per_node, dim3(64), 0, stream_, d_best_, d_node_first_, d_node_items_, max_items_,
                          F_, d_cand_);
@@ -416,7 +433,7 @@ class ExactSortBuilder : public TreeBuilder {
                            d_work_, d_n_work_, d_lefts_, d_left_bits_, max_items_);
         hipLaunchKernelGGL((k_ex_offsets<unsigned>), per_node, dim3(64), 0, stream_, d_lefts_, d_left_off_,
                            d_node_first_, d_node_items_, max_items_);
-        if (pair_)
+        if (harr_)
           hipLaunchKernelGGL((k_ex_scatter<true>), per_item, dim3(kExThreads), 0, stream_, lists, d_ids_[b], d_ranks_[b],
                              d_lg_[b], d_lh_[b], stride_, d_left_bits_, d_work_, d_n_work_, d_left_off_,
                              d_seg_[state], d_seg_[state ^ 1], max_items_);
@@ -441,6 +458,8 @@ class ExactSortBuilder : public TreeBuilder {
   size_t n_ = 0, stride_ = 0;
   int F_ = 0, K_ = 1, D_ = 2;
   bool pair_ = false, f64_ = false, inspect_ = false, sampling_ = false;
+  bool pack_ = false;  // logistic gradients packed into one float per row
+  bool harr_ = false;  // the gradients are two arrays (g, h)
   unsigned max_items_ = 0;
   hipStream_t stream_ = nullptr;
   std::default_random_engine rnd_;

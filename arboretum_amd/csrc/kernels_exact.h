@@ -85,21 +85,44 @@ __device__ __forceinline__ void ExLoad8(const T *__restrict__ base, unsigned p0,
 }
 
 // The fixed-point gradients of the rows at the places [p0, p0 + kExPer) of feature f's list, zero past `end`.
-template <bool PAIR>
+// PACK: one float per row holds both (logistic gradients of 0/1 labels, PackGrad); no h lists.
+template <bool PAIR, bool PACK>
 __device__ __forceinline__ void ExLoadSums(const ExLists &ls, size_t fbase, unsigned p0, unsigned end, int sg, int sh,
                                            ExSum *v) {
   float gv[kExPer], hv[kExPer];
   ExLoad8(ls.g + fbase, p0, end, 0.0f, gv);
-  if (PAIR) ExLoad8(ls.h + fbase, p0, end, 0.0f, hv);
+  if (PAIR && !PACK) ExLoad8(ls.h + fbase, p0, end, 0.0f, hv);
 #pragma unroll
   for (int j = 0; j < kExPer; ++j) {
-    v[j].g = p0 + j < end ? ToFixed(gv[j], sg) : 0;
-    v[j].h = PAIR && p0 + j < end ? ToFixed(hv[j], sh) : 0;
+    float g1 = gv[j], h1 = PAIR && !PACK ? hv[j] : 0.0f;
+    if (PACK) UnpackGrad(gv[j], &g1, &h1);
+    v[j].g = p0 + j < end ? ToFixed(g1, sg) : 0;
+    v[j].h = PAIR && p0 + j < end ? ToFixed(h1, sh) : 0;
+  }
+}
+
+// Sum of the fixed-point gradients of all rows from packed logistic gradients: the totals of
+// the root.  tot[0].g / .h must be zero at launch; integer sums, any order.
+__global__ void __launch_bounds__(256)
+k_ex_sum_packed(const float *__restrict__ packed, size_t n, const int *__restrict__ shifts, NodeSum *__restrict__ tot) {
+  const int sg = shifts[0], sh = shifts[1];
+  long long a = 0, b = 0;
+  for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (size_t)gridDim.x * blockDim.x) {
+    float g1, h1;
+    UnpackGrad(packed[i], &g1, &h1);
+    a += ToFixed(g1, sg);
+    b += ToFixed(h1, sh);
+  }
+  a = WaveSumLL(a);
+  b = WaveSumLL(b);
+  if ((threadIdx.x & 63) == 0) {
+    atomicAdd(reinterpret_cast<unsigned long long *>(&tot[0].g), (unsigned long long)a);
+    atomicAdd(reinterpret_cast<unsigned long long *>(&tot[0].h), (unsigned long long)b);
   }
 }
 
 // grid (items, F): the sum of the gradients over every work item's piece of every feature's list.
-template <bool PAIR>
+template <bool PAIR, bool PACK>
 __global__ void __launch_bounds__(kExThreads)
 k_ex_partial(const ExLists ls, size_t stride, const int *__restrict__ shifts, const WorkItem *__restrict__ work,
              const unsigned *__restrict__ n_work, ExSum *__restrict__ part, unsigned max_items) {
@@ -108,7 +131,7 @@ k_ex_partial(const ExLists ls, size_t stride, const int *__restrict__ shifts, co
   if (w >= *n_work) return;
   const WorkItem it = work[w];
   ExSum v[kExPer];
-  ExLoadSums<PAIR>(ls, (size_t)f * stride, it.begin + threadIdx.x * kExPer, it.end, shifts[0], shifts[1], v);
+  ExLoadSums<PAIR, PACK>(ls, (size_t)f * stride, it.begin + threadIdx.x * kExPer, it.end, shifts[0], shifts[1], v);
   ExSum mine = v[0];
 #pragma unroll
   for (int j = 1; j < kExPer; ++j) mine = mine + v[j];
@@ -193,7 +216,7 @@ __device__ __forceinline__ bool ExBetter(float og, int ob, float gain, int bin) 
 // sums of the node's items before it), the gain wherever the rank changes to the next place of the
 // node, and the best candidate of the piece, ties to the highest rank.
 // best: [F][max_items].
-template <bool PAIR, bool F64>
+template <bool PAIR, bool F64, bool PACK>
 __global__ void __launch_bounds__(kExThreads)
 k_ex_scan(const ExLists ls, size_t stride, const int *__restrict__ shifts,
           const WorkItem *__restrict__ work, const unsigned *__restrict__ n_work, const ExSum *__restrict__ off,
@@ -210,7 +233,7 @@ k_ex_scan(const ExLists ls, size_t stride, const int *__restrict__ shifts,
   const int sg = shifts[0], sh = shifts[1];
   const unsigned p0 = it.begin + threadIdx.x * kExPer;
   ExSum v[kExPer];
-  ExLoadSums<PAIR>(ls, fbase, p0, it.end, sg, sh, v);
+  ExLoadSums<PAIR, PACK>(ls, fbase, p0, it.end, sg, sh, v);
   // ranks at this thread's places and at the one after them (which may lie in the next item)
   unsigned rk[kExPer + 1];
   ExLoad8(ls.ranks + fbase, p0, node_end, 0u, rk);
@@ -355,7 +378,8 @@ k_ex_count(const unsigned *__restrict__ ids, size_t stride, const unsigned long 
 }
 
 // grid (items, F): the stable partition of every piece into the lists of the two children, with
-// the rank and the gradients of every row next to its id.  The piece is put in order in LDS
+// the rank and the gradients of every row next to its id (PAIR here: the lists hold h beside g;
+// packed gradients are one word, like g alone).  The piece is put in order in LDS
 // (the rows that go left, then the others) and written out from there, so that the stores of a
 // wave are consecutive.
 // left_off: rows of the node's earlier pieces that go left; seg_start / seg_next: first place of
