@@ -4,11 +4,35 @@
 #include <atomic>
 #include <cmath>
 #include <cstring>
+#include <exception>
 #include <limits>
+#include <mutex>
 #include <stdexcept>
 #include <thread>
 
 namespace arb {
+
+namespace {
+// Runs the workers on threads of their own (the caller's included) and hands the first
+// exception of any of them back to the caller instead of ending the process.
+void RunWorkers(size_t workers, const std::function<void(size_t)> &work) {
+  std::exception_ptr failed;
+  std::mutex guard;
+  auto run = [&](size_t t) {
+    try {
+      work(t);
+    } catch (...) {
+      std::lock_guard<std::mutex> lock(guard);
+      if (!failed) failed = std::current_exception();
+    }
+  };
+  std::vector<std::thread> th;
+  for (size_t t = 1; t < workers; ++t) th.emplace_back(run, t);
+  run(0);
+  for (auto &t : th) t.join();
+  if (failed) std::rethrow_exception(failed);
+}
+}  // namespace
 
 void ParallelFor(size_t n, const std::function<void(size_t, size_t)> &fn) {
   unsigned hw = std::thread::hardware_concurrency();
@@ -17,27 +41,20 @@ void ParallelFor(size_t n, const std::function<void(size_t, size_t)> &fn) {
     fn(0, n);
     return;
   }
-  std::vector<std::thread> th;
-  size_t chunk = (n + nt - 1) / nt;
-  for (size_t t = 0; t < nt; ++t) {
-    size_t b = t * chunk, e = std::min(n, b + chunk);
-    if (b >= e) break;
-    th.emplace_back([&fn, b, e] { fn(b, e); });
-  }
-  for (auto &t : th) t.join();
+  const size_t chunk = (n + nt - 1) / nt;
+  RunWorkers(nt, [&](size_t t) {
+    const size_t b = t * chunk, e = std::min(n, b + chunk);
+    if (b < e) fn(b, e);
+  });
 }
 
 void ParallelTasks(size_t n, const std::function<void(size_t)> &fn) {
   const unsigned hw = std::thread::hardware_concurrency();
   const size_t nt = std::max<size_t>(1, std::min<size_t>({(size_t)(hw ? hw : 1), (size_t)16, n}));
   std::atomic<size_t> next{0};
-  auto run = [&]() {
+  RunWorkers(nt, [&](size_t) {
     for (size_t i = next++; i < n; i = next++) fn(i);
-  };
-  std::vector<std::thread> th;
-  for (size_t t = 1; t < nt; ++t) th.emplace_back(run);
-  run();
-  for (auto &t : th) t.join();
+  });
 }
 
 namespace {

@@ -159,6 +159,7 @@ class ExactSortBuilder : public TreeBuilder {
     d_g_ = DevAlloc<float>(n_ * K_);
     d_h_ = harr_ ? DevAlloc<float>(n_ * K_) : nullptr;
     d_leaf_ = DevAlloc<unsigned>(n_);
+    HIP_OK(hipMemsetAsync(d_leaf_, 0, n_ * sizeof(unsigned), stream_));  // (asked for before the first tree: the root)
     d_node_of_ = DevAlloc<unsigned>(n_);
     if (!data->y.empty()) HIP_OK(hipMemcpy(d_y_, data->y.data(), n_ * sizeof(float), hipMemcpyHostToDevice));
     if (!data->labels.empty()) HIP_OK(hipMemcpy(d_labels_, data->labels.data(), n_, hipMemcpyHostToDevice));
