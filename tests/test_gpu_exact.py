@@ -194,6 +194,26 @@ def test_sorted_lists_on_random_configurations(arb, oracle, seed):
 
 
 @pytest.mark.parametrize("objective", [0, 1])
+def test_sorted_lists_over_many_work_items(arb, oracle, objective):
+    # a million rows: several hundred work items per list at the root (the sums and left counts of a
+    # node's items are scanned in rounds of 64), many rows per distinct value, nodes of every size
+    n = 1_000_000
+    rng = np.random.default_rng(21 + objective)
+    X = np.empty((n, 3), np.float32)
+    X[:, 0] = np.round(rng.normal(size=n) * 9000.0)            # about 50 000 distinct values
+    X[:, 1] = np.round(rng.exponential(size=n) * 3000.0)       # skewed: many rows share the small values
+    X[:, 2] = rng.integers(0, 7, size=n)
+    s = np.tanh(X[:, 0] / 9000.0) + (X[:, 1] > 2000.0) + 0.2 * X[:, 2]
+    y = (s + 0.3 * rng.normal(size=n)).astype(np.float32) if objective == 0 else \
+        (rng.random(n) < 1 / (1 + np.exp(-(s - 1.0)))).astype(np.float32)
+    cfg = {"objective": objective, "method": 0, "internals": {"double_precision": True},
+           "tree": {"max_depth": 6, "eta": 0.3, "lambda": 1.0, "min_child_weight": 1.0}}
+    ob = oracle.Booster(X, y=y, config=cfg)
+    assert 4096 < ob.params.hist_size < 65536
+    _same_trees(ob, arb.Garden(cfg, arb.DMatrix(X, y=y)), 2)
+
+
+@pytest.mark.parametrize("objective", [0, 1])
 def test_sorted_lists_match_the_checker_beyond_16_bit_ranks(arb, oracle, objective):
     # 100 000 distinct values per feature: the checker's exact mode with 32-bit ranks
     n = 100000
